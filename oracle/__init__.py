@@ -1,0 +1,214 @@
+"""ctypes front end of the CPU oracle (TEST INFRASTRUCTURE ONLY).
+
+`load()` returns a thin numpy wrapper over ``oracle/liboracle.so`` (this repo's
+restatement of the reference CPU algorithms, built by ``oracle/Makefile``);
+`load_ref()` returns the same wrapper over ``oracle/_ref/libtagi_ref.so`` (the
+reference's own sources compiled in place) or ``None`` when that library was not
+built. Only tests, the smoke test and the benchmark's CPU-baseline leg may
+import this package; the shipped library never does.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_F = ctypes.POINTER(ctypes.c_float)
+_I = ctypes.POINTER(ctypes.c_int)
+
+
+def _fp(a):
+    if a is None:
+        return ctypes.cast(None, _F)
+    assert a.dtype == np.float32 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(_F)
+
+
+def _ip(a):
+    assert a.dtype == np.int32 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(_I)
+
+
+def f32(x):
+    return np.ascontiguousarray(x, dtype=np.float32)
+
+
+def build(ref=False):
+    """Compile liboracle.so (and, with ref=True, _ref/libtagi_ref.so)."""
+    targets = ["all"] + (["ref"] if ref else [])
+    subprocess.run(["make", "-C", _HERE, "-j8"] + targets, check=True,
+                   stdout=subprocess.DEVNULL)
+
+
+class Oracle:
+    """Numpy-in / numpy-out calls; `prefix` selects oracle_* or ref_* symbols."""
+
+    def __init__(self, path, prefix):
+        self.lib = ctypes.CDLL(path)
+        self.prefix = prefix
+        self.is_ref = prefix == "ref_"
+        for name in ("cap_factor",):
+            getattr(self.lib, prefix + name).restype = ctypes.c_float
+
+    def _fn(self, name):
+        return getattr(self.lib, self.prefix + name)
+
+    # ---- linear ---------------------------------------------------------
+    def linear_fwd(self, mu_w, var_w, mu_b, var_b, mu_a, var_a, threads=1):
+        N, K = mu_w.shape
+        B = mu_a.shape[0]
+        bias = mu_b is not None
+        mu_z = np.empty((B, N), np.float32)
+        var_z = np.empty((B, N), np.float32)
+        self._fn("linear_fwd")(_fp(mu_w), _fp(var_w), _fp(mu_b), _fp(var_b),
+                               _fp(mu_a), _fp(var_a), K, N, B, int(bias),
+                               threads, _fp(mu_z), _fp(var_z))
+        return mu_z, var_z
+
+    def linear_bwd_dz(self, mu_w, jcb, dmu, dvar, threads=1):
+        N, K = mu_w.shape
+        B = dmu.shape[0]
+        om = np.empty((B, K), np.float32)
+        ov = np.empty((B, K), np.float32)
+        self._fn("linear_bwd_dz")(_fp(mu_w), _fp(jcb), _fp(dmu), _fp(dvar), K,
+                                  N, B, threads, _fp(om), _fp(ov))
+        return om, ov
+
+    def linear_bwd_dw(self, var_w, mu_a, dmu, dvar, threads=1):
+        N, K = var_w.shape
+        B = dmu.shape[0]
+        om = np.empty((N, K), np.float32)
+        ov = np.empty((N, K), np.float32)
+        self._fn("linear_bwd_dw")(_fp(var_w), _fp(mu_a), _fp(dmu), _fp(dvar),
+                                  K, N, B, threads, _fp(om), _fp(ov))
+        return om, ov
+
+    def linear_bwd_db(self, var_b, dmu, dvar, threads=1):
+        B, N = dmu.shape
+        om = np.empty(N, np.float32)
+        ov = np.empty(N, np.float32)
+        self._fn("linear_bwd_db")(_fp(var_b), _fp(dmu), _fp(dvar), N, B,
+                                  threads, _fp(om), _fp(ov))
+        return om, ov
+
+    # ---- conv index tables -------------------------------------------------
+    def conv2d_out_size(self, kernel, stride, wi, hi, pad, pad_type):
+        wo, ho = ctypes.c_int(0), ctypes.c_int(0)
+        rc = self._fn("conv2d_out_size")(kernel, stride, wi, hi, pad, pad_type,
+                                         ctypes.byref(wo), ctypes.byref(ho))
+        if rc != 0:
+            raise ValueError("invalid conv2d geometry")
+        return wo.value, ho.value
+
+    def conv2d_build_idx(self, kernel, stride, wi, hi, pad, pad_type,
+                         param_pad_idx):
+        wo, ho = self.conv2d_out_size(kernel, stride, wi, hi, pad, pad_type)
+        k2 = kernel * kernel
+        fm = np.zeros(wo * ho * k2, np.int32)
+        zw = np.zeros(wi * hi * k2 + 16, np.int32)
+        zud = np.zeros(wi * hi * k2 + 16, np.int32)
+        w, h = ctypes.c_int(0), ctypes.c_int(0)
+        rc = self._fn("conv2d_build_idx")(kernel, stride, wi, hi, wo, ho, pad,
+                                          pad_type, param_pad_idx, _ip(fm),
+                                          _ip(zw), _ip(zud), ctypes.byref(w),
+                                          ctypes.byref(h))
+        if rc != 0:
+            raise ValueError("conv2d index construction failed (%d)" % rc)
+        n = w.value * h.value
+        return dict(Fmwa_2=fm, FCzwa_1=zw[:n].copy(), Szz_ud=zud[:n].copy(),
+                    w=w.value, h=h.value, wo=wo, ho=ho)
+
+    # ---- conv ---------------------------------------------------------------
+    def conv2d_fwd(self, mu_w, var_w, mu_b, var_b, mu_a, var_a, aidx, woho,
+                   fo, wihi, fi, ki, B, threads=1):
+        bias = mu_b is not None
+        mu_z = np.empty(B * fo * woho, np.float32)
+        var_z = np.empty(B * fo * woho, np.float32)
+        self._fn("conv2d_fwd")(_fp(mu_w), _fp(var_w), _fp(mu_b), _fp(var_b),
+                               _fp(mu_a), _fp(var_a), _ip(aidx), woho, fo,
+                               wihi, fi, ki, B, int(bias), threads, _fp(mu_z),
+                               _fp(var_z))
+        return mu_z, var_z
+
+    def conv2d_bwd_dz(self, mu_w, jcb, dmu, dvar, zw_idx, zud_idx, woho, fo,
+                      wihi, fi, ki, nr, B, threads=1):
+        tmp = np.empty(B * fi * wihi, np.float32)
+        om = np.empty(B * fi * wihi, np.float32)
+        ov = np.empty(B * fi * wihi, np.float32)
+        self._fn("conv2d_bwd_dz")(_fp(mu_w), _fp(jcb), _fp(dmu), _fp(dvar),
+                                  _ip(zw_idx), _ip(zud_idx), woho, fo, wihi,
+                                  fi, ki, nr, B, threads, _fp(tmp), _fp(om),
+                                  _fp(ov))
+        return om, ov
+
+    def conv2d_bwd_dw(self, var_w, var_b, mu_a, dmu, dvar, aidx, B, fo, woho,
+                      wihi, fi, ki, threads=1):
+        bias = var_b is not None
+        nw = ki * ki * fi * fo
+        t1 = np.empty(B * fo * woho, np.float32)
+        t2 = np.empty(B * fo * woho, np.float32)
+        om = np.empty(nw, np.float32)
+        ov = np.empty(nw, np.float32)
+        bm = np.zeros(fo, np.float32)
+        bv = np.zeros(fo, np.float32)
+        self._fn("conv2d_bwd_dw")(_fp(var_w), _fp(var_b), _fp(mu_a), _fp(dmu),
+                                  _fp(dvar), _ip(aidx), B, fo, woho, wihi, fi,
+                                  ki, int(bias), threads, _fp(t1), _fp(t2),
+                                  _fp(om), _fp(ov), _fp(bm), _fp(bv))
+        return (om, ov, bm, bv) if bias else (om, ov, None, None)
+
+    # ---- update / output / relu ----------------------------------------------
+    def cap_factor(self, batch_size, prev=1.0):
+        return float(self._fn("cap_factor")(int(batch_size),
+                                            ctypes.c_float(prev)))
+
+    def param_update(self, mu, var, dmu, dvar, cap, weights=True):
+        """In place on copies; returns (mu, var, clamped_count)."""
+        mu, var = mu.copy(), var.copy()
+        args = [_fp(mu), _fp(var), _fp(dmu), _fp(dvar),
+                ctypes.c_size_t(mu.size), ctypes.c_float(cap)]
+        if self.is_ref:
+            args.append(int(weights))
+        cnt = self._fn("param_update")(*args)
+        return mu, var, (cnt if weights else 0)
+
+    def out_update_dense(self, mu_a, var_a, jcb, obs, var_obs, dmu, dvar):
+        dmu, dvar = dmu.copy(), dvar.copy()
+        self._fn("out_update_dense")(_fp(mu_a), _fp(var_a), _fp(jcb), _fp(obs),
+                                     _fp(var_obs), obs.size, _fp(dmu),
+                                     _fp(dvar))
+        return dmu, dvar
+
+    def out_update_indexed(self, mu_a, var_a, jcb, obs, var_obs, sel, n_obs,
+                           n_enc, dmu, dvar):
+        dmu, dvar = dmu.copy(), dvar.copy()
+        args = [_fp(mu_a), _fp(var_a), _fp(jcb), _fp(obs), _fp(var_obs),
+                _ip(sel), n_obs, n_enc, obs.size]
+        if self.is_ref:
+            args.append(int(mu_a.size))
+        args += [_fp(dmu), _fp(dvar)]
+        self._fn("out_update_indexed")(*args)
+        return dmu, dvar
+
+    def relu_fwd(self, mu_z, var_z):
+        mu_a = np.empty_like(mu_z)
+        jcb = np.empty_like(mu_z)
+        var_a = np.empty_like(mu_z)
+        self._fn("relu_fwd")(_fp(mu_z), _fp(var_z), mu_z.size, _fp(mu_a),
+                             _fp(jcb), _fp(var_a))
+        return mu_a, var_a, jcb
+
+
+def load():
+    path = os.path.join(_HERE, "liboracle.so")
+    if not os.path.exists(path):
+        build()
+    return Oracle(path, "oracle_")
+
+
+def load_ref():
+    path = os.path.join(_HERE, "_ref", "libtagi_ref.so")
+    if not os.path.exists(path):
+        return None
+    return Oracle(path, "ref_")

@@ -1,0 +1,249 @@
+// extern "C" wrappers around the reference's own CPU functions, compiled by
+// oracle/Makefile together with the reference sources where they lie (the
+// REF variable, by default /root/reference) into oracle/_ref/libtagi_ref.so.
+// TEST INFRASTRUCTURE ONLY: used to validate tagi_oracle.cpp bit for bit and to
+// write the golden vectors under tests/golden/. It carries the same signatures
+// as tagi_oracle.h with a `ref_` prefix. No reference source is copied here:
+// this file only includes the reference headers and calls into them.
+#include <cstring>
+#include <stdexcept>
+#include <vector>
+
+#include "activation.h"
+#include "base_layer.h"
+#include "base_output_updater.h"
+#include "conv2d_layer.h"
+#include "linear_layer.h"
+
+namespace {
+std::vector<float> vec(const float *p, size_t n) {
+    return p ? std::vector<float>(p, p + n) : std::vector<float>();
+}
+std::vector<int> ivec(const int *p, size_t n) { return std::vector<int>(p, p + n); }
+void put(const std::vector<float> &v, float *out) {
+    std::memcpy(out, v.data(), v.size() * sizeof(float));
+}
+}  // namespace
+
+extern "C" {
+
+void ref_linear_fwd(const float *mu_w, const float *var_w, const float *mu_b,
+                    const float *var_b, const float *mu_a, const float *var_a,
+                    int K, int N, int B, int bias, int threads, float *mu_z,
+                    float *var_z) {
+    auto mw = vec(mu_w, (size_t)N * K), vw = vec(var_w, (size_t)N * K);
+    auto mb = vec(bias ? mu_b : nullptr, N), vb = vec(bias ? var_b : nullptr, N);
+    auto ma = vec(mu_a, (size_t)B * K), va = vec(var_a, (size_t)B * K);
+    std::vector<float> mz((size_t)B * N), vz((size_t)B * N);
+    if (threads > 1)
+        linear_fwd_mean_var_mp(mw, vw, mb, vb, ma, va, K, N, B, bias != 0, threads, mz, vz);
+    else
+        linear_fwd_mean_var(mw, vw, mb, vb, ma, va, 0, N * B, K, N, B, bias != 0, mz, vz);
+    put(mz, mu_z);
+    put(vz, var_z);
+}
+
+void ref_linear_bwd_dz(const float *mu_w, const float *jcb, const float *delta_mu,
+                       const float *delta_var, int K, int N, int B, int threads,
+                       float *delta_mu_z, float *delta_var_z) {
+    auto mw = vec(mu_w, (size_t)N * K), jc = vec(jcb, (size_t)B * K);
+    auto dm = vec(delta_mu, (size_t)B * N), dv = vec(delta_var, (size_t)B * N);
+    std::vector<float> om((size_t)B * K), ov((size_t)B * K);
+    if (threads > 1)
+        linear_bwd_fc_delta_z_mp(mw, jc, dm, dv, K, N, B, threads, om, ov);
+    else
+        linear_bwd_fc_delta_z(mw, jc, dm, dv, K, N, B, 0, B * K, om, ov);
+    put(om, delta_mu_z);
+    put(ov, delta_var_z);
+}
+
+void ref_linear_bwd_dw(const float *var_w, const float *mu_a, const float *delta_mu,
+                       const float *delta_var, int K, int N, int B, int threads,
+                       float *delta_mu_w, float *delta_var_w) {
+    auto vw = vec(var_w, (size_t)N * K), ma = vec(mu_a, (size_t)B * K);
+    auto dm = vec(delta_mu, (size_t)B * N), dv = vec(delta_var, (size_t)B * N);
+    std::vector<float> om((size_t)N * K), ov((size_t)N * K);
+    if (threads > 1)
+        linear_bwd_fc_delta_w_mp(vw, ma, dm, dv, K, N, B, threads, om, ov);
+    else
+        linear_bwd_fc_delta_w(vw, ma, dm, dv, K, N, B, 0, K * N, om, ov);
+    put(om, delta_mu_w);
+    put(ov, delta_var_w);
+}
+
+void ref_linear_bwd_db(const float *var_b, const float *delta_mu, const float *delta_var,
+                       int N, int B, int threads, float *delta_mu_b, float *delta_var_b) {
+    auto vb = vec(var_b, N);
+    auto dm = vec(delta_mu, (size_t)B * N), dv = vec(delta_var, (size_t)B * N);
+    std::vector<float> om(N), ov(N);
+    if (threads > 1)
+        linear_bwd_fc_delta_b_mp(vb, dm, dv, N, B, threads, om, ov);
+    else
+        linear_bwd_fc_delta_b(vb, dm, dv, N, B, 0, N, om, ov);
+    put(om, delta_mu_b);
+    put(ov, delta_var_b);
+}
+
+int ref_conv2d_out_size(int kernel, int stride, int wi, int hi, int pad, int pad_type,
+                        int *wo, int *ho) {
+    try {
+        std::tie(*wo, *ho) = compute_downsample_img_size_v2(kernel, stride, wi, hi, pad, pad_type);
+    } catch (const std::exception &) {
+        return -1;
+    }
+    return 0;
+}
+
+int ref_conv2d_build_idx(int kernel, int stride, int wi, int hi, int wo, int ho, int pad,
+                         int pad_type, int param_pad_idx, int *Fmwa_2, int *FCzwa_1,
+                         int *Szz_ud, int *w, int *h) {
+    try {
+        Conv2dIndex idx =
+            get_conv2d_idx(kernel, stride, wi, hi, wo, ho, pad, pad_type, -1, -1, param_pad_idx);
+        std::memcpy(Fmwa_2, idx.Fmwa_2_idx.data(), idx.Fmwa_2_idx.size() * sizeof(int));
+        std::memcpy(FCzwa_1, idx.FCzwa_1_idx.data(), idx.FCzwa_1_idx.size() * sizeof(int));
+        std::memcpy(Szz_ud, idx.Szz_ud_idx.data(), idx.Szz_ud_idx.size() * sizeof(int));
+        *w = idx.w;
+        *h = idx.h;
+    } catch (const std::exception &) {
+        return -1;
+    }
+    return 0;
+}
+
+void ref_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
+                    const float *var_b, const float *mu_a, const float *var_a,
+                    const int *aidx, int woho, int fo, int wihi, int fi, int ki, int B,
+                    int bias, int threads, float *mu_z, float *var_z) {
+    const size_t nw = (size_t)ki * ki * fi * fo;
+    auto mw = vec(mu_w, nw), vw = vec(var_w, nw);
+    auto mb = vec(bias ? mu_b : nullptr, fo), vb = vec(bias ? var_b : nullptr, fo);
+    auto ma = vec(mu_a, (size_t)B * fi * wihi), va = vec(var_a, (size_t)B * fi * wihi);
+    auto ai = ivec(aidx, (size_t)woho * ki * ki);
+    std::vector<float> mz((size_t)B * fo * woho), vz((size_t)B * fo * woho);
+    const int pad_idx = wihi * fi * B + 1;
+    if (threads > 1)
+        conv2d_fwd_mean_var_mp(mw, vw, mb, vb, ma, va, ai, woho, fo, wihi, fi, ki, B, pad_idx,
+                               bias != 0, threads, mz, vz);
+    else
+        conv2d_fwd_mean_var(mw, vw, mb, vb, ma, va, ai, woho, fo, wihi, fi, ki, B, pad_idx,
+                            bias != 0, 0, woho * B * fo, mz, vz);
+    put(mz, mu_z);
+    put(vz, var_z);
+}
+
+void ref_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *delta_mu_out,
+                       const float *delta_var_out, const int *zw_idx, const int *zud_idx,
+                       int woho, int fo, int wihi, int fi, int ki, int nr, int B, int threads,
+                       float *tmp, float *delta_mu, float *delta_var) {
+    const size_t nw = (size_t)ki * ki * fi * fo;
+    auto mw = vec(mu_w, nw);
+    auto jc = vec(jcb, (size_t)B * fi * wihi);
+    auto dm = vec(delta_mu_out, (size_t)B * fo * woho), dv = vec(delta_var_out, (size_t)B * fo * woho);
+    auto zw = ivec(zw_idx, (size_t)wihi * nr), zud = ivec(zud_idx, (size_t)wihi * nr);
+    std::vector<float> t1((size_t)B * fi * wihi), om((size_t)B * fi * wihi), ov((size_t)B * fi * wihi);
+    permute_jacobian(jc, wihi, fi, B, t1);
+    const int pad_idx = woho * fo * B + 1;
+    if (threads > 1)
+        conv2d_bwd_delta_z_mp(mw, t1, dm, dv, zw, zud, woho, fo, wihi, fi, ki, nr, nr * fo, B,
+                              pad_idx, threads, om, ov);
+    else
+        conv2d_bwd_delta_z(mw, t1, dm, dv, zw, zud, woho, fo, wihi, fi, ki, nr, nr * fo, B,
+                           pad_idx, 0, wihi * B * fi, om, ov);
+    put(t1, tmp);
+    put(om, delta_mu);
+    put(ov, delta_var);
+}
+
+void ref_conv2d_bwd_dw(const float *var_w, const float *var_b, const float *mu_a,
+                       const float *delta_mu_out, const float *delta_var_out, const int *aidx,
+                       int B, int fo, int woho, int wihi, int fi, int ki, int bias, int threads,
+                       float *tmp_1, float *tmp_2, float *delta_mu_w, float *delta_var_w,
+                       float *delta_mu_b, float *delta_var_b) {
+    const size_t nw = (size_t)ki * ki * fi * fo;
+    auto vw = vec(var_w, nw);
+    auto vb = vec(bias ? var_b : nullptr, fo);
+    auto ma = vec(mu_a, (size_t)B * fi * wihi);
+    auto dm = vec(delta_mu_out, (size_t)B * fo * woho), dv = vec(delta_var_out, (size_t)B * fo * woho);
+    auto ai = ivec(aidx, (size_t)woho * ki * ki);
+    std::vector<float> t1((size_t)B * fo * woho), t2((size_t)B * fo * woho), om(nw), ov(nw);
+    permute_delta(dm, dv, woho, woho * fo, B, t1, t2);
+    const int pad_idx = wihi * fi * B + 1;
+    if (threads > 1)
+        conv2d_bwd_delta_w_mp(vw, ma, t1, t2, ai, B, fo, woho, wihi, fi, ki, pad_idx, threads, om, ov);
+    else
+        conv2d_bwd_delta_w(vw, ma, t1, t2, ai, B, fo, woho, wihi, fi, ki, pad_idx, 0, (int)nw, om, ov);
+    put(t1, tmp_1);
+    put(t2, tmp_2);
+    put(om, delta_mu_w);
+    put(ov, delta_var_w);
+    if (bias) {
+        std::vector<float> bm(fo), bv(fo);
+        conv2d_bwd_delta_b(vb, t1, t2, woho * B, fo, bm, bv);
+        put(bm, delta_mu_b);
+        put(bv, delta_var_b);
+    }
+}
+
+float ref_cap_factor(int batch_size, float prev) {
+    BaseLayer layer;
+    layer.cap_factor_update = prev;
+    layer.set_cap_factor_udapte(batch_size);
+    return layer.cap_factor_update;
+}
+
+// weights != 0: BaseLayer::update_weights, else BaseLayer::update_biases
+int ref_param_update(float *mu, float *var, const float *delta_mu, const float *delta_var,
+                     size_t n, float cap_factor, int weights) {
+    BaseLayer layer;
+    layer.cap_factor_update = cap_factor;
+    layer.bias = true;
+    if (weights) {
+        layer.mu_w = vec(mu, n); layer.var_w = vec(var, n);
+        layer.delta_mu_w = vec(delta_mu, n); layer.delta_var_w = vec(delta_var, n);
+        layer.update_weights();
+        put(layer.mu_w, mu); put(layer.var_w, var);
+        return layer.get_neg_var_w_counter();
+    }
+    layer.mu_b = vec(mu, n); layer.var_b = vec(var, n);
+    layer.delta_mu_b = vec(delta_mu, n); layer.delta_var_b = vec(delta_var, n);
+    layer.update_biases();
+    put(layer.mu_b, mu); put(layer.var_b, var);
+    return 0;
+}
+
+void ref_out_update_dense(const float *mu_a, const float *var_a, const float *jcb,
+                          const float *obs, const float *var_obs, int n, float *delta_mu,
+                          float *delta_var) {
+    auto ma = vec(mu_a, n), va = vec(var_a, n), jc = vec(jcb, n), ob = vec(obs, n), vo = vec(var_obs, n);
+    auto dm = vec(delta_mu, n), dv = vec(delta_var, n);
+    compute_delta_z_output(ma, va, jc, ob, vo, 0, n, dm, dv);
+    put(dm, delta_mu);
+    put(dv, delta_var);
+}
+
+// n_states = block_size * n_obs floats in the state / delta arrays
+void ref_out_update_indexed(const float *mu_a, const float *var_a, const float *jcb,
+                            const float *obs, const float *var_obs, const int *selected_idx,
+                            int n_obs, int n_enc, int n, int n_states, float *delta_mu,
+                            float *delta_var) {
+    auto ma = vec(mu_a, n_states), va = vec(var_a, n_states), jc = vec(jcb, n_states);
+    auto ob = vec(obs, n), vo = vec(var_obs, n);
+    auto si = ivec(selected_idx, n);
+    auto dm = vec(delta_mu, n_states), dv = vec(delta_var, n_states);
+    compute_selected_delta_z_output(ma, va, jc, ob, vo, si, n_obs, n_enc, 0, n, dm, dv);
+    put(dm, delta_mu);
+    put(dv, delta_var);
+}
+
+void ref_relu_fwd(const float *mu_z, const float *var_z, int n, float *mu_a, float *jcb,
+                  float *var_a) {
+    auto mz = vec(mu_z, n), vz = vec(var_z, n);
+    std::vector<float> ma(n), jc(n), va(n);
+    relu_mean_var(mz, vz, 0, n, ma, jc, va);
+    put(ma, mu_a);
+    put(jc, jcb);
+    put(va, var_a);
+}
+
+}  // extern "C"
