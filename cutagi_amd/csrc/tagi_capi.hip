@@ -1,0 +1,464 @@
+// C ABI of the backend (include/tagi_hip.h): argument checks, kernel selection
+// by shape, and the per-device workspace for split-reduction partial sums.
+#include <cstdint>
+#include <cstring>
+#include <mutex>
+
+#include "../../include/tagi_hip.h"
+#include "tagi_internal.h"
+
+using namespace tagi;
+
+namespace {
+
+constexpr int ABI_VERSION = 100;
+constexpr int MAX_DEVICES = 16;
+constexpr int NUM_CU = 256;  // MI355X
+
+#define TAGI_TRY(expr)                          \
+    do {                                        \
+        hipError_t _e = (expr);                 \
+        if (_e != hipSuccess) return (int)_e;   \
+    } while (0)
+
+struct Workspace {
+    float *ptr = nullptr;
+    size_t bytes = 0;
+};
+Workspace g_ws[MAX_DEVICES];
+std::mutex g_ws_mutex;
+
+// Grow-only. Reallocation waits for the device, so buffers still in use by
+// queued kernels are never freed under them.
+int workspace_get(size_t bytes, float **out) {
+    int dev = 0;
+    TAGI_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) return TAGI_ERR_NO_DEVICE;
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    Workspace &w = g_ws[dev];
+    if (w.bytes < bytes) {
+        TAGI_TRY(hipDeviceSynchronize());
+        if (w.ptr != nullptr) TAGI_TRY(hipFree(w.ptr));
+        w.ptr = nullptr;
+        w.bytes = 0;
+        const size_t want = (bytes + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
+        TAGI_TRY(hipMalloc(reinterpret_cast<void **>(&w.ptr), want));
+        w.bytes = want;
+    }
+    *out = w.ptr;
+    return TAGI_OK;
+}
+
+struct Tuning {
+    int fwd_splits = -1;
+    int dz_splits = -1;
+    int dw_splits = -1;
+    int gemv_max_batch = -1;
+    int tile = -1;
+    int conv_dw_splits = -1;
+};
+Tuning g_tune;
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+int pick_tile(int rows) {
+    // tile ids: 0 = 128x128, 1 = 64x128, 2 = 32x128 (rows x columns)
+    if (g_tune.tile >= 0 && g_tune.tile < gemm_tile_count()) return g_tune.tile;
+    if (rows > 64) return 0;
+    if (rows > 32) return 1;
+    return 2;
+}
+
+// Reduction slices so that a launch reaches about one workgroup per CU, while
+// every slice keeps at least `min_tiles` k-tiles of work.
+int pick_splits(int tiles, int reduction, int forced, int min_tiles = 8) {
+    const int kt = gemm_k_tile();
+    const int k_tiles = ceil_div(reduction, kt);
+    int s = forced > 0 ? forced : ceil_div(NUM_CU, tiles);
+    const int cap = k_tiles / min_tiles > 0 ? k_tiles / min_tiles : 1;
+    if (forced <= 0 && s > cap) s = cap;
+    if (s > k_tiles) s = k_tiles;
+    if (s < 1) s = 1;
+    return s;
+}
+
+int gemv_max_batch() { return g_tune.gemv_max_batch >= 0 ? g_tune.gemv_max_batch : 16; }
+
+// Tiled MFMA launch + (when sliced) the fold of the partial sums.
+int run_gemm(GemmMode mode, GemmParams p, bool vec, int forced_splits, hipStream_t stream) {
+    const int tile = pick_tile(p.M);
+    const int tiles = ceil_div(p.M, gemm_tile_rows(tile)) * ceil_div(p.N, gemm_tile_cols(tile));
+    const int kt = gemm_k_tile();
+    int splits = (mode == GEMM_DW && forced_splits <= 0) ? 1
+                                                          : pick_splits(tiles, p.R, forced_splits);
+    int per = ceil_div(ceil_div(p.R, splits), kt) * kt;
+    splits = ceil_div(p.R, per);
+    p.splits = splits;
+    p.r_per_split = per;
+    if (splits > 1) {
+        float *ws = nullptr;
+        const size_t part = (size_t)splits * p.M * p.N;
+        int rc = workspace_get(2 * part * sizeof(float), &ws);
+        if (rc != TAGI_OK) return rc;
+        p.ws0 = ws;
+        p.ws1 = ws + part;
+    }
+    TAGI_TRY(launch_gemm(mode, tile, vec, p, stream));
+    if (splits > 1) {
+        TAGI_TRY(launch_reduce_splits(mode == GEMM_FWD ? EPI_BIAS : EPI_SCALE, p.ws0, p.ws1,
+                                      splits, p.M, p.N, p.e0, p.e1, p.out0, p.out1, p.ldo,
+                                      stream));
+    }
+    return TAGI_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int tagi_hip_version(void) { return ABI_VERSION; }
+
+int tagi_hip_device_count(int *count) {
+    if (count == nullptr) return TAGI_ERR_INVALID_ARG;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) {
+        *count = 0;
+        (void)hipGetLastError();
+        return e == hipErrorNoDevice ? TAGI_OK : (int)e;
+    }
+    *count = n;
+    return TAGI_OK;
+}
+
+const char *tagi_hip_error_string(int code) {
+    switch (code) {
+        case TAGI_OK: return "ok";
+        case TAGI_ERR_INVALID_ARG: return "tagi: invalid argument";
+        case TAGI_ERR_UNSUPPORTED: return "tagi: unsupported shape";
+        case TAGI_ERR_NO_DEVICE: return "tagi: no usable device";
+        default: break;
+    }
+    if (code > 0) return hipGetErrorString((hipError_t)code);
+    return "tagi: unknown error";
+}
+
+int tagi_hip_workspace_reserve(size_t bytes) {
+    float *p = nullptr;
+    return workspace_get(bytes, &p);
+}
+
+int tagi_hip_shutdown(void) {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    int cur = 0;
+    if (hipGetDevice(&cur) != hipSuccess) return TAGI_OK;
+    for (int d = 0; d < MAX_DEVICES; d++) {
+        if (g_ws[d].ptr == nullptr) continue;
+        TAGI_TRY(hipSetDevice(d));
+        TAGI_TRY(hipDeviceSynchronize());
+        TAGI_TRY(hipFree(g_ws[d].ptr));
+        g_ws[d] = Workspace();
+    }
+    TAGI_TRY(hipSetDevice(cur));
+    return TAGI_OK;
+}
+
+int tagi_hip_tune(const char *key, int value) {
+    if (key == nullptr) return TAGI_ERR_INVALID_ARG;
+    if (!strcmp(key, "linear.fwd.splits")) g_tune.fwd_splits = value;
+    else if (!strcmp(key, "linear.dz.splits")) g_tune.dz_splits = value;
+    else if (!strcmp(key, "linear.dw.splits")) g_tune.dw_splits = value;
+    else if (!strcmp(key, "linear.gemv_max_batch")) g_tune.gemv_max_batch = value;
+    else if (!strcmp(key, "linear.tile")) g_tune.tile = value;
+    else if (!strcmp(key, "conv2d.dw.splits")) g_tune.conv_dw_splits = value;
+    else return TAGI_ERR_INVALID_ARG;
+    return TAGI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Linear
+// ---------------------------------------------------------------------------
+
+int tagi_linear_fwd(const float *mu_w, const float *var_w, const float *mu_b, const float *var_b,
+                    const float *mu_a, const float *var_a, int K, int N, int B, int bias,
+                    float *mu_z, float *var_z, void *stream_) {
+    if (!mu_w || !var_w || !mu_a || !var_a || !mu_z || !var_z) return TAGI_ERR_INVALID_ARG;
+    if (K <= 0 || N <= 0 || B <= 0) return TAGI_ERR_INVALID_ARG;
+    if (bias && (!mu_b || !var_b)) return TAGI_ERR_INVALID_ARG;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const float *e0 = bias ? mu_b : nullptr, *e1 = bias ? var_b : nullptr;
+    const bool vec = (K % 4 == 0) && aligned16(mu_w) && aligned16(var_w) && aligned16(mu_a) &&
+                     aligned16(var_a);
+
+    if (B <= gemv_max_batch() && vec) {
+        const int blocks = ceil_div(N, gemv_fwd_rows_per_block());
+        int splits = g_tune.fwd_splits > 0 ? g_tune.fwd_splits : ceil_div(4 * NUM_CU, blocks);
+        const int max_splits = ceil_div(K, 4 * gemv_fwd_k_step());
+        if (splits > max_splits) splits = max_splits;
+        if (splits < 1) splits = 1;
+        int per = ceil_div(ceil_div(K, splits), gemv_fwd_k_step()) * gemv_fwd_k_step();
+        splits = ceil_div(K, per);
+        float *ws = nullptr;
+        const size_t part = (size_t)splits * B * N;
+        int rc = workspace_get(2 * part * sizeof(float), &ws);
+        if (rc != TAGI_OK) return rc;
+        TAGI_TRY(launch_gemv_fwd(mu_w, var_w, mu_a, var_a, K, N, B, splits, ws, ws + part, stream));
+        TAGI_TRY(launch_reduce_splits(EPI_BIAS, ws, ws + part, splits, B, N, e0, e1, mu_z, var_z, N,
+                                      stream));
+        return TAGI_OK;
+    }
+
+    GemmParams p = {};
+    p.x0 = mu_a; p.x1 = var_a; p.y0 = mu_w; p.y1 = var_w;
+    p.M = B; p.N = N; p.R = K; p.ldx = K; p.ldy = K;
+    p.out0 = mu_z; p.out1 = var_z; p.ldo = N;
+    p.e0 = e0; p.e1 = e1;
+    return run_gemm(GEMM_FWD, p, vec, g_tune.fwd_splits, stream);
+}
+
+int tagi_linear_bwd_dz(const float *mu_w, const float *jcb, const float *delta_mu,
+                       const float *delta_var, int K, int N, int B, float *delta_mu_z,
+                       float *delta_var_z, void *stream_) {
+    if (!mu_w || !jcb || !delta_mu || !delta_var || !delta_mu_z || !delta_var_z)
+        return TAGI_ERR_INVALID_ARG;
+    if (K <= 0 || N <= 0 || B <= 0) return TAGI_ERR_INVALID_ARG;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const bool vec = (K % 4 == 0) && (N % 4 == 0) && aligned16(mu_w) && aligned16(delta_mu) &&
+                     aligned16(delta_var);
+
+    if (B <= gemv_max_batch() && vec) {
+        const int blocks = ceil_div(K, gemv_dz_cols_per_block());
+        int splits = g_tune.dz_splits > 0 ? g_tune.dz_splits : ceil_div(4 * NUM_CU, blocks);
+        const int max_splits = ceil_div(N, 4 * gemv_dz_n_step());
+        if (splits > max_splits) splits = max_splits;
+        if (splits < 1) splits = 1;
+        int per = ceil_div(ceil_div(N, splits), gemv_dz_n_step()) * gemv_dz_n_step();
+        splits = ceil_div(N, per);
+        float *ws = nullptr;
+        const size_t part = (size_t)splits * B * K;
+        int rc = workspace_get(2 * part * sizeof(float), &ws);
+        if (rc != TAGI_OK) return rc;
+        TAGI_TRY(launch_gemv_dz(mu_w, delta_mu, delta_var, K, N, B, splits, ws, ws + part, stream));
+        TAGI_TRY(launch_reduce_splits(EPI_SCALE, ws, ws + part, splits, B, K, jcb, nullptr,
+                                      delta_mu_z, delta_var_z, K, stream));
+        return TAGI_OK;
+    }
+
+    GemmParams p = {};
+    p.x0 = delta_mu; p.x1 = delta_var; p.y0 = mu_w; p.y1 = nullptr;
+    p.M = B; p.N = K; p.R = N; p.ldx = N; p.ldy = K;
+    p.out0 = delta_mu_z; p.out1 = delta_var_z; p.ldo = K;
+    p.e0 = jcb; p.e1 = nullptr;
+    return run_gemm(GEMM_DZ, p, vec, g_tune.dz_splits, stream);
+}
+
+int tagi_linear_bwd_dw(const float *var_w, const float *mu_a, const float *delta_mu,
+                       const float *delta_var, int K, int N, int B, float *delta_mu_w,
+                       float *delta_var_w, void *stream_) {
+    if (!var_w || !mu_a || !delta_mu || !delta_var || !delta_mu_w || !delta_var_w)
+        return TAGI_ERR_INVALID_ARG;
+    if (K <= 0 || N <= 0 || B <= 0) return TAGI_ERR_INVALID_ARG;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const bool k_vec = (K % 4 == 0) && aligned16(mu_a) && aligned16(var_w) &&
+                       aligned16(delta_mu_w) && aligned16(delta_var_w);
+
+    if (B <= gemv_max_batch() && k_vec) {
+        TAGI_TRY(launch_gemv_dw(var_w, mu_a, delta_mu, delta_var, K, N, B, delta_mu_w, delta_var_w,
+                                stream));
+        return TAGI_OK;
+    }
+
+    const bool vec = k_vec && (N % 4 == 0) && aligned16(delta_mu) && aligned16(delta_var);
+    GemmParams p = {};
+    p.x0 = delta_mu; p.x1 = delta_var; p.y0 = mu_a; p.y1 = nullptr;
+    p.M = N; p.N = K; p.R = B; p.ldx = N; p.ldy = K;
+    p.out0 = delta_mu_w; p.out1 = delta_var_w; p.ldo = K;
+    p.e0 = var_w; p.e1 = nullptr;
+    return run_gemm(GEMM_DW, p, vec, g_tune.dw_splits, stream);
+}
+
+int tagi_linear_bwd_db(const float *var_b, const float *delta_mu, const float *delta_var, int N,
+                       int B, float *delta_mu_b, float *delta_var_b, void *stream_) {
+    if (!var_b || !delta_mu || !delta_var || !delta_mu_b || !delta_var_b)
+        return TAGI_ERR_INVALID_ARG;
+    if (N <= 0 || B <= 0) return TAGI_ERR_INVALID_ARG;
+    TAGI_TRY(launch_bias_delta(var_b, delta_mu, delta_var, N, B, delta_mu_b, delta_var_b,
+                               static_cast<hipStream_t>(stream_)));
+    return TAGI_OK;
+}
+
+int tagi_linear_bwd(const float *mu_w, const float *var_w, const float *var_b, const float *mu_a,
+                    const float *jcb, const float *delta_mu, const float *delta_var, int K, int N,
+                    int B, int bias, int state_update, int param_update, float *delta_mu_z,
+                    float *delta_var_z, float *delta_mu_w, float *delta_var_w, float *delta_mu_b,
+                    float *delta_var_b, void *stream) {
+    int rc = TAGI_OK;
+    if (state_update) {
+        rc = tagi_linear_bwd_dz(mu_w, jcb, delta_mu, delta_var, K, N, B, delta_mu_z, delta_var_z,
+                                stream);
+        if (rc != TAGI_OK) return rc;
+    }
+    if (param_update) {
+        rc = tagi_linear_bwd_dw(var_w, mu_a, delta_mu, delta_var, K, N, B, delta_mu_w, delta_var_w,
+                                stream);
+        if (rc != TAGI_OK) return rc;
+        if (bias) {
+            rc = tagi_linear_bwd_db(var_b, delta_mu, delta_var, N, B, delta_mu_b, delta_var_b,
+                                    stream);
+        }
+    }
+    return rc;
+}
+
+// ---------------------------------------------------------------------------
+// Conv2d
+// ---------------------------------------------------------------------------
+
+int tagi_conv2d_out_size(int kernel, int stride, int wi, int hi, int pad, int pad_type, int *wo,
+                         int *ho) {
+    if (!wo || !ho) return TAGI_ERR_INVALID_ARG;
+    return conv2d_out_size(kernel, stride, wi, hi, pad, pad_type, wo, ho) == 0
+               ? TAGI_OK
+               : TAGI_ERR_INVALID_ARG;
+}
+
+int tagi_conv2d_build_idx(int kernel, int stride, int wi, int hi, int pad, int pad_type,
+                          int param_pad_idx, int *Fmwa_2, int *FCzwa_1, int *Szz_ud, int *w,
+                          int *h) {
+    if (!Fmwa_2 || !FCzwa_1 || !Szz_ud || !w || !h) return TAGI_ERR_INVALID_ARG;
+    return conv2d_build_idx(kernel, stride, wi, hi, pad, pad_type, param_pad_idx, Fmwa_2, FCzwa_1,
+                            Szz_ud, w, h) == 0
+               ? TAGI_OK
+               : TAGI_ERR_INVALID_ARG;
+}
+
+int tagi_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b, const float *var_b,
+                    const float *mu_a, const float *var_a, const int *aidx, int woho, int fo,
+                    int wihi, int fi, int ki, int B, int bias, float *mu_z, float *var_z,
+                    void *stream_) {
+    if (!mu_w || !var_w || !mu_a || !var_a || !aidx || !mu_z || !var_z)
+        return TAGI_ERR_INVALID_ARG;
+    if (woho <= 0 || fo <= 0 || wihi <= 0 || fi <= 0 || ki <= 0 || B <= 0)
+        return TAGI_ERR_INVALID_ARG;
+    if (bias && (!mu_b || !var_b)) return TAGI_ERR_INVALID_ARG;
+    TAGI_TRY(launch_conv2d_fwd(mu_w, var_w, mu_b, var_b, mu_a, var_a, aidx, woho, fo, wihi, fi, ki,
+                               B, bias, mu_z, var_z, static_cast<hipStream_t>(stream_)));
+    return TAGI_OK;
+}
+
+int tagi_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *delta_mu_out,
+                       const float *delta_var_out, const int *zw_idx, const int *zud_idx, int woho,
+                       int fo, int wihi, int fi, int ki, int nr, int B, float *delta_mu,
+                       float *delta_var, void *stream_) {
+    if (!mu_w || !jcb || !delta_mu_out || !delta_var_out || !zw_idx || !zud_idx || !delta_mu ||
+        !delta_var)
+        return TAGI_ERR_INVALID_ARG;
+    if (woho <= 0 || fo <= 0 || wihi <= 0 || fi <= 0 || ki <= 0 || nr <= 0 || B <= 0)
+        return TAGI_ERR_INVALID_ARG;
+    float *ws = nullptr;
+    int rc = workspace_get((size_t)ki * ki * wihi * sizeof(int), &ws);
+    if (rc != TAGI_OK) return rc;
+    TAGI_TRY(launch_conv2d_bwd_dz(mu_w, jcb, delta_mu_out, delta_var_out, zw_idx, zud_idx, woho,
+                                  fo, wihi, fi, ki, nr, B, reinterpret_cast<int *>(ws), delta_mu,
+                                  delta_var, static_cast<hipStream_t>(stream_)));
+    return TAGI_OK;
+}
+
+int tagi_conv2d_bwd_dw(const float *var_w, const float *var_b, const float *mu_a,
+                       const float *delta_mu_out, const float *delta_var_out, const int *aidx,
+                       int B, int fo, int woho, int wihi, int fi, int ki, int bias,
+                       float *delta_mu_w, float *delta_var_w, float *delta_mu_b,
+                       float *delta_var_b, void *stream_) {
+    if (!var_w || !mu_a || !delta_mu_out || !delta_var_out || !aidx || !delta_mu_w ||
+        !delta_var_w)
+        return TAGI_ERR_INVALID_ARG;
+    if (woho <= 0 || fo <= 0 || wihi <= 0 || fi <= 0 || ki <= 0 || B <= 0)
+        return TAGI_ERR_INVALID_ARG;
+    if (bias && (!var_b || !delta_mu_b || !delta_var_b)) return TAGI_ERR_INVALID_ARG;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+
+    // The reduction runs over all B*woho output positions while the result is
+    // only fo x (ki*ki*fi): slice the reduction to fill the GPU.
+    const int red = B * woho;
+    const int out_tiles = ceil_div(fo, 64) * ceil_div(ki * ki * fi, 64);
+    int splits = g_tune.conv_dw_splits > 0 ? g_tune.conv_dw_splits
+                                           : ceil_div(4 * NUM_CU, out_tiles);
+    const int max_splits = ceil_div(red, 256);
+    if (splits > max_splits) splits = max_splits;
+    if (splits < 1) splits = 1;
+    float *ws = nullptr;
+    const size_t part = (size_t)splits * fo * ki * ki * fi;
+    const int chunks = 64;  // slices of the (b, o) range in the bias reduction
+    int rc = workspace_get((2 * part + 2 * (size_t)chunks * fo) * sizeof(float), &ws);
+    if (rc != TAGI_OK) return rc;
+    TAGI_TRY(launch_conv2d_bwd_dw(var_w, mu_a, delta_mu_out, delta_var_out, aidx, B, fo, woho, wihi,
+                                  fi, ki, splits, ws, ws + part, delta_mu_w, delta_var_w, stream));
+    if (bias) {
+        TAGI_TRY(launch_conv2d_bwd_db(var_b, delta_mu_out, delta_var_out, B, fo, woho, chunks,
+                                      ws + 2 * part, delta_mu_b, delta_var_b, stream));
+    }
+    return TAGI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Layer glue, update, output updater, ReLU
+// ---------------------------------------------------------------------------
+
+int tagi_store_states(const float *mu_a, const float *jcb, size_t n_in, float *bwd_mu_a,
+                      float *bwd_jcb, float *out_jcb, size_t n_out, void *stream_) {
+    if (n_in > 0 && (!mu_a || !jcb || !bwd_mu_a || !bwd_jcb)) return TAGI_ERR_INVALID_ARG;
+    if (n_out > 0 && !out_jcb) return TAGI_ERR_INVALID_ARG;
+    TAGI_TRY(launch_store_states(mu_a, jcb, n_in, bwd_mu_a, bwd_jcb, out_jcb, n_out,
+                                 static_cast<hipStream_t>(stream_)));
+    return TAGI_OK;
+}
+
+int tagi_param_update(const float *delta_mu, const float *delta_var, float cap_factor, size_t n,
+                      float *mu, float *var, int *neg_var_count, void *stream_) {
+    if (n > 0 && (!delta_mu || !delta_var || !mu || !var)) return TAGI_ERR_INVALID_ARG;
+    if (!(cap_factor > 0.0f)) return TAGI_ERR_INVALID_ARG;
+    TAGI_TRY(launch_param_update(delta_mu, delta_var, cap_factor, n, mu, var, neg_var_count,
+                                 static_cast<hipStream_t>(stream_)));
+    return TAGI_OK;
+}
+
+float tagi_cap_factor(int batch_size, float prev) {
+    if (batch_size == 1) return 0.1f;
+    if (batch_size > 1 && batch_size < 256) return 2.0f;
+    if (batch_size >= 256) return 3.0f;
+    return prev;
+}
+
+int tagi_out_update_dense(const float *mu_a, const float *var_a, const float *jcb,
+                          const float *obs, const float *var_obs, int n, float *delta_mu,
+                          float *delta_var, void *stream_) {
+    if (n < 0) return TAGI_ERR_INVALID_ARG;
+    if (n > 0 && (!mu_a || !var_a || !jcb || !obs || !var_obs || !delta_mu || !delta_var))
+        return TAGI_ERR_INVALID_ARG;
+    TAGI_TRY(launch_out_update_dense(mu_a, var_a, jcb, obs, var_obs, n, delta_mu, delta_var,
+                                     static_cast<hipStream_t>(stream_)));
+    return TAGI_OK;
+}
+
+int tagi_out_update_indexed(const float *mu_a, const float *var_a, const float *jcb,
+                            const float *obs, const float *var_obs, const int *selected_idx,
+                            int n_obs, int n_enc, int n, float *delta_mu, float *delta_var,
+                            void *stream_) {
+    if (n < 0 || n_obs <= 0 || n_enc <= 0) return TAGI_ERR_INVALID_ARG;
+    if (n > 0 && (!mu_a || !var_a || !jcb || !obs || !var_obs || !selected_idx || !delta_mu ||
+                  !delta_var))
+        return TAGI_ERR_INVALID_ARG;
+    TAGI_TRY(launch_out_update_indexed(mu_a, var_a, jcb, obs, var_obs, selected_idx, n_obs, n_enc,
+                                       n, delta_mu, delta_var, static_cast<hipStream_t>(stream_)));
+    return TAGI_OK;
+}
+
+int tagi_relu_fwd(const float *mu_z, const float *var_z, size_t n, float *mu_a, float *jcb,
+                  float *var_a, void *stream_) {
+    if (n > 0 && (!mu_z || !var_z || !mu_a || !jcb || !var_a)) return TAGI_ERR_INVALID_ARG;
+    TAGI_TRY(launch_relu(mu_z, var_z, n, mu_a, jcb, var_a, static_cast<hipStream_t>(stream_)));
+    return TAGI_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,181 @@
+// Small bandwidth-bound kernels around the TAGI layers: bias innovation, state
+// bookkeeping, capped parameter step, output innovation and ReLU. gfx950.
+#include "tagi_internal.h"
+
+namespace tagi {
+namespace {
+
+constexpr int TPB = 256;
+
+inline unsigned blocks_for(size_t n, int per_block) {
+    return (unsigned)((n + per_block - 1) / per_block);
+}
+
+// delta_b[n] = var_b[n] * sum_b delta[b][n]. Block = 64 columns x 4 batch
+// slices; consecutive lanes read consecutive columns, the 4 slices meet in LDS.
+__global__ __launch_bounds__(TPB) void bias_delta_kernel(
+    const float *__restrict__ var_b, const float *__restrict__ dmu,
+    const float *__restrict__ dvar, int N, int B, float *__restrict__ dmu_b,
+    float *__restrict__ dvar_b) {
+    __shared__ float s0[4][64], s1[4][64];
+    const int c = threadIdx.x & 63, slice = threadIdx.x >> 6;
+    const int n = blockIdx.x * 64 + c;
+    float a0 = 0.f, a1 = 0.f;
+    if (n < N) {
+        for (int b = slice; b < B; b += 4) {
+            a0 += dmu[(size_t)b * N + n];
+            a1 += dvar[(size_t)b * N + n];
+        }
+    }
+    s0[slice][c] = a0;
+    s1[slice][c] = a1;
+    __syncthreads();
+    if (slice == 0 && n < N) {
+        const float m = (s0[0][c] + s0[1][c]) + (s0[2][c] + s0[3][c]);
+        const float v = (s1[0][c] + s1[1][c]) + (s1[2][c] + s1[3][c]);
+        const float vb = var_b[n];
+        dmu_b[n] = m * vb;
+        dvar_b[n] = v * vb * vb;
+    }
+}
+
+__global__ __launch_bounds__(TPB) void store_states_kernel(
+    const float *__restrict__ mu_a, const float *__restrict__ jcb, size_t n_in,
+    float *__restrict__ bwd_mu_a, float *__restrict__ bwd_jcb, float *__restrict__ out_jcb,
+    size_t n_out) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i < n_in) {
+        bwd_mu_a[i] = mu_a[i];
+        bwd_jcb[i] = jcb[i];
+    }
+    if (i < n_out) out_jcb[i] = 1.0f;
+}
+
+// p += sign(d) * min(|d|, sqrt(var)/cap); var <= 0 -> 1e-5 and counted. One
+// atomic per wave: the clamped lanes are counted with a ballot.
+__global__ __launch_bounds__(TPB) void param_update_kernel(
+    const float *__restrict__ dmu, const float *__restrict__ dvar, float cap, size_t n,
+    float *__restrict__ mu, float *__restrict__ var, int *__restrict__ neg_count) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    bool clamped = false;
+    if (i < n) {
+        const float dm = dmu[i], dv = dvar[i], v = var[i];
+        const float sm = (float)((dm > 0.f) - (dm < 0.f));
+        const float sv = (float)((dv > 0.f) - (dv < 0.f));
+        const float bar = sqrtf(v) / cap;
+        mu[i] += sm * fminf(fabsf(dm), bar);
+        float nv = v + sv * fminf(fabsf(dv), bar);
+        if (nv <= 0.0f) {
+            nv = 1E-5f;
+            clamped = true;
+        }
+        var[i] = nv;
+    }
+    if (neg_count != nullptr) {
+        const unsigned long long mask = __ballot(clamped);
+        if (mask != 0ull && (threadIdx.x & 63) == 0) atomicAdd(neg_count, __popcll(mask));
+    }
+}
+
+__global__ __launch_bounds__(TPB) void out_update_dense_kernel(
+    const float *__restrict__ mu_a, const float *__restrict__ var_a,
+    const float *__restrict__ jcb, const float *__restrict__ obs,
+    const float *__restrict__ var_obs, int n, float *__restrict__ dmu,
+    float *__restrict__ dvar) {
+    const int col = blockIdx.x * TPB + threadIdx.x;
+    if (col >= n) return;
+    const float t = jcb[col] / (var_a[col] + var_obs[col]);
+    if (isinf(t) || isnan(t) || isnan(obs[col])) {
+        dmu[col] = 0.f;
+        dvar[col] = 0.f;
+    } else {
+        dmu[col] = t * (obs[col] - mu_a[col]);
+        dvar[col] = -t * jcb[col];
+    }
+}
+
+__global__ __launch_bounds__(TPB) void out_update_indexed_kernel(
+    const float *__restrict__ mu_a, const float *__restrict__ var_a,
+    const float *__restrict__ jcb, const float *__restrict__ obs,
+    const float *__restrict__ var_obs, const int *__restrict__ sel, int n_obs, int n_enc, int n,
+    float *__restrict__ dmu, float *__restrict__ dvar) {
+    const int col = blockIdx.x * TPB + threadIdx.x;
+    if (col >= n) return;
+    const int idx = sel[col] + (col / n_enc) * n_obs - 1;  // sel is 1-based
+    const float t = jcb[idx] / (var_a[idx] + var_obs[col]);
+    if (isinf(t) || isnan(t)) {
+        dmu[idx] = 0.f;
+        dvar[idx] = 0.f;
+    } else {
+        dmu[idx] = t * (obs[col] - mu_a[idx]);
+        dvar[idx] = -t * jcb[idx];
+    }
+}
+
+// No __restrict__: the call may run in place (mu_a == mu_z, var_a == var_z).
+__global__ __launch_bounds__(TPB) void relu_kernel(const float *mu_z, const float *var_z,
+                                                   size_t n, float *mu_a, float *jcb,
+                                                   float *var_a) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n) return;
+    const float m = fmaxf(mu_z[i], 0.f);
+    const float v = var_z[i];
+    mu_a[i] = m;
+    jcb[i] = (m == 0.f) ? 0.f : 1.f;
+    var_a[i] = (m == 0.f) ? 0.f : v;
+}
+
+}  // namespace
+
+hipError_t launch_bias_delta(const float *var_b, const float *dmu, const float *dvar, int N,
+                             int B, float *dmu_b, float *dvar_b, hipStream_t stream) {
+    hipLaunchKernelGGL(bias_delta_kernel, dim3(blocks_for(N, 64)), dim3(TPB), 0, stream, var_b,
+                       dmu, dvar, N, B, dmu_b, dvar_b);
+    return hipGetLastError();
+}
+
+hipError_t launch_store_states(const float *mu_a, const float *jcb, size_t n_in, float *bwd_mu_a,
+                               float *bwd_jcb, float *out_jcb, size_t n_out, hipStream_t stream) {
+    const size_t n = n_in > n_out ? n_in : n_out;
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(store_states_kernel, dim3(blocks_for(n, TPB)), dim3(TPB), 0, stream, mu_a,
+                       jcb, n_in, bwd_mu_a, bwd_jcb, out_jcb, n_out);
+    return hipGetLastError();
+}
+
+hipError_t launch_param_update(const float *dmu, const float *dvar, float cap, size_t n, float *mu,
+                               float *var, int *neg_count, hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(param_update_kernel, dim3(blocks_for(n, TPB)), dim3(TPB), 0, stream, dmu,
+                       dvar, cap, n, mu, var, neg_count);
+    return hipGetLastError();
+}
+
+hipError_t launch_out_update_dense(const float *mu_a, const float *var_a, const float *jcb,
+                                   const float *obs, const float *var_obs, int n, float *dmu,
+                                   float *dvar, hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(out_update_dense_kernel, dim3(blocks_for(n, TPB)), dim3(TPB), 0, stream,
+                       mu_a, var_a, jcb, obs, var_obs, n, dmu, dvar);
+    return hipGetLastError();
+}
+
+hipError_t launch_out_update_indexed(const float *mu_a, const float *var_a, const float *jcb,
+                                     const float *obs, const float *var_obs, const int *sel,
+                                     int n_obs, int n_enc, int n, float *dmu, float *dvar,
+                                     hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(out_update_indexed_kernel, dim3(blocks_for(n, TPB)), dim3(TPB), 0, stream,
+                       mu_a, var_a, jcb, obs, var_obs, sel, n_obs, n_enc, n, dmu, dvar);
+    return hipGetLastError();
+}
+
+hipError_t launch_relu(const float *mu_z, const float *var_z, size_t n, float *mu_a, float *jcb,
+                       float *var_a, hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(relu_kernel, dim3(blocks_for(n, TPB)), dim3(TPB), 0, stream, mu_z, var_z, n, mu_a,
+                       jcb, var_a);
+    return hipGetLastError();
+}
+
+}  // namespace tagi

@@ -1,0 +1,180 @@
+// Tiled fp32-MFMA kernels for the three TAGI Linear contractions, gfx950: the
+// problem definitions that plug the Linear operands into tagi_mfma_tile.h.
+//
+//   FWD: D[b][n]  = sum_k act[b][k] * w[n][k]; the variance is one GEMM over the
+//        concatenated reduction [var_w | mu_w^2] x [var_a + mu_a^2 ; var_a] that
+//        shares the LDS tiles of the mean GEMM (squares and sums are formed in
+//        registers from the staged mu/var tiles). Both operands k-contiguous.
+//   DZ : D[b][k'] = sum_n delta[b][n] * w[n][k'] (variance with w^2); delta is
+//        k-contiguous, w is staged [n][k'] as it lies in memory.
+//   DW : D[n][k'] = sum_b delta[b][n] * act[b][k'] (variance with act^2); both
+//        operands are staged [b][...] as they lie in memory.
+#include "tagi_internal.h"
+#include "tagi_mfma_tile.h"
+
+namespace tagi {
+namespace {
+
+// Four elements of a row-major matrix `base` (leading dimension ld): along the
+// reduction (KC) at (row, r..r+3), or along the rows at (row..row+3, r) where the
+// reduction index is the slow one. Zero outside [0,rows) x [.., r_end).
+template <bool KC, bool VEC>
+__device__ __forceinline__ float4 load4(const float *__restrict__ base, int ld, int row, int rows,
+                                        int r, int r_end) {
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (VEC) {
+        if (row < rows && r < r_end) {
+            const float *q = KC ? base + (size_t)row * ld + r : base + (size_t)r * ld + row;
+            v = *reinterpret_cast<const float4 *>(q);
+        }
+    } else {
+        float c[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (KC) {
+                if (row < rows && r + j < r_end) c[j] = base[(size_t)row * ld + r + j];
+            } else {
+                if (r < r_end && row + j < rows) c[j] = base[(size_t)r * ld + row + j];
+            }
+        }
+        v = make_float4(c[0], c[1], c[2], c[3]);
+    }
+    return v;
+}
+
+template <int MODE, bool VEC>
+struct LinearProblem {
+    using Params = GemmParams;
+    static constexpr bool XK = (MODE != GEMM_DW);
+    static constexpr bool YK = (MODE == GEMM_FWD);
+    static constexpr int NX = 2;
+    static constexpr int NY = (MODE == GEMM_FWD) ? 2 : 1;
+    static constexpr int FLAVOR = (MODE == GEMM_FWD) ? FLAVOR_FWD_ACT_ROWS : FLAVOR_DELTA_ROWS;
+
+    __device__ static __forceinline__ float4 load_x(const Params &p, int arr, int m, int r,
+                                                    int r_end) {
+        return load4<XK, VEC>(arr ? p.x1 : p.x0, p.ldx, m, p.M, r, r_end);
+    }
+    __device__ static __forceinline__ float4 load_y(const Params &p, int arr, int n, int r,
+                                                    int r_end) {
+        return load4<YK, VEC>(arr ? p.y1 : p.y0, p.ldy, n, p.N, r, r_end);
+    }
+    __device__ static __forceinline__ void store(const Params &p, int m, int n, float a0,
+                                                 float a1) {
+        const size_t at = (size_t)m * p.ldo + n;
+        if (MODE == GEMM_FWD) {
+            if (p.e0 != nullptr) {
+                a0 += p.e0[n];
+                a1 += p.e1[n];
+            }
+        } else {
+            const float e = p.e0[at];
+            a0 *= e;
+            a1 *= e * e;
+        }
+        p.out0[at] = a0;
+        p.out1[at] = a1;
+    }
+};
+
+template <int EPI, bool VEC>
+__global__ __launch_bounds__(256) void reduce_splits_kernel(const float *__restrict__ ws0,
+                                                            const float *__restrict__ ws1,
+                                                            int splits, int M, int N,
+                                                            const float *__restrict__ e0,
+                                                            const float *__restrict__ e1,
+                                                            float *__restrict__ out0,
+                                                            float *__restrict__ out1, int ldo) {
+    const size_t total = (size_t)M * N;
+    constexpr int W = VEC ? 4 : 1;
+    const size_t idx = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * W;
+    if (idx >= total) return;
+    float s0[W], s1[W];
+#pragma unroll
+    for (int c = 0; c < W; c++) s0[c] = s1[c] = 0.f;
+    for (int s = 0; s < splits; s++) {
+        if constexpr (VEC) {
+            const float4 a = *reinterpret_cast<const float4 *>(ws0 + s * total + idx);
+            const float4 b = *reinterpret_cast<const float4 *>(ws1 + s * total + idx);
+            s0[0] += a.x; s0[1] += a.y; s0[2] += a.z; s0[3] += a.w;
+            s1[0] += b.x; s1[1] += b.y; s1[2] += b.z; s1[3] += b.w;
+        } else {
+            s0[0] += ws0[s * total + idx];
+            s1[0] += ws1[s * total + idx];
+        }
+    }
+    const int row = (int)(idx / N), col = (int)(idx % N);
+    const size_t at = (size_t)row * ldo + col;
+#pragma unroll
+    for (int c = 0; c < W; c++) {
+        if (EPI == EPI_BIAS) {
+            if (e0 != nullptr) {
+                s0[c] += e0[col + c];
+                s1[c] += e1[col + c];
+            }
+        } else {
+            const float e = e0[at + c];
+            s0[c] *= e;
+            s1[c] *= e * e;
+        }
+    }
+    if constexpr (VEC) {
+        *reinterpret_cast<float4 *>(out0 + at) = make_float4(s0[0], s0[1], s0[2], s0[3]);
+        *reinterpret_cast<float4 *>(out1 + at) = make_float4(s1[0], s1[1], s1[2], s1[3]);
+    } else {
+        out0[at] = s0[0];
+        out1[at] = s1[0];
+    }
+}
+
+template <int MODE>
+hipError_t launch_mode(int tile, bool vec, const GemmParams &p, hipStream_t stream) {
+    if (vec) return launch_tiles<LinearProblem<MODE, true>>(tile, p, stream);
+    return launch_tiles<LinearProblem<MODE, false>>(tile, p, stream);
+}
+
+}  // namespace
+
+int gemm_tile_rows(int tile) { return tile_rows(tile); }
+int gemm_tile_cols(int tile) { return tile_cols(tile); }
+int gemm_tile_count() { return TILE_COUNT; }
+int gemm_k_tile() { return KT; }
+
+hipError_t launch_gemm(GemmMode mode, int tile, bool vec, const GemmParams &p,
+                       hipStream_t stream) {
+    switch (mode) {
+        case GEMM_FWD: return launch_mode<GEMM_FWD>(tile, vec, p, stream);
+        case GEMM_DZ: return launch_mode<GEMM_DZ>(tile, vec, p, stream);
+        case GEMM_DW: return launch_mode<GEMM_DW>(tile, vec, p, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+hipError_t launch_reduce_splits(Epilogue epi, const float *ws0, const float *ws1, int splits,
+                                int M, int N, const float *e0, const float *e1, float *out0,
+                                float *out1, int ldo, hipStream_t stream) {
+    const size_t total = (size_t)M * N;
+    auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
+    const bool vec = (N % 4 == 0) && (ldo % 4 == 0) && al(ws0) && al(ws1) && al(out0) &&
+                     al(out1) && (epi == EPI_BIAS || al(e0));
+    const size_t items = vec ? total / 4 : total;
+    dim3 grid((unsigned)((items + 255) / 256)), block(256);
+    if (epi == EPI_BIAS) {
+        if (vec)
+            hipLaunchKernelGGL((reduce_splits_kernel<EPI_BIAS, true>), grid, block, 0, stream, ws0,
+                               ws1, splits, M, N, e0, e1, out0, out1, ldo);
+        else
+            hipLaunchKernelGGL((reduce_splits_kernel<EPI_BIAS, false>), grid, block, 0, stream,
+                               ws0, ws1, splits, M, N, e0, e1, out0, out1, ldo);
+    } else {
+        if (vec)
+            hipLaunchKernelGGL((reduce_splits_kernel<EPI_SCALE, true>), grid, block, 0, stream,
+                               ws0, ws1, splits, M, N, e0, e1, out0, out1, ldo);
+        else
+            hipLaunchKernelGGL((reduce_splits_kernel<EPI_SCALE, false>), grid, block, 0, stream,
+                               ws0, ws1, splits, M, N, e0, e1, out0, out1, ldo);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace tagi

@@ -1,0 +1,109 @@
+// Internal launcher interface between the C ABI (tagi_capi.hip) and the kernel
+// translation units. Not installed; the public surface is include/tagi_hip.h.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+
+namespace tagi {
+
+// Which contraction of the layer a tiled GEMM launch computes.
+//   FWD: D[b][n]  = sum_k  act[b][k] * w[n][k]      (mean; variance with 2 terms)
+//   DZ : D[b][k'] = sum_n  delta[b][n] * w[n][k']   (variance with w^2)
+//   DW : D[n][k'] = sum_b  delta[b][n] * act[b][k'] (variance with act^2)
+enum GemmMode { GEMM_FWD = 0, GEMM_DZ = 1, GEMM_DW = 2 };
+
+// Epilogue applied to the two accumulators (mean-like `0`, variance-like `1`).
+//   EPI_BIAS : out0 = acc0 + e0[col], out1 = acc1 + e1[col]   (e0 == nullptr: none)
+//   EPI_SCALE: out0 = acc0 * e0[row][col], out1 = acc1 * e0[row][col]^2
+enum Epilogue { EPI_BIAS = 0, EPI_SCALE = 1 };
+
+struct GemmParams {
+    const float *x0, *x1;  // row-side operands (FWD: mu_a,var_a; DZ/DW: delta_mu,delta_var)
+    const float *y0, *y1;  // column-side operands (FWD: mu_w,var_w; DZ: mu_w; DW: mu_a)
+    int M, N, R;           // D is M x N, reduction length R
+    int ldx, ldy;          // leading dimensions of the operands as stored
+    float *out0, *out1;    // M x N, leading dimension ldo
+    int ldo;
+    const float *e0, *e1;  // epilogue operands, see Epilogue
+    int splits;            // number of reduction slices (gridDim.y)
+    int r_per_split;       // reduction elements per slice, multiple of the k-tile
+    float *ws0, *ws1;      // [splits][M][N] partial sums when splits > 1
+};
+
+// Tile shapes the tiled kernels are instantiated for (indices 0..count-1).
+int gemm_tile_count();
+int gemm_tile_rows(int tile);
+int gemm_tile_cols(int tile);
+int gemm_k_tile();
+
+// Launches the tiled MFMA kernel. `vec` selects 16-byte global loads (the caller
+// guarantees the alignment rules); partial sums go to ws0/ws1 when splits > 1
+// and the caller then runs reduce_splits.
+hipError_t launch_gemm(GemmMode mode, int tile, bool vec, const GemmParams &p,
+                       hipStream_t stream);
+
+// out = epilogue(sum over splits of ws[s]) for the two accumulators.
+hipError_t launch_reduce_splits(Epilogue epi, const float *ws0, const float *ws1,
+                                int splits, int M, int N, const float *e0,
+                                const float *e1, float *out0, float *out1, int ldo,
+                                hipStream_t stream);
+
+// Skinny-batch (B <= 16) streaming kernels: weights are read once from HBM
+// straight into MFMA operand layout, nothing is staged in LDS.
+hipError_t launch_gemv_fwd(const float *mu_w, const float *var_w, const float *mu_a,
+                           const float *var_a, int K, int N, int B, int splits,
+                           float *ws0, float *ws1, hipStream_t stream);
+hipError_t launch_gemv_dz(const float *mu_w, const float *dmu, const float *dvar, int K,
+                          int N, int B, int splits, float *ws0, float *ws1,
+                          hipStream_t stream);
+hipError_t launch_gemv_dw(const float *var_w, const float *mu_a, const float *dmu,
+                          const float *dvar, int K, int N, int B, float *dmu_w,
+                          float *dvar_w, hipStream_t stream);
+int gemv_fwd_rows_per_block();
+int gemv_fwd_k_step();
+int gemv_dz_cols_per_block();
+int gemv_dz_n_step();
+
+// Elementwise / small kernels
+hipError_t launch_bias_delta(const float *var_b, const float *dmu, const float *dvar, int N,
+                             int B, float *dmu_b, float *dvar_b, hipStream_t stream);
+hipError_t launch_store_states(const float *mu_a, const float *jcb, size_t n_in,
+                               float *bwd_mu_a, float *bwd_jcb, float *out_jcb, size_t n_out,
+                               hipStream_t stream);
+hipError_t launch_param_update(const float *dmu, const float *dvar, float cap, size_t n,
+                               float *mu, float *var, int *neg_count, hipStream_t stream);
+hipError_t launch_out_update_dense(const float *mu_a, const float *var_a, const float *jcb,
+                                   const float *obs, const float *var_obs, int n, float *dmu,
+                                   float *dvar, hipStream_t stream);
+hipError_t launch_out_update_indexed(const float *mu_a, const float *var_a, const float *jcb,
+                                     const float *obs, const float *var_obs, const int *sel,
+                                     int n_obs, int n_enc, int n, float *dmu, float *dvar,
+                                     hipStream_t stream);
+hipError_t launch_relu(const float *mu_z, const float *var_z, size_t n, float *mu_a, float *jcb,
+                       float *var_a, hipStream_t stream);
+
+// Conv2d (implicit GEMM through the index tables)
+hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
+                             const float *var_b, const float *mu_a, const float *var_a,
+                             const int *aidx, int woho, int fo, int wihi, int fi, int ki, int B,
+                             int bias, float *mu_z, float *var_z, hipStream_t stream);
+hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *dmu,
+                                const float *dvar, const int *zw_idx, const int *zud_idx,
+                                int woho, int fo, int wihi, int fi, int ki, int nr, int B,
+                                int *scratch, float *out_dmu, float *out_dvar,
+                                hipStream_t stream);
+hipError_t launch_conv2d_bwd_dw(const float *var_w, const float *mu_a, const float *dmu,
+                                const float *dvar, const int *aidx, int B, int fo, int woho,
+                                int wihi, int fi, int ki, int splits, float *ws0, float *ws1,
+                                float *dmu_w, float *dvar_w, hipStream_t stream);
+hipError_t launch_conv2d_bwd_db(const float *var_b, const float *dmu, const float *dvar, int B,
+                                int fo, int woho, int chunks, float *scratch, float *dmu_b,
+                                float *dvar_b, hipStream_t stream);
+
+// Host-side index tables (tagi_conv_idx.cpp)
+int conv2d_out_size(int kernel, int stride, int wi, int hi, int pad, int pad_type, int *wo,
+                    int *ho);
+int conv2d_build_idx(int kernel, int stride, int wi, int hi, int pad, int pad_type,
+                     int param_pad_idx, int *Fmwa_2, int *FCzwa_1, int *Szz_ud, int *w, int *h);
+
+}  // namespace tagi

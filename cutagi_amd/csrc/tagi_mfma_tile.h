@@ -1,0 +1,289 @@
+// Workgroup-tiled fp32 MFMA core shared by the Linear and Conv2d contractions,
+// gfx950 (v_mfma_f32_32x32x2_f32, 64-lane waves).
+//
+// A workgroup owns a BM x BN tile of an output PAIR (accumulator 0: the
+// mean-like sum, accumulator 1: the variance-like sum), walks its slice of the
+// reduction in k-tiles of KT elements staged through LDS (global -> registers ->
+// LDS, the next k-tile's global loads in flight while the current one is
+// multiplied), and each of its WM x WN waves multiplies (BM/WM) x (BN/WN)
+// sub-tiles.
+//
+// A `Problem` type supplies the operands and the epilogue:
+//   Params                      kernel argument (must hold M, N, R, splits,
+//                               r_per_split, ws0, ws1)
+//   XK / YK                     is the row-side / column-side operand staged with
+//                               its reduction index contiguous ([row][KT+4], read
+//                               back with one 16-byte LDS load), or with the row
+//                               index contiguous ([k][rows+4], read back with four
+//                               4-byte loads)?  Either way lane l of a 32-row
+//                               fragment holds reduction elements kk+4*(l/32)+t,
+//                               t = 0..3, and the t-th of four MFMAs consumes
+//                               component t, so both sides agree on k.
+//   NX / NY                     number of arrays on each side (1 or 2)
+//   FLAVOR                      how the MFMA operands are formed, see Flavor
+//   load_x(p, arr, m, r, r_end) four elements of row-side array `arr`: rows m,
+//                               reduction r..r+3 when XK, rows m..m+3 at reduction
+//                               r otherwise; zero outside the problem
+//   load_y(p, arr, n, r, r_end) the same for the column side
+//   store(p, m, n, acc0, acc1)  final epilogue of one output element
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace tagi {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+// Which products feed the two accumulators (x = row side, y = column side):
+enum Flavor {
+    // acc0 += x0*y0 ; acc1 += (x1 + x0^2)*y1 + x1*y0^2   rows: (mu_a,var_a), cols: (mu_w,var_w)
+    FLAVOR_FWD_ACT_ROWS = 0,
+    // acc0 += x0*y0 ; acc1 += x1*(y1 + y0^2) + x0^2*y1   rows: (mu_w,var_w), cols: (mu_a,var_a)
+    FLAVOR_FWD_W_ROWS = 1,
+    // acc0 += x0*y0 ; acc1 += x1*y0^2                    rows: (delta_mu,delta_var), cols: (v)
+    FLAVOR_DELTA_ROWS = 2,
+    // acc0 += x0*y0 ; acc1 += x0^2*y1                    rows: (w), cols: (delta_mu,delta_var)
+    FLAVOR_DELTA_COLS = 3,
+};
+
+constexpr int KT = 32;  // reduction elements per LDS stage
+
+template <bool KC, int ROWS>
+struct TileGeom {
+    static constexpr int stride = KC ? KT + 4 : ROWS + 4;
+    static constexpr int floats = KC ? ROWS * stride : KT * stride;
+};
+
+__device__ __forceinline__ float comp4(const float4 &v, int t) {
+    return t == 0 ? v.x : t == 1 ? v.y : t == 2 ? v.z : v.w;
+}
+__device__ __forceinline__ float4 sq4(const float4 &a) {
+    return make_float4(a.x * a.x, a.y * a.y, a.z * a.z, a.w * a.w);
+}
+__device__ __forceinline__ float4 add_sq4(const float4 &v, const float4 &m) {
+    return make_float4(v.x + m.x * m.x, v.y + m.y * m.y, v.z + m.z * m.z, v.w + m.w * m.w);
+}
+
+// Position of the f-th float4 of a staged tile: (row, k) of its first element.
+template <bool KC, int ROWS>
+__device__ __forceinline__ void tile_pos(int f, int &row, int &k) {
+    if (KC) {
+        row = f / (KT / 4);
+        k = (f % (KT / 4)) * 4;
+    } else {
+        k = f / (ROWS / 4);
+        row = (f % (ROWS / 4)) * 4;
+    }
+}
+
+template <bool KC, int ROWS>
+__device__ __forceinline__ float4 read_frag(const float *lds, int row, int kk, int lane) {
+    constexpr int S = TileGeom<KC, ROWS>::stride;
+    const int k = kk + 4 * (lane >> 5);
+    if (KC) {
+        return *reinterpret_cast<const float4 *>(lds + (row + (lane & 31)) * S + k);
+    } else {
+        const float *q = lds + k * S + row + (lane & 31);
+        return make_float4(q[0], q[S], q[2 * S], q[3 * S]);
+    }
+}
+
+template <class P, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM *WN * 64) void mfma_tile_kernel(typename P::Params p) {
+    constexpr bool XK = P::XK, YK = P::YK;
+    constexpr int NX = P::NX, NY = P::NY, FL = P::FLAVOR;
+    constexpr int NT = WM * WN * 64;
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int XS = TileGeom<XK, BM>::stride, YS = TileGeom<YK, BN>::stride;
+    constexpr int XF = TileGeom<XK, BM>::floats, YF = TileGeom<YK, BN>::floats;
+    constexpr int LX = BM * KT / 4 / NT, LY = BN * KT / 4 / NT;
+    static_assert(LX >= 1 && LY >= 1, "tile too small for the thread count");
+
+    __shared__ __attribute__((aligned(16))) float lds_x[NX][XF];
+    __shared__ __attribute__((aligned(16))) float lds_y[NY][YF];
+
+    const int tiles_n = (p.N + BN - 1) / BN;
+    const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+    const int split = blockIdx.y;
+    const int r_begin = split * p.r_per_split;
+    const int r_end = min(p.R, r_begin + p.r_per_split);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wrow = (wave / WN) * (TM * 32), wcol = (wave % WN) * (TN * 32);
+
+    floatx16 acc0[TM][TN], acc1[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                acc0[i][j][v] = 0.f;
+                acc1[i][j][v] = 0.f;
+            }
+
+    float4 rx[NX][LX], ry[NY][LY];
+
+    auto fetch = [&](int r0) {
+#pragma unroll
+        for (int a = 0; a < NX; a++)
+#pragma unroll
+            for (int i = 0; i < LX; i++) {
+                int row, k;
+                tile_pos<XK, BM>(tid + i * NT, row, k);
+                rx[a][i] = P::load_x(p, a, m0 + row, r0 + k, r_end);
+            }
+#pragma unroll
+        for (int a = 0; a < NY; a++)
+#pragma unroll
+            for (int i = 0; i < LY; i++) {
+                int row, k;
+                tile_pos<YK, BN>(tid + i * NT, row, k);
+                ry[a][i] = P::load_y(p, a, n0 + row, r0 + k, r_end);
+            }
+    };
+    auto commit = [&]() {
+#pragma unroll
+        for (int a = 0; a < NX; a++)
+#pragma unroll
+            for (int i = 0; i < LX; i++) {
+                int row, k;
+                tile_pos<XK, BM>(tid + i * NT, row, k);
+                *reinterpret_cast<float4 *>(&lds_x[a][XK ? row * XS + k : k * XS + row]) = rx[a][i];
+            }
+#pragma unroll
+        for (int a = 0; a < NY; a++)
+#pragma unroll
+            for (int i = 0; i < LY; i++) {
+                int row, k;
+                tile_pos<YK, BN>(tid + i * NT, row, k);
+                *reinterpret_cast<float4 *>(&lds_y[a][YK ? row * YS + k : k * YS + row]) = ry[a][i];
+            }
+    };
+
+    if (r_begin < r_end) {
+        fetch(r_begin);
+        commit();
+    }
+    __syncthreads();
+
+    for (int r0 = r_begin; r0 < r_end; r0 += KT) {
+        const bool more = r0 + KT < r_end;
+        if (more) fetch(r0 + KT);
+
+#pragma unroll
+        for (int kk = 0; kk < KT; kk += 8) {
+            // MFMA operand fragments: mean (A0,B0), variance (A1,B1) [+ (A2,B2)]
+            float4 A0[TM], A1[TM], A2[TM], B0[TN], B1[TN], B2[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+                const float4 x0 = read_frag<XK, BM>(lds_x[0], wrow + i * 32, kk, lane);
+                float4 x1 = x0;
+                if (NX == 2) x1 = read_frag<XK, BM>(lds_x[NX - 1], wrow + i * 32, kk, lane);
+                A0[i] = x0;
+                if (FL == FLAVOR_FWD_ACT_ROWS) {
+                    A1[i] = add_sq4(x1, x0);
+                    A2[i] = x1;
+                } else if (FL == FLAVOR_FWD_W_ROWS) {
+                    A1[i] = x1;
+                    A2[i] = sq4(x0);
+                } else if (FL == FLAVOR_DELTA_ROWS) {
+                    A1[i] = x1;
+                } else {
+                    A1[i] = sq4(x0);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                const float4 y0 = read_frag<YK, BN>(lds_y[0], wcol + j * 32, kk, lane);
+                float4 y1 = y0;
+                if (NY == 2) y1 = read_frag<YK, BN>(lds_y[NY - 1], wcol + j * 32, kk, lane);
+                B0[j] = y0;
+                if (FL == FLAVOR_FWD_ACT_ROWS) {
+                    B1[j] = y1;
+                    B2[j] = sq4(y0);
+                } else if (FL == FLAVOR_FWD_W_ROWS) {
+                    B1[j] = add_sq4(y1, y0);
+                    B2[j] = y1;
+                } else if (FL == FLAVOR_DELTA_ROWS) {
+                    B1[j] = sq4(y0);
+                } else {
+                    B1[j] = y1;
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) {
+                        acc0[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                            comp4(A0[i], t), comp4(B0[j], t), acc0[i][j], 0, 0, 0);
+                        acc1[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                            comp4(A1[i], t), comp4(B1[j], t), acc1[i][j], 0, 0, 0);
+                        if (FL == FLAVOR_FWD_ACT_ROWS || FL == FLAVOR_FWD_W_ROWS)
+                            acc1[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                                comp4(A2[i], t), comp4(B2[j], t), acc1[i][j], 0, 0, 0);
+                    }
+        }
+        __syncthreads();
+        if (more) {
+            commit();
+            __syncthreads();
+        }
+    }
+
+    // Accumulator register v of lane l is D[8*(v/4) + 4*(l/32) + v%4][l%32]: lanes
+    // run along the output columns.
+    const bool partial = p.splits > 1;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int col = n0 + wcol + j * 32 + (lane & 31);
+            if (col >= p.N) continue;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = m0 + wrow + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                if (row >= p.M) continue;
+                if (partial) {
+                    const size_t at = ((size_t)split * p.M + row) * p.N + col;
+                    p.ws0[at] = acc0[i][j][v];
+                    p.ws1[at] = acc1[i][j][v];
+                } else {
+                    P::store(p, row, col, acc0[i][j][v], acc1[i][j][v]);
+                }
+            }
+        }
+}
+
+// Launch over a (tiles, splits) grid for one of the instantiated tile shapes.
+enum TileShape { TILE_128x128 = 0, TILE_64x128 = 1, TILE_32x128 = 2, TILE_64x64 = 3, TILE_COUNT = 4 };
+
+inline int tile_rows(int t) { return t == TILE_128x128 ? 128 : t == TILE_32x128 ? 32 : 64; }
+inline int tile_cols(int t) { return t == TILE_64x64 ? 64 : 128; }
+
+template <class P>
+hipError_t launch_tiles(int tile, const typename P::Params &p, hipStream_t stream) {
+    const int tiles = ((p.M + tile_rows(tile) - 1) / tile_rows(tile)) *
+                      ((p.N + tile_cols(tile) - 1) / tile_cols(tile));
+    dim3 grid(tiles, p.splits);
+    switch (tile) {
+        case TILE_128x128:
+            hipLaunchKernelGGL((mfma_tile_kernel<P, 128, 128, 2, 4>), grid, dim3(512), 0, stream, p);
+            break;
+        case TILE_64x128:
+            hipLaunchKernelGGL((mfma_tile_kernel<P, 64, 128, 2, 4>), grid, dim3(512), 0, stream, p);
+            break;
+        case TILE_32x128:
+            hipLaunchKernelGGL((mfma_tile_kernel<P, 32, 128, 1, 4>), grid, dim3(256), 0, stream, p);
+            break;
+        case TILE_64x64:
+            hipLaunchKernelGGL((mfma_tile_kernel<P, 64, 64, 2, 2>), grid, dim3(256), 0, stream, p);
+            break;
+        default:
+            return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace tagi

@@ -1,0 +1,198 @@
+/*
+ * tagi_hip.h - C ABI of the MI355X (gfx950) backend for the TAGI Linear and
+ * Conv2d hot path.
+ *
+ * The reference (cuTAGI) has no C ABI: its GPU layers link C++ classes against
+ * CUDA kernels directly. Each entry point below replaces one kernel-dispatch
+ * function of that code and is what a binding of the reference would call in
+ * its place; the reference interface is cited per function (paths relative to
+ * the reference tree).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer to fp32 (or int32 for index tables)
+ *     unless it is marked "host";
+ *   - layouts are the reference's: weights [N][K] row-major (conv: OIHW),
+ *     activations [B][K] (conv: NCHW), outputs [B][N];
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     calls only enqueue work and never synchronise, except where noted;
+ *   - every function returns TAGI_OK (0) or a negative TAGI_ERR_* code, or a
+ *     positive hipError_t when the HIP runtime failed; nothing throws;
+ *     tagi_hip_error_string() describes any of them;
+ *   - the library owns no user buffer. It keeps one grow-only device workspace
+ *     per GPU for split-reduction partial sums (see tagi_hip_workspace_reserve).
+ */
+#ifndef TAGI_HIP_H
+#define TAGI_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TAGI_OK 0
+#define TAGI_ERR_INVALID_ARG (-1) /* null pointer, non-positive size, ... */
+#define TAGI_ERR_UNSUPPORTED (-2) /* shape outside what the kernels cover */
+#define TAGI_ERR_NO_DEVICE (-3)
+
+/* ---- runtime ------------------------------------------------------------ */
+
+/* ABI version of this header (major * 100 + minor). */
+int tagi_hip_version(void);
+/* replaces get_cuda_device_count (src/cuda_utils.cpp) as used by
+ * Sequential::to_device (src/sequential.cpp:32-73). */
+int tagi_hip_device_count(int *count /* host, out */);
+const char *tagi_hip_error_string(int code);
+/* Grow the current device's workspace to at least `bytes` now (synchronises the
+ * device if it has to reallocate). Optional: entry points grow it on demand. */
+int tagi_hip_workspace_reserve(size_t bytes);
+/* Free the workspaces of all devices. */
+int tagi_hip_shutdown(void);
+/* Kernel-selection knobs for experiments ("linear.splitk", "linear.path", ...);
+ * value < 0 restores the built-in heuristic. Unknown keys are an error. */
+int tagi_hip_tune(const char *key /* host */, int value);
+
+/* ---- Linear -------------------------------------------------------------- */
+
+/* mu_z = mu_a * mu_w^T + mu_b ; var_z = (var_a + mu_a^2) * var_w^T
+ *                                        + var_a * (mu_w^2)^T + var_b
+ * replaces linear_forward_cuda (src/linear_layer_cuda.cu:12-73) and the kernels
+ * it dispatches (include/linear_cuda_kernel.cuh:50-573).
+ * mu_b/var_b may be NULL when bias == 0. */
+int tagi_linear_fwd(const float *mu_w, const float *var_w, const float *mu_b,
+                    const float *var_b, const float *mu_a, const float *var_a,
+                    int K, int N, int B, int bias, float *mu_z, float *var_z,
+                    void *stream);
+
+/* delta_mu_z = (delta_mu * mu_w) .* jcb ; delta_var_z = (delta_var * mu_w^2) .* jcb^2
+ * replaces linear_state_backward_cuda (src/linear_layer_cuda.cu:75-121). */
+int tagi_linear_bwd_dz(const float *mu_w, const float *jcb,
+                       const float *delta_mu, const float *delta_var, int K,
+                       int N, int B, float *delta_mu_z, float *delta_var_z,
+                       void *stream);
+
+/* delta_mu_w = (delta_mu^T * mu_a) .* var_w ; delta_var_w = (delta_var^T * mu_a^2) .* var_w^2
+ * replaces linear_weight_backward_cuda (src/linear_layer_cuda.cu:123-168). */
+int tagi_linear_bwd_dw(const float *var_w, const float *mu_a,
+                       const float *delta_mu, const float *delta_var, int K,
+                       int N, int B, float *delta_mu_w, float *delta_var_w,
+                       void *stream);
+
+/* delta_mu_b = colsum(delta_mu) .* var_b ; delta_var_b = colsum(delta_var) .* var_b^2
+ * replaces the linear_bwd_delta_b launch of LinearCuda::backward
+ * (src/linear_layer_cuda.cu:311-321, kernel include/linear_cuda_kernel.cuh:1492-1519). */
+int tagi_linear_bwd_db(const float *var_b, const float *delta_mu,
+                       const float *delta_var, int N, int B, float *delta_mu_b,
+                       float *delta_var_b, void *stream);
+
+/* The whole of LinearCuda::backward (src/linear_layer_cuda.cu:273-323) in one
+ * call: the state update when state_update != 0, the weight update when
+ * param_update != 0 and the bias update when additionally bias != 0. */
+int tagi_linear_bwd(const float *mu_w, const float *var_w, const float *var_b,
+                    const float *mu_a, const float *jcb, const float *delta_mu,
+                    const float *delta_var, int K, int N, int B, int bias,
+                    int state_update, int param_update, float *delta_mu_z,
+                    float *delta_var_z, float *delta_mu_w, float *delta_var_w,
+                    float *delta_mu_b, float *delta_var_b, void *stream);
+
+/* ---- Conv2d -------------------------------------------------------------- */
+
+/* Output size of a convolution; replaces compute_downsample_img_size_v2
+ * (src/conv2d_layer.cpp:581-628). Host only. TAGI_ERR_INVALID_ARG where the
+ * reference throws (stride does not divide). */
+int tagi_conv2d_out_size(int kernel, int stride, int wi, int hi, int pad,
+                         int pad_type, int *wo /* host */, int *ho /* host */);
+
+/* Index tables of a convolution, on the host, int32 and 1-based exactly as
+ * get_conv2d_idx builds them (src/conv2d_layer.cpp:656-719 over
+ * src/indices.cpp): Fmwa_2 [wo*ho][k*k] (padding = -1), FCzwa_1 [w][h]
+ * (padding = param_pad_idx) and Szz_ud [h][w] (padding = -1).
+ * Capacity needed: Fmwa_2 wo*ho*k*k ints, the other two wi*hi*k*k ints each.
+ * All pointers host. Square images only, like the reference. */
+int tagi_conv2d_build_idx(int kernel, int stride, int wi, int hi, int pad,
+                          int pad_type, int param_pad_idx, int *Fmwa_2,
+                          int *FCzwa_1, int *Szz_ud, int *w, int *h);
+
+/* Forward through the Fmwa_2 table (device copy `aidx`); replaces
+ * conv2d_forward_cuda (src/conv2d_layer_cuda.cu:22-88).
+ * mu_a/var_a [B][fi][wihi], weights [fo][fi*ki*ki], out [B][fo][woho]. */
+int tagi_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
+                    const float *var_b, const float *mu_a, const float *var_a,
+                    const int *aidx, int woho, int fo, int wihi, int fi,
+                    int ki, int B, int bias, float *mu_z, float *var_z,
+                    void *stream);
+
+/* State backward through FCzwa_1 (`zw_idx`, [wihi][nr]) and Szz_ud (`zud_idx`,
+ * [nr][wihi]); replaces conv2d_state_backward_cuda
+ * (src/conv2d_layer_cuda.cu:90-147) including the Jacobian permutation
+ * Conv2dCuda::backward runs before it (src/conv2d_layer_cuda.cu:501-509):
+ * `jcb` is the un-permuted [B][fi][wihi] Jacobian. Requires every input pixel
+ * to be covered (w == wihi), as the reference's kernels assume. */
+int tagi_conv2d_bwd_dz(const float *mu_w, const float *jcb,
+                       const float *delta_mu_out, const float *delta_var_out,
+                       const int *zw_idx, const int *zud_idx, int woho, int fo,
+                       int wihi, int fi, int ki, int nr, int B,
+                       float *delta_mu, float *delta_var, void *stream);
+
+/* Weight (and, with bias != 0, bias) backward through Fmwa_2; replaces
+ * conv2d_param_backward_cuda (src/conv2d_layer_cuda.cu:149-227) including its
+ * delta permutation, and the bias reduction of Conv2dCuda::backward (478-498): delta_*_out are the un-permuted [B][fo][woho] deltas. */
+int tagi_conv2d_bwd_dw(const float *var_w, const float *var_b,
+                       const float *mu_a, const float *delta_mu_out,
+                       const float *delta_var_out, const int *aidx, int B,
+                       int fo, int woho, int wihi, int fi, int ki, int bias,
+                       float *delta_mu_w, float *delta_var_w,
+                       float *delta_mu_b, float *delta_var_b, void *stream);
+
+/* ---- layer glue ------------------------------------------------------------ */
+
+/* Keep what the backward pass needs and reset the output Jacobian; replaces
+ * BaseLayerCuda::store_states_for_training_cuda
+ * (src/base_layer_cuda.cu:464-486): bwd_mu_a/bwd_jcb <- first n_in entries of
+ * mu_a/jcb, out_jcb[0..n_out) <- 1. */
+int tagi_store_states(const float *mu_a, const float *jcb, size_t n_in,
+                      float *bwd_mu_a, float *bwd_jcb, float *out_jcb,
+                      size_t n_out, void *stream);
+
+/* Capped parameter step, p += sign(d) * min(|d|, sqrt(var)/cap), with
+ * var <= 0 -> 1e-5; replaces device_weight_update / device_bias_update
+ * (src/base_layer_cuda.cu:56-103). neg_var_count (device int, may be NULL) is
+ * incremented once per clamped variance; the caller zeroes it. */
+int tagi_param_update(const float *delta_mu, const float *delta_var,
+                      float cap_factor, size_t n, float *mu, float *var,
+                      int *neg_var_count, void *stream);
+
+/* Cap factor for a batch size (src/base_layer.cpp:164-187); `prev` is returned
+ * for batch sizes below 1. Host only. */
+float tagi_cap_factor(int batch_size, float prev);
+
+/* ---- output updater -------------------------------------------------------- */
+
+/* delta_mu = jcb/(var_a+var_obs) * (obs-mu_a), delta_var = -jcb^2/(var_a+var_obs),
+ * inf/nan -> 0; replaces update_delta_z_cuda (src/output_updater_cuda.cu:27-44).
+ * The caller zeroes the delta buffers first, as reset_zeros does. */
+int tagi_out_update_dense(const float *mu_a, const float *var_a,
+                          const float *jcb, const float *obs,
+                          const float *var_obs, int n, float *delta_mu,
+                          float *delta_var, void *stream);
+
+/* The same for the selected (1-based) output indices of hierarchical softmax;
+ * replaces update_delta_z_using_indices_cuda (src/output_updater_cuda.cu:3-26). */
+int tagi_out_update_indexed(const float *mu_a, const float *var_a,
+                            const float *jcb, const float *obs,
+                            const float *var_obs, const int *selected_idx,
+                            int n_obs, int n_enc, int n, float *delta_mu,
+                            float *delta_var, void *stream);
+
+/* ---- ReLU -------------------------------------------------------------------- */
+
+/* mu_a = max(mu_z, 0); jcb, var_a = (0, 0) where that is 0, else (1, var_z);
+ * replaces relu_mean_var_cuda (src/activation_cuda.cu), CPU form
+ * src/activation.cpp:7-29. In place allowed. */
+int tagi_relu_fwd(const float *mu_z, const float *var_z, size_t n, float *mu_a,
+                  float *jcb, float *var_a, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TAGI_HIP_H */

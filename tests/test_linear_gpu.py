@@ -1,0 +1,77 @@
+"""Parity of the HIP Linear path (through the C ABI) against the CPU oracle."""
+import numpy as np
+import pytest
+
+from util import assert_close, linear_inputs
+
+pytestmark = pytest.mark.gpu
+
+# (K, N, B): tiled path (aligned / ragged / odd), skinny path, layer shapes of
+# the MLP configuration, and the reference's odd-size smoke shape (785 -> 6000)
+# scaled down.
+SHAPES = [
+    (256, 256, 128), (512, 384, 256), (100, 36, 40), (785, 600, 16), (784, 128, 32),
+    (128, 128, 32), (128, 11, 32), (64, 32, 1), (256, 512, 8), (1024, 256, 5),
+    (516, 260, 16), (130, 70, 17), (5, 3, 2), (4, 4, 4), (333, 129, 77),
+]
+
+
+def _dev(d):
+    import torch
+    return {k: (None if v is None else torch.from_numpy(v).cuda()) for k, v in d.items()}
+
+
+@pytest.mark.parametrize("K,N,B", SHAPES)
+@pytest.mark.parametrize("bias", [True, False])
+def test_linear_forward(oracle_lib, K, N, B, bias):
+    import cutagi_amd.functional as F
+    d = linear_inputs(K, N, B, seed=K + N + B, bias=bias)
+    t = _dev(d)
+    mu_z, var_z = F.linear_fwd(t["mu_w"], t["var_w"], t["mu_b"], t["var_b"], t["mu_a"], t["var_a"])
+    ref_mu, ref_var = oracle_lib.linear_fwd(d["mu_w"], d["var_w"], d["mu_b"], d["var_b"],
+                                            d["mu_a"], d["var_a"], threads=4)
+    assert_close(mu_z.cpu().numpy(), ref_mu, "mu_z")
+    assert_close(var_z.cpu().numpy(), ref_var, "var_z")
+    assert float(var_z.min()) >= 0.0
+
+
+@pytest.mark.parametrize("K,N,B", SHAPES)
+def test_linear_backward(oracle_lib, K, N, B):
+    import cutagi_amd.functional as F
+    d = linear_inputs(K, N, B, seed=7 * K + N + B, bias=True, jcb_random=True)
+    t = _dev(d)
+    out = F.linear_bwd(t["mu_w"], t["var_w"], t["var_b"], t["mu_a"], t["jcb"], t["delta_mu"],
+                       t["delta_var"])
+    dz = oracle_lib.linear_bwd_dz(d["mu_w"], d["jcb"], d["delta_mu"], d["delta_var"], threads=4)
+    dw = oracle_lib.linear_bwd_dw(d["var_w"], d["mu_a"], d["delta_mu"], d["delta_var"], threads=4)
+    db = oracle_lib.linear_bwd_db(d["var_b"], d["delta_mu"], d["delta_var"])
+    names = ["delta_mu_z", "delta_var_z", "delta_mu_w", "delta_var_w", "delta_mu_b", "delta_var_b"]
+    for name, got, ref in zip(names, out, dz + dw + db):
+        assert_close(got.cpu().numpy(), ref, name)
+    # innovations of the variance keep the sign of delta_var (<= 0)
+    assert float(out[1].max()) <= 0.0 and float(out[3].max()) <= 0.0 and float(out[5].max()) <= 0.0
+
+
+def test_linear_backward_skips(oracle_lib):
+    """state_update / param_update switches of LinearCuda::backward."""
+    import torch
+    import cutagi_amd.functional as F
+    d = linear_inputs(64, 32, 8, seed=3)
+    t = _dev(d)
+    out = F.linear_bwd(t["mu_w"], t["var_w"], t["var_b"], t["mu_a"], t["jcb"], t["delta_mu"],
+                       t["delta_var"], state_update=False)
+    assert out[0] is None and out[2] is not None
+    out = F.linear_bwd(t["mu_w"], t["var_w"], t["var_b"], t["mu_a"], t["jcb"], t["delta_mu"],
+                       t["delta_var"], param_update=False)
+    assert out[2] is None and out[4] is None and out[0] is not None
+    torch.cuda.synchronize()
+
+
+def test_size_mismatch_raises():
+    """The reference throws on an input-size mismatch (Linear::forward)."""
+    import cutagi_amd.functional as F
+    d = linear_inputs(64, 32, 8, seed=3)
+    t = _dev(d)
+    with pytest.raises(ValueError):
+        F.linear_fwd(t["mu_w"], t["var_w"], t["mu_b"], t["var_b"], t["mu_a"][:, :32].contiguous(),
+                     t["var_a"][:, :32].contiguous())

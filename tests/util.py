@@ -1,0 +1,69 @@
+"""Shared helpers of the parity tests: the error metric and seeded inputs."""
+import numpy as np
+
+# Tolerance of the parity gate: max_i |x_i - ref_i| / max(|ref_i|, rms(ref)).
+# Normalising small entries by the tensor's rms keeps reordering noise on
+# near-zero means (absolute error ~1e-6) from reading as a large relative error.
+TOL = 1e-4
+
+
+def rel_err(x, ref):
+    x = np.asarray(x, dtype=np.float64).ravel()
+    ref = np.asarray(ref, dtype=np.float64).ravel()
+    assert x.shape == ref.shape
+    if ref.size == 0:
+        return 0.0
+    rms = np.sqrt(np.mean(ref * ref))
+    denom = np.maximum(np.abs(ref), max(rms, 1e-30))
+    return float(np.max(np.abs(x - ref) / denom))
+
+
+def assert_close(x, ref, what, tol=TOL):
+    e = rel_err(x, ref)
+    assert np.all(np.isfinite(np.asarray(x))), what + ": non-finite values"
+    assert e <= tol, "%s: rel err %.3e > %.1e" % (what, e, tol)
+    return e
+
+
+def linear_inputs(K, N, B, seed=0, bias=True, jcb_random=False):
+    """Distributions of the benchmark configurations: mu_a ~ N(0,1),
+    var_a ~ U(0.01,0.1), mu_w ~ N(0,1/K), var_w ~ 1/K (jittered so that a wrong
+    index shows), delta_mu ~ N(0,1e-2), delta_var ~ -U(0,1e-3)."""
+    rng = np.random.default_rng(seed)
+    f = np.float32
+    d = dict(
+        mu_w=rng.normal(0, K ** -0.5, (N, K)).astype(f),
+        var_w=(rng.uniform(0.5, 1.5, (N, K)) / K).astype(f),
+        mu_a=rng.normal(0, 1, (B, K)).astype(f),
+        var_a=rng.uniform(0.01, 0.1, (B, K)).astype(f),
+        delta_mu=rng.normal(0, 0.1, (B, N)).astype(f),
+        delta_var=(-rng.uniform(0, 1e-3, (B, N))).astype(f),
+        jcb=(rng.uniform(0, 1, (B, K)) if jcb_random else np.ones((B, K))).astype(f),
+    )
+    if bias:
+        d["mu_b"] = rng.normal(0, 0.5, N).astype(f)
+        d["var_b"] = (rng.uniform(0.5, 1.5, N) / K).astype(f)
+    else:
+        d["mu_b"] = d["var_b"] = None
+    return d
+
+
+def conv_inputs(fi, fo, ki, wihi, woho, B, seed=0, bias=False, jcb_random=False):
+    rng = np.random.default_rng(seed)
+    f = np.float32
+    k2 = ki * ki
+    d = dict(
+        mu_w=rng.normal(0, (k2 * fi) ** -0.5, fo * fi * k2).astype(f),
+        var_w=(rng.uniform(0.5, 1.5, fo * fi * k2) / (k2 * fi)).astype(f),
+        mu_a=rng.normal(0, 1, B * fi * wihi).astype(f),
+        var_a=rng.uniform(0.01, 0.1, B * fi * wihi).astype(f),
+        delta_mu=rng.normal(0, 0.1, B * fo * woho).astype(f),
+        delta_var=(-rng.uniform(0, 1e-3, B * fo * woho)).astype(f),
+        jcb=(rng.uniform(0, 1, B * fi * wihi) if jcb_random else np.ones(B * fi * wihi)).astype(f),
+    )
+    if bias:
+        d["mu_b"] = rng.normal(0, 0.5, fo).astype(f)
+        d["var_b"] = (rng.uniform(0.5, 1.5, fo) / (k2 * fi)).astype(f)
+    else:
+        d["mu_b"] = d["var_b"] = None
+    return d
