@@ -1,0 +1,225 @@
+#!/usr/bin/env python3
+"""Benchmark of the TAGI Linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm|skinny]
+
+A step is one forward + backward (delta_z, delta_w, delta_b) of a single TAGI
+Linear layer on synthetic inputs that are resident in HBM before the timed
+region starts. The default workload is the dense one the headline metric is
+quoted on (4096 -> 4096, batch 256, fp32); `--workload skinny` times the
+HBM-bound one (8192 -> 8192, batch 8) and reports GB/s. The default run also
+times the skinny workload and the CPU baseline and attaches them to the same
+JSON line.
+
+Prints ONE JSON line. `roofline` is computed for the dominant kernel from its
+algorithmic work and its average duration measured with HIP events on the
+stream the kernels run on; `cpu_baseline` is the CPU oracle (a bit-identical
+restatement of the reference's multithreaded CPU path) timed on this host.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E peak
+
+WORKLOADS = {
+    # name: (K, N, B, bound)
+    "gemm": (4096, 4096, 256, "mfma"),
+    "skinny": (8192, 8192, 8, "hbm"),
+}
+
+
+def make_inputs(K, N, B, device):
+    """Distributions of the benchmark configuration, seed 0."""
+    import torch
+    g = torch.Generator(device=device)
+    g.manual_seed(0)
+    randn = lambda *s: torch.randn(*s, device=device, generator=g)
+    rand = lambda *s: torch.rand(*s, device=device, generator=g)
+    return dict(
+        mu_w=randn(N, K) * K ** -0.5,
+        var_w=torch.full((N, K), 1.0 / K, device=device),
+        mu_b=torch.zeros(N, device=device),
+        var_b=torch.full((N,), 1.0 / K, device=device),
+        mu_a=randn(B, K),
+        var_a=rand(B, K) * 0.09 + 0.01,
+        jcb=torch.ones(B, K, device=device),
+        delta_mu=randn(B, N) * 0.1,
+        delta_var=-rand(B, N) * 1e-3,
+    )
+
+
+def run_workload(name, steps, warmup):
+    import torch
+    import cutagi_amd.functional as F
+
+    K, N, B, bound = WORKLOADS[name]
+    dev = torch.device("cuda:0")
+    t = make_inputs(K, N, B, dev)
+    out_z = (torch.empty(B, N, device=dev), torch.empty(B, N, device=dev))
+    out_dz = (torch.empty(B, K, device=dev), torch.empty(B, K, device=dev))
+    out_dw = (torch.empty(N, K, device=dev), torch.empty(N, K, device=dev))
+    out_db = (torch.empty(N, device=dev), torch.empty(N, device=dev))
+
+    phases = [
+        ("fwd", lambda: F.linear_fwd(t["mu_w"], t["var_w"], t["mu_b"], t["var_b"], t["mu_a"],
+                                     t["var_a"], out=out_z)),
+        ("bwd_dz", lambda: F.linear_bwd_dz(t["mu_w"], t["jcb"], t["delta_mu"], t["delta_var"],
+                                           out=out_dz)),
+        ("bwd_dw", lambda: F.linear_bwd_dw(t["var_w"], t["mu_a"], t["delta_mu"], t["delta_var"],
+                                           out=out_dw)),
+        ("bwd_db", lambda: F.linear_bwd_db(t["var_b"], t["delta_mu"], t["delta_var"],
+                                           out=out_db)),
+    ]
+
+    def step():
+        for _, fn in phases:
+            fn()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+
+    # timed region: exactly `steps` steps between two synchronisations
+    t0 = time.perf_counter()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = e0.elapsed_time(e1) / steps
+
+    # second pass: per-phase durations with HIP events on the same stream
+    marks = [[torch.cuda.Event(enable_timing=True) for _ in range(len(phases) + 1)]
+             for _ in range(steps)]
+    for s in range(steps):
+        marks[s][0].record()
+        for i, (_, fn) in enumerate(phases):
+            fn()
+            marks[s][i + 1].record()
+    torch.cuda.synchronize()
+    phase_ms = {}
+    for i, (pname, _) in enumerate(phases):
+        phase_ms[pname] = sum(m[i].elapsed_time(m[i + 1]) for m in marks) / steps
+
+    flops = {"fwd": 6.0 * B * N * K, "bwd_dz": 4.0 * B * N * K, "bwd_dw": 4.0 * B * N * K}
+    bytes_ = {"fwd": 2.0 * N * K * 4, "bwd_dz": 1.0 * N * K * 4, "bwd_dw": 3.0 * N * K * 4}
+    dominant = max(flops, key=lambda p: phase_ms[p])
+    if bound == "mfma":
+        achieved = flops[dominant] / (phase_ms[dominant] * 1e-3) / 1e12
+        roof = dict(bound="mfma", kernel=dominant, achieved=round(achieved, 2),
+                    peak=FP32_MFMA_PEAK_TFLOPS, unit="TFLOP/s",
+                    frac=round(achieved / FP32_MFMA_PEAK_TFLOPS, 4), traffic=None)
+        value = 14.0 * B * N * K / (ms_per_step * 1e-3) / 1e12
+        unit = "TFLOP/s"
+        peak = FP32_MFMA_PEAK_TFLOPS
+    else:
+        achieved = bytes_[dominant] / (phase_ms[dominant] * 1e-3) / 1e9
+        roof = dict(bound="hbm", kernel=dominant, achieved=round(achieved, 1), peak=HBM_PEAK_GBS,
+                    unit="GB/s", frac=round(achieved / HBM_PEAK_GBS, 4), traffic=None)
+        value = 6.0 * N * K * 4 / (ms_per_step * 1e-3) / 1e9
+        unit = "GB/s"
+        peak = HBM_PEAK_GBS
+    roof["kernel_ms"] = round(phase_ms[dominant], 5)
+    return dict(name=name, K=K, N=N, B=B, value=value, unit=unit, frac_of_peak=value / peak,
+                ms_per_step=ms_per_step, wall_ms=wall_ms, phase_ms=phase_ms, roofline=roof)
+
+
+def cpu_baseline(name):
+    """One full step of the same workload on the host cores, through the oracle."""
+    import numpy as np
+    import oracle
+
+    K, N, B, _ = WORKLOADS[name]
+    lib = oracle.load()
+    threads = max(1, min(16, os.cpu_count() or 1))
+    rng = np.random.default_rng(0)
+    f = np.float32
+    mu_w = (rng.standard_normal((N, K)) * K ** -0.5).astype(f)
+    var_w = np.full((N, K), 1.0 / K, f)
+    mu_b = np.zeros(N, f)
+    var_b = np.full(N, 1.0 / K, f)
+    mu_a = rng.standard_normal((B, K)).astype(f)
+    var_a = rng.uniform(0.01, 0.1, (B, K)).astype(f)
+    jcb = np.ones((B, K), f)
+    dmu = (rng.standard_normal((B, N)) * 0.1).astype(f)
+    dvar = (-rng.uniform(0, 1e-3, (B, N))).astype(f)
+    t0 = time.perf_counter()
+    lib.linear_fwd(mu_w, var_w, mu_b, var_b, mu_a, var_a, threads)
+    lib.linear_bwd_dz(mu_w, jcb, dmu, dvar, threads)
+    lib.linear_bwd_dw(var_w, mu_a, dmu, dvar, threads)
+    lib.linear_bwd_db(var_b, dmu, dvar, threads)
+    dt = time.perf_counter() - t0
+    return dict(value=round(14.0 * B * N * K / dt / 1e12, 5), unit="TFLOP/s", cores=threads,
+                kind="port", seconds=round(dt, 3),
+                sample="1 full forward+backward step of the %s workload (K=%d, N=%d, B=%d), "
+                       "reference thread fan-out with %d std::threads" % (name, K, N, B, threads))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="gemm")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary workload")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path "
+              "(run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (torch.cuda.is_available() is False)", file=sys.stderr)
+        sys.exit(1)
+
+    main_res = run_workload(args.workload, args.steps, args.warmup)
+    line = {
+        "metric": "TAGI Linear fwd+bwd TFLOP/s (% fp32 MFMA peak) 4096^2,B=256; GB/s at B=8",
+        "value": round(main_res["value"], 3),
+        "unit": main_res["unit"],
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(main_res["ms_per_step"], 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "TAGI Linear %d->%d, batch %d, fp32, forward + backward "
+                               "(delta_z, delta_w, delta_b)" % (main_res["K"], main_res["N"],
+                                                                main_res["B"]),
+                   "name": main_res["name"]},
+        "frac_of_peak": round(main_res["frac_of_peak"], 4),
+        "phase_ms": {k: round(v, 5) for k, v in main_res["phase_ms"].items()},
+        "roofline": main_res["roofline"],
+    }
+    if not args.no_extra:
+        other = "skinny" if args.workload == "gemm" else "gemm"
+        r = run_workload(other, args.steps, args.warmup)
+        line["extra"] = {other: {
+            "workload": "TAGI Linear %d->%d, batch %d" % (r["K"], r["N"], r["B"]),
+            "value": round(r["value"], 3), "unit": r["unit"],
+            "frac_of_peak": round(r["frac_of_peak"], 4),
+            "ms_per_step": round(r["ms_per_step"], 5),
+            "phase_ms": {k: round(v, 5) for k, v in r["phase_ms"].items()},
+            "roofline": r["roofline"]}}
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(args.workload)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

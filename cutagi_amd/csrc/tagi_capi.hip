@@ -56,6 +56,7 @@ struct Tuning {
     int gemv_max_batch = -1;
     int tile = -1;
     int conv_dw_splits = -1;
+    int gemv_swz = -1;
 };
 Tuning g_tune;
 
@@ -65,17 +66,18 @@ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 int pick_tile(int rows) {
     // tile ids: 0 = 128x128, 1 = 64x128, 2 = 32x128 (rows x columns)
     if (g_tune.tile >= 0 && g_tune.tile < gemm_tile_count()) return g_tune.tile;
-    if (rows > 64) return 0;
+    // 64x128 keeps the accumulators small enough for two workgroups per CU,
+    // which measures faster than one 128x128 workgroup on every shape tried
     if (rows > 32) return 1;
     return 2;
 }
 
-// Reduction slices so that a launch reaches about one workgroup per CU, while
+// Reduction slices so that a launch reaches about two workgroups per CU, while
 // every slice keeps at least `min_tiles` k-tiles of work.
 int pick_splits(int tiles, int reduction, int forced, int min_tiles = 8) {
     const int kt = gemm_k_tile();
     const int k_tiles = ceil_div(reduction, kt);
-    int s = forced > 0 ? forced : ceil_div(NUM_CU, tiles);
+    int s = forced > 0 ? forced : ceil_div(2 * NUM_CU, tiles);
     const int cap = k_tiles / min_tiles > 0 ? k_tiles / min_tiles : 1;
     if (forced <= 0 && s > cap) s = cap;
     if (s > k_tiles) s = k_tiles;
@@ -172,6 +174,7 @@ int tagi_hip_tune(const char *key, int value) {
     else if (!strcmp(key, "linear.gemv_max_batch")) g_tune.gemv_max_batch = value;
     else if (!strcmp(key, "linear.tile")) g_tune.tile = value;
     else if (!strcmp(key, "conv2d.dw.splits")) g_tune.conv_dw_splits = value;
+    else if (!strcmp(key, "linear.gemv.swizzle")) g_tune.gemv_swz = value;
     else return TAGI_ERR_INVALID_ARG;
     return TAGI_OK;
 }
@@ -192,18 +195,23 @@ int tagi_linear_fwd(const float *mu_w, const float *var_w, const float *mu_b, co
                      aligned16(var_a);
 
     if (B <= gemv_max_batch() && vec) {
+        // slices: short enough for the LDS-resident activations, and enough of
+        // them for about two workgroups per CU
         const int blocks = ceil_div(N, gemv_fwd_rows_per_block());
-        int splits = g_tune.fwd_splits > 0 ? g_tune.fwd_splits : ceil_div(4 * NUM_CU, blocks);
-        const int max_splits = ceil_div(K, 4 * gemv_fwd_k_step());
+        const int step = gemv_fwd_k_step();
+        int splits = g_tune.fwd_splits > 0 ? g_tune.fwd_splits : ceil_div(2 * NUM_CU, blocks);
+        const int max_splits = ceil_div(K, 4 * step);
         if (splits > max_splits) splits = max_splits;
-        if (splits < 1) splits = 1;
-        int per = ceil_div(ceil_div(K, splits), gemv_fwd_k_step()) * gemv_fwd_k_step();
+        const int min_splits = ceil_div(K, gemv_fwd_max_slice(B));
+        if (splits < min_splits) splits = min_splits;
+        int per = ceil_div(ceil_div(K, splits), step) * step;
         splits = ceil_div(K, per);
         float *ws = nullptr;
         const size_t part = (size_t)splits * B * N;
         int rc = workspace_get(2 * part * sizeof(float), &ws);
         if (rc != TAGI_OK) return rc;
-        TAGI_TRY(launch_gemv_fwd(mu_w, var_w, mu_a, var_a, K, N, B, splits, ws, ws + part, stream));
+        TAGI_TRY(launch_gemv_fwd(mu_w, var_w, mu_a, var_a, K, N, B, splits,
+                                 g_tune.gemv_swz >= 0 ? g_tune.gemv_swz : 3, ws, ws + part, stream));
         TAGI_TRY(launch_reduce_splits(EPI_BIAS, ws, ws + part, splits, B, N, e0, e1, mu_z, var_z, N,
                                       stream));
         return TAGI_OK;
@@ -229,11 +237,13 @@ int tagi_linear_bwd_dz(const float *mu_w, const float *jcb, const float *delta_m
 
     if (B <= gemv_max_batch() && vec) {
         const int blocks = ceil_div(K, gemv_dz_cols_per_block());
-        int splits = g_tune.dz_splits > 0 ? g_tune.dz_splits : ceil_div(4 * NUM_CU, blocks);
-        const int max_splits = ceil_div(N, 4 * gemv_dz_n_step());
+        const int step = gemv_dz_n_step();
+        int splits = g_tune.dz_splits > 0 ? g_tune.dz_splits : ceil_div(NUM_CU, blocks);
+        const int max_splits = ceil_div(N, 2 * step);
         if (splits > max_splits) splits = max_splits;
-        if (splits < 1) splits = 1;
-        int per = ceil_div(ceil_div(N, splits), gemv_dz_n_step()) * gemv_dz_n_step();
+        const int min_splits = ceil_div(N, gemv_dz_max_slice(B));
+        if (splits < min_splits) splits = min_splits;
+        int per = ceil_div(ceil_div(N, splits), step) * step;
         splits = ceil_div(N, per);
         float *ws = nullptr;
         const size_t part = (size_t)splits * B * K;

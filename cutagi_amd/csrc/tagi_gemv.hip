@@ -1,13 +1,14 @@
 // Skinny-batch (B <= 16) kernels of the TAGI Linear layer, gfx950.
 //
 // With a handful of samples every weight is used only B times, so the layer is
-// bound by streaming the weight matrices from HBM once. Nothing is staged in
-// LDS: each lane loads 16 bytes of a weight row straight into the operand
-// layout of v_mfma_f32_16x16x4_f32 (A[i][k]: lane = i + 16*k, B[k][j]: lane =
-// j + 16*k, D[i][j]: register i%4 of lane j + 16*(i/4)), the batch sits in the
-// 16 columns of the MFMA (columns >= B are fed zeros), and the reduction over
-// the streamed dimension happens inside the matrix core. The weight backward
-// has no reduction worth an MFMA (length B) and is a pure VALU streaming kernel.
+// bound by streaming the weight matrices from HBM once. Each lane loads 16 bytes
+// of a weight row straight into the operand layout of v_mfma_f32_4x4x1_16b_f32,
+// chosen because its 16 independent 4x4 blocks let a load instruction cover whole
+// cache lines (4 rows x 256 B forward, 1 row x 1 KB backward) while the batch
+// sits in the 4 columns of a block (groups of 4 samples, rows beyond B are fed
+// zeros). The few activations / innovations a workgroup needs live in LDS. The
+// weight backward has no reduction worth an MFMA (length B) and is a pure VALU
+// streaming kernel.
 //
 // Reduction slices (gridDim.y) write partial sums [slice][B][cols]; the caller
 // folds them, together with the bias or Jacobian epilogue, in reduce_splits.
@@ -26,168 +27,349 @@ __device__ __forceinline__ float4 zero4() { return make_float4(0.f, 0.f, 0.f, 0.
 __device__ __forceinline__ float comp(const float4 &v, int t) {
     return t == 0 ? v.x : t == 1 ? v.y : t == 2 ? v.z : v.w;
 }
-__device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
-}
 
 // ---------------------------------------------------------------------------
-// Forward. A wave owns 16 output rows (weight rows n0..n0+15) and one reduction
-// slice; lane (i = l%16, g = l/16) reads U consecutive float4 of row n0+i
-// starting at k = kb + 4*U*g, so one row is read in runs of 64*U bytes and the
-// four lanes of a row cover 256*U bytes between them. MFMA (u, t) multiplies
-// k = kb + 4*U*g + 4*u + t on both operands.
+// Forward, v_mfma_f32_4x4x1_16b_f32: 16 independent 4x4 outer products per
+// instruction, A_blk[i] taken from lane 4*blk+i, B_blk[j] from lane 4*blk+j,
+// D_blk[i][j] in register i of lane 4*blk+j.
+//
+// Lane (blk = l/4, i = l%4) streams weight row n0+4*rg+i and holds the float4 at
+// k = kb + 4*blk, so one load instruction covers 4 rows x 256 contiguous bytes
+// (8 full cache lines). Block blk multiplies reduction elements kb+4*blk+t
+// (t = 0..3, one MFMA each) against the activations of samples j+4*h, which the
+// workgroup keeps in LDS for its whole reduction slice. The 16 blocks hold
+// partial sums over different k; they meet in one cross-lane reduction when the
+// slice is finished.
 // ---------------------------------------------------------------------------
-constexpr int FWD_U = 4;
-constexpr int FWD_ROWS_PER_BLOCK = 64;  // 4 waves x 16 rows
-constexpr int FWD_KSTEP = 16 * FWD_U;
+constexpr int FWD_WAVES = 8;
+constexpr int FWD_RG = 2;                                  // row groups of 4 per wave
+constexpr int FWD_ROWS_PER_BLOCK = FWD_WAVES * FWD_RG * 4;  // 64
+constexpr int FWD_KSTEP = 64;   // reduction elements per register stage
+constexpr int FWD_KROUND = 2 * FWD_KSTEP;  // slices are whole pairs of stages
+constexpr int FWD_LDS_PAD = 8;  // row stride % 32 == 8: conflict-free 16-byte reads
 
-struct FwdRegs {
-    float4 wm[FWD_U], wv[FWD_U], am[FWD_U], av[FWD_U];
-};
-
-__device__ __forceinline__ void fwd_load(FwdRegs &r, const float *wm, const float *wv,
-                                         const float *am, const float *av, bool row_ok,
-                                         bool act_ok, int k, int k_end) {
-#pragma unroll
-    for (int u = 0; u < FWD_U; u++) {
-        const int kk = k + 4 * u;
-        const bool in = kk < k_end;
-        r.wm[u] = (row_ok && in) ? ld4(wm + kk) : zero4();
-        r.wv[u] = (row_ok && in) ? ld4(wv + kk) : zero4();
-        r.am[u] = (act_ok && in) ? ld4(am + kk) : zero4();
-        r.av[u] = (act_ok && in) ? ld4(av + kk) : zero4();
-    }
+__device__ __forceinline__ floatx4 mfma4(float a, float b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_4x4x1f32(a, b, c, 0, 0, 0);
 }
 
-__global__ __launch_bounds__(256) void gemv_fwd_kernel(
+template <int H>
+__global__ __launch_bounds__(FWD_WAVES * 64) void gemv_fwd_kernel(
     const float *__restrict__ mu_w, const float *__restrict__ var_w,
     const float *__restrict__ mu_a, const float *__restrict__ var_a, int K, int N, int B,
-    int k_per_split, float *__restrict__ ws0, float *__restrict__ ws1) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int i = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * FWD_ROWS_PER_BLOCK + wave * 16;
-    const int split = blockIdx.y;
+    int k_per_split, int splits, int swz, float *__restrict__ ws0, float *__restrict__ ws1) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int S = k_per_split + FWD_LDS_PAD;  // LDS row stride
+    float *s_mu = lds, *s_var = lds + 4 * H * S;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int blk = lane >> 2, i = lane & 3;
+    // Workgroup -> (row block, reduction slice). Workgroups are handed to the 8
+    // XCDs round-robin; with the slice as the fast index inside an XCD, the
+    // workgroups resident on one XCD cover all slices (all 4 KB windows of a
+    // weight row) instead of crowding into one.
+    int row_block, split;
+    const int id = blockIdx.x, row_blocks = gridDim.x / splits;
+    if ((swz & 1) && row_blocks % 8 == 0) {
+        const int xcd = id & 7, local = id >> 3;
+        split = local % splits;
+        row_block = (local / splits) * 8 + xcd;
+    } else {
+        row_block = id % row_blocks;
+        split = id / row_blocks;
+    }
     const int k_begin = split * k_per_split;
-    const int k_end = min(K, k_begin + k_per_split);
-    const int row = n0 + i;
-    const bool row_ok = row < N, act_ok = i < B;
-    const float *wm = mu_w + (size_t)(row_ok ? row : 0) * K;
-    const float *wv = var_w + (size_t)(row_ok ? row : 0) * K;
-    const float *am = mu_a + (size_t)(act_ok ? i : 0) * K;
-    const float *av = var_a + (size_t)(act_ok ? i : 0) * K;
+    const int kr = min(K, k_begin + k_per_split) - k_begin;  // this slice's length
+    // each wave walks its slice from a different starting point (sums commute)
+    const int rot = (swz & 2) ? ((row_block * FWD_WAVES + wave) * FWD_KROUND) % k_per_split : 0;
 
-    floatx4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
-    FwdRegs cur, nxt;
-    const int koff = 4 * FWD_U * g;
-    fwd_load(cur, wm, wv, am, av, row_ok, act_ok, k_begin + koff, k_end);
-    for (int kb = k_begin; kb < k_end; kb += FWD_KSTEP) {
-        fwd_load(nxt, wm, wv, am, av, row_ok, act_ok, kb + FWD_KSTEP + koff, k_end);
-#pragma unroll
-        for (int u = 0; u < FWD_U; u++) {
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-                const float w = comp(cur.wm[u], t), v = comp(cur.wv[u], t);
-                const float a = comp(cur.am[u], t), s = comp(cur.av[u], t);
-                acc0 = mfma16(w, a, acc0);
-                acc1 = mfma16(v, s + a * a, acc1);
-                acc1 = mfma16(w * w, s, acc1);
-            }
+    // stage the slice of the activations: [sample][k], zero beyond B and kr
+    const int k4s = k_per_split / 4;
+    for (int e = tid; e < 4 * H * k4s; e += FWD_WAVES * 64) {
+        const int b = e / k4s, k = (e - b * k4s) * 4;
+        float4 m = zero4(), v = zero4();
+        if (b < B && k < kr) {
+            m = ld4(mu_a + (size_t)b * K + k_begin + k);
+            v = ld4(var_a + (size_t)b * K + k_begin + k);
         }
-        cur = nxt;
+        *reinterpret_cast<float4 *>(s_mu + b * S + k) = m;
+        *reinterpret_cast<float4 *>(s_var + b * S + k) = v;
     }
 
-    // D[i = row][j = sample]: lane (j = l%16, q = l/16) holds rows n0 + 4q + 0..3
-    const int j = lane & 15, q = lane >> 4;
-    if (j < B) {
-        const size_t base = ((size_t)split * B + j) * N + n0 + 4 * q;
+    // Weight loads are never predicated (a predicated load costs a branch and
+    // makes the compiler wait for every outstanding load): rows beyond N read row
+    // N-1 and are dropped at the end, reduction elements beyond the slice read the
+    // last float4 of the row and meet zero activations.
+    const int n0 = row_block * FWD_ROWS_PER_BLOCK + wave * (FWD_RG * 4);
+    const float *wm[FWD_RG], *wv[FWD_RG];
 #pragma unroll
-        for (int v = 0; v < 4; v++) {
-            if (n0 + 4 * q + v < N) {
-                ws0[base + v] = acc0[v];
-                ws1[base + v] = acc1[v];
+    for (int rg = 0; rg < FWD_RG; rg++) {
+        const int row = min(n0 + 4 * rg + i, N - 1);
+        wm[rg] = mu_w + (size_t)row * K;
+        wv[rg] = var_w + (size_t)row * K;
+    }
+    const int k_lane = k_begin + 4 * blk, k_last = K - 4;
+
+    floatx4 acc0[FWD_RG][H], acc1[FWD_RG][H];
+#pragma unroll
+    for (int rg = 0; rg < FWD_RG; rg++)
+#pragma unroll
+        for (int h = 0; h < H; h++) {
+            acc0[rg][h] = (floatx4){0.f, 0.f, 0.f, 0.f};
+            acc1[rg][h] = (floatx4){0.f, 0.f, 0.f, 0.f};
+        }
+
+    // Two register stages used in turn (no copies between them, so a stage's
+    // loads stay in flight while the other stage is multiplied).
+    float4 am_[2][FWD_RG], av_[2][FWD_RG];
+    auto load = [&](float4(&m)[FWD_RG], float4(&v)[FWD_RG], int kb) {
+        const int k = min(k_lane + kb, k_last);
+#pragma unroll
+        for (int rg = 0; rg < FWD_RG; rg++) {
+            m[rg] = ld4(wm[rg] + k);
+            v[rg] = ld4(wv[rg] + k);
+        }
+    };
+    auto multiply = [&](const float4(&cm)[FWD_RG], const float4(&cv)[FWD_RG], int kb) {
+        float4 am[H], as[H], av[H];
+#pragma unroll
+        for (int h = 0; h < H; h++) {
+            am[h] = *reinterpret_cast<const float4 *>(s_mu + (i + 4 * h) * S + kb + 4 * blk);
+            av[h] = *reinterpret_cast<const float4 *>(s_var + (i + 4 * h) * S + kb + 4 * blk);
+            as[h] = make_float4(av[h].x + am[h].x * am[h].x, av[h].y + am[h].y * am[h].y,
+                                av[h].z + am[h].z * am[h].z, av[h].w + am[h].w * am[h].w);
+        }
+#pragma unroll
+        for (int rg = 0; rg < FWD_RG; rg++) {
+            const float4 q = make_float4(cm[rg].x * cm[rg].x, cm[rg].y * cm[rg].y,
+                                         cm[rg].z * cm[rg].z, cm[rg].w * cm[rg].w);
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+#pragma unroll
+                for (int h = 0; h < H; h++) {
+                    acc0[rg][h] = mfma4(comp(cm[rg], t), comp(am[h], t), acc0[rg][h]);
+                    acc1[rg][h] = mfma4(comp(cv[rg], t), comp(as[h], t), acc1[rg][h]);
+                    acc1[rg][h] = mfma4(comp(q, t), comp(av[h], t), acc1[rg][h]);
+                }
+        }
+    };
+
+    // k_per_split is a multiple of two stages and the staged activations are zero
+    // beyond the slice, so the loop needs no tail handling; `pos` is the rotated
+    // position inside the slice.
+    const int span = (swz & 2) ? k_per_split : kr;
+    auto wrap = [&](int p) { return p >= k_per_split ? p - k_per_split : p; };
+    load(am_[0], av_[0], rot);
+    __syncthreads();
+    for (int kb = 0; kb < span; kb += 2 * FWD_KSTEP) {
+        const int p0 = wrap(rot + kb), p1 = p0 + FWD_KSTEP, p2 = wrap(p0 + 2 * FWD_KSTEP);
+        // the barriers keep the scheduler from sinking a stage's loads below the
+        // MFMAs they are meant to overlap
+        load(am_[1], av_[1], p1);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(am_[0], av_[0], p0);
+        __builtin_amdgcn_sched_barrier(0);
+        load(am_[0], av_[0], p2);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(am_[1], av_[1], p1);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // sum the 16 blocks (lanes with equal l%4), then lanes 0..3 (sample j = l%4)
+    // hold D[row n0+4*rg+v][sample j+4*h] in register v
+#pragma unroll
+    for (int rg = 0; rg < FWD_RG; rg++)
+#pragma unroll
+        for (int h = 0; h < H; h++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                float x0 = acc0[rg][h][v], x1 = acc1[rg][h][v];
+#pragma unroll
+                for (int m = 4; m < 64; m <<= 1) {
+                    x0 += __shfl_xor(x0, m);
+                    x1 += __shfl_xor(x1, m);
+                }
+                acc0[rg][h][v] = x0;
+                acc1[rg][h][v] = x1;
             }
+    if (blk == 0) {
+#pragma unroll
+        for (int h = 0; h < H; h++) {
+            const int b = i + 4 * h;
+            if (b >= B) continue;
+#pragma unroll
+            for (int rg = 0; rg < FWD_RG; rg++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const int n = n0 + 4 * rg + v;
+                    if (n < N) {
+                        const size_t at = ((size_t)split * B + b) * N + n;
+                        ws0[at] = acc0[rg][h][v];
+                        ws1[at] = acc1[rg][h][v];
+                    }
+                }
         }
     }
 }
 
 // ---------------------------------------------------------------------------
-// State backward. A wave owns 64 consecutive input columns k' and one slice of
-// the reduction over output rows n; lane (i = l%16, g = l/16) reads the float4
-// W[n][c0 + 4i .. 4i+3] of rows n = nb + 4g + u (u = 0..3), i.e. every row is
-// read in 256-byte runs. Component t of the float4 feeds accumulator t, whose
-// row i is column c0 + 4i + t; the MFMA reduces over the four rows held by the
-// four lane groups.
+// State backward, same instruction. A wave owns 256 consecutive input columns
+// (lane l: the float4 at c0 + 4*l, so one load instruction is one contiguous
+// kilobyte of a weight row) and a range of output rows n; the MFMA for row n
+// multiplies A_blk[i] = w[n][c0 + 16*blk + 4*i + t] by B_blk[j] = delta[j+4*h][n]
+// and accumulates over the rows in place: register v of lane (blk, j) of
+// accumulator (t, h) is column c0 + 16*blk + 4*v + t of sample j+4*h. The eight
+// waves of a workgroup split its row slice and meet in an LDS tree reduction,
+// so only gridDim.y partial sums per output reach memory.
 // ---------------------------------------------------------------------------
-constexpr int DZ_COLS_PER_BLOCK = 256;  // 4 waves x 64 columns
-constexpr int DZ_NSTEP = 16;
+constexpr int DZ_WAVES = 8;
+constexpr int DZ_COLS_PER_BLOCK = 256;
+constexpr int DZ_STAGE = 8;  // rows in flight per wave and pipeline stage
+constexpr int DZ_NSTEP = DZ_WAVES * 2 * DZ_STAGE;  // slices: whole pairs of stages per wave
 
-struct DzRegs {
-    float4 w[4];
-    float4 dm, dv;
-};
-
-__device__ __forceinline__ void dz_load(DzRegs &r, const float *w, size_t ldw, bool col_ok,
-                                        const float *dm, const float *dv, bool act_ok, int n,
-                                        int n_end) {
-#pragma unroll
-    for (int u = 0; u < 4; u++)
-        r.w[u] = (col_ok && n + u < n_end) ? ld4(w + (size_t)(n + u) * ldw) : zero4();
-    const bool in = act_ok && n < n_end;
-    r.dm = in ? ld4(dm + n) : zero4();
-    r.dv = in ? ld4(dv + n) : zero4();
-}
-
-__global__ __launch_bounds__(256) void gemv_dz_kernel(
+template <int H>
+__global__ __launch_bounds__(DZ_WAVES * 64) void gemv_dz_kernel(
     const float *__restrict__ mu_w, const float *__restrict__ dmu,
     const float *__restrict__ dvar, int K, int N, int B, int n_per_split,
     float *__restrict__ ws0, float *__restrict__ ws1) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int i = lane & 15, g = lane >> 4;
-    const int c0 = blockIdx.x * DZ_COLS_PER_BLOCK + wave * 64;
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int S = n_per_split + 4;
+    float *s_dm = lds, *s_dv = lds + 4 * H * S;
+
+    // rows per pipeline stage: fewer for large batches, whose accumulators need
+    // the registers
+    constexpr int STAGE = H <= 2 ? DZ_STAGE : DZ_STAGE / 2;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int j = lane & 3;
     const int split = blockIdx.y;
     const int n_begin = split * n_per_split;
-    const int n_end = min(N, n_begin + n_per_split);
-    const int col = c0 + 4 * i;
-    const bool col_ok = col < K, act_ok = i < B;
-    const float *w = mu_w + (col_ok ? col : 0);
-    const float *dm = dmu + (size_t)(act_ok ? i : 0) * N;
-    const float *dv = dvar + (size_t)(act_ok ? i : 0) * N;
+    const int nr = min(N, n_begin + n_per_split) - n_begin;
 
-    floatx4 acc0[4], acc1[4];
-#pragma unroll
-    for (int t = 0; t < 4; t++) {
-        acc0[t] = (floatx4){0.f, 0.f, 0.f, 0.f};
-        acc1[t] = (floatx4){0.f, 0.f, 0.f, 0.f};
+    // stage this slice of the innovations: [sample][n], zero beyond B and nr
+    const int n4s = n_per_split / 4;
+    for (int e = tid; e < 4 * H * n4s; e += DZ_WAVES * 64) {
+        const int b = e / n4s, n = (e - b * n4s) * 4;
+        float4 m = zero4(), v = zero4();
+        if (b < B && n < nr) {
+            m = ld4(dmu + (size_t)b * N + n_begin + n);
+            v = ld4(dvar + (size_t)b * N + n_begin + n);
+        }
+        *reinterpret_cast<float4 *>(s_dm + b * S + n) = m;
+        *reinterpret_cast<float4 *>(s_dv + b * S + n) = v;
     }
-    DzRegs cur, nxt;
-    dz_load(cur, w, K, col_ok, dm, dv, act_ok, n_begin + 4 * g, n_end);
-    for (int nb = n_begin; nb < n_end; nb += DZ_NSTEP) {
-        dz_load(nxt, w, K, col_ok, dm, dv, act_ok, nb + DZ_NSTEP + 4 * g, n_end);
+
+    // Weight loads are never predicated: columns beyond K read column K-4 and are
+    // dropped at the end, rows beyond N read row N-1 and meet zero innovations.
+    const int col = min(blockIdx.x * DZ_COLS_PER_BLOCK + 4 * lane, K - 4);
+    // rows of this wave: local [r_lo, r_hi)
+    const int per_wave = n_per_split / DZ_WAVES;  // multiple of DZ_STAGE
+    const int r_lo = wave * per_wave, r_hi = min(nr, r_lo + per_wave);
+    const float *w = mu_w + col;
+    const int n_last = N - 1;
+
+    floatx4 acc0[4][H], acc1[4][H];
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            const float d0 = comp(cur.dm, u), d1 = comp(cur.dv, u);
+    for (int t = 0; t < 4; t++)
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
-                const float x = comp(cur.w[u], t);
-                acc0[t] = mfma16(x, d0, acc0[t]);
-                acc1[t] = mfma16(x * x, d1, acc1[t]);
+        for (int h = 0; h < H; h++) {
+            acc0[t][h] = (floatx4){0.f, 0.f, 0.f, 0.f};
+            acc1[t][h] = (floatx4){0.f, 0.f, 0.f, 0.f};
+        }
+
+    // Two register stages used in turn, as in the forward kernel.
+    float4 st[2][STAGE];
+    auto load = [&](float4(&x)[STAGE], int r) {
+#pragma unroll
+        for (int u = 0; u < STAGE; u++)
+            x[u] = ld4(w + (size_t)min(n_begin + r + u, n_last) * K);
+    };
+    auto multiply = [&](const float4(&cur)[STAGE], int r) {
+#pragma unroll
+        for (int g = 0; g < STAGE / 4; g++) {
+            float4 dm[H], dv[H];
+#pragma unroll
+            for (int h = 0; h < H; h++) {
+                dm[h] = *reinterpret_cast<const float4 *>(s_dm + (j + 4 * h) * S + r + 4 * g);
+                dv[h] = *reinterpret_cast<const float4 *>(s_dv + (j + 4 * h) * S + r + 4 * g);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const float4 x = cur[4 * g + u];
+                const float4 q = make_float4(x.x * x.x, x.y * x.y, x.z * x.z, x.w * x.w);
+#pragma unroll
+                for (int t = 0; t < 4; t++)
+#pragma unroll
+                    for (int h = 0; h < H; h++) {
+                        acc0[t][h] = mfma4(comp(x, t), comp(dm[h], u), acc0[t][h]);
+                        acc1[t][h] = mfma4(comp(q, t), comp(dv[h], u), acc1[t][h]);
+                    }
             }
         }
-        cur = nxt;
+    };
+
+    load(st[0], r_lo);
+    __syncthreads();
+    for (int r = r_lo; r < r_hi; r += 2 * STAGE) {
+        load(st[1], r + STAGE);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(st[0], r);
+        __builtin_amdgcn_sched_barrier(0);
+        load(st[0], r + 2 * STAGE);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(st[1], r + STAGE);
+        __builtin_amdgcn_sched_barrier(0);
     }
 
-    // D_t[i][j]: lane (j = l%16, q = l/16), register v -> i = 4q + v, i.e. column
-    // c0 + 16q + 4v + t: 16 consecutive columns per lane.
-    const int j = lane & 15, q = lane >> 4;
-    if (j < B) {
-        const size_t base = ((size_t)split * B + j) * K + c0 + 16 * q;
+    // tree reduction over the 8 waves through LDS (reusing the staging area):
+    // slot layout [slot][value][lane]
+    constexpr int NV = 4 * H * 4 * 2;  // values per lane
+    __syncthreads();
+    float *slot = lds;
 #pragma unroll
-        for (int v = 0; v < 4; v++) {
-            if (c0 + 16 * q + 4 * v < K) {  // K % 4 == 0 on this path
-                *reinterpret_cast<float4 *>(ws0 + base + 4 * v) =
-                    make_float4(acc0[0][v], acc0[1][v], acc0[2][v], acc0[3][v]);
-                *reinterpret_cast<float4 *>(ws1 + base + 4 * v) =
-                    make_float4(acc1[0][v], acc1[1][v], acc1[2][v], acc1[3][v]);
+    for (int half = DZ_WAVES / 2; half >= 1; half >>= 1) {
+        if (wave >= half && wave < 2 * half) {
+            float *dst = slot + (size_t)(wave - half) * NV * 64 + lane;
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+#pragma unroll
+                for (int h = 0; h < H; h++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        dst[((t * H + h) * 4 + v) * 2 * 64] = acc0[t][h][v];
+                        dst[(((t * H + h) * 4 + v) * 2 + 1) * 64] = acc1[t][h][v];
+                    }
+        }
+        __syncthreads();
+        if (wave < half) {
+            const float *src = slot + (size_t)wave * NV * 64 + lane;
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+#pragma unroll
+                for (int h = 0; h < H; h++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        acc0[t][h][v] += src[((t * H + h) * 4 + v) * 2 * 64];
+                        acc1[t][h][v] += src[(((t * H + h) * 4 + v) * 2 + 1) * 64];
+                    }
+        }
+        __syncthreads();
+    }
+
+    if (wave == 0) {
+        const int blk = lane >> 2;
+        const int c = blockIdx.x * DZ_COLS_PER_BLOCK + 16 * blk;
+#pragma unroll
+        for (int h = 0; h < H; h++) {
+            const int b = j + 4 * h;
+            if (b >= B) continue;
+            const size_t base = ((size_t)split * B + b) * K + c;
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                if (c + 4 * v < K) {  // K % 4 == 0 on this path
+                    *reinterpret_cast<float4 *>(ws0 + base + 4 * v) = make_float4(
+                        acc0[0][h][v], acc0[1][h][v], acc0[2][h][v], acc0[3][h][v]);
+                    *reinterpret_cast<float4 *>(ws1 + base + 4 * v) = make_float4(
+                        acc1[0][h][v], acc1[1][h][v], acc1[2][h][v], acc1[3][h][v]);
+                }
             }
         }
     }
@@ -257,18 +439,74 @@ __global__ __launch_bounds__(256) void gemv_dw_kernel(
 }  // namespace
 
 int gemv_fwd_rows_per_block() { return FWD_ROWS_PER_BLOCK; }
-int gemv_fwd_k_step() { return FWD_KSTEP; }
+int gemv_fwd_k_step() { return FWD_KROUND; }
 int gemv_dz_cols_per_block() { return DZ_COLS_PER_BLOCK; }
 int gemv_dz_n_step() { return DZ_NSTEP; }
 
+// Largest reduction slice whose staged activations / innovations fit in LDS.
+int gemv_fwd_max_slice(int B) {
+    const int H = (B + 3) / 4;
+    return (72 * 1024 / (2 * 4 * H * 4) - FWD_LDS_PAD) / FWD_KROUND * FWD_KROUND;
+}
+int gemv_dz_max_slice(int B) {
+    const int H = (B + 3) / 4;
+    return (72 * 1024 / (2 * 4 * H * 4) - 4) / DZ_NSTEP * DZ_NSTEP;
+}
+
+template <int H>
+static hipError_t fwd_launch(const float *mu_w, const float *var_w, const float *mu_a,
+                             const float *var_a, int K, int N, int B, int per, int splits,
+                             int swz, float *ws0, float *ws1, hipStream_t stream) {
+    const size_t lds = (size_t)2 * 4 * H * (per + FWD_LDS_PAD) * sizeof(float);
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_fwd_kernel<H>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    dim3 grid(((N + FWD_ROWS_PER_BLOCK - 1) / FWD_ROWS_PER_BLOCK) * splits), block(FWD_WAVES * 64);
+    hipLaunchKernelGGL(gemv_fwd_kernel<H>, grid, block, lds, stream, mu_w, var_w, mu_a, var_a, K, N,
+                       B, per, splits, swz, ws0, ws1);
+    return hipGetLastError();
+}
+
 hipError_t launch_gemv_fwd(const float *mu_w, const float *var_w, const float *mu_a,
-                           const float *var_a, int K, int N, int B, int splits, float *ws0,
-                           float *ws1, hipStream_t stream) {
+                           const float *var_a, int K, int N, int B, int splits, int swz,
+                           float *ws0, float *ws1, hipStream_t stream) {
     int per = (K + splits - 1) / splits;
-    per = (per + FWD_KSTEP - 1) / FWD_KSTEP * FWD_KSTEP;
-    dim3 grid((N + FWD_ROWS_PER_BLOCK - 1) / FWD_ROWS_PER_BLOCK, splits), block(256);
-    hipLaunchKernelGGL(gemv_fwd_kernel, grid, block, 0, stream, mu_w, var_w, mu_a, var_a, K, N, B,
-                       per, ws0, ws1);
+    per = (per + FWD_KROUND - 1) / FWD_KROUND * FWD_KROUND;
+    if (per > gemv_fwd_max_slice(B)) return hipErrorInvalidValue;
+    switch ((B + 3) / 4) {
+        case 1: return fwd_launch<1>(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1,
+                                       stream);
+        case 2: return fwd_launch<2>(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1,
+                                       stream);
+        case 3: return fwd_launch<3>(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1,
+                                       stream);
+        case 4: return fwd_launch<4>(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1,
+                                       stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+template <int H>
+static hipError_t dz_launch(const float *mu_w, const float *dmu, const float *dvar, int K, int N,
+                            int B, int per, int splits, float *ws0, float *ws1,
+                            hipStream_t stream) {
+    size_t lds = (size_t)2 * 4 * H * (per + 4) * sizeof(float);
+    const size_t red = (size_t)(DZ_WAVES / 2) * (4 * H * 4 * 2) * 64 * sizeof(float);
+    if (red > lds) lds = red;
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_dz_kernel<H>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    dim3 grid((K + DZ_COLS_PER_BLOCK - 1) / DZ_COLS_PER_BLOCK, splits), block(DZ_WAVES * 64);
+    hipLaunchKernelGGL(gemv_dz_kernel<H>, grid, block, lds, stream, mu_w, dmu, dvar, K, N, B, per,
+                       ws0, ws1);
     return hipGetLastError();
 }
 
@@ -276,10 +514,14 @@ hipError_t launch_gemv_dz(const float *mu_w, const float *dmu, const float *dvar
                           int B, int splits, float *ws0, float *ws1, hipStream_t stream) {
     int per = (N + splits - 1) / splits;
     per = (per + DZ_NSTEP - 1) / DZ_NSTEP * DZ_NSTEP;
-    dim3 grid((K + DZ_COLS_PER_BLOCK - 1) / DZ_COLS_PER_BLOCK, splits), block(256);
-    hipLaunchKernelGGL(gemv_dz_kernel, grid, block, 0, stream, mu_w, dmu, dvar, K, N, B, per, ws0,
-                       ws1);
-    return hipGetLastError();
+    if (per > gemv_dz_max_slice(B)) return hipErrorInvalidValue;
+    switch ((B + 3) / 4) {
+        case 1: return dz_launch<1>(mu_w, dmu, dvar, K, N, B, per, splits, ws0, ws1, stream);
+        case 2: return dz_launch<2>(mu_w, dmu, dvar, K, N, B, per, splits, ws0, ws1, stream);
+        case 3: return dz_launch<3>(mu_w, dmu, dvar, K, N, B, per, splits, ws0, ws1, stream);
+        case 4: return dz_launch<4>(mu_w, dmu, dvar, K, N, B, per, splits, ws0, ws1, stream);
+    }
+    return hipErrorInvalidValue;
 }
 
 hipError_t launch_gemv_dw(const float *var_w, const float *mu_a, const float *dmu,

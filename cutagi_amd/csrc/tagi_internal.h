@@ -51,7 +51,7 @@ hipError_t launch_reduce_splits(Epilogue epi, const float *ws0, const float *ws1
 // Skinny-batch (B <= 16) streaming kernels: weights are read once from HBM
 // straight into MFMA operand layout, nothing is staged in LDS.
 hipError_t launch_gemv_fwd(const float *mu_w, const float *var_w, const float *mu_a,
-                           const float *var_a, int K, int N, int B, int splits,
+                           const float *var_a, int K, int N, int B, int splits, int swz,
                            float *ws0, float *ws1, hipStream_t stream);
 hipError_t launch_gemv_dz(const float *mu_w, const float *dmu, const float *dvar, int K,
                           int N, int B, int splits, float *ws0, float *ws1,
@@ -63,6 +63,8 @@ int gemv_fwd_rows_per_block();
 int gemv_fwd_k_step();
 int gemv_dz_cols_per_block();
 int gemv_dz_n_step();
+int gemv_fwd_max_slice(int B);  // longest reduction slice whose activations fit in LDS
+int gemv_dz_max_slice(int B);
 
 // Elementwise / small kernels
 hipError_t launch_bias_delta(const float *var_b, const float *dmu, const float *dvar, int N,
