@@ -11,18 +11,20 @@ inline unsigned blocks_for(size_t n, int per_block) {
     return (unsigned)((n + per_block - 1) / per_block);
 }
 
-// delta_b[n] = var_b[n] * sum_b delta[b][n]. Block = 64 columns x 4 batch
-// slices; consecutive lanes read consecutive columns, the 4 slices meet in LDS.
-__global__ __launch_bounds__(TPB) void bias_delta_kernel(
+// delta_b[n] = var_b[n] * sum_b delta[b][n]. Block = 64 columns x 16 batch
+// slices (one wave each): consecutive lanes read consecutive columns, the slices
+// meet in LDS and are folded in a fixed order.
+constexpr int BIAS_SLICES = 16;
+__global__ __launch_bounds__(64 * BIAS_SLICES) void bias_delta_kernel(
     const float *__restrict__ var_b, const float *__restrict__ dmu,
     const float *__restrict__ dvar, int N, int B, float *__restrict__ dmu_b,
     float *__restrict__ dvar_b) {
-    __shared__ float s0[4][64], s1[4][64];
+    __shared__ float s0[BIAS_SLICES][64], s1[BIAS_SLICES][64];
     const int c = threadIdx.x & 63, slice = threadIdx.x >> 6;
     const int n = blockIdx.x * 64 + c;
     float a0 = 0.f, a1 = 0.f;
     if (n < N) {
-        for (int b = slice; b < B; b += 4) {
+        for (int b = slice; b < B; b += BIAS_SLICES) {
             a0 += dmu[(size_t)b * N + n];
             a1 += dvar[(size_t)b * N + n];
         }
@@ -31,8 +33,12 @@ __global__ __launch_bounds__(TPB) void bias_delta_kernel(
     s1[slice][c] = a1;
     __syncthreads();
     if (slice == 0 && n < N) {
-        const float m = (s0[0][c] + s0[1][c]) + (s0[2][c] + s0[3][c]);
-        const float v = (s1[0][c] + s1[1][c]) + (s1[2][c] + s1[3][c]);
+        float m = 0.f, v = 0.f;
+#pragma unroll
+        for (int s = 0; s < BIAS_SLICES; s++) {
+            m += s0[s][c];
+            v += s1[s][c];
+        }
         const float vb = var_b[n];
         dmu_b[n] = m * vb;
         dvar_b[n] = v * vb * vb;
@@ -129,7 +135,7 @@ __global__ __launch_bounds__(TPB) void relu_kernel(const float *mu_z, const floa
 
 hipError_t launch_bias_delta(const float *var_b, const float *dmu, const float *dvar, int N,
                              int B, float *dmu_b, float *dvar_b, hipStream_t stream) {
-    hipLaunchKernelGGL(bias_delta_kernel, dim3(blocks_for(N, 64)), dim3(TPB), 0, stream, var_b,
+    hipLaunchKernelGGL(bias_delta_kernel, dim3(blocks_for(N, 64)), dim3(64 * BIAS_SLICES), 0, stream, var_b,
                        dmu, dvar, N, B, dmu_b, dvar_b);
     return hipGetLastError();
 }

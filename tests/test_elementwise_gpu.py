@@ -1,0 +1,93 @@
+"""Parity of the small kernels (update, output updater, ReLU, state bookkeeping)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _t(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+@pytest.mark.parametrize("cap", [0.1, 2.0, 3.0])
+def test_param_update(oracle_lib, cap):
+    import torch
+    import cutagi_amd.functional as F
+    rng = np.random.default_rng(int(cap * 10))
+    n = 100003
+    mu = rng.normal(0, 1, n).astype(np.float32)
+    var = rng.uniform(1e-4, 1, n).astype(np.float32)
+    dmu = rng.normal(0, 1, n).astype(np.float32)
+    dvar = rng.normal(0, 0.5, n).astype(np.float32)
+    dmu[::7] = 0.0
+    dvar[::11] = 0.0
+    ref_mu, ref_var, ref_cnt = oracle_lib.param_update(mu, var, dmu, dvar, cap)
+    t_mu, t_var = _t(mu), _t(var)
+    cnt = torch.zeros(1, dtype=torch.int32, device="cuda")
+    F.param_update(_t(dmu), _t(dvar), cap, t_mu, t_var, cnt)
+    # identical up to the last bit of sqrt/divide; the clamp decisions must agree
+    np.testing.assert_allclose(t_mu.cpu().numpy(), ref_mu, rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(t_var.cpu().numpy(), ref_var, rtol=1e-6, atol=1e-7)
+    assert int(cnt.item()) == ref_cnt
+    assert ref_cnt > 0 or cap > 1.0
+    assert float(t_var.min()) > 0.0
+
+
+def test_out_update_dense_and_indexed(oracle_lib):
+    import torch
+    import cutagi_amd.functional as F
+    rng = np.random.default_rng(5)
+    B, n_obs, n_enc = 32, 11, 4
+    mu_a = rng.normal(0, 1, B * n_obs).astype(np.float32)
+    var_a = rng.uniform(0.1, 1, B * n_obs).astype(np.float32)
+    jcb = np.ones(B * n_obs, np.float32)
+    # dense
+    obs = rng.normal(0, 1, B * n_obs).astype(np.float32)
+    obs[5] = np.nan
+    var_obs = np.ones(B * n_obs, np.float32)
+    var_obs[9] = -var_a[9]  # division by zero -> inf -> zeroed
+    z = np.zeros(B * n_obs, np.float32)
+    ref = oracle_lib.out_update_dense(mu_a, var_a, jcb, obs, var_obs, z, z)
+    dm, dv = _t(z), _t(z)
+    F.out_update_dense(_t(mu_a), _t(var_a), _t(jcb), _t(obs), _t(var_obs), dm, dv)
+    np.testing.assert_allclose(dm.cpu().numpy(), ref[0], rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(dv.cpu().numpy(), ref[1], rtol=1e-6, atol=1e-7)
+    assert ref[0][5] == 0 and ref[0][9] == 0
+    # indexed: 4 distinct 1-based positions per sample
+    sel = np.concatenate([rng.choice(n_obs, n_enc, replace=False) + 1 for _ in range(B)]).astype(np.int32)
+    y = rng.normal(0, 1, B * n_enc).astype(np.float32)
+    vy = np.ones(B * n_enc, np.float32)
+    ref = oracle_lib.out_update_indexed(mu_a, var_a, jcb, y, vy, sel, n_obs, n_enc, z, z)
+    dm, dv = _t(z), _t(z)
+    F.out_update_indexed(_t(mu_a), _t(var_a), _t(jcb), _t(y), _t(vy), _t(sel), n_obs, n_enc, dm, dv)
+    np.testing.assert_allclose(dm.cpu().numpy(), ref[0], rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(dv.cpu().numpy(), ref[1], rtol=1e-6, atol=1e-7)
+    assert np.count_nonzero(ref[0]) == B * n_enc
+
+
+def test_relu_and_store_states(oracle_lib):
+    import torch
+    import cutagi_amd.functional as F
+    rng = np.random.default_rng(6)
+    n = 5000
+    mu_z = rng.normal(0, 1, n).astype(np.float32)
+    mu_z[::13] = 0.0
+    var_z = rng.uniform(0.1, 1, n).astype(np.float32)
+    ref = oracle_lib.relu_fwd(mu_z, var_z)
+    got = F.relu_fwd(_t(mu_z), _t(var_z))
+    for g, r in zip(got, ref):
+        assert np.array_equal(g.cpu().numpy(), r)
+    # in place
+    a, v = _t(mu_z), _t(var_z)
+    j = torch.empty_like(a)
+    F.relu_fwd(a, v, a, j, v)
+    assert np.array_equal(a.cpu().numpy(), ref[0]) and np.array_equal(v.cpu().numpy(), ref[1])
+    # store_states: copies the first n_in entries and resets the output Jacobian
+    mu_a, jcb = _t(mu_z), _t(var_z)
+    bm, bj = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+    oj = torch.zeros(2 * n, device="cuda")
+    F.store_states(mu_a, jcb, 3000, bm, bj, oj, 7000)
+    assert torch.equal(bm[:3000], mu_a[:3000]) and float(bm[3000:].abs().max()) == 0.0
+    assert torch.equal(bj[:3000], jcb[:3000])
+    assert float(oj[:7000].min()) == 1.0 and float(oj[7000:].max()) == 0.0
