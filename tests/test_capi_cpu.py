@@ -1,0 +1,65 @@
+"""The C-ABI library without a GPU: it loads, exports every function the header
+declares, and its host-only entry points and argument checks behave."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "tagi_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tagi_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from cutagi_amd import capi
+    names = _declared()
+    assert len(names) >= 20
+    for n in names:
+        assert hasattr(capi.lib, n), "missing export: " + n
+        assert n in capi.SIGNATURES, "binding missing for: " + n
+    assert sorted(capi.SIGNATURES) == names
+    assert capi.version() == 100
+
+
+def test_error_strings_and_device_count():
+    from cutagi_amd import capi
+    assert capi.lib.tagi_hip_error_string(0) == b"ok"
+    assert b"invalid" in capi.lib.tagi_hip_error_string(capi.ERR_INVALID_ARG)
+    assert capi.device_count() >= 0
+
+
+def test_null_and_bad_sizes_are_rejected_before_any_launch():
+    from cutagi_amd import capi
+    L = capi.lib
+    one = ctypes.c_void_p(16)  # never dereferenced: the size check fires first
+    assert L.tagi_linear_fwd(None, one, one, one, one, one, 4, 4, 4, 1, one, one, None) == capi.ERR_INVALID_ARG
+    assert L.tagi_linear_fwd(one, one, one, one, one, one, 0, 4, 4, 1, one, one, None) == capi.ERR_INVALID_ARG
+    assert L.tagi_linear_fwd(one, one, None, None, one, one, 4, 4, 4, 1, one, one, None) == capi.ERR_INVALID_ARG
+    assert L.tagi_linear_bwd_dz(one, one, one, one, 4, -1, 4, one, one, None) == capi.ERR_INVALID_ARG
+    assert L.tagi_linear_bwd_dw(one, one, one, None, 4, 4, 4, one, one, None) == capi.ERR_INVALID_ARG
+    assert L.tagi_param_update(one, one, 0.0, 4, one, one, None, None) == capi.ERR_INVALID_ARG
+    assert L.tagi_hip_tune(b"no.such.key", 1) == capi.ERR_INVALID_ARG
+    with pytest.raises(capi.TagiHipError):
+        capi.check(capi.ERR_INVALID_ARG)
+
+
+def test_host_only_entry_points(oracle_lib):
+    from cutagi_amd import capi
+    for b in (-1, 0, 1, 2, 255, 256, 5000):
+        assert capi.cap_factor(b, 1.25) == pytest.approx(oracle_lib.cap_factor(b, 1.25))
+    assert capi.conv2d_out_size(3, 1, 32, 32, 1, 1) == (32, 32)
+    assert capi.conv2d_out_size(3, 2, 32, 32, 1, 2) == (16, 16)
+    assert capi.conv2d_out_size(2, 2, 32, 32, 0, 1) == (16, 16)
+    with pytest.raises(capi.TagiHipError):   # stride does not divide: the reference throws
+        capi.conv2d_out_size(3, 2, 8, 8, 0, 1)
+    a = capi.conv2d_build_idx(3, 1, 32, 32, 1, 1, 64 * 64 * 9 + 1)
+    b = oracle_lib.conv2d_build_idx(3, 1, 32, 32, 1, 1, 64 * 64 * 9 + 1)
+    for key in ("Fmwa_2", "FCzwa_1", "Szz_ud", "w", "h"):
+        assert np.array_equal(a[key], b[key])
+    assert (a["w"], a["h"]) == (1024, 9)

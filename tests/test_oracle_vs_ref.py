@@ -1,0 +1,103 @@
+"""The CPU oracle against the reference's own sources compiled in place
+(oracle/_ref, built by `make -C oracle ref` where the reference tree is mounted):
+bit-for-bit on seeded inputs, serial and threaded. Skipped where that library
+does not exist."""
+import numpy as np
+import pytest
+
+from util import conv_inputs, linear_inputs
+
+
+@pytest.fixture(scope="module")
+def ref(ref_lib):
+    if ref_lib is None:
+        pytest.skip("oracle/_ref/libtagi_ref.so not built (no reference tree here)")
+    return ref_lib
+
+
+def _eq(a, b):
+    return all(np.array_equal(x, y, equal_nan=True) for x, y in zip(a, b))
+
+
+@pytest.mark.parametrize("K,N,B", [(5, 3, 2), (784, 128, 32), (129, 67, 9), (512, 256, 64),
+                                   (1000, 11, 7), (64, 64, 1)])
+@pytest.mark.parametrize("threads", [1, 4, 7])
+def test_linear(oracle_lib, ref, K, N, B, threads):
+    d = linear_inputs(K, N, B, seed=K + N + B + threads, jcb_random=True)
+    for bias in (True, False):
+        mb, vb = (d["mu_b"], d["var_b"]) if bias else (None, None)
+        assert _eq(oracle_lib.linear_fwd(d["mu_w"], d["var_w"], mb, vb, d["mu_a"], d["var_a"], threads),
+                   ref.linear_fwd(d["mu_w"], d["var_w"], mb, vb, d["mu_a"], d["var_a"], threads))
+    a = (d["mu_w"], d["jcb"], d["delta_mu"], d["delta_var"], threads)
+    assert _eq(oracle_lib.linear_bwd_dz(*a), ref.linear_bwd_dz(*a))
+    a = (d["var_w"], d["mu_a"], d["delta_mu"], d["delta_var"], threads)
+    assert _eq(oracle_lib.linear_bwd_dw(*a), ref.linear_bwd_dw(*a))
+    a = (d["var_b"], d["delta_mu"], d["delta_var"], threads)
+    assert _eq(oracle_lib.linear_bwd_db(*a), ref.linear_bwd_db(*a))
+
+
+GEOMS = [(k, s, p, pt, wi) for k in (1, 2, 3, 4, 5) for s in (1, 2) for p in (0, 1, 2)
+         for pt in (1, 2) for wi in (4, 7, 8, 12)]
+
+
+def test_index_tables_sweep(oracle_lib, ref):
+    """Every geometry both sides accept gives identical tables; both reject the
+    same geometries (the reference throws where the stride does not divide)."""
+    from cutagi_amd import capi
+    checked = 0
+    for g in GEOMS:
+        k, s, p, pt, wi = g
+        if k > wi:
+            continue
+        try:
+            b = ref.conv2d_build_idx(k, s, wi, wi, p, pt, 1234)
+        except ValueError:
+            with pytest.raises(ValueError):
+                oracle_lib.conv2d_build_idx(k, s, wi, wi, p, pt, 1234)
+            continue
+        a = oracle_lib.conv2d_build_idx(k, s, wi, wi, p, pt, 1234)
+        c = capi.conv2d_build_idx(k, s, wi, wi, p, pt, 1234)
+        for key in ("Fmwa_2", "FCzwa_1", "Szz_ud", "w", "h", "wo", "ho"):
+            assert np.array_equal(a[key], b[key]), (g, key)
+            assert np.array_equal(c[key], b[key]), (g, key, "product builder")
+        checked += 1
+    assert checked > 100
+
+
+@pytest.mark.parametrize("geom", [(3, 1, 1, 1, 8, 3, 4, 2), (3, 2, 1, 2, 8, 4, 6, 2),
+                                  (2, 2, 0, 1, 8, 4, 4, 3), (5, 1, 2, 1, 9, 2, 3, 1),
+                                  (3, 1, 1, 1, 16, 8, 8, 2), (4, 2, 1, 1, 10, 3, 5, 2)])
+@pytest.mark.parametrize("threads", [1, 3])
+def test_conv(oracle_lib, ref, geom, threads):
+    k, s, p, pt, wi, fi, fo, B = geom
+    idx = ref.conv2d_build_idx(k, s, wi, wi, p, pt, k * k * fi * fo + 1)
+    wihi, woho = wi * wi, idx["wo"] * idx["ho"]
+    d = conv_inputs(fi, fo, k, wihi, woho, B, seed=sum(geom) + threads, bias=True, jcb_random=True)
+    a = (d["mu_w"], d["var_w"], d["mu_b"], d["var_b"], d["mu_a"], d["var_a"], idx["Fmwa_2"], woho,
+         fo, wihi, fi, k, B, threads)
+    assert _eq(oracle_lib.conv2d_fwd(*a), ref.conv2d_fwd(*a))
+    a = (d["mu_w"], d["jcb"], d["delta_mu"], d["delta_var"], idx["FCzwa_1"], idx["Szz_ud"], woho,
+         fo, wihi, fi, k, idx["h"], B, threads)
+    assert _eq(oracle_lib.conv2d_bwd_dz(*a), ref.conv2d_bwd_dz(*a))
+    a = (d["var_w"], d["var_b"], d["mu_a"], d["delta_mu"], d["delta_var"], idx["Fmwa_2"], B, fo,
+         woho, wihi, fi, k, threads)
+    assert _eq(oracle_lib.conv2d_bwd_dw(*a), ref.conv2d_bwd_dw(*a))
+
+
+def test_update_output_relu(oracle_lib, ref):
+    rng = np.random.default_rng(3)
+    n = 20000
+    mu = rng.normal(0, 1, n).astype(np.float32)
+    var = rng.uniform(1e-5, 1, n).astype(np.float32)
+    dmu = rng.normal(0, 1, n).astype(np.float32)
+    dvar = rng.normal(0, 0.5, n).astype(np.float32)
+    for cap in (0.1, 2.0, 3.0):
+        for w in (True, False):
+            a = oracle_lib.param_update(mu, var, dmu, dvar, cap, w)
+            b = ref.param_update(mu, var, dmu, dvar, cap, w)
+            assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1]) and a[2] == b[2]
+    for bs in (-3, 0, 1, 2, 100, 255, 256, 100000):
+        assert oracle_lib.cap_factor(bs, 1.5) == ref.cap_factor(bs, 1.5)
+    m = rng.normal(0, 1, 999).astype(np.float32)
+    v = rng.uniform(0, 1, 999).astype(np.float32)
+    assert _eq(oracle_lib.relu_fwd(m, v), ref.relu_fwd(m, v))
