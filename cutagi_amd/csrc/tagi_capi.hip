@@ -57,6 +57,8 @@ struct Tuning {
     int tile = -1;
     int conv_dw_splits = -1;
     int gemv_swz = -1;
+    int gemv_fwd_variant = -1;
+    int gemv_rev = -1;  // bit 0: state backward, bit 1: weight backward walk rows from the end
 };
 Tuning g_tune;
 
@@ -175,6 +177,8 @@ int tagi_hip_tune(const char *key, int value) {
     else if (!strcmp(key, "linear.tile")) g_tune.tile = value;
     else if (!strcmp(key, "conv2d.dw.splits")) g_tune.conv_dw_splits = value;
     else if (!strcmp(key, "linear.gemv.swizzle")) g_tune.gemv_swz = value;
+    else if (!strcmp(key, "linear.gemv.fwd_variant")) g_tune.gemv_fwd_variant = value;
+    else if (!strcmp(key, "linear.gemv.reverse")) g_tune.gemv_rev = value;
     else return TAGI_ERR_INVALID_ARG;
     return TAGI_OK;
 }
@@ -197,7 +201,11 @@ int tagi_linear_fwd(const float *mu_w, const float *var_w, const float *mu_b, co
     if (B <= gemv_max_batch() && vec) {
         // slices: short enough for the LDS-resident activations, and enough of
         // them for about two workgroups per CU
-        const int blocks = ceil_div(N, gemv_fwd_rows_per_block());
+        const int variant = (g_tune.gemv_fwd_variant >= 0 &&
+                             g_tune.gemv_fwd_variant < gemv_fwd_variants())
+                                ? g_tune.gemv_fwd_variant
+                                : 0;
+        const int blocks = ceil_div(N, gemv_fwd_rows_per_block(variant));
         const int step = gemv_fwd_k_step();
         int splits = g_tune.fwd_splits > 0 ? g_tune.fwd_splits : ceil_div(2 * NUM_CU, blocks);
         const int max_splits = ceil_div(K, 4 * step);
@@ -211,7 +219,8 @@ int tagi_linear_fwd(const float *mu_w, const float *var_w, const float *mu_b, co
         int rc = workspace_get(2 * part * sizeof(float), &ws);
         if (rc != TAGI_OK) return rc;
         TAGI_TRY(launch_gemv_fwd(mu_w, var_w, mu_a, var_a, K, N, B, splits,
-                                 g_tune.gemv_swz >= 0 ? g_tune.gemv_swz : 3, ws, ws + part, stream));
+                                 g_tune.gemv_swz >= 0 ? g_tune.gemv_swz : 3, variant, ws,
+                                 ws + part, stream));
         TAGI_TRY(launch_reduce_splits(EPI_BIAS, ws, ws + part, splits, B, N, e0, e1, mu_z, var_z, N,
                                       stream));
         return TAGI_OK;
@@ -249,7 +258,9 @@ int tagi_linear_bwd_dz(const float *mu_w, const float *jcb, const float *delta_m
         const size_t part = (size_t)splits * B * K;
         int rc = workspace_get(2 * part * sizeof(float), &ws);
         if (rc != TAGI_OK) return rc;
-        TAGI_TRY(launch_gemv_dz(mu_w, delta_mu, delta_var, K, N, B, splits, ws, ws + part, stream));
+        TAGI_TRY(launch_gemv_dz(mu_w, delta_mu, delta_var, K, N, B, splits,
+                                (g_tune.gemv_rev >= 0 ? g_tune.gemv_rev : 0) & 1, ws, ws + part,
+                                stream));
         TAGI_TRY(launch_reduce_splits(EPI_SCALE, ws, ws + part, splits, B, K, jcb, nullptr,
                                       delta_mu_z, delta_var_z, K, stream));
         return TAGI_OK;
@@ -274,8 +285,9 @@ int tagi_linear_bwd_dw(const float *var_w, const float *mu_a, const float *delta
                        aligned16(delta_mu_w) && aligned16(delta_var_w);
 
     if (B <= gemv_max_batch() && k_vec) {
-        TAGI_TRY(launch_gemv_dw(var_w, mu_a, delta_mu, delta_var, K, N, B, delta_mu_w, delta_var_w,
-                                stream));
+        TAGI_TRY(launch_gemv_dw(var_w, mu_a, delta_mu, delta_var, K, N, B,
+                                ((g_tune.gemv_rev >= 0 ? g_tune.gemv_rev : 0) >> 1) & 1,
+                                delta_mu_w, delta_var_w, stream));
         return TAGI_OK;
     }
 

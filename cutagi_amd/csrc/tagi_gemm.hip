@@ -78,7 +78,7 @@ struct LinearProblem {
 };
 
 template <int EPI, bool VEC>
-__global__ __launch_bounds__(256) void reduce_splits_kernel(const float *__restrict__ ws0,
+__global__ __launch_bounds__(64) void reduce_splits_kernel(const float *__restrict__ ws0,
                                                             const float *__restrict__ ws1,
                                                             int splits, int M, int N,
                                                             const float *__restrict__ e0,
@@ -92,6 +92,9 @@ __global__ __launch_bounds__(256) void reduce_splits_kernel(const float *__restr
     float s0[W], s1[W];
 #pragma unroll
     for (int c = 0; c < W; c++) s0[c] = s1[c] = 0.f;
+    // slices are folded in index order (deterministic); the unroll keeps several
+    // slices' loads in flight
+#pragma unroll 8
     for (int s = 0; s < splits; s++) {
         if constexpr (VEC) {
             const float4 a = *reinterpret_cast<const float4 *>(ws0 + s * total + idx);
@@ -158,7 +161,7 @@ hipError_t launch_reduce_splits(Epilogue epi, const float *ws0, const float *ws1
     const bool vec = (N % 4 == 0) && (ldo % 4 == 0) && al(ws0) && al(ws1) && al(out0) &&
                      al(out1) && (epi == EPI_BIAS || al(e0));
     const size_t items = vec ? total / 4 : total;
-    dim3 grid((unsigned)((items + 255) / 256)), block(256);
+    dim3 grid((unsigned)((items + 63) / 64)), block(64);
     if (epi == EPI_BIAS) {
         if (vec)
             hipLaunchKernelGGL((reduce_splits_kernel<EPI_BIAS, true>), grid, block, 0, stream, ws0,

@@ -42,22 +42,24 @@ __device__ __forceinline__ float comp(const float4 &v, int t) {
 // slice is finished.
 // ---------------------------------------------------------------------------
 constexpr int FWD_WAVES = 8;
-constexpr int FWD_RG = 2;                                  // row groups of 4 per wave
-constexpr int FWD_ROWS_PER_BLOCK = FWD_WAVES * FWD_RG * 4;  // 64
-constexpr int FWD_KSTEP = 64;   // reduction elements per register stage
-constexpr int FWD_KROUND = 2 * FWD_KSTEP;  // slices are whole pairs of stages
-constexpr int FWD_LDS_PAD = 8;  // row stride % 32 == 8: conflict-free 16-byte reads
+constexpr int FWD_KCHUNK = 64;    // reduction elements one load instruction covers per row
+constexpr int FWD_KROUND = 512;   // slices are multiples of this (two stages of any variant)
+constexpr int FWD_LDS_PAD = 8;    // row stride % 32 == 8: conflict-free 16-byte reads
 
 __device__ __forceinline__ floatx4 mfma4(float a, float b, floatx4 c) {
     return __builtin_amdgcn_mfma_f32_4x4x1f32(a, b, c, 0, 0, 0);
 }
 
-template <int H>
+// H: groups of 4 samples; RG: groups of 4 rows per wave; C: 64-element chunks per
+// row and register stage (a stage holds RG*C float4 of each weight array).
+template <int H, int RG, int C>
 __global__ __launch_bounds__(FWD_WAVES * 64) void gemv_fwd_kernel(
     const float *__restrict__ mu_w, const float *__restrict__ var_w,
     const float *__restrict__ mu_a, const float *__restrict__ var_a, int K, int N, int B,
     int k_per_split, int splits, int swz, float *__restrict__ ws0, float *__restrict__ ws1) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
+    constexpr int ROWS_PER_BLOCK = FWD_WAVES * RG * 4;
+    constexpr int KSTEP = FWD_KCHUNK * C;  // reduction elements per register stage
     const int S = k_per_split + FWD_LDS_PAD;  // LDS row stride
     float *s_mu = lds, *s_var = lds + 4 * H * S;
 
@@ -65,8 +67,8 @@ __global__ __launch_bounds__(FWD_WAVES * 64) void gemv_fwd_kernel(
     const int blk = lane >> 2, i = lane & 3;
     // Workgroup -> (row block, reduction slice). Workgroups are handed to the 8
     // XCDs round-robin; with the slice as the fast index inside an XCD, the
-    // workgroups resident on one XCD cover all slices (all 4 KB windows of a
-    // weight row) instead of crowding into one.
+    // workgroups resident on one XCD cover all slices (all windows of a weight
+    // row) instead of crowding into one.
     int row_block, split;
     const int id = blockIdx.x, row_blocks = gridDim.x / splits;
     if ((swz & 1) && row_blocks % 8 == 0) {
@@ -80,7 +82,7 @@ __global__ __launch_bounds__(FWD_WAVES * 64) void gemv_fwd_kernel(
     const int k_begin = split * k_per_split;
     const int kr = min(K, k_begin + k_per_split) - k_begin;  // this slice's length
     // each wave walks its slice from a different starting point (sums commute)
-    const int rot = (swz & 2) ? ((row_block * FWD_WAVES + wave) * FWD_KROUND) % k_per_split : 0;
+    const int rot = (swz & 2) ? ((row_block * FWD_WAVES + wave) * 2 * KSTEP) % k_per_split : 0;
 
     // stage the slice of the activations: [sample][k], zero beyond B and kr
     const int k4s = k_per_split / 4;
@@ -99,19 +101,19 @@ __global__ __launch_bounds__(FWD_WAVES * 64) void gemv_fwd_kernel(
     // makes the compiler wait for every outstanding load): rows beyond N read row
     // N-1 and are dropped at the end, reduction elements beyond the slice read the
     // last float4 of the row and meet zero activations.
-    const int n0 = row_block * FWD_ROWS_PER_BLOCK + wave * (FWD_RG * 4);
-    const float *wm[FWD_RG], *wv[FWD_RG];
+    const int n0 = row_block * ROWS_PER_BLOCK + wave * (RG * 4);
+    const float *wm[RG], *wv[RG];
 #pragma unroll
-    for (int rg = 0; rg < FWD_RG; rg++) {
+    for (int rg = 0; rg < RG; rg++) {
         const int row = min(n0 + 4 * rg + i, N - 1);
         wm[rg] = mu_w + (size_t)row * K;
         wv[rg] = var_w + (size_t)row * K;
     }
     const int k_lane = k_begin + 4 * blk, k_last = K - 4;
 
-    floatx4 acc0[FWD_RG][H], acc1[FWD_RG][H];
+    floatx4 acc0[RG][H], acc1[RG][H];
 #pragma unroll
-    for (int rg = 0; rg < FWD_RG; rg++)
+    for (int rg = 0; rg < RG; rg++)
 #pragma unroll
         for (int h = 0; h < H; h++) {
             acc0[rg][h] = (floatx4){0.f, 0.f, 0.f, 0.f};
@@ -120,64 +122,71 @@ __global__ __launch_bounds__(FWD_WAVES * 64) void gemv_fwd_kernel(
 
     // Two register stages used in turn (no copies between them, so a stage's
     // loads stay in flight while the other stage is multiplied).
-    float4 am_[2][FWD_RG], av_[2][FWD_RG];
-    auto load = [&](float4(&m)[FWD_RG], float4(&v)[FWD_RG], int kb) {
-        const int k = min(k_lane + kb, k_last);
+    float4 sm[2][RG][C], sv[2][RG][C];
+    auto load = [&](float4(&m)[RG][C], float4(&v)[RG][C], int kb) {
 #pragma unroll
-        for (int rg = 0; rg < FWD_RG; rg++) {
-            m[rg] = ld4(wm[rg] + k);
-            v[rg] = ld4(wv[rg] + k);
+        for (int c = 0; c < C; c++) {
+            const int k = min(k_lane + kb + FWD_KCHUNK * c, k_last);
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) {
+                m[rg][c] = ld4(wm[rg] + k);
+                v[rg][c] = ld4(wv[rg] + k);
+            }
         }
     };
-    auto multiply = [&](const float4(&cm)[FWD_RG], const float4(&cv)[FWD_RG], int kb) {
-        float4 am[H], as[H], av[H];
+    auto multiply = [&](const float4(&cm)[RG][C], const float4(&cv)[RG][C], int kb) {
 #pragma unroll
-        for (int h = 0; h < H; h++) {
-            am[h] = *reinterpret_cast<const float4 *>(s_mu + (i + 4 * h) * S + kb + 4 * blk);
-            av[h] = *reinterpret_cast<const float4 *>(s_var + (i + 4 * h) * S + kb + 4 * blk);
-            as[h] = make_float4(av[h].x + am[h].x * am[h].x, av[h].y + am[h].y * am[h].y,
-                                av[h].z + am[h].z * am[h].z, av[h].w + am[h].w * am[h].w);
-        }
+        for (int c = 0; c < C; c++) {
+            float4 am[H], as[H], av[H];
+            const int at = kb + FWD_KCHUNK * c + 4 * blk;
 #pragma unroll
-        for (int rg = 0; rg < FWD_RG; rg++) {
-            const float4 q = make_float4(cm[rg].x * cm[rg].x, cm[rg].y * cm[rg].y,
-                                         cm[rg].z * cm[rg].z, cm[rg].w * cm[rg].w);
+            for (int h = 0; h < H; h++) {
+                am[h] = *reinterpret_cast<const float4 *>(s_mu + (i + 4 * h) * S + at);
+                av[h] = *reinterpret_cast<const float4 *>(s_var + (i + 4 * h) * S + at);
+                as[h] = make_float4(av[h].x + am[h].x * am[h].x, av[h].y + am[h].y * am[h].y,
+                                    av[h].z + am[h].z * am[h].z, av[h].w + am[h].w * am[h].w);
+            }
 #pragma unroll
-            for (int t = 0; t < 4; t++)
+            for (int rg = 0; rg < RG; rg++) {
+                const float4 w = cm[rg][c], u = cv[rg][c];
+                const float4 q = make_float4(w.x * w.x, w.y * w.y, w.z * w.z, w.w * w.w);
 #pragma unroll
-                for (int h = 0; h < H; h++) {
-                    acc0[rg][h] = mfma4(comp(cm[rg], t), comp(am[h], t), acc0[rg][h]);
-                    acc1[rg][h] = mfma4(comp(cv[rg], t), comp(as[h], t), acc1[rg][h]);
-                    acc1[rg][h] = mfma4(comp(q, t), comp(av[h], t), acc1[rg][h]);
-                }
+                for (int t = 0; t < 4; t++)
+#pragma unroll
+                    for (int h = 0; h < H; h++) {
+                        acc0[rg][h] = mfma4(comp(w, t), comp(am[h], t), acc0[rg][h]);
+                        acc1[rg][h] = mfma4(comp(u, t), comp(as[h], t), acc1[rg][h]);
+                        acc1[rg][h] = mfma4(comp(q, t), comp(av[h], t), acc1[rg][h]);
+                    }
+            }
         }
     };
 
     // k_per_split is a multiple of two stages and the staged activations are zero
-    // beyond the slice, so the loop needs no tail handling; `pos` is the rotated
-    // position inside the slice.
-    const int span = (swz & 2) ? k_per_split : kr;
+    // beyond the slice, so the loop needs no tail handling; positions are inside
+    // the slice, rotated by `rot`.
+    const int span = (swz & 2) ? k_per_split : (kr + 2 * KSTEP - 1) / (2 * KSTEP) * (2 * KSTEP);
     auto wrap = [&](int p) { return p >= k_per_split ? p - k_per_split : p; };
-    load(am_[0], av_[0], rot);
+    load(sm[0], sv[0], rot);
     __syncthreads();
-    for (int kb = 0; kb < span; kb += 2 * FWD_KSTEP) {
-        const int p0 = wrap(rot + kb), p1 = p0 + FWD_KSTEP, p2 = wrap(p0 + 2 * FWD_KSTEP);
+    for (int kb = 0; kb < span; kb += 2 * KSTEP) {
+        const int p0 = wrap(rot + kb), p1 = p0 + KSTEP, p2 = wrap(p0 + 2 * KSTEP);
         // the barriers keep the scheduler from sinking a stage's loads below the
         // MFMAs they are meant to overlap
-        load(am_[1], av_[1], p1);
+        load(sm[1], sv[1], p1);
         __builtin_amdgcn_sched_barrier(0);
-        multiply(am_[0], av_[0], p0);
+        multiply(sm[0], sv[0], p0);
         __builtin_amdgcn_sched_barrier(0);
-        load(am_[0], av_[0], p2);
+        load(sm[0], sv[0], p2);
         __builtin_amdgcn_sched_barrier(0);
-        multiply(am_[1], av_[1], p1);
+        multiply(sm[1], sv[1], p1);
         __builtin_amdgcn_sched_barrier(0);
     }
 
     // sum the 16 blocks (lanes with equal l%4), then lanes 0..3 (sample j = l%4)
     // hold D[row n0+4*rg+v][sample j+4*h] in register v
 #pragma unroll
-    for (int rg = 0; rg < FWD_RG; rg++)
+    for (int rg = 0; rg < RG; rg++)
 #pragma unroll
         for (int h = 0; h < H; h++)
 #pragma unroll
@@ -197,7 +206,7 @@ __global__ __launch_bounds__(FWD_WAVES * 64) void gemv_fwd_kernel(
             const int b = i + 4 * h;
             if (b >= B) continue;
 #pragma unroll
-            for (int rg = 0; rg < FWD_RG; rg++)
+            for (int rg = 0; rg < RG; rg++)
 #pragma unroll
                 for (int v = 0; v < 4; v++) {
                     const int n = n0 + 4 * rg + v;
@@ -229,7 +238,7 @@ constexpr int DZ_NSTEP = DZ_WAVES * 2 * DZ_STAGE;  // slices: whole pairs of sta
 template <int H>
 __global__ __launch_bounds__(DZ_WAVES * 64) void gemv_dz_kernel(
     const float *__restrict__ mu_w, const float *__restrict__ dmu,
-    const float *__restrict__ dvar, int K, int N, int B, int n_per_split,
+    const float *__restrict__ dvar, int K, int N, int B, int n_per_split, int rev,
     float *__restrict__ ws0, float *__restrict__ ws1) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int S = n_per_split + 4;
@@ -240,7 +249,9 @@ __global__ __launch_bounds__(DZ_WAVES * 64) void gemv_dz_kernel(
     constexpr int STAGE = H <= 2 ? DZ_STAGE : DZ_STAGE / 2;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int j = lane & 3;
-    const int split = blockIdx.y;
+    // Row slices are walked from the end of the matrix: a forward pass that just
+    // ran left the last weight rows in the memory-side cache.
+    const int split = rev ? gridDim.y - 1 - blockIdx.y : blockIdx.y;
     const int n_begin = split * n_per_split;
     const int nr = min(N, n_begin + n_per_split) - n_begin;
 
@@ -379,21 +390,46 @@ __global__ __launch_bounds__(DZ_WAVES * 64) void gemv_dz_kernel(
 // Weight backward. delta_w[n][k'] = var_w[n][k'] * sum_b delta[b][n] * a[b][k'].
 // A lane keeps a[b][k'..k'+3] and its squares for all b in registers and walks
 // rows; the 2*B innovations of a row are wave-uniform and come from LDS as
-// broadcast reads. Per row a wave reads 1 KB of var_w and writes 2 KB.
+// broadcast reads. Per row a wave reads 1 KB of var_w and writes 2 KB
+// (non-temporal: the results are not read again by this kernel).
+//
+// EXACT (K % 256 == 0 and N % rows-per-block == 0): no predicate anywhere, and
+// the var_w rows move through two register stages of DW_STAGE rows used in turn,
+// so a stage's loads are in flight while the other stage is multiplied and
+// stored. The general variant guards every row and column.
 // ---------------------------------------------------------------------------
 constexpr int DW_COLS_PER_BLOCK = 256;  // 64 lanes x 4 columns, shared by the 4 waves
-constexpr int DW_ROWS_PER_BLOCK = 64;   // 16 rows per wave
+constexpr int DW_ROWS_PER_BLOCK = 128;  // 32 rows per wave
+constexpr int DW_STAGE = 4;
 
 template <int BMAX>
+__device__ __forceinline__ void dw_row(const float4 &vw, const float (*s_dm)[BMAX],
+                                       const float (*s_dv)[BMAX], int r, const float4 (&a)[BMAX],
+                                       const float4 (&a2)[BMAX], float *pm, float *pv) {
+    float4 sm = zero4(), sv = zero4();
+#pragma unroll
+    for (int b = 0; b < BMAX; b++) {
+        const float d0 = s_dm[r][b], d1 = s_dv[r][b];
+        sm.x += d0 * a[b].x; sm.y += d0 * a[b].y; sm.z += d0 * a[b].z; sm.w += d0 * a[b].w;
+        sv.x += d1 * a2[b].x; sv.y += d1 * a2[b].y; sv.z += d1 * a2[b].z; sv.w += d1 * a2[b].w;
+    }
+    const floatx4 om = {sm.x * vw.x, sm.y * vw.y, sm.z * vw.z, sm.w * vw.w};
+    const floatx4 ov = {sv.x * vw.x * vw.x, sv.y * vw.y * vw.y, sv.z * vw.z * vw.z,
+                        sv.w * vw.w * vw.w};
+    __builtin_nontemporal_store(om, reinterpret_cast<floatx4 *>(pm));
+    __builtin_nontemporal_store(ov, reinterpret_cast<floatx4 *>(pv));
+}
+
+template <int BMAX, bool EXACT>
 __global__ __launch_bounds__(256) void gemv_dw_kernel(
     const float *__restrict__ var_w, const float *__restrict__ mu_a,
-    const float *__restrict__ dmu, const float *__restrict__ dvar, int K, int N, int B,
+    const float *__restrict__ dmu, const float *__restrict__ dvar, int K, int N, int B, int rev,
     float *__restrict__ dmu_w, float *__restrict__ dvar_w) {
     __shared__ __attribute__((aligned(16))) float s_dm[DW_ROWS_PER_BLOCK][BMAX];
     __shared__ __attribute__((aligned(16))) float s_dv[DW_ROWS_PER_BLOCK][BMAX];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = blockIdx.x * DW_COLS_PER_BLOCK + lane * 4;
-    const int n0 = blockIdx.y * DW_ROWS_PER_BLOCK;
+    const int n0 = (rev ? gridDim.y - 1 - blockIdx.y : blockIdx.y) * DW_ROWS_PER_BLOCK;
 
     for (int e = threadIdx.x; e < DW_ROWS_PER_BLOCK * BMAX; e += 256) {
         const int b = e / DW_ROWS_PER_BLOCK, r = e % DW_ROWS_PER_BLOCK;
@@ -402,7 +438,7 @@ __global__ __launch_bounds__(256) void gemv_dw_kernel(
         s_dv[r][b] = ok ? dvar[(size_t)b * N + n0 + r] : 0.f;
     }
 
-    const bool col_ok = col < K;  // K % 4 == 0 on this path
+    const bool col_ok = EXACT || col < K;  // K % 4 == 0 on this path
     float4 a[BMAX], a2[BMAX];
 #pragma unroll
     for (int b = 0; b < BMAX; b++) {
@@ -410,35 +446,58 @@ __global__ __launch_bounds__(256) void gemv_dw_kernel(
         a2[b] = make_float4(a[b].x * a[b].x, a[b].y * a[b].y, a[b].z * a[b].z, a[b].w * a[b].w);
     }
     __syncthreads();
-    if (!col_ok) return;
 
     constexpr int RPW = DW_ROWS_PER_BLOCK / 4;
-#pragma unroll 4
-    for (int rr = 0; rr < RPW; rr++) {
-        const int r = wave * RPW + rr;
-        const int n = n0 + r;
-        if (n >= N) break;
-        const float4 vw = ld4(var_w + (size_t)n * K + col);
-        float4 sm = zero4(), sv = zero4();
+    const int r0 = wave * RPW;
+    if (EXACT) {
+        const float *src = var_w + (size_t)(n0 + r0) * K + col;
+        float *dm = dmu_w + (size_t)(n0 + r0) * K + col;
+        float *dv = dvar_w + (size_t)(n0 + r0) * K + col;
+        float4 st[2][DW_STAGE];
+        auto load = [&](float4(&x)[DW_STAGE], int rr) {
 #pragma unroll
-        for (int b = 0; b < BMAX; b++) {
-            const float d0 = s_dm[r][b], d1 = s_dv[r][b];
-            sm.x += d0 * a[b].x; sm.y += d0 * a[b].y; sm.z += d0 * a[b].z; sm.w += d0 * a[b].w;
-            sv.x += d1 * a2[b].x; sv.y += d1 * a2[b].y; sv.z += d1 * a2[b].z; sv.w += d1 * a2[b].w;
+            for (int u = 0; u < DW_STAGE; u++) x[u] = ld4(src + (size_t)(rr + u) * K);
+        };
+        auto flush = [&](const float4(&x)[DW_STAGE], int rr) {
+#pragma unroll
+            for (int u = 0; u < DW_STAGE; u++)
+                dw_row<BMAX>(x[u], s_dm, s_dv, r0 + rr + u, a, a2, dm + (size_t)(rr + u) * K,
+                             dv + (size_t)(rr + u) * K);
+        };
+        load(st[0], 0);
+#pragma unroll 1
+        for (int rr = 0; rr < RPW; rr += 2 * DW_STAGE) {
+            load(st[1], rr + DW_STAGE);
+            __builtin_amdgcn_sched_barrier(0);
+            flush(st[0], rr);
+            __builtin_amdgcn_sched_barrier(0);
+            // the last pair prefetches nothing new: re-reads its own first rows
+            load(st[0], rr + 2 * DW_STAGE < RPW ? rr + 2 * DW_STAGE : rr);
+            __builtin_amdgcn_sched_barrier(0);
+            flush(st[1], rr + DW_STAGE);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        float4 om = make_float4(sm.x * vw.x, sm.y * vw.y, sm.z * vw.z, sm.w * vw.w);
-        float4 ov = make_float4(sv.x * vw.x * vw.x, sv.y * vw.y * vw.y, sv.z * vw.z * vw.z,
-                                sv.w * vw.w * vw.w);
-        floatx4 *pm = reinterpret_cast<floatx4 *>(dmu_w + (size_t)n * K + col);
-        floatx4 *pv = reinterpret_cast<floatx4 *>(dvar_w + (size_t)n * K + col);
-        __builtin_nontemporal_store((floatx4){om.x, om.y, om.z, om.w}, pm);
-        __builtin_nontemporal_store((floatx4){ov.x, ov.y, ov.z, ov.w}, pv);
+    } else {
+        if (!col_ok) return;
+        for (int rr = 0; rr < RPW; rr++) {
+            const int n = n0 + r0 + rr;
+            if (n >= N) break;
+            const float4 vw = ld4(var_w + (size_t)n * K + col);
+            dw_row<BMAX>(vw, s_dm, s_dv, r0 + rr, a, a2, dmu_w + (size_t)n * K + col,
+                         dvar_w + (size_t)n * K + col);
+        }
     }
 }
 
 }  // namespace
 
-int gemv_fwd_rows_per_block() { return FWD_ROWS_PER_BLOCK; }
+// Forward variants (row groups per wave, chunks per stage), by index.
+constexpr int FWD_VARIANTS = 4;
+static const int kFwdRG[FWD_VARIANTS] = {2, 2, 1, 1};
+static const int kFwdC[FWD_VARIANTS] = {1, 2, 2, 4};
+
+int gemv_fwd_variants() { return FWD_VARIANTS; }
+int gemv_fwd_rows_per_block(int variant) { return FWD_WAVES * kFwdRG[variant] * 4; }
 int gemv_fwd_k_step() { return FWD_KROUND; }
 int gemv_dz_cols_per_block() { return DZ_COLS_PER_BLOCK; }
 int gemv_dz_n_step() { return DZ_NSTEP; }
@@ -453,46 +512,58 @@ int gemv_dz_max_slice(int B) {
     return (72 * 1024 / (2 * 4 * H * 4) - 4) / DZ_NSTEP * DZ_NSTEP;
 }
 
-template <int H>
+template <int H, int RG, int C>
 static hipError_t fwd_launch(const float *mu_w, const float *var_w, const float *mu_a,
                              const float *var_a, int K, int N, int B, int per, int splits,
                              int swz, float *ws0, float *ws1, hipStream_t stream) {
     const size_t lds = (size_t)2 * 4 * H * (per + FWD_LDS_PAD) * sizeof(float);
     static bool configured = false;
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_fwd_kernel<H>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipError_t e =
+            hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_fwd_kernel<H, RG, C>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
         configured = true;
     }
-    dim3 grid(((N + FWD_ROWS_PER_BLOCK - 1) / FWD_ROWS_PER_BLOCK) * splits), block(FWD_WAVES * 64);
-    hipLaunchKernelGGL(gemv_fwd_kernel<H>, grid, block, lds, stream, mu_w, var_w, mu_a, var_a, K, N,
-                       B, per, splits, swz, ws0, ws1);
+    constexpr int rows = FWD_WAVES * RG * 4;
+    dim3 grid(((N + rows - 1) / rows) * splits), block(FWD_WAVES * 64);
+    hipLaunchKernelGGL((gemv_fwd_kernel<H, RG, C>), grid, block, lds, stream, mu_w, var_w, mu_a,
+                       var_a, K, N, B, per, splits, swz, ws0, ws1);
     return hipGetLastError();
+}
+
+template <int H>
+static hipError_t fwd_variant(int variant, const float *mu_w, const float *var_w,
+                              const float *mu_a, const float *var_a, int K, int N, int B, int per,
+                              int splits, int swz, float *ws0, float *ws1, hipStream_t stream) {
+    switch (variant) {
+        case 0: return fwd_launch<H, 2, 1>(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1, stream);
+        case 1: return fwd_launch<H, 2, 2>(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1, stream);
+        case 2: return fwd_launch<H, 1, 2>(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1, stream);
+        case 3: return fwd_launch<H, 1, 4>(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1, stream);
+    }
+    return hipErrorInvalidValue;
 }
 
 hipError_t launch_gemv_fwd(const float *mu_w, const float *var_w, const float *mu_a,
                            const float *var_a, int K, int N, int B, int splits, int swz,
-                           float *ws0, float *ws1, hipStream_t stream) {
+                           int variant, float *ws0, float *ws1, hipStream_t stream) {
     int per = (K + splits - 1) / splits;
     per = (per + FWD_KROUND - 1) / FWD_KROUND * FWD_KROUND;
-    if (per > gemv_fwd_max_slice(B)) return hipErrorInvalidValue;
+    if (per > gemv_fwd_max_slice(B) || variant < 0 || variant >= FWD_VARIANTS)
+        return hipErrorInvalidValue;
     switch ((B + 3) / 4) {
-        case 1: return fwd_launch<1>(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1,
-                                       stream);
-        case 2: return fwd_launch<2>(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1,
-                                       stream);
-        case 3: return fwd_launch<3>(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1,
-                                       stream);
-        case 4: return fwd_launch<4>(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1,
-                                       stream);
+        case 1: return fwd_variant<1>(variant, mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1, stream);
+        case 2: return fwd_variant<2>(variant, mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1, stream);
+        case 3: return fwd_variant<3>(variant, mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1, stream);
+        case 4: return fwd_variant<4>(variant, mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1, stream);
     }
     return hipErrorInvalidValue;
 }
 
 template <int H>
 static hipError_t dz_launch(const float *mu_w, const float *dmu, const float *dvar, int K, int N,
-                            int B, int per, int splits, float *ws0, float *ws1,
+                            int B, int per, int splits, int rev, float *ws0, float *ws1,
                             hipStream_t stream) {
     size_t lds = (size_t)2 * 4 * H * (per + 4) * sizeof(float);
     const size_t red = (size_t)(DZ_WAVES / 2) * (4 * H * 4 * 2) * 64 * sizeof(float);
@@ -506,39 +577,49 @@ static hipError_t dz_launch(const float *mu_w, const float *dmu, const float *dv
     }
     dim3 grid((K + DZ_COLS_PER_BLOCK - 1) / DZ_COLS_PER_BLOCK, splits), block(DZ_WAVES * 64);
     hipLaunchKernelGGL(gemv_dz_kernel<H>, grid, block, lds, stream, mu_w, dmu, dvar, K, N, B, per,
-                       ws0, ws1);
+                       rev, ws0, ws1);
     return hipGetLastError();
 }
 
 hipError_t launch_gemv_dz(const float *mu_w, const float *dmu, const float *dvar, int K, int N,
-                          int B, int splits, float *ws0, float *ws1, hipStream_t stream) {
+                          int B, int splits, int rev, float *ws0, float *ws1,
+                          hipStream_t stream) {
     int per = (N + splits - 1) / splits;
     per = (per + DZ_NSTEP - 1) / DZ_NSTEP * DZ_NSTEP;
     if (per > gemv_dz_max_slice(B)) return hipErrorInvalidValue;
     switch ((B + 3) / 4) {
-        case 1: return dz_launch<1>(mu_w, dmu, dvar, K, N, B, per, splits, ws0, ws1, stream);
-        case 2: return dz_launch<2>(mu_w, dmu, dvar, K, N, B, per, splits, ws0, ws1, stream);
-        case 3: return dz_launch<3>(mu_w, dmu, dvar, K, N, B, per, splits, ws0, ws1, stream);
-        case 4: return dz_launch<4>(mu_w, dmu, dvar, K, N, B, per, splits, ws0, ws1, stream);
+        case 1: return dz_launch<1>(mu_w, dmu, dvar, K, N, B, per, splits, rev, ws0, ws1, stream);
+        case 2: return dz_launch<2>(mu_w, dmu, dvar, K, N, B, per, splits, rev, ws0, ws1, stream);
+        case 3: return dz_launch<3>(mu_w, dmu, dvar, K, N, B, per, splits, rev, ws0, ws1, stream);
+        case 4: return dz_launch<4>(mu_w, dmu, dvar, K, N, B, per, splits, rev, ws0, ws1, stream);
     }
     return hipErrorInvalidValue;
 }
 
-hipError_t launch_gemv_dw(const float *var_w, const float *mu_a, const float *dmu,
-                          const float *dvar, int K, int N, int B, float *dmu_w, float *dvar_w,
-                          hipStream_t stream) {
-    dim3 grid((K + DW_COLS_PER_BLOCK - 1) / DW_COLS_PER_BLOCK,
-              (N + DW_ROWS_PER_BLOCK - 1) / DW_ROWS_PER_BLOCK),
-        block(256);
-    if (B <= 4)
-        hipLaunchKernelGGL(gemv_dw_kernel<4>, grid, block, 0, stream, var_w, mu_a, dmu, dvar, K, N,
-                           B, dmu_w, dvar_w);
-    else if (B <= 8)
-        hipLaunchKernelGGL(gemv_dw_kernel<8>, grid, block, 0, stream, var_w, mu_a, dmu, dvar, K, N,
-                           B, dmu_w, dvar_w);
+template <int BMAX>
+static void dw_launch(bool exact, dim3 grid, hipStream_t stream, const float *var_w,
+                      const float *mu_a, const float *dmu, const float *dvar, int K, int N, int B,
+                      int rev, float *dmu_w, float *dvar_w) {
+    if (exact)
+        hipLaunchKernelGGL((gemv_dw_kernel<BMAX, true>), grid, dim3(256), 0, stream, var_w, mu_a,
+                           dmu, dvar, K, N, B, rev, dmu_w, dvar_w);
     else
-        hipLaunchKernelGGL(gemv_dw_kernel<16>, grid, block, 0, stream, var_w, mu_a, dmu, dvar, K,
-                           N, B, dmu_w, dvar_w);
+        hipLaunchKernelGGL((gemv_dw_kernel<BMAX, false>), grid, dim3(256), 0, stream, var_w, mu_a,
+                           dmu, dvar, K, N, B, rev, dmu_w, dvar_w);
+}
+
+hipError_t launch_gemv_dw(const float *var_w, const float *mu_a, const float *dmu,
+                          const float *dvar, int K, int N, int B, int rev, float *dmu_w,
+                          float *dvar_w, hipStream_t stream) {
+    dim3 grid((K + DW_COLS_PER_BLOCK - 1) / DW_COLS_PER_BLOCK,
+              (N + DW_ROWS_PER_BLOCK - 1) / DW_ROWS_PER_BLOCK);
+    const bool exact = (K % DW_COLS_PER_BLOCK == 0) && (N % DW_ROWS_PER_BLOCK == 0);
+    if (B <= 4)
+        dw_launch<4>(exact, grid, stream, var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w);
+    else if (B <= 8)
+        dw_launch<8>(exact, grid, stream, var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w);
+    else
+        dw_launch<16>(exact, grid, stream, var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w);
     return hipGetLastError();
 }
 

@@ -52,14 +52,15 @@ hipError_t launch_reduce_splits(Epilogue epi, const float *ws0, const float *ws1
 // straight into MFMA operand layout, nothing is staged in LDS.
 hipError_t launch_gemv_fwd(const float *mu_w, const float *var_w, const float *mu_a,
                            const float *var_a, int K, int N, int B, int splits, int swz,
-                           float *ws0, float *ws1, hipStream_t stream);
+                           int variant, float *ws0, float *ws1, hipStream_t stream);
 hipError_t launch_gemv_dz(const float *mu_w, const float *dmu, const float *dvar, int K,
-                          int N, int B, int splits, float *ws0, float *ws1,
+                          int N, int B, int splits, int rev, float *ws0, float *ws1,
                           hipStream_t stream);
 hipError_t launch_gemv_dw(const float *var_w, const float *mu_a, const float *dmu,
-                          const float *dvar, int K, int N, int B, float *dmu_w,
+                          const float *dvar, int K, int N, int B, int rev, float *dmu_w,
                           float *dvar_w, hipStream_t stream);
-int gemv_fwd_rows_per_block();
+int gemv_fwd_variants();
+int gemv_fwd_rows_per_block(int variant);
 int gemv_fwd_k_step();
 int gemv_dz_cols_per_block();
 int gemv_dz_n_step();
