@@ -45,5 +45,36 @@ def build(extra_flags=(), objdir=None, lib=LIB):
     return lib
 
 
+HOST_SOURCES = ["states.cpp", "layers.cpp", "sequential.cpp", "bindings.cpp"]
+
+
+def build_host():
+    """The C++ host classes (BaseLayer / Linear / Conv2d / Sequential / OutputUpdater
+    mirrors) and their pybind11 module `cutagi`, linked against libtagi_hip.so."""
+    import sysconfig
+    import pybind11
+    host = os.path.join(HERE, "host")
+    objdir = os.path.join(HERE, "build", "host")
+    os.makedirs(objdir, exist_ok=True)
+    ext = sysconfig.get_config_var("EXT_SUFFIX")
+    out = os.path.join(HERE, "cutagi" + ext)
+    flags = ["-O2", "-std=c++17", "-fPIC", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include",
+             "-I" + pybind11.get_include(), "-I" + sysconfig.get_paths()["include"],
+             "-fvisibility=hidden"]
+
+    def comp(src):
+        obj = os.path.join(objdir, src.replace(".cpp", ".o"))
+        subprocess.run(["g++"] + flags + ["-c", os.path.join(host, src), "-o", obj], check=True)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        objs = list(pool.map(comp, HOST_SOURCES))
+    subprocess.run(["g++", "-shared", "-o", out] + objs +
+                   ["-L" + HERE, "-ltagi_hip", "-L/opt/rocm/lib", "-lamdhip64",
+                    "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"], check=True)
+    return out
+
+
 if __name__ == "__main__":
     print(build())
+    print(build_host())

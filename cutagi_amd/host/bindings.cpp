@@ -1,0 +1,212 @@
+// pybind11 module `cutagi`: the Python surface of the reference's extension
+// module (src/bindings/*.cpp) for the classes on the hot path, with the same
+// class, method and argument names, so that pytagi-style code runs unchanged.
+#include <pybind11/numpy.h>
+#include <pybind11/pybind11.h>
+#include <pybind11/stl.h>
+
+#include <cstring>
+
+#include "../../include/tagi_hip.h"
+#include "sequential.h"
+
+namespace py = pybind11;
+using namespace tagi_host;
+
+namespace {
+std::vector<float> to_vec(const py::array_t<float, py::array::c_style | py::array::forcecast> &a) {
+    std::vector<float> v(a.size());
+    if (a.size()) std::memcpy(v.data(), a.data(), a.size() * sizeof(float));
+    return v;
+}
+py::array_t<float> to_np(const std::vector<float> &v) { return py::array_t<float>(v.size(), v.data()); }
+}  // namespace
+
+PYBIND11_MODULE(cutagi, m) {
+    m.doc() = "TAGI Linear/Conv2d hot path on MI355X (HIP backend)";
+
+    py::class_<BaseHiddenStates, std::shared_ptr<BaseHiddenStates>>(m, "BaseHiddenStates")
+        .def(py::init<size_t, size_t>())
+        .def(py::init<>())
+        .def_readwrite("mu_a", &BaseHiddenStates::mu_a)
+        .def_readwrite("var_a", &BaseHiddenStates::var_a)
+        .def_readwrite("jcb", &BaseHiddenStates::jcb)
+        .def_readwrite("size", &BaseHiddenStates::size)
+        .def_readwrite("block_size", &BaseHiddenStates::block_size)
+        .def_readwrite("actual_size", &BaseHiddenStates::actual_size)
+        .def_readwrite("width", &BaseHiddenStates::width)
+        .def_readwrite("height", &BaseHiddenStates::height)
+        .def_readwrite("depth", &BaseHiddenStates::depth)
+        .def("set_input_x", &BaseHiddenStates::set_input_x)
+        .def("get_name", &BaseHiddenStates::get_name)
+        .def("set_size", &BaseHiddenStates::set_size)
+        .def("swap", &BaseHiddenStates::swap)
+        .def("copy_from", &BaseHiddenStates::copy_from, py::arg("source"), py::arg("num_data") = -1);
+    py::class_<HiddenStateHip, BaseHiddenStates, std::shared_ptr<HiddenStateHip>>(m, "HiddenStateCuda")
+        .def(py::init<size_t, size_t, int>(), py::arg("size"), py::arg("block_size"),
+             py::arg("device_idx") = 0)
+        .def("to_host", py::overload_cast<>(&HiddenStateHip::to_host))
+        .def("to_device", &HiddenStateHip::to_device);
+
+    py::class_<BaseDeltaStates, std::shared_ptr<BaseDeltaStates>>(m, "BaseDeltaStates")
+        .def(py::init<size_t, size_t>())
+        .def(py::init<>())
+        .def_readwrite("delta_mu", &BaseDeltaStates::delta_mu)
+        .def_readwrite("delta_var", &BaseDeltaStates::delta_var)
+        .def_readwrite("size", &BaseDeltaStates::size)
+        .def_readwrite("block_size", &BaseDeltaStates::block_size)
+        .def_readwrite("actual_size", &BaseDeltaStates::actual_size)
+        .def("get_name", &BaseDeltaStates::get_name)
+        .def("reset_zeros", &BaseDeltaStates::reset_zeros)
+        .def("copy_from", &BaseDeltaStates::copy_from, py::arg("source"), py::arg("num_data") = -1)
+        .def("set_size", &BaseDeltaStates::set_size)
+        .def("swap", &BaseDeltaStates::swap);
+    py::class_<DeltaStateHip, BaseDeltaStates, std::shared_ptr<DeltaStateHip>>(m, "DeltaStateCuda")
+        .def(py::init<size_t, size_t, int>(), py::arg("size"), py::arg("block_size"),
+             py::arg("device_idx") = 0)
+        .def("to_host", &DeltaStateHip::to_host)
+        .def("to_device", &DeltaStateHip::to_device);
+
+    py::class_<BaseLayer, std::shared_ptr<BaseLayer>>(m, "BaseLayer")
+        .def_readwrite("input_size", &BaseLayer::input_size)
+        .def_readwrite("output_size", &BaseLayer::output_size)
+        .def_readwrite("in_width", &BaseLayer::in_width)
+        .def_readwrite("in_height", &BaseLayer::in_height)
+        .def_readwrite("in_channels", &BaseLayer::in_channels)
+        .def_readwrite("out_width", &BaseLayer::out_width)
+        .def_readwrite("out_height", &BaseLayer::out_height)
+        .def_readwrite("out_channels", &BaseLayer::out_channels)
+        .def_readwrite("bias", &BaseLayer::bias)
+        .def_readwrite("num_weights", &BaseLayer::num_weights)
+        .def_readwrite("num_biases", &BaseLayer::num_biases)
+        .def_readwrite("mu_w", &BaseLayer::mu_w)
+        .def_readwrite("var_w", &BaseLayer::var_w)
+        .def_readwrite("mu_b", &BaseLayer::mu_b)
+        .def_readwrite("var_b", &BaseLayer::var_b)
+        .def_readwrite("delta_mu_w", &BaseLayer::delta_mu_w)
+        .def_readwrite("delta_var_w", &BaseLayer::delta_var_w)
+        .def_readwrite("delta_mu_b", &BaseLayer::delta_mu_b)
+        .def_readwrite("delta_var_b", &BaseLayer::delta_var_b)
+        .def_readwrite("num_threads", &BaseLayer::num_threads)
+        .def_readwrite("training", &BaseLayer::training)
+        .def_readwrite("param_update", &BaseLayer::param_update)
+        .def_readwrite("cap_factor_update", &BaseLayer::cap_factor_update)
+        .def_readwrite("device", &BaseLayer::device)
+        .def("forward", &BaseLayer::forward)
+        .def("backward", &BaseLayer::backward, py::arg("input_delta_states"),
+             py::arg("output_delta_states"), py::arg("temp_states"), py::arg("state_udapte") = true)
+        .def("get_layer_info", &BaseLayer::get_layer_info)
+        .def("get_layer_name", &BaseLayer::get_layer_name)
+        .def("get_max_num_states", &BaseLayer::get_max_num_states)
+        .def("preinit_layer", &BaseLayer::preinit_layer)
+        .def("params_to_host",
+             [](BaseLayer &l) {
+                 if (auto *d = dynamic_cast<BaseLayerHip *>(&l)) d->params_to_host();
+             })
+        .def("params_to_device",
+             [](BaseLayer &l) {
+                 if (auto *d = dynamic_cast<BaseLayerHip *>(&l)) d->params_to_device();
+             })
+        .def("delta_params_to_host", [](BaseLayer &l) {
+            if (auto *d = dynamic_cast<BaseLayerHip *>(&l)) d->delta_params_to_host();
+        });
+
+    py::class_<Linear, BaseLayer, std::shared_ptr<Linear>>(m, "Linear")
+        .def(py::init<size_t, size_t, bool, float, float, std::string, int>(), py::arg("ip_size"),
+             py::arg("op_size"), py::arg("bias") = true, py::arg("gain_weight") = 1.0f,
+             py::arg("gain_bias") = 1.0f, py::arg("method") = "He", py::arg("device_idx") = 0)
+        .def("init_weight_bias", &Linear::init_weight_bias);
+    py::class_<Conv2d, BaseLayer, std::shared_ptr<Conv2d>>(m, "Conv2d")
+        .def(py::init<size_t, size_t, size_t, bool, int, int, int, size_t, size_t, float, float,
+                      std::string, int>(),
+             py::arg("in_channels"), py::arg("out_channels"), py::arg("kernel_size"),
+             py::arg("bias") = true, py::arg("stride") = 1, py::arg("padding") = 0,
+             py::arg("padding_type") = 1, py::arg("in_width") = 0, py::arg("in_height") = 0,
+             py::arg("gain_weight") = 1.0f, py::arg("gain_bias") = 1.0f,
+             py::arg("init_method") = "He", py::arg("device_idx") = 0)
+        .def("init_weight_bias", &Conv2d::init_weight_bias);
+    py::class_<ReLU, BaseLayer, std::shared_ptr<ReLU>>(m, "ReLU").def(py::init<>());
+
+    py::class_<OutputUpdater, std::shared_ptr<OutputUpdater>>(m, "OutputUpdater")
+        .def(py::init<const std::string>())
+        .def("update", &OutputUpdater::update, py::arg("output_states"), py::arg("mu_obs"),
+             py::arg("var_obs"), py::arg("delta_states"))
+        .def("update_using_indices", &OutputUpdater::update_using_indices,
+             py::arg("output_states"), py::arg("mu_obs"), py::arg("var_obs"),
+             py::arg("selected_idx"), py::arg("delta_states"))
+        .def_readwrite("device", &OutputUpdater::device);
+
+    py::class_<Sequential, std::shared_ptr<Sequential>>(m, "Sequential")
+        .def(py::init<>())
+        .def(py::init([](const std::vector<std::shared_ptr<BaseLayer>> &layers) {
+            auto seq = std::make_shared<Sequential>();
+            for (const auto &layer : layers) seq->add_layer(layer);
+            seq->add_layers();
+            return seq;
+        }))
+        .def_readwrite("layers", &Sequential::layers)
+        .def_readwrite("output_z_buffer", &Sequential::output_z_buffer)
+        .def_readwrite("input_delta_z_buffer", &Sequential::input_delta_z_buffer)
+        .def_readwrite("output_delta_z_buffer", &Sequential::output_delta_z_buffer)
+        .def_readwrite("z_buffer_size", &Sequential::z_buffer_size)
+        .def_readwrite("z_buffer_block_size", &Sequential::z_buffer_block_size)
+        .def_readwrite("input_size", &Sequential::input_size)
+        .def_readwrite("num_samples", &Sequential::num_samples)
+        .def_readwrite("training", &Sequential::training)
+        .def_readwrite("param_update", &Sequential::param_update)
+        .def_readwrite("device", &Sequential::device)
+        .def_readwrite("input_state_update", &Sequential::input_state_update)
+        .def_readwrite("num_threads", &Sequential::num_threads)
+        .def("to_device", &Sequential::to_device)
+        .def("params_to_host", &Sequential::params_to_host)
+        .def("params_to_device", &Sequential::params_to_device)
+        .def("set_threads", &Sequential::set_threads)
+        .def("train", &Sequential::train)
+        .def("eval", &Sequential::eval)
+        .def("forward",
+             [](Sequential &self, py::object arg1, py::object arg2) {
+                 if (py::isinstance<BaseHiddenStates>(arg1)) {
+                     self.forward(arg1.cast<BaseHiddenStates &>());
+                     return;
+                 }
+                 auto mu = to_vec(arg1.cast<py::array_t<float, py::array::c_style | py::array::forcecast>>());
+                 std::vector<float> var;
+                 if (!arg2.is_none())
+                     var = to_vec(arg2.cast<py::array_t<float, py::array::c_style | py::array::forcecast>>());
+                 self.forward(mu, var);
+             },
+             py::arg("mu_x"), py::arg("var_x") = py::none())
+        .def("backward", &Sequential::backward)
+        .def("step", &Sequential::step)
+        .def("output_to_host", &Sequential::output_to_host)
+        .def("delta_z_to_host", &Sequential::delta_z_to_host)
+        .def("set_delta_z",
+             [](Sequential &self, py::array_t<float, py::array::c_style | py::array::forcecast> mu,
+                py::array_t<float, py::array::c_style | py::array::forcecast> var) {
+                 auto m_ = to_vec(mu), v_ = to_vec(var);
+                 self.set_delta_z(m_, v_);
+             },
+             py::arg("delta_mu"), py::arg("delta_var"))
+        .def("get_layer_stack_info", &Sequential::get_layer_stack_info)
+        .def("preinit_layer", &Sequential::preinit_layer)
+        .def("get_neg_var_w_counter", &Sequential::get_neg_var_w_counter)
+        .def("save", &Sequential::save)
+        .def("load", &Sequential::load)
+        .def("params_from", &Sequential::params_from)
+        .def("parameters", &Sequential::parameters)
+        .def("state_dict", &Sequential::state_dict)
+        .def("load_state_dict", &Sequential::load_state_dict)
+        .def("get_outputs",
+             [](Sequential &self) {
+                 auto r = self.get_outputs_vec();
+                 return std::make_tuple(to_np(std::get<0>(r)), to_np(std::get<1>(r)));
+             })
+        .def("get_input_states", [](Sequential &self) {
+            auto r = self.get_input_states_vec();
+            return std::make_tuple(to_np(std::get<0>(r)), to_np(std::get<1>(r)));
+        });
+
+    m.def("manual_seed", &manual_seed);
+    m.def("is_cuda_available", &is_cuda_available);
+    m.def("get_cuda_device_count", &get_cuda_device_count);
+}

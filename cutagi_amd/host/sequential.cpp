@@ -1,0 +1,403 @@
+// Sequential and OutputUpdater: see sequential.h.
+#include "sequential.h"
+
+#include <fstream>
+#include <sstream>
+
+#include "../../include/tagi_hip.h"
+#include "logger.h"
+
+namespace tagi_host {
+
+constexpr int PACK_SIZE = 4;  // state buffers are sized in multiples of 4 floats
+
+int get_cuda_device_count() {
+    int n = 0;
+    if (tagi_hip_device_count(&n) != TAGI_OK) return 0;
+    return n;
+}
+bool is_cuda_available() { return get_cuda_device_count() > 0; }
+
+// ---- OutputUpdater ------------------------------------------------------------------
+OutputUpdater::OutputUpdater(const std::string model_device) : device(model_device) {
+    const size_t colon = model_device.find(':');
+    if (colon != std::string::npos) {
+        this->device_idx = std::stoi(model_device.substr(colon + 1));
+        this->device = model_device.substr(0, colon);
+    }
+    if (this->device == "hip") this->device = "cuda";
+    if (this->device == "cuda")
+        this->obs = std::make_shared<ObservationHip>(this->device_idx);
+    else
+        this->obs = std::make_shared<BaseObservation>();
+}
+
+ObservationHip *OutputUpdater::device_obs() {
+    auto *o = dynamic_cast<ObservationHip *>(this->obs.get());
+    if (o == nullptr)
+        LOG(LogLevel::ERROR,
+            "OutputUpdater(\"" + device + "\"): this library computes on the GPU only; "
+            "construct it with the model's device (\"cuda\")");
+    return o;
+}
+
+void OutputUpdater::update(BaseHiddenStates &output_states, std::vector<float> &mu_obs,
+                           std::vector<float> &var_obs, BaseDeltaStates &delta_states) {
+    ObservationHip *o = this->device_obs();
+    auto *out = dynamic_cast<HiddenStateHip *>(&output_states);
+    auto *delta = dynamic_cast<DeltaStateHip *>(&delta_states);
+    if (out == nullptr || delta == nullptr)
+        LOG(LogLevel::ERROR, "OutputUpdater needs device state buffers");
+    if (mu_obs.size() != var_obs.size() || mu_obs.size() > out->size || mu_obs.size() > delta->size)
+        LOG(LogLevel::ERROR, "Observation size does not fit the output buffers");
+    o->set_obs(mu_obs, var_obs);
+    o->block_size = output_states.block_size;
+    o->size = mu_obs.size();
+    o->actual_size = mu_obs.size() / output_states.block_size;
+    o->to_device();
+    delta->reset_zeros();
+    TAGI_OK_OR_THROW(tagi_out_update_dense(out->d_mu_a, out->d_var_a, out->d_jcb, o->d_mu_obs,
+                                           o->d_var_obs, (int)o->size, delta->d_delta_mu,
+                                           delta->d_delta_var, nullptr));
+}
+
+void OutputUpdater::update_using_indices(BaseHiddenStates &output_states,
+                                         std::vector<float> &mu_obs, std::vector<float> &var_obs,
+                                         std::vector<int> &selected_idx,
+                                         BaseDeltaStates &delta_states) {
+    ObservationHip *o = this->device_obs();
+    auto *out = dynamic_cast<HiddenStateHip *>(&output_states);
+    auto *delta = dynamic_cast<DeltaStateHip *>(&delta_states);
+    if (out == nullptr || delta == nullptr)
+        LOG(LogLevel::ERROR, "OutputUpdater needs device state buffers");
+    if (mu_obs.size() != var_obs.size() || selected_idx.size() != mu_obs.size() ||
+        output_states.block_size == 0 || mu_obs.size() % output_states.block_size != 0)
+        LOG(LogLevel::ERROR, "Observations, variances and indices must have one size, a multiple "
+                             "of the batch size");
+    const int n_obs = (int)output_states.actual_size;
+    for (int idx : selected_idx)
+        if (idx < 1 || idx > n_obs)
+            LOG(LogLevel::ERROR, "Selected index " + std::to_string(idx) + " outside 1.." +
+                                     std::to_string(n_obs));
+    o->set_obs(mu_obs, var_obs);
+    o->set_selected_idx(selected_idx);
+    o->block_size = output_states.block_size;
+    o->size = mu_obs.size();
+    o->actual_size = mu_obs.size() / output_states.block_size;
+    o->idx_size = selected_idx.size();
+    o->to_device();
+    const int n_enc = (int)(o->idx_size / output_states.block_size);
+    delta->reset_zeros();
+    TAGI_OK_OR_THROW(tagi_out_update_indexed(out->d_mu_a, out->d_var_a, out->d_jcb, o->d_mu_obs,
+                                             o->d_var_obs, o->d_selected_idx, n_obs, n_enc,
+                                             (int)o->size, delta->d_delta_mu, delta->d_delta_var,
+                                             nullptr));
+}
+
+// ---- Sequential -----------------------------------------------------------------------
+void Sequential::add_layer(std::shared_ptr<BaseLayer> layer) {
+    if (this->device == "cpu")
+        this->layers.push_back(layer);
+    else if (this->device == "cuda")
+        this->layers.push_back(layer->to_cuda(this->device_idx));
+    else
+        LOG(LogLevel::ERROR, "Invalid device: [" + this->device + "]");
+}
+
+void Sequential::add_layers() {
+    if (this->layers.empty()) return;
+    this->compute_input_output_size();
+    this->set_buffer_size();
+}
+
+void Sequential::switch_to_cuda() {
+    for (auto &layer : this->layers) layer = layer->to_cuda(this->device_idx);
+}
+
+// reference: src/sequential.cpp:32-73. "hip" is accepted as a synonym of "cuda".
+void Sequential::to_device(const std::string &new_device) {
+    if (new_device == "cpu") {
+        this->device = "cpu";
+        return;
+    }
+    std::string name = new_device;
+    int idx = 0;
+    const size_t colon = new_device.find(':');
+    if (colon != std::string::npos) {
+        name = new_device.substr(0, colon);
+        try {
+            idx = std::stoi(new_device.substr(colon + 1));
+        } catch (const std::exception &) {
+            LOG(LogLevel::ERROR, "Invalid device index format in: [" + new_device + "]");
+        }
+    }
+    if (name == "hip") name = "cuda";
+    if (name != "cuda") LOG(LogLevel::ERROR, "Invalid device: [" + new_device + "]");
+    const int count = get_cuda_device_count();
+    if (count == 0) LOG(LogLevel::ERROR, "CUDA is not available");
+    if (idx < 0 || idx >= count)
+        LOG(LogLevel::ERROR, "Invalid CUDA device index: " + std::to_string(idx) +
+                                 ". Available devices: " + std::to_string(count));
+    const bool already = this->device == "cuda";
+    this->device = name;
+    this->device_idx = idx;
+    if (!already) this->switch_to_cuda();
+    this->compute_input_output_size();
+    this->set_buffer_size();
+}
+
+void Sequential::params_to_host() {
+    for (auto &layer : layers)
+        if (auto *l = dynamic_cast<BaseLayerHip *>(layer.get())) l->params_to_host();
+}
+void Sequential::params_to_device() {
+    for (auto &layer : layers)
+        if (auto *l = dynamic_cast<BaseLayerHip *>(layer.get())) l->params_to_device();
+}
+
+void Sequential::set_buffer_size() {
+    int per_sample = this->z_buffer_block_size > 0 ? this->z_buffer_size / this->z_buffer_block_size
+                                                   : this->z_buffer_size;
+    for (auto &layer : layers) per_sample = std::max(per_sample, layer->get_max_num_states());
+    per_sample = (per_sample + PACK_SIZE - 1) / PACK_SIZE * PACK_SIZE;
+    this->z_buffer_size =
+        this->z_buffer_block_size > 0 ? per_sample * this->z_buffer_block_size : per_sample;
+}
+
+void Sequential::compute_input_output_size() {
+    int w = (int)layers.front()->in_width, h = (int)layers.front()->in_height;
+    int d = (int)layers.front()->in_channels;
+    for (auto &layer : layers) {
+        layer->compute_input_output_size(InitArgs(w, h, d));
+        w = (int)layer->out_width;
+        h = (int)layer->out_height;
+        d = (int)layer->out_channels;
+    }
+}
+
+void Sequential::require_device(const char *what) const {
+    if (this->device != "cuda")
+        LOG(LogLevel::ERROR, std::string(what) + ": this library computes on the GPU only; call "
+                                                 "to_device(\"cuda\") first");
+}
+
+void Sequential::init_output_state_buffer() {
+    output_z_buffer = std::make_shared<HiddenStateHip>(z_buffer_size, z_buffer_block_size, device_idx);
+    input_z_buffer = std::make_shared<HiddenStateHip>(z_buffer_size, z_buffer_block_size, device_idx);
+    temp_states = std::make_shared<TempStateHip>(0, z_buffer_block_size, device_idx);
+}
+
+void Sequential::init_delta_state_buffer() {
+    output_delta_z_buffer =
+        std::make_shared<DeltaStateHip>(z_buffer_size, z_buffer_block_size, device_idx);
+    input_delta_z_buffer =
+        std::make_shared<DeltaStateHip>(z_buffer_size, z_buffer_block_size, device_idx);
+}
+
+// Lazy allocation at the first batch, regrowth when the batch size changes
+// (reference: src/sequential.cpp:290-318).
+void Sequential::prepare_buffers(int batch_size) {
+    if (this->z_buffer_block_size == 0) {
+        this->z_buffer_block_size = batch_size;
+        this->z_buffer_size = batch_size * this->z_buffer_size;
+        this->init_output_state_buffer();
+        if (this->training) this->init_delta_state_buffer();
+    }
+    if (batch_size != this->z_buffer_block_size) {
+        this->z_buffer_size = batch_size * (this->z_buffer_size / this->z_buffer_block_size);
+        this->z_buffer_block_size = batch_size;
+        this->input_z_buffer->set_size(this->z_buffer_size, batch_size);
+        this->output_z_buffer->set_size(this->z_buffer_size, batch_size);
+        if (this->training) {
+            this->input_delta_z_buffer->set_size(this->z_buffer_size, batch_size);
+            this->output_delta_z_buffer->set_size(this->z_buffer_size, batch_size);
+        }
+    }
+    if (this->training && !this->input_delta_z_buffer) this->init_delta_state_buffer();
+}
+
+void Sequential::set_threads(unsigned n) {
+    this->num_threads = n;
+    for (auto &layer : layers) layer->set_threads(n);
+}
+void Sequential::train() {
+    this->training = true;
+    for (auto &layer : layers) layer->train();
+}
+void Sequential::eval() {
+    this->training = false;
+    for (auto &layer : layers) layer->eval();
+}
+std::string Sequential::get_device() { return this->device; }
+
+void Sequential::forward(const std::vector<float> &mu_x, const std::vector<float> &var_x) {
+    this->require_device("forward");
+    const int in_size = this->layers.front()->get_input_size();
+    if (in_size <= 0 || mu_x.size() % in_size != 0)
+        LOG(LogLevel::ERROR, "Input size mismatch: " + std::to_string(in_size) + " vs " +
+                                 std::to_string(mu_x.size()));
+    const int batch_size = (int)(mu_x.size() / in_size);
+    this->prepare_buffers(batch_size);
+    this->input_z_buffer->set_input_x(mu_x, var_x, batch_size);
+    for (auto &layer : layers) {
+        layer->forward(*input_z_buffer, *output_z_buffer, *temp_states);
+        std::swap(input_z_buffer, output_z_buffer);
+    }
+    std::swap(output_z_buffer, input_z_buffer);
+}
+
+void Sequential::forward(BaseHiddenStates &input_states) {
+    this->require_device("forward");
+    this->prepare_buffers((int)input_states.block_size);
+    layers.front()->forward(input_states, *input_z_buffer, *temp_states);
+    for (size_t i = 1; i < layers.size(); i++) {
+        layers[i]->forward(*input_z_buffer, *output_z_buffer, *temp_states);
+        std::swap(input_z_buffer, output_z_buffer);
+    }
+    std::swap(output_z_buffer, input_z_buffer);
+}
+
+// reference: src/sequential.cpp:387-411. Activations do not consume a delta
+// buffer; the first layer propagates to its input only on request.
+void Sequential::backward() {
+    this->require_device("backward");
+    for (size_t i = layers.size() - 1; i >= 1; i--) {
+        BaseLayer *layer = layers[i].get();
+        layer->backward(*input_delta_z_buffer, *output_delta_z_buffer, *temp_states);
+        if (layer->get_layer_type() != LayerType::Activation)
+            std::swap(input_delta_z_buffer, output_delta_z_buffer);
+    }
+    layers.front()->backward(*input_delta_z_buffer, *output_delta_z_buffer, *temp_states,
+                             this->input_state_update);
+}
+
+void Sequential::step() {
+    this->require_device("step");
+    for (auto &layer : layers) {
+        if (layer->get_layer_type() == LayerType::Activation) continue;
+        layer->update_weights();
+        layer->update_biases();
+    }
+}
+
+std::string Sequential::get_layer_stack_info() const {
+    std::stringstream ss;
+    for (const auto &layer : layers)
+        if (layer) ss << layer->get_layer_info() << "\n";
+    return ss.str();
+}
+
+void Sequential::preinit_layer() {
+    for (auto &layer : layers)
+        if (layer) layer->preinit_layer();
+}
+
+void Sequential::save(const std::string &filename) {
+    std::ofstream file(filename, std::ios::binary);
+    if (!file.is_open()) LOG(LogLevel::ERROR, "Failed to open file for saving");
+    for (auto &layer : layers) layer->save(file);
+}
+
+void Sequential::load(const std::string &filename) {
+    this->preinit_layer();
+    std::ifstream file(filename, std::ios::binary);
+    if (!file.is_open()) LOG(LogLevel::ERROR, "Failed to open file for loading");
+    for (auto &layer : layers) layer->load(file);
+}
+
+std::vector<ParameterTuple> Sequential::parameters() {
+    std::vector<ParameterTuple> params;
+    for (auto &layer : layers) {
+        if (layer->get_layer_type() == LayerType::Activation) continue;
+        auto p = layer->parameters();
+        params.insert(params.end(), p.begin(), p.end());
+    }
+    return params;
+}
+
+ParameterMap Sequential::state_dict() {
+    ParameterMap sd;
+    for (size_t i = 0; i < layers.size(); i++) {
+        if (layers[i]->get_layer_type() == LayerType::Activation) continue;
+        auto p = layers[i]->get_parameters_as_map(std::to_string(i));
+        sd.insert(p.begin(), p.end());
+    }
+    return sd;
+}
+
+void Sequential::load_state_dict(const ParameterMap &sd) {
+    for (size_t i = 0; i < layers.size(); i++) {
+        if (layers[i]->get_layer_type() == LayerType::Activation) continue;
+        layers[i]->load_parameters_from_map(sd, std::to_string(i));
+    }
+}
+
+void Sequential::params_from(const Sequential &ref) {
+    if (layers.size() != ref.layers.size()) LOG(LogLevel::ERROR, "Model architecture is different.");
+    for (size_t i = 0; i < layers.size(); i++) {
+        BaseLayer *src = ref.layers[i].get();
+        if (auto *s = dynamic_cast<BaseLayerHip *>(src)) s->params_to_host();
+        layers[i]->num_weights = src->num_weights;
+        layers[i]->num_biases = src->num_biases;
+        layers[i]->mu_w = src->mu_w;
+        layers[i]->var_w = src->var_w;
+        layers[i]->mu_b = src->mu_b;
+        layers[i]->var_b = src->var_b;
+        if (auto *d = dynamic_cast<BaseLayerHip *>(layers[i].get()))
+            if (d->d_mu_w != nullptr) d->params_to_device();
+    }
+}
+
+std::unordered_map<std::string, int> Sequential::get_neg_var_w_counter() {
+    std::unordered_map<std::string, int> counter;
+    for (size_t i = 0; i < layers.size(); i++) {
+        if (layers[i]->get_layer_type() == LayerType::Activation) continue;
+        counter[layers[i]->get_layer_name() + "." + std::to_string(i)] =
+            layers[i]->get_neg_var_w_counter();
+    }
+    return counter;
+}
+
+void Sequential::output_to_host() {
+    if (auto *o = dynamic_cast<HiddenStateHip *>(output_z_buffer.get())) o->to_host();
+}
+
+void Sequential::delta_z_to_host() {
+    if (auto *d = dynamic_cast<DeltaStateHip *>(input_delta_z_buffer.get())) d->to_host();
+    if (auto *d = dynamic_cast<DeltaStateHip *>(output_delta_z_buffer.get())) d->to_host();
+}
+
+// reference: src/sequential.cpp:499-515 (the vectors replace the host copy of the
+// input delta buffer and must have its capacity)
+void Sequential::set_delta_z(std::vector<float> &delta_mu, std::vector<float> &delta_var) {
+    auto *d = dynamic_cast<DeltaStateHip *>(input_delta_z_buffer.get());
+    if (d == nullptr) LOG(LogLevel::ERROR, "set_delta_z needs a forward pass in training mode first");
+    if (delta_mu.size() != d->size || delta_var.size() != d->size)
+        LOG(LogLevel::ERROR, "set_delta_z: vectors must have the buffer size " +
+                                 std::to_string(d->size));
+    d->delta_mu = delta_mu;
+    d->delta_var = delta_var;
+    d->to_device();
+}
+
+std::tuple<std::vector<float>, std::vector<float>> Sequential::get_outputs_vec() {
+    auto *o = dynamic_cast<HiddenStateHip *>(output_z_buffer.get());
+    if (o == nullptr) LOG(LogLevel::ERROR, "get_outputs needs a forward pass first");
+    const size_t n = o->block_size * layers.back()->output_size;
+    o->to_host(n);  // only the part that holds outputs, not the whole capacity
+    return {std::vector<float>(o->mu_a.begin(), o->mu_a.begin() + n),
+            std::vector<float>(o->var_a.begin(), o->var_a.begin() + n)};
+}
+
+// innovations that reached the model's input (needs input_state_update)
+std::tuple<std::vector<float>, std::vector<float>> Sequential::get_input_states_vec() {
+    if (!this->input_state_update) LOG(LogLevel::ERROR, "input_state_update is set to False.");
+    auto *d = dynamic_cast<DeltaStateHip *>(output_delta_z_buffer.get());
+    if (d == nullptr) LOG(LogLevel::ERROR, "get_input_states needs a backward pass first");
+    d->to_host();
+    const size_t n = this->z_buffer_block_size * layers.front()->input_size;
+    return {std::vector<float>(d->delta_mu.begin(), d->delta_mu.begin() + n),
+            std::vector<float>(d->delta_var.begin(), d->delta_var.begin() + n)};
+}
+
+}  // namespace tagi_host

@@ -1,0 +1,98 @@
+// Model driver and output updater, mirroring the reference's Sequential
+// (include/sequential.h, src/sequential.cpp:25-73,102-448,574-768) and
+// OutputUpdater (include/base_output_updater.h, src/base_output_updater.cpp:269-386,
+// src/output_updater_cuda.cu:146-223).
+#pragma once
+#include <memory>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "layers.h"
+
+namespace tagi_host {
+
+bool is_cuda_available();
+int get_cuda_device_count();
+
+class OutputUpdater {
+   public:
+    std::string device = "cpu";
+    int device_idx = 0;
+    std::shared_ptr<BaseObservation> obs;
+
+    explicit OutputUpdater(const std::string model_device);
+    void update(BaseHiddenStates &output_states, std::vector<float> &mu_obs,
+                std::vector<float> &var_obs, BaseDeltaStates &delta_states);
+    void update_using_indices(BaseHiddenStates &output_states, std::vector<float> &mu_obs,
+                              std::vector<float> &var_obs, std::vector<int> &selected_idx,
+                              BaseDeltaStates &delta_states);
+
+   private:
+    ObservationHip *device_obs();
+};
+
+class Sequential {
+   public:
+    std::shared_ptr<BaseHiddenStates> output_z_buffer, input_z_buffer;
+    std::shared_ptr<BaseDeltaStates> output_delta_z_buffer, input_delta_z_buffer;
+    std::shared_ptr<BaseTempStates> temp_states;
+
+    int z_buffer_size = 0;        // per-sample capacity until the first forward, then x batch
+    int z_buffer_block_size = 0;  // batch size the buffers were made for
+    int num_samples = 0;
+    int input_size = 0;
+    bool training = true;
+    bool param_update = true;
+    bool input_state_update = false;
+    unsigned num_threads = 1;
+    std::string device = "cpu";
+    int device_idx = 0;
+    std::vector<std::shared_ptr<BaseLayer>> layers;
+
+    Sequential() = default;
+    void add_layer(std::shared_ptr<BaseLayer> layer);
+    void add_layers();  // call once after the last add_layer
+
+    void to_device(const std::string &new_device);
+    void params_to_host();
+    void params_to_device();
+    void set_threads(unsigned num_threads);
+    void train();
+    void eval();
+    std::string get_device();
+
+    void forward(const std::vector<float> &mu_x,
+                 const std::vector<float> &var_x = std::vector<float>());
+    void forward(BaseHiddenStates &input_states);
+    void backward();
+    void step();
+
+    std::string get_layer_stack_info() const;
+    void preinit_layer();
+    void save(const std::string &filename);
+    void load(const std::string &filename);
+    std::vector<ParameterTuple> parameters();
+    ParameterMap state_dict();
+    void load_state_dict(const ParameterMap &state_dict);
+    void params_from(const Sequential &ref_model);
+    std::unordered_map<std::string, int> get_neg_var_w_counter();
+
+    void output_to_host();
+    void delta_z_to_host();
+    void set_delta_z(std::vector<float> &delta_mu, std::vector<float> &delta_var);
+    // first batch*outputs entries of the output buffer, copied to the host
+    std::tuple<std::vector<float>, std::vector<float>> get_outputs_vec();
+    std::tuple<std::vector<float>, std::vector<float>> get_input_states_vec();
+
+   private:
+    void switch_to_cuda();
+    void compute_input_output_size();
+    void set_buffer_size();
+    void init_output_state_buffer();
+    void init_delta_state_buffer();
+    void prepare_buffers(int batch_size);
+    void require_device(const char *what) const;
+};
+
+}  // namespace tagi_host

@@ -1,0 +1,363 @@
+// Host and device state containers: see states.h. Device buffers are plain
+// hipMalloc allocations owned by the object that made them; copies are
+// synchronous hipMemcpy on the null stream, which also orders them after every
+// kernel the layers queued there.
+#include "states.h"
+
+#include <algorithm>
+
+#include "logger.h"
+
+namespace tagi_host {
+
+namespace {
+float *dev_alloc(size_t n, int device_idx) {
+    float *p = nullptr;
+    if (n == 0) return p;
+    HIP_OK(hipSetDevice(device_idx));
+    HIP_OK(hipMalloc(reinterpret_cast<void **>(&p), n * sizeof(float)));
+    return p;
+}
+void dev_free(float *&p) {
+    if (p != nullptr) (void)hipFree(p);
+    p = nullptr;
+}
+void h2d(float *dst, const float *src, size_t n) {
+    if (n) HIP_OK(hipMemcpy(dst, src, n * sizeof(float), hipMemcpyHostToDevice));
+}
+void d2h(float *dst, const float *src, size_t n) {
+    if (n) HIP_OK(hipMemcpy(dst, src, n * sizeof(float), hipMemcpyDeviceToHost));
+}
+void d2d(float *dst, const float *src, size_t n) {
+    if (n) HIP_OK(hipMemcpy(dst, src, n * sizeof(float), hipMemcpyDeviceToDevice));
+}
+}  // namespace
+
+// ---- BaseHiddenStates (reference: src/data_struct.cpp:6-95) ---------------------
+BaseHiddenStates::BaseHiddenStates(size_t n, size_t m, int device_idx)
+    : mu_a(n, 0.0f), var_a(n, 0.0f), jcb(n, 1.0f), size(n), block_size(m), device_idx(device_idx) {
+    this->actual_size = m ? n / m : 0;
+}
+
+void BaseHiddenStates::set_input_x(const std::vector<float> &mu_x, const std::vector<float> &var_x,
+                                   size_t block_size) {
+    const size_t n = mu_x.size();
+    this->actual_size = n / block_size;
+    this->block_size = block_size;
+    std::copy(mu_x.begin(), mu_x.end(), this->mu_a.begin());
+    std::fill(this->jcb.begin(), this->jcb.begin() + n, 1.0f);
+    if (var_x.size() == n)
+        std::copy(var_x.begin(), var_x.end(), this->var_a.begin());
+    else
+        std::fill(this->var_a.begin(), this->var_a.begin() + n, 0.0f);
+}
+
+void BaseHiddenStates::set_size(size_t new_size, size_t new_block_size) {
+    if (new_size > this->size) {
+        this->size = new_size;
+        this->mu_a.resize(new_size, 0.0f);
+        this->var_a.resize(new_size, 0.0f);
+        this->jcb.resize(new_size, 1.0f);
+    }
+    this->block_size = new_block_size;
+    this->actual_size = new_size / new_block_size;
+}
+
+void BaseHiddenStates::swap(BaseHiddenStates &other) {
+    std::swap(mu_a, other.mu_a);
+    std::swap(var_a, other.var_a);
+    std::swap(jcb, other.jcb);
+    std::swap(size, other.size);
+    std::swap(block_size, other.block_size);
+    std::swap(actual_size, other.actual_size);
+    std::swap(width, other.width);
+    std::swap(height, other.height);
+    std::swap(depth, other.depth);
+}
+
+void BaseHiddenStates::copy_from(const BaseHiddenStates &source, int num_data) {
+    if (num_data == -1) num_data = (int)std::min(source.size, this->size);
+    std::copy_n(source.mu_a.begin(), num_data, this->mu_a.begin());
+    std::copy_n(source.var_a.begin(), num_data, this->var_a.begin());
+    std::copy_n(source.jcb.begin(), num_data, this->jcb.begin());
+    this->block_size = source.block_size;
+    this->actual_size = source.actual_size;
+    this->width = source.width;
+    this->height = source.height;
+    this->depth = source.depth;
+}
+
+// ---- BaseDeltaStates (src/data_struct.cpp:100-160) ------------------------------
+BaseDeltaStates::BaseDeltaStates(size_t n, size_t m, int device_idx)
+    : delta_mu(n, 0.0f), delta_var(n, 0.0f), size(n), block_size(m), device_idx(device_idx) {
+    this->actual_size = m ? n / m : 0;
+}
+
+void BaseDeltaStates::reset_zeros() {
+    std::fill(delta_mu.begin(), delta_mu.end(), 0.0f);
+    std::fill(delta_var.begin(), delta_var.end(), 0.0f);
+}
+
+void BaseDeltaStates::copy_from(const BaseDeltaStates &source, int num_data) {
+    if (num_data == -1) num_data = (int)std::min(source.size, this->size);
+    std::copy_n(source.delta_mu.begin(), num_data, this->delta_mu.begin());
+    std::copy_n(source.delta_var.begin(), num_data, this->delta_var.begin());
+    this->block_size = source.block_size;
+}
+
+void BaseDeltaStates::set_size(size_t new_size, size_t new_block_size) {
+    if (new_size > this->size) {
+        this->size = new_size;
+        this->reset_zeros();
+        this->delta_mu.resize(new_size, 0.0f);
+        this->delta_var.resize(new_size, 0.0f);
+    }
+    this->block_size = new_block_size;
+    this->actual_size = new_size / new_block_size;
+}
+
+void BaseDeltaStates::swap(BaseDeltaStates &other) {
+    std::swap(delta_mu, other.delta_mu);
+    std::swap(delta_var, other.delta_var);
+    std::swap(size, other.size);
+    std::swap(block_size, other.block_size);
+    std::swap(actual_size, other.actual_size);
+}
+
+// ---- BaseTempStates / BaseBackwardStates / BaseObservation ----------------------
+BaseTempStates::BaseTempStates(size_t n, size_t m, int device_idx)
+    : tmp_1(n, 0.0f), tmp_2(n, 0.0f), size(n), block_size(m), device_idx(device_idx) {
+    this->actual_size = m ? n / m : 0;
+}
+
+void BaseTempStates::set_size(size_t new_size, size_t new_block_size) {
+    if (new_size > this->size) {
+        this->size = new_size;
+        this->tmp_1.resize(new_size, 0.0f);
+        this->tmp_2.resize(new_size, 0.0f);
+    }
+    this->block_size = new_block_size;
+    this->actual_size = new_size / new_block_size;
+}
+
+BaseBackwardStates::BaseBackwardStates(int num) : mu_a(num, 0.0f), jcb(num, 1.0f), size(num) {}
+
+void BaseBackwardStates::set_size(size_t new_size) {
+    if (new_size > this->size) {
+        this->size = new_size;
+        this->mu_a.resize(new_size, 0.0f);
+        this->jcb.resize(new_size, 1.0f);
+    }
+}
+
+void BaseObservation::set_obs(std::vector<float> &mu, std::vector<float> &var) {
+    this->mu_obs = mu;
+    this->var_obs = var;
+}
+void BaseObservation::set_selected_idx(std::vector<int> &idx) { this->selected_idx = idx; }
+
+// ---- HiddenStateHip (reference: src/data_struct_cuda.cu:9-200) ------------------
+HiddenStateHip::HiddenStateHip(size_t n, size_t m, int device_idx)
+    : BaseHiddenStates(n, m, device_idx) {
+    this->allocate_memory();
+}
+HiddenStateHip::~HiddenStateHip() { this->deallocate_memory(); }
+
+void HiddenStateHip::allocate_memory() {
+    this->deallocate_memory();
+    d_mu_a = dev_alloc(size, device_idx);
+    d_var_a = dev_alloc(size, device_idx);
+    d_jcb = dev_alloc(size, device_idx);
+    this->to_device();
+}
+void HiddenStateHip::deallocate_memory() {
+    dev_free(d_mu_a);
+    dev_free(d_var_a);
+    dev_free(d_jcb);
+}
+void HiddenStateHip::to_device() { this->chunks_to_device(this->size); }
+void HiddenStateHip::chunks_to_device(size_t n) {
+    h2d(d_mu_a, mu_a.data(), n);
+    h2d(d_var_a, var_a.data(), n);
+    h2d(d_jcb, jcb.data(), n);
+}
+void HiddenStateHip::to_host() { this->to_host(this->size); }
+void HiddenStateHip::to_host(size_t n) {
+    n = std::min(n, this->size);
+    d2h(mu_a.data(), d_mu_a, n);
+    d2h(var_a.data(), d_var_a, n);
+    d2h(jcb.data(), d_jcb, n);
+}
+void HiddenStateHip::set_input_x(const std::vector<float> &mu_x, const std::vector<float> &var_x,
+                                 size_t block_size) {
+    if (mu_x.size() > this->size)
+        LOG(LogLevel::ERROR, "Input of " + std::to_string(mu_x.size()) +
+                                 " values exceeds the state buffer of " + std::to_string(size));
+    BaseHiddenStates::set_input_x(mu_x, var_x, block_size);
+    this->chunks_to_device(mu_x.size());
+}
+void HiddenStateHip::set_size(size_t new_size, size_t new_block_size) {
+    if (new_size > this->size) {
+        BaseHiddenStates::set_size(new_size, new_block_size);
+        HIP_OK(hipDeviceSynchronize());
+        this->allocate_memory();
+    } else {
+        this->block_size = new_block_size;
+        this->actual_size = new_size / new_block_size;
+    }
+}
+void HiddenStateHip::swap(BaseHiddenStates &other) {
+    auto *o = dynamic_cast<HiddenStateHip *>(&other);
+    if (o == nullptr) LOG(LogLevel::ERROR, "Swap needs two device hidden states");
+    BaseHiddenStates::swap(other);
+    std::swap(d_mu_a, o->d_mu_a);
+    std::swap(d_var_a, o->d_var_a);
+    std::swap(d_jcb, o->d_jcb);
+}
+void HiddenStateHip::copy_from(const BaseHiddenStates &source, int num_data) {
+    auto *s = dynamic_cast<const HiddenStateHip *>(&source);
+    if (s == nullptr) LOG(LogLevel::ERROR, "Copy needs a device hidden state as source");
+    if (num_data == -1) num_data = (int)std::min(source.size, this->size);
+    d2d(d_mu_a, s->d_mu_a, num_data);
+    d2d(d_var_a, s->d_var_a, num_data);
+    d2d(d_jcb, s->d_jcb, num_data);
+    this->block_size = source.block_size;
+    this->actual_size = source.actual_size;
+    this->width = source.width;
+    this->height = source.height;
+    this->depth = source.depth;
+}
+
+// ---- DeltaStateHip (src/data_struct_cuda.cu:205-330) -----------------------------
+DeltaStateHip::DeltaStateHip(size_t n, size_t m, int device_idx) : BaseDeltaStates(n, m, device_idx) {
+    this->allocate_memory();
+}
+DeltaStateHip::~DeltaStateHip() { this->deallocate_memory(); }
+void DeltaStateHip::allocate_memory() {
+    this->deallocate_memory();
+    d_delta_mu = dev_alloc(size, device_idx);
+    d_delta_var = dev_alloc(size, device_idx);
+    this->to_device();
+}
+void DeltaStateHip::deallocate_memory() {
+    dev_free(d_delta_mu);
+    dev_free(d_delta_var);
+}
+void DeltaStateHip::to_device() {
+    h2d(d_delta_mu, delta_mu.data(), size);
+    h2d(d_delta_var, delta_var.data(), size);
+}
+void DeltaStateHip::to_host() {
+    d2h(delta_mu.data(), d_delta_mu, size);
+    d2h(delta_var.data(), d_delta_var, size);
+}
+void DeltaStateHip::reset_zeros() {
+    if (size == 0) return;
+    HIP_OK(hipMemsetAsync(d_delta_mu, 0, size * sizeof(float), nullptr));
+    HIP_OK(hipMemsetAsync(d_delta_var, 0, size * sizeof(float), nullptr));
+}
+void DeltaStateHip::copy_from(const BaseDeltaStates &source, int num_data) {
+    auto *s = dynamic_cast<const DeltaStateHip *>(&source);
+    if (s == nullptr) LOG(LogLevel::ERROR, "Copy needs a device delta state as source");
+    if (num_data == -1) num_data = (int)std::min(source.size, this->size);
+    d2d(d_delta_mu, s->d_delta_mu, num_data);
+    d2d(d_delta_var, s->d_delta_var, num_data);
+    this->block_size = source.block_size;
+}
+void DeltaStateHip::set_size(size_t new_size, size_t new_block_size) {
+    if (new_size > this->size) {
+        this->size = new_size;
+        this->delta_mu.assign(new_size, 0.0f);
+        this->delta_var.assign(new_size, 0.0f);
+        HIP_OK(hipDeviceSynchronize());
+        this->allocate_memory();
+    }
+    this->block_size = new_block_size;
+    this->actual_size = new_size / new_block_size;
+}
+void DeltaStateHip::swap(BaseDeltaStates &other) {
+    auto *o = dynamic_cast<DeltaStateHip *>(&other);
+    if (o == nullptr) LOG(LogLevel::ERROR, "Swap needs two device delta states");
+    BaseDeltaStates::swap(other);
+    std::swap(d_delta_mu, o->d_delta_mu);
+    std::swap(d_delta_var, o->d_delta_var);
+}
+
+// ---- TempStateHip / BackwardStateHip / ObservationHip ----------------------------
+TempStateHip::TempStateHip(size_t n, size_t m, int device_idx) : BaseTempStates(n, m, device_idx) {
+    this->allocate_memory();
+}
+TempStateHip::~TempStateHip() { this->deallocate_memory(); }
+void TempStateHip::allocate_memory() {
+    this->deallocate_memory();
+    d_tmp_1 = dev_alloc(size, device_idx);
+    d_tmp_2 = dev_alloc(size, device_idx);
+}
+void TempStateHip::deallocate_memory() {
+    dev_free(d_tmp_1);
+    dev_free(d_tmp_2);
+}
+void TempStateHip::set_size(size_t new_size, size_t new_block_size) {
+    if (new_size > this->size) {
+        BaseTempStates::set_size(new_size, new_block_size);
+        HIP_OK(hipDeviceSynchronize());
+        this->allocate_memory();
+    } else {
+        this->block_size = new_block_size;
+        this->actual_size = new_size / new_block_size;
+    }
+}
+
+BackwardStateHip::~BackwardStateHip() { this->deallocate_memory(); }
+void BackwardStateHip::allocate_memory() {
+    this->deallocate_memory();
+    d_mu_a = dev_alloc(size, device_idx);
+    d_jcb = dev_alloc(size, device_idx);
+}
+void BackwardStateHip::deallocate_memory() {
+    dev_free(d_mu_a);
+    dev_free(d_jcb);
+}
+void BackwardStateHip::to_host() {
+    mu_a.resize(size);
+    jcb.resize(size);
+    d2h(mu_a.data(), d_mu_a, size);
+    d2h(jcb.data(), d_jcb, size);
+}
+void BackwardStateHip::set_size(size_t new_size) {
+    if (new_size > this->size) {
+        this->size = new_size;
+        HIP_OK(hipDeviceSynchronize());
+        this->allocate_memory();
+    }
+}
+
+ObservationHip::~ObservationHip() {
+    dev_free(d_mu_obs);
+    dev_free(d_var_obs);
+    if (d_selected_idx != nullptr) (void)hipFree(d_selected_idx);
+}
+void ObservationHip::to_device() {
+    const size_t n = mu_obs.size(), ni = selected_idx.size();
+    if (n > cap_obs) {
+        HIP_OK(hipDeviceSynchronize());
+        dev_free(d_mu_obs);
+        dev_free(d_var_obs);
+        d_mu_obs = dev_alloc(n, device_idx);
+        d_var_obs = dev_alloc(n, device_idx);
+        cap_obs = n;
+    }
+    if (ni > cap_idx) {
+        HIP_OK(hipDeviceSynchronize());
+        if (d_selected_idx != nullptr) (void)hipFree(d_selected_idx);
+        HIP_OK(hipMalloc(reinterpret_cast<void **>(&d_selected_idx), ni * sizeof(int)));
+        cap_idx = ni;
+    }
+    h2d(d_mu_obs, mu_obs.data(), n);
+    h2d(d_var_obs, var_obs.data(), n);
+    if (ni)
+        HIP_OK(hipMemcpy(d_selected_idx, selected_idx.data(), ni * sizeof(int),
+                         hipMemcpyHostToDevice));
+}
+
+}  // namespace tagi_host

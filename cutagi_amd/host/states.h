@@ -1,0 +1,175 @@
+// State containers the layers exchange, mirroring the reference's
+// include/data_struct.h:14-202 (host side) and include/data_struct_cuda.cuh:9-139
+// (device side): same member names, same grow-only sizing, pointer-swapping
+// ping-pong. The *Hip classes add raw device pointers next to the host vectors;
+// the host vectors are refreshed only by an explicit to_host().
+#pragma once
+#include <hip/hip_runtime_api.h>
+
+#include <string>
+#include <tuple>
+#include <unordered_map>
+#include <vector>
+
+namespace tagi_host {
+
+using ParameterTuple =
+    std::tuple<std::vector<float>, std::vector<float>, std::vector<float>, std::vector<float>>;
+using ParameterMap = std::unordered_map<std::string, ParameterTuple>;
+
+class BaseHiddenStates {
+   public:
+    std::vector<float> mu_a, var_a, jcb;
+    size_t size = 0;         // capacity in floats
+    size_t block_size = 0;   // batch size
+    size_t actual_size = 0;  // features per sample currently held
+    size_t width = 0, height = 0, depth = 0;
+    int device_idx = 0;
+
+    BaseHiddenStates(size_t n, size_t m, int device_idx = 0);
+    BaseHiddenStates() = default;
+    virtual ~BaseHiddenStates() = default;
+    virtual std::string get_name() const { return "BaseHiddenStates"; }
+    virtual void set_input_x(const std::vector<float> &mu_x, const std::vector<float> &var_x,
+                             size_t block_size);
+    virtual void set_size(size_t size, size_t block_size);
+    virtual void swap(BaseHiddenStates &other);
+    virtual void copy_from(const BaseHiddenStates &source, int num_data = -1);
+};
+
+class BaseDeltaStates {
+   public:
+    std::vector<float> delta_mu, delta_var;
+    size_t size = 0, block_size = 0, actual_size = 0;
+    int device_idx = 0;
+
+    BaseDeltaStates(size_t n, size_t m, int device_idx = 0);
+    BaseDeltaStates() = default;
+    virtual ~BaseDeltaStates() = default;
+    virtual std::string get_name() const { return "BaseDeltaStates"; }
+    virtual void reset_zeros();
+    virtual void copy_from(const BaseDeltaStates &source, int num_data = -1);
+    virtual void set_size(size_t size, size_t block_size);
+    virtual void swap(BaseDeltaStates &other);
+};
+
+class BaseTempStates {
+   public:
+    std::vector<float> tmp_1, tmp_2;
+    size_t size = 0, block_size = 0, actual_size = 0;
+    int device_idx = 0;
+
+    BaseTempStates(size_t n, size_t m, int device_idx = 0);
+    BaseTempStates() = default;
+    virtual ~BaseTempStates() = default;
+    virtual std::string get_name() const { return "BaseTempStates"; }
+    virtual void set_size(size_t size, size_t block_size);
+};
+
+class BaseBackwardStates {
+   public:
+    std::vector<float> mu_a, jcb;
+    size_t size = 0;
+    int device_idx = 0;
+
+    explicit BaseBackwardStates(int num);
+    BaseBackwardStates() = default;
+    virtual ~BaseBackwardStates() = default;
+    virtual std::string get_name() const { return "BaseBackwardStates"; }
+    virtual void set_size(size_t size);
+};
+
+class BaseObservation {
+   public:
+    std::vector<float> mu_obs, var_obs;
+    std::vector<int> selected_idx;
+    size_t size = 0, block_size = 0, actual_size = 0, idx_size = 0;
+    int device_idx = 0;
+
+    BaseObservation() = default;
+    virtual ~BaseObservation() = default;
+    virtual std::string get_name() const { return "BaseObservation"; }
+    void set_obs(std::vector<float> &mu_obs, std::vector<float> &var_obs);
+    void set_selected_idx(std::vector<int> &selected_idx);
+};
+
+// ---- device side ---------------------------------------------------------------
+
+class HiddenStateHip : public BaseHiddenStates {
+   public:
+    float *d_mu_a = nullptr, *d_var_a = nullptr, *d_jcb = nullptr;
+
+    HiddenStateHip(size_t n, size_t m, int device_idx = 0);
+    HiddenStateHip() = default;
+    ~HiddenStateHip() override;
+    std::string get_name() const override { return "HiddenStateCuda"; }
+    void set_input_x(const std::vector<float> &mu_x, const std::vector<float> &var_x,
+                     size_t block_size) override;
+    void allocate_memory();
+    void deallocate_memory();
+    void to_device();
+    void chunks_to_device(size_t chunk_size);
+    void to_host();
+    void to_host(size_t n);  // first n entries only
+    void set_size(size_t size, size_t block_size) override;
+    void swap(BaseHiddenStates &other) override;
+    void copy_from(const BaseHiddenStates &source, int num_data = -1) override;
+};
+
+class DeltaStateHip : public BaseDeltaStates {
+   public:
+    float *d_delta_mu = nullptr, *d_delta_var = nullptr;
+
+    DeltaStateHip(size_t n, size_t m, int device_idx = 0);
+    DeltaStateHip() = default;
+    ~DeltaStateHip() override;
+    std::string get_name() const override { return "DeltaStateCuda"; }
+    void allocate_memory();
+    void deallocate_memory();
+    void to_device();
+    void to_host();
+    void reset_zeros() override;
+    void copy_from(const BaseDeltaStates &source, int num_data = -1) override;
+    void set_size(size_t size, size_t block_size) override;
+    void swap(BaseDeltaStates &other) override;
+};
+
+class TempStateHip : public BaseTempStates {
+   public:
+    float *d_tmp_1 = nullptr, *d_tmp_2 = nullptr;
+
+    TempStateHip(size_t n, size_t m, int device_idx = 0);
+    TempStateHip() = default;
+    ~TempStateHip() override;
+    std::string get_name() const override { return "TempStateCuda"; }
+    void allocate_memory();
+    void deallocate_memory();
+    void set_size(size_t size, size_t block_size) override;
+};
+
+class BackwardStateHip : public BaseBackwardStates {
+   public:
+    float *d_mu_a = nullptr, *d_jcb = nullptr;
+
+    BackwardStateHip() = default;
+    ~BackwardStateHip() override;
+    std::string get_name() const override { return "BackwardStateCuda"; }
+    void allocate_memory();
+    void deallocate_memory();
+    void to_host();
+    void set_size(size_t size) override;
+};
+
+class ObservationHip : public BaseObservation {
+   public:
+    float *d_mu_obs = nullptr, *d_var_obs = nullptr;
+    int *d_selected_idx = nullptr;
+    size_t cap_obs = 0, cap_idx = 0;
+
+    explicit ObservationHip(int device_idx = 0) { this->device_idx = device_idx; }
+    ~ObservationHip() override;
+    std::string get_name() const override { return "ObservationCuda"; }
+    void to_device();  // grows the device arrays as needed, then copies
+};
+
+}  // namespace tagi_host
