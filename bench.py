@@ -33,6 +33,8 @@ WORKLOADS = {
     "gemm": (4096, 4096, 256, "mfma"),
     "skinny": (8192, 8192, 8, "hbm"),
 }
+# Conv2d 3x3, stride 1, pad 1, 64 -> 64 channels on 32x32 maps, batch 128, no bias
+CONV = dict(fi=64, fo=64, k=3, stride=1, pad=1, pad_type=1, wi=32, B=128)
 
 
 def make_inputs(K, N, B, device):
@@ -133,6 +135,63 @@ def run_workload(name, steps, warmup):
                 ms_per_step=ms_per_step, wall_ms=wall_ms, phase_ms=phase_ms, roofline=roof)
 
 
+def run_conv(steps, warmup):
+    """Conv2d forward + backward (delta_w, delta_z) through the index tables."""
+    import torch
+    import cutagi_amd.functional as F
+    from cutagi_amd import capi
+
+    c = CONV
+    fi, fo, k, wi, B = c["fi"], c["fo"], c["k"], c["wi"], c["B"]
+    idx = capi.conv2d_build_idx(k, c["stride"], wi, wi, c["pad"], c["pad_type"], k * k * fi * fo + 1)
+    wihi, woho = wi * wi, idx["wo"] * idx["ho"]
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev)
+    g.manual_seed(0)
+    randn = lambda n: torch.randn(n, device=dev, generator=g)
+    rand = lambda n: torch.rand(n, device=dev, generator=g)
+    R = k * k * fi
+    mu_w, var_w = randn(fo * R) * R ** -0.5, torch.full((fo * R,), 1.0 / R, device=dev)
+    mu_a, var_a = randn(B * fi * wihi), rand(B * fi * wihi) * 0.09 + 0.01
+    jcb = torch.ones(B * fi * wihi, device=dev)
+    dmu, dvar = randn(B * fo * woho) * 0.1, -rand(B * fo * woho) * 1e-3
+    t = {n: torch.from_numpy(idx[n]).to(dev) for n in ("Fmwa_2", "FCzwa_1", "Szz_ud")}
+
+    def step():
+        F.conv2d_fwd(mu_w, var_w, None, None, mu_a, var_a, t["Fmwa_2"], woho, fo, wihi, fi, k, B)
+        F.conv2d_bwd_dw(var_w, None, mu_a, dmu, dvar, t["Fmwa_2"], B, fo, woho, wihi, fi, k)
+        F.conv2d_bwd_dz(mu_w, jcb, dmu, dvar, t["FCzwa_1"], t["Szz_ud"], woho, fo, wihi, fi, k,
+                        idx["h"], B)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    tflops = 14.0 * fo * (B * woho) * R / (ms * 1e-3) / 1e12
+    return dict(workload="TAGI Conv2d 3x3 s1 p1, 64->64 channels, 32x32 maps, batch 128, no bias, "
+                         "forward + backward", value=round(tflops, 3), unit="TFLOP/s",
+                frac_of_peak=round(tflops / FP32_MFMA_PEAK_TFLOPS, 4), ms_per_step=round(ms, 5))
+
+
+def calibrate_copy():
+    """A plain device copy of known size (1 GiB read + 1 GiB written), so that
+    hardware byte counters of a profiler run can be scaled."""
+    import torch
+    a = torch.empty(1 << 28, device="cuda:0")
+    b = torch.empty_like(a)
+    a.fill_(1.0)
+    torch.cuda.synchronize()
+    for _ in range(5):
+        b.copy_(a)
+    torch.cuda.synchronize()
+
+
 def cpu_baseline(name):
     """One full step of the same workload on the host cores, through the oracle."""
     import numpy as np
@@ -171,7 +230,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="gemm")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-extra", action="store_true", help="skip the secondary workload")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run a plain 1 GiB device copy (reference for byte counters)")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -216,6 +277,9 @@ def main():
             "ms_per_step": round(r["ms_per_step"], 5),
             "phase_ms": {k: round(v, 5) for k, v in r["phase_ms"].items()},
             "roofline": r["roofline"]}}
+        line["extra"]["conv"] = run_conv(max(5, args.steps // 2), args.warmup)
+    if args.calibrate:
+        calibrate_copy()
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(args.workload)
     print(json.dumps(line))

@@ -58,7 +58,9 @@ struct Tuning {
     int conv_dw_splits = -1;
     int gemv_swz = -1;
     int gemv_fwd_variant = -1;
-    int gemv_rev = -1;  // bit 0: state backward, bit 1: weight backward walk rows from the end
+    // bits 0-1: state backward, bits 2-3: weight backward; low bit of each pair:
+    // walk rows from the end, high bit: XCD-aware column mapping
+    int gemv_rev = -1;
 };
 Tuning g_tune;
 
@@ -259,7 +261,7 @@ int tagi_linear_bwd_dz(const float *mu_w, const float *jcb, const float *delta_m
         int rc = workspace_get(2 * part * sizeof(float), &ws);
         if (rc != TAGI_OK) return rc;
         TAGI_TRY(launch_gemv_dz(mu_w, delta_mu, delta_var, K, N, B, splits,
-                                (g_tune.gemv_rev >= 0 ? g_tune.gemv_rev : 0) & 1, ws, ws + part,
+                                (g_tune.gemv_rev >= 0 ? g_tune.gemv_rev : 8) & 3, ws, ws + part,
                                 stream));
         TAGI_TRY(launch_reduce_splits(EPI_SCALE, ws, ws + part, splits, B, K, jcb, nullptr,
                                       delta_mu_z, delta_var_z, K, stream));
@@ -286,7 +288,7 @@ int tagi_linear_bwd_dw(const float *var_w, const float *mu_a, const float *delta
 
     if (B <= gemv_max_batch() && k_vec) {
         TAGI_TRY(launch_gemv_dw(var_w, mu_a, delta_mu, delta_var, K, N, B,
-                                ((g_tune.gemv_rev >= 0 ? g_tune.gemv_rev : 0) >> 1) & 1,
+                                ((g_tune.gemv_rev >= 0 ? g_tune.gemv_rev : 8) >> 2) & 3,
                                 delta_mu_w, delta_var_w, stream));
         return TAGI_OK;
     }
@@ -405,7 +407,7 @@ int tagi_conv2d_bwd_dw(const float *var_w, const float *var_b, const float *mu_a
     const int red = B * woho;
     const int out_tiles = ceil_div(fo, 64) * ceil_div(ki * ki * fi, 64);
     int splits = g_tune.conv_dw_splits > 0 ? g_tune.conv_dw_splits
-                                           : ceil_div(4 * NUM_CU, out_tiles);
+                                           : ceil_div(8 * NUM_CU, out_tiles);
     const int max_splits = ceil_div(red, 256);
     if (splits > max_splits) splits = max_splits;
     if (splits < 1) splits = 1;

@@ -170,7 +170,10 @@ __global__ __launch_bounds__(FWD_WAVES * 64) void gemv_fwd_kernel(
     load(sm[0], sv[0], rot);
     __syncthreads();
     for (int kb = 0; kb < span; kb += 2 * KSTEP) {
-        const int p0 = wrap(rot + kb), p1 = p0 + KSTEP, p2 = wrap(p0 + 2 * KSTEP);
+        // (the last pair has nothing left to prefetch: it re-reads the stage that
+        // was just loaded, which is still in cache, instead of new memory)
+        const int p0 = wrap(rot + kb), p1 = p0 + KSTEP;
+        const int p2 = kb + 2 * KSTEP < span ? wrap(p0 + 2 * KSTEP) : p1;
         // the barriers keep the scheduler from sinking a stage's loads below the
         // MFMAs they are meant to overlap
         load(sm[1], sv[1], p1);
@@ -251,7 +254,19 @@ __global__ __launch_bounds__(DZ_WAVES * 64) void gemv_dz_kernel(
     const int j = lane & 3;
     // Row slices are walked from the end of the matrix: a forward pass that just
     // ran left the last weight rows in the memory-side cache.
-    const int split = rev ? gridDim.y - 1 - blockIdx.y : blockIdx.y;
+    // Workgroup -> (column slab, row slice). Consecutive workgroup ids go to the 8
+    // XCDs round-robin; mode 1 gives each XCD runs of 4 adjacent column slabs (4 KB
+    // of every row, i.e. all of its L2 channels) instead of every 8th slab.
+    int slab = blockIdx.x, split_raw = blockIdx.y;
+    if ((rev & 2) && gridDim.x % 32 == 0) {
+        const int id = blockIdx.y * gridDim.x + blockIdx.x;
+        const int xcd = id & 7, local = id >> 3;        // local: 0 .. gridDim.x*gridDim.y/8
+        const int groups = gridDim.x / 32;               // groups of 32 slabs (8 XCDs x 4)
+        const int g = local % groups, rest = local / groups;
+        slab = g * 32 + xcd * 4 + (rest & 3);
+        split_raw = rest >> 2;
+    }
+    const int split = (rev & 1) ? gridDim.y - 1 - split_raw : split_raw;
     const int n_begin = split * n_per_split;
     const int nr = min(N, n_begin + n_per_split) - n_begin;
 
@@ -270,7 +285,7 @@ __global__ __launch_bounds__(DZ_WAVES * 64) void gemv_dz_kernel(
 
     // Weight loads are never predicated: columns beyond K read column K-4 and are
     // dropped at the end, rows beyond N read row N-1 and meet zero innovations.
-    const int col = min(blockIdx.x * DZ_COLS_PER_BLOCK + 4 * lane, K - 4);
+    const int col = min(slab * DZ_COLS_PER_BLOCK + 4 * lane, K - 4);
     // rows of this wave: local [r_lo, r_hi)
     const int per_wave = n_per_split / DZ_WAVES;  // multiple of DZ_STAGE
     const int r_lo = wave * per_wave, r_hi = min(nr, r_lo + per_wave);
@@ -324,7 +339,8 @@ __global__ __launch_bounds__(DZ_WAVES * 64) void gemv_dz_kernel(
         __builtin_amdgcn_sched_barrier(0);
         multiply(st[0], r);
         __builtin_amdgcn_sched_barrier(0);
-        load(st[0], r + 2 * STAGE);
+        // (nothing left to prefetch in the last pair: re-read the cached stage)
+        load(st[0], r + 2 * STAGE < r_hi ? r + 2 * STAGE : r + STAGE);
         __builtin_amdgcn_sched_barrier(0);
         multiply(st[1], r + STAGE);
         __builtin_amdgcn_sched_barrier(0);
@@ -367,7 +383,7 @@ __global__ __launch_bounds__(DZ_WAVES * 64) void gemv_dz_kernel(
 
     if (wave == 0) {
         const int blk = lane >> 2;
-        const int c = blockIdx.x * DZ_COLS_PER_BLOCK + 16 * blk;
+        const int c = slab * DZ_COLS_PER_BLOCK + 16 * blk;
 #pragma unroll
         for (int h = 0; h < H; h++) {
             const int b = j + 4 * h;
@@ -428,8 +444,18 @@ __global__ __launch_bounds__(256) void gemv_dw_kernel(
     __shared__ __attribute__((aligned(16))) float s_dm[DW_ROWS_PER_BLOCK][BMAX];
     __shared__ __attribute__((aligned(16))) float s_dv[DW_ROWS_PER_BLOCK][BMAX];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int col = blockIdx.x * DW_COLS_PER_BLOCK + lane * 4;
-    const int n0 = (rev ? gridDim.y - 1 - blockIdx.y : blockIdx.y) * DW_ROWS_PER_BLOCK;
+    // same XCD-aware choice of the column block as in the state backward
+    int cblock = blockIdx.x, rblock = blockIdx.y;
+    if ((rev & 2) && gridDim.x % 32 == 0) {
+        const int id = blockIdx.y * gridDim.x + blockIdx.x;
+        const int xcd = id & 7, local = id >> 3;
+        const int groups = gridDim.x / 32;
+        const int g = local % groups, rest = local / groups;
+        cblock = g * 32 + xcd * 4 + (rest & 3);
+        rblock = rest >> 2;
+    }
+    const int col = cblock * DW_COLS_PER_BLOCK + lane * 4;
+    const int n0 = ((rev & 1) ? gridDim.y - 1 - rblock : rblock) * DW_ROWS_PER_BLOCK;
 
     for (int e = threadIdx.x; e < DW_ROWS_PER_BLOCK * BMAX; e += 256) {
         const int b = e / DW_ROWS_PER_BLOCK, r = e % DW_ROWS_PER_BLOCK;
