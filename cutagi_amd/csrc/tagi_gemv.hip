@@ -23,6 +23,20 @@ namespace {
 __device__ __forceinline__ float4 ld4(const float *p) {
     return *reinterpret_cast<const float4 *>(p);
 }
+// Streaming (non-temporal) load for weights that a kernel reads exactly once.
+// Measured on the forward + backward sequence at 8192 x 8192, batch 8: with the
+// forward and the state backward streaming their weights this way the whole step
+// takes 288 us instead of 307 us; the weight backward is faster with plain loads.
+__device__ __forceinline__ float4 ldnt4(const float *p) {
+    const floatx4 v = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(p));
+    return make_float4(v[0], v[1], v[2], v[3]);
+}
+#ifndef TAGI_NT_MASK
+#define TAGI_NT_MASK 3  // bit 0: forward, bit 1: state backward, bit 2: weight backward
+#endif
+__device__ __forceinline__ float4 ldw_fwd(const float *p) { return (TAGI_NT_MASK & 1) ? ldnt4(p) : ld4(p); }
+__device__ __forceinline__ float4 ldw_dz(const float *p) { return (TAGI_NT_MASK & 2) ? ldnt4(p) : ld4(p); }
+__device__ __forceinline__ float4 ldw_dw(const float *p) { return (TAGI_NT_MASK & 4) ? ldnt4(p) : ld4(p); }
 __device__ __forceinline__ float4 zero4() { return make_float4(0.f, 0.f, 0.f, 0.f); }
 __device__ __forceinline__ float comp(const float4 &v, int t) {
     return t == 0 ? v.x : t == 1 ? v.y : t == 2 ? v.z : v.w;
@@ -129,8 +143,8 @@ __global__ __launch_bounds__(FWD_WAVES * 64) void gemv_fwd_kernel(
             const int k = min(k_lane + kb + FWD_KCHUNK * c, k_last);
 #pragma unroll
             for (int rg = 0; rg < RG; rg++) {
-                m[rg][c] = ld4(wm[rg] + k);
-                v[rg][c] = ld4(wv[rg] + k);
+                m[rg][c] = ldw_fwd(wm[rg] + k);
+                v[rg][c] = ldw_fwd(wv[rg] + k);
             }
         }
     };
@@ -306,7 +320,7 @@ __global__ __launch_bounds__(DZ_WAVES * 64) void gemv_dz_kernel(
     auto load = [&](float4(&x)[STAGE], int r) {
 #pragma unroll
         for (int u = 0; u < STAGE; u++)
-            x[u] = ld4(w + (size_t)min(n_begin + r + u, n_last) * K);
+            x[u] = ldw_dz(w + (size_t)min(n_begin + r + u, n_last) * K);
     };
     auto multiply = [&](const float4(&cur)[STAGE], int r) {
 #pragma unroll
@@ -482,7 +496,7 @@ __global__ __launch_bounds__(256) void gemv_dw_kernel(
         float4 st[2][DW_STAGE];
         auto load = [&](float4(&x)[DW_STAGE], int rr) {
 #pragma unroll
-            for (int u = 0; u < DW_STAGE; u++) x[u] = ld4(src + (size_t)(rr + u) * K);
+            for (int u = 0; u < DW_STAGE; u++) x[u] = ldw_dw(src + (size_t)(rr + u) * K);
         };
         auto flush = [&](const float4(&x)[DW_STAGE], int rr) {
 #pragma unroll
