@@ -80,9 +80,14 @@ def run_workload(name, steps, warmup):
                                            out=out_db)),
     ]
 
+    out_bwd = list(out_dz + out_dw + out_db)
+
     def step():
-        for _, fn in phases:
-            fn()
+        # what one training step of the layer runs: the forward call, then the one
+        # backward call that LinearCuda::backward maps to (delta_z, delta_w, delta_b)
+        phases[0][1]()
+        F.linear_bwd(t["mu_w"], t["var_w"], t["var_b"], t["mu_a"], t["jcb"], t["delta_mu"],
+                     t["delta_var"], out=out_bwd)
 
     for _ in range(warmup):
         step()

@@ -276,9 +276,12 @@ int tagi_linear_bwd_dz(const float *mu_w, const float *jcb, const float *delta_m
     return run_gemm(GEMM_DZ, p, vec, g_tune.dz_splits, stream);
 }
 
-int tagi_linear_bwd_dw(const float *var_w, const float *mu_a, const float *delta_mu,
-                       const float *delta_var, int K, int N, int B, float *delta_mu_w,
-                       float *delta_var_w, void *stream_) {
+// Weight backward; when the bias pointers are given and the skinny-batch kernel
+// runs, that kernel also writes the bias innovations and *bias_done is set.
+static int linear_bwd_dw_impl(const float *var_w, const float *mu_a, const float *delta_mu,
+                              const float *delta_var, int K, int N, int B, float *delta_mu_w,
+                              float *delta_var_w, const float *var_b, float *delta_mu_b,
+                              float *delta_var_b, bool *bias_done, void *stream_) {
     if (!var_w || !mu_a || !delta_mu || !delta_var || !delta_mu_w || !delta_var_w)
         return TAGI_ERR_INVALID_ARG;
     if (K <= 0 || N <= 0 || B <= 0) return TAGI_ERR_INVALID_ARG;
@@ -289,7 +292,8 @@ int tagi_linear_bwd_dw(const float *var_w, const float *mu_a, const float *delta
     if (B <= gemv_max_batch() && k_vec) {
         TAGI_TRY(launch_gemv_dw(var_w, mu_a, delta_mu, delta_var, K, N, B,
                                 ((g_tune.gemv_rev >= 0 ? g_tune.gemv_rev : 8) >> 2) & 3,
-                                delta_mu_w, delta_var_w, stream));
+                                delta_mu_w, delta_var_w, var_b, delta_mu_b, delta_var_b, stream));
+        if (bias_done) *bias_done = var_b != nullptr;
         return TAGI_OK;
     }
 
@@ -300,6 +304,13 @@ int tagi_linear_bwd_dw(const float *var_w, const float *mu_a, const float *delta
     p.out0 = delta_mu_w; p.out1 = delta_var_w; p.ldo = K;
     p.e0 = var_w; p.e1 = nullptr;
     return run_gemm(GEMM_DW, p, vec, g_tune.dw_splits, stream);
+}
+
+int tagi_linear_bwd_dw(const float *var_w, const float *mu_a, const float *delta_mu,
+                       const float *delta_var, int K, int N, int B, float *delta_mu_w,
+                       float *delta_var_w, void *stream) {
+    return linear_bwd_dw_impl(var_w, mu_a, delta_mu, delta_var, K, N, B, delta_mu_w, delta_var_w,
+                              nullptr, nullptr, nullptr, nullptr, stream);
 }
 
 int tagi_linear_bwd_db(const float *var_b, const float *delta_mu, const float *delta_var, int N,
@@ -324,10 +335,13 @@ int tagi_linear_bwd(const float *mu_w, const float *var_w, const float *var_b, c
         if (rc != TAGI_OK) return rc;
     }
     if (param_update) {
-        rc = tagi_linear_bwd_dw(var_w, mu_a, delta_mu, delta_var, K, N, B, delta_mu_w, delta_var_w,
+        if (bias && (!var_b || !delta_mu_b || !delta_var_b)) return TAGI_ERR_INVALID_ARG;
+        bool bias_done = false;
+        rc = linear_bwd_dw_impl(var_w, mu_a, delta_mu, delta_var, K, N, B, delta_mu_w, delta_var_w,
+                                bias ? var_b : nullptr, delta_mu_b, delta_var_b, &bias_done,
                                 stream);
         if (rc != TAGI_OK) return rc;
-        if (bias) {
+        if (bias && !bias_done) {
             rc = tagi_linear_bwd_db(var_b, delta_mu, delta_var, N, B, delta_mu_b, delta_var_b,
                                     stream);
         }

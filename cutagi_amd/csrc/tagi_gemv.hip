@@ -284,6 +284,21 @@ __global__ __launch_bounds__(DZ_WAVES * 64) void gemv_dz_kernel(
     const int n_begin = split * n_per_split;
     const int nr = min(N, n_begin + n_per_split) - n_begin;
 
+    // Weight loads are never predicated: columns beyond K read column K-4 and are
+    // dropped at the end, rows beyond N read row N-1 and meet zero innovations.
+    const int col = min(slab * DZ_COLS_PER_BLOCK + 4 * lane, K - 4);
+    // rows of this wave: local [r_lo, r_hi)
+    const int per_wave = n_per_split / DZ_WAVES;  // multiple of DZ_STAGE
+    const int r_lo = wave * per_wave, r_hi = min(nr, r_lo + per_wave);
+    const float *w = mu_w + col;
+    const int n_last = N - 1;
+    // Two register stages used in turn, as in the forward kernel.
+    float4 st[2][STAGE];
+    auto load = [&](float4(&x)[STAGE], int r) {
+#pragma unroll
+        for (int u = 0; u < STAGE; u++)
+            x[u] = ldw_dz(w + (size_t)min(n_begin + r + u, n_last) * K);
+    };
     // stage this slice of the innovations: [sample][n], zero beyond B and nr
     const int n4s = n_per_split / 4;
     for (int e = tid; e < 4 * H * n4s; e += DZ_WAVES * 64) {
@@ -297,15 +312,6 @@ __global__ __launch_bounds__(DZ_WAVES * 64) void gemv_dz_kernel(
         *reinterpret_cast<float4 *>(s_dv + b * S + n) = v;
     }
 
-    // Weight loads are never predicated: columns beyond K read column K-4 and are
-    // dropped at the end, rows beyond N read row N-1 and meet zero innovations.
-    const int col = min(slab * DZ_COLS_PER_BLOCK + 4 * lane, K - 4);
-    // rows of this wave: local [r_lo, r_hi)
-    const int per_wave = n_per_split / DZ_WAVES;  // multiple of DZ_STAGE
-    const int r_lo = wave * per_wave, r_hi = min(nr, r_lo + per_wave);
-    const float *w = mu_w + col;
-    const int n_last = N - 1;
-
     floatx4 acc0[4][H], acc1[4][H];
 #pragma unroll
     for (int t = 0; t < 4; t++)
@@ -315,13 +321,6 @@ __global__ __launch_bounds__(DZ_WAVES * 64) void gemv_dz_kernel(
             acc1[t][h] = (floatx4){0.f, 0.f, 0.f, 0.f};
         }
 
-    // Two register stages used in turn, as in the forward kernel.
-    float4 st[2][STAGE];
-    auto load = [&](float4(&x)[STAGE], int r) {
-#pragma unroll
-        for (int u = 0; u < STAGE; u++)
-            x[u] = ldw_dz(w + (size_t)min(n_begin + r + u, n_last) * K);
-    };
     auto multiply = [&](const float4(&cur)[STAGE], int r) {
 #pragma unroll
         for (int g = 0; g < STAGE / 4; g++) {
@@ -454,7 +453,8 @@ template <int BMAX, bool EXACT>
 __global__ __launch_bounds__(256) void gemv_dw_kernel(
     const float *__restrict__ var_w, const float *__restrict__ mu_a,
     const float *__restrict__ dmu, const float *__restrict__ dvar, int K, int N, int B, int rev,
-    float *__restrict__ dmu_w, float *__restrict__ dvar_w) {
+    float *__restrict__ dmu_w, float *__restrict__ dvar_w, const float *__restrict__ var_b,
+    float *__restrict__ dmu_b, float *__restrict__ dvar_b) {
     __shared__ __attribute__((aligned(16))) float s_dm[DW_ROWS_PER_BLOCK][BMAX];
     __shared__ __attribute__((aligned(16))) float s_dv[DW_ROWS_PER_BLOCK][BMAX];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -471,6 +471,14 @@ __global__ __launch_bounds__(256) void gemv_dw_kernel(
     const int col = cblock * DW_COLS_PER_BLOCK + lane * 4;
     const int n0 = ((rev & 1) ? gridDim.y - 1 - rblock : rblock) * DW_ROWS_PER_BLOCK;
 
+    constexpr int RPW = DW_ROWS_PER_BLOCK / 4;
+    const int r0 = wave * RPW;
+    const float *src = var_w + (size_t)(n0 + r0) * K + col;
+    float4 st[2][DW_STAGE];
+    auto load = [&](float4(&x)[DW_STAGE], int rr) {
+#pragma unroll
+        for (int u = 0; u < DW_STAGE; u++) x[u] = ldw_dw(src + (size_t)(rr + u) * K);
+    };
     for (int e = threadIdx.x; e < DW_ROWS_PER_BLOCK * BMAX; e += 256) {
         const int b = e / DW_ROWS_PER_BLOCK, r = e % DW_ROWS_PER_BLOCK;
         const bool ok = b < B && n0 + r < N;
@@ -487,17 +495,25 @@ __global__ __launch_bounds__(256) void gemv_dw_kernel(
     }
     __syncthreads();
 
-    constexpr int RPW = DW_ROWS_PER_BLOCK / 4;
-    const int r0 = wave * RPW;
+    // Bias innovations ride along: the staged innovations of this row block are
+    // all that delta_b needs, so the first column block folds them over the batch.
+    if (var_b != nullptr && cblock == 0 && threadIdx.x < DW_ROWS_PER_BLOCK &&
+        n0 + (int)threadIdx.x < N) {
+        const int r = threadIdx.x;
+        float sm = 0.f, sv = 0.f;
+#pragma unroll
+        for (int b = 0; b < BMAX; b++) {
+            sm += s_dm[r][b];
+            sv += s_dv[r][b];
+        }
+        const float vb = var_b[n0 + r];
+        dmu_b[n0 + r] = sm * vb;
+        dvar_b[n0 + r] = sv * vb * vb;
+    }
+
     if (EXACT) {
-        const float *src = var_w + (size_t)(n0 + r0) * K + col;
         float *dm = dmu_w + (size_t)(n0 + r0) * K + col;
         float *dv = dvar_w + (size_t)(n0 + r0) * K + col;
-        float4 st[2][DW_STAGE];
-        auto load = [&](float4(&x)[DW_STAGE], int rr) {
-#pragma unroll
-            for (int u = 0; u < DW_STAGE; u++) x[u] = ldw_dw(src + (size_t)(rr + u) * K);
-        };
         auto flush = [&](const float4(&x)[DW_STAGE], int rr) {
 #pragma unroll
             for (int u = 0; u < DW_STAGE; u++)
@@ -639,27 +655,32 @@ hipError_t launch_gemv_dz(const float *mu_w, const float *dmu, const float *dvar
 template <int BMAX>
 static void dw_launch(bool exact, dim3 grid, hipStream_t stream, const float *var_w,
                       const float *mu_a, const float *dmu, const float *dvar, int K, int N, int B,
-                      int rev, float *dmu_w, float *dvar_w) {
+                      int rev, float *dmu_w, float *dvar_w, const float *var_b, float *dmu_b,
+                      float *dvar_b) {
     if (exact)
         hipLaunchKernelGGL((gemv_dw_kernel<BMAX, true>), grid, dim3(256), 0, stream, var_w, mu_a,
-                           dmu, dvar, K, N, B, rev, dmu_w, dvar_w);
+                           dmu, dvar, K, N, B, rev, dmu_w, dvar_w, var_b, dmu_b, dvar_b);
     else
         hipLaunchKernelGGL((gemv_dw_kernel<BMAX, false>), grid, dim3(256), 0, stream, var_w, mu_a,
-                           dmu, dvar, K, N, B, rev, dmu_w, dvar_w);
+                           dmu, dvar, K, N, B, rev, dmu_w, dvar_w, var_b, dmu_b, dvar_b);
 }
 
 hipError_t launch_gemv_dw(const float *var_w, const float *mu_a, const float *dmu,
                           const float *dvar, int K, int N, int B, int rev, float *dmu_w,
-                          float *dvar_w, hipStream_t stream) {
+                          float *dvar_w, const float *var_b, float *dmu_b, float *dvar_b,
+                          hipStream_t stream) {
     dim3 grid((K + DW_COLS_PER_BLOCK - 1) / DW_COLS_PER_BLOCK,
               (N + DW_ROWS_PER_BLOCK - 1) / DW_ROWS_PER_BLOCK);
     const bool exact = (K % DW_COLS_PER_BLOCK == 0) && (N % DW_ROWS_PER_BLOCK == 0);
     if (B <= 4)
-        dw_launch<4>(exact, grid, stream, var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w);
+        dw_launch<4>(exact, grid, stream, var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w,
+                      var_b, dmu_b, dvar_b);
     else if (B <= 8)
-        dw_launch<8>(exact, grid, stream, var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w);
+        dw_launch<8>(exact, grid, stream, var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w,
+                      var_b, dmu_b, dvar_b);
     else
-        dw_launch<16>(exact, grid, stream, var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w);
+        dw_launch<16>(exact, grid, stream, var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w,
+                      var_b, dmu_b, dvar_b);
     return hipGetLastError();
 }
 

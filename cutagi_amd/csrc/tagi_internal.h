@@ -58,7 +58,8 @@ hipError_t launch_gemv_dz(const float *mu_w, const float *dmu, const float *dvar
                           hipStream_t stream);
 hipError_t launch_gemv_dw(const float *var_w, const float *mu_a, const float *dmu,
                           const float *dvar, int K, int N, int B, int rev, float *dmu_w,
-                          float *dvar_w, hipStream_t stream);
+                          float *dvar_w, const float *var_b, float *dmu_b, float *dvar_b,
+                          hipStream_t stream);
 int gemv_fwd_variants();
 int gemv_fwd_rows_per_block(int variant);
 int gemv_fwd_k_step();
