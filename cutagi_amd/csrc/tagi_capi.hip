@@ -353,6 +353,14 @@ int tagi_linear_bwd(const float *mu_w, const float *var_w, const float *var_b, c
 // Conv2d
 // ---------------------------------------------------------------------------
 
+// The conv kernels keep element offsets inside one tensor in 32 bits and stage a
+// per-tap table of 128 columns in LDS.
+static bool conv_sizes_ok(int B, int fo, int woho, int fi, int wihi, int ki) {
+    const long long lim = 0x7fffffffLL;
+    return (long long)B * fo * woho < lim && (long long)B * fi * wihi < lim &&
+           (long long)ki * ki * fi * fo < lim && (long long)ki * ki * 128 * 4 <= 64 * 1024;
+}
+
 int tagi_conv2d_out_size(int kernel, int stride, int wi, int hi, int pad, int pad_type, int *wo,
                          int *ho) {
     if (!wo || !ho) return TAGI_ERR_INVALID_ARG;
@@ -380,6 +388,7 @@ int tagi_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b, co
     if (woho <= 0 || fo <= 0 || wihi <= 0 || fi <= 0 || ki <= 0 || B <= 0)
         return TAGI_ERR_INVALID_ARG;
     if (bias && (!mu_b || !var_b)) return TAGI_ERR_INVALID_ARG;
+    if (!conv_sizes_ok(B, fo, woho, fi, wihi, ki)) return TAGI_ERR_UNSUPPORTED;
     TAGI_TRY(launch_conv2d_fwd(mu_w, var_w, mu_b, var_b, mu_a, var_a, aidx, woho, fo, wihi, fi, ki,
                                B, bias, mu_z, var_z, static_cast<hipStream_t>(stream_)));
     return TAGI_OK;
@@ -394,12 +403,10 @@ int tagi_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *delta_m
         return TAGI_ERR_INVALID_ARG;
     if (woho <= 0 || fo <= 0 || wihi <= 0 || fi <= 0 || ki <= 0 || nr <= 0 || B <= 0)
         return TAGI_ERR_INVALID_ARG;
-    float *ws = nullptr;
-    int rc = workspace_get((size_t)ki * ki * wihi * sizeof(int), &ws);
-    if (rc != TAGI_OK) return rc;
+    if (!conv_sizes_ok(B, fo, woho, fi, wihi, ki)) return TAGI_ERR_UNSUPPORTED;
     TAGI_TRY(launch_conv2d_bwd_dz(mu_w, jcb, delta_mu_out, delta_var_out, zw_idx, zud_idx, woho,
-                                  fo, wihi, fi, ki, nr, B, reinterpret_cast<int *>(ws), delta_mu,
-                                  delta_var, static_cast<hipStream_t>(stream_)));
+                                  fo, wihi, fi, ki, nr, B, delta_mu, delta_var,
+                                  static_cast<hipStream_t>(stream_)));
     return TAGI_OK;
 }
 
@@ -414,6 +421,7 @@ int tagi_conv2d_bwd_dw(const float *var_w, const float *var_b, const float *mu_a
     if (woho <= 0 || fo <= 0 || wihi <= 0 || fi <= 0 || ki <= 0 || B <= 0)
         return TAGI_ERR_INVALID_ARG;
     if (bias && (!var_b || !delta_mu_b || !delta_var_b)) return TAGI_ERR_INVALID_ARG;
+    if (!conv_sizes_ok(B, fo, woho, fi, wihi, ki)) return TAGI_ERR_UNSUPPORTED;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
 
     // The reduction runs over all B*woho output positions while the result is

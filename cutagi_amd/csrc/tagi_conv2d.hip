@@ -11,8 +11,10 @@
 // information as the reference's FCzwa_1 / Szz_ud pair (per input pixel, the
 // list of (tap, output pixel) occurrences), re-keyed by tap so that the weight
 // operand of the state backward does not depend on the pixel and the contraction
-// is a plain GEMM. The permutations the reference runs as separate passes
-// (Jacobian, deltas) are folded into the operand addressing.
+// is a plain GEMM; each workgroup re-keys the lists of its own pixels in LDS.
+// The permutations the reference runs as separate passes (Jacobian, deltas) are
+// folded into the operand addressing. Offsets inside one tensor are 32-bit: the
+// entry points refuse tensors of 2^31 elements or more.
 #include "tagi_internal.h"
 #include "tagi_mfma_tile.h"
 
@@ -24,28 +26,67 @@ struct ConvParams {
     const float *a0, *a1;  // mu_a, var_a        [B][fi][wihi]
     const float *d0, *d1;  // delta_mu, delta_var [B][fo][woho]
     const float *e0, *e1;  // forward: mu_b, var_b [fo] (or null); states: jcb; weights: var_w
-    const int *idx;        // forward/weights: Fmwa_2 [woho][k2]; states: inv [k2][wihi]
+    const int *idx;        // forward/weights: Fmwa_2 [woho][k2]; states: FCzwa_1 [wihi][nr]
+    const int *idx2;       // states: Szz_ud [nr][wihi]
     float *out0, *out1;
-    int woho, fo, wihi, fi, k2, B;
+    int woho, fo, wihi, fi, k2, B, nr;
     int M, N, R, splits, r_per_split;
     float *ws0, *ws1;
 };
 
-template <bool VEC>
-__device__ __forceinline__ float4 load_rows_kc(const float *__restrict__ base, int ld, int row,
-                                               int rows, int r, int r_end) {
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (row >= rows) return v;
-    if (VEC) {
-        if (r < r_end) v = *reinterpret_cast<const float4 *>(base + (size_t)row * ld + r);
-    } else {
-        float c[4] = {0.f, 0.f, 0.f, 0.f};
+// All operand loads below are unconditional: an element outside the problem (or
+// a padding tap) reads element 0 of its array and is replaced by zero afterwards.
+// Loads under a branch would each wait for their index to arrive before the next
+// one is issued; this way a thread's loads of one k-tile are all in flight at once.
+
+// ---- gathered column operand staged [k][column] -------------------------------
+// The four columns of a thread are fixed for the whole kernel, only the reduction
+// index (channel, tap) moves. The prologue leaves in LDS, for every tap t and
+// local column c, the 0-based offset inside one channel map that tap t of column c
+// reads (tab[t*BN + c], -1 = nothing); Ctx keeps the image base of the columns.
+struct GatherCtx {
+    int img[4];
+    int bn;
+    const int *tab;
+};
+
+__device__ __forceinline__ float4 gather_cols(const float *__restrict__ src, const GatherCtx &ctx,
+                                              int row, int r, int r_end, int R, int k2,
+                                              int cstride) {
+    const int rr = min(r, R - 1);
+    const int ch = rr / k2, t = rr - ch * k2;
+    const int4 off = *reinterpret_cast<const int4 *>(ctx.tab + t * ctx.bn + row);
+    const int o[4] = {off.x, off.y, off.z, off.w};
+    const bool live = r < r_end;
+    float c[4];
 #pragma unroll
-        for (int j = 0; j < 4; j++)
-            if (r + j < r_end) c[j] = base[(size_t)row * ld + r + j];
-        v = make_float4(c[0], c[1], c[2], c[3]);
+    for (int j = 0; j < 4; j++) {
+        const bool ok = live && o[j] >= 0;
+        const float v = src[ok ? ctx.img[j] + ch * cstride + o[j] : 0];
+        c[j] = ok ? v : 0.f;
     }
-    return v;
+    return make_float4(c[0], c[1], c[2], c[3]);
+}
+
+// Four consecutive reduction elements of row `m` of a [rows][R] matrix.
+template <bool VEC>
+__device__ __forceinline__ float4 load_rows_kc(const float *__restrict__ base, int R, int m,
+                                               int rows, int r, int r_end) {
+    const bool row_ok = m < rows;
+    const size_t at = (size_t)(row_ok ? m : 0) * R;
+    if (VEC) {  // R % 4 == 0, 16-byte aligned base
+        const bool ok = row_ok && r < r_end;
+        const float4 v = *reinterpret_cast<const float4 *>(base + at + (ok ? r : 0));
+        return ok ? v : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    float c[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const bool ok = row_ok && r + j < r_end;
+        const float v = base[at + (ok ? r + j : 0)];
+        c[j] = ok ? v : 0.f;
+    }
+    return make_float4(c[0], c[1], c[2], c[3]);
 }
 
 // ---- forward ---------------------------------------------------------------
@@ -54,33 +95,39 @@ __device__ __forceinline__ float4 load_rows_kc(const float *__restrict__ base, i
 template <bool VEC>
 struct ConvFwdProblem {
     using Params = ConvParams;
-    static constexpr bool XK = true, YK = false;
+    using Ctx = GatherCtx;
+    static constexpr bool XK = true, YK = false, PROLOGUE_WRITES_LDS = true;
     static constexpr int NX = 2, NY = 2, FLAVOR = FLAVOR_FWD_W_ROWS;
 
-    __device__ static __forceinline__ float4 load_x(const Params &p, int arr, int m, int r,
-                                                    int r_end) {
-        return load_rows_kc<VEC>(arr ? p.w1 : p.w0, p.R, m, p.M, r, r_end);
+    static size_t extra_lds_bytes(const Params &p, int, int bn) {
+        return (size_t)p.k2 * bn * sizeof(int);
     }
-    __device__ static __forceinline__ float4 load_y(const Params &p, int arr, int n, int r,
-                                                    int r_end) {
-        float c[4] = {0.f, 0.f, 0.f, 0.f};
-        if (r < r_end) {
-            const float *__restrict__ act = arr ? p.a1 : p.a0;
-            const int ch = r / p.k2, t = r - ch * p.k2;
-            int b = n / p.woho, o = n - b * p.woho;
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                if (n + j < p.N) {
-                    const int a = p.idx[o * p.k2 + t];
-                    if (a > -1) c[j] = act[((size_t)b * p.fi + ch) * p.wihi + a - 1];
-                }
-                if (++o == p.woho) {
-                    o = 0;
-                    b++;
-                }
+    __device__ static __forceinline__ void prologue(const Params &p, Ctx &ctx, int *tab, int tid,
+                                                    int nthreads, int, int n0, int, int bn, int,
+                                                    int) {
+        for (int e = tid; e < p.k2 * bn; e += nthreads) {
+            const int t = e / bn, c = e - t * bn, n = n0 + c;
+            int off = -1;
+            if (n < p.N) {
+                const int a = p.idx[(n % p.woho) * p.k2 + t];
+                if (a > -1) off = a - 1;
             }
+            tab[e] = off;
         }
-        return make_float4(c[0], c[1], c[2], c[3]);
+        const int row = (tid % (bn / 4)) * 4;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            ctx.img[j] = n0 + row + j < p.N ? ((n0 + row + j) / p.woho) * p.fi * p.wihi : 0;
+        ctx.bn = bn;
+        ctx.tab = tab;
+    }
+    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &, int arr, int, int m0,
+                                                    int row, int r, int r_end) {
+        return load_rows_kc<VEC>(arr ? p.w1 : p.w0, p.R, m0 + row, p.M, r, r_end);
+    }
+    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &ctx, int arr, int,
+                                                    int, int row, int r, int r_end) {
+        return gather_cols(arr ? p.a1 : p.a0, ctx, row, r, r_end, p.R, p.k2, p.wihi);
     }
     __device__ static __forceinline__ void store(const Params &p, int m, int n, float a0,
                                                  float a1) {
@@ -97,51 +144,93 @@ struct ConvFwdProblem {
 
 // ---- weight backward ---------------------------------------------------------
 // rows: deltas [fo][(b,o)]; columns: gathered activations [(c,t)][(b,o)]; both
-// have the reduction (b,o) as their fast index.
+// have the reduction (b,o) as their fast index. A thread's column (channel, tap)
+// is fixed per slot; the four reduction positions of a slot move by one k-tile
+// per visit, and the table entries for the NEXT visit are requested right after
+// the current visit's gathers, so that the table lookup is never waited for.
+constexpr int DW_SLOTS = 4;  // most column slots a thread can have (32x128 tile)
+
 template <bool VEC>
 struct ConvDwProblem {
     using Params = ConvParams;
-    static constexpr bool XK = true, YK = true;
+    struct Ctx {
+        int cb[DW_SLOTS];       // channel offset ch*wihi of the slot's column, -1: no column
+        int tap[DW_SLOTS];
+        int nidx[DW_SLOTS][4];  // table entries of the next visit
+        int nimg[DW_SLOTS][4];  // image offsets b*fi*wihi of the next visit
+    };
+    static constexpr bool XK = true, YK = true, PROLOGUE_WRITES_LDS = false;
     static constexpr int NX = 2, NY = 1, FLAVOR = FLAVOR_DELTA_ROWS;
 
-    __device__ static __forceinline__ float4 load_x(const Params &p, int arr, int m, int r,
-                                                    int r_end) {
-        float c[4] = {0.f, 0.f, 0.f, 0.f};
-        if (m < p.M && r < r_end) {
-            const float *__restrict__ d = arr ? p.d1 : p.d0;
-            int b = r / p.woho, o = r - b * p.woho;
-            if (VEC) {  // woho % 4 == 0: the four positions share the image
-                return *reinterpret_cast<const float4 *>(d + ((size_t)b * p.fo + m) * p.woho + o);
-            }
+    static size_t extra_lds_bytes(const Params &, int, int) { return 0; }
+
+    __device__ static __forceinline__ void lookup(const Params &p, Ctx &ctx, int i, int r) {
+        const int rr = min(r, p.R - 1);  // positions past the end repeat the last one
+        int b = rr / p.woho, o = rr - b * p.woho;
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                if (r + j < r_end) c[j] = d[((size_t)b * p.fo + m) * p.woho + o];
-                if (++o == p.woho) {
-                    o = 0;
-                    b++;
-                }
+        for (int j = 0; j < 4; j++) {
+            ctx.nidx[i][j] = p.idx[o * p.k2 + ctx.tap[i]];
+            ctx.nimg[i][j] = b * p.fi * p.wihi;
+            if (rr + j + 1 < p.R && ++o == p.woho) {
+                o = 0;
+                b++;
+            }
+        }
+    }
+    __device__ static __forceinline__ void prologue(const Params &p, Ctx &ctx, int *, int tid,
+                                                    int nthreads, int, int n0, int, int bn,
+                                                    int r_begin, int) {
+        const int slots = bn * KT / 4 / nthreads;
+#pragma unroll
+        for (int i = 0; i < DW_SLOTS; i++) {
+            if (i >= slots) break;
+            const int f = tid + i * nthreads;
+            const int n = n0 + f / (KT / 4);
+            const int nn = min(n, p.N - 1);
+            const int ch = nn / p.k2;
+            ctx.tap[i] = nn - ch * p.k2;
+            ctx.cb[i] = n < p.N ? ch * p.wihi : -1;
+            lookup(p, ctx, i, r_begin + (f % (KT / 4)) * 4);
+        }
+    }
+    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &, int arr, int, int m0,
+                                                    int row, int r, int r_end) {
+        const float *__restrict__ d = arr ? p.d1 : p.d0;
+        const int m = m0 + row;
+        const bool row_ok = m < p.M;
+        const int mm = row_ok ? m : 0;
+        const int rr = min(r, p.R - 1);
+        int b = rr / p.woho, o = rr - b * p.woho;
+        if (VEC) {  // woho % 4 == 0: the four positions share the image
+            const bool ok = row_ok && r < r_end;
+            const float4 v = *reinterpret_cast<const float4 *>(
+                d + (ok ? ((size_t)b * p.fo + mm) * p.woho + o : 0));
+            return ok ? v : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        float c[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const bool ok = row_ok && r + j < r_end;
+            const float v = d[ok ? ((size_t)b * p.fo + mm) * p.woho + o : 0];
+            c[j] = ok ? v : 0.f;
+            if (++o == p.woho) {
+                o = 0;
+                b++;
             }
         }
         return make_float4(c[0], c[1], c[2], c[3]);
     }
-    __device__ static __forceinline__ float4 load_y(const Params &p, int arr, int n, int r,
-                                                    int r_end) {
-        float c[4] = {0.f, 0.f, 0.f, 0.f};
-        if (n < p.N && r < r_end) {
-            const int ch = n / p.k2, t = n - ch * p.k2;
-            int b = r / p.woho, o = r - b * p.woho;
+    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &ctx, int, int i, int,
+                                                    int, int r, int r_end) {
+        float c[4];
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                if (r + j < r_end) {
-                    const int a = p.idx[o * p.k2 + t];
-                    if (a > -1) c[j] = p.a0[((size_t)b * p.fi + ch) * p.wihi + a - 1];
-                }
-                if (++o == p.woho) {
-                    o = 0;
-                    b++;
-                }
-            }
+        for (int j = 0; j < 4; j++) {
+            const int a = ctx.nidx[i][j];
+            const bool ok = ctx.cb[i] >= 0 && r + j < r_end && a > -1;
+            const float v = p.a0[ok ? ctx.nimg[i][j] + ctx.cb[i] + a - 1 : 0];
+            c[j] = ok ? v : 0.f;
         }
+        lookup(p, ctx, i, r + KT);
         return make_float4(c[0], c[1], c[2], c[3]);
     }
     __device__ static __forceinline__ void store(const Params &p, int m, int n, float a0,
@@ -155,47 +244,60 @@ struct ConvDwProblem {
 
 // ---- state backward -----------------------------------------------------------
 // rows: weights re-indexed [c][(fo,t)]; columns: gathered deltas [(fo,t)][(b,p)].
+// The reference's FCzwa_1 / Szz_ud pair lists, per input pixel, the (tap, output
+// pixel) occurrences; the prologue re-keys the lists of the tile's pixels by tap
+// (each tap meets a pixel at most once), which is the table gather_cols wants.
 struct ConvDzProblem {
     using Params = ConvParams;
-    static constexpr bool XK = true, YK = false;
+    using Ctx = GatherCtx;
+    static constexpr bool XK = true, YK = false, PROLOGUE_WRITES_LDS = true;
     static constexpr int NX = 1, NY = 2, FLAVOR = FLAVOR_DELTA_COLS;
 
-    __device__ static __forceinline__ float4 load_x(const Params &p, int, int m, int r,
-                                                    int r_end) {
-        float c[4] = {0.f, 0.f, 0.f, 0.f};
-        if (m < p.M) {
-            int f = r / p.k2, t = r - f * p.k2;
+    static size_t extra_lds_bytes(const Params &p, int, int bn) {
+        return (size_t)p.k2 * bn * sizeof(int);
+    }
+    __device__ static __forceinline__ void prologue(const Params &p, Ctx &ctx, int *tab, int tid,
+                                                    int nthreads, int, int n0, int, int bn, int,
+                                                    int) {
+        for (int e = tid; e < p.k2 * bn; e += nthreads) tab[e] = -1;
+        __syncthreads();
+        for (int e = tid; e < p.nr * bn; e += nthreads) {
+            const int j = e / bn, c = e - j * bn, n = n0 + c;
+            if (n < p.N) {
+                const int px = n % p.wihi;
+                const int tap = p.idx[px * p.nr + j], o = p.idx2[j * p.wihi + px];
+                if (o > -1 && tap >= 1 && tap <= p.k2) tab[(tap - 1) * bn + c] = o - 1;
+            }
+        }
+        const int row = (tid % (bn / 4)) * 4;
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                if (r + j < r_end) c[j] = p.w0[((size_t)f * p.fi + m) * p.k2 + t];
-                if (++t == p.k2) {
-                    t = 0;
-                    f++;
-                }
+        for (int j = 0; j < 4; j++)
+            ctx.img[j] = n0 + row + j < p.N ? ((n0 + row + j) / p.wihi) * p.fo * p.woho : 0;
+        ctx.bn = bn;
+        ctx.tab = tab;
+    }
+    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &, int, int, int m0,
+                                                    int row, int r, int r_end) {
+        const int m = m0 + row;
+        const bool row_ok = m < p.M;
+        const int rr = min(r, p.R - 1);
+        int f = rr / p.k2, t = rr - f * p.k2;
+        float c[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const bool ok = row_ok && r + j < r_end;
+            const float v = p.w0[ok ? ((size_t)f * p.fi + m) * p.k2 + t : 0];
+            c[j] = ok ? v : 0.f;
+            if (++t == p.k2) {
+                t = 0;
+                f++;
             }
         }
         return make_float4(c[0], c[1], c[2], c[3]);
     }
-    __device__ static __forceinline__ float4 load_y(const Params &p, int arr, int n, int r,
-                                                    int r_end) {
-        float c[4] = {0.f, 0.f, 0.f, 0.f};
-        if (r < r_end) {
-            const float *__restrict__ d = arr ? p.d1 : p.d0;
-            const int f = r / p.k2, t = r - f * p.k2;
-            int b = n / p.wihi, px = n - b * p.wihi;
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                if (n + j < p.N) {
-                    const int o = p.idx[t * p.wihi + px];
-                    if (o > -1) c[j] = d[((size_t)b * p.fo + f) * p.woho + o];
-                }
-                if (++px == p.wihi) {
-                    px = 0;
-                    b++;
-                }
-            }
-        }
-        return make_float4(c[0], c[1], c[2], c[3]);
+    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &ctx, int arr, int,
+                                                    int, int row, int r, int r_end) {
+        return gather_cols(arr ? p.d1 : p.d0, ctx, row, r, r_end, p.R, p.k2, p.woho);
     }
     __device__ static __forceinline__ void store(const Params &p, int m, int n, float a0,
                                                  float a1) {
@@ -206,23 +308,6 @@ struct ConvDzProblem {
         p.out1[at] = a1 * e * e;
     }
 };
-
-// inv[t][p] = 0-based output pixel whose tap t reads input pixel p, else -1,
-// from FCzwa_1 (zw, [wihi][nr], 1-based taps) and Szz_ud (zud, [nr][wihi],
-// 1-based output pixels, -1 = none).
-__global__ __launch_bounds__(256) void conv_inv_fill_kernel(int *inv, int n) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i < n) inv[i] = -1;
-}
-__global__ __launch_bounds__(256) void conv_inv_build_kernel(const int *__restrict__ zw,
-                                                             const int *__restrict__ zud, int wihi,
-                                                             int nr, int k2, int *inv) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= wihi * nr) return;
-    const int px = i / nr, j = i - px * nr;
-    const int tap = zw[px * nr + j], o = zud[j * wihi + px];
-    if (o > -1 && tap >= 1 && tap <= k2) inv[(tap - 1) * wihi + px] = o - 1;
-}
 
 // Bias innovation: per-channel sums over (b, o) in two stages.
 __global__ __launch_bounds__(256) void conv_bias_partial_kernel(const float *__restrict__ dmu,
@@ -296,21 +381,15 @@ hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float 
     return launch_tiles<ConvFwdProblem<false>>(tile, p, stream);
 }
 
-// `scratch` holds ki*ki*wihi ints for the re-keyed table.
 hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *dmu,
                                 const float *dvar, const int *zw_idx, const int *zud_idx,
                                 int woho, int fo, int wihi, int fi, int ki, int nr, int B,
-                                int *scratch, float *out_dmu, float *out_dvar,
-                                hipStream_t stream) {
+                                float *out_dmu, float *out_dvar, hipStream_t stream) {
     const int k2 = ki * ki;
-    hipLaunchKernelGGL(conv_inv_fill_kernel, dim3(ceil_div(k2 * wihi, 256)), dim3(256), 0, stream,
-                       scratch, k2 * wihi);
-    hipLaunchKernelGGL(conv_inv_build_kernel, dim3(ceil_div(nr * wihi, 256)), dim3(256), 0, stream,
-                       zw_idx, zud_idx, wihi, nr, k2, scratch);
     ConvParams p = {};
-    p.w0 = mu_w; p.d0 = dmu; p.d1 = dvar; p.e0 = jcb; p.idx = scratch;
+    p.w0 = mu_w; p.d0 = dmu; p.d1 = dvar; p.e0 = jcb; p.idx = zw_idx; p.idx2 = zud_idx;
     p.out0 = out_dmu; p.out1 = out_dvar;
-    p.woho = woho; p.fo = fo; p.wihi = wihi; p.fi = fi; p.k2 = k2; p.B = B;
+    p.woho = woho; p.fo = fo; p.wihi = wihi; p.fi = fi; p.k2 = k2; p.B = B; p.nr = nr;
     p.M = fi; p.N = B * wihi; p.R = k2 * fo; p.splits = 1;
     p.r_per_split = ceil_div(p.R, KT) * KT;
     const int tile = fi > 64 ? TILE_128x128 : fi > 32 ? TILE_64x128 : TILE_32x128;

@@ -51,13 +51,19 @@ struct LinearProblem {
     static constexpr int NY = (MODE == GEMM_FWD) ? 2 : 1;
     static constexpr int FLAVOR = (MODE == GEMM_FWD) ? FLAVOR_FWD_ACT_ROWS : FLAVOR_DELTA_ROWS;
 
-    __device__ static __forceinline__ float4 load_x(const Params &p, int arr, int m, int r,
-                                                    int r_end) {
-        return load4<XK, VEC>(arr ? p.x1 : p.x0, p.ldx, m, p.M, r, r_end);
+    using Ctx = TileNoCtx;
+    static constexpr bool PROLOGUE_WRITES_LDS = false;
+    static size_t extra_lds_bytes(const Params &, int, int) { return 0; }
+    __device__ static __forceinline__ void prologue(const Params &, Ctx &, int *, int, int, int,
+                                                    int, int, int, int, int) {}
+
+    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &, int arr, int, int m0,
+                                                    int row, int r, int r_end) {
+        return load4<XK, VEC>(arr ? p.x1 : p.x0, p.ldx, m0 + row, p.M, r, r_end);
     }
-    __device__ static __forceinline__ float4 load_y(const Params &p, int arr, int n, int r,
-                                                    int r_end) {
-        return load4<YK, VEC>(arr ? p.y1 : p.y0, p.ldy, n, p.N, r, r_end);
+    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &, int arr, int, int n0,
+                                                    int row, int r, int r_end) {
+        return load4<YK, VEC>(arr ? p.y1 : p.y0, p.ldy, n0 + row, p.N, r, r_end);
     }
     __device__ static __forceinline__ void store(const Params &p, int m, int n, float a0,
                                                  float a1) {

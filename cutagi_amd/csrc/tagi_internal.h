@@ -94,8 +94,7 @@ hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float 
 hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *dmu,
                                 const float *dvar, const int *zw_idx, const int *zud_idx,
                                 int woho, int fo, int wihi, int fi, int ki, int nr, int B,
-                                int *scratch, float *out_dmu, float *out_dvar,
-                                hipStream_t stream);
+                                float *out_dmu, float *out_dvar, hipStream_t stream);
 hipError_t launch_conv2d_bwd_dw(const float *var_w, const float *mu_a, const float *dmu,
                                 const float *dvar, const int *aidx, int B, int fo, int woho,
                                 int wihi, int fi, int ki, int splits, float *ws0, float *ws1,

@@ -21,10 +21,19 @@
 //                               component t, so both sides agree on k.
 //   NX / NY                     number of arrays on each side (1 or 2)
 //   FLAVOR                      how the MFMA operands are formed, see Flavor
-//   load_x(p, arr, m, r, r_end) four elements of row-side array `arr`: rows m,
-//                               reduction r..r+3 when XK, rows m..m+3 at reduction
-//                               r otherwise; zero outside the problem
-//   load_y(p, arr, n, r, r_end) the same for the column side
+//   Ctx                         per-thread state that lives across the k-tiles
+//                               (TileNoCtx when a problem needs none)
+//   extra_lds_bytes(p, BM, BN)  host: dynamic LDS the prologue wants (index tables)
+//   prologue(p, ctx, extra, tid, nthreads, m0, n0, BM, BN, r_begin, r_end)
+//                               runs once before the first load; a barrier follows
+//   load_x(p, ctx, arr, i, m0, row, r, r_end)
+//                               four elements of row-side array `arr` for the
+//                               thread's i-th slot: row m0+row, reduction r..r+3
+//                               when XK; rows m0+row..+3 at reduction r otherwise;
+//                               zero outside the problem. Slots are visited for
+//                               consecutive k-tiles in increasing order, so Ctx may
+//                               carry what the next tile's loads need.
+//   load_y(p, ctx, arr, i, n0, row, r, r_end)   the same for the column side
 //   store(p, m, n, acc0, acc1)  final epilogue of one output element
 #pragma once
 #include <hip/hip_runtime.h>
@@ -46,6 +55,8 @@ enum Flavor {
 };
 
 constexpr int KT = 32;  // reduction elements per LDS stage
+
+struct TileNoCtx {};
 
 template <bool KC, int ROWS>
 struct TileGeom {
@@ -100,6 +111,7 @@ __global__ __launch_bounds__(WM *WN * 64) void mfma_tile_kernel(typename P::Para
 
     __shared__ __attribute__((aligned(16))) float lds_x[NX][XF];
     __shared__ __attribute__((aligned(16))) float lds_y[NY][YF];
+    extern __shared__ __attribute__((aligned(16))) int lds_extra[];
 
     const int tiles_n = (p.N + BN - 1) / BN;
     const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
@@ -122,6 +134,8 @@ __global__ __launch_bounds__(WM *WN * 64) void mfma_tile_kernel(typename P::Para
             }
 
     float4 rx[NX][LX], ry[NY][LY];
+    typename P::Ctx ctx;
+    P::prologue(p, ctx, lds_extra, tid, NT, m0, n0, BM, BN, r_begin, r_end);
 
     auto fetch = [&](int r0) {
 #pragma unroll
@@ -130,7 +144,7 @@ __global__ __launch_bounds__(WM *WN * 64) void mfma_tile_kernel(typename P::Para
             for (int i = 0; i < LX; i++) {
                 int row, k;
                 tile_pos<XK, BM>(tid + i * NT, row, k);
-                rx[a][i] = P::load_x(p, a, m0 + row, r0 + k, r_end);
+                rx[a][i] = P::load_x(p, ctx, a, i, m0, row, r0 + k, r_end);
             }
 #pragma unroll
         for (int a = 0; a < NY; a++)
@@ -138,7 +152,7 @@ __global__ __launch_bounds__(WM *WN * 64) void mfma_tile_kernel(typename P::Para
             for (int i = 0; i < LY; i++) {
                 int row, k;
                 tile_pos<YK, BN>(tid + i * NT, row, k);
-                ry[a][i] = P::load_y(p, a, n0 + row, r0 + k, r_end);
+                ry[a][i] = P::load_y(p, ctx, a, i, n0, row, r0 + k, r_end);
             }
     };
     auto commit = [&]() {
@@ -160,6 +174,7 @@ __global__ __launch_bounds__(WM *WN * 64) void mfma_tile_kernel(typename P::Para
             }
     };
 
+    if (P::PROLOGUE_WRITES_LDS) __syncthreads();
     if (r_begin < r_end) {
         fetch(r_begin);
         commit();
@@ -262,28 +277,41 @@ enum TileShape { TILE_128x128 = 0, TILE_64x128 = 1, TILE_32x128 = 2, TILE_64x64 
 inline int tile_rows(int t) { return t == TILE_128x128 ? 128 : t == TILE_32x128 ? 32 : 64; }
 inline int tile_cols(int t) { return t == TILE_64x64 ? 64 : 128; }
 
+// Dynamic LDS a problem may ask for on top of the staged tiles.
+constexpr size_t kTileExtraLdsMax = 64 * 1024;
+
+template <class P, int BM, int BN, int WM, int WN>
+hipError_t launch_tile(dim3 grid, size_t extra, const typename P::Params &p, hipStream_t stream) {
+    if (extra > 0) {
+        // static + dynamic LDS beyond 64 KB has to be allowed once per kernel
+        static bool allowed = false;
+        if (!allowed) {
+            hipError_t e = hipFuncSetAttribute(
+                reinterpret_cast<const void *>(mfma_tile_kernel<P, BM, BN, WM, WN>),
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTileExtraLdsMax);
+            if (e != hipSuccess) return e;
+            allowed = true;
+        }
+    }
+    hipLaunchKernelGGL((mfma_tile_kernel<P, BM, BN, WM, WN>), grid, dim3(WM * WN * 64), extra,
+                       stream, p);
+    return hipGetLastError();
+}
+
 template <class P>
 hipError_t launch_tiles(int tile, const typename P::Params &p, hipStream_t stream) {
     const int tiles = ((p.M + tile_rows(tile) - 1) / tile_rows(tile)) *
                       ((p.N + tile_cols(tile) - 1) / tile_cols(tile));
     dim3 grid(tiles, p.splits);
+    const size_t extra = P::extra_lds_bytes(p, tile_rows(tile), tile_cols(tile));
+    if (extra > kTileExtraLdsMax) return hipErrorInvalidValue;
     switch (tile) {
-        case TILE_128x128:
-            hipLaunchKernelGGL((mfma_tile_kernel<P, 128, 128, 2, 4>), grid, dim3(512), 0, stream, p);
-            break;
-        case TILE_64x128:
-            hipLaunchKernelGGL((mfma_tile_kernel<P, 64, 128, 2, 4>), grid, dim3(512), 0, stream, p);
-            break;
-        case TILE_32x128:
-            hipLaunchKernelGGL((mfma_tile_kernel<P, 32, 128, 1, 4>), grid, dim3(256), 0, stream, p);
-            break;
-        case TILE_64x64:
-            hipLaunchKernelGGL((mfma_tile_kernel<P, 64, 64, 2, 2>), grid, dim3(256), 0, stream, p);
-            break;
-        default:
-            return hipErrorInvalidValue;
+        case TILE_128x128: return launch_tile<P, 128, 128, 2, 4>(grid, extra, p, stream);
+        case TILE_64x128: return launch_tile<P, 64, 128, 2, 4>(grid, extra, p, stream);
+        case TILE_32x128: return launch_tile<P, 32, 128, 1, 4>(grid, extra, p, stream);
+        case TILE_64x64: return launch_tile<P, 64, 64, 2, 2>(grid, extra, p, stream);
     }
-    return hipGetLastError();
+    return hipErrorInvalidValue;
 }
 
 }  // namespace tagi
