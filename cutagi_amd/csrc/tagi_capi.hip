@@ -54,6 +54,7 @@ struct Tuning {
     int dz_splits = -1;
     int dw_splits = -1;
     int gemv_max_batch = -1;
+    int conv_dw_tile = -1;
     int tile = -1;
     int conv_dw_splits = -1;
     int gemv_swz = -1;
@@ -176,6 +177,7 @@ int tagi_hip_tune(const char *key, int value) {
     else if (!strcmp(key, "linear.dz.splits")) g_tune.dz_splits = value;
     else if (!strcmp(key, "linear.dw.splits")) g_tune.dw_splits = value;
     else if (!strcmp(key, "linear.gemv_max_batch")) g_tune.gemv_max_batch = value;
+    else if (!strcmp(key, "conv2d.dw.tile")) g_tune.conv_dw_tile = value;
     else if (!strcmp(key, "linear.tile")) g_tune.tile = value;
     else if (!strcmp(key, "conv2d.dw.splits")) g_tune.conv_dw_splits = value;
     else if (!strcmp(key, "linear.gemv.swizzle")) g_tune.gemv_swz = value;
@@ -427,9 +429,16 @@ int tagi_conv2d_bwd_dw(const float *var_w, const float *var_b, const float *mu_a
     // The reduction runs over all B*woho output positions while the result is
     // only fo x (ki*ki*fi): slice the reduction to fill the GPU.
     const int red = B * woho;
-    const int out_tiles = ceil_div(fo, 64) * ceil_div(ki * ki * fi, 64);
-    int splits = g_tune.conv_dw_splits > 0 ? g_tune.conv_dw_splits
-                                           : ceil_div(8 * NUM_CU, out_tiles);
+    const int tile = (g_tune.conv_dw_tile >= 0 && g_tune.conv_dw_tile < gemm_tile_count())
+                         ? g_tune.conv_dw_tile
+                         : 3;  // 64 x 64
+    const int out_tiles =
+        ceil_div(fo, gemm_tile_rows(tile)) * ceil_div(ki * ki * fi, gemm_tile_cols(tile));
+    // (three full rounds of resident workgroups: a partly filled last round
+    // costs as much time as a full one)
+    int splits = g_tune.conv_dw_splits > 0
+                     ? g_tune.conv_dw_splits
+                     : 3 * conv2d_bwd_dw_blocks_per_cu(tile) * NUM_CU / out_tiles;
     const int max_splits = ceil_div(red, 256);
     if (splits > max_splits) splits = max_splits;
     if (splits < 1) splits = 1;
@@ -439,7 +448,7 @@ int tagi_conv2d_bwd_dw(const float *var_w, const float *var_b, const float *mu_a
     int rc = workspace_get((2 * part + 2 * (size_t)chunks * fo) * sizeof(float), &ws);
     if (rc != TAGI_OK) return rc;
     TAGI_TRY(launch_conv2d_bwd_dw(var_w, mu_a, delta_mu_out, delta_var_out, aidx, B, fo, woho, wihi,
-                                  fi, ki, splits, ws, ws + part, delta_mu_w, delta_var_w, stream));
+                                  fi, ki, tile, splits, ws, ws + part, delta_mu_w, delta_var_w, stream));
     if (bias) {
         TAGI_TRY(launch_conv2d_bwd_db(var_b, delta_mu_out, delta_var_out, B, fo, woho, chunks,
                                       ws + 2 * part, delta_mu_b, delta_var_b, stream));

@@ -96,7 +96,7 @@ template <bool VEC>
 struct ConvFwdProblem {
     using Params = ConvParams;
     using Ctx = GatherCtx;
-    static constexpr bool XK = true, YK = false, PROLOGUE_WRITES_LDS = true;
+    static constexpr bool XK = true, YK = false, PROLOGUE_WRITES_LDS = true, SPLIT_PER_XCD = false;
     static constexpr int NX = 2, NY = 2, FLAVOR = FLAVOR_FWD_W_ROWS;
 
     static size_t extra_lds_bytes(const Params &p, int, int bn) {
@@ -159,7 +159,7 @@ struct ConvDwProblem {
         int nidx[DW_SLOTS][4];  // table entries of the next visit
         int nimg[DW_SLOTS][4];  // image offsets b*fi*wihi of the next visit
     };
-    static constexpr bool XK = true, YK = true, PROLOGUE_WRITES_LDS = false;
+    static constexpr bool XK = true, YK = true, PROLOGUE_WRITES_LDS = false, SPLIT_PER_XCD = true;
     static constexpr int NX = 2, NY = 1, FLAVOR = FLAVOR_DELTA_ROWS;
 
     static size_t extra_lds_bytes(const Params &, int, int) { return 0; }
@@ -250,7 +250,7 @@ struct ConvDwProblem {
 struct ConvDzProblem {
     using Params = ConvParams;
     using Ctx = GatherCtx;
-    static constexpr bool XK = true, YK = false, PROLOGUE_WRITES_LDS = true;
+    static constexpr bool XK = true, YK = false, PROLOGUE_WRITES_LDS = true, SPLIT_PER_XCD = false;
     static constexpr int NX = 1, NY = 2, FLAVOR = FLAVOR_DELTA_COLS;
 
     static size_t extra_lds_bytes(const Params &p, int, int bn) {
@@ -396,9 +396,40 @@ hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float
     return launch_tiles<ConvDzProblem>(tile, p, stream);
 }
 
+// Workgroups of the weight-backward kernel that one CU holds at a time.
+int conv2d_bwd_dw_blocks_per_cu(int tile) {
+    static int cached[TILE_COUNT] = {};
+    if (tile < 0 || tile >= TILE_COUNT) return 1;
+    if (cached[tile] == 0) {
+        int n = 0;
+        hipError_t e = hipErrorInvalidValue;
+        using P = ConvDwProblem<true>;
+        switch (tile) {
+            case TILE_128x128:
+                e = hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                    &n, reinterpret_cast<const void *>(mfma_tile_kernel<P, 128, 128, 2, 4>), 512, 0);
+                break;
+            case TILE_64x128:
+                e = hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                    &n, reinterpret_cast<const void *>(mfma_tile_kernel<P, 64, 128, 2, 4>), 512, 0);
+                break;
+            case TILE_32x128:
+                e = hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                    &n, reinterpret_cast<const void *>(mfma_tile_kernel<P, 32, 128, 1, 4>), 256, 0);
+                break;
+            case TILE_64x64:
+                e = hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                    &n, reinterpret_cast<const void *>(mfma_tile_kernel<P, 64, 64, 2, 2>), 256, 0);
+                break;
+        }
+        cached[tile] = (e == hipSuccess && n >= 1) ? n : 1;
+    }
+    return cached[tile];
+}
+
 hipError_t launch_conv2d_bwd_dw(const float *var_w, const float *mu_a, const float *dmu,
                                 const float *dvar, const int *aidx, int B, int fo, int woho,
-                                int wihi, int fi, int ki, int splits, float *ws0, float *ws1,
+                                int wihi, int fi, int ki, int tile, int splits, float *ws0, float *ws1,
                                 float *dmu_w, float *dvar_w, hipStream_t stream) {
     ConvParams p = {};
     p.a0 = mu_a; p.d0 = dmu; p.d1 = dvar; p.e0 = var_w; p.idx = aidx;
@@ -410,8 +441,8 @@ hipError_t launch_conv2d_bwd_dw(const float *var_w, const float *mu_a, const flo
     p.r_per_split = per;
     p.ws0 = ws0; p.ws1 = ws1;
     const bool vec = (woho % 4 == 0) && aligned16(dmu) && aligned16(dvar);
-    hipError_t e = vec ? launch_tiles<ConvDwProblem<true>>(TILE_64x64, p, stream)
-                       : launch_tiles<ConvDwProblem<false>>(TILE_64x64, p, stream);
+    hipError_t e = vec ? launch_tiles<ConvDwProblem<true>>(tile, p, stream)
+                       : launch_tiles<ConvDwProblem<false>>(tile, p, stream);
     if (e != hipSuccess) return e;
     if (p.splits > 1)
         e = launch_reduce_splits(EPI_SCALE, ws0, ws1, p.splits, p.M, p.N, var_w, nullptr, dmu_w,

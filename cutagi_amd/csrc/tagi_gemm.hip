@@ -52,7 +52,7 @@ struct LinearProblem {
     static constexpr int FLAVOR = (MODE == GEMM_FWD) ? FLAVOR_FWD_ACT_ROWS : FLAVOR_DELTA_ROWS;
 
     using Ctx = TileNoCtx;
-    static constexpr bool PROLOGUE_WRITES_LDS = false;
+    static constexpr bool PROLOGUE_WRITES_LDS = false, SPLIT_PER_XCD = false;
     static size_t extra_lds_bytes(const Params &, int, int) { return 0; }
     __device__ static __forceinline__ void prologue(const Params &, Ctx &, int *, int, int, int,
                                                     int, int, int, int, int) {}

@@ -95,9 +95,10 @@ hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float
                                 const float *dvar, const int *zw_idx, const int *zud_idx,
                                 int woho, int fo, int wihi, int fi, int ki, int nr, int B,
                                 float *out_dmu, float *out_dvar, hipStream_t stream);
+int conv2d_bwd_dw_blocks_per_cu(int tile);
 hipError_t launch_conv2d_bwd_dw(const float *var_w, const float *mu_a, const float *dmu,
                                 const float *dvar, const int *aidx, int B, int fo, int woho,
-                                int wihi, int fi, int ki, int splits, float *ws0, float *ws1,
+                                int wihi, int fi, int ki, int tile, int splits, float *ws0, float *ws1,
                                 float *dmu_w, float *dvar_w, hipStream_t stream);
 hipError_t launch_conv2d_bwd_db(const float *var_b, const float *dmu, const float *dvar, int B,
                                 int fo, int woho, int chunks, float *scratch, float *dmu_b,

@@ -21,6 +21,7 @@
 //                               component t, so both sides agree on k.
 //   NX / NY                     number of arrays on each side (1 or 2)
 //   FLAVOR                      how the MFMA operands are formed, see Flavor
+//   SPLIT_PER_XCD               map all tiles of a reduction slice to one XCD
 //   Ctx                         per-thread state that lives across the k-tiles
 //                               (TileNoCtx when a problem needs none)
 //   extra_lds_bytes(p, BM, BN)  host: dynamic LDS the prologue wants (index tables)
@@ -114,8 +115,17 @@ __global__ __launch_bounds__(WM *WN * 64) void mfma_tile_kernel(typename P::Para
     extern __shared__ __attribute__((aligned(16))) int lds_extra[];
 
     const int tiles_n = (p.N + BN - 1) / BN;
-    const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
-    const int split = blockIdx.y;
+    int tile = blockIdx.x, split = blockIdx.y;
+    if (P::SPLIT_PER_XCD && gridDim.y % 8 == 0) {
+        // Workgroups are handed to the 8 XCDs round-robin in launch order. Give all
+        // tiles of one reduction slice to one XCD, so that the operands they share
+        // are fetched into one L2 instead of eight.
+        const int id = blockIdx.y * gridDim.x + blockIdx.x;
+        const int q = id >> 3;
+        tile = q % gridDim.x;
+        split = (q / gridDim.x) * 8 + (id & 7);
+    }
+    const int m0 = (tile / tiles_n) * BM, n0 = (tile % tiles_n) * BN;
     const int r_begin = split * p.r_per_split;
     const int r_end = min(p.R, r_begin + p.r_per_split);
 
