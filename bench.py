@@ -33,6 +33,21 @@ WORKLOADS = {
     "gemm": (4096, 4096, 256, "mfma"),
     "skinny": (8192, 8192, 8, "hbm"),
 }
+# HBM bytes per launch of the dominant kernel of each workload: FETCH_SIZE and
+# WRITE_SIZE of two `rocprofv3 --pmc` runs of this script, each scaled by what the
+# same counter reads for a plain 1 GiB copy (x2.000 and x1.000; `--calibrate` adds
+# that copy to a run). Counters cannot be read from inside this process, so the
+# figures of the last profiled build are carried here; the summaries are under
+# profiles/.
+MEASURED_TRAFFIC_BYTES = {
+    ("gemm", "fwd"): 235.0e6,      # algorithmic 151.0e6
+    ("gemm", "bwd_dw"): 284.0e6,   # algorithmic 213.9e6
+    ("gemm", "bwd_dz"): 168.0e6,   # algorithmic 88.1e6
+    ("skinny", "fwd"): 562.5e6,    # algorithmic 536.9e6
+    ("skinny", "bwd_dz"): 286.5e6, # algorithmic 268.4e6
+    ("skinny", "bwd_dw"): 818.4e6, # algorithmic 805.3e6
+}
+
 # Conv2d 3x3, stride 1, pad 1, 64 -> 64 channels on 32x32 maps, batch 128, no bias
 CONV = dict(fi=64, fo=64, k=3, stride=1, pad=1, pad_type=1, wi=32, B=128)
 
@@ -135,6 +150,7 @@ def run_workload(name, steps, warmup):
         value = 6.0 * N * K * 4 / (ms_per_step * 1e-3) / 1e9
         unit = "GB/s"
         peak = HBM_PEAK_GBS
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get((name, dominant))
     roof["kernel_ms"] = round(phase_ms[dominant], 5)
     return dict(name=name, K=K, N=N, B=B, value=value, unit=unit, frac_of_peak=value / peak,
                 ms_per_step=ms_per_step, wall_ms=wall_ms, phase_ms=phase_ms, roofline=roof)

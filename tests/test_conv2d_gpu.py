@@ -8,7 +8,7 @@ pytestmark = pytest.mark.gpu
 
 # (kernel, stride, pad, pad_type, wi, fi, fo, B): the geometries of the ResNet-18
 # configuration (3x3 s1 p1, 3x3 s2 p1 type 2, 2x2 s2 shortcut), odd channel
-# counts (27 = 3*9 reduction, the first ResNet conv), 1x1 and 5x5 kernels.
+# counts (27 = 3*9 reduction, the first ResNet conv), 1x1, 5x5 and 7x7 kernels.
 GEOMS = [
     (3, 1, 1, 1, 8, 4, 8, 3),
     (3, 1, 1, 1, 16, 3, 16, 2),
@@ -20,6 +20,7 @@ GEOMS = [
     (3, 1, 1, 1, 32, 16, 32, 2),
     (3, 1, 1, 1, 12, 70, 66, 1),
     (4, 2, 1, 1, 10, 3, 5, 2),
+    (7, 2, 3, 1, 17, 3, 40, 2),  # per-tap table + staged tiles exceed 64 KB of LDS
 ]
 
 
