@@ -199,6 +199,97 @@ class Oracle:
                              _fp(jcb), _fp(var_a))
         return mu_a, var_a, jcb
 
+    # ---- mixture relu -----------------------------------------------------
+    def mixture_relu_fwd(self, mu_z, var_z, threads=1):
+        n = mu_z.size
+        mu_a, jcb, var_a = (np.empty(n, np.float32) for _ in range(3))
+        self._fn("mixture_relu_fwd")(_fp(mu_z), _fp(var_z), n, threads, _fp(mu_a), _fp(jcb),
+                                     _fp(var_a))
+        return mu_a, var_a, jcb
+
+    # ---- batch norm ---------------------------------------------------------
+    def batchnorm2d_stats(self, mu_a, var_a, wihi, fi, B, momentum, mu_ra, var_ra, threads=1):
+        """Returns (mu_s, var_s, mu_ra, var_ra): batch statistics and the updated
+        running averages (the inputs mu_ra/var_ra are not modified)."""
+        mu_s, var_s, tmp = (np.empty(fi, np.float32) for _ in range(3))
+        mu_ra, var_ra = f32(mu_ra).copy(), f32(var_ra).copy()
+        self._fn("batchnorm2d_stats")(_fp(mu_a), _fp(var_a), wihi, fi, B,
+                                      ctypes.c_float(momentum), threads, _fp(tmp), _fp(mu_s),
+                                      _fp(var_s), _fp(mu_ra), _fp(var_ra))
+        return mu_s, var_s, mu_ra, var_ra
+
+    def batchnorm2d_fwd(self, mu_w, var_w, mu_b, var_b, mu_a, var_a, mu_norm, var_norm, eps,
+                        wihi, fi, B, threads=1):
+        mu_z, var_z = np.empty(B * fi * wihi, np.float32), np.empty(B * fi * wihi, np.float32)
+        self._fn("batchnorm2d_fwd")(_fp(mu_w), _fp(var_w), _fp(mu_b), _fp(var_b), _fp(mu_a),
+                                    _fp(var_a), _fp(mu_norm), _fp(var_norm),
+                                    int(mu_b is not None), ctypes.c_float(eps), wihi, fi, B,
+                                    threads, _fp(mu_z), _fp(var_z))
+        return mu_z, var_z
+
+    def batchnorm2d_bwd_dz(self, mu_w, jcb, var_norm, dmu, dvar, eps, wihi, fi, B, threads=1):
+        om, ov = np.empty(B * fi * wihi, np.float32), np.empty(B * fi * wihi, np.float32)
+        self._fn("batchnorm2d_bwd_dz")(_fp(mu_w), _fp(jcb), _fp(var_norm), _fp(dmu), _fp(dvar),
+                                       ctypes.c_float(eps), wihi, fi, B, threads, _fp(om),
+                                       _fp(ov))
+        return om, ov
+
+    def batchnorm2d_bwd_dw(self, var_w, var_b, mu_a, mu_norm, var_norm, dmu, dvar, eps, wihi,
+                           fi, B, threads=1):
+        n = B * fi * wihi
+        t1, t2 = np.empty(n, np.float32), np.empty(n, np.float32)
+        ow, ovw, ob, ovb = (np.zeros(fi, np.float32) for _ in range(4))
+        bias = var_b is not None
+        self._fn("batchnorm2d_bwd_dw")(_fp(var_w), _fp(var_b), _fp(mu_a), _fp(mu_norm),
+                                       _fp(var_norm), _fp(dmu), _fp(dvar), ctypes.c_float(eps),
+                                       wihi, fi, B, int(bias), threads, _fp(t1), _fp(t2),
+                                       _fp(ow), _fp(ovw), _fp(ob), _fp(ovb))
+        return (ow, ovw, ob, ovb) if bias else (ow, ovw, None, None)
+
+    # ---- average pooling -------------------------------------------------------
+    def avgpool2d_build_idx(self, kernel, stride, wi, hi, pad, pad_type):
+        wo, ho = self.conv2d_out_size(kernel, stride, wi, hi, pad, pad_type)
+        k2 = kernel * kernel
+        pool = np.zeros(wo * ho * k2, np.int32)
+        zud = np.zeros(wi * hi * k2 + 16, np.int32)
+        w, h, ov = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
+        rc = self._fn("avgpool2d_build_idx")(kernel, stride, wi, hi, wo, ho, pad, pad_type,
+                                             _ip(pool), _ip(zud), ctypes.byref(w),
+                                             ctypes.byref(h), ctypes.byref(ov))
+        if rc != 0:
+            raise RuntimeError("avgpool2d_build_idx failed (%d)" % rc)
+        return dict(pool_idx=pool, z_ud_idx=zud[:w.value * h.value].copy(), w=w.value,
+                    h=h.value, overlap=bool(ov.value), wo=wo, ho=ho)
+
+    def avgpool2d_fwd(self, mu_a, var_a, pool_idx, woho, wihi, ki, n_out, overlap, threads=1):
+        mu_z, var_z = np.empty(n_out, np.float32), np.empty(n_out, np.float32)
+        self._fn("avgpool2d_fwd")(_fp(mu_a), _fp(var_a), _ip(pool_idx), woho, wihi, ki, n_out,
+                                  mu_a.size, int(overlap), threads, _fp(mu_z), _fp(var_z))
+        return mu_z, var_z
+
+    def avgpool2d_bwd_dz(self, jcb, dmu, dvar, z_ud_idx, woho, wihi, ki, nr, wo, overlap,
+                         threads=1):
+        n_in = jcb.size
+        om, ov = np.zeros(n_in, np.float32), np.zeros(n_in, np.float32)
+        zud = z_ud_idx if z_ud_idx.size else np.zeros(1, np.int32)
+        self._fn("avgpool2d_bwd_dz")(_fp(jcb), _fp(dmu), _fp(dvar), _ip(zud), woho, wihi, ki, nr,
+                                     wo, n_in, dmu.size, int(overlap), threads, _fp(om),
+                                     _fp(ov))
+        return om, ov
+
+    # ---- residual connection ----------------------------------------------------
+    def add_shortcut(self, mu_s, var_s, mu_a, var_a):
+        mu_a, var_a = f32(mu_a).copy(), f32(var_a).copy()
+        self._fn("add_shortcut")(_fp(mu_s), _fp(var_s), mu_a.size, _fp(mu_a), _fp(var_a))
+        return mu_a, var_a
+
+    def add_shortcut_delta(self, mu_s, var_s, jcb_s, mu_a, var_a):
+        mu_a, var_a = f32(mu_a).copy(), f32(var_a).copy()
+        self._fn("add_shortcut_delta")(_fp(mu_s), _fp(var_s), _fp(jcb_s), mu_a.size, _fp(mu_a),
+                                       _fp(var_a))
+        return mu_a, var_a
+
+
 
 def load():
     path = os.path.join(_HERE, "liboracle.so")

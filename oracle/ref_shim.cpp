@@ -14,6 +14,87 @@
 #include "base_output_updater.h"
 #include "conv2d_layer.h"
 #include "linear_layer.h"
+#include "pooling_layer.h"
+
+// Free functions the reference defines in its .cpp files without declaring them
+// in a header (src/batchnorm_layer.cpp:15-354,457-775, src/resnet_block.cpp:8-31,
+// src/common.cpp:360-378): declared here so that they can be called.
+void running_mean_var(const std::vector<float> &mu_s, const std::vector<float> &var_s,
+                      float momentum, int start_chunk, int end_chunk,
+                      std::vector<float> &mu_ra, std::vector<float> &var_ra);
+void running_mean_var_mp(const std::vector<float> &mu_s, const std::vector<float> &var_s,
+                         float momentum, int num_states, const int num_threads,
+                         std::vector<float> &mu_ra, std::vector<float> &var_ra);
+void batchnorm2d_stat_mean_var(const std::vector<float> &mu_a, const std::vector<float> &var_a,
+                               int wihi, int fi, int batch_size, int start_chunk, int end_chunk,
+                               std::vector<float> &mu_s, std::vector<float> &var_s);
+void batchnorm2d_stat_mean_var_mp(const std::vector<float> &mu_a,
+                                  const std::vector<float> &var_a, int wihi, int fi,
+                                  int batch_size, const int num_threads,
+                                  std::vector<float> &mu_s, std::vector<float> &var_s);
+void batchnorm2d_sample_var(const std::vector<float> &mu_a, const std::vector<float> &mu_s,
+                            const std::vector<float> &var_s, int wihi, int fi, int batch_size,
+                            int start_chunk, int end_chunk, std::vector<float> &var);
+void batchnorm2d_sample_var_mp(const std::vector<float> &mu_a, const std::vector<float> &mu_s,
+                               const std::vector<float> &var_s, int wihi, int fi,
+                               int batch_size, const int num_threads, std::vector<float> &var);
+void batchnorm2d_fwd_mean_var(const std::vector<float> &mu_w, const std::vector<float> &var_w,
+                              const std::vector<float> &mu_b, const std::vector<float> &var_b,
+                              const std::vector<float> &mu_a, const std::vector<float> &var_a,
+                              const std::vector<float> &mu_ra, const std::vector<float> &var_ra,
+                              bool bias, float epsilon, int wihi, int fi, int batch_size,
+                              int start_chunk, int end_chunk, std::vector<float> &mu_z,
+                              std::vector<float> &var_z);
+void batchnorm2d_fwd_mean_var_mp(const std::vector<float> &mu_w, const std::vector<float> &var_w,
+                                 const std::vector<float> &mu_b, const std::vector<float> &var_b,
+                                 const std::vector<float> &mu_a, const std::vector<float> &var_a,
+                                 const std::vector<float> &mu_ra,
+                                 const std::vector<float> &var_ra, bool bias, float epsilon,
+                                 int wihi, int fi, int batch_size, const int num_threads,
+                                 std::vector<float> &mu_z, std::vector<float> &var_z);
+void batchnorm2d_bwd_delta_z(const std::vector<float> &mu_w, const std::vector<float> &jcb,
+                             const std::vector<float> &var_ra,
+                             const std::vector<float> &delta_mu_out,
+                             const std::vector<float> &delta_var_out, float epsilon, int wihi,
+                             int fi, int batch_size, int start_chunk, int end_chunk,
+                             std::vector<float> &delta_mu, std::vector<float> &delta_var);
+void batchnorm2d_bwd_delta_z_mp(const std::vector<float> &mu_w, const std::vector<float> &jcb,
+                                const std::vector<float> &var_ra,
+                                const std::vector<float> &delta_mu_out,
+                                const std::vector<float> &delta_var_out, float epsilon, int wihi,
+                                int fi, int batch_size, const int num_threads,
+                                std::vector<float> &delta_mu, std::vector<float> &delta_var);
+void batchnorm2d_bwd_delta_w(const std::vector<float> &var_w, const std::vector<float> &mu_a,
+                             const std::vector<float> &mu_ra, const std::vector<float> &var_ra,
+                             const std::vector<float> &delta_mu_out,
+                             const std::vector<float> &delta_var_out, float epsilon, int wihi,
+                             int fi, int batch_size, int start_chunk, int end_chunk,
+                             std::vector<float> &delta_mu_w, std::vector<float> &delta_var_w);
+void batchnorm2d_bwd_delta_w_mp(const std::vector<float> &var_w, const std::vector<float> &mu_a,
+                                const std::vector<float> &mu_ra,
+                                const std::vector<float> &var_ra,
+                                const std::vector<float> &delta_mu_out,
+                                const std::vector<float> &delta_var_out, float epsilon, int wihi,
+                                int fi, int batch_size, const int num_threads,
+                                std::vector<float> &delta_mu_w, std::vector<float> &delta_var_w);
+void batchnorm2d_bwd_delta_b(const std::vector<float> &var_b,
+                             const std::vector<float> &delta_mu_out,
+                             const std::vector<float> &delta_var_out, float epsilon, int wihi,
+                             int fi, int start_chunk, int end_chunk,
+                             std::vector<float> &delta_mu_b, std::vector<float> &delta_var_b);
+void batchnorm2d_bwd_delta_b_mp(const std::vector<float> &var_b,
+                                const std::vector<float> &delta_mu_out,
+                                const std::vector<float> &delta_var_out, float epsilon, int wihi,
+                                int fi, int batch_size, const int num_threads,
+                                std::vector<float> &delta_mu_b, std::vector<float> &delta_var_b);
+void delta_param_sum(const std::vector<float> &delta_mu_e, const std::vector<float> &delta_var_e,
+                     int wihi, int fi, int batch_size, std::vector<float> &delta_mu,
+                     std::vector<float> &delta_var);
+void add_shortcut_mean_var(const std::vector<float> &mu_s, const std::vector<float> &var_s,
+                           int num_states, std::vector<float> &mu_a, std::vector<float> &var_a);
+void add_shortcut_delta(const std::vector<float> &mu_s, const std::vector<float> &var_s,
+                        const std::vector<float> &jcb_s, int num_states,
+                        std::vector<float> &mu_a, std::vector<float> &var_a);
 
 namespace {
 std::vector<float> vec(const float *p, size_t n) {
@@ -243,6 +324,186 @@ void ref_relu_fwd(const float *mu_z, const float *var_z, int n, float *mu_a, flo
     relu_mean_var(mz, vz, 0, n, ma, jc, va);
     put(ma, mu_a);
     put(jc, jcb);
+    put(va, var_a);
+}
+
+void ref_mixture_relu_fwd(const float *mu_z, const float *var_z, int n, int threads,
+                          float *mu_a, float *jcb, float *var_a) {
+    auto mz = vec(mu_z, n), vz = vec(var_z, n);
+    std::vector<float> ma(n), jc(n), va(n);
+    if (threads > 1)
+        mixture_relu_mean_var_mp(mz, vz, n, threads, ma, jc, va);
+    else
+        mixture_relu_mean_var(mz, vz, 0, n, ma, jc, va);
+    put(ma, mu_a);
+    put(jc, jcb);
+    put(va, var_a);
+}
+
+void ref_batchnorm2d_stats(const float *mu_a, const float *var_a, int wihi, int fi, int B,
+                           float momentum, int threads, float *var_s_tmp, float *mu_s,
+                           float *var_s, float *mu_ra, float *var_ra) {
+    const size_t n = (size_t)B * fi * wihi;
+    auto ma = vec(mu_a, n), va = vec(var_a, n);
+    std::vector<float> ms(fi), tmp(fi), vs(fi);
+    auto mra = vec(mu_ra, fi), vra = vec(var_ra, fi);
+    if (threads > 1) {
+        batchnorm2d_stat_mean_var_mp(ma, va, wihi, fi, B, threads, ms, tmp);
+        batchnorm2d_sample_var_mp(ma, ms, tmp, wihi, fi, B, threads, vs);
+        running_mean_var_mp(ms, vs, momentum, fi, threads, mra, vra);
+    } else {
+        batchnorm2d_stat_mean_var(ma, va, wihi, fi, B, 0, fi, ms, tmp);
+        batchnorm2d_sample_var(ma, ms, tmp, wihi, fi, B, 0, fi, vs);
+        running_mean_var(ms, vs, momentum, 0, fi, mra, vra);
+    }
+    put(tmp, var_s_tmp);
+    put(ms, mu_s);
+    put(vs, var_s);
+    put(mra, mu_ra);
+    put(vra, var_ra);
+}
+
+void ref_batchnorm2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
+                         const float *var_b, const float *mu_a, const float *var_a,
+                         const float *mu_norm, const float *var_norm, int bias, float epsilon,
+                         int wihi, int fi, int B, int threads, float *mu_z, float *var_z) {
+    const size_t n = (size_t)B * fi * wihi;
+    auto mw = vec(mu_w, fi), vw = vec(var_w, fi);
+    auto mb = vec(bias ? mu_b : nullptr, fi), vb = vec(bias ? var_b : nullptr, fi);
+    auto ma = vec(mu_a, n), va = vec(var_a, n), mn = vec(mu_norm, fi), vn = vec(var_norm, fi);
+    std::vector<float> mz(n), vz(n);
+    if (threads > 1)
+        batchnorm2d_fwd_mean_var_mp(mw, vw, mb, vb, ma, va, mn, vn, bias != 0, epsilon, wihi, fi,
+                                    B, threads, mz, vz);
+    else
+        batchnorm2d_fwd_mean_var(mw, vw, mb, vb, ma, va, mn, vn, bias != 0, epsilon, wihi, fi, B,
+                                 0, fi * B, mz, vz);
+    put(mz, mu_z);
+    put(vz, var_z);
+}
+
+void ref_batchnorm2d_bwd_dz(const float *mu_w, const float *jcb, const float *var_norm,
+                            const float *delta_mu_out, const float *delta_var_out,
+                            float epsilon, int wihi, int fi, int B, int threads,
+                            float *delta_mu, float *delta_var) {
+    const size_t n = (size_t)B * fi * wihi;
+    auto mw = vec(mu_w, fi), jc = vec(jcb, n), vn = vec(var_norm, fi);
+    auto dm = vec(delta_mu_out, n), dv = vec(delta_var_out, n);
+    std::vector<float> om(n), ov(n);
+    if (threads > 1)
+        batchnorm2d_bwd_delta_z_mp(mw, jc, vn, dm, dv, epsilon, wihi, fi, B, threads, om, ov);
+    else
+        batchnorm2d_bwd_delta_z(mw, jc, vn, dm, dv, epsilon, wihi, fi, B, 0, fi * B, om, ov);
+    put(om, delta_mu);
+    put(ov, delta_var);
+}
+
+void ref_batchnorm2d_bwd_dw(const float *var_w, const float *var_b, const float *mu_a,
+                            const float *mu_norm, const float *var_norm,
+                            const float *delta_mu_out, const float *delta_var_out,
+                            float epsilon, int wihi, int fi, int B, int bias, int threads,
+                            float *tmp_1, float *tmp_2, float *delta_mu_w, float *delta_var_w,
+                            float *delta_mu_b, float *delta_var_b) {
+    const size_t n = (size_t)B * fi * wihi;
+    auto vw = vec(var_w, fi), vb = vec(bias ? var_b : nullptr, fi), ma = vec(mu_a, n);
+    auto mn = vec(mu_norm, fi), vn = vec(var_norm, fi);
+    auto dm = vec(delta_mu_out, n), dv = vec(delta_var_out, n);
+    std::vector<float> t1(n), t2(n), ow(fi), ovw(fi), ob(fi), ovb(fi);
+    if (threads > 1)
+        batchnorm2d_bwd_delta_w_mp(vw, ma, mn, vn, dm, dv, epsilon, wihi, fi, B, threads, t1, t2);
+    else
+        batchnorm2d_bwd_delta_w(vw, ma, mn, vn, dm, dv, epsilon, wihi, fi, B, 0, fi * B, t1, t2);
+    delta_param_sum(t1, t2, wihi, fi, B, ow, ovw);
+    put(ow, delta_mu_w);
+    put(ovw, delta_var_w);
+    if (!bias) return;
+    if (threads > 1)
+        batchnorm2d_bwd_delta_b_mp(vb, dm, dv, epsilon, wihi, fi, B, threads, t1, t2);
+    else
+        batchnorm2d_bwd_delta_b(vb, dm, dv, epsilon, wihi, fi, 0, fi * B, t1, t2);
+    delta_param_sum(t1, t2, wihi, fi, B, ob, ovb);
+    put(ob, delta_mu_b);
+    put(ovb, delta_var_b);
+}
+
+int ref_avgpool2d_build_idx(int kernel, int stride, int wi, int hi, int wo, int ho, int pad,
+                            int pad_type, int *pool_idx, int *z_ud_idx, int *w, int *h,
+                            int *overlap) {
+    try {
+        Pool2dIndex idx = get_pool_index(kernel, stride, wi, hi, wo, ho, pad, pad_type, -1, -1);
+        std::memcpy(pool_idx, idx.pool_idx.data(), idx.pool_idx.size() * sizeof(int));
+        std::memcpy(z_ud_idx, idx.z_ud_idx.data(), idx.z_ud_idx.size() * sizeof(int));
+        // AvgPool2d::lazy_index_init (src/pooling_layer.cpp:186-210)
+        *overlap = !(kernel == stride || kernel == wi);
+        *w = idx.z_ud_idx.empty() ? 0 : idx.w;
+        *h = idx.z_ud_idx.empty() ? 0 : idx.h;
+        return 0;
+    } catch (const std::exception &) {
+        return -1;
+    }
+}
+
+void ref_avgpool2d_fwd(const float *mu_a, const float *var_a, const int *pool_idx, int woho,
+                       int wihi, int ki, int n_out, int n_in, int overlap, int threads,
+                       float *mu_z, float *var_z) {
+    auto ma = vec(mu_a, n_in), va = vec(var_a, n_in);
+    auto idx = ivec(pool_idx, (size_t)ki * ki * woho);
+    std::vector<float> mz(n_out), vz(n_out);
+    if (overlap) {
+        if (threads > 1)
+            avgpool2d_fwd_overlapped_mean_var_mp(ma, va, idx, woho, wihi, ki, n_out, n_in + 1,
+                                                 threads, mz, vz);
+        else
+            avgpool2d_fwd_overlapped_mean_var(ma, va, idx, woho, wihi, ki, n_out, n_in + 1, 0,
+                                              n_out, mz, vz);
+    } else {
+        if (threads > 1)
+            avgpool2d_fwd_mean_var_mp(ma, va, idx, woho, wihi, ki, n_out, threads, mz, vz);
+        else
+            avgpool2d_fwd_mean_var(ma, va, idx, woho, wihi, ki, n_out, 0, n_out, mz, vz);
+    }
+    put(mz, mu_z);
+    put(vz, var_z);
+}
+
+void ref_avgpool2d_bwd_dz(const float *jcb, const float *delta_mu_out,
+                          const float *delta_var_out, const int *z_ud_idx, int woho, int wihi,
+                          int ki, int nr, int wo, int n_in, int n_out, int overlap, int threads,
+                          float *delta_mu, float *delta_var) {
+    auto jc = vec(jcb, n_in), dm = vec(delta_mu_out, n_out), dv = vec(delta_var_out, n_out);
+    std::vector<float> om(n_in), ov(n_in);
+    if (overlap) {
+        auto idx = ivec(z_ud_idx, (size_t)nr * wihi);
+        if (threads > 1)
+            avgpool2d_bwd_overlapped_delta_z_mp(jc, dm, dv, idx, woho, wihi, ki, nr, n_in,
+                                                n_out + 1, threads, om, ov);
+        else
+            avgpool2d_bwd_overlapped_delta_z(jc, dm, dv, idx, woho, wihi, ki, nr, n_in,
+                                             n_out + 1, 0, n_in, om, ov);
+    } else {
+        const int nums = n_in / (ki * wo);  // src/pooling_layer.cpp:162-164
+        if (threads > 1)
+            avgpool2d_bwd_delta_z_mp(jc, dm, dv, wo, ki, nums, threads, om, ov);
+        else
+            avgpool2d_bwd_delta_z(jc, dm, dv, wo, ki, nums, 0, ki * wo * nums, om, ov);
+    }
+    put(om, delta_mu);
+    put(ov, delta_var);
+}
+
+void ref_add_shortcut(const float *mu_s, const float *var_s, int n, float *mu_a, float *var_a) {
+    auto ms = vec(mu_s, n), vs = vec(var_s, n), ma = vec(mu_a, n), va = vec(var_a, n);
+    add_shortcut_mean_var(ms, vs, n, ma, va);
+    put(ma, mu_a);
+    put(va, var_a);
+}
+
+void ref_add_shortcut_delta(const float *mu_s, const float *var_s, const float *jcb_s, int n,
+                            float *mu_a, float *var_a) {
+    auto ms = vec(mu_s, n), vs = vec(var_s, n), js = vec(jcb_s, n);
+    auto ma = vec(mu_a, n), va = vec(var_a, n);
+    add_shortcut_delta(ms, vs, js, n, ma, va);
+    put(ma, mu_a);
     put(va, var_a);
 }
 

@@ -535,4 +535,285 @@ void oracle_relu_fwd(const float *mu_z, const float *var_z, int n, float *mu_a,
     }
 }
 
+// ---------------------------------------------------------------------------
+// MixtureReLU
+// ---------------------------------------------------------------------------
+
+// src/activation.cpp:152-178; normcdf_cpu is src/common.cpp:315-319.
+void oracle_mixture_relu_fwd(const float *mu_z, const float *var_z, int n,
+                             int threads, float *mu_a, float *jcb,
+                             float *var_a) {
+    fan_out(n, threads, [=](int lo, int hi) {
+        constexpr float SQRT_2PI = 2.5066282746310002f;
+        for (int i = lo; i < hi; i++) {
+            const float m = mu_z[i];
+            const float sd = powf(var_z[i], 0.5);
+            const float alpha = m / sd;
+            const float pdf = (1.0f / SQRT_2PI) * expf(-0.5f * alpha * alpha);
+            const float cdf = 0.5f * erfcf(-alpha * 0.7071067811865475f);
+            const float t = m * cdf + sd * pdf;
+            mu_a[i] = fmaxf(0.000001f, t);
+            var_a[i] = fmaxf(0.000001f, -t * t + 2 * t * m - m * sd * pdf +
+                                            (var_z[i] - m * m) * cdf);
+            jcb[i] = cdf;
+        }
+    });
+}
+
+// ---------------------------------------------------------------------------
+// BatchNorm2d
+// ---------------------------------------------------------------------------
+
+void oracle_batchnorm2d_stats(const float *mu_a, const float *var_a, int wihi,
+                              int fi, int B, float momentum, int threads,
+                              float *var_s_tmp, float *mu_s, float *var_s,
+                              float *mu_ra, float *var_ra) {
+    // src/batchnorm_layer.cpp:127-147
+    fan_out(fi, threads, [=](int lo, int hi) {
+        for (int col = lo; col < hi; col++) {
+            float sum_mu = 0, sum_var = 0;
+            for (int i = 0; i < wihi * B; i++) {
+                const int at = (i / wihi) * wihi * fi + i % wihi + col * wihi;
+                sum_mu += mu_a[at];
+                sum_var += var_a[at];
+            }
+            mu_s[col] = sum_mu / (wihi * B);
+            var_s_tmp[col] = sum_var;
+        }
+    });
+    // src/batchnorm_layer.cpp:149-168
+    fan_out(fi, threads, [=](int lo, int hi) {
+        for (int col = lo; col < hi; col++) {
+            float sum = 0;
+            for (int i = 0; i < wihi * B; i++) {
+                const int at = (i / wihi) * wihi * fi + i % wihi + col * wihi;
+                sum += (mu_a[at] - mu_s[col]) * (mu_a[at] - mu_s[col]);
+            }
+            var_s[col] = (sum + var_s_tmp[col]) / (wihi * B - 1);
+        }
+    });
+    // src/batchnorm_layer.cpp:15-26
+    fan_out(fi, threads, [=](int lo, int hi) {
+        for (int col = lo; col < hi; col++) {
+            mu_ra[col] = mu_ra[col] * momentum + mu_s[col] * (1 - momentum);
+            var_ra[col] = var_ra[col] * momentum + var_s[col] * (1 - momentum);
+        }
+    });
+}
+
+// src/batchnorm_layer.cpp:170-206: rows are (sample, channel) pairs
+void oracle_batchnorm2d_fwd(const float *mu_w, const float *var_w,
+                            const float *mu_b, const float *var_b,
+                            const float *mu_a, const float *var_a,
+                            const float *mu_norm, const float *var_norm,
+                            int bias, float epsilon, int wihi, int fi, int B,
+                            int threads, float *mu_z, float *var_z) {
+    fan_out(fi * B, threads, [=](int lo, int hi) {
+        for (int row = lo; row < hi; row++) {
+            const float inv = 1.0f / std::sqrt(var_norm[row % fi] + epsilon);
+            const float mra = mu_norm[row % fi];
+            const float mw = mu_w[row % fi];
+            for (int col = 0; col < wihi; col++) {
+                const int at = col + row * wihi;
+                const float d = mu_a[at] - mra;
+                mu_z[at] = inv * d * mw;
+                var_z[at] = inv * inv * (var_a[at] * (mw * mw + var_w[row % fi]) +
+                                         var_w[row % fi] * d * d);
+                if (bias) {
+                    mu_z[at] += mu_b[row % fi];
+                    var_z[at] += var_b[row % fi];
+                }
+            }
+        }
+    });
+}
+
+// src/batchnorm_layer.cpp:233-255
+void oracle_batchnorm2d_bwd_dz(const float *mu_w, const float *jcb,
+                               const float *var_norm, const float *delta_mu_out,
+                               const float *delta_var_out, float epsilon,
+                               int wihi, int fi, int B, int threads,
+                               float *delta_mu, float *delta_var) {
+    fan_out(fi * B, threads, [=](int lo, int hi) {
+        for (int row = lo; row < hi; row++) {
+            const float inv = 1.0f / std::sqrt(var_norm[row % fi] + epsilon);
+            for (int col = 0; col < wihi; col++) {
+                const int at = col + row * wihi;
+                const float tmp = inv * mu_w[row % fi] * jcb[at];
+                delta_mu[at] = tmp * delta_mu_out[at];
+                delta_var[at] = tmp * delta_var_out[at] * tmp;
+            }
+        }
+    });
+}
+
+namespace {
+// src/common.cpp:360-378 (single-threaded in the reference)
+void param_sum(const float *e_mu, const float *e_var, int wihi, int fi, int B,
+               float *out_mu, float *out_var) {
+    for (int col = 0; col < fi; col++) {
+        float s_mu = 0.0f, s_var = 0.0f;
+        for (int i = 0; i < wihi * B; i++) {
+            const int at = (i / wihi) * wihi * fi + i % wihi + col * wihi;
+            s_mu += e_mu[at];
+            s_var += e_var[at];
+        }
+        out_mu[col] = s_mu;
+        out_var[col] = s_var;
+    }
+}
+}  // namespace
+
+void oracle_batchnorm2d_bwd_dw(const float *var_w, const float *var_b,
+                               const float *mu_a, const float *mu_norm,
+                               const float *var_norm, const float *delta_mu_out,
+                               const float *delta_var_out, float epsilon,
+                               int wihi, int fi, int B, int bias, int threads,
+                               float *tmp_1, float *tmp_2, float *delta_mu_w,
+                               float *delta_var_w, float *delta_mu_b,
+                               float *delta_var_b) {
+    // src/batchnorm_layer.cpp:307-332
+    fan_out(fi * B, threads, [=](int lo, int hi) {
+        for (int row = lo; row < hi; row++) {
+            const float inv = 1.0f / std::sqrt(var_norm[row % fi] + epsilon);
+            const float mra = mu_norm[row % fi];
+            for (int col = 0; col < wihi; col++) {
+                const int at = col + row * wihi;
+                const float tmp = inv * (mu_a[at] - mra) * var_w[row % fi];
+                tmp_1[at] = tmp * delta_mu_out[at];
+                tmp_2[at] = tmp * delta_var_out[at] * tmp;
+            }
+        }
+    });
+    param_sum(tmp_1, tmp_2, wihi, fi, B, delta_mu_w, delta_var_w);
+    if (!bias) return;
+    // src/batchnorm_layer.cpp:334-354
+    fan_out(fi * B, threads, [=](int lo, int hi) {
+        for (int row = lo; row < hi; row++) {
+            for (int col = 0; col < wihi; col++) {
+                const float tmp = var_b[row % fi];
+                tmp_1[col + row * wihi] = tmp * delta_mu_out[col + row * wihi];
+                tmp_2[col + row * wihi] = tmp * delta_var_out[col + row * wihi] * tmp;
+            }
+        }
+    });
+    param_sum(tmp_1, tmp_2, wihi, fi, B, delta_mu_b, delta_var_b);
+}
+
+// ---------------------------------------------------------------------------
+// AvgPool2d
+// ---------------------------------------------------------------------------
+
+// src/pooling_layer.cpp:453-484: the receptive-field table of the conv layer,
+// transposed to [tap][output pixel]; the per-input-pixel list of output pixels
+// only when windows overlap.
+int oracle_avgpool2d_build_idx(int kernel, int stride, int wi, int hi, int wo,
+                               int ho, int pad, int pad_type, int *pool_idx,
+                               int *z_ud_idx, int *w, int *h, int *overlap) {
+    const int k2 = kernel * kernel;
+    std::vector<int> fm((size_t)wo * ho * k2), zw((size_t)wi * hi * k2), zud((size_t)wi * hi * k2);
+    int rc = oracle_conv2d_build_idx(kernel, stride, wi, hi, wo, ho, pad, pad_type, k2 + 1,
+                                     fm.data(), zw.data(), zud.data(), w, h);
+    if (rc != 0) return rc;
+    for (int o = 0; o < wo * ho; o++)
+        for (int t = 0; t < k2; t++) pool_idx[(size_t)t * wo * ho + o] = fm[(size_t)o * k2 + t];
+    // AvgPool2d::lazy_index_init (src/pooling_layer.cpp:186-190)
+    *overlap = !(kernel == stride || kernel == wi);
+    if (*overlap) {
+        for (int i = 0; i < *w * *h; i++) z_ud_idx[i] = zud[i];
+    } else {
+        *w = 0;
+        *h = 0;
+    }
+    return 0;
+}
+
+void oracle_avgpool2d_fwd(const float *mu_a, const float *var_a,
+                          const int *pool_idx, int woho, int wihi, int ki,
+                          int n_out, int n_in, int overlap, int threads,
+                          float *mu_z, float *var_z) {
+    const int ki2 = ki * ki;
+    fan_out(n_out, threads, [=](int lo, int hi) {
+        for (int col = lo; col < hi; col++) {
+            float s_mu = 0, s_var = 0;
+            for (int i = 0; i < ki2; i++) {
+                if (overlap) {  // src/pooling_layer.cpp:201-225
+                    int a = pool_idx[col % woho + woho * i];
+                    if (a > -1) {
+                        a += (col / woho) * wihi;
+                        s_mu += mu_a[a - 1];
+                        s_var += var_a[a - 1];
+                    }
+                } else {  // src/pooling_layer.cpp:259-280
+                    const int a = pool_idx[col % woho + woho * i] + (col / woho) * wihi - 1;
+                    s_mu += mu_a[a];
+                    s_var += var_a[a];
+                }
+            }
+            mu_z[col] = s_mu / ki2;
+            var_z[col] = s_var / (ki2 * ki2);
+        }
+    });
+}
+
+void oracle_avgpool2d_bwd_dz(const float *jcb, const float *delta_mu_out,
+                             const float *delta_var_out, const int *z_ud_idx,
+                             int woho, int wihi, int ki, int nr, int wo,
+                             int n_in, int n_out, int overlap, int threads,
+                             float *delta_mu, float *delta_var) {
+    const int ki2 = ki * ki;
+    if (overlap) {  // src/pooling_layer.cpp:316-340
+        fan_out(n_in, threads, [=](int lo, int hi) {
+            for (int col = lo; col < hi; col++) {
+                float s_mu = 0, s_var = 0;
+                for (int i = 0; i < nr; i++) {
+                    int z = z_ud_idx[col % wihi + wihi * i];
+                    if (z > -1) {
+                        z += (col / wihi) * woho;
+                        s_mu += delta_mu_out[z - 1];
+                        s_var += delta_var_out[z - 1];
+                    }
+                }
+                delta_mu[col] = s_mu * jcb[col] / ki2;
+                delta_var[col] = s_var * jcb[col] * jcb[col] / (ki2 * ki2);
+            }
+        });
+        return;
+    }
+    // src/pooling_layer.cpp:379-399 with k = n_in / (ki*wo) (line 163-164)
+    const int m = ki * wo;
+    const int k = n_in / m;
+    fan_out(k * m, threads, [=](int lo, int hi) {
+        for (int j = lo; j < hi; j++) {
+            const int row = j / k, col = j % k;
+            const int at = row + col * m, src = row / ki + (col / ki) * wo;
+            delta_mu[at] = delta_mu_out[src] * jcb[at] / ki2;
+            delta_var[at] = delta_var_out[src] * jcb[at] * jcb[at] / (ki2 * ki2);
+        }
+    });
+}
+
+// ---------------------------------------------------------------------------
+// Residual connection
+// ---------------------------------------------------------------------------
+
+// src/resnet_block.cpp:8-18
+void oracle_add_shortcut(const float *mu_s, const float *var_s, int n,
+                         float *mu_a, float *var_a) {
+    for (int i = 0; i < n; i++) {
+        mu_a[i] += mu_s[i];
+        var_a[i] += var_s[i];
+    }
+}
+
+// src/resnet_block.cpp:20-31
+void oracle_add_shortcut_delta(const float *mu_s, const float *var_s,
+                               const float *jcb_s, int n, float *mu_a,
+                               float *var_a) {
+    for (int i = 0; i < n; i++) {
+        mu_a[i] += mu_s[i] * jcb_s[i];
+        var_a[i] += var_s[i] * jcb_s[i] * jcb_s[i];
+    }
+}
+
 }  // extern "C"

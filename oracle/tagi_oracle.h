@@ -1,5 +1,6 @@
 /*
- * CPU oracle for the TAGI Linear / Conv2d hot path.
+ * CPU oracle for the TAGI Linear / Conv2d hot path and the layers around it
+ * (MixtureReLU, BatchNorm2d, AvgPool2d, residual adds).
  *
  * TEST INFRASTRUCTURE ONLY. This is a plain C++ restatement of the reference
  * CPU algorithms (cuTAGI, src/*.cpp), used as the checker in tests, in the
@@ -119,6 +120,83 @@ void oracle_out_update_indexed(const float *mu_a, const float *var_a,
 /* reference: src/activation.cpp:7-29 */
 void oracle_relu_fwd(const float *mu_z, const float *var_z, int n, float *mu_a,
                      float *jcb, float *var_a);
+
+/* ---- MixtureReLU ---------------------------------------------------------- */
+/* reference: src/activation.cpp:152-178 (+ _mp 180-212) */
+void oracle_mixture_relu_fwd(const float *mu_z, const float *var_z, int n,
+                             int threads, float *mu_a, float *jcb,
+                             float *var_a);
+
+/* ---- BatchNorm2d ----------------------------------------------------------- */
+/* Batch statistics of a [B][fi][wihi] tensor, training mode. reference:
+ * batchnorm2d_stat_mean_var (src/batchnorm_layer.cpp:127-147), then
+ * batchnorm2d_sample_var (149-168), then running_mean_var (15-26) with the
+ * given momentum. var_s_tmp holds fi floats (the sums of var_a).
+ * A fully-connected input is the case wihi = 1, fi = features. */
+void oracle_batchnorm2d_stats(const float *mu_a, const float *var_a, int wihi,
+                              int fi, int B, float momentum, int threads,
+                              float *var_s_tmp, float *mu_s, float *var_s,
+                              float *mu_ra, float *var_ra);
+/* reference: src/batchnorm_layer.cpp:170-206 (+ _mp 521-556). mu_norm/var_norm
+ * are the batch statistics (training) or the running averages (inference). */
+void oracle_batchnorm2d_fwd(const float *mu_w, const float *var_w,
+                            const float *mu_b, const float *var_b,
+                            const float *mu_a, const float *var_a,
+                            const float *mu_norm, const float *var_norm,
+                            int bias, float epsilon, int wihi, int fi, int B,
+                            int threads, float *mu_z, float *var_z);
+/* reference: src/batchnorm_layer.cpp:233-255 (+ _mp 593-626) */
+void oracle_batchnorm2d_bwd_dz(const float *mu_w, const float *jcb,
+                               const float *var_norm, const float *delta_mu_out,
+                               const float *delta_var_out, float epsilon,
+                               int wihi, int fi, int B, int threads,
+                               float *delta_mu, float *delta_var);
+/* reference: batchnorm2d_bwd_delta_w (src/batchnorm_layer.cpp:307-332) and,
+ * when bias != 0, batchnorm2d_bwd_delta_b (334-354), each followed by
+ * delta_param_sum (src/common.cpp:360-378). tmp_1/tmp_2: B*fi*wihi floats. */
+void oracle_batchnorm2d_bwd_dw(const float *var_w, const float *var_b,
+                               const float *mu_a, const float *mu_norm,
+                               const float *var_norm, const float *delta_mu_out,
+                               const float *delta_var_out, float epsilon,
+                               int wihi, int fi, int B, int bias, int threads,
+                               float *tmp_1, float *tmp_2, float *delta_mu_w,
+                               float *delta_var_w, float *delta_mu_b,
+                               float *delta_var_b);
+
+/* ---- AvgPool2d -------------------------------------------------------------- */
+/* reference: get_pool_index (src/pooling_layer.cpp:453-484) as
+ * AvgPool2d::lazy_index_init calls it (pad indices -1). pool_idx is
+ * [kernel*kernel][wo*ho] (1-based input pixel, -1 = padding); z_ud_idx is
+ * [h][w] (1-based output pixel, -1 = none) and is only filled for overlapping
+ * windows (*overlap = 1), as the reference leaves it empty otherwise.
+ * Caller provides pool_idx[wo*ho*k*k] and z_ud_idx[wi*hi*k*k]. */
+int oracle_avgpool2d_build_idx(int kernel, int stride, int wi, int hi, int wo,
+                               int ho, int pad, int pad_type, int *pool_idx,
+                               int *z_ud_idx, int *w, int *h, int *overlap);
+/* reference: avgpool2d_fwd_overlapped_mean_var (src/pooling_layer.cpp:201-225)
+ * when overlap != 0, else avgpool2d_fwd_mean_var (259-280); n_out = woho*fo*B,
+ * n_in = wihi*fo*B */
+void oracle_avgpool2d_fwd(const float *mu_a, const float *var_a,
+                          const int *pool_idx, int woho, int wihi, int ki,
+                          int n_out, int n_in, int overlap, int threads,
+                          float *mu_z, float *var_z);
+/* reference: avgpool2d_bwd_overlapped_delta_z (src/pooling_layer.cpp:316-340)
+ * when overlap != 0 (nr = rows of z_ud_idx), else avgpool2d_bwd_delta_z
+ * (379-399) with wo the output width; n_in = wihi*fi*B, n_out = woho*fi*B */
+void oracle_avgpool2d_bwd_dz(const float *jcb, const float *delta_mu_out,
+                             const float *delta_var_out, const int *z_ud_idx,
+                             int woho, int wihi, int ki, int nr, int wo,
+                             int n_in, int n_out, int overlap, int threads,
+                             float *delta_mu, float *delta_var);
+
+/* ---- Residual connection ------------------------------------------------------ */
+/* reference: add_shortcut_mean_var (src/resnet_block.cpp:8-18) */
+void oracle_add_shortcut(const float *mu_s, const float *var_s, int n,
+                         float *mu_a, float *var_a);
+/* reference: add_shortcut_delta (src/resnet_block.cpp:20-31) */
+void oracle_add_shortcut_delta(const float *mu_s, const float *var_s,
+                               const float *jcb_s, int n, float *mu_a,
+                               float *var_a);
 
 #ifdef __cplusplus
 }

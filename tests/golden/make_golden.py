@@ -15,7 +15,7 @@ sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 sys.path.insert(0, os.path.dirname(HERE))
 
 import oracle  # noqa: E402
-from util import conv_inputs, linear_inputs  # noqa: E402
+from util import batchnorm_inputs, conv_inputs, linear_inputs, pool_inputs  # noqa: E402
 
 # (kernel, stride, pad, pad_type, wi): every geometry of the Conv2d and ResNet-18
 # configurations plus a few odd ones
@@ -27,6 +27,64 @@ IDX_GEOMS = [(3, 1, 1, 1, 32), (3, 1, 1, 1, 16), (3, 1, 1, 1, 8), (3, 1, 1, 1, 4
 LINEAR_SHAPES = [(5, 3, 2), (7, 4, 1), (33, 17, 9), (784, 32, 8), (128, 11, 32), (96, 64, 16)]
 CONV_GEOMS = [(3, 1, 1, 1, 8, 3, 4, 2), (3, 2, 1, 2, 8, 4, 6, 2), (2, 2, 0, 1, 8, 4, 4, 3),
               (5, 1, 2, 1, 9, 2, 3, 1)]
+# (wihi, fi, B) of the batch-norm vectors; (kernel, stride, pad, pad_type, wi, fo, B)
+# of the pooling vectors (global pooling with the default stride -1 is the
+# ResNet-18 head)
+BN_SHAPES = [(16, 8, 4), (64, 3, 5), (1, 37, 6), (9, 5, 2)]
+POOL_GEOMS = [(4, -1, 0, 0, 4, 8, 3), (2, 2, 0, 0, 8, 3, 2), (3, 2, 1, 2, 8, 3, 2),
+              (3, 1, 1, 1, 6, 2, 2), (2, 1, 0, 0, 5, 3, 1)]
+
+
+def layer_vectors(lib):
+    """Outputs of MixtureReLU, BatchNorm2d, AvgPool2d and the residual adds."""
+    out = {}
+    rng = np.random.default_rng(23)
+    mz = (rng.standard_normal(2048) * 3).astype(np.float32)
+    vz = rng.uniform(1e-4, 4.0, 2048).astype(np.float32)
+    out["mrelu_mu_z"], out["mrelu_var_z"] = mz, vz
+    out["mrelu_mu_a"], out["mrelu_var_a"], out["mrelu_jcb"] = lib.mixture_relu_fwd(mz, vz, 1)
+    for (wihi, fi, B) in BN_SHAPES:
+        d = batchnorm_inputs(wihi, fi, B, seed=wihi * 5 + fi * 3 + B)
+        t = "bn_%d_%d_%d" % (wihi, fi, B)
+        for mom in (0.0, 0.9):
+            r = lib.batchnorm2d_stats(d["mu_a"], d["var_a"], wihi, fi, B, mom, d["mu_ra"],
+                                      d["var_ra"], 2)
+            for key, a in zip(("mu_s", "var_s", "mu_ra", "var_ra"), r):
+                out["%s_m%g_%s" % (t, mom, key)] = a
+        mu_s, var_s = r[0], r[1]
+        out[t + "_mu_z"], out[t + "_var_z"] = lib.batchnorm2d_fwd(
+            d["mu_w"], d["var_w"], d["mu_b"], d["var_b"], d["mu_a"], d["var_a"], mu_s, var_s,
+            1e-5, wihi, fi, B, 2)
+        out[t + "_nobias_mu_z"], out[t + "_nobias_var_z"] = lib.batchnorm2d_fwd(
+            d["mu_w"], d["var_w"], None, None, d["mu_a"], d["var_a"], mu_s, var_s, 1e-5, wihi,
+            fi, B, 1)
+        out[t + "_dz_mu"], out[t + "_dz_var"] = lib.batchnorm2d_bwd_dz(
+            d["mu_w"], d["jcb"], var_s, d["dmu"], d["dvar"], 1e-5, wihi, fi, B, 2)
+        r = lib.batchnorm2d_bwd_dw(d["var_w"], d["var_b"], d["mu_a"], mu_s, var_s, d["dmu"],
+                                   d["dvar"], 1e-5, wihi, fi, B, 2)
+        out[t + "_dw_mu"], out[t + "_dw_var"], out[t + "_db_mu"], out[t + "_db_var"] = r
+    for g in POOL_GEOMS:
+        k, s, p, pt, wi, fo, B = g
+        idx = lib.avgpool2d_build_idx(k, s, wi, wi, p, pt)
+        wihi, woho = wi * wi, idx["wo"] * idx["ho"]
+        d = pool_inputs(wihi, woho, fo, B, seed=sum(g))
+        t = "pool_" + "_".join(map(str, g))
+        out[t + "_pool_idx"] = idx["pool_idx"]
+        out[t + "_z_ud_idx"] = idx["z_ud_idx"] if idx["overlap"] else np.zeros(0, np.int32)
+        out[t + "_meta"] = np.array([idx["w"] if idx["overlap"] else 0,
+                                     idx["h"] if idx["overlap"] else 0, idx["wo"], idx["ho"],
+                                     int(idx["overlap"])], np.int32)
+        out[t + "_mu_z"], out[t + "_var_z"] = lib.avgpool2d_fwd(
+            d["mu_a"], d["var_a"], idx["pool_idx"], woho, wihi, k, B * fo * woho, idx["overlap"], 2)
+        out[t + "_dz_mu"], out[t + "_dz_var"] = lib.avgpool2d_bwd_dz(
+            d["jcb"], d["dmu"], d["dvar"], idx["z_ud_idx"], woho, wihi, k, idx["h"], idx["wo"],
+            idx["overlap"], 2)
+    v = [rng.standard_normal(777).astype(np.float32) for _ in range(5)]
+    for i, a in enumerate(v):
+        out["sc_in%d" % i] = a
+    out["sc_mu"], out["sc_var"] = lib.add_shortcut(v[0], v[1], v[2], v[3])
+    out["scd_mu"], out["scd_var"] = lib.add_shortcut_delta(v[0], v[1], v[4], v[2], v[3])
+    return out
 
 
 def main():
@@ -121,7 +179,8 @@ def main():
     out["relu_mu_z"], out["relu_var_z"] = mz, vz
     out["relu_mu_a"], out["relu_var_a"], out["relu_jcb"] = ref.relu_fwd(mz, vz)
     np.savez_compressed(os.path.join(HERE, "misc.npz"), **out)
-    for f in ("conv_idx.npz", "linear.npz", "conv.npz", "misc.npz"):
+    np.savez_compressed(os.path.join(HERE, "layers.npz"), **layer_vectors(ref))
+    for f in ("conv_idx.npz", "linear.npz", "conv.npz", "misc.npz", "layers.npz"):
         print(f, os.path.getsize(os.path.join(HERE, f)))
 
 

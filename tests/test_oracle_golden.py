@@ -5,7 +5,7 @@ import os
 import numpy as np
 import pytest
 
-from golden.make_golden import CONV_GEOMS, IDX_GEOMS, LINEAR_SHAPES
+from golden.make_golden import CONV_GEOMS, IDX_GEOMS, LINEAR_SHAPES, layer_vectors
 from util import conv_inputs, linear_inputs
 
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
@@ -108,3 +108,13 @@ def test_update_output_relu(oracle_lib):
     r = oracle_lib.relu_fwd(g["relu_mu_z"], g["relu_var_z"])
     _same(r[0], g["relu_mu_a"], "relu mu"); _same(r[1], g["relu_var_a"], "relu var")
     _same(r[2], g["relu_jcb"], "relu jcb")
+
+
+def test_layer_vectors(oracle_lib):
+    """MixtureReLU, BatchNorm2d, AvgPool2d (tables and arithmetic) and the
+    residual adds: the oracle reproduces every stored reference output."""
+    g = _load("layers.npz")
+    mine = layer_vectors(oracle_lib)
+    assert set(mine) == set(g.files)
+    for key in g.files:
+        _same(mine[key], g[key], key)

@@ -5,7 +5,7 @@ dropped term, a transposed operand or a wrong index fails one of these."""
 import numpy as np
 import pytest
 
-from util import assert_close, conv_inputs, linear_inputs
+from util import assert_close, conv_inputs, linear_inputs, rel_err
 
 
 @pytest.mark.parametrize("K,N,B", [(37, 19, 5), (128, 64, 16), (300, 11, 32)])
@@ -172,3 +172,111 @@ def test_output_updater_closed_form(oracle_lib):
         gi = float(jcb[i]) / (float(var_a[i]) + 0.5)
         assert dm[i] == pytest.approx(gi * (float(yy[c]) - float(mu_a[i])), rel=1e-5)
         assert dv[i] == pytest.approx(-gi * float(jcb[i]), rel=1e-5)
+
+
+# ---- layers around the hot path ----------------------------------------------------
+
+def test_mixture_relu_is_rectified_gaussian(oracle_lib):
+    """Moments of max(z, 0) for z ~ N(mu, var): E = mu*Phi + sd*phi,
+    E[a^2] = (mu^2 + var)*Phi + mu*sd*phi; the Jacobian is Phi."""
+    from scipy.special import ndtr
+    rng = np.random.default_rng(3)
+    mu = (rng.standard_normal(5000) * 2).astype(np.float32)
+    var = rng.uniform(0.05, 3.0, 5000).astype(np.float32)
+    mu_a, var_a, jcb = oracle_lib.mixture_relu_fwd(mu, var, 2)
+    m, v = mu.astype(np.float64), var.astype(np.float64)
+    sd = np.sqrt(v)
+    al = m / sd
+    Phi, phi = ndtr(al), np.exp(-0.5 * al * al) / np.sqrt(2 * np.pi)
+    e1 = m * Phi + sd * phi
+    e2 = (m * m + v) * Phi + m * sd * phi
+    assert rel_err(jcb, Phi) < 1e-5
+    assert rel_err(mu_a, np.maximum(e1, 1e-6)) < 1e-5
+    assert rel_err(var_a, np.maximum(e2 - e1 * e1, 1e-6)) < 2e-4  # cancellation in fp32
+    assert mu_a.min() >= 1e-6 and var_a.min() >= 1e-6
+
+
+@pytest.mark.parametrize("wihi,fi,B", [(16, 6, 5), (1, 19, 7), (49, 3, 2)])
+def test_batchnorm2d_closed_forms(oracle_lib, wihi, fi, B):
+    from util import batchnorm_inputs
+    d = batchnorm_inputs(wihi, fi, B, seed=wihi + fi)
+    x = d["mu_a"].astype(np.float64).reshape(B, fi, wihi)
+    vx = d["var_a"].astype(np.float64).reshape(B, fi, wihi)
+    n = B * wihi
+    mean = x.mean(axis=(0, 2))
+    var = (((x - mean[None, :, None]) ** 2).sum(axis=(0, 2)) + vx.sum(axis=(0, 2))) / (n - 1)
+    mu_s, var_s, mu_ra, var_ra = oracle_lib.batchnorm2d_stats(
+        d["mu_a"], d["var_a"], wihi, fi, B, 0.9, d["mu_ra"], d["var_ra"], 2)
+    assert rel_err(mu_s, mean) < 1e-5 and rel_err(var_s, var) < 1e-5
+    assert rel_err(mu_ra, 0.9 * d["mu_ra"] + 0.1 * mean) < 1e-5
+    assert rel_err(var_ra, 0.9 * d["var_ra"] + 0.1 * var) < 1e-5
+    # momentum 0 replaces the running averages by the batch statistics
+    r0 = oracle_lib.batchnorm2d_stats(d["mu_a"], d["var_a"], wihi, fi, B, 0.0, d["mu_ra"],
+                                      d["var_ra"], 1)
+    assert np.array_equal(r0[2], r0[0]) and np.array_equal(r0[3], r0[1])
+
+    c = lambda a: a.astype(np.float64)[None, :, None]
+    inv = 1.0 / np.sqrt(c(var_s) + 1e-5)
+    xt = x - c(mu_s)
+    mu_z = inv * xt * c(d["mu_w"]) + c(d["mu_b"])
+    var_z = inv ** 2 * (vx * (c(d["mu_w"]) ** 2 + c(d["var_w"])) + c(d["var_w"]) * xt ** 2) + c(d["var_b"])
+    got = oracle_lib.batchnorm2d_fwd(d["mu_w"], d["var_w"], d["mu_b"], d["var_b"], d["mu_a"],
+                                     d["var_a"], mu_s, var_s, 1e-5, wihi, fi, B, 3)
+    assert rel_err(got[0], mu_z) < 1e-5 and rel_err(got[1], var_z) < 1e-5
+    assert got[1].min() >= 0
+
+    dm = d["dmu"].astype(np.float64).reshape(B, fi, wihi)
+    dv = d["dvar"].astype(np.float64).reshape(B, fi, wihi)
+    j = d["jcb"].astype(np.float64).reshape(B, fi, wihi)
+    t = inv * c(d["mu_w"]) * j
+    got = oracle_lib.batchnorm2d_bwd_dz(d["mu_w"], d["jcb"], var_s, d["dmu"], d["dvar"], 1e-5,
+                                        wihi, fi, B, 2)
+    assert rel_err(got[0], t * dm) < 1e-5 and rel_err(got[1], t * t * dv) < 1e-5
+    tw = inv * xt * c(d["var_w"])
+    got = oracle_lib.batchnorm2d_bwd_dw(d["var_w"], d["var_b"], d["mu_a"], mu_s, var_s, d["dmu"],
+                                        d["dvar"], 1e-5, wihi, fi, B, 2)
+    assert rel_err(got[0], (tw * dm).sum(axis=(0, 2))) < 1e-4
+    assert rel_err(got[1], (tw * tw * dv).sum(axis=(0, 2))) < 1e-4
+    vb = d["var_b"].astype(np.float64)
+    assert rel_err(got[2], vb * dm.sum(axis=(0, 2))) < 1e-4
+    assert rel_err(got[3], vb * vb * dv.sum(axis=(0, 2))) < 1e-4
+    # the mean path is what torch's batch norm computes with these statistics
+    import torch
+    ref = torch.nn.functional.batch_norm(
+        torch.from_numpy(x.reshape(B, fi, wihi, 1)), torch.from_numpy(c(mu_s).ravel()),
+        torch.from_numpy(c(var_s).ravel()), torch.from_numpy(c(d["mu_w"]).ravel()),
+        torch.from_numpy(c(d["mu_b"]).ravel()), training=False, eps=1e-5)
+    assert rel_err(mu_z, ref.numpy()) < 1e-9
+
+
+@pytest.mark.parametrize("geom", [(4, -1, 0, 0, 4), (2, 2, 0, 0, 8), (3, 2, 1, 1, 9),
+                                  (3, 1, 1, 1, 6), (2, 1, 0, 0, 5)])
+def test_avgpool2d_is_torch_avg_pool(oracle_lib, geom):
+    """Mean: torch's avg_pool2d with the padding counted in the divisor;
+    variance: the same window sum divided by k^4; backward: its adjoint times
+    the Jacobian (squared for the variance)."""
+    import torch
+    from util import pool_inputs
+    k, s, p, pt, wi = geom
+    idx = oracle_lib.avgpool2d_build_idx(k, s, wi, wi, p, pt)
+    fo, B = 3, 2
+    wihi, woho = wi * wi, idx["wo"] * idx["ho"]
+    d = pool_inputs(wihi, woho, fo, B, seed=sum(geom))
+    stride = k if s < 0 else s
+    x = torch.from_numpy(d["mu_a"].astype(np.float64)).reshape(B, fo, wi, wi).requires_grad_(True)
+    v = torch.from_numpy(d["var_a"].astype(np.float64)).reshape(B, fo, wi, wi).requires_grad_(True)
+    pool = lambda a: torch.nn.functional.avg_pool2d(a, k, stride, p, count_include_pad=True)
+    ym, yv = pool(x), pool(v) / (k * k)
+    got = oracle_lib.avgpool2d_fwd(d["mu_a"], d["var_a"], idx["pool_idx"], woho, wihi, k,
+                                   B * fo * woho, idx["overlap"], 2)
+    assert rel_err(got[0], ym.detach().numpy()) < 1e-5
+    assert rel_err(got[1], yv.detach().numpy()) < 1e-5
+    dm = torch.from_numpy(d["dmu"].astype(np.float64)).reshape(ym.shape)
+    dv = torch.from_numpy(d["dvar"].astype(np.float64)).reshape(ym.shape)
+    gm, = torch.autograd.grad(ym, x, dm)
+    gv, = torch.autograd.grad(yv, v, dv)   # adjoint of (window sum)/k^4, times k^2 below
+    j = d["jcb"].astype(np.float64).reshape(B, fo, wi, wi)
+    got = oracle_lib.avgpool2d_bwd_dz(d["jcb"], d["dmu"], d["dvar"], idx["z_ud_idx"], woho, wihi,
+                                      k, idx["h"], idx["wo"], idx["overlap"], 2)
+    assert rel_err(got[0], gm.numpy() * j) < 1e-5
+    assert rel_err(got[1], gv.numpy() * j * j) < 1e-5

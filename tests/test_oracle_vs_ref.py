@@ -5,7 +5,7 @@ does not exist."""
 import numpy as np
 import pytest
 
-from util import conv_inputs, linear_inputs
+from util import batchnorm_inputs, conv_inputs, linear_inputs, pool_inputs
 
 
 @pytest.fixture(scope="module")
@@ -101,3 +101,68 @@ def test_update_output_relu(oracle_lib, ref):
     m = rng.normal(0, 1, 999).astype(np.float32)
     v = rng.uniform(0, 1, 999).astype(np.float32)
     assert _eq(oracle_lib.relu_fwd(m, v), ref.relu_fwd(m, v))
+
+
+# ---- layers around the hot path: MixtureReLU, BatchNorm2d, AvgPool2d, residual adds ----
+
+@pytest.mark.parametrize("threads", [1, 4])
+def test_mixture_relu(oracle_lib, ref, threads):
+    rng = np.random.default_rng(11 + threads)
+    mu_z = (rng.standard_normal(4099) * 3).astype(np.float32)
+    var_z = rng.uniform(1e-4, 4.0, 4099).astype(np.float32)
+    assert _eq(oracle_lib.mixture_relu_fwd(mu_z, var_z, threads),
+               ref.mixture_relu_fwd(mu_z, var_z, threads))
+
+
+@pytest.mark.parametrize("wihi,fi,B", [(16, 8, 4), (64, 3, 5), (1, 37, 6), (9, 5, 2)])
+@pytest.mark.parametrize("threads", [1, 3])
+def test_batchnorm2d(oracle_lib, ref, wihi, fi, B, threads):
+    d = batchnorm_inputs(wihi, fi, B, seed=wihi + fi + B + threads)
+    for momentum in (0.0, 0.9):
+        a = (d["mu_a"], d["var_a"], wihi, fi, B, momentum, d["mu_ra"], d["var_ra"], threads)
+        so, sr = oracle_lib.batchnorm2d_stats(*a), ref.batchnorm2d_stats(*a)
+        assert _eq(so, sr)
+    mu_s, var_s = so[0], so[1]
+    for bias in (True, False):
+        mb, vb = (d["mu_b"], d["var_b"]) if bias else (None, None)
+        a = (d["mu_w"], d["var_w"], mb, vb, d["mu_a"], d["var_a"], mu_s, var_s, 1e-5, wihi, fi, B,
+             threads)
+        assert _eq(oracle_lib.batchnorm2d_fwd(*a), ref.batchnorm2d_fwd(*a))
+        a = (d["var_w"], vb, d["mu_a"], mu_s, var_s, d["dmu"], d["dvar"], 1e-5, wihi, fi, B, threads)
+        x, y = oracle_lib.batchnorm2d_bwd_dw(*a), ref.batchnorm2d_bwd_dw(*a)
+        assert _eq(x[:2], y[:2]) and (not bias or _eq(x[2:], y[2:]))
+    a = (d["mu_w"], d["jcb"], var_s, d["dmu"], d["dvar"], 1e-5, wihi, fi, B, threads)
+    assert _eq(oracle_lib.batchnorm2d_bwd_dz(*a), ref.batchnorm2d_bwd_dz(*a))
+
+
+# (kernel, stride, pad, pad_type, wi): global pooling with the default stride -1,
+# non-overlapping windows, overlapping windows with and without padding
+POOLS = [(4, -1, 0, 0, 4), (2, 2, 0, 0, 8), (3, 2, 1, 2, 8), (3, 1, 1, 1, 6), (2, 1, 0, 0, 5),
+         (8, -1, 0, 0, 8), (3, 2, 1, 1, 9)]
+
+
+@pytest.mark.parametrize("geom", POOLS)
+@pytest.mark.parametrize("threads", [1, 4])
+def test_avgpool2d(oracle_lib, ref, geom, threads):
+    k, s, p, pt, wi = geom
+    a, b = oracle_lib.avgpool2d_build_idx(k, s, wi, wi, p, pt), ref.avgpool2d_build_idx(k, s, wi, wi, p, pt)
+    assert np.array_equal(a["pool_idx"], b["pool_idx"])
+    assert a["overlap"] == b["overlap"] and (a["wo"], a["ho"]) == (b["wo"], b["ho"])
+    if a["overlap"]:
+        assert np.array_equal(a["z_ud_idx"], b["z_ud_idx"]) and (a["w"], a["h"]) == (b["w"], b["h"])
+    fo, B = 3, 2
+    wihi, woho = wi * wi, a["wo"] * a["ho"]
+    d = pool_inputs(wihi, woho, fo, B, seed=sum(geom) + threads)
+    mu_a, var_a, jcb, dmu, dvar = d["mu_a"], d["var_a"], d["jcb"], d["dmu"], d["dvar"]
+    args = (mu_a, var_a, a["pool_idx"], woho, wihi, k, B * fo * woho, a["overlap"], threads)
+    assert _eq(oracle_lib.avgpool2d_fwd(*args), ref.avgpool2d_fwd(*args))
+    args = (jcb, dmu, dvar, a["z_ud_idx"], woho, wihi, k, a["h"], a["wo"], a["overlap"], threads)
+    assert _eq(oracle_lib.avgpool2d_bwd_dz(*args), ref.avgpool2d_bwd_dz(*args))
+
+
+def test_shortcut_adds(oracle_lib, ref):
+    rng = np.random.default_rng(5)
+    v = [rng.standard_normal(1001).astype(np.float32) for _ in range(5)]
+    assert _eq(oracle_lib.add_shortcut(v[0], v[1], v[2], v[3]), ref.add_shortcut(v[0], v[1], v[2], v[3]))
+    assert _eq(oracle_lib.add_shortcut_delta(v[0], v[1], v[4], v[2], v[3]),
+               ref.add_shortcut_delta(v[0], v[1], v[4], v[2], v[3]))

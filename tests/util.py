@@ -67,3 +67,30 @@ def conv_inputs(fi, fo, ki, wihi, woho, B, seed=0, bias=False, jcb_random=False)
     else:
         d["mu_b"] = d["var_b"] = None
     return d
+
+
+def batchnorm_inputs(wihi, fi, B, seed=0):
+    """A [B][fi][wihi] activation tensor with per-channel parameters, running
+    averages and incoming innovations (jittered so that a wrong index shows)."""
+    rng = np.random.default_rng(seed)
+    n = B * fi * wihi
+    f = np.float32
+    return dict(
+        mu_a=rng.standard_normal(n).astype(f), var_a=rng.uniform(0.01, 0.5, n).astype(f),
+        jcb=rng.uniform(0.0, 1.0, n).astype(f),
+        mu_w=(1 + 0.1 * rng.standard_normal(fi)).astype(f),
+        var_w=rng.uniform(0.01, 0.1, fi).astype(f),
+        mu_b=(0.1 * rng.standard_normal(fi)).astype(f), var_b=rng.uniform(0.01, 0.1, fi).astype(f),
+        mu_ra=rng.standard_normal(fi).astype(f), var_ra=rng.uniform(0.5, 2.0, fi).astype(f),
+        dmu=(0.1 * rng.standard_normal(n)).astype(f), dvar=(-rng.uniform(0, 1e-2, n)).astype(f))
+
+
+def pool_inputs(wihi, woho, fo, B, seed=0):
+    rng = np.random.default_rng(seed)
+    f = np.float32
+    return dict(
+        mu_a=rng.standard_normal(B * fo * wihi).astype(f),
+        var_a=rng.uniform(0.01, 0.5, B * fo * wihi).astype(f),
+        jcb=rng.uniform(0, 1, B * fo * wihi).astype(f),
+        dmu=rng.standard_normal(B * fo * woho).astype(f),
+        dvar=(-rng.uniform(0, 1e-2, B * fo * woho)).astype(f))
