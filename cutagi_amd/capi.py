@@ -47,6 +47,15 @@ SIGNATURES = {
     "tagi_out_update_dense": (_i, [_vp] * 5 + [_i] + [_vp] * 3),
     "tagi_out_update_indexed": (_i, [_vp] * 6 + [_i] * 3 + [_vp] * 3),
     "tagi_relu_fwd": (_i, [_vp, _vp, _sz, _vp, _vp, _vp, _vp]),
+    "tagi_mixture_relu_fwd": (_i, [_vp, _vp, _sz, _vp, _vp, _vp, _vp]),
+    "tagi_batchnorm2d_stats": (_i, [_vp, _vp, _i, _i, _i, _f] + [_vp] * 5),
+    "tagi_batchnorm2d_fwd": (_i, [_vp] * 8 + [_i, _f, _i, _i, _i] + [_vp] * 3),
+    "tagi_batchnorm2d_bwd": (_i, [_vp] * 9 + [_f] + [_i] * 6 + [_vp] * 7),
+    "tagi_avgpool2d_build_idx": (_i, [_i] * 6 + [_ip] * 5),
+    "tagi_avgpool2d_fwd": (_i, [_vp] * 3 + [_i] * 4 + [_vp] * 3),
+    "tagi_avgpool2d_bwd_dz": (_i, [_vp] * 4 + [_i] * 7 + [_vp] * 3),
+    "tagi_add_shortcut": (_i, [_vp, _vp, _sz, _vp, _vp, _vp]),
+    "tagi_add_shortcut_delta": (_i, [_vp, _vp, _vp, _sz, _vp, _vp, _vp]),
 }
 
 
@@ -110,6 +119,22 @@ def conv2d_out_size(kernel, stride, wi, hi, pad, pad_type):
     check(lib.tagi_conv2d_out_size(kernel, stride, wi, hi, pad, pad_type,
                                    ctypes.byref(wo), ctypes.byref(ho)))
     return wo.value, ho.value
+
+
+def avgpool2d_build_idx(kernel, stride, wi, hi, pad, pad_type):
+    """Host pooling tables as numpy int32 arrays (see tagi_avgpool2d_build_idx)."""
+    import numpy as np
+    wo, ho = conv2d_out_size(kernel, stride, wi, hi, pad, pad_type)
+    k2 = kernel * kernel
+    pool = np.zeros(wo * ho * k2, np.int32)
+    zud = np.zeros(wi * hi * k2, np.int32)
+    w, h, ov = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
+    as_ip = lambda a: a.ctypes.data_as(_ip)
+    check(lib.tagi_avgpool2d_build_idx(kernel, stride, wi, hi, pad, pad_type, as_ip(pool),
+                                       as_ip(zud), ctypes.byref(w), ctypes.byref(h),
+                                       ctypes.byref(ov)))
+    return dict(pool_idx=pool, z_ud_idx=zud[:w.value * h.value].copy(), w=w.value, h=h.value,
+                overlap=bool(ov.value), wo=wo, ho=ho)
 
 
 def conv2d_build_idx(kernel, stride, wi, hi, pad, pad_type, param_pad_idx):

@@ -13,7 +13,6 @@ namespace {
 
 constexpr int ABI_VERSION = 100;
 constexpr int MAX_DEVICES = 16;
-constexpr int NUM_CU = 256;  // MI355X
 
 #define TAGI_TRY(expr)                          \
     do {                                        \
@@ -513,6 +512,130 @@ int tagi_relu_fwd(const float *mu_z, const float *var_z, size_t n, float *mu_a, 
                   float *var_a, void *stream_) {
     if (n > 0 && (!mu_z || !var_z || !mu_a || !jcb || !var_a)) return TAGI_ERR_INVALID_ARG;
     TAGI_TRY(launch_relu(mu_z, var_z, n, mu_a, jcb, var_a, static_cast<hipStream_t>(stream_)));
+    return TAGI_OK;
+}
+
+// ---------------------------------------------------------------------------
+// MixtureReLU, BatchNorm2d, AvgPool2d, residual adds
+// ---------------------------------------------------------------------------
+
+int tagi_mixture_relu_fwd(const float *mu_z, const float *var_z, size_t n, float *mu_a,
+                          float *jcb, float *var_a, void *stream) {
+    if (!mu_z || !var_z || !mu_a || !jcb || !var_a) return TAGI_ERR_INVALID_ARG;
+    if (n == 0) return TAGI_OK;
+    TAGI_TRY(launch_mixture_relu(mu_z, var_z, n, mu_a, jcb, var_a,
+                                 static_cast<hipStream_t>(stream)));
+    return TAGI_OK;
+}
+
+static bool bn_sizes_ok(int wihi, int fi, int B) {
+    return wihi > 0 && fi > 0 && B > 0 && fi <= 65535 &&
+           (long long)wihi * fi * B < 0x7fffffffLL;
+}
+
+int tagi_batchnorm2d_stats(const float *mu_a, const float *var_a, int wihi, int fi, int B,
+                           float momentum, float *mu_s, float *var_s, float *mu_ra,
+                           float *var_ra, void *stream) {
+    if (!mu_a || !var_a || !mu_s || !var_s || !mu_ra || !var_ra) return TAGI_ERR_INVALID_ARG;
+    if (!bn_sizes_ok(wihi, fi, B)) return TAGI_ERR_INVALID_ARG;
+    float *ws = nullptr;
+    int rc = workspace_get(batchnorm2d_scratch_floats(fi, B) * sizeof(float), &ws);
+    if (rc != TAGI_OK) return rc;
+    TAGI_TRY(launch_batchnorm2d_stats(mu_a, var_a, wihi, fi, B, momentum, ws, mu_s, var_s, mu_ra,
+                                      var_ra, static_cast<hipStream_t>(stream)));
+    return TAGI_OK;
+}
+
+int tagi_batchnorm2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
+                         const float *var_b, const float *mu_a, const float *var_a,
+                         const float *mu_norm, const float *var_norm, int bias, float epsilon,
+                         int wihi, int fi, int B, float *mu_z, float *var_z, void *stream) {
+    if (!mu_w || !var_w || !mu_a || !var_a || !mu_norm || !var_norm || !mu_z || !var_z)
+        return TAGI_ERR_INVALID_ARG;
+    if (bias && (!mu_b || !var_b)) return TAGI_ERR_INVALID_ARG;
+    if (!bn_sizes_ok(wihi, fi, B)) return TAGI_ERR_INVALID_ARG;
+    TAGI_TRY(launch_batchnorm2d_fwd(mu_w, var_w, bias ? mu_b : nullptr, bias ? var_b : nullptr,
+                                    mu_a, var_a, mu_norm, var_norm, epsilon, wihi, fi, B, mu_z,
+                                    var_z, static_cast<hipStream_t>(stream)));
+    return TAGI_OK;
+}
+
+int tagi_batchnorm2d_bwd(const float *mu_w, const float *var_w, const float *var_b,
+                         const float *mu_a, const float *jcb, const float *mu_norm,
+                         const float *var_norm, const float *delta_mu_out,
+                         const float *delta_var_out, float epsilon, int wihi, int fi, int B,
+                         int bias, int state_update, int param_update, float *delta_mu,
+                         float *delta_var, float *delta_mu_w, float *delta_var_w,
+                         float *delta_mu_b, float *delta_var_b, void *stream) {
+    if (!mu_w || !var_w || !mu_norm || !var_norm || !delta_mu_out || !delta_var_out)
+        return TAGI_ERR_INVALID_ARG;
+    if (state_update && (!jcb || !delta_mu || !delta_var)) return TAGI_ERR_INVALID_ARG;
+    if (param_update && (!mu_a || !delta_mu_w || !delta_var_w)) return TAGI_ERR_INVALID_ARG;
+    if (param_update && bias && (!var_b || !delta_mu_b || !delta_var_b))
+        return TAGI_ERR_INVALID_ARG;
+    if (!bn_sizes_ok(wihi, fi, B)) return TAGI_ERR_INVALID_ARG;
+    if (!state_update && !param_update) return TAGI_OK;
+    float *ws = nullptr;
+    int rc = workspace_get(batchnorm2d_scratch_floats(fi, B) * sizeof(float), &ws);
+    if (rc != TAGI_OK) return rc;
+    TAGI_TRY(launch_batchnorm2d_bwd(mu_w, var_w, bias ? var_b : nullptr, mu_a, jcb, mu_norm,
+                                    var_norm, delta_mu_out, delta_var_out, epsilon, wihi, fi, B,
+                                    state_update, param_update, ws, delta_mu, delta_var,
+                                    delta_mu_w, delta_var_w, delta_mu_b, delta_var_b,
+                                    static_cast<hipStream_t>(stream)));
+    return TAGI_OK;
+}
+
+int tagi_avgpool2d_build_idx(int kernel, int stride, int wi, int hi, int pad, int pad_type,
+                             int *pool_idx, int *z_ud_idx, int *w, int *h, int *overlap) {
+    if (!pool_idx || !z_ud_idx || !w || !h || !overlap) return TAGI_ERR_INVALID_ARG;
+    return avgpool2d_build_idx(kernel, stride, wi, hi, pad, pad_type, pool_idx, z_ud_idx, w, h,
+                               overlap) == 0
+               ? TAGI_OK
+               : TAGI_ERR_INVALID_ARG;
+}
+
+int tagi_avgpool2d_fwd(const float *mu_a, const float *var_a, const int *pool_idx, int woho,
+                       int wihi, int ki, int n_out, float *mu_z, float *var_z, void *stream) {
+    if (!mu_a || !var_a || !pool_idx || !mu_z || !var_z) return TAGI_ERR_INVALID_ARG;
+    if (woho <= 0 || wihi <= 0 || ki <= 0 || n_out <= 0 || n_out % woho != 0)
+        return TAGI_ERR_INVALID_ARG;
+    TAGI_TRY(launch_avgpool2d_fwd(mu_a, var_a, pool_idx, woho, wihi, ki, n_out, mu_z, var_z,
+                                  static_cast<hipStream_t>(stream)));
+    return TAGI_OK;
+}
+
+int tagi_avgpool2d_bwd_dz(const float *jcb, const float *delta_mu_out, const float *delta_var_out,
+                          const int *z_ud_idx, int woho, int wihi, int ki, int nr, int wo,
+                          int n_in, int overlap, float *delta_mu, float *delta_var,
+                          void *stream) {
+    if (!jcb || !delta_mu_out || !delta_var_out || !delta_mu || !delta_var)
+        return TAGI_ERR_INVALID_ARG;
+    if (woho <= 0 || wihi <= 0 || ki <= 0 || n_in <= 0 || n_in % wihi != 0)
+        return TAGI_ERR_INVALID_ARG;
+    if (overlap && (!z_ud_idx || nr <= 0)) return TAGI_ERR_INVALID_ARG;
+    if (!overlap && (wo <= 0 || n_in % (ki * wo) != 0)) return TAGI_ERR_INVALID_ARG;
+    TAGI_TRY(launch_avgpool2d_bwd(jcb, delta_mu_out, delta_var_out, z_ud_idx, woho, wihi, ki, nr,
+                                  wo, n_in, overlap, delta_mu, delta_var,
+                                  static_cast<hipStream_t>(stream)));
+    return TAGI_OK;
+}
+
+int tagi_add_shortcut(const float *mu_s, const float *var_s, size_t n, float *mu_a, float *var_a,
+                      void *stream) {
+    if (!mu_s || !var_s || !mu_a || !var_a) return TAGI_ERR_INVALID_ARG;
+    if (n == 0) return TAGI_OK;
+    TAGI_TRY(launch_add_shortcut(mu_s, var_s, nullptr, n, mu_a, var_a,
+                                 static_cast<hipStream_t>(stream)));
+    return TAGI_OK;
+}
+
+int tagi_add_shortcut_delta(const float *mu_s, const float *var_s, const float *jcb_s, size_t n,
+                            float *mu_a, float *var_a, void *stream) {
+    if (!mu_s || !var_s || !jcb_s || !mu_a || !var_a) return TAGI_ERR_INVALID_ARG;
+    if (n == 0) return TAGI_OK;
+    TAGI_TRY(launch_add_shortcut(mu_s, var_s, jcb_s, n, mu_a, var_a,
+                                 static_cast<hipStream_t>(stream)));
     return TAGI_OK;
 }
 

@@ -24,12 +24,16 @@ namespace tagi {
 
 int conv2d_out_size(int kernel, int stride, int wi, int hi, int pad, int pad_type, int *wo,
                     int *ho) {
-    if (kernel <= 0 || stride <= 0 || wi <= 0 || hi <= 0 || pad < 0) return -1;
+    // A negative stride is what the pooling layers pass by default ("stride =
+    // kernel"); the reference's formula then only works out for a window that
+    // covers the whole image (nom = 0), which is how global pooling is written.
+    if (kernel <= 0 || stride == 0 || wi <= 0 || hi <= 0 || pad < 0) return -1;
     const int extra = pad_type == 1 ? 2 * pad : pad_type == 2 ? pad : 0;
     const int nom_w = wi - kernel + extra, nom_h = hi - kernel + extra;
     if (nom_w < 0 || nom_h < 0 || nom_w % stride != 0 || nom_h % stride != 0) return -1;
     *wo = nom_w / stride + 1;
     *ho = nom_h / stride + 1;
+    if (*wo < 1 || *ho < 1) return -1;
     return 0;
 }
 
@@ -81,6 +85,34 @@ int conv2d_build_idx(int kernel, int stride, int wi, int hi, int pad, int pad_ty
         }
     *w_out = w;
     *h_out = h;
+    return 0;
+}
+
+// Pooling tables (reference: get_pool_index, src/pooling_layer.cpp:453-484, as
+// AvgPool2d::lazy_index_init calls it): the receptive-field table transposed to
+// [tap][output pixel], and -- only for overlapping windows -- the per-input-pixel
+// list of output pixels [h][w].
+int avgpool2d_build_idx(int kernel, int stride, int wi, int hi, int pad, int pad_type,
+                        int *pool_idx, int *z_ud_idx, int *w_out, int *h_out, int *overlap) {
+    int wo = 0, ho = 0;
+    if (conv2d_out_size(kernel, stride, wi, hi, pad, pad_type, &wo, &ho) != 0) return -1;
+    const int k2 = kernel * kernel;
+    std::vector<int> fm((size_t)wo * ho * k2), zw((size_t)wi * hi * k2), zud((size_t)wi * hi * k2);
+    int w = 0, h = 0;
+    if (conv2d_build_idx(kernel, stride, wi, hi, pad, pad_type, k2 + 1, fm.data(), zw.data(),
+                         zud.data(), &w, &h) != 0)
+        return -1;
+    for (int o = 0; o < wo * ho; o++)
+        for (int t = 0; t < k2; t++) pool_idx[(size_t)t * wo * ho + o] = fm[(size_t)o * k2 + t];
+    *overlap = !(kernel == stride || kernel == wi);
+    if (*overlap) {
+        for (int i = 0; i < w * h; i++) z_ud_idx[i] = zud[i];
+        *w_out = w;
+        *h_out = h;
+    } else {
+        *w_out = 0;
+        *h_out = 0;
+    }
     return 0;
 }
 

@@ -6,6 +6,8 @@
 
 namespace tagi {
 
+constexpr int NUM_CU = 256;  // MI355X
+
 // Which contraction of the layer a tiled GEMM launch computes.
 //   FWD: D[b][n]  = sum_k  act[b][k] * w[n][k]      (mean; variance with 2 terms)
 //   DZ : D[b][k'] = sum_n  delta[b][n] * w[n][k']   (variance with w^2)
@@ -86,6 +88,36 @@ hipError_t launch_out_update_indexed(const float *mu_a, const float *var_a, cons
 hipError_t launch_relu(const float *mu_z, const float *var_z, size_t n, float *mu_a, float *jcb,
                        float *var_a, hipStream_t stream);
 
+// Layers between the contractions (tagi_layers.hip)
+hipError_t launch_mixture_relu(const float *mu_z, const float *var_z, size_t n, float *mu_a,
+                               float *jcb, float *var_a, hipStream_t stream);
+size_t batchnorm2d_scratch_floats(int fi, int B);
+hipError_t launch_batchnorm2d_stats(const float *mu_a, const float *var_a, int wihi, int fi,
+                                    int B, float momentum, float *scratch, float *mu_s,
+                                    float *var_s, float *mu_ra, float *var_ra,
+                                    hipStream_t stream);
+hipError_t launch_batchnorm2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
+                                  const float *var_b, const float *mu_a, const float *var_a,
+                                  const float *mu_norm, const float *var_norm, float epsilon,
+                                  int wihi, int fi, int B, float *mu_z, float *var_z,
+                                  hipStream_t stream);
+hipError_t launch_batchnorm2d_bwd(const float *mu_w, const float *var_w, const float *var_b,
+                                  const float *mu_a, const float *jcb, const float *mu_norm,
+                                  const float *var_norm, const float *dmu_out,
+                                  const float *dvar_out, float epsilon, int wihi, int fi, int B,
+                                  int state_update, int param_update, float *scratch, float *dmu,
+                                  float *dvar, float *dmu_w, float *dvar_w, float *dmu_b,
+                                  float *dvar_b, hipStream_t stream);
+hipError_t launch_avgpool2d_fwd(const float *mu_a, const float *var_a, const int *pool_idx,
+                                int woho, int wihi, int ki, int n_out, float *mu_z, float *var_z,
+                                hipStream_t stream);
+hipError_t launch_avgpool2d_bwd(const float *jcb, const float *dmu_out, const float *dvar_out,
+                                const int *z_ud_idx, int woho, int wihi, int ki, int nr, int wo,
+                                int n_in, int overlap, float *dmu, float *dvar,
+                                hipStream_t stream);
+hipError_t launch_add_shortcut(const float *mu_s, const float *var_s, const float *jcb_s,
+                               size_t n, float *mu_a, float *var_a, hipStream_t stream);
+
 // Conv2d (implicit GEMM through the index tables)
 hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
                              const float *var_b, const float *mu_a, const float *var_a,
@@ -109,5 +141,7 @@ int conv2d_out_size(int kernel, int stride, int wi, int hi, int pad, int pad_typ
                     int *ho);
 int conv2d_build_idx(int kernel, int stride, int wi, int hi, int pad, int pad_type,
                      int param_pad_idx, int *Fmwa_2, int *FCzwa_1, int *Szz_ud, int *w, int *h);
+int avgpool2d_build_idx(int kernel, int stride, int wi, int hi, int pad, int pad_type,
+                        int *pool_idx, int *z_ud_idx, int *w, int *h, int *overlap);
 
 }  // namespace tagi

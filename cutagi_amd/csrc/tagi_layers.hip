@@ -1,0 +1,394 @@
+// The layers that sit between the Linear / Conv2d contractions of a TAGI
+// network: MixtureReLU, BatchNorm2d (statistics, normalisation, backward),
+// AvgPool2d and the residual adds. All of them are bandwidth-bound passes over
+// [B][channels][pixels] tensors; gfx950.
+#include "tagi_internal.h"
+
+namespace tagi {
+namespace {
+
+constexpr int TPB = 256;
+
+inline unsigned blocks_for(size_t n, int per_block) {
+    return (unsigned)((n + per_block - 1) / per_block);
+}
+
+// ---------------------------------------------------------------------------
+// MixtureReLU: moments of max(z, 0) for z ~ N(mu, var), floored at 1e-6; the
+// Jacobian is the probability mass above zero.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(TPB) void mixture_relu_kernel(const float *__restrict__ mu_z,
+                                                           const float *__restrict__ var_z,
+                                                           size_t n, float *__restrict__ mu_a,
+                                                           float *__restrict__ jcb,
+                                                           float *__restrict__ var_a) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n) return;
+    constexpr float INV_SQRT_2PI = 1.0f / 2.5066282746310002f;
+    const float m = mu_z[i], v = var_z[i];
+    const float sd = sqrtf(v);
+    const float alpha = m / sd;
+    const float pdf = INV_SQRT_2PI * expf(-0.5f * alpha * alpha);
+    const float cdf = 0.5f * erfcf(-alpha * 0.7071067811865475f);
+    const float t = m * cdf + sd * pdf;
+    mu_a[i] = fmaxf(0.000001f, t);
+    var_a[i] = fmaxf(0.000001f, -t * t + 2.f * t * m - m * sd * pdf + (v - m * m) * cdf);
+    jcb[i] = cdf;
+}
+
+// ---------------------------------------------------------------------------
+// Block-wide sums of up to four values, folded in a fixed order.
+// ---------------------------------------------------------------------------
+template <int NV>
+__device__ __forceinline__ void block_sum(float (&v)[NV], float (*s)[TPB / 64]) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) v[k] += __shfl_down(v[k], off, 64);
+        if (lane == 0) s[k][wave] = v[k];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+        float t = 0.f;
+#pragma unroll
+        for (int w = 0; w < TPB / 64; w++) t += s[k][w];
+        v[k] = t;
+    }
+    __syncthreads();
+}
+
+// ---------------------------------------------------------------------------
+// BatchNorm2d statistics. Workgroup (chunk, channel) owns the samples
+// [b_lo, b_hi) of one channel: element count, mean, sum of squared deviations
+// from that mean, and the sum of the activation variances. The chunks of a
+// channel are merged pairwise in index order (Chan et al.), which keeps the
+// two-pass accuracy of the reference's "mean first, then deviations".
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(TPB) void bn_stats_partial_kernel(
+    const float *__restrict__ mu_a, const float *__restrict__ var_a, int wihi, int fi, int B,
+    int b_per_chunk, float *__restrict__ part) {
+    __shared__ float s[2][TPB / 64];
+    const int c = blockIdx.y, chunk = blockIdx.x, chunks = gridDim.x;
+    const int b_lo = chunk * b_per_chunk, b_hi = min(B, b_lo + b_per_chunk);
+    const int count = max(0, b_hi - b_lo) * wihi;
+
+    float v[2] = {0.f, 0.f};
+    for (int i = threadIdx.x; i < count; i += TPB) {
+        const int b = b_lo + i / wihi, p = i % wihi;
+        const size_t at = ((size_t)b * fi + c) * wihi + p;
+        v[0] += mu_a[at];
+        v[1] += var_a[at];
+    }
+    block_sum<2>(v, s);
+    const float mean = count > 0 ? v[0] / count : 0.f;
+    const float sum_var = v[1];
+
+    float d[1] = {0.f};
+    for (int i = threadIdx.x; i < count; i += TPB) {
+        const int b = b_lo + i / wihi, p = i % wihi;
+        const float x = mu_a[((size_t)b * fi + c) * wihi + p] - mean;
+        d[0] += x * x;
+    }
+    block_sum<1>(d, s);
+    if (threadIdx.x == 0) {
+        float *o = part + ((size_t)c * chunks + chunk) * 4;
+        o[0] = (float)count;
+        o[1] = mean;
+        o[2] = d[0];
+        o[3] = sum_var;
+    }
+}
+
+__global__ __launch_bounds__(64) void bn_stats_final_kernel(const float *__restrict__ part,
+                                                            int fi, int chunks, float momentum,
+                                                            float *__restrict__ mu_s,
+                                                            float *__restrict__ var_s,
+                                                            float *__restrict__ mu_ra,
+                                                            float *__restrict__ var_ra) {
+    const int c = blockIdx.x * 64 + threadIdx.x;
+    if (c >= fi) return;
+    float n = 0.f, mean = 0.f, m2 = 0.f, sum_var = 0.f;
+    for (int q = 0; q < chunks; q++) {
+        const float *o = part + ((size_t)c * chunks + q) * 4;
+        const float nb = o[0];
+        if (nb <= 0.f) continue;
+        const float delta = o[1] - mean, tot = n + nb;
+        mean += delta * (nb / tot);
+        m2 += o[2] + delta * delta * (n * nb / tot);
+        n = tot;
+        sum_var += o[3];
+    }
+    const float var = (m2 + sum_var) / (n - 1.f);
+    mu_s[c] = mean;
+    var_s[c] = var;
+    mu_ra[c] = mu_ra[c] * momentum + mean * (1.f - momentum);
+    var_ra[c] = var_ra[c] * momentum + var * (1.f - momentum);
+}
+
+// z = (a - mean) / sqrt(var + eps) * w + b with Gaussian w, b and a.
+__global__ __launch_bounds__(TPB) void bn_fwd_kernel(
+    const float *__restrict__ mu_w, const float *__restrict__ var_w,
+    const float *__restrict__ mu_b, const float *__restrict__ var_b,
+    const float *__restrict__ mu_a, const float *__restrict__ var_a,
+    const float *__restrict__ mu_norm, const float *__restrict__ var_norm, float epsilon,
+    int wihi, int fi, size_t n, float *__restrict__ mu_z, float *__restrict__ var_z) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n) return;
+    const int c = (int)((i / wihi) % fi);
+    const float inv = 1.0f / sqrtf(var_norm[c] + epsilon);
+    const float mw = mu_w[c], vw = var_w[c];
+    const float d = mu_a[i] - mu_norm[c];
+    float mz = inv * d * mw;
+    float vz = inv * inv * (var_a[i] * (mw * mw + vw) + vw * d * d);
+    if (mu_b != nullptr) {
+        mz += mu_b[c];
+        vz += var_b[c];
+    }
+    mu_z[i] = mz;
+    var_z[i] = vz;
+}
+
+// Backward of one (chunk, channel): the state innovations element by element,
+// and partial sums of the four parameter innovations of the channel.
+__global__ __launch_bounds__(TPB) void bn_bwd_partial_kernel(
+    const float *__restrict__ mu_w, const float *__restrict__ var_w,
+    const float *__restrict__ mu_a, const float *__restrict__ jcb,
+    const float *__restrict__ mu_norm, const float *__restrict__ var_norm,
+    const float *__restrict__ dmu_out, const float *__restrict__ dvar_out, float epsilon,
+    int wihi, int fi, int B, int b_per_chunk, int state_update, int param_update,
+    float *__restrict__ dmu, float *__restrict__ dvar, float *__restrict__ part) {
+    __shared__ float s[4][TPB / 64];
+    const int c = blockIdx.y, chunk = blockIdx.x, chunks = gridDim.x;
+    const int b_lo = chunk * b_per_chunk, b_hi = min(B, b_lo + b_per_chunk);
+    const int count = max(0, b_hi - b_lo) * wihi;
+    const float inv = 1.0f / sqrtf(var_norm[c] + epsilon);
+    const float mean = mu_norm[c], mw = mu_w[c], vw = var_w[c];
+
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int i = threadIdx.x; i < count; i += TPB) {
+        const int b = b_lo + i / wihi, p = i % wihi;
+        const size_t at = ((size_t)b * fi + c) * wihi + p;
+        const float dm = dmu_out[at], dv = dvar_out[at];
+        if (state_update) {
+            const float t = inv * mw * jcb[at];
+            dmu[at] = t * dm;
+            dvar[at] = t * dv * t;
+        }
+        if (param_update) {
+            const float t = inv * (mu_a[at] - mean) * vw;
+            v[0] += t * dm;
+            v[1] += t * dv * t;
+            v[2] += dm;
+            v[3] += dv;
+        }
+    }
+    if (!param_update) return;
+    block_sum<4>(v, s);
+    if (threadIdx.x < 4) part[((size_t)c * chunks + chunk) * 4 + threadIdx.x] = v[threadIdx.x];
+}
+
+__global__ __launch_bounds__(64) void bn_bwd_final_kernel(const float *__restrict__ part,
+                                                          const float *__restrict__ var_b, int fi,
+                                                          int chunks, float *__restrict__ dmu_w,
+                                                          float *__restrict__ dvar_w,
+                                                          float *__restrict__ dmu_b,
+                                                          float *__restrict__ dvar_b) {
+    const int c = blockIdx.x * 64 + threadIdx.x;
+    if (c >= fi) return;
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int q = 0; q < chunks; q++) {
+        const float *o = part + ((size_t)c * chunks + q) * 4;
+#pragma unroll
+        for (int k = 0; k < 4; k++) v[k] += o[k];
+    }
+    dmu_w[c] = v[0];
+    dvar_w[c] = v[1];
+    if (var_b != nullptr) {
+        const float vb = var_b[c];
+        dmu_b[c] = vb * v[2];
+        dvar_b[c] = vb * v[3] * vb;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// AvgPool2d. pool_idx [k*k][woho]: 1-based input pixel under tap t of output
+// pixel o (-1: padding, which still counts in the divisor); z_ud_idx [nr][wihi]:
+// the output pixels an input pixel contributes to (overlapping windows only).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(TPB) void avgpool_fwd_kernel(const float *__restrict__ mu_a,
+                                                          const float *__restrict__ var_a,
+                                                          const int *__restrict__ pool_idx,
+                                                          int woho, int wihi, int ki2, int n_out,
+                                                          float *__restrict__ mu_z,
+                                                          float *__restrict__ var_z) {
+    const int col = blockIdx.x * TPB + threadIdx.x;
+    if (col >= n_out) return;
+    const int o = col % woho;
+    const size_t base = (size_t)(col / woho) * wihi;
+    float sm = 0.f, sv = 0.f;
+    for (int t = 0; t < ki2; t++) {
+        const int a = pool_idx[o + woho * t];
+        if (a > -1) {
+            sm += mu_a[base + a - 1];
+            sv += var_a[base + a - 1];
+        }
+    }
+    mu_z[col] = sm / ki2;
+    var_z[col] = sv / (ki2 * ki2);
+}
+
+__global__ __launch_bounds__(TPB) void avgpool_bwd_overlap_kernel(
+    const float *__restrict__ jcb, const float *__restrict__ dmu_out,
+    const float *__restrict__ dvar_out, const int *__restrict__ z_ud_idx, int woho, int wihi,
+    int ki2, int nr, int n_in, float *__restrict__ dmu, float *__restrict__ dvar) {
+    const int col = blockIdx.x * TPB + threadIdx.x;
+    if (col >= n_in) return;
+    const int p = col % wihi;
+    const size_t base = (size_t)(col / wihi) * woho;
+    float sm = 0.f, sv = 0.f;
+    for (int i = 0; i < nr; i++) {
+        const int z = z_ud_idx[p + wihi * i];
+        if (z > -1) {
+            sm += dmu_out[base + z - 1];
+            sv += dvar_out[base + z - 1];
+        }
+    }
+    const float j = jcb[col];
+    dmu[col] = sm * j / ki2;
+    dvar[col] = sv * j * j / (ki2 * ki2);
+}
+
+// Windows that tile the image: input element `at` lies in row at % (ki*wo) of
+// image-row block at / (ki*wo); its window is (row / ki, block / ki).
+__global__ __launch_bounds__(TPB) void avgpool_bwd_tiled_kernel(
+    const float *__restrict__ jcb, const float *__restrict__ dmu_out,
+    const float *__restrict__ dvar_out, int wo, int ki, int n_in, float *__restrict__ dmu,
+    float *__restrict__ dvar) {
+    const int at = blockIdx.x * TPB + threadIdx.x;
+    if (at >= n_in) return;
+    const int m = ki * wo, ki2 = ki * ki;
+    const int row = at % m, blk = at / m;
+    const int src = row / ki + (blk / ki) * wo;
+    const float j = jcb[at];
+    dmu[at] = dmu_out[src] * j / ki2;
+    dvar[at] = dvar_out[src] * j * j / (ki2 * ki2);
+}
+
+// ---------------------------------------------------------------------------
+// Residual connection
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(TPB) void add_shortcut_kernel(const float *__restrict__ mu_s,
+                                                           const float *__restrict__ var_s,
+                                                           const float *__restrict__ jcb_s,
+                                                           size_t n, float *__restrict__ mu_a,
+                                                           float *__restrict__ var_a) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n) return;
+    if (jcb_s != nullptr) {
+        const float j = jcb_s[i];
+        mu_a[i] += mu_s[i] * j;
+        var_a[i] += var_s[i] * j * j;
+    } else {
+        mu_a[i] += mu_s[i];
+        var_a[i] += var_s[i];
+    }
+}
+
+// Samples per chunk so that a channel-major grid has about 4 workgroups per CU.
+int bn_chunks(int fi, int B, int *b_per_chunk) {
+    int chunks = (4 * NUM_CU + fi - 1) / fi;
+    if (chunks > B) chunks = B;
+    if (chunks < 1) chunks = 1;
+    *b_per_chunk = (B + chunks - 1) / chunks;
+    return (B + *b_per_chunk - 1) / *b_per_chunk;
+}
+
+}  // namespace
+
+hipError_t launch_mixture_relu(const float *mu_z, const float *var_z, size_t n, float *mu_a,
+                               float *jcb, float *var_a, hipStream_t stream) {
+    hipLaunchKernelGGL(mixture_relu_kernel, dim3(blocks_for(n, TPB)), dim3(TPB), 0, stream, mu_z,
+                       var_z, n, mu_a, jcb, var_a);
+    return hipGetLastError();
+}
+
+size_t batchnorm2d_scratch_floats(int fi, int B) {
+    int per = 0;
+    return (size_t)bn_chunks(fi, B, &per) * fi * 4;
+}
+
+hipError_t launch_batchnorm2d_stats(const float *mu_a, const float *var_a, int wihi, int fi,
+                                    int B, float momentum, float *scratch, float *mu_s,
+                                    float *var_s, float *mu_ra, float *var_ra,
+                                    hipStream_t stream) {
+    int per = 0;
+    const int chunks = bn_chunks(fi, B, &per);
+    hipLaunchKernelGGL(bn_stats_partial_kernel, dim3(chunks, fi), dim3(TPB), 0, stream, mu_a,
+                       var_a, wihi, fi, B, per, scratch);
+    hipLaunchKernelGGL(bn_stats_final_kernel, dim3((fi + 63) / 64), dim3(64), 0, stream, scratch,
+                       fi, chunks, momentum, mu_s, var_s, mu_ra, var_ra);
+    return hipGetLastError();
+}
+
+hipError_t launch_batchnorm2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
+                                  const float *var_b, const float *mu_a, const float *var_a,
+                                  const float *mu_norm, const float *var_norm, float epsilon,
+                                  int wihi, int fi, int B, float *mu_z, float *var_z,
+                                  hipStream_t stream) {
+    const size_t n = (size_t)B * fi * wihi;
+    hipLaunchKernelGGL(bn_fwd_kernel, dim3(blocks_for(n, TPB)), dim3(TPB), 0, stream, mu_w, var_w,
+                       mu_b, var_b, mu_a, var_a, mu_norm, var_norm, epsilon, wihi, fi, n, mu_z,
+                       var_z);
+    return hipGetLastError();
+}
+
+hipError_t launch_batchnorm2d_bwd(const float *mu_w, const float *var_w, const float *var_b,
+                                  const float *mu_a, const float *jcb, const float *mu_norm,
+                                  const float *var_norm, const float *dmu_out,
+                                  const float *dvar_out, float epsilon, int wihi, int fi, int B,
+                                  int state_update, int param_update, float *scratch, float *dmu,
+                                  float *dvar, float *dmu_w, float *dvar_w, float *dmu_b,
+                                  float *dvar_b, hipStream_t stream) {
+    int per = 0;
+    const int chunks = bn_chunks(fi, B, &per);
+    hipLaunchKernelGGL(bn_bwd_partial_kernel, dim3(chunks, fi), dim3(TPB), 0, stream, mu_w, var_w,
+                       mu_a, jcb, mu_norm, var_norm, dmu_out, dvar_out, epsilon, wihi, fi, B, per,
+                       state_update, param_update, dmu, dvar, scratch);
+    if (param_update)
+        hipLaunchKernelGGL(bn_bwd_final_kernel, dim3((fi + 63) / 64), dim3(64), 0, stream, scratch,
+                           var_b, fi, chunks, dmu_w, dvar_w, dmu_b, dvar_b);
+    return hipGetLastError();
+}
+
+hipError_t launch_avgpool2d_fwd(const float *mu_a, const float *var_a, const int *pool_idx,
+                                int woho, int wihi, int ki, int n_out, float *mu_z, float *var_z,
+                                hipStream_t stream) {
+    hipLaunchKernelGGL(avgpool_fwd_kernel, dim3(blocks_for(n_out, TPB)), dim3(TPB), 0, stream,
+                       mu_a, var_a, pool_idx, woho, wihi, ki * ki, n_out, mu_z, var_z);
+    return hipGetLastError();
+}
+
+hipError_t launch_avgpool2d_bwd(const float *jcb, const float *dmu_out, const float *dvar_out,
+                                const int *z_ud_idx, int woho, int wihi, int ki, int nr, int wo,
+                                int n_in, int overlap, float *dmu, float *dvar,
+                                hipStream_t stream) {
+    if (overlap)
+        hipLaunchKernelGGL(avgpool_bwd_overlap_kernel, dim3(blocks_for(n_in, TPB)), dim3(TPB), 0,
+                           stream, jcb, dmu_out, dvar_out, z_ud_idx, woho, wihi, ki * ki, nr, n_in,
+                           dmu, dvar);
+    else
+        hipLaunchKernelGGL(avgpool_bwd_tiled_kernel, dim3(blocks_for(n_in, TPB)), dim3(TPB), 0,
+                           stream, jcb, dmu_out, dvar_out, wo, ki, n_in, dmu, dvar);
+    return hipGetLastError();
+}
+
+hipError_t launch_add_shortcut(const float *mu_s, const float *var_s, const float *jcb_s,
+                               size_t n, float *mu_a, float *var_a, hipStream_t stream) {
+    hipLaunchKernelGGL(add_shortcut_kernel, dim3(blocks_for(n, TPB)), dim3(TPB), 0, stream, mu_s,
+                       var_s, jcb_s, n, mu_a, var_a);
+    return hipGetLastError();
+}
+
+}  // namespace tagi

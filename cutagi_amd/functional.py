@@ -173,3 +173,90 @@ def relu_fwd(mu_z, var_z, mu_a=None, jcb=None, var_a=None):
     capi.check(capi.lib.tagi_relu_fwd(capi.ptr(mu_z), capi.ptr(var_z), mu_z.numel(),
                                       capi.ptr(mu_a), capi.ptr(jcb), capi.ptr(var_a), _stream()))
     return mu_a, var_a, jcb
+
+
+def mixture_relu_fwd(mu_z, var_z, mu_a=None, jcb=None, var_a=None):
+    _chk(mu_z, var_z, mu_a, jcb, var_a)
+    mu_a = torch.empty_like(mu_z) if mu_a is None else mu_a
+    jcb = torch.empty_like(mu_z) if jcb is None else jcb
+    var_a = torch.empty_like(mu_z) if var_a is None else var_a
+    capi.check(capi.lib.tagi_mixture_relu_fwd(capi.ptr(mu_z), capi.ptr(var_z), mu_z.numel(),
+                                              capi.ptr(mu_a), capi.ptr(jcb), capi.ptr(var_a),
+                                              _stream()))
+    return mu_a, var_a, jcb
+
+
+def batchnorm2d_stats(mu_a, var_a, wihi, fi, B, momentum, mu_ra, var_ra):
+    """Batch statistics (returned) and the running averages (updated in place)."""
+    _chk(mu_a, var_a, mu_ra, var_ra)
+    mu_s, var_s = torch.empty(fi, device=mu_a.device), torch.empty(fi, device=mu_a.device)
+    capi.check(capi.lib.tagi_batchnorm2d_stats(capi.ptr(mu_a), capi.ptr(var_a), wihi, fi, B,
+                                               momentum, capi.ptr(mu_s), capi.ptr(var_s),
+                                               capi.ptr(mu_ra), capi.ptr(var_ra), _stream()))
+    return mu_s, var_s
+
+
+def batchnorm2d_fwd(mu_w, var_w, mu_b, var_b, mu_a, var_a, mu_norm, var_norm, eps, wihi, fi, B):
+    _chk(mu_w, var_w, mu_b, var_b, mu_a, var_a, mu_norm, var_norm)
+    mu_z, var_z = torch.empty_like(mu_a), torch.empty_like(mu_a)
+    capi.check(capi.lib.tagi_batchnorm2d_fwd(capi.ptr(mu_w), capi.ptr(var_w), capi.ptr(mu_b),
+                                             capi.ptr(var_b), capi.ptr(mu_a), capi.ptr(var_a),
+                                             capi.ptr(mu_norm), capi.ptr(var_norm),
+                                             int(mu_b is not None), eps, wihi, fi, B,
+                                             capi.ptr(mu_z), capi.ptr(var_z), _stream()))
+    return mu_z, var_z
+
+
+def batchnorm2d_bwd(mu_w, var_w, var_b, mu_a, jcb, mu_norm, var_norm, delta_mu, delta_var, eps,
+                    wihi, fi, B, state_update=True, param_update=True):
+    """Returns (dz_mu, dz_var, dw_mu, dw_var, db_mu, db_var); entries not asked for are None."""
+    _chk(mu_w, var_w, var_b, mu_a, jcb, mu_norm, var_norm, delta_mu, delta_var)
+    dev = mu_w.device
+    bias = var_b is not None
+    out = [None] * 6
+    if state_update:
+        out[0], out[1] = torch.empty_like(delta_mu), torch.empty_like(delta_mu)
+    if param_update:
+        out[2], out[3] = torch.empty(fi, device=dev), torch.empty(fi, device=dev)
+        if bias:
+            out[4], out[5] = torch.empty(fi, device=dev), torch.empty(fi, device=dev)
+    capi.check(capi.lib.tagi_batchnorm2d_bwd(
+        capi.ptr(mu_w), capi.ptr(var_w), capi.ptr(var_b), capi.ptr(mu_a), capi.ptr(jcb),
+        capi.ptr(mu_norm), capi.ptr(var_norm), capi.ptr(delta_mu), capi.ptr(delta_var), eps, wihi,
+        fi, B, int(bias), int(state_update), int(param_update), *[capi.ptr(t) for t in out],
+        _stream()))
+    return tuple(out)
+
+
+def avgpool2d_fwd(mu_a, var_a, pool_idx, woho, wihi, ki, n_out):
+    _chk(mu_a, var_a, pool_idx)
+    mu_z, var_z = torch.empty(n_out, device=mu_a.device), torch.empty(n_out, device=mu_a.device)
+    capi.check(capi.lib.tagi_avgpool2d_fwd(capi.ptr(mu_a), capi.ptr(var_a), capi.ptr(pool_idx),
+                                           woho, wihi, ki, n_out, capi.ptr(mu_z), capi.ptr(var_z),
+                                           _stream()))
+    return mu_z, var_z
+
+
+def avgpool2d_bwd_dz(jcb, delta_mu, delta_var, z_ud_idx, woho, wihi, ki, nr, wo, overlap):
+    _chk(jcb, delta_mu, delta_var, z_ud_idx)
+    om, ov = torch.empty_like(jcb), torch.empty_like(jcb)
+    capi.check(capi.lib.tagi_avgpool2d_bwd_dz(capi.ptr(jcb), capi.ptr(delta_mu),
+                                              capi.ptr(delta_var), capi.ptr(z_ud_idx), woho, wihi,
+                                              ki, nr, wo, jcb.numel(), int(overlap), capi.ptr(om),
+                                              capi.ptr(ov), _stream()))
+    return om, ov
+
+
+def add_shortcut(mu_s, var_s, mu_a, var_a):
+    """In place on mu_a/var_a."""
+    _chk(mu_s, var_s, mu_a, var_a)
+    capi.check(capi.lib.tagi_add_shortcut(capi.ptr(mu_s), capi.ptr(var_s), mu_a.numel(),
+                                          capi.ptr(mu_a), capi.ptr(var_a), _stream()))
+
+
+def add_shortcut_delta(mu_s, var_s, jcb_s, mu_a, var_a):
+    """In place on mu_a/var_a."""
+    _chk(mu_s, var_s, jcb_s, mu_a, var_a)
+    capi.check(capi.lib.tagi_add_shortcut_delta(capi.ptr(mu_s), capi.ptr(var_s), capi.ptr(jcb_s),
+                                                mu_a.numel(), capi.ptr(mu_a), capi.ptr(var_a),
+                                                _stream()))

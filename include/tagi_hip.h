@@ -192,6 +192,101 @@ int tagi_out_update_indexed(const float *mu_a, const float *var_a,
 int tagi_relu_fwd(const float *mu_z, const float *var_z, size_t n, float *mu_a,
                   float *jcb, float *var_a, void *stream);
 
+/* ---- MixtureReLU ------------------------------------------------------------- */
+
+/* Moments of max(z, 0) for z ~ N(mu_z, var_z), both floored at 1e-6; jcb = P(z > 0).
+ * Replaces mixture_relu_mean_var_cuda as MixtureReLUCuda::forward launches it
+ * (src/activation_cuda.cu:130-150, 726-760); CPU form src/activation.cpp:152-178.
+ * In place allowed. */
+int tagi_mixture_relu_fwd(const float *mu_z, const float *var_z, size_t n,
+                          float *mu_a, float *jcb, float *var_a, void *stream);
+
+/* ---- BatchNorm2d ------------------------------------------------------------- */
+/* Tensors are [B][fi][wihi]; a fully-connected input is wihi = 1, fi = features.
+ * Parameters, statistics and running averages are [fi]. */
+
+/* Training-mode statistics: mu_s = mean over (B, wihi), var_s = (sum of squared
+ * deviations + sum of var_a) / (B*wihi - 1), then mu_ra/var_ra <- ra*momentum +
+ * s*(1 - momentum). Replaces the reduction sequence of BatchNorm2dCuda::forward
+ * (src/batchnorm_layer_cuda.cu:915-948); CPU form src/batchnorm_layer.cpp:15-26,
+ * 127-168. Uses the workspace. */
+int tagi_batchnorm2d_stats(const float *mu_a, const float *var_a, int wihi,
+                           int fi, int B, float momentum, float *mu_s,
+                           float *var_s, float *mu_ra, float *var_ra,
+                           void *stream);
+
+/* mu_z = (mu_a - mu_norm)/sqrt(var_norm + eps) * mu_w (+ mu_b); var_z likewise
+ * with Gaussian weights. mu_norm/var_norm: batch statistics when training, running
+ * averages otherwise. Replaces batchnorm2d_fwd_mean_var_cuda
+ * (src/batchnorm_layer_cuda.cu:507-543, launched at 950-959); CPU form
+ * src/batchnorm_layer.cpp:170-206. */
+int tagi_batchnorm2d_fwd(const float *mu_w, const float *var_w,
+                         const float *mu_b, const float *var_b,
+                         const float *mu_a, const float *var_a,
+                         const float *mu_norm, const float *var_norm, int bias,
+                         float epsilon, int wihi, int fi, int B, float *mu_z,
+                         float *var_z, void *stream);
+
+/* All of BatchNorm2dCuda::backward (src/batchnorm_layer_cuda.cu:969-1102) in one
+ * call: state innovations (state_update) and the per-channel weight / bias
+ * innovations (param_update; bias ones only when bias != 0). mu_a and jcb are the
+ * layer's stored input states. CPU form src/batchnorm_layer.cpp:233-255, 307-354
+ * and delta_param_sum (src/common.cpp:360-378). Uses the workspace. */
+int tagi_batchnorm2d_bwd(const float *mu_w, const float *var_w,
+                         const float *var_b, const float *mu_a,
+                         const float *jcb, const float *mu_norm,
+                         const float *var_norm, const float *delta_mu_out,
+                         const float *delta_var_out, float epsilon, int wihi,
+                         int fi, int B, int bias, int state_update,
+                         int param_update, float *delta_mu, float *delta_var,
+                         float *delta_mu_w, float *delta_var_w,
+                         float *delta_mu_b, float *delta_var_b, void *stream);
+
+/* ---- AvgPool2d ---------------------------------------------------------------- */
+
+/* Host tables of a pooling layer, as AvgPool2d::lazy_index_init builds them
+ * (src/pooling_layer.cpp:186-210 over get_pool_index, 453-484): pool_idx
+ * [kernel*kernel][wo*ho] (1-based input pixel, -1 = padding) and, only when the
+ * windows overlap (*overlap = 1), z_ud_idx [h][w] (1-based output pixel, -1 =
+ * none). Caller provides pool_idx[wo*ho*k*k] and z_ud_idx[wi*hi*k*k]. The output
+ * size comes from tagi_conv2d_out_size; stride -1 (the pooling default) is valid
+ * for a window that covers the whole image. */
+int tagi_avgpool2d_build_idx(int kernel, int stride, int wi, int hi, int pad,
+                             int pad_type, int *pool_idx, int *z_ud_idx, int *w,
+                             int *h, int *overlap);
+
+/* mu_z = window sum / k^2, var_z = window sum / k^4 (padding counts in the
+ * divisor); n_out = woho*channels*B. Replaces avgpool2d_fwd_*_mean_var_cuda
+ * (src/pooling_layer_cuda.cu:13-64, launched at 167-218); CPU form
+ * src/pooling_layer.cpp:201-225, 259-280. */
+int tagi_avgpool2d_fwd(const float *mu_a, const float *var_a,
+                       const int *pool_idx, int woho, int wihi, int ki,
+                       int n_out, float *mu_z, float *var_z, void *stream);
+
+/* State innovations of the pooling layer; n_in = wihi*channels*B. overlap != 0
+ * walks z_ud_idx (nr rows); otherwise the windows tile the image and wo (output
+ * width) is enough. Replaces avgpool2d_bwd_*_delta_z_cuda
+ * (src/pooling_layer_cuda.cu:66-120, launched at 220-270); CPU form
+ * src/pooling_layer.cpp:316-340, 379-399. */
+int tagi_avgpool2d_bwd_dz(const float *jcb, const float *delta_mu_out,
+                          const float *delta_var_out, const int *z_ud_idx,
+                          int woho, int wihi, int ki, int nr, int wo, int n_in,
+                          int overlap, float *delta_mu, float *delta_var,
+                          void *stream);
+
+/* ---- residual connection -------------------------------------------------------- */
+
+/* mu_a += mu_s, var_a += var_s; replaces add_shortcut_mean_var_cuda
+ * (src/resnet_block_cuda.cu:7-18); CPU form src/resnet_block.cpp:8-18. */
+int tagi_add_shortcut(const float *mu_s, const float *var_s, size_t n,
+                      float *mu_a, float *var_a, void *stream);
+
+/* mu_a += mu_s*jcb_s, var_a += var_s*jcb_s^2; replaces add_shortcut_delta_cuda
+ * (src/resnet_block_cuda.cu:20-33); CPU form src/resnet_block.cpp:20-31. */
+int tagi_add_shortcut_delta(const float *mu_s, const float *var_s,
+                            const float *jcb_s, size_t n, float *mu_a,
+                            float *var_a, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
