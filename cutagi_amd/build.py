@@ -45,7 +45,7 @@ def build(extra_flags=(), objdir=None, lib=LIB):
     return lib
 
 
-HOST_SOURCES = ["states.cpp", "layers.cpp", "sequential.cpp", "bindings.cpp"]
+HOST_SOURCES = ["states.cpp", "layers.cpp", "blocks.cpp", "sequential.cpp", "bindings.cpp"]
 
 
 def build_host():

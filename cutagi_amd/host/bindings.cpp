@@ -8,6 +8,7 @@
 #include <cstring>
 
 #include "../../include/tagi_hip.h"
+#include "blocks.h"
 #include "sequential.h"
 
 namespace py = pybind11;
@@ -99,17 +100,9 @@ PYBIND11_MODULE(cutagi, m) {
         .def("get_layer_name", &BaseLayer::get_layer_name)
         .def("get_max_num_states", &BaseLayer::get_max_num_states)
         .def("preinit_layer", &BaseLayer::preinit_layer)
-        .def("params_to_host",
-             [](BaseLayer &l) {
-                 if (auto *d = dynamic_cast<BaseLayerHip *>(&l)) d->params_to_host();
-             })
-        .def("params_to_device",
-             [](BaseLayer &l) {
-                 if (auto *d = dynamic_cast<BaseLayerHip *>(&l)) d->params_to_device();
-             })
-        .def("delta_params_to_host", [](BaseLayer &l) {
-            if (auto *d = dynamic_cast<BaseLayerHip *>(&l)) d->delta_params_to_host();
-        });
+        .def("params_to_host", &BaseLayer::params_to_host)
+        .def("params_to_device", &BaseLayer::params_to_device)
+        .def("delta_params_to_host", &BaseLayer::delta_params_to_host);
 
     py::class_<Linear, BaseLayer, std::shared_ptr<Linear>>(m, "Linear")
         .def(py::init<size_t, size_t, bool, float, float, std::string, int>(), py::arg("ip_size"),
@@ -126,6 +119,40 @@ PYBIND11_MODULE(cutagi, m) {
              py::arg("init_method") = "He", py::arg("device_idx") = 0)
         .def("init_weight_bias", &Conv2d::init_weight_bias);
     py::class_<ReLU, BaseLayer, std::shared_ptr<ReLU>>(m, "ReLU").def(py::init<>());
+    py::class_<MixtureReLU, BaseLayer, std::shared_ptr<MixtureReLU>>(m, "MixtureReLU")
+        .def(py::init<>());
+    // argument names and defaults of the reference's binding
+    // (src/bindings/norm_layer_bindings.cpp:31-42)
+    py::class_<BatchNorm2d, BaseLayer, std::shared_ptr<BatchNorm2d>>(m, "BatchNorm2d")
+        .def(py::init<int, float, float, bool, float, float>(), py::arg("num_features"),
+             py::arg("eps") = 1e-4f, py::arg("mometum") = 0.9f, py::arg("bias") = true,
+             py::arg("gain_weight") = 1.0f, py::arg("gain_bias") = 1.0f)
+        .def_readwrite("mu_ra", &BatchNorm2d::mu_ra)
+        .def_readwrite("var_ra", &BatchNorm2d::var_ra)
+        .def("init_weight_bias", &BatchNorm2d::init_weight_bias);
+    py::class_<BatchNorm2dHip, BaseLayer, std::shared_ptr<BatchNorm2dHip>>(m, "BatchNorm2dCuda")
+        .def("get_norm_mean_var", &BatchNorm2dHip::get_norm_mean_var);
+    py::class_<AvgPool2d, BaseLayer, std::shared_ptr<AvgPool2d>>(m, "AvgPool2d")
+        .def(py::init<size_t, int, int, int, int>(), py::arg("kernel_size"),
+             py::arg("stride") = -1, py::arg("padding") = 0, py::arg("padding_type") = 0,
+             py::arg("device_idx") = 0);
+    py::class_<LayerBlock, BaseLayer, std::shared_ptr<LayerBlock>>(m, "LayerBlock")
+        .def(py::init<>())
+        .def(py::init([](const std::vector<std::shared_ptr<BaseLayer>> &layers) {
+            return std::make_shared<LayerBlock>(layers);
+        }))
+        .def("add_layer", &LayerBlock::add_layer)
+        .def("switch_to_cuda", &LayerBlock::switch_to_cuda)
+        .def_readwrite("layers", &LayerBlock::layers);
+    py::class_<ResNetBlock, BaseLayer, std::shared_ptr<ResNetBlock>>(m, "ResNetBlock")
+        .def(py::init<std::shared_ptr<BaseLayer>, std::shared_ptr<BaseLayer>>(),
+             py::arg("main_block"), py::arg("shortcut") = nullptr)
+        .def_readwrite("main_block", &ResNetBlock::main_block)
+        .def_readwrite("shortcut", &ResNetBlock::shortcut)
+        .def_readwrite("input_z", &ResNetBlock::input_z)
+        .def_readwrite("input_delta_z", &ResNetBlock::input_delta_z)
+        .def_readwrite("shortcut_output_z", &ResNetBlock::shortcut_output_z)
+        .def_readwrite("shortcut_output_delta_z", &ResNetBlock::shortcut_output_delta_z);
 
     py::class_<OutputUpdater, std::shared_ptr<OutputUpdater>>(m, "OutputUpdater")
         .def(py::init<const std::string>())

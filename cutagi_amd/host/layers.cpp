@@ -7,51 +7,11 @@
 #include <cstring>
 
 #include "../../include/tagi_hip.h"
+#include "host_util.h"
 #include "logger.h"
 
 namespace tagi_host {
 
-namespace {
-template <typename T>
-T *dev_alloc_t(size_t n, int device_idx) {
-    T *p = nullptr;
-    if (n == 0) return p;
-    HIP_OK(hipSetDevice(device_idx));
-    HIP_OK(hipMalloc(reinterpret_cast<void **>(&p), n * sizeof(T)));
-    return p;
-}
-template <typename T>
-void dev_free_t(T *&p) {
-    if (p != nullptr) (void)hipFree(p);
-    p = nullptr;
-}
-void h2d(float *dst, const std::vector<float> &src) {
-    if (!src.empty())
-        HIP_OK(hipMemcpy(dst, src.data(), src.size() * sizeof(float), hipMemcpyHostToDevice));
-}
-void d2h(std::vector<float> &dst, const float *src, size_t n) {
-    dst.resize(n);
-    if (n) HIP_OK(hipMemcpy(dst.data(), src, n * sizeof(float), hipMemcpyDeviceToHost));
-}
-void write_floats(std::ofstream &f, const std::vector<float> &v) {
-    f.write(reinterpret_cast<const char *>(v.data()), v.size() * sizeof(float));
-}
-void read_floats(std::ifstream &f, std::vector<float> &v) {
-    f.read(reinterpret_cast<char *>(v.data()), v.size() * sizeof(float));
-}
-template <typename T>
-T *as(BaseHiddenStates &s) {
-    auto *p = dynamic_cast<T *>(&s);
-    if (p == nullptr) LOG(LogLevel::ERROR, "Device layer received host state buffers");
-    return p;
-}
-template <typename T>
-T *as(BaseDeltaStates &s) {
-    auto *p = dynamic_cast<T *>(&s);
-    if (p == nullptr) LOG(LogLevel::ERROR, "Device layer received host delta buffers");
-    return p;
-}
-}  // namespace
 
 void manual_seed(int seed) { SeedManager::get_instance().set_seed(seed); }
 

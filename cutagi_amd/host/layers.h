@@ -16,7 +16,7 @@
 
 namespace tagi_host {
 
-enum class LayerType { Base, Linear, Conv2d, Activation };
+enum class LayerType { Base, Linear, Conv2d, Activation, Pool2d, Norm, LayerBlock, ResNetBlock };
 
 class InitArgs {
    public:
@@ -105,6 +105,11 @@ class BaseLayer {
     virtual std::vector<ParameterTuple> parameters();
     virtual void preinit_layer() {}
     virtual int get_neg_var_w_counter() { return neg_var_w_counter; }
+    // host <-> device copies of the parameters; layers without device storage
+    // have nothing to move, blocks pass the call on to their members
+    virtual void params_to_device() {}
+    virtual void params_to_host() {}
+    virtual void delta_params_to_host() {}
 
    protected:
     [[noreturn]] void no_cpu_path(const char *what) const;
@@ -133,9 +138,9 @@ class BaseLayerHip : public BaseLayer {
     std::vector<ParameterTuple> parameters() override;
     int get_neg_var_w_counter() override;
 
-    virtual void params_to_device();
-    virtual void params_to_host();
-    virtual void delta_params_to_host();
+    void params_to_device() override;
+    void params_to_host() override;
+    void delta_params_to_host() override;
     void copy_params_from(const BaseLayer &source);
 
    protected:

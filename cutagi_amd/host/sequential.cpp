@@ -147,12 +147,10 @@ void Sequential::to_device(const std::string &new_device) {
 }
 
 void Sequential::params_to_host() {
-    for (auto &layer : layers)
-        if (auto *l = dynamic_cast<BaseLayerHip *>(layer.get())) l->params_to_host();
+    for (auto &layer : layers) layer->params_to_host();
 }
 void Sequential::params_to_device() {
-    for (auto &layer : layers)
-        if (auto *l = dynamic_cast<BaseLayerHip *>(layer.get())) l->params_to_device();
+    for (auto &layer : layers) layer->params_to_device();
 }
 
 void Sequential::set_buffer_size() {
@@ -308,7 +306,9 @@ void Sequential::load(const std::string &filename) {
 std::vector<ParameterTuple> Sequential::parameters() {
     std::vector<ParameterTuple> params;
     for (auto &layer : layers) {
-        if (layer->get_layer_type() == LayerType::Activation) continue;
+        if (layer->get_layer_type() == LayerType::Activation ||
+            layer->get_layer_type() == LayerType::Pool2d)
+            continue;
         auto p = layer->parameters();
         params.insert(params.end(), p.begin(), p.end());
     }
@@ -318,7 +318,9 @@ std::vector<ParameterTuple> Sequential::parameters() {
 ParameterMap Sequential::state_dict() {
     ParameterMap sd;
     for (size_t i = 0; i < layers.size(); i++) {
-        if (layers[i]->get_layer_type() == LayerType::Activation) continue;
+        if (layers[i]->get_layer_type() == LayerType::Activation ||
+            layers[i]->get_layer_type() == LayerType::Pool2d)
+            continue;
         auto p = layers[i]->get_parameters_as_map(std::to_string(i));
         sd.insert(p.begin(), p.end());
     }
@@ -327,7 +329,9 @@ ParameterMap Sequential::state_dict() {
 
 void Sequential::load_state_dict(const ParameterMap &sd) {
     for (size_t i = 0; i < layers.size(); i++) {
-        if (layers[i]->get_layer_type() == LayerType::Activation) continue;
+        if (layers[i]->get_layer_type() == LayerType::Activation ||
+            layers[i]->get_layer_type() == LayerType::Pool2d)
+            continue;
         layers[i]->load_parameters_from_map(sd, std::to_string(i));
     }
 }
