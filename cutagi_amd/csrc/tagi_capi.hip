@@ -54,6 +54,7 @@ struct Tuning {
     int dw_splits = -1;
     int gemv_max_batch = -1;
     int conv_dw_tile = -1;
+    int conv_splits = -1;
     int tile = -1;
     int conv_dw_splits = -1;
     int gemv_swz = -1;
@@ -177,6 +178,7 @@ int tagi_hip_tune(const char *key, int value) {
     else if (!strcmp(key, "linear.dw.splits")) g_tune.dw_splits = value;
     else if (!strcmp(key, "linear.gemv_max_batch")) g_tune.gemv_max_batch = value;
     else if (!strcmp(key, "conv2d.dw.tile")) g_tune.conv_dw_tile = value;
+    else if (!strcmp(key, "conv2d.splits")) g_tune.conv_splits = value;
     else if (!strcmp(key, "linear.tile")) g_tune.tile = value;
     else if (!strcmp(key, "conv2d.dw.splits")) g_tune.conv_dw_splits = value;
     else if (!strcmp(key, "linear.gemv.swizzle")) g_tune.gemv_swz = value;
@@ -390,8 +392,18 @@ int tagi_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b, co
         return TAGI_ERR_INVALID_ARG;
     if (bias && (!mu_b || !var_b)) return TAGI_ERR_INVALID_ARG;
     if (!conv_sizes_ok(B, fo, woho, fi, wihi, ki)) return TAGI_ERR_UNSUPPORTED;
+    int tile = 0, splits = 1;
+    conv2d_plan(fo, B * woho, ki * ki * fi, &tile, &splits);
+    if (g_tune.conv_splits > 0) splits = g_tune.conv_splits;
+    float *ws = nullptr;
+    const size_t part = splits > 1 ? (size_t)splits * fo * B * woho : 0;
+    if (part) {
+        int rc = workspace_get(2 * part * sizeof(float), &ws);
+        if (rc != TAGI_OK) return rc;
+    }
     TAGI_TRY(launch_conv2d_fwd(mu_w, var_w, mu_b, var_b, mu_a, var_a, aidx, woho, fo, wihi, fi, ki,
-                               B, bias, mu_z, var_z, static_cast<hipStream_t>(stream_)));
+                               B, bias, tile, splits, ws, ws + part, mu_z, var_z,
+                               static_cast<hipStream_t>(stream_)));
     return TAGI_OK;
 }
 
@@ -405,9 +417,18 @@ int tagi_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *delta_m
     if (woho <= 0 || fo <= 0 || wihi <= 0 || fi <= 0 || ki <= 0 || nr <= 0 || B <= 0)
         return TAGI_ERR_INVALID_ARG;
     if (!conv_sizes_ok(B, fo, woho, fi, wihi, ki)) return TAGI_ERR_UNSUPPORTED;
+    int tile = 0, splits = 1;
+    conv2d_plan(fi, B * wihi, ki * ki * fo, &tile, &splits);
+    if (g_tune.conv_splits > 0) splits = g_tune.conv_splits;
+    float *ws = nullptr;
+    const size_t part = splits > 1 ? (size_t)splits * fi * B * wihi : 0;
+    if (part) {
+        int rc = workspace_get(2 * part * sizeof(float), &ws);
+        if (rc != TAGI_OK) return rc;
+    }
     TAGI_TRY(launch_conv2d_bwd_dz(mu_w, jcb, delta_mu_out, delta_var_out, zw_idx, zud_idx, woho,
-                                  fo, wihi, fi, ki, nr, B, delta_mu, delta_var,
-                                  static_cast<hipStream_t>(stream_)));
+                                  fo, wihi, fi, ki, nr, B, tile, splits, ws, ws + part, delta_mu,
+                                  delta_var, static_cast<hipStream_t>(stream_)));
     return TAGI_OK;
 }
 

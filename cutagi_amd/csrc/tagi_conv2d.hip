@@ -364,36 +364,65 @@ inline bool aligned16(const void *q) { return (reinterpret_cast<uintptr_t>(q) & 
 
 }  // namespace
 
+// Tile shape and number of reduction slices of the forward / state-backward
+// GEMMs: M rows (output or input channels), N columns (batch x pixels), R
+// reduction (taps x channels). Late ResNet stages have few columns and a long
+// reduction; slicing it keeps every CU busy.
+void conv2d_plan(int M, int N, int R, int *tile, int *splits) {
+    *tile = M > 32 ? TILE_64x128 : TILE_32x128;
+    const int tiles = ceil_div(M, tile_rows(*tile)) * ceil_div(N, tile_cols(*tile));
+    const int k_tiles = ceil_div(R, KT);
+    int s = ceil_div(2 * NUM_CU, tiles);
+    const int cap = k_tiles / 8 > 0 ? k_tiles / 8 : 1;  // at least 8 k-tiles per slice
+    if (s > cap) s = cap;
+    if (s < 1) s = 1;
+    const int per = ceil_div(ceil_div(R, s), KT) * KT;
+    *splits = ceil_div(R, per);
+}
+
+namespace {
+template <class P>
+hipError_t run_sliced(int tile, int splits, float *ws0, float *ws1, ConvParams &p,
+                      hipStream_t stream) {
+    const int per = ceil_div(ceil_div(p.R, splits), KT) * KT;
+    p.splits = ceil_div(p.R, per);
+    p.r_per_split = per;
+    p.ws0 = ws0;
+    p.ws1 = ws1;
+    hipError_t e = launch_tiles<P>(tile, p, stream);
+    if (e != hipSuccess || p.splits == 1) return e;
+    return launch_reduce_store<P>(p, stream);
+}
+}  // namespace
+
 hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
                              const float *var_b, const float *mu_a, const float *var_a,
                              const int *aidx, int woho, int fo, int wihi, int fi, int ki, int B,
-                             int bias, float *mu_z, float *var_z, hipStream_t stream) {
+                             int bias, int tile, int splits, float *ws0, float *ws1, float *mu_z,
+                             float *var_z, hipStream_t stream) {
     ConvParams p = {};
     p.w0 = mu_w; p.w1 = var_w; p.a0 = mu_a; p.a1 = var_a;
     p.e0 = bias ? mu_b : nullptr; p.e1 = bias ? var_b : nullptr;
     p.idx = aidx; p.out0 = mu_z; p.out1 = var_z;
     p.woho = woho; p.fo = fo; p.wihi = wihi; p.fi = fi; p.k2 = ki * ki; p.B = B;
-    p.M = fo; p.N = B * woho; p.R = p.k2 * fi; p.splits = 1;
-    p.r_per_split = ceil_div(p.R, KT) * KT;
-    const int tile = fo > 64 ? TILE_128x128 : fo > 32 ? TILE_64x128 : TILE_32x128;
+    p.M = fo; p.N = B * woho; p.R = p.k2 * fi;
     const bool vec = (p.R % 4 == 0) && aligned16(mu_w) && aligned16(var_w);
-    if (vec) return launch_tiles<ConvFwdProblem<true>>(tile, p, stream);
-    return launch_tiles<ConvFwdProblem<false>>(tile, p, stream);
+    if (vec) return run_sliced<ConvFwdProblem<true>>(tile, splits, ws0, ws1, p, stream);
+    return run_sliced<ConvFwdProblem<false>>(tile, splits, ws0, ws1, p, stream);
 }
 
 hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *dmu,
                                 const float *dvar, const int *zw_idx, const int *zud_idx,
                                 int woho, int fo, int wihi, int fi, int ki, int nr, int B,
-                                float *out_dmu, float *out_dvar, hipStream_t stream) {
+                                int tile, int splits, float *ws0, float *ws1, float *out_dmu,
+                                float *out_dvar, hipStream_t stream) {
     const int k2 = ki * ki;
     ConvParams p = {};
     p.w0 = mu_w; p.d0 = dmu; p.d1 = dvar; p.e0 = jcb; p.idx = zw_idx; p.idx2 = zud_idx;
     p.out0 = out_dmu; p.out1 = out_dvar;
     p.woho = woho; p.fo = fo; p.wihi = wihi; p.fi = fi; p.k2 = k2; p.B = B; p.nr = nr;
-    p.M = fi; p.N = B * wihi; p.R = k2 * fo; p.splits = 1;
-    p.r_per_split = ceil_div(p.R, KT) * KT;
-    const int tile = fi > 64 ? TILE_128x128 : fi > 32 ? TILE_64x128 : TILE_32x128;
-    return launch_tiles<ConvDzProblem>(tile, p, stream);
+    p.M = fi; p.N = B * wihi; p.R = k2 * fo;
+    return run_sliced<ConvDzProblem>(tile, splits, ws0, ws1, p, stream);
 }
 
 // Workgroups of the weight-backward kernel that one CU holds at a time.

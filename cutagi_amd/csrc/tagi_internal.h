@@ -119,14 +119,17 @@ hipError_t launch_add_shortcut(const float *mu_s, const float *var_s, const floa
                                size_t n, float *mu_a, float *var_a, hipStream_t stream);
 
 // Conv2d (implicit GEMM through the index tables)
+void conv2d_plan(int M, int N, int R, int *tile, int *splits);
 hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
                              const float *var_b, const float *mu_a, const float *var_a,
                              const int *aidx, int woho, int fo, int wihi, int fi, int ki, int B,
-                             int bias, float *mu_z, float *var_z, hipStream_t stream);
+                             int bias, int tile, int splits, float *ws0, float *ws1, float *mu_z,
+                             float *var_z, hipStream_t stream);
 hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *dmu,
                                 const float *dvar, const int *zw_idx, const int *zud_idx,
                                 int woho, int fo, int wihi, int fi, int ki, int nr, int B,
-                                float *out_dmu, float *out_dvar, hipStream_t stream);
+                                int tile, int splits, float *ws0, float *ws1, float *out_dmu,
+                                float *out_dvar, hipStream_t stream);
 int conv2d_bwd_dw_blocks_per_cu(int tile);
 hipError_t launch_conv2d_bwd_dw(const float *var_w, const float *mu_a, const float *dmu,
                                 const float *dvar, const int *aidx, int B, int fo, int woho,

@@ -281,6 +281,30 @@ __global__ __launch_bounds__(WM *WN * 64) void mfma_tile_kernel(typename P::Para
         }
 }
 
+// Folds the partial sums of a sliced reduction (ws0/ws1 [split][M][N]) in slice
+// order and hands every output element to the problem's epilogue.
+template <class P>
+__global__ __launch_bounds__(256) void reduce_store_kernel(typename P::Params p) {
+    const size_t total = (size_t)p.M * p.N;
+    const size_t at = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (at >= total) return;
+    float s0 = 0.f, s1 = 0.f;
+#pragma unroll 4
+    for (int s = 0; s < p.splits; s++) {
+        s0 += p.ws0[s * total + at];
+        s1 += p.ws1[s * total + at];
+    }
+    P::store(p, (int)(at / p.N), (int)(at % p.N), s0, s1);
+}
+
+template <class P>
+hipError_t launch_reduce_store(const typename P::Params &p, hipStream_t stream) {
+    const size_t total = (size_t)p.M * p.N;
+    hipLaunchKernelGGL((reduce_store_kernel<P>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                       stream, p);
+    return hipGetLastError();
+}
+
 // Launch over a (tiles, splits) grid for one of the instantiated tile shapes.
 enum TileShape { TILE_128x128 = 0, TILE_64x128 = 1, TILE_32x128 = 2, TILE_64x64 = 3, TILE_COUNT = 4 };
 

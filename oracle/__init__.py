@@ -290,6 +290,15 @@ class Oracle:
         return mu_a, var_a
 
 
+    # ---- hierarchical softmax (reference build only) -----------------------------
+    def class_to_obs(self, n_classes):
+        n_obs = int(np.ceil(np.log2(n_classes)))
+        obs = np.zeros(n_classes * n_obs, np.float32)
+        idx = np.zeros(n_classes * n_obs, np.int32)
+        a, b = ctypes.c_int(0), ctypes.c_int(0)
+        self._fn("class_to_obs")(n_classes, _fp(obs), _ip(idx), ctypes.byref(a), ctypes.byref(b))
+        return obs.reshape(n_classes, n_obs), idx.reshape(n_classes, n_obs), a.value, b.value
+
 
 def load():
     path = os.path.join(_HERE, "liboracle.so")

@@ -13,6 +13,7 @@
 #include "base_layer.h"
 #include "base_output_updater.h"
 #include "conv2d_layer.h"
+#include "cost.h"
 #include "linear_layer.h"
 #include "pooling_layer.h"
 
@@ -505,6 +506,16 @@ void ref_add_shortcut_delta(const float *mu_s, const float *var_s, const float *
     add_shortcut_delta(ms, vs, js, n, ma, va);
     put(ma, mu_a);
     put(va, var_a);
+}
+
+// Hierarchical-softmax label encoding (src/cost.cpp:76-143). obs and idx hold
+// n_classes * ceil(log2(n_classes)) entries.
+void ref_class_to_obs(int n_classes, float *obs, int *idx, int *n_obs, int *len) {
+    HRCSoftmax hs = class_to_obs(n_classes);
+    std::memcpy(obs, hs.obs.data(), hs.obs.size() * sizeof(float));
+    std::memcpy(idx, hs.idx.data(), hs.idx.size() * sizeof(int));
+    *n_obs = (int)hs.n_obs;
+    *len = (int)hs.len;
 }
 
 }  // extern "C"

@@ -21,6 +21,8 @@ GEOMS = [
     (3, 1, 1, 1, 12, 70, 66, 1),
     (4, 2, 1, 1, 10, 3, 5, 2),
     (7, 2, 3, 1, 17, 3, 40, 2),  # per-tap table + staged tiles exceed 64 KB of LDS
+    (3, 1, 1, 1, 4, 128, 96, 3),  # late-stage shape: few pixels, long reduction (sliced)
+    (2, 2, 0, 1, 8, 64, 130, 2),  # projection shortcut, more than 128 output channels
 ]
 
 

@@ -61,3 +61,26 @@ def test_host_state_containers():
     d.delta_mu = [1.0] * 8
     d.reset_zeros()
     assert d.delta_mu == [0.0] * 8
+
+
+def test_hierarchical_softmax_ten_classes():
+    """The encoding for 10 classes, as the compiled reference's class_to_obs(10)
+    gives it: 4 observations per label among 11 outputs."""
+    import numpy as np
+    from cutagi_amd.resnet import hrc_softmax
+    obs, idx, n_obs, length = hrc_softmax(10)
+    assert (n_obs, length) == (4, 11)
+    assert idx.tolist() == [[1, 2, 4, 7], [1, 2, 4, 7], [1, 2, 4, 8], [1, 2, 4, 8], [1, 2, 5, 9],
+                            [1, 2, 5, 9], [1, 2, 5, 10], [1, 2, 5, 10], [1, 3, 6, 11], [1, 3, 6, 11]]
+    bits = [[(c >> s) & 1 for s in (3, 2, 1, 0)] for c in range(10)]
+    assert np.array_equal(obs, np.where(np.array(bits) == 1, -1.0, 1.0).astype(np.float32))
+
+
+def test_resnet18_builds_on_the_host():
+    from cutagi_amd.resnet import resnet18_cifar10
+    net = resnet18_cifar10()
+    info = net.get_layer_stack_info().split()
+    assert info[0] == "Conv2d(3,64,32,32,3)" and info[-1] == "Linear(512,11)"
+    assert info[-2] == "AvgPool2d(512,512,1,1,4)"
+    assert net.z_buffer_size == 64 * 32 * 32
+    assert len(net.layers) == 13

@@ -166,3 +166,14 @@ def test_shortcut_adds(oracle_lib, ref):
     assert _eq(oracle_lib.add_shortcut(v[0], v[1], v[2], v[3]), ref.add_shortcut(v[0], v[1], v[2], v[3]))
     assert _eq(oracle_lib.add_shortcut_delta(v[0], v[1], v[4], v[2], v[3]),
                ref.add_shortcut_delta(v[0], v[1], v[4], v[2], v[3]))
+
+
+@pytest.mark.parametrize("n_classes", [2, 3, 5, 8, 10, 17, 33, 100, 1000])
+def test_hierarchical_softmax_encoding(ref, n_classes):
+    """cutagi_amd.resnet.hrc_softmax (what a training script feeds the output
+    updater) against the reference's class_to_obs."""
+    from cutagi_amd.resnet import hrc_softmax
+    obs, idx, n_obs, length = hrc_softmax(n_classes)
+    r_obs, r_idx, r_n, r_len = ref.class_to_obs(n_classes)
+    assert (n_obs, length) == (r_n, r_len)
+    assert np.array_equal(obs, r_obs) and np.array_equal(idx, r_idx)
