@@ -8,8 +8,8 @@ Linear layer on synthetic inputs that are resident in HBM before the timed
 region starts. The default workload is the dense one the headline metric is
 quoted on (4096 -> 4096, batch 256, fp32); `--workload skinny` times the
 HBM-bound one (8192 -> 8192, batch 8) and reports GB/s. The default run also
-times the skinny workload and the CPU baseline and attaches them to the same
-JSON line.
+times the skinny workload, the Conv2d workload, one training step of the CIFAR
+ResNet-18 and the CPU baseline, and attaches them to the same JSON line.
 
 Prints ONE JSON line. `roofline` is computed for the dominant kernel from its
 algorithmic work and its average duration measured with HIP events on the
@@ -200,6 +200,49 @@ def run_conv(steps, warmup):
                 frac_of_peak=round(tflops / FP32_MFMA_PEAK_TFLOPS, 4), ms_per_step=round(ms, 5))
 
 
+def run_resnet(steps, warmup, B=128):
+    """One training step of the CIFAR ResNet-18 (forward, hierarchical-softmax output
+    update, backward, parameter step) through the host classes, batch 128. Inputs
+    are handed over as host arrays, as the reference's API takes them, so the
+    figure includes their copy to the device."""
+    import numpy as np
+    import torch
+    from cutagi_amd import cutagi
+    from cutagi_amd.resnet import hrc_softmax, resnet18_cifar10
+
+    cutagi.manual_seed(0)
+    net = resnet18_cifar10(cutagi)
+    net.to_device("cuda")
+    updater = cutagi.OutputUpdater(net.device)
+    obs, idx, n_obs, _ = hrc_softmax(10)
+    rng = np.random.default_rng(0)
+    x = rng.normal(0, 1, (B, 3 * 32 * 32)).astype(np.float32)
+    labels = rng.integers(0, 10, B)
+    y, sel = obs[labels].ravel().tolist(), idx[labels].ravel().tolist()
+    var_y = [1.0] * (B * n_obs)
+
+    def step():
+        net.forward(x)
+        updater.update_using_indices(net.output_z_buffer, y, var_y, sel, net.input_delta_z_buffer)
+        net.backward()
+        net.step()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    mu, var = net.get_outputs()
+    ok = bool(np.all(np.isfinite(mu)) and var.min() >= 0)
+    return dict(workload="TAGI ResNet-18 (CIFAR: 3x32x32 input, BatchNorm, MixtureReLU, 11 "
+                         "hierarchical-softmax outputs), batch %d, one training step" % B,
+                value=round(B / (ms * 1e-3), 1), unit="images/s", ms_per_step=round(ms, 3),
+                outputs_finite_and_variances_nonnegative=ok)
+
+
 def calibrate_copy():
     """A plain device copy of known size (1 GiB read + 1 GiB written), so that
     hardware byte counters of a profiler run can be scaled."""
@@ -299,6 +342,7 @@ def main():
             "phase_ms": {k: round(v, 5) for k, v in r["phase_ms"].items()},
             "roofline": r["roofline"]}}
         line["extra"]["conv"] = run_conv(max(5, args.steps // 2), args.warmup)
+        line["extra"]["resnet18"] = run_resnet(max(5, args.steps // 5), 3)
     if args.calibrate:
         calibrate_copy()
     if not args.no_cpu:

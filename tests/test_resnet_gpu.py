@@ -144,3 +144,38 @@ def test_resnet_checkpoint_and_eval(tmp_path, oracle_lib):
     net2.forward(x)
     assert np.array_equal(net.get_outputs()[0], net2.get_outputs()[0])
     assert np.all(np.isfinite(net.get_outputs()[0]))
+
+
+def test_resnet18_full_size_step():
+    """The ResNet-18 configuration at its real size (batch 128): one training step
+    through the host classes. Too large for the CPU emulation; checked through what
+    holds at any size: finite outputs, non-negative output variances, every
+    parameter variance positive after the step, running variances positive."""
+    from cutagi_amd import cutagi
+    from cutagi_amd.resnet import hrc_softmax, resnet18_cifar10
+    B = 128
+    cutagi.manual_seed(0)
+    net = resnet18_cifar10(cutagi)
+    net.to_device("cuda")
+    updater = cutagi.OutputUpdater(net.device)
+    obs, idx, n_obs, n_out = hrc_softmax(10)
+    rng = np.random.default_rng(0)
+    x = rng.normal(0, 1, (B, 3 * 32 * 32)).astype(np.float32)
+    labels = rng.integers(0, 10, B)
+    for _ in range(2):
+        net.forward(x)
+        mu, var = net.get_outputs()
+        assert mu.shape == (B * n_out,) and np.all(np.isfinite(mu)) and np.all(np.isfinite(var))
+        assert var.min() >= 0
+        updater.update_using_indices(net.output_z_buffer, obs[labels].ravel().tolist(),
+                                     [1.0] * (B * n_obs), idx[labels].ravel().tolist(),
+                                     net.input_delta_z_buffer)
+        net.backward()
+        net.step()
+    sd = net.state_dict()
+    assert len(sd) == 41  # 20 convolutions, 20 batch norms, 1 linear
+    for key, (mu_w, var_w, mu_b, var_b) in sd.items():
+        assert np.all(np.isfinite(mu_w)) and min(var_w) > 0, key
+        if len(var_b):
+            assert np.all(np.isfinite(mu_b)) and min(var_b) > 0, key
+    assert min(net.layers[2].get_norm_mean_var()[1]) > 0
