@@ -55,6 +55,7 @@ struct Tuning {
     int gemv_max_batch = -1;
     int conv_dw_tile = -1;
     int conv_splits = -1;
+    int conv_tile = -1;
     int tile = -1;
     int conv_dw_splits = -1;
     int gemv_swz = -1;
@@ -179,6 +180,7 @@ int tagi_hip_tune(const char *key, int value) {
     else if (!strcmp(key, "linear.gemv_max_batch")) g_tune.gemv_max_batch = value;
     else if (!strcmp(key, "conv2d.dw.tile")) g_tune.conv_dw_tile = value;
     else if (!strcmp(key, "conv2d.splits")) g_tune.conv_splits = value;
+    else if (!strcmp(key, "conv2d.tile")) g_tune.conv_tile = value;
     else if (!strcmp(key, "linear.tile")) g_tune.tile = value;
     else if (!strcmp(key, "conv2d.dw.splits")) g_tune.conv_dw_splits = value;
     else if (!strcmp(key, "linear.gemv.swizzle")) g_tune.gemv_swz = value;
@@ -239,9 +241,11 @@ int tagi_linear_fwd(const float *mu_w, const float *var_w, const float *mu_b, co
     return run_gemm(GEMM_FWD, p, vec, g_tune.fwd_splits, stream);
 }
 
-int tagi_linear_bwd_dz(const float *mu_w, const float *jcb, const float *delta_mu,
-                       const float *delta_var, int K, int N, int B, float *delta_mu_z,
-                       float *delta_var_z, void *stream_) {
+// State backward; with `defer` given and the skinny-batch kernel running, the
+// slices are left unfolded and described in *defer for a later kernel to fold.
+static int linear_bwd_dz_impl(const float *mu_w, const float *jcb, const float *delta_mu,
+                              const float *delta_var, int K, int N, int B, float *delta_mu_z,
+                              float *delta_var_z, DzFold *defer, void *stream_) {
     if (!mu_w || !jcb || !delta_mu || !delta_var || !delta_mu_z || !delta_var_z)
         return TAGI_ERR_INVALID_ARG;
     if (K <= 0 || N <= 0 || B <= 0) return TAGI_ERR_INVALID_ARG;
@@ -266,6 +270,12 @@ int tagi_linear_bwd_dz(const float *mu_w, const float *jcb, const float *delta_m
         TAGI_TRY(launch_gemv_dz(mu_w, delta_mu, delta_var, K, N, B, splits,
                                 (g_tune.gemv_rev >= 0 ? g_tune.gemv_rev : 8) & 3, ws, ws + part,
                                 stream));
+        if (defer != nullptr && aligned16(jcb) && aligned16(delta_mu_z) && aligned16(delta_var_z)) {
+            defer->ws0 = ws; defer->ws1 = ws + part; defer->jcb = jcb;
+            defer->out0 = delta_mu_z; defer->out1 = delta_var_z;
+            defer->splits = splits; defer->total = (size_t)B * K;
+            return TAGI_OK;
+        }
         TAGI_TRY(launch_reduce_splits(EPI_SCALE, ws, ws + part, splits, B, K, jcb, nullptr,
                                       delta_mu_z, delta_var_z, K, stream));
         return TAGI_OK;
@@ -279,12 +289,20 @@ int tagi_linear_bwd_dz(const float *mu_w, const float *jcb, const float *delta_m
     return run_gemm(GEMM_DZ, p, vec, g_tune.dz_splits, stream);
 }
 
+int tagi_linear_bwd_dz(const float *mu_w, const float *jcb, const float *delta_mu,
+                       const float *delta_var, int K, int N, int B, float *delta_mu_z,
+                       float *delta_var_z, void *stream) {
+    return linear_bwd_dz_impl(mu_w, jcb, delta_mu, delta_var, K, N, B, delta_mu_z, delta_var_z,
+                              nullptr, stream);
+}
+
 // Weight backward; when the bias pointers are given and the skinny-batch kernel
 // runs, that kernel also writes the bias innovations and *bias_done is set.
 static int linear_bwd_dw_impl(const float *var_w, const float *mu_a, const float *delta_mu,
                               const float *delta_var, int K, int N, int B, float *delta_mu_w,
                               float *delta_var_w, const float *var_b, float *delta_mu_b,
-                              float *delta_var_b, bool *bias_done, void *stream_) {
+                              float *delta_var_b, bool *bias_done, const DzFold *fold,
+                              bool *fold_done, void *stream_) {
     if (!var_w || !mu_a || !delta_mu || !delta_var || !delta_mu_w || !delta_var_w)
         return TAGI_ERR_INVALID_ARG;
     if (K <= 0 || N <= 0 || B <= 0) return TAGI_ERR_INVALID_ARG;
@@ -295,8 +313,10 @@ static int linear_bwd_dw_impl(const float *var_w, const float *mu_a, const float
     if (B <= gemv_max_batch() && k_vec) {
         TAGI_TRY(launch_gemv_dw(var_w, mu_a, delta_mu, delta_var, K, N, B,
                                 ((g_tune.gemv_rev >= 0 ? g_tune.gemv_rev : 8) >> 2) & 3,
-                                delta_mu_w, delta_var_w, var_b, delta_mu_b, delta_var_b, stream));
+                                delta_mu_w, delta_var_w, var_b, delta_mu_b, delta_var_b, fold,
+                                stream));
         if (bias_done) *bias_done = var_b != nullptr;
+        if (fold_done) *fold_done = fold != nullptr;
         return TAGI_OK;
     }
 
@@ -313,7 +333,7 @@ int tagi_linear_bwd_dw(const float *var_w, const float *mu_a, const float *delta
                        const float *delta_var, int K, int N, int B, float *delta_mu_w,
                        float *delta_var_w, void *stream) {
     return linear_bwd_dw_impl(var_w, mu_a, delta_mu, delta_var, K, N, B, delta_mu_w, delta_var_w,
-                              nullptr, nullptr, nullptr, nullptr, stream);
+                              nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, stream);
 }
 
 int tagi_linear_bwd_db(const float *var_b, const float *delta_mu, const float *delta_var, int N,
@@ -332,22 +352,32 @@ int tagi_linear_bwd(const float *mu_w, const float *var_w, const float *var_b, c
                     float *delta_var_z, float *delta_mu_w, float *delta_var_w, float *delta_mu_b,
                     float *delta_var_b, void *stream) {
     int rc = TAGI_OK;
+    if (param_update && bias && (!var_b || !delta_mu_b || !delta_var_b))
+        return TAGI_ERR_INVALID_ARG;
+    DzFold fold;
     if (state_update) {
-        rc = tagi_linear_bwd_dz(mu_w, jcb, delta_mu, delta_var, K, N, B, delta_mu_z, delta_var_z,
-                                stream);
+        rc = linear_bwd_dz_impl(mu_w, jcb, delta_mu, delta_var, K, N, B, delta_mu_z, delta_var_z,
+                                param_update ? &fold : nullptr, stream);
         if (rc != TAGI_OK) return rc;
     }
+    const bool pending = fold.ws0 != nullptr;
+    bool fold_done = false;
     if (param_update) {
-        if (bias && (!var_b || !delta_mu_b || !delta_var_b)) return TAGI_ERR_INVALID_ARG;
         bool bias_done = false;
         rc = linear_bwd_dw_impl(var_w, mu_a, delta_mu, delta_var, K, N, B, delta_mu_w, delta_var_w,
                                 bias ? var_b : nullptr, delta_mu_b, delta_var_b, &bias_done,
-                                stream);
+                                pending ? &fold : nullptr, &fold_done, stream);
         if (rc != TAGI_OK) return rc;
         if (bias && !bias_done) {
             rc = tagi_linear_bwd_db(var_b, delta_mu, delta_var, N, B, delta_mu_b, delta_var_b,
                                     stream);
+            if (rc != TAGI_OK) return rc;
         }
+    }
+    if (pending && !fold_done) {  // the weight backward took the tiled path: fold here
+        TAGI_TRY(launch_reduce_splits(EPI_SCALE, fold.ws0, fold.ws1, fold.splits, B, K, fold.jcb,
+                                      nullptr, fold.out0, fold.out1, K,
+                                      static_cast<hipStream_t>(stream)));
     }
     return rc;
 }
@@ -395,6 +425,7 @@ int tagi_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b, co
     int tile = 0, splits = 1;
     conv2d_plan(fo, B * woho, ki * ki * fi, &tile, &splits);
     if (g_tune.conv_splits > 0) splits = g_tune.conv_splits;
+    if (g_tune.conv_tile >= 0 && g_tune.conv_tile < gemm_tile_count()) tile = g_tune.conv_tile;
     float *ws = nullptr;
     const size_t part = splits > 1 ? (size_t)splits * fo * B * woho : 0;
     if (part) {
@@ -420,6 +451,7 @@ int tagi_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *delta_m
     int tile = 0, splits = 1;
     conv2d_plan(fi, B * wihi, ki * ki * fo, &tile, &splits);
     if (g_tune.conv_splits > 0) splits = g_tune.conv_splits;
+    if (g_tune.conv_tile >= 0 && g_tune.conv_tile < gemm_tile_count()) tile = g_tune.conv_tile;
     float *ws = nullptr;
     const size_t part = splits > 1 ? (size_t)splits * fi * B * wihi : 0;
     if (part) {

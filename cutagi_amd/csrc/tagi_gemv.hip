@@ -454,8 +454,33 @@ __global__ __launch_bounds__(256) void gemv_dw_kernel(
     const float *__restrict__ var_w, const float *__restrict__ mu_a,
     const float *__restrict__ dmu, const float *__restrict__ dvar, int K, int N, int B, int rev,
     float *__restrict__ dmu_w, float *__restrict__ dvar_w, const float *__restrict__ var_b,
-    float *__restrict__ dmu_b, float *__restrict__ dvar_b) {
+    float *__restrict__ dmu_b, float *__restrict__ dvar_b, DzFold fold) {
     __shared__ __attribute__((aligned(16))) float s_dm[DW_ROWS_PER_BLOCK][BMAX];
+    // The state backward that ran before this kernel may have left its slices
+    // unfolded: every workgroup folds its share of them first (a few float4 each),
+    // which saves a launch of its own for that.
+    if (fold.ws0 != nullptr) {
+        const size_t items = fold.total / 4;
+        const size_t nwg = (size_t)gridDim.x * gridDim.y;
+        const size_t per = (items + nwg - 1) / nwg;
+        const size_t wg = (size_t)blockIdx.y * gridDim.x + blockIdx.x;
+        for (size_t it = threadIdx.x; it < per; it += 256) {
+            const size_t at = (wg * per + it) * 4;
+            if (at >= fold.total) break;
+            float4 m = zero4(), v = zero4();
+            for (int sl = 0; sl < fold.splits; sl++) {
+                const float4 a = ld4(fold.ws0 + sl * fold.total + at);
+                const float4 b = ld4(fold.ws1 + sl * fold.total + at);
+                m.x += a.x; m.y += a.y; m.z += a.z; m.w += a.w;
+                v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
+            }
+            const float4 j = ld4(fold.jcb + at);
+            *reinterpret_cast<float4 *>(fold.out0 + at) =
+                make_float4(m.x * j.x, m.y * j.y, m.z * j.z, m.w * j.w);
+            *reinterpret_cast<float4 *>(fold.out1 + at) = make_float4(
+                v.x * j.x * j.x, v.y * j.y * j.y, v.z * j.z * j.z, v.w * j.w * j.w);
+        }
+    }
     __shared__ __attribute__((aligned(16))) float s_dv[DW_ROWS_PER_BLOCK][BMAX];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     // same XCD-aware choice of the column block as in the state backward
@@ -656,31 +681,32 @@ template <int BMAX>
 static void dw_launch(bool exact, dim3 grid, hipStream_t stream, const float *var_w,
                       const float *mu_a, const float *dmu, const float *dvar, int K, int N, int B,
                       int rev, float *dmu_w, float *dvar_w, const float *var_b, float *dmu_b,
-                      float *dvar_b) {
+                      float *dvar_b, const DzFold &fold) {
     if (exact)
         hipLaunchKernelGGL((gemv_dw_kernel<BMAX, true>), grid, dim3(256), 0, stream, var_w, mu_a,
-                           dmu, dvar, K, N, B, rev, dmu_w, dvar_w, var_b, dmu_b, dvar_b);
+                           dmu, dvar, K, N, B, rev, dmu_w, dvar_w, var_b, dmu_b, dvar_b, fold);
     else
         hipLaunchKernelGGL((gemv_dw_kernel<BMAX, false>), grid, dim3(256), 0, stream, var_w, mu_a,
-                           dmu, dvar, K, N, B, rev, dmu_w, dvar_w, var_b, dmu_b, dvar_b);
+                           dmu, dvar, K, N, B, rev, dmu_w, dvar_w, var_b, dmu_b, dvar_b, fold);
 }
 
 hipError_t launch_gemv_dw(const float *var_w, const float *mu_a, const float *dmu,
                           const float *dvar, int K, int N, int B, int rev, float *dmu_w,
                           float *dvar_w, const float *var_b, float *dmu_b, float *dvar_b,
-                          hipStream_t stream) {
+                          const DzFold *fold_in, hipStream_t stream) {
+    const DzFold fold = fold_in ? *fold_in : DzFold();
     dim3 grid((K + DW_COLS_PER_BLOCK - 1) / DW_COLS_PER_BLOCK,
               (N + DW_ROWS_PER_BLOCK - 1) / DW_ROWS_PER_BLOCK);
     const bool exact = (K % DW_COLS_PER_BLOCK == 0) && (N % DW_ROWS_PER_BLOCK == 0);
     if (B <= 4)
         dw_launch<4>(exact, grid, stream, var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w,
-                      var_b, dmu_b, dvar_b);
+                      var_b, dmu_b, dvar_b, fold);
     else if (B <= 8)
         dw_launch<8>(exact, grid, stream, var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w,
-                      var_b, dmu_b, dvar_b);
+                      var_b, dmu_b, dvar_b, fold);
     else
         dw_launch<16>(exact, grid, stream, var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w,
-                      var_b, dmu_b, dvar_b);
+                      var_b, dmu_b, dvar_b, fold);
     return hipGetLastError();
 }
 

@@ -58,10 +58,19 @@ hipError_t launch_gemv_fwd(const float *mu_w, const float *var_w, const float *m
 hipError_t launch_gemv_dz(const float *mu_w, const float *dmu, const float *dvar, int K,
                           int N, int B, int splits, int rev, float *ws0, float *ws1,
                           hipStream_t stream);
+// Partial sums of a sliced state backward that a later kernel folds:
+// out = (sum over slices of ws) * jcb (mean) and * jcb^2 (variance).
+struct DzFold {
+    const float *ws0 = nullptr, *ws1 = nullptr;  // [splits][total]
+    const float *jcb = nullptr;
+    float *out0 = nullptr, *out1 = nullptr;
+    int splits = 0;
+    size_t total = 0;  // B * K, a multiple of 4
+};
 hipError_t launch_gemv_dw(const float *var_w, const float *mu_a, const float *dmu,
                           const float *dvar, int K, int N, int B, int rev, float *dmu_w,
                           float *dvar_w, const float *var_b, float *dmu_b, float *dvar_b,
-                          hipStream_t stream);
+                          const DzFold *fold, hipStream_t stream);
 int gemv_fwd_variants();
 int gemv_fwd_rows_per_block(int variant);
 int gemv_fwd_k_step();
