@@ -121,6 +121,7 @@ struct ConvFwdProblem {
         ctx.bn = bn;
         ctx.tab = tab;
     }
+    __device__ static __forceinline__ void next_tile(const Params &, Ctx &) {}
     __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &, int arr, int, int m0,
                                                     int row, int r, int r_end) {
         return load_rows_kc<VEC>(arr ? p.w1 : p.w0, p.R, m0 + row, p.M, r, r_end);
@@ -193,6 +194,7 @@ struct ConvDwProblem {
             lookup(p, ctx, i, r_begin + (f % (KT / 4)) * 4);
         }
     }
+    __device__ static __forceinline__ void next_tile(const Params &, Ctx &) {}
     __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &, int arr, int, int m0,
                                                     int row, int r, int r_end) {
         const float *__restrict__ d = arr ? p.d1 : p.d0;
@@ -242,6 +244,102 @@ struct ConvDwProblem {
     }
 };
 
+// The same contraction when every group of four reduction positions lies in one
+// image (woho % 4 == 0, 16-byte aligned innovations): all positions of a thread
+// move together, so the thread keeps (pixel, image offsets) of its group in
+// registers and advances them by one k-tile per visit instead of dividing; the
+// innovations are one 16-byte load.
+struct ConvDwVecProblem {
+    using Params = ConvParams;
+    struct Ctx {
+        int o;      // pixel of the group in the tile being fetched
+        int xoff;   // b*fo*woho + o of that group
+        int img;    // b*fi*wihi
+        int xrow[2];            // m*woho of the row slots, -1: no row
+        int cb[DW_SLOTS];       // ch*wihi of the column slots, -1: no column
+        int tap[DW_SLOTS];
+        int nidx[DW_SLOTS][4];  // table entries of the tile being fetched
+    };
+    static constexpr bool XK = true, YK = true, PROLOGUE_WRITES_LDS = false, SPLIT_PER_XCD = true;
+    static constexpr int NX = 2, NY = 1, FLAVOR = FLAVOR_DELTA_ROWS;
+
+    static size_t extra_lds_bytes(const Params &, int, int) { return 0; }
+
+    __device__ static __forceinline__ void lookup(const Params &p, Ctx &ctx, int i, int o) {
+        const int *q = p.idx + (size_t)(o * p.k2 + ctx.tap[i]);
+#pragma unroll
+        for (int j = 0; j < 4; j++) ctx.nidx[i][j] = q[j * p.k2];
+    }
+    __device__ static __forceinline__ void prologue(const Params &p, Ctx &ctx, int *, int tid,
+                                                    int nthreads, int m0, int n0, int bm, int bn,
+                                                    int r_begin, int) {
+        const int r = min(r_begin + (tid % (KT / 4)) * 4, p.R - 4);
+        const int b = r / p.woho;
+        ctx.o = r - b * p.woho;
+        ctx.xoff = b * p.fo * p.woho + ctx.o;
+        ctx.img = b * p.fi * p.wihi;
+        const int xslots = bm * KT / 4 / nthreads, yslots = bn * KT / 4 / nthreads;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            if (i >= xslots) break;
+            const int m = m0 + (tid + i * nthreads) / (KT / 4);
+            ctx.xrow[i] = m < p.M ? m * p.woho : -1;
+        }
+#pragma unroll
+        for (int i = 0; i < DW_SLOTS; i++) {
+            if (i >= yslots) break;
+            const int n = n0 + (tid + i * nthreads) / (KT / 4);
+            const int nn = min(n, p.N - 1);
+            const int ch = nn / p.k2;
+            ctx.tap[i] = nn - ch * p.k2;
+            ctx.cb[i] = n < p.N ? ch * p.wihi : -1;
+            lookup(p, ctx, i, ctx.o);
+        }
+    }
+    __device__ static __forceinline__ void next_tile(const Params &p, Ctx &ctx) {
+        ctx.o += KT;
+        ctx.xoff += KT;
+        while (ctx.o >= p.woho) {
+            ctx.o -= p.woho;
+            ctx.img += p.fi * p.wihi;
+            ctx.xoff += (p.fo - 1) * p.woho;
+        }
+    }
+    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &ctx, int arr, int i, int,
+                                                    int, int r, int r_end) {
+        const bool ok = r < r_end && ctx.xrow[i] >= 0;
+        const float *__restrict__ d = arr ? p.d1 : p.d0;
+        const float4 v = *reinterpret_cast<const float4 *>(d + (ok ? ctx.xrow[i] + ctx.xoff : 0));
+        return ok ? v : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &ctx, int, int i, int,
+                                                    int, int r, int r_end) {
+        const bool live = r < r_end && ctx.cb[i] >= 0;
+        const int base = ctx.img + ctx.cb[i] - 1;
+        float c[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int a = ctx.nidx[i][j];
+            const bool ok = live && a > -1;
+            const float v = p.a0[ok ? base + a : 0];
+            c[j] = ok ? v : 0.f;
+        }
+        // table entries of the next k-tile (always inside the table: the pixel
+        // index wraps, and a group of four never straddles its end)
+        int o = ctx.o + KT;
+        while (o >= p.woho) o -= p.woho;
+        lookup(p, ctx, i, o);
+        return make_float4(c[0], c[1], c[2], c[3]);
+    }
+    __device__ static __forceinline__ void store(const Params &p, int m, int n, float a0,
+                                                 float a1) {
+        const size_t at = (size_t)m * p.N + n;
+        const float e = p.e0[at];
+        p.out0[at] = a0 * e;
+        p.out1[at] = a1 * e * e;
+    }
+};
+
 // ---- state backward -----------------------------------------------------------
 // rows: weights re-indexed [c][(fo,t)]; columns: gathered deltas [(fo,t)][(b,p)].
 // The reference's FCzwa_1 / Szz_ud pair lists, per input pixel, the (tap, output
@@ -276,6 +374,7 @@ struct ConvDzProblem {
         ctx.bn = bn;
         ctx.tab = tab;
     }
+    __device__ static __forceinline__ void next_tile(const Params &, Ctx &) {}
     __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &, int, int, int m0,
                                                     int row, int r, int r_end) {
         const int m = m0 + row;
@@ -432,7 +531,7 @@ int conv2d_bwd_dw_blocks_per_cu(int tile) {
     if (cached[tile] == 0) {
         int n = 0;
         hipError_t e = hipErrorInvalidValue;
-        using P = ConvDwProblem<true>;
+        using P = ConvDwVecProblem;
         switch (tile) {
             case TILE_128x128:
                 e = hipOccupancyMaxActiveBlocksPerMultiprocessor(
@@ -470,7 +569,7 @@ hipError_t launch_conv2d_bwd_dw(const float *var_w, const float *mu_a, const flo
     p.r_per_split = per;
     p.ws0 = ws0; p.ws1 = ws1;
     const bool vec = (woho % 4 == 0) && aligned16(dmu) && aligned16(dvar);
-    hipError_t e = vec ? launch_tiles<ConvDwProblem<true>>(tile, p, stream)
+    hipError_t e = vec ? launch_tiles<ConvDwVecProblem>(tile, p, stream)
                        : launch_tiles<ConvDwProblem<false>>(tile, p, stream);
     if (e != hipSuccess) return e;
     if (p.splits > 1)

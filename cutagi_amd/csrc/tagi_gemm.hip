@@ -56,6 +56,7 @@ struct LinearProblem {
     static size_t extra_lds_bytes(const Params &, int, int) { return 0; }
     __device__ static __forceinline__ void prologue(const Params &, Ctx &, int *, int, int, int,
                                                     int, int, int, int, int) {}
+    __device__ static __forceinline__ void next_tile(const Params &, Ctx &) {}
 
     __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &, int arr, int, int m0,
                                                     int row, int r, int r_end) {

@@ -35,6 +35,7 @@
 //                               consecutive k-tiles in increasing order, so Ctx may
 //                               carry what the next tile's loads need.
 //   load_y(p, ctx, arr, i, n0, row, r, r_end)   the same for the column side
+//   next_tile(p, ctx)           runs after all loads of a k-tile were issued
 //   store(p, m, n, acc0, acc1)  final epilogue of one output element
 #pragma once
 #include <hip/hip_runtime.h>
@@ -164,6 +165,7 @@ __global__ __launch_bounds__(WM *WN * 64) void mfma_tile_kernel(typename P::Para
                 tile_pos<YK, BN>(tid + i * NT, row, k);
                 ry[a][i] = P::load_y(p, ctx, a, i, n0, row, r0 + k, r_end);
             }
+        P::next_tile(p, ctx);
     };
     auto commit = [&]() {
 #pragma unroll
