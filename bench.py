@@ -72,6 +72,21 @@ def make_inputs(K, N, B, device):
     )
 
 
+def warm_up(step, warmup, min_seconds=0.3):
+    """`warmup` untimed steps, and more of them until the GPU has worked for
+    `min_seconds`: a handful of sub-millisecond steps right after start-up would
+    otherwise be timed on clocks that are still ramping."""
+    import torch
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < min_seconds:
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
+
+
 def run_workload(name, steps, warmup):
     import torch
     import cutagi_amd.functional as F
@@ -104,9 +119,7 @@ def run_workload(name, steps, warmup):
         F.linear_bwd(t["mu_w"], t["var_w"], t["var_b"], t["mu_a"], t["jcb"], t["delta_mu"],
                      t["delta_var"], out=out_bwd)
 
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
+    warm_up(step, warmup)
 
     # timed region: exactly `steps` steps between two synchronisations
     t0 = time.perf_counter()
@@ -184,9 +197,7 @@ def run_conv(steps, warmup):
         F.conv2d_bwd_dz(mu_w, jcb, dmu, dvar, t["FCzwa_1"], t["Szz_ud"], woho, fo, wihi, fi, k,
                         idx["h"], B)
 
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
+    warm_up(step, warmup)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(steps):
