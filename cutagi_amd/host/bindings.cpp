@@ -196,11 +196,17 @@ PYBIND11_MODULE(cutagi, m) {
                      self.forward(arg1.cast<BaseHiddenStates &>());
                      return;
                  }
-                 auto mu = to_vec(arg1.cast<py::array_t<float, py::array::c_style | py::array::forcecast>>());
-                 std::vector<float> var;
-                 if (!arg2.is_none())
-                     var = to_vec(arg2.cast<py::array_t<float, py::array::c_style | py::array::forcecast>>());
-                 self.forward(mu, var);
+                 // numpy memory goes to the device as it is (no intermediate vector)
+                 using Arr = py::array_t<float, py::array::c_style | py::array::forcecast>;
+                 Arr mu = arg1.cast<Arr>();
+                 if (arg2.is_none()) {
+                     self.forward(mu.data(), nullptr, (size_t)mu.size());
+                 } else {
+                     Arr var = arg2.cast<Arr>();
+                     if (var.size() != mu.size())
+                         throw std::runtime_error("Input mean and variance differ in size");
+                     self.forward(mu.data(), var.data(), (size_t)mu.size());
+                 }
              },
              py::arg("mu_x"), py::arg("var_x") = py::none())
         .def("backward", &Sequential::backward)

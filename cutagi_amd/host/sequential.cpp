@@ -229,14 +229,21 @@ void Sequential::eval() {
 std::string Sequential::get_device() { return this->device; }
 
 void Sequential::forward(const std::vector<float> &mu_x, const std::vector<float> &var_x) {
+    if (!var_x.empty() && var_x.size() != mu_x.size())
+        LOG(LogLevel::ERROR, "Input mean and variance differ in size");
+    this->forward(mu_x.data(), var_x.empty() ? nullptr : var_x.data(), mu_x.size());
+}
+
+void Sequential::forward(const float *mu_x, const float *var_x, size_t n) {
     this->require_device("forward");
     const int in_size = this->layers.front()->get_input_size();
-    if (in_size <= 0 || mu_x.size() % in_size != 0)
+    if (in_size <= 0 || n == 0 || n % in_size != 0)
         LOG(LogLevel::ERROR, "Input size mismatch: " + std::to_string(in_size) + " vs " +
-                                 std::to_string(mu_x.size()));
-    const int batch_size = (int)(mu_x.size() / in_size);
+                                 std::to_string(n));
+    const int batch_size = (int)(n / in_size);
     this->prepare_buffers(batch_size);
-    this->input_z_buffer->set_input_x(mu_x, var_x, batch_size);
+    auto *in = dynamic_cast<HiddenStateHip *>(this->input_z_buffer.get());
+    in->set_input_raw(mu_x, var_x, n, batch_size);
     for (auto &layer : layers) {
         layer->forward(*input_z_buffer, *output_z_buffer, *temp_states);
         std::swap(input_z_buffer, output_z_buffer);

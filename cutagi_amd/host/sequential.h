@@ -64,6 +64,8 @@ class Sequential {
 
     void forward(const std::vector<float> &mu_x,
                  const std::vector<float> &var_x = std::vector<float>());
+    // n values per array; var_x may be null (zero input variance)
+    void forward(const float *mu_x, const float *var_x, size_t n);
     void forward(BaseHiddenStates &input_states);
     void backward();
     void step();

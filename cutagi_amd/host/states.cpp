@@ -4,6 +4,8 @@
 // kernel the layers queued there.
 #include "states.h"
 
+#include "../../include/tagi_hip.h"
+
 #include <algorithm>
 
 #include "logger.h"
@@ -193,8 +195,28 @@ void HiddenStateHip::set_input_x(const std::vector<float> &mu_x, const std::vect
     if (mu_x.size() > this->size)
         LOG(LogLevel::ERROR, "Input of " + std::to_string(mu_x.size()) +
                                  " values exceeds the state buffer of " + std::to_string(size));
-    BaseHiddenStates::set_input_x(mu_x, var_x, block_size);
-    this->chunks_to_device(mu_x.size());
+    this->set_input_raw(mu_x.data(), var_x.size() == mu_x.size() ? var_x.data() : nullptr,
+                        mu_x.size(), block_size);
+}
+// The reference fills host vectors first and then copies all three of them
+// (src/data_struct_cuda.cu:58-80): three host passes and three transfers per
+// batch. Here only what the caller supplied crosses the bus.
+void HiddenStateHip::set_input_raw(const float *mu_x, const float *var_x, size_t n,
+                                   size_t new_block_size) {
+    if (n > this->size)
+        LOG(LogLevel::ERROR, "Input of " + std::to_string(n) +
+                                 " values exceeds the state buffer of " + std::to_string(size));
+    if (n == 0 || new_block_size == 0) LOG(LogLevel::ERROR, "Empty input");
+    this->actual_size = n / new_block_size;
+    this->block_size = new_block_size;
+    HIP_OK(hipSetDevice(device_idx));
+    HIP_OK(hipMemcpy(d_mu_a, mu_x, n * sizeof(float), hipMemcpyHostToDevice));
+    if (var_x != nullptr)
+        HIP_OK(hipMemcpy(d_var_a, var_x, n * sizeof(float), hipMemcpyHostToDevice));
+    else
+        HIP_OK(hipMemsetAsync(d_var_a, 0, n * sizeof(float), nullptr));
+    if (tagi_store_states(nullptr, nullptr, 0, nullptr, nullptr, d_jcb, n, nullptr) != TAGI_OK)
+        LOG(LogLevel::ERROR, "Cannot initialise the input Jacobian");
 }
 void HiddenStateHip::set_size(size_t new_size, size_t new_block_size) {
     if (new_size > this->size) {

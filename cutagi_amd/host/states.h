@@ -109,6 +109,10 @@ class HiddenStateHip : public BaseHiddenStates {
     void deallocate_memory();
     void to_device();
     void chunks_to_device(size_t chunk_size);
+    // Inputs straight from caller memory to the device: mean copied, variance
+    // copied or (var_x == nullptr) cleared on the device, Jacobian set to one by a
+    // kernel. The host mirrors are not touched.
+    void set_input_raw(const float *mu_x, const float *var_x, size_t n, size_t block_size);
     void to_host();
     void to_host(size_t n);  // first n entries only
     void set_size(size_t size, size_t block_size) override;
