@@ -32,6 +32,7 @@ struct ConvParams {
     int woho, fo, wihi, fi, k2, B, nr;
     int M, N, R, splits, r_per_split;
     float *ws0, *ws1;
+    int group_loads;  // 0: never use the sixteen-byte group loads
 };
 
 // All operand loads below are unconditional: an element outside the problem (or
@@ -44,48 +45,121 @@ struct ConvParams {
 // index (channel, tap) moves. The prologue leaves in LDS, for every tap t and
 // local column c, the 0-based offset inside one channel map that tap t of column c
 // reads (tab[t*BN + c], -1 = nothing); Ctx keeps the image base of the columns.
+// Where the four columns of a thread read four CONSECUTIVE elements for every tap
+// (stride-1 geometry, groups that do not straddle an image), one unaligned 16-byte
+// load replaces the four gathers: the prologue also leaves, per tap and group of
+// four columns, (first offset, validity mask) in LDS (qtab), and a flag telling
+// whether every group of the tile has that form. Otherwise the tile gathers
+// element by element.
 struct GatherCtx {
     int img[4];
     int bn;
     const int *tab;
+    const int *qtab;
+    int fast;      // wave-uniform: all groups of this tile are consecutive
+    int ymask[4];  // per column slot: which of the four loaded values are real
+    int xok[2];    // per row slot: the loaded values are real
 };
 
-__device__ __forceinline__ float4 gather_cols(const float *__restrict__ src, const GatherCtx &ctx,
-                                              int row, int r, int r_end, int R, int k2,
-                                              int cstride) {
+__device__ __forceinline__ float4 keep_masked(const float4 &v, int mask) {
+    return make_float4((mask & 1) ? v.x : 0.f, (mask & 2) ? v.y : 0.f, (mask & 4) ? v.z : 0.f,
+                       (mask & 8) ? v.w : 0.f);
+}
+
+typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
+
+// Second half of the prologue: tab[t*bn + c] is complete (a barrier was passed).
+// `pix` = pixels per image of the column index, `src_pix` = elements per channel
+// map of the gathered tensor, B = images. A group whose 16-byte window could leave
+// the tensor (it starts before the first element of image 0 or ends after the
+// last element of image B-1) makes the whole tile gather element by element.
+__device__ __forceinline__ void build_group_table(GatherCtx &ctx, int *tab, int k2, int bn, int n0,
+                                                  int N, int pix, int src_pix, int B, int tid,
+                                                  int nthreads, int allow) {
+    int *qtab = tab + k2 * bn, *flag = qtab + k2 * (bn / 4);
+    if (tid == 0) *flag = (allow && src_pix >= 4) ? 0 : 1;
+    __syncthreads();
+    for (int e = tid; e < k2 * (bn / 4); e += nthreads) {
+        const int t = e / (bn / 4), c = (e - t * (bn / 4)) * 4, n = n0 + c;
+        const int4 off = *reinterpret_cast<const int4 *>(tab + t * bn + c);
+        const int o[4] = {off.x, off.y, off.z, off.w};
+        int mask = 0, base = 0;
+        bool ok = true;
+#pragma unroll
+        for (int j = 3; j >= 0; j--)
+            if (o[j] >= 0) {
+                mask |= 1 << j;
+                base = o[j] - j;
+            }
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if (o[j] >= 0 && o[j] != base + j) ok = false;
+        if (mask != 0) {
+            const int b = n / pix;
+            if (n + 3 >= N || b != (n + 3) / pix) ok = false;
+            if (b == 0 && base < 0) ok = false;
+            if (b == B - 1 && base + 3 > src_pix - 1) ok = false;
+        }
+        qtab[e] = ok ? (((base + 4) << 4) | mask) : 0;
+        if (!ok) *flag = 1;
+    }
+    __syncthreads();
+    ctx.qtab = qtab;
+    ctx.fast = __builtin_amdgcn_readfirstlane(*flag == 0 ? 1 : 0);
+}
+
+// Loads the slot's four values and records in ctx.ymask[slot] which of them are
+// real; nothing here depends on the loaded data (see fix_y).
+__device__ __forceinline__ float4 gather_cols(const float *__restrict__ src, GatherCtx &ctx,
+                                              int fast, int slot, int row, int r, int r_end,
+                                              int R, int k2, int cstride) {
     const int rr = min(r, R - 1);
     const int ch = rr / k2, t = rr - ch * k2;
+    const bool live = r < r_end;
+    if (fast) {
+        const int e = ctx.qtab[t * (ctx.bn >> 2) + (row >> 2)];
+        ctx.ymask[slot] = live ? (e & 15) : 0;
+        // an empty group has first offset 0; either way the window lies inside the
+        // tensor (the prologue has checked the groups at its two ends)
+        const float4u v =
+            *reinterpret_cast<const float4u *>(src + (ctx.img[0] + ch * cstride + (e >> 4) - 4));
+        return make_float4(v.x, v.y, v.z, v.w);
+    }
     const int4 off = *reinterpret_cast<const int4 *>(ctx.tab + t * ctx.bn + row);
     const int o[4] = {off.x, off.y, off.z, off.w};
-    const bool live = r < r_end;
     float c[4];
+    int mask = 0;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const bool ok = live && o[j] >= 0;
-        const float v = src[ok ? ctx.img[j] + ch * cstride + o[j] : 0];
-        c[j] = ok ? v : 0.f;
+        mask |= ok ? (1 << j) : 0;
+        c[j] = src[ok ? ctx.img[j] + ch * cstride + o[j] : 0];
     }
+    ctx.ymask[slot] = mask;
     return make_float4(c[0], c[1], c[2], c[3]);
 }
 
-// Four consecutive reduction elements of row `m` of a [rows][R] matrix.
+// Four consecutive reduction elements of row `m` of a [rows][R] matrix; *mask says
+// which of them are real (the others were read from a clamped address).
 template <bool VEC>
 __device__ __forceinline__ float4 load_rows_kc(const float *__restrict__ base, int R, int m,
-                                               int rows, int r, int r_end) {
+                                               int rows, int r, int r_end, int *mask) {
     const bool row_ok = m < rows;
     const size_t at = (size_t)(row_ok ? m : 0) * R;
     if (VEC) {  // R % 4 == 0, 16-byte aligned base
         const bool ok = row_ok && r < r_end;
-        const float4 v = *reinterpret_cast<const float4 *>(base + at + (ok ? r : 0));
-        return ok ? v : make_float4(0.f, 0.f, 0.f, 0.f);
+        *mask = ok ? 15 : 0;
+        return *reinterpret_cast<const float4 *>(base + at + (ok ? r : 0));
     }
     float c[4];
+    int bits = 0;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const bool ok = row_ok && r + j < r_end;
-        const float v = base[at + (ok ? r + j : 0)];
-        c[j] = ok ? v : 0.f;
+        bits |= ok ? (1 << j) : 0;
+        c[j] = base[at + (ok ? r + j : 0)];
     }
+    *mask = bits;
     return make_float4(c[0], c[1], c[2], c[3]);
 }
 
@@ -97,10 +171,12 @@ struct ConvFwdProblem {
     using Params = ConvParams;
     using Ctx = GatherCtx;
     static constexpr bool XK = true, YK = false, PROLOGUE_WRITES_LDS = true, SPLIT_PER_XCD = false;
+    static constexpr int VARIANTS = 2;  // 1: sixteen-byte loads of consecutive groups
+    __device__ static __forceinline__ bool variant(const Ctx &ctx) { return ctx.fast != 0; }
     static constexpr int NX = 2, NY = 2, FLAVOR = FLAVOR_FWD_W_ROWS;
 
     static size_t extra_lds_bytes(const Params &p, int, int bn) {
-        return (size_t)p.k2 * bn * sizeof(int);
+        return ((size_t)p.k2 * bn + (size_t)p.k2 * (bn / 4) + 4) * sizeof(int);
     }
     __device__ static __forceinline__ void prologue(const Params &p, Ctx &ctx, int *tab, int tid,
                                                     int nthreads, int, int n0, int, int bn, int,
@@ -120,15 +196,23 @@ struct ConvFwdProblem {
             ctx.img[j] = n0 + row + j < p.N ? ((n0 + row + j) / p.woho) * p.fi * p.wihi : 0;
         ctx.bn = bn;
         ctx.tab = tab;
+        build_group_table(ctx, tab, p.k2, bn, n0, p.N, p.woho, p.wihi, p.B, tid, nthreads,
+                          p.group_loads);
     }
     __device__ static __forceinline__ void next_tile(const Params &, Ctx &) {}
-    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &, int arr, int, int m0,
-                                                    int row, int r, int r_end) {
-        return load_rows_kc<VEC>(arr ? p.w1 : p.w0, p.R, m0 + row, p.M, r, r_end);
+    __device__ static __forceinline__ float4 fix_x(const Ctx &ctx, int i, const float4 &v) {
+        return keep_masked(v, ctx.xok[i]);
     }
-    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &ctx, int arr, int,
+    __device__ static __forceinline__ float4 fix_y(const Ctx &ctx, int i, const float4 &v) {
+        return keep_masked(v, ctx.ymask[i]);
+    }
+    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &ctx, int V, int arr, int i,
+                                                    int m0, int row, int r, int r_end) {
+        return load_rows_kc<VEC>(arr ? p.w1 : p.w0, p.R, m0 + row, p.M, r, r_end, &ctx.xok[i]);
+    }
+    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &ctx, int V, int arr, int i,
                                                     int, int row, int r, int r_end) {
-        return gather_cols(arr ? p.a1 : p.a0, ctx, row, r, r_end, p.R, p.k2, p.wihi);
+        return gather_cols(arr ? p.a1 : p.a0, ctx, V, i, row, r, r_end, p.R, p.k2, p.wihi);
     }
     __device__ static __forceinline__ void store(const Params &p, int m, int n, float a0,
                                                  float a1) {
@@ -161,6 +245,7 @@ struct ConvDwProblem {
         int nimg[DW_SLOTS][4];  // image offsets b*fi*wihi of the next visit
     };
     static constexpr bool XK = true, YK = true, PROLOGUE_WRITES_LDS = false, SPLIT_PER_XCD = true;
+    static constexpr int VARIANTS = 1;
     static constexpr int NX = 2, NY = 1, FLAVOR = FLAVOR_DELTA_ROWS;
 
     static size_t extra_lds_bytes(const Params &, int, int) { return 0; }
@@ -195,7 +280,9 @@ struct ConvDwProblem {
         }
     }
     __device__ static __forceinline__ void next_tile(const Params &, Ctx &) {}
-    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &, int arr, int, int m0,
+    __device__ static __forceinline__ float4 fix_x(const Ctx &, int, const float4 &v) { return v; }
+    __device__ static __forceinline__ float4 fix_y(const Ctx &, int, const float4 &v) { return v; }
+    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &, int V, int arr, int, int m0,
                                                     int row, int r, int r_end) {
         const float *__restrict__ d = arr ? p.d1 : p.d0;
         const int m = m0 + row;
@@ -222,7 +309,7 @@ struct ConvDwProblem {
         }
         return make_float4(c[0], c[1], c[2], c[3]);
     }
-    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &ctx, int, int i, int,
+    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &ctx, int V, int, int i, int,
                                                     int, int r, int r_end) {
         float c[4];
 #pragma unroll
@@ -259,8 +346,11 @@ struct ConvDwVecProblem {
         int cb[DW_SLOTS];       // ch*wihi of the column slots, -1: no column
         int tap[DW_SLOTS];
         int nidx[DW_SLOTS][4];  // table entries of the tile being fetched
+        int xok[2];             // masks of the values in flight, applied by fix_x / fix_y
+        int ymask[DW_SLOTS];
     };
     static constexpr bool XK = true, YK = true, PROLOGUE_WRITES_LDS = false, SPLIT_PER_XCD = true;
+    static constexpr int VARIANTS = 1;
     static constexpr int NX = 2, NY = 1, FLAVOR = FLAVOR_DELTA_ROWS;
 
     static size_t extra_lds_bytes(const Params &, int, int) { return 0; }
@@ -305,25 +395,33 @@ struct ConvDwVecProblem {
             ctx.xoff += (p.fo - 1) * p.woho;
         }
     }
-    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &ctx, int arr, int i, int,
+    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &ctx, int V, int arr, int i, int,
                                                     int, int r, int r_end) {
         const bool ok = r < r_end && ctx.xrow[i] >= 0;
         const float *__restrict__ d = arr ? p.d1 : p.d0;
-        const float4 v = *reinterpret_cast<const float4 *>(d + (ok ? ctx.xrow[i] + ctx.xoff : 0));
-        return ok ? v : make_float4(0.f, 0.f, 0.f, 0.f);
+        ctx.xok[i] = ok ? 15 : 0;
+        return *reinterpret_cast<const float4 *>(d + (ok ? ctx.xrow[i] + ctx.xoff : 0));
     }
-    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &ctx, int, int i, int,
+    __device__ static __forceinline__ float4 fix_x(const Ctx &ctx, int i, const float4 &v) {
+        return keep_masked(v, ctx.xok[i]);
+    }
+    __device__ static __forceinline__ float4 fix_y(const Ctx &ctx, int i, const float4 &v) {
+        return keep_masked(v, ctx.ymask[i]);
+    }
+    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &ctx, int V, int, int i, int,
                                                     int, int r, int r_end) {
         const bool live = r < r_end && ctx.cb[i] >= 0;
         const int base = ctx.img + ctx.cb[i] - 1;
         float c[4];
+        int mask = 0;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int a = ctx.nidx[i][j];
             const bool ok = live && a > -1;
-            const float v = p.a0[ok ? base + a : 0];
-            c[j] = ok ? v : 0.f;
+            mask |= ok ? (1 << j) : 0;
+            c[j] = p.a0[ok ? base + a : 0];
         }
+        ctx.ymask[i] = mask;
         // table entries of the next k-tile (always inside the table: the pixel
         // index wraps, and a group of four never straddles its end)
         int o = ctx.o + KT;
@@ -349,10 +447,12 @@ struct ConvDzProblem {
     using Params = ConvParams;
     using Ctx = GatherCtx;
     static constexpr bool XK = true, YK = false, PROLOGUE_WRITES_LDS = true, SPLIT_PER_XCD = false;
+    static constexpr int VARIANTS = 2;  // 1: sixteen-byte loads of consecutive groups
+    __device__ static __forceinline__ bool variant(const Ctx &ctx) { return ctx.fast != 0; }
     static constexpr int NX = 1, NY = 2, FLAVOR = FLAVOR_DELTA_COLS;
 
     static size_t extra_lds_bytes(const Params &p, int, int bn) {
-        return (size_t)p.k2 * bn * sizeof(int);
+        return ((size_t)p.k2 * bn + (size_t)p.k2 * (bn / 4) + 4) * sizeof(int);
     }
     __device__ static __forceinline__ void prologue(const Params &p, Ctx &ctx, int *tab, int tid,
                                                     int nthreads, int, int n0, int, int bn, int,
@@ -373,30 +473,40 @@ struct ConvDzProblem {
             ctx.img[j] = n0 + row + j < p.N ? ((n0 + row + j) / p.wihi) * p.fo * p.woho : 0;
         ctx.bn = bn;
         ctx.tab = tab;
+        build_group_table(ctx, tab, p.k2, bn, n0, p.N, p.wihi, p.woho, p.B, tid, nthreads,
+                          p.group_loads);
     }
     __device__ static __forceinline__ void next_tile(const Params &, Ctx &) {}
-    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &, int, int, int m0,
+    __device__ static __forceinline__ float4 fix_x(const Ctx &ctx, int i, const float4 &v) {
+        return keep_masked(v, ctx.xok[i]);
+    }
+    __device__ static __forceinline__ float4 fix_y(const Ctx &ctx, int i, const float4 &v) {
+        return keep_masked(v, ctx.ymask[i]);
+    }
+    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &ctx, int V, int, int i, int m0,
                                                     int row, int r, int r_end) {
         const int m = m0 + row;
         const bool row_ok = m < p.M;
         const int rr = min(r, p.R - 1);
         int f = rr / p.k2, t = rr - f * p.k2;
         float c[4];
+        int mask = 0;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const bool ok = row_ok && r + j < r_end;
-            const float v = p.w0[ok ? ((size_t)f * p.fi + m) * p.k2 + t : 0];
-            c[j] = ok ? v : 0.f;
+            mask |= ok ? (1 << j) : 0;
+            c[j] = p.w0[ok ? ((size_t)f * p.fi + m) * p.k2 + t : 0];
             if (++t == p.k2) {
                 t = 0;
                 f++;
             }
         }
+        ctx.xok[i] = mask;
         return make_float4(c[0], c[1], c[2], c[3]);
     }
-    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &ctx, int arr, int,
+    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &ctx, int V, int arr, int i,
                                                     int, int row, int r, int r_end) {
-        return gather_cols(arr ? p.d1 : p.d0, ctx, row, r, r_end, p.R, p.k2, p.woho);
+        return gather_cols(arr ? p.d1 : p.d0, ctx, V, i, row, r, r_end, p.R, p.k2, p.woho);
     }
     __device__ static __forceinline__ void store(const Params &p, int m, int n, float a0,
                                                  float a1) {
@@ -494,6 +604,8 @@ hipError_t run_sliced(int tile, int splits, float *ws0, float *ws1, ConvParams &
 }
 }  // namespace
 
+int g_conv2d_group_loads = 1;
+
 hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
                              const float *var_b, const float *mu_a, const float *var_a,
                              const int *aidx, int woho, int fo, int wihi, int fi, int ki, int B,
@@ -505,6 +617,7 @@ hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float 
     p.idx = aidx; p.out0 = mu_z; p.out1 = var_z;
     p.woho = woho; p.fo = fo; p.wihi = wihi; p.fi = fi; p.k2 = ki * ki; p.B = B;
     p.M = fo; p.N = B * woho; p.R = p.k2 * fi;
+    p.group_loads = g_conv2d_group_loads;
     const bool vec = (p.R % 4 == 0) && aligned16(mu_w) && aligned16(var_w);
     if (vec) return run_sliced<ConvFwdProblem<true>>(tile, splits, ws0, ws1, p, stream);
     return run_sliced<ConvFwdProblem<false>>(tile, splits, ws0, ws1, p, stream);
@@ -521,6 +634,7 @@ hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float
     p.out0 = out_dmu; p.out1 = out_dvar;
     p.woho = woho; p.fo = fo; p.wihi = wihi; p.fi = fi; p.k2 = k2; p.B = B; p.nr = nr;
     p.M = fi; p.N = B * wihi; p.R = k2 * fo;
+    p.group_loads = g_conv2d_group_loads;
     return run_sliced<ConvDzProblem>(tile, splits, ws0, ws1, p, stream);
 }
 

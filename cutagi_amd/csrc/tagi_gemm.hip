@@ -53,16 +53,19 @@ struct LinearProblem {
 
     using Ctx = TileNoCtx;
     static constexpr bool PROLOGUE_WRITES_LDS = false, SPLIT_PER_XCD = false;
+    static constexpr int VARIANTS = 1;
     static size_t extra_lds_bytes(const Params &, int, int) { return 0; }
     __device__ static __forceinline__ void prologue(const Params &, Ctx &, int *, int, int, int,
                                                     int, int, int, int, int) {}
     __device__ static __forceinline__ void next_tile(const Params &, Ctx &) {}
+    __device__ static __forceinline__ float4 fix_x(const Ctx &, int, const float4 &v) { return v; }
+    __device__ static __forceinline__ float4 fix_y(const Ctx &, int, const float4 &v) { return v; }
 
-    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &, int arr, int, int m0,
+    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &, int, int arr, int, int m0,
                                                     int row, int r, int r_end) {
         return load4<XK, VEC>(arr ? p.x1 : p.x0, p.ldx, m0 + row, p.M, r, r_end);
     }
-    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &, int arr, int, int n0,
+    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &, int, int arr, int, int n0,
                                                     int row, int r, int r_end) {
         return load4<YK, VEC>(arr ? p.y1 : p.y0, p.ldy, n0 + row, p.N, r, r_end);
     }

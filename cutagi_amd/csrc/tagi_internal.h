@@ -129,6 +129,9 @@ hipError_t launch_add_shortcut(const float *mu_s, const float *var_s, const floa
 
 // Conv2d (implicit GEMM through the index tables)
 void conv2d_plan(int M, int N, int R, int *tile, int *splits);
+// 0 switches the sixteen-byte group loads of the conv2d gathers off (tuning knob).
+extern int g_conv2d_group_loads;
+
 hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
                              const float *var_b, const float *mu_a, const float *var_a,
                              const int *aidx, int woho, int fo, int wihi, int fi, int ki, int B,

@@ -27,15 +27,21 @@
 //   extra_lds_bytes(p, BM, BN)  host: dynamic LDS the prologue wants (index tables)
 //   prologue(p, ctx, extra, tid, nthreads, m0, n0, BM, BN, r_begin, r_end)
 //                               runs once before the first load; a barrier follows
-//   load_x(p, ctx, arr, i, m0, row, r, r_end)
+//   VARIANTS, variant(ctx)      number of loader variants (1 or 2) and, after the
+//                               prologue, which one this workgroup uses (uniform)
+//   load_x(p, ctx, V, arr, i, m0, row, r, r_end)
 //                               four elements of row-side array `arr` for the
 //                               thread's i-th slot: row m0+row, reduction r..r+3
 //                               when XK; rows m0+row..+3 at reduction r otherwise;
 //                               zero outside the problem. Slots are visited for
 //                               consecutive k-tiles in increasing order, so Ctx may
 //                               carry what the next tile's loads need.
-//   load_y(p, ctx, arr, i, n0, row, r, r_end)   the same for the column side
+//   load_y(p, ctx, V, arr, i, n0, row, r, r_end)   the same for the column side
 //   next_tile(p, ctx)           runs after all loads of a k-tile were issued
+//   fix_x(ctx, i, v) / fix_y    applied to slot i's loaded values when they are
+//                               written to LDS, i.e. after the MFMAs of the previous
+//                               k-tile: masking done here instead of right after the
+//                               load keeps the loads in flight during the MFMAs
 //   store(p, m, n, acc0, acc1)  final epilogue of one output element
 #pragma once
 #include <hip/hip_runtime.h>
@@ -100,36 +106,21 @@ __device__ __forceinline__ float4 read_frag(const float *lds, int row, int kk, i
     }
 }
 
-template <class P, int BM, int BN, int WM, int WN>
-__global__ __launch_bounds__(WM *WN * 64) void mfma_tile_kernel(typename P::Params p) {
+// Everything a workgroup does after its prologue, instantiated once per loader
+// variant V (a problem whose prologue chooses between two ways of loading gets two
+// copies of the loop instead of a branch at every load).
+template <class P, int BM, int BN, int WM, int WN, int V>
+__device__ __forceinline__ void mfma_tile_body(const typename P::Params &p, typename P::Ctx &ctx,
+                                               float (*lds_x)[TileGeom<P::XK, BM>::floats],
+                                               float (*lds_y)[TileGeom<P::YK, BN>::floats],
+                                               int m0, int n0, int split, int r_begin,
+                                               int r_end) {
     constexpr bool XK = P::XK, YK = P::YK;
     constexpr int NX = P::NX, NY = P::NY, FL = P::FLAVOR;
     constexpr int NT = WM * WN * 64;
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     constexpr int XS = TileGeom<XK, BM>::stride, YS = TileGeom<YK, BN>::stride;
-    constexpr int XF = TileGeom<XK, BM>::floats, YF = TileGeom<YK, BN>::floats;
     constexpr int LX = BM * KT / 4 / NT, LY = BN * KT / 4 / NT;
-    static_assert(LX >= 1 && LY >= 1, "tile too small for the thread count");
-
-    __shared__ __attribute__((aligned(16))) float lds_x[NX][XF];
-    __shared__ __attribute__((aligned(16))) float lds_y[NY][YF];
-    extern __shared__ __attribute__((aligned(16))) int lds_extra[];
-
-    const int tiles_n = (p.N + BN - 1) / BN;
-    int tile = blockIdx.x, split = blockIdx.y;
-    if (P::SPLIT_PER_XCD && gridDim.y % 8 == 0) {
-        // Workgroups are handed to the 8 XCDs round-robin in launch order. Give all
-        // tiles of one reduction slice to one XCD, so that the operands they share
-        // are fetched into one L2 instead of eight.
-        const int id = blockIdx.y * gridDim.x + blockIdx.x;
-        const int q = id >> 3;
-        tile = q % gridDim.x;
-        split = (q / gridDim.x) * 8 + (id & 7);
-    }
-    const int m0 = (tile / tiles_n) * BM, n0 = (tile % tiles_n) * BN;
-    const int r_begin = split * p.r_per_split;
-    const int r_end = min(p.R, r_begin + p.r_per_split);
-
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wrow = (wave / WN) * (TM * 32), wcol = (wave % WN) * (TN * 32);
 
@@ -145,8 +136,6 @@ __global__ __launch_bounds__(WM *WN * 64) void mfma_tile_kernel(typename P::Para
             }
 
     float4 rx[NX][LX], ry[NY][LY];
-    typename P::Ctx ctx;
-    P::prologue(p, ctx, lds_extra, tid, NT, m0, n0, BM, BN, r_begin, r_end);
 
     auto fetch = [&](int r0) {
 #pragma unroll
@@ -155,7 +144,7 @@ __global__ __launch_bounds__(WM *WN * 64) void mfma_tile_kernel(typename P::Para
             for (int i = 0; i < LX; i++) {
                 int row, k;
                 tile_pos<XK, BM>(tid + i * NT, row, k);
-                rx[a][i] = P::load_x(p, ctx, a, i, m0, row, r0 + k, r_end);
+                rx[a][i] = P::load_x(p, ctx, V, a, i, m0, row, r0 + k, r_end);
             }
 #pragma unroll
         for (int a = 0; a < NY; a++)
@@ -163,7 +152,7 @@ __global__ __launch_bounds__(WM *WN * 64) void mfma_tile_kernel(typename P::Para
             for (int i = 0; i < LY; i++) {
                 int row, k;
                 tile_pos<YK, BN>(tid + i * NT, row, k);
-                ry[a][i] = P::load_y(p, ctx, a, i, n0, row, r0 + k, r_end);
+                ry[a][i] = P::load_y(p, ctx, V, a, i, n0, row, r0 + k, r_end);
             }
         P::next_tile(p, ctx);
     };
@@ -174,7 +163,8 @@ __global__ __launch_bounds__(WM *WN * 64) void mfma_tile_kernel(typename P::Para
             for (int i = 0; i < LX; i++) {
                 int row, k;
                 tile_pos<XK, BM>(tid + i * NT, row, k);
-                *reinterpret_cast<float4 *>(&lds_x[a][XK ? row * XS + k : k * XS + row]) = rx[a][i];
+                *reinterpret_cast<float4 *>(&lds_x[a][XK ? row * XS + k : k * XS + row]) =
+                    P::fix_x(ctx, i, rx[a][i]);
             }
 #pragma unroll
         for (int a = 0; a < NY; a++)
@@ -182,11 +172,11 @@ __global__ __launch_bounds__(WM *WN * 64) void mfma_tile_kernel(typename P::Para
             for (int i = 0; i < LY; i++) {
                 int row, k;
                 tile_pos<YK, BN>(tid + i * NT, row, k);
-                *reinterpret_cast<float4 *>(&lds_y[a][YK ? row * YS + k : k * YS + row]) = ry[a][i];
+                *reinterpret_cast<float4 *>(&lds_y[a][YK ? row * YS + k : k * YS + row]) =
+                    P::fix_y(ctx, i, ry[a][i]);
             }
     };
 
-    if (P::PROLOGUE_WRITES_LDS) __syncthreads();
     if (r_begin < r_end) {
         fetch(r_begin);
         commit();
@@ -282,6 +272,52 @@ __global__ __launch_bounds__(WM *WN * 64) void mfma_tile_kernel(typename P::Para
             }
         }
 }
+
+
+template <class P, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM *WN * 64) void mfma_tile_kernel(typename P::Params p) {
+    constexpr bool XK = P::XK, YK = P::YK;
+    constexpr int NX = P::NX, NY = P::NY, FL = P::FLAVOR;
+    constexpr int NT = WM * WN * 64;
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int XS = TileGeom<XK, BM>::stride, YS = TileGeom<YK, BN>::stride;
+    constexpr int XF = TileGeom<XK, BM>::floats, YF = TileGeom<YK, BN>::floats;
+    constexpr int LX = BM * KT / 4 / NT, LY = BN * KT / 4 / NT;
+    static_assert(LX >= 1 && LY >= 1, "tile too small for the thread count");
+
+    __shared__ __attribute__((aligned(16))) float lds_x[NX][XF];
+    __shared__ __attribute__((aligned(16))) float lds_y[NY][YF];
+    extern __shared__ __attribute__((aligned(16))) int lds_extra[];
+
+    const int tiles_n = (p.N + BN - 1) / BN;
+    int tile = blockIdx.x, split = blockIdx.y;
+    if (P::SPLIT_PER_XCD && gridDim.y % 8 == 0) {
+        // Workgroups are handed to the 8 XCDs round-robin in launch order. Give all
+        // tiles of one reduction slice to one XCD, so that the operands they share
+        // are fetched into one L2 instead of eight.
+        const int id = blockIdx.y * gridDim.x + blockIdx.x;
+        const int q = id >> 3;
+        tile = q % gridDim.x;
+        split = (q / gridDim.x) * 8 + (id & 7);
+    }
+    const int m0 = (tile / tiles_n) * BM, n0 = (tile % tiles_n) * BN;
+    const int r_begin = split * p.r_per_split;
+    const int r_end = min(p.R, r_begin + p.r_per_split);
+
+    typename P::Ctx ctx;
+    P::prologue(p, ctx, lds_extra, threadIdx.x, NT, m0, n0, BM, BN, r_begin, r_end);
+    if (P::PROLOGUE_WRITES_LDS) __syncthreads();
+    if constexpr (P::VARIANTS > 1) {
+        if (P::variant(ctx)) {
+            mfma_tile_body<P, BM, BN, WM, WN, 1>(p, ctx, lds_x, lds_y, m0, n0, split, r_begin,
+                                                 r_end);
+            return;
+        }
+    }
+    mfma_tile_body<P, BM, BN, WM, WN, 0>(p, ctx, lds_x, lds_y, m0, n0, split, r_begin, r_end);
+}
+
+
 
 // Folds the partial sums of a sliced reduction (ws0/ws1 [split][M][N]) in slice
 // order and hands every output element to the problem's epilogue.
