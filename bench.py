@@ -45,7 +45,7 @@ MEASURED_TRAFFIC_BYTES = {
     ("gemm", "bwd_dz"): 168.0e6,   # algorithmic 88.1e6
     ("skinny", "fwd"): 562.5e6,    # algorithmic 536.9e6
     ("skinny", "bwd_dz"): 286.5e6, # algorithmic 268.4e6
-    ("skinny", "bwd_dw"): 818.4e6, # algorithmic 805.3e6
+    ("skinny", "bwd_dw"): 820.7e6, # algorithmic 805.3e6
 }
 
 # Conv2d 3x3, stride 1, pad 1, 64 -> 64 channels on 32x32 maps, batch 128, no bias
@@ -309,6 +309,8 @@ def main():
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="gemm")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--extra", default="linear,conv,resnet18",
+                    help="comma-separated secondary workloads to run (linear, conv, resnet18)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain 1 GiB device copy (reference for byte counters)")
     args = ap.parse_args()
@@ -345,17 +347,22 @@ def main():
         "phase_ms": {k: round(v, 5) for k, v in main_res["phase_ms"].items()},
         "roofline": main_res["roofline"],
     }
-    if not args.no_extra:
+    extras = [] if args.no_extra else [e for e in args.extra.split(",") if e]
+    if extras:
+        line["extra"] = {}
+    if "linear" in extras:
         other = "skinny" if args.workload == "gemm" else "gemm"
         r = run_workload(other, args.steps, args.warmup)
-        line["extra"] = {other: {
+        line["extra"][other] = {
             "workload": "TAGI Linear %d->%d, batch %d" % (r["K"], r["N"], r["B"]),
             "value": round(r["value"], 3), "unit": r["unit"],
             "frac_of_peak": round(r["frac_of_peak"], 4),
             "ms_per_step": round(r["ms_per_step"], 5),
             "phase_ms": {k: round(v, 5) for k, v in r["phase_ms"].items()},
-            "roofline": r["roofline"]}}
+            "roofline": r["roofline"]}
+    if "conv" in extras:
         line["extra"]["conv"] = run_conv(max(5, args.steps // 2), args.warmup)
+    if "resnet18" in extras:
         line["extra"]["resnet18"] = run_resnet(max(5, args.steps // 5), 3)
     if args.calibrate:
         calibrate_copy()

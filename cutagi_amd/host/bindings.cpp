@@ -225,6 +225,8 @@ PYBIND11_MODULE(cutagi, m) {
         .def("get_neg_var_w_counter", &Sequential::get_neg_var_w_counter)
         .def("save", &Sequential::save)
         .def("load", &Sequential::load)
+        .def("save_csv", &Sequential::save_csv)
+        .def("load_csv", &Sequential::load_csv)
         .def("params_from", &Sequential::params_from)
         .def("parameters", &Sequential::parameters)
         .def("state_dict", &Sequential::state_dict)

@@ -21,6 +21,10 @@ class MixtureReLU : public BaseLayer {
     std::string get_layer_info() const override { return "MixtureReLU()"; }
     std::string get_layer_name() const override { return "MixtureReLU"; }
     LayerType get_layer_type() const override { return LayerType::Activation; }
+    // Activations own no section of a checkpoint file (reference:
+    // include/activation.h:142-144).
+    void save(std::ofstream &) override {}
+    void load(std::ifstream &) override {}
     std::unique_ptr<BaseLayer> to_cuda(int device_idx = 0) override;
 };
 
@@ -30,6 +34,10 @@ class MixtureReLUHip : public BaseLayer {
     std::string get_layer_info() const override { return "MixtureReLU()"; }
     std::string get_layer_name() const override { return "MixtureReLUCuda"; }
     LayerType get_layer_type() const override { return LayerType::Activation; }
+    // Activations own no section of a checkpoint file (reference:
+    // include/activation.h:142-144).
+    void save(std::ofstream &) override {}
+    void load(std::ifstream &) override {}
     void forward(BaseHiddenStates &input_states, BaseHiddenStates &output_states,
                  BaseTempStates &temp_states) override;
     void backward(BaseDeltaStates &, BaseDeltaStates &, BaseTempStates &, bool = true) override {}

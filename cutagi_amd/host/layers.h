@@ -240,6 +240,10 @@ class ReLU : public BaseLayer {
     std::string get_layer_info() const override { return "ReLU()"; }
     std::string get_layer_name() const override { return "ReLU"; }
     LayerType get_layer_type() const override { return LayerType::Activation; }
+    // Activations own no section of a checkpoint file (reference:
+    // include/activation.h:142-144).
+    void save(std::ofstream &) override {}
+    void load(std::ifstream &) override {}
     std::unique_ptr<BaseLayer> to_cuda(int device_idx = 0) override;
 };
 
@@ -249,6 +253,10 @@ class ReLUHip : public BaseLayer {
     std::string get_layer_info() const override { return "Relu()"; }
     std::string get_layer_name() const override { return "ReLUCuda"; }
     LayerType get_layer_type() const override { return LayerType::Activation; }
+    // Activations own no section of a checkpoint file (reference:
+    // include/activation.h:142-144).
+    void save(std::ofstream &) override {}
+    void load(std::ifstream &) override {}
     void forward(BaseHiddenStates &input_states, BaseHiddenStates &output_states,
                  BaseTempStates &temp_states) override;
     // Nothing to propagate: the Jacobian rides in the hidden state and is applied

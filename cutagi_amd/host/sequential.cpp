@@ -1,6 +1,8 @@
 // Sequential and OutputUpdater: see sequential.h.
 #include "sequential.h"
 
+#include <sys/stat.h>
+
 #include <fstream>
 #include <sstream>
 
@@ -297,7 +299,18 @@ void Sequential::preinit_layer() {
         if (layer) layer->preinit_layer();
 }
 
+// Creates the directory part of `filename` when it does not exist yet (one level,
+// as the reference's create_directory does, src/common.cpp:57-73).
+static void make_parent_directory(const std::string &filename) {
+    const size_t cut = filename.find_last_of("\\/");
+    if (cut == std::string::npos || cut == 0) return;
+    const std::string dir = filename.substr(0, cut);
+    struct stat st;
+    if (stat(dir.c_str(), &st) == -1) mkdir(dir.c_str(), 0777);
+}
+
 void Sequential::save(const std::string &filename) {
+    make_parent_directory(filename);
     std::ofstream file(filename, std::ios::binary);
     if (!file.is_open()) LOG(LogLevel::ERROR, "Failed to open file for saving");
     for (auto &layer : layers) layer->save(file);
@@ -308,6 +321,80 @@ void Sequential::load(const std::string &filename) {
     std::ifstream file(filename, std::ios::binary);
     if (!file.is_open()) LOG(LogLevel::ERROR, "Failed to open file for loading");
     for (auto &layer : layers) layer->load(file);
+}
+
+// Text checkpoint (reference: Sequential::save_csv / load_csv,
+// src/sequential.cpp:612-709 over write_csv / read_csv, include/common.h:135-207):
+// four files `<filename>_1_mw.csv`, `_2_Sw.csv`, `_3_mb.csv`, `_4_Sb.csv`, each the
+// concatenation over the top-level layers of that parameter vector, one value
+// per line in the stream's default float format (six significant digits). As in
+// the reference only the vectors the top-level layers hold themselves are
+// written: the members of a LayerBlock / ResNetBlock keep theirs and are skipped.
+static void write_csv_column(const std::string &path, const std::vector<float> &v) {
+    std::ofstream file(path);
+    if (!file.is_open()) LOG(LogLevel::ERROR, "Failed to open file for saving: " + path);
+    for (float x : v) file << x << "\n";
+}
+
+static void read_csv_column(const std::string &path, std::vector<float> &v) {
+    std::ifstream file(path);
+    if (!file.is_open()) LOG(LogLevel::ERROR, "Could not open the file: " + path);
+    size_t count = 0;
+    std::string line, cell;
+    while (count < v.size() && std::getline(file, line)) {
+        std::stringstream row(line);
+        while (count < v.size() && std::getline(row, cell, ',')) {
+            std::stringstream value(cell);
+            float d = 0.0f;
+            value >> d;
+            v[count++] = d;
+        }
+    }
+    if (count != v.size())
+        LOG(LogLevel::ERROR, "There is missing data in " + path + ": expected " +
+                                 std::to_string(v.size()) + " values, found " +
+                                 std::to_string(count));
+}
+
+void Sequential::save_csv(const std::string &filename) {
+    make_parent_directory(filename);
+    std::vector<float> mu_w, var_w, mu_b, var_b;
+    for (auto &layer : layers) {
+        layer->params_to_host();
+        mu_w.insert(mu_w.end(), layer->mu_w.begin(), layer->mu_w.end());
+        var_w.insert(var_w.end(), layer->var_w.begin(), layer->var_w.end());
+        mu_b.insert(mu_b.end(), layer->mu_b.begin(), layer->mu_b.end());
+        var_b.insert(var_b.end(), layer->var_b.begin(), layer->var_b.end());
+    }
+    write_csv_column(filename + "_1_mw.csv", mu_w);
+    write_csv_column(filename + "_2_Sw.csv", var_w);
+    write_csv_column(filename + "_3_mb.csv", mu_b);
+    write_csv_column(filename + "_4_Sb.csv", var_b);
+}
+
+void Sequential::load_csv(const std::string &filename) {
+    size_t num_weights = 0, num_biases = 0;
+    for (auto &layer : layers) {
+        num_weights += layer->mu_w.size();
+        num_biases += layer->mu_b.size();
+    }
+    std::vector<float> mu_w(num_weights), var_w(num_weights), mu_b(num_biases), var_b(num_biases);
+    read_csv_column(filename + "_1_mw.csv", mu_w);
+    read_csv_column(filename + "_2_Sw.csv", var_w);
+    read_csv_column(filename + "_3_mb.csv", mu_b);
+    read_csv_column(filename + "_4_Sb.csv", var_b);
+    size_t w0 = 0, b0 = 0;
+    for (auto &layer : layers) {
+        const size_t nw = layer->mu_w.size(), nb = layer->mu_b.size();
+        std::copy(mu_w.begin() + w0, mu_w.begin() + w0 + nw, layer->mu_w.begin());
+        std::copy(var_w.begin() + w0, var_w.begin() + w0 + nw, layer->var_w.begin());
+        std::copy(mu_b.begin() + b0, mu_b.begin() + b0 + nb, layer->mu_b.begin());
+        std::copy(var_b.begin() + b0, var_b.begin() + b0 + nb, layer->var_b.begin());
+        w0 += nw;
+        b0 += nb;
+        if (auto *d = dynamic_cast<BaseLayerHip *>(layer.get()))
+            if (d->d_mu_w != nullptr) d->params_to_device();
+    }
 }
 
 std::vector<ParameterTuple> Sequential::parameters() {

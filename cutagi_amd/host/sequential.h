@@ -74,6 +74,8 @@ class Sequential {
     void preinit_layer();
     void save(const std::string &filename);
     void load(const std::string &filename);
+    void save_csv(const std::string &filename);
+    void load_csv(const std::string &filename);
     std::vector<ParameterTuple> parameters();
     ParameterMap state_dict();
     void load_state_dict(const ParameterMap &state_dict);

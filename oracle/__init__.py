@@ -299,6 +299,35 @@ class Oracle:
         self._fn("class_to_obs")(n_classes, _fp(obs), _ip(idx), ctypes.byref(a), ctypes.byref(b))
         return obs.reshape(n_classes, n_obs), idx.reshape(n_classes, n_obs), a.value, b.value
 
+    # ---- checkpoint files (reference build only) -----------------------------------
+    def checkpoint_save(self, model, path):
+        """Writes the reference's binary checkpoint of zoo model `model` with the
+        parameter pattern value(leaf, array, i) = leaf+1 + 0.1*(array+1) + 1e-4*i."""
+        fn = self._fn("checkpoint_save")
+        fn.restype = ctypes.c_int
+        return fn(int(model), os.fsencode(path))
+
+    def checkpoint_load(self, model, path, capacity=1 << 16):
+        """Loads a binary checkpoint with the reference's loader; returns all
+        parameters leaf by leaf in saving order, or None if the loader threw."""
+        fn = self._fn("checkpoint_load")
+        fn.restype = ctypes.c_int
+        out = np.zeros(capacity, np.float32)
+        n = fn(int(model), os.fsencode(path), _fp(out), capacity)
+        return None if n < 0 else out[:n].copy()
+
+    def write_csv(self, path, data):
+        fn = self._fn("write_csv")
+        fn.restype = ctypes.c_int
+        data = f32(data)
+        return fn(os.fsencode(path), _fp(data), data.size)
+
+    def read_csv(self, path, n):
+        fn = self._fn("read_csv")
+        fn.restype = ctypes.c_int
+        out = np.zeros(n, np.float32)
+        return out if fn(os.fsencode(path), _fp(out), n) == 0 else None
+
 
 def load():
     path = os.path.join(_HERE, "liboracle.so")

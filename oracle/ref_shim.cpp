@@ -6,6 +6,8 @@
 // as tagi_oracle.h with a `ref_` prefix. No reference source is copied here:
 // this file only includes the reference headers and calls into them.
 #include <cstring>
+#include <fstream>
+#include <memory>
 #include <stdexcept>
 #include <vector>
 
@@ -15,7 +17,10 @@
 #include "conv2d_layer.h"
 #include "cost.h"
 #include "linear_layer.h"
+#include "batchnorm_layer.h"
+#include "layer_block.h"
 #include "pooling_layer.h"
+#include "resnet_block.h"
 
 // Free functions the reference defines in its .cpp files without declaring them
 // in a header (src/batchnorm_layer.cpp:15-354,457-775, src/resnet_block.cpp:8-31,
@@ -516,6 +521,142 @@ void ref_class_to_obs(int n_classes, float *obs, int *idx, int *n_obs, int *len)
     std::memcpy(idx, hs.idx.data(), hs.idx.size() * sizeof(int));
     *n_obs = (int)hs.n_obs;
     *len = (int)hs.len;
+}
+
+// ---- checkpoint files ---------------------------------------------------------
+// Two small models built from the reference's own layer classes, sized the way
+// Sequential::compute_input_output_size does it (src/sequential.cpp:144-164), to
+// write and read the reference's binary checkpoint (BaseLayer::save/load,
+// src/base_layer.cpp:230-297; BatchNorm2d adds its running averages,
+// src/batchnorm_layer.cpp:1143-1230; blocks save their members in order,
+// src/layer_block.cpp, src/resnet_block.cpp:299-317).
+//   model 0: Linear(13,7) ReLU Linear(7,3)
+//   model 1: Conv2d(3,4,k3,p1) BatchNorm2d(4) MixtureReLU
+//            ResNetBlock(main: Conv2d(4,8,k3,s2,p1 type 2) ReLU BatchNorm2d(8);
+//                        shortcut: Conv2d(4,8,k2,s2)) AvgPool2d(4) Linear(8,5)
+}  // extern "C"
+
+namespace {
+struct Zoo {
+    std::vector<std::shared_ptr<BaseLayer>> top;
+    std::vector<BaseLayer *> leaves;  // in the order their parameters are saved
+};
+
+Zoo make_zoo(int model) {
+    Zoo z;
+    auto leaf = [&](std::shared_ptr<BaseLayer> l) {
+        z.leaves.push_back(l.get());
+        return l;
+    };
+    if (model == 0) {
+        z.top.push_back(leaf(std::make_shared<Linear>(13, 7)));
+        z.top.push_back(leaf(std::make_shared<ReLU>()));
+        z.top.push_back(leaf(std::make_shared<Linear>(7, 3)));
+    } else {
+        z.top.push_back(leaf(std::make_shared<Conv2d>(3, 4, 3, false, 1, 1, 1, 8, 8)));
+        z.top.push_back(leaf(std::make_shared<BatchNorm2d>(4)));
+        z.top.push_back(leaf(std::make_shared<MixtureReLU>()));
+        auto main = std::make_shared<LayerBlock>();
+        main->add_layer(leaf(std::make_shared<Conv2d>(4, 8, 3, false, 2, 1, 2)));
+        main->add_layer(leaf(std::make_shared<ReLU>()));
+        main->add_layer(leaf(std::make_shared<BatchNorm2d>(8)));
+        auto shortcut = std::make_shared<LayerBlock>();
+        shortcut->add_layer(leaf(std::make_shared<Conv2d>(4, 8, 2, false, 2)));
+        z.top.push_back(std::make_shared<ResNetBlock>(main, shortcut));
+        z.top.push_back(leaf(std::make_shared<AvgPool2d>(4)));
+        z.top.push_back(leaf(std::make_shared<Linear>(8, 5)));
+    }
+    int w = z.top.front()->in_width, h = z.top.front()->in_height,
+        d = z.top.front()->in_channels;
+    for (auto &l : z.top) {
+        InitArgs args(w, h, d);
+        l->compute_input_output_size(args);
+        w = l->out_width;
+        h = l->out_height;
+        d = l->out_channels;
+    }
+    for (auto &l : z.top) l->preinit_layer();
+    return z;
+}
+
+std::vector<std::vector<float> *> arrays_of(BaseLayer *l) {
+    std::vector<std::vector<float> *> a = {&l->mu_w, &l->var_w, &l->mu_b, &l->var_b};
+    if (auto *bn = dynamic_cast<BatchNorm2d *>(l)) {
+        a.push_back(&bn->mu_ra);
+        a.push_back(&bn->var_ra);
+    }
+    return a;
+}
+}  // namespace
+
+extern "C" {
+
+// Fills every parameter of the model with value(leaf, array, i) =
+// (leaf + 1) + 0.1 * (array + 1) + 1e-4 * i and saves it. Returns the number of
+// floats written, -1 on failure.
+int ref_checkpoint_save(int model, const char *path) {
+    try {
+        Zoo z = make_zoo(model);
+        int total = 0;
+        for (size_t L = 0; L < z.leaves.size(); L++) {
+            auto arrs = arrays_of(z.leaves[L]);
+            for (size_t a = 0; a < arrs.size(); a++)
+                for (size_t i = 0; i < arrs[a]->size(); i++, total++)
+                    (*arrs[a])[i] = (float)(L + 1) + 0.1f * (float)(a + 1) + 1e-4f * (float)i;
+        }
+        std::ofstream file(path, std::ios::binary);
+        if (!file.is_open()) return -1;
+        for (auto &l : z.top) l->save(file);
+        return total;
+    } catch (const std::exception &) {
+        return -1;
+    }
+}
+
+// Loads a checkpoint into a freshly built model and writes its parameters, leaf
+// by leaf in saving order, to out. Returns the number of floats, -1 on failure
+// (a layer name that does not match throws in the reference).
+int ref_checkpoint_load(int model, const char *path, float *out, int capacity) {
+    try {
+        Zoo z = make_zoo(model);
+        std::ifstream file(path, std::ios::binary);
+        if (!file.is_open()) return -1;
+        for (auto &l : z.top) l->load(file);
+        int n = 0;
+        for (auto *l : z.leaves)
+            for (auto *arr : arrays_of(l))
+                for (float v : *arr) {
+                    if (n >= capacity) return -1;
+                    out[n++] = v;
+                }
+        return n;
+    } catch (const std::exception &) {
+        return -1;
+    }
+}
+
+// The text format of Sequential::save_csv / load_csv (src/sequential.cpp:612-709):
+// one value per line through write_csv / read_csv (include/common.h:135-207).
+int ref_write_csv(const char *path, const float *data, int n) {
+    try {
+        std::vector<float> v(data, data + n);
+        write_csv(std::string(path), v);
+        return 0;
+    } catch (const std::exception &) {
+        return -1;
+    }
+}
+
+int ref_read_csv(const char *path, float *out, int n) {
+    try {
+        std::vector<float> v(n);
+        std::string name(path);
+        read_csv(name, v, 1, false);
+        std::memcpy(out, v.data(), n * sizeof(float));
+        return 0;
+    } catch (const std::exception &) {
+        return -1;
+    }
 }
 
 }  // extern "C"
