@@ -229,8 +229,9 @@ def run_resnet(steps, warmup, B=128):
     rng = np.random.default_rng(0)
     x = rng.normal(0, 1, (B, 3 * 32 * 32)).astype(np.float32)
     labels = rng.integers(0, 10, B)
-    y, sel = obs[labels].ravel().tolist(), idx[labels].ravel().tolist()
-    var_y = [1.0] * (B * n_obs)
+    y = np.ascontiguousarray(obs[labels].ravel(), np.float32)
+    sel = np.ascontiguousarray(idx[labels].ravel(), np.int32)
+    var_y = np.ones(B * n_obs, np.float32)
 
     def step():
         net.forward(x)

@@ -15,6 +15,9 @@ namespace py = pybind11;
 using namespace tagi_host;
 
 namespace {
+using FloatArray = py::array_t<float, py::array::c_style>;
+using IntArray = py::array_t<int, py::array::c_style>;
+
 std::vector<float> to_vec(const py::array_t<float, py::array::c_style | py::array::forcecast> &a) {
     std::vector<float> v(a.size());
     if (a.size()) std::memcpy(v.data(), a.data(), a.size() * sizeof(float));
@@ -156,8 +159,31 @@ PYBIND11_MODULE(cutagi, m) {
 
     py::class_<OutputUpdater, std::shared_ptr<OutputUpdater>>(m, "OutputUpdater")
         .def(py::init<const std::string>())
+        // float32 / int32 numpy arrays are read in place; anything else (lists, as in
+        // the reference's binding, or arrays of another type) goes through std::vector
+        .def("update",
+             [](OutputUpdater &self, BaseHiddenStates &out, const FloatArray &mu,
+                const FloatArray &var, BaseDeltaStates &delta) {
+                 if (mu.size() != var.size())
+                     throw std::runtime_error("Observation size does not fit the output buffers");
+                 self.update_raw(out, mu.data(), var.data(), (size_t)mu.size(), delta);
+             },
+             py::arg("output_states"), py::arg("mu_obs").noconvert(),
+             py::arg("var_obs").noconvert(), py::arg("delta_states"))
         .def("update", &OutputUpdater::update, py::arg("output_states"), py::arg("mu_obs"),
              py::arg("var_obs"), py::arg("delta_states"))
+        .def("update_using_indices",
+             [](OutputUpdater &self, BaseHiddenStates &out, const FloatArray &mu,
+                const FloatArray &var, const IntArray &idx, BaseDeltaStates &delta) {
+                 if (mu.size() != var.size() || mu.size() != idx.size())
+                     throw std::runtime_error("Observations, variances and indices must have "
+                                              "one size, a multiple of the batch size");
+                 self.update_using_indices_raw(out, mu.data(), var.data(), idx.data(),
+                                               (size_t)mu.size(), delta);
+             },
+             py::arg("output_states"), py::arg("mu_obs").noconvert(),
+             py::arg("var_obs").noconvert(), py::arg("selected_idx").noconvert(),
+             py::arg("delta_states"))
         .def("update_using_indices", &OutputUpdater::update_using_indices,
              py::arg("output_states"), py::arg("mu_obs"), py::arg("var_obs"),
              py::arg("selected_idx"), py::arg("delta_states"))

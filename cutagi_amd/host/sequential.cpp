@@ -45,18 +45,24 @@ ObservationHip *OutputUpdater::device_obs() {
 
 void OutputUpdater::update(BaseHiddenStates &output_states, std::vector<float> &mu_obs,
                            std::vector<float> &var_obs, BaseDeltaStates &delta_states) {
+    if (mu_obs.size() != var_obs.size())
+        LOG(LogLevel::ERROR, "Observation size does not fit the output buffers");
+    this->update_raw(output_states, mu_obs.data(), var_obs.data(), mu_obs.size(), delta_states);
+}
+
+void OutputUpdater::update_raw(BaseHiddenStates &output_states, const float *mu_obs,
+                               const float *var_obs, size_t n, BaseDeltaStates &delta_states) {
     ObservationHip *o = this->device_obs();
     auto *out = dynamic_cast<HiddenStateHip *>(&output_states);
     auto *delta = dynamic_cast<DeltaStateHip *>(&delta_states);
     if (out == nullptr || delta == nullptr)
         LOG(LogLevel::ERROR, "OutputUpdater needs device state buffers");
-    if (mu_obs.size() != var_obs.size() || mu_obs.size() > out->size || mu_obs.size() > delta->size)
+    if (n > out->size || n > delta->size)
         LOG(LogLevel::ERROR, "Observation size does not fit the output buffers");
-    o->set_obs(mu_obs, var_obs);
     o->block_size = output_states.block_size;
-    o->size = mu_obs.size();
-    o->actual_size = mu_obs.size() / output_states.block_size;
-    o->to_device();
+    o->size = n;
+    o->actual_size = output_states.block_size ? n / output_states.block_size : 0;
+    o->upload(mu_obs, var_obs, n, nullptr, 0);
     delta->reset_zeros();
     TAGI_OK_OR_THROW(tagi_out_update_dense(out->d_mu_a, out->d_var_a, out->d_jcb, o->d_mu_obs,
                                            o->d_var_obs, (int)o->size, delta->d_delta_mu,
@@ -67,27 +73,35 @@ void OutputUpdater::update_using_indices(BaseHiddenStates &output_states,
                                          std::vector<float> &mu_obs, std::vector<float> &var_obs,
                                          std::vector<int> &selected_idx,
                                          BaseDeltaStates &delta_states) {
+    if (mu_obs.size() != var_obs.size() || selected_idx.size() != mu_obs.size())
+        LOG(LogLevel::ERROR, "Observations, variances and indices must have one size, a multiple "
+                             "of the batch size");
+    this->update_using_indices_raw(output_states, mu_obs.data(), var_obs.data(),
+                                   selected_idx.data(), mu_obs.size(), delta_states);
+}
+
+void OutputUpdater::update_using_indices_raw(BaseHiddenStates &output_states,
+                                             const float *mu_obs, const float *var_obs,
+                                             const int *selected_idx, size_t n,
+                                             BaseDeltaStates &delta_states) {
     ObservationHip *o = this->device_obs();
     auto *out = dynamic_cast<HiddenStateHip *>(&output_states);
     auto *delta = dynamic_cast<DeltaStateHip *>(&delta_states);
     if (out == nullptr || delta == nullptr)
         LOG(LogLevel::ERROR, "OutputUpdater needs device state buffers");
-    if (mu_obs.size() != var_obs.size() || selected_idx.size() != mu_obs.size() ||
-        output_states.block_size == 0 || mu_obs.size() % output_states.block_size != 0)
+    if (output_states.block_size == 0 || n % output_states.block_size != 0)
         LOG(LogLevel::ERROR, "Observations, variances and indices must have one size, a multiple "
                              "of the batch size");
     const int n_obs = (int)output_states.actual_size;
-    for (int idx : selected_idx)
-        if (idx < 1 || idx > n_obs)
-            LOG(LogLevel::ERROR, "Selected index " + std::to_string(idx) + " outside 1.." +
-                                     std::to_string(n_obs));
-    o->set_obs(mu_obs, var_obs);
-    o->set_selected_idx(selected_idx);
+    for (size_t i = 0; i < n; i++)
+        if (selected_idx[i] < 1 || selected_idx[i] > n_obs)
+            LOG(LogLevel::ERROR, "Selected index " + std::to_string(selected_idx[i]) +
+                                     " outside 1.." + std::to_string(n_obs));
     o->block_size = output_states.block_size;
-    o->size = mu_obs.size();
-    o->actual_size = mu_obs.size() / output_states.block_size;
-    o->idx_size = selected_idx.size();
-    o->to_device();
+    o->size = n;
+    o->actual_size = n / output_states.block_size;
+    o->idx_size = n;
+    o->upload(mu_obs, var_obs, n, selected_idx, n);
     const int n_enc = (int)(o->idx_size / output_states.block_size);
     delta->reset_zeros();
     TAGI_OK_OR_THROW(tagi_out_update_indexed(out->d_mu_a, out->d_var_a, out->d_jcb, o->d_mu_obs,

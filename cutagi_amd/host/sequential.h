@@ -27,6 +27,13 @@ class OutputUpdater {
     void update_using_indices(BaseHiddenStates &output_states, std::vector<float> &mu_obs,
                               std::vector<float> &var_obs, std::vector<int> &selected_idx,
                               BaseDeltaStates &delta_states);
+    // The same two updates with the observations read straight from caller memory
+    // (what the Python binding passes for float32 / int32 numpy arrays).
+    void update_raw(BaseHiddenStates &output_states, const float *mu_obs, const float *var_obs,
+                    size_t n, BaseDeltaStates &delta_states);
+    void update_using_indices_raw(BaseHiddenStates &output_states, const float *mu_obs,
+                                  const float *var_obs, const int *selected_idx, size_t n,
+                                  BaseDeltaStates &delta_states);
 
    private:
     ObservationHip *device_obs();

@@ -359,8 +359,7 @@ ObservationHip::~ObservationHip() {
     dev_free(d_var_obs);
     if (d_selected_idx != nullptr) (void)hipFree(d_selected_idx);
 }
-void ObservationHip::to_device() {
-    const size_t n = mu_obs.size(), ni = selected_idx.size();
+void ObservationHip::reserve(size_t n, size_t ni) {
     if (n > cap_obs) {
         HIP_OK(hipDeviceSynchronize());
         dev_free(d_mu_obs);
@@ -375,11 +374,17 @@ void ObservationHip::to_device() {
         HIP_OK(hipMalloc(reinterpret_cast<void **>(&d_selected_idx), ni * sizeof(int)));
         cap_idx = ni;
     }
-    h2d(d_mu_obs, mu_obs.data(), n);
-    h2d(d_var_obs, var_obs.data(), n);
-    if (ni)
-        HIP_OK(hipMemcpy(d_selected_idx, selected_idx.data(), ni * sizeof(int),
-                         hipMemcpyHostToDevice));
+}
+void ObservationHip::upload(const float *mu, const float *var, size_t n, const int *idx,
+                            size_t ni) {
+    this->reserve(n, ni);
+    h2d(d_mu_obs, mu, n);
+    h2d(d_var_obs, var, n);
+    if (ni) HIP_OK(hipMemcpy(d_selected_idx, idx, ni * sizeof(int), hipMemcpyHostToDevice));
+}
+void ObservationHip::to_device() {
+    this->upload(mu_obs.data(), var_obs.data(), mu_obs.size(), selected_idx.data(),
+                 selected_idx.size());
 }
 
 }  // namespace tagi_host

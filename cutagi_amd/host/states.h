@@ -174,6 +174,11 @@ class ObservationHip : public BaseObservation {
     ~ObservationHip() override;
     std::string get_name() const override { return "ObservationCuda"; }
     void to_device();  // grows the device arrays as needed, then copies
+    // Same, straight from caller memory (no host mirror is kept): n observations and
+    // variances, n_idx selected indices (idx may be null with n_idx = 0).
+    void upload(const float *mu, const float *var, size_t n, const int *idx, size_t n_idx);
+   private:
+    void reserve(size_t n, size_t n_idx);
 };
 
 }  // namespace tagi_host

@@ -177,3 +177,59 @@ def test_errors_and_checkpoint_round_trip(tmp_path):
     with pytest.raises(RuntimeError):
         cutagi.OutputUpdater("cpu").update(net.output_z_buffer, [0.0] * 12, [1.0] * 12,
                                            net.input_delta_z_buffer)
+
+
+def test_output_updater_reads_numpy_arrays_in_place():
+    """float32 / int32 numpy arrays take the binding's direct path; lists (the
+    reference's binding) and arrays of another type take the std::vector path.
+    Both give the same innovations, and wrong sizes or indices raise."""
+    from cutagi_amd import cutagi
+    cutagi.manual_seed(2)
+    rng = np.random.default_rng(2)
+    B, N = 16, 11
+    net = cutagi.Sequential([cutagi.Linear(20, N)])
+    net.to_device("cuda")
+    net.forward(rng.normal(0, 1, (B, 20)).astype(np.float32))
+    upd = cutagi.OutputUpdater(net.device)
+    d = net.input_delta_z_buffer
+
+    def deltas():
+        d.to_host()
+        return np.array(d.delta_mu[:B * N], np.float32), np.array(d.delta_var[:B * N], np.float32)
+
+    y = rng.normal(0, 1, B * N).astype(np.float32)
+    v = rng.uniform(0.5, 1.5, B * N).astype(np.float32)
+    upd.update(net.output_z_buffer, y.tolist(), v.tolist(), d)
+    want = deltas()
+    upd.update(net.output_z_buffer, y, v, d)
+    got = deltas()
+    assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
+    upd.update(net.output_z_buffer, y.astype(np.float64), v.astype(np.float64), d)  # converted
+    got = deltas()
+    assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
+
+    n_enc = 4
+    ys = rng.normal(0, 1, B * n_enc).astype(np.float32)
+    vs = np.ones(B * n_enc, np.float32)
+    sel = rng.integers(1, N + 1, B * n_enc).astype(np.int32)
+    upd.update_using_indices(net.output_z_buffer, ys.tolist(), vs.tolist(), sel.tolist(), d)
+    want = deltas()
+    assert np.any(want[0] != 0)
+    upd.update_using_indices(net.output_z_buffer, ys, vs, sel, d)
+    got = deltas()
+    assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
+    upd.update_using_indices(net.output_z_buffer, ys, vs, sel.astype(np.int64), d)  # converted
+    got = deltas()
+    assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
+
+    with pytest.raises(RuntimeError):
+        upd.update(net.output_z_buffer, y, v[:-1], d)
+    with pytest.raises(RuntimeError):
+        upd.update_using_indices(net.output_z_buffer, ys, vs, sel[:-1], d)
+    bad = sel.copy()
+    bad[5] = N + 1
+    with pytest.raises(RuntimeError):
+        upd.update_using_indices(net.output_z_buffer, ys, vs, bad, d)
+    bad[5] = 0
+    with pytest.raises(RuntimeError):
+        upd.update_using_indices(net.output_z_buffer, ys, vs, bad, d)
