@@ -172,6 +172,7 @@ struct ConvFwdProblem {
     using Ctx = GatherCtx;
     static constexpr bool XK = true, YK = false, PROLOGUE_WRITES_LDS = true, SPLIT_PER_XCD = false;
     static constexpr int VARIANTS = 2;  // 1: sixteen-byte loads of consecutive groups
+    static constexpr bool FIT_TWO_WORKGROUPS = true;
     __device__ static __forceinline__ bool variant(const Ctx &ctx) { return ctx.fast != 0; }
     static constexpr int NX = 2, NY = 2, FLAVOR = FLAVOR_FWD_W_ROWS;
 
@@ -246,6 +247,7 @@ struct ConvDwProblem {
     };
     static constexpr bool XK = true, YK = true, PROLOGUE_WRITES_LDS = false, SPLIT_PER_XCD = true;
     static constexpr int VARIANTS = 1;
+    static constexpr bool FIT_TWO_WORKGROUPS = false;
     static constexpr int NX = 2, NY = 1, FLAVOR = FLAVOR_DELTA_ROWS;
 
     static size_t extra_lds_bytes(const Params &, int, int) { return 0; }
@@ -351,6 +353,7 @@ struct ConvDwVecProblem {
     };
     static constexpr bool XK = true, YK = true, PROLOGUE_WRITES_LDS = false, SPLIT_PER_XCD = true;
     static constexpr int VARIANTS = 1;
+    static constexpr bool FIT_TWO_WORKGROUPS = false;
     static constexpr int NX = 2, NY = 1, FLAVOR = FLAVOR_DELTA_ROWS;
 
     static size_t extra_lds_bytes(const Params &, int, int) { return 0; }
@@ -448,6 +451,7 @@ struct ConvDzProblem {
     using Ctx = GatherCtx;
     static constexpr bool XK = true, YK = false, PROLOGUE_WRITES_LDS = true, SPLIT_PER_XCD = false;
     static constexpr int VARIANTS = 2;  // 1: sixteen-byte loads of consecutive groups
+    static constexpr bool FIT_TWO_WORKGROUPS = false;
     __device__ static __forceinline__ bool variant(const Ctx &ctx) { return ctx.fast != 0; }
     static constexpr int NX = 1, NY = 2, FLAVOR = FLAVOR_DELTA_COLS;
 

@@ -27,6 +27,7 @@
 //   extra_lds_bytes(p, BM, BN)  host: dynamic LDS the prologue wants (index tables)
 //   prologue(p, ctx, extra, tid, nthreads, m0, n0, BM, BN, r_begin, r_end)
 //                               runs once before the first load; a barrier follows
+//   FIT_TWO_WORKGROUPS         see tile_min_waves
 //   VARIANTS, variant(ctx)      number of loader variants (1 or 2) and, after the
 //                               prologue, which one this workgroup uses (uniform)
 //   load_x(p, ctx, V, arr, i, m0, row, r, r_end)
@@ -104,6 +105,14 @@ __device__ __forceinline__ float4 read_frag(const float *lds, int row, int kk, i
         const float *q = lds + k * S + row + (lane & 31);
         return make_float4(q[0], q[S], q[2 * S], q[3 * S]);
     }
+}
+
+// Waves per SIMD the register allocation has to leave room for. Two 8-wave
+// workgroups on a CU need four (at most 128 registers per lane); a problem whose
+// 64x128 kernel would land just above that asks for it with FIT_TWO_WORKGROUPS.
+template <class P>
+constexpr int tile_min_waves(int bm, int bn, int waves) {
+    return (P::FIT_TWO_WORKGROUPS && waves == 8 && bm * bn <= 64 * 128) ? 4 : (waves + 3) / 4;
 }
 
 // Everything a workgroup does after its prologue, instantiated once per loader
@@ -275,7 +284,9 @@ __device__ __forceinline__ void mfma_tile_body(const typename P::Params &p, type
 
 
 template <class P, int BM, int BN, int WM, int WN>
-__global__ __launch_bounds__(WM *WN * 64) void mfma_tile_kernel(typename P::Params p) {
+__global__ __launch_bounds__(WM *WN * 64)
+__attribute__((amdgpu_waves_per_eu(tile_min_waves<P>(BM, BN, WM * WN))))
+void mfma_tile_kernel(typename P::Params p) {
     constexpr bool XK = P::XK, YK = P::YK;
     constexpr int NX = P::NX, NY = P::NY, FL = P::FLAVOR;
     constexpr int NT = WM * WN * 64;
