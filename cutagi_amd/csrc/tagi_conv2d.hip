@@ -172,7 +172,10 @@ struct ConvFwdProblem {
     using Ctx = GatherCtx;
     static constexpr bool XK = true, YK = false, PROLOGUE_WRITES_LDS = true, SPLIT_PER_XCD = false;
     static constexpr int VARIANTS = 2;  // 1: sixteen-byte loads of consecutive groups
-    static constexpr bool FIT_TWO_WORKGROUPS = true;
+    // 130 registers without the request: one 64x128 workgroup per CU instead of two
+    static constexpr int min_waves_per_simd(int bm, int bn, int waves) {
+        return waves == 8 && bm * bn <= 64 * 128 ? 4 : 0;
+    }
     __device__ static __forceinline__ bool variant(const Ctx &ctx) { return ctx.fast != 0; }
     static constexpr int NX = 2, NY = 2, FLAVOR = FLAVOR_FWD_W_ROWS;
 
@@ -247,7 +250,7 @@ struct ConvDwProblem {
     };
     static constexpr bool XK = true, YK = true, PROLOGUE_WRITES_LDS = false, SPLIT_PER_XCD = true;
     static constexpr int VARIANTS = 1;
-    static constexpr bool FIT_TWO_WORKGROUPS = false;
+    static constexpr int min_waves_per_simd(int, int, int) { return 0; }
     static constexpr int NX = 2, NY = 1, FLAVOR = FLAVOR_DELTA_ROWS;
 
     static size_t extra_lds_bytes(const Params &, int, int) { return 0; }
@@ -353,7 +356,9 @@ struct ConvDwVecProblem {
     };
     static constexpr bool XK = true, YK = true, PROLOGUE_WRITES_LDS = false, SPLIT_PER_XCD = true;
     static constexpr int VARIANTS = 1;
-    static constexpr bool FIT_TWO_WORKGROUPS = false;
+    // (asking for four or five 64x64 workgroups per CU instead of three measured
+    // no gain)
+    static constexpr int min_waves_per_simd(int, int, int) { return 0; }
     static constexpr int NX = 2, NY = 1, FLAVOR = FLAVOR_DELTA_ROWS;
 
     static size_t extra_lds_bytes(const Params &, int, int) { return 0; }
@@ -451,7 +456,7 @@ struct ConvDzProblem {
     using Ctx = GatherCtx;
     static constexpr bool XK = true, YK = false, PROLOGUE_WRITES_LDS = true, SPLIT_PER_XCD = false;
     static constexpr int VARIANTS = 2;  // 1: sixteen-byte loads of consecutive groups
-    static constexpr bool FIT_TWO_WORKGROUPS = false;
+    static constexpr int min_waves_per_simd(int, int, int) { return 0; }
     __device__ static __forceinline__ bool variant(const Ctx &ctx) { return ctx.fast != 0; }
     static constexpr int NX = 1, NY = 2, FLAVOR = FLAVOR_DELTA_COLS;
 

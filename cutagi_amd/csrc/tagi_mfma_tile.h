@@ -27,7 +27,8 @@
 //   extra_lds_bytes(p, BM, BN)  host: dynamic LDS the prologue wants (index tables)
 //   prologue(p, ctx, extra, tid, nthreads, m0, n0, BM, BN, r_begin, r_end)
 //                               runs once before the first load; a barrier follows
-//   FIT_TWO_WORKGROUPS         see tile_min_waves
+//   min_waves_per_simd(BM, BN, waves)
+//                               occupancy the register allocation must allow (0: none)
 //   VARIANTS, variant(ctx)      number of loader variants (1 or 2) and, after the
 //                               prologue, which one this workgroup uses (uniform)
 //   load_x(p, ctx, V, arr, i, m0, row, r, r_end)
@@ -107,12 +108,15 @@ __device__ __forceinline__ float4 read_frag(const float *lds, int row, int kk, i
     }
 }
 
-// Waves per SIMD the register allocation has to leave room for. Two 8-wave
-// workgroups on a CU need four (at most 128 registers per lane); a problem whose
-// 64x128 kernel would land just above that asks for it with FIT_TWO_WORKGROUPS.
+// Waves per SIMD the register allocation has to leave room for: what the
+// workgroup size implies, or more where the problem asks for it (two 8-wave
+// workgroups on a CU need four, i.e. at most 128 registers per lane; a kernel that
+// would land just above such a step loses a whole workgroup per CU).
 template <class P>
 constexpr int tile_min_waves(int bm, int bn, int waves) {
-    return (P::FIT_TWO_WORKGROUPS && waves == 8 && bm * bn <= 64 * 128) ? 4 : (waves + 3) / 4;
+    return P::min_waves_per_simd(bm, bn, waves) > (waves + 3) / 4
+               ? P::min_waves_per_simd(bm, bn, waves)
+               : (waves + 3) / 4;
 }
 
 // Everything a workgroup does after its prologue, instantiated once per loader
