@@ -182,6 +182,7 @@ int tagi_hip_tune(const char *key, int value) {
     else if (!strcmp(key, "conv2d.splits")) g_tune.conv_splits = value;
     else if (!strcmp(key, "conv2d.tile")) g_tune.conv_tile = value;
     else if (!strcmp(key, "conv2d.group_loads")) g_conv2d_group_loads = value;
+    else if (!strcmp(key, "conv2d.stencil")) g_conv2d_stencil = value;
     else if (!strcmp(key, "linear.tile")) g_tune.tile = value;
     else if (!strcmp(key, "conv2d.dw.splits")) g_tune.conv_dw_splits = value;
     else if (!strcmp(key, "linear.gemv.swizzle")) g_tune.gemv_swz = value;

@@ -15,6 +15,8 @@
 // The permutations the reference runs as separate passes (Jacobian, deltas) are
 // folded into the operand addressing. Offsets inside one tensor are 32-bit: the
 // entry points refuse tensors of 2^31 elements or more.
+#include <type_traits>
+
 #include "tagi_internal.h"
 #include "tagi_mfma_tile.h"
 
@@ -527,6 +529,14 @@ struct ConvDzProblem {
     }
 };
 
+}  // namespace
+}  // namespace tagi
+
+#include "tagi_conv_stencil.h"
+
+namespace tagi {
+namespace {
+
 // Bias innovation: per-channel sums over (b, o) in two stages.
 __global__ __launch_bounds__(256) void conv_bias_partial_kernel(const float *__restrict__ dmu,
                                                                 const float *__restrict__ dvar,
@@ -599,21 +609,27 @@ void conv2d_plan(int M, int N, int R, int *tile, int *splits) {
 }
 
 namespace {
-template <class P>
-hipError_t run_sliced(int tile, int splits, float *ws0, float *ws1, ConvParams &p,
+// `stencil`: map width when the regular-stencil kernel applies (slices are then
+// whole groups of 32 channels: a multiple of its 72-step and of the table-driven
+// loop's 32-step k-tile), 0 otherwise.
+template <class P, bool DZ>
+hipError_t run_sliced(int tile, int splits, int stencil, float *ws0, float *ws1, ConvParams &p,
                       hipStream_t stream) {
-    const int per = ceil_div(ceil_div(p.R, splits), KT) * KT;
+    const int unit = stencil ? 288 : KT;
+    const int per = ceil_div(ceil_div(p.R, splits), unit) * unit;
     p.splits = ceil_div(p.R, per);
     p.r_per_split = per;
     p.ws0 = ws0;
     p.ws1 = ws1;
-    hipError_t e = launch_tiles<P>(tile, p, stream);
+    hipError_t e = stencil ? launch_conv_stencil<DZ>(stencil, p, stream)
+                           : launch_tiles<P>(tile, p, stream);
     if (e != hipSuccess || p.splits == 1) return e;
     return launch_reduce_store<P>(p, stream);
 }
 }  // namespace
 
 int g_conv2d_group_loads = 1;
+int g_conv2d_stencil = 1;
 
 hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
                              const float *var_b, const float *mu_a, const float *var_a,
@@ -628,8 +644,13 @@ hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float 
     p.M = fo; p.N = B * woho; p.R = p.k2 * fi;
     p.group_loads = g_conv2d_group_loads;
     const bool vec = (p.R % 4 == 0) && aligned16(mu_w) && aligned16(var_w);
-    if (vec) return run_sliced<ConvFwdProblem<true>>(tile, splits, ws0, ws1, p, stream);
-    return run_sliced<ConvFwdProblem<false>>(tile, splits, ws0, ws1, p, stream);
+    // 3x3, stride 1, "same" padding on a square map (the kernel verifies the table)
+    int stencil = 0;
+    if (g_conv2d_stencil && vec && ki == 3 && woho == wihi && fi % 8 == 0 && fo % 64 == 0 &&
+        tile == TILE_64x128 && aligned16(mu_a) && aligned16(var_a))
+        stencil = stencil_width(wihi);
+    if (vec) return run_sliced<ConvFwdProblem<true>, false>(tile, splits, stencil, ws0, ws1, p, stream);
+    return run_sliced<ConvFwdProblem<false>, false>(tile, splits, 0, ws0, ws1, p, stream);
 }
 
 hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *dmu,
@@ -644,7 +665,11 @@ hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float
     p.woho = woho; p.fo = fo; p.wihi = wihi; p.fi = fi; p.k2 = k2; p.B = B; p.nr = nr;
     p.M = fi; p.N = B * wihi; p.R = k2 * fo;
     p.group_loads = g_conv2d_group_loads;
-    return run_sliced<ConvDzProblem>(tile, splits, ws0, ws1, p, stream);
+    int stencil = 0;
+    if (g_conv2d_stencil && ki == 3 && nr == 9 && woho == wihi && fo % 8 == 0 && fi % 64 == 0 &&
+        tile == TILE_64x128 && aligned16(mu_w) && aligned16(dmu) && aligned16(dvar))
+        stencil = stencil_width(wihi);
+    return run_sliced<ConvDzProblem, true>(tile, splits, stencil, ws0, ws1, p, stream);
 }
 
 // Workgroups of the weight-backward kernel that one CU holds at a time.

@@ -1,0 +1,331 @@
+// Conv2d forward and state backward for the geometry that carries almost all of
+// a ResNet's work: 3x3 kernel, stride 1, one pixel of padding on every side, on
+// square maps of width 4, 8, 16 or 32. For it the reference's index tables
+// (src/conv2d_layer.cpp:274-323, 363-404 read them per tap) describe a regular
+// stencil: tap (ky, kx) of output pixel (y, x) reads input pixel (y+ky-1, x+kx-1),
+// and nothing outside the map. Each workgroup first CHECKS that against the
+// tables it was given, for its own pixels; only then does it take the path below,
+// otherwise the table-driven kernel body runs (included from tagi_conv2d.hip, so
+// any table still gives the table's result).
+//
+// What the regular stencil buys: a 128-pixel tile is 128/W whole image rows, so
+// instead of gathering nine shifted copies of every channel map (nine loads and
+// nine table lookups per element) the workgroup stages each channel's rows ONCE,
+// with a zero halo, and the nine taps are nine constant offsets into that patch
+// when the MFMA operand is read from LDS. The k-tile is 8 channels x 9 taps = 72
+// reduction steps; MFMA k-halves (lanes 0-31 / 32-63) take an even / odd channel
+// at the same tap, so one LDS address per lane plus an immediate per step reaches
+// every operand.
+//
+// Included by tagi_conv2d.hip after ConvParams, ConvFwdProblem and ConvDzProblem.
+#pragma once
+
+namespace tagi {
+namespace {
+
+template <int WIDTH>
+struct StencilGeom {
+    static constexpr int W = WIDTH, H = WIDTH;     // square maps
+    static constexpr int BM = 64, BN = 128;        // output tile: rows x pixels
+    static constexpr int KC = 8;                   // channels per k-tile
+    static constexpr int NR = BN / W;              // image rows per tile
+    static constexpr int RPI = NR < H ? NR : H;    // rows of one image among them
+    static constexpr int SEGS = NR / RPI;          // images (segments) per tile
+    // One patch row: [3 unused][left halo][W values][right halo = cell 0 of the
+    // next row]; values start 16-byte aligned. Unused and halo cells stay zero.
+    static constexpr int XO = 4;
+    static constexpr int RS = W + 4;
+    // Rows r = -1 .. RPI of a segment; the pad of the narrowest map moves the
+    // second image of a 32-pixel column block onto other LDS banks.
+    static constexpr int SEG = (RPI + 2) * RS + (W == 4 ? 4 : 0);
+    static constexpr int CS = SEGS * SEG + 4;      // one channel (+ the last row's halo cell)
+    static constexpr int PATCH = KC * CS;          // floats per staged array
+    static constexpr int UNITS = KC * SEGS * (RPI + 2) * (W / 4);  // 16-byte loads per array
+    // Weight tile [64 rows][2 halves][36 steps], row stride 76: eight consecutive
+    // rows start on eight different groups of four banks.
+    static constexpr int AS = 76;
+    static constexpr int A_VEC = BM * KC * 9 / 4;  // 16-byte loads per weight array
+    static_assert(UNITS <= 512 && BN % W == 0 && NR % RPI == 0 && H % RPI == 0, "tile geometry");
+};
+
+// Does the table describe the regular stencil for the pixels n0 .. n0+127? Every
+// thread checks a share and returns its verdict.
+template <bool DZ, int WIDTH>
+__device__ __forceinline__ bool stencil_tables_ok(const ConvParams &p, int n0, int tid,
+                                                  int nthreads) {
+    constexpr int W = WIDTH, H = WIDTH;
+    bool ok = true;
+    if (!DZ) {
+        // Fmwa_2 [woho][9]: 1-based input pixel under tap t of output pixel o, -1 = padding
+        for (int e = tid; e < 128 * 9; e += nthreads) {
+            const int c = e / 9, t = e - c * 9, n = n0 + c;
+            if (n >= p.N) continue;
+            const int o = n % p.woho, y = o / W, x = o - y * W;
+            const int iy = y + t / 3 - 1, ix = x + t % 3 - 1;
+            const int want = (iy >= 0 && iy < H && ix >= 0 && ix < W) ? iy * W + ix + 1 : -1;
+            ok = ok && p.idx[o * 9 + t] == want;
+        }
+    } else {
+        // FCzwa_1 [wihi][nr] / Szz_ud [nr][wihi]: per input pixel the (tap, output
+        // pixel) pairs that touch it, in any order. Regular stencil: tap t touches
+        // pixel (y, x) from output pixel (y-ky+1, x-kx+1) when that lies in the map.
+        for (int c = tid; c < 128; c += nthreads) {
+            const int n = n0 + c;
+            if (n >= p.N) continue;
+            const int px = n % p.wihi, y = px / W, x = px - y * W;
+            int seen = 0, want = 0;
+            for (int t = 0; t < 9; t++) {
+                const int qy = y - t / 3 + 1, qx = x - t % 3 + 1;
+                if (qy >= 0 && qy < H && qx >= 0 && qx < W) want |= 1 << t;
+            }
+            for (int j = 0; j < p.nr; j++) {
+                const int o = p.idx2[j * p.wihi + px];
+                if (o <= -1) continue;
+                const int tap = p.idx[px * p.nr + j];
+                if (tap < 1 || tap > 9 || (seen >> (tap - 1) & 1)) {
+                    ok = false;
+                    continue;
+                }
+                const int t = tap - 1, qy = y - t / 3 + 1, qx = x - t % 3 + 1;
+                ok = ok && qy >= 0 && qy < H && qx >= 0 && qx < W && o == qy * W + qx + 1;
+                seen |= 1 << t;
+            }
+            ok = ok && seen == want;
+        }
+    }
+    return ok;
+}
+
+// The tile loop on a verified stencil. `lds` holds the weight tile(s) followed by
+// the two patches. r_begin / r_end are multiples of 72 (whole channels of 9 taps,
+// 8 at a time).
+template <bool DZ, int WIDTH>
+__device__ __forceinline__ void stencil_body(const ConvParams &p, float *lds, int m0, int n0,
+                                             int split, int r_begin, int r_end) {
+    using G = StencilGeom<WIDTH>;
+    using P = typename std::conditional<DZ, ConvDzProblem, ConvFwdProblem<true>>::type;
+    constexpr int W = G::W, H = G::H, NA = DZ ? 1 : 2, NT = 512;
+    constexpr int SLOTS = (G::A_VEC + NT - 1) / NT;  // 3
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wrow = (wave / 4) * 32, wcol = (wave % 4) * 32, half = lane >> 5;
+    float *lds_a = lds;                       // [NA][64][AS]
+    float *lds_p = lds + NA * 64 * G::AS;     // [2][PATCH]
+    // gathered tensor: activations [B][fi][W*H] (forward), innovations [B][fo][W*H]
+    const float *src0 = DZ ? p.d0 : p.a0, *src1 = DZ ? p.d1 : p.a1;
+    const int CH = DZ ? p.fo : p.fi;
+    const int c_begin = r_begin / 9, c_end = r_end / 9;
+
+    for (int i = tid; i < 2 * G::PATCH; i += NT) lds_p[i] = 0.f;
+
+    // this thread's 16 bytes of the patch: channel c, segment, patch row pr, column 4*x4
+    int u = tid < G::UNITS ? tid : 0;
+    const int x4 = u % (W / 4);
+    u /= (W / 4);
+    const int pr = u % (G::RPI + 2);
+    u /= (G::RPI + 2);
+    const int seg = u % G::SEGS, pc = u / G::SEGS;
+    const int grow = n0 / W + seg * G::RPI;  // first image row of the segment, counted over the batch
+    const int img = grow / H, y = grow % H + pr - 1;
+    const bool unit_ok = tid < G::UNITS && y >= 0 && y < H && img < p.B;
+    // a unit outside the map loads element 0 instead and is never written
+    size_t punit = unit_ok ? ((size_t)img * CH + c_begin + pc) * (W * H) + y * W + 4 * x4 : 0;
+    const size_t pstep = unit_ok ? (size_t)G::KC * (W * H) : 0;
+    const int pdst = pc * G::CS + seg * G::SEG + pr * G::RS + G::XO + 4 * x4;
+
+    // this thread's 16-byte pieces of the weight tile and where their four values go
+    // in the [row][half][step] layout
+    size_t aunit[SLOTS];
+    int adst[SLOTS][4];
+    bool a_ok[SLOTS];
+    const size_t astep = DZ ? (size_t)G::KC * p.fi * 9 : (size_t)G::KC * 9;
+#pragma unroll
+    for (int i = 0; i < SLOTS; i++) {
+        const int idx = tid + i * NT;
+        a_ok[i] = idx < G::A_VEC;
+        const int id = a_ok[i] ? idx : 0;
+        if (!DZ) {
+            // rows = output channels, 72 consecutive values of w[row][c*9 + t]
+            const int row = id / 18, q = id - row * 18;
+            aunit[i] = (size_t)(m0 + row) * p.R + (size_t)c_begin * 9 + 4 * q;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int kk = 4 * q + e, c = kk / 9, t = kk - c * 9;
+                adst[i][e] = row * G::AS + (c & 1) * 36 + (c >> 1) * 9 + t;
+            }
+        } else {
+            // rows = input channels; for one output channel f the values
+            // w[f][(m0+row)*9 + t] of the 64 rows are 576 consecutive floats
+            const int f = id / 144, q = id - f * 144;
+            aunit[i] = (size_t)(c_begin + f) * p.fi * 9 + (size_t)m0 * 9 + 4 * q;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int flat = 4 * q + e, row = flat / 9, t = flat - row * 9;
+                adst[i][e] = row * G::AS + (f & 1) * 36 + (f >> 1) * 9 + t;
+            }
+        }
+        if (!a_ok[i]) aunit[i] = 0;
+    }
+
+    floatx16 acc0[1][1], acc1[1][1];
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        acc0[0][0][v] = 0.f;
+        acc1[0][0][v] = 0.f;
+    }
+
+    float4 ra[NA][SLOTS], rp[2];
+    auto fetch = [&]() {
+#pragma unroll
+        for (int i = 0; i < SLOTS; i++) {
+            ra[0][i] = *reinterpret_cast<const float4 *>(p.w0 + aunit[i]);
+            if (NA == 2) ra[NA - 1][i] = *reinterpret_cast<const float4 *>(p.w1 + aunit[i]);
+            if (a_ok[i]) aunit[i] += astep;
+        }
+        rp[0] = *reinterpret_cast<const float4 *>(src0 + punit);
+        rp[1] = *reinterpret_cast<const float4 *>(src1 + punit);
+        punit += pstep;
+    };
+    auto commit = [&]() {
+#pragma unroll
+        for (int a = 0; a < NA; a++)
+#pragma unroll
+            for (int i = 0; i < SLOTS; i++)
+                if (a_ok[i]) {
+                    float *dst = lds_a + a * 64 * G::AS;
+                    dst[adst[i][0]] = ra[a][i].x;
+                    dst[adst[i][1]] = ra[a][i].y;
+                    dst[adst[i][2]] = ra[a][i].z;
+                    dst[adst[i][3]] = ra[a][i].w;
+                }
+        if (unit_ok) {
+            *reinterpret_cast<float4 *>(lds_p + pdst) = rp[0];
+            *reinterpret_cast<float4 *>(lds_p + G::PATCH + pdst) = rp[1];
+        }
+    };
+
+    // operand addresses of this lane
+    const int pix = wcol + (lane & 31), prow = pix / W, px = pix - prow * W;
+    const float *b0 = lds_p + half * G::CS + (prow / G::RPI) * G::SEG + (prow % G::RPI) * G::RS +
+                      G::XO - 1 + px;
+    const float *b1 = b0 + G::PATCH;
+    const float *a0 = lds_a + (wrow + (lane & 31)) * G::AS + half * 36;
+    const float *a1 = a0 + 64 * G::AS;
+
+    __syncthreads();  // patch zeroed
+    if (c_begin < c_end) {
+        fetch();
+        commit();
+    }
+    __syncthreads();
+
+    for (int c0 = c_begin; c0 < c_end; c0 += G::KC) {
+        const bool more = c0 + G::KC < c_end;
+        if (more) fetch();
+#pragma unroll
+        for (int g = 0; g < 9; g++) {
+            const float4 am = *reinterpret_cast<const float4 *>(a0 + 4 * g);
+            float4 av = am;
+            if (NA == 2) av = *reinterpret_cast<const float4 *>(a1 + 4 * g);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int s = 4 * g + e, pair = s / 9, t = s - pair * 9, ky = t / 3, kx = t - ky * 3;
+                const int off = pair * 2 * G::CS +
+                                (DZ ? (2 - ky) * G::RS + (2 - kx) : ky * G::RS + kx);
+                const float w = comp4(am, e), y0 = b0[off], y1 = b1[off];
+                if (!DZ) {
+                    // mean: mu_w mu_a; variance: var_w (var_a + mu_a^2) + mu_w^2 var_a
+                    acc0[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(w, y0, acc0[0][0], 0, 0, 0);
+                    acc1[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(comp4(av, e), y0 * y0 + y1,
+                                                                      acc1[0][0], 0, 0, 0);
+                    acc1[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(w * w, y1, acc1[0][0], 0, 0, 0);
+                } else {
+                    // mean: mu_w delta_mu; variance: mu_w^2 delta_var
+                    acc0[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(w, y0, acc0[0][0], 0, 0, 0);
+                    acc1[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(w * w, y1, acc1[0][0], 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();
+        if (more) {
+            commit();
+            __syncthreads();
+        }
+    }
+    tile_epilogue<P, 64, 128, 2, 4>(p, acc0, acc1, m0, n0, split);
+}
+
+// One 64 x 128 tile per workgroup of 8 waves: verified stencil -> stencil_body,
+// anything else -> the table-driven loop of the generic tile kernel.
+template <bool DZ, int WIDTH>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4)))
+void conv_stencil_kernel(ConvParams p) {
+    using G = StencilGeom<WIDTH>;
+    using P = typename std::conditional<DZ, ConvDzProblem, ConvFwdProblem<true>>::type;
+    constexpr int XF = TileGeom<P::XK, 64>::floats, YF = TileGeom<P::YK, 128>::floats;
+    constexpr int GENERIC = P::NX * XF + P::NY * YF;
+    constexpr int STENCIL = (DZ ? 1 : 2) * 64 * G::AS + 2 * G::PATCH;
+    __shared__ __attribute__((aligned(16))) float lds[GENERIC > STENCIL ? GENERIC : STENCIL];
+    extern __shared__ __attribute__((aligned(16))) int lds_extra[];
+
+    const int tiles_n = (p.N + 127) / 128;
+    const int tile = blockIdx.x, split = blockIdx.y;
+    const int m0 = (tile / tiles_n) * 64, n0 = (tile % tiles_n) * 128;
+    const int r_begin = split * p.r_per_split;
+    const int r_end = min(p.R, r_begin + p.r_per_split);
+
+    if (threadIdx.x == 0) lds_extra[0] = 1;
+    __syncthreads();
+    if (!stencil_tables_ok<DZ, WIDTH>(p, n0, threadIdx.x, 512)) lds_extra[0] = 0;
+    __syncthreads();
+    const int regular = __builtin_amdgcn_readfirstlane(lds_extra[0]);
+    __syncthreads();  // the table-driven prologue reuses lds_extra
+    if (regular) {
+        stencil_body<DZ, WIDTH>(p, lds, m0, n0, split, r_begin, r_end);
+        return;
+    }
+    typename P::Ctx ctx;
+    P::prologue(p, ctx, lds_extra, threadIdx.x, 512, m0, n0, 64, 128, r_begin, r_end);
+    __syncthreads();
+    mfma_tile_body<P, 64, 128, 2, 4, 0>(p, ctx, reinterpret_cast<float (*)[XF]>(lds),
+                                        reinterpret_cast<float (*)[YF]>(lds + P::NX * XF), m0, n0,
+                                        split, r_begin, r_end);
+}
+
+// Map width for which the stencil kernel exists, 0 otherwise (pixels = width^2).
+inline int stencil_width(int pixels) {
+    for (int w : {4, 8, 16, 32})
+        if (w * w == pixels) return w;
+    return 0;
+}
+
+template <bool DZ>
+hipError_t launch_conv_stencil(int width, const ConvParams &p, hipStream_t stream) {
+    using P = typename std::conditional<DZ, ConvDzProblem, ConvFwdProblem<true>>::type;
+    const dim3 grid(((p.M + 63) / 64) * ((p.N + 127) / 128), p.splits);
+    const size_t extra = P::extra_lds_bytes(p, 64, 128);
+    if (extra > kTileExtraLdsMax) return hipErrorInvalidValue;
+#define TAGI_LAUNCH_STENCIL(WD)                                                                  \
+    case WD: {                                                                                   \
+        static bool allowed = false;                                                             \
+        if (!allowed) {                                                                          \
+            hipError_t e = hipFuncSetAttribute(                                                  \
+                reinterpret_cast<const void *>(conv_stencil_kernel<DZ, WD>),                     \
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTileExtraLdsMax);              \
+            if (e != hipSuccess) return e;                                                       \
+            allowed = true;                                                                      \
+        }                                                                                        \
+        hipLaunchKernelGGL((conv_stencil_kernel<DZ, WD>), grid, dim3(512), extra, stream, p);    \
+        return hipGetLastError();                                                                \
+    }
+    switch (width) {
+        TAGI_LAUNCH_STENCIL(4)
+        TAGI_LAUNCH_STENCIL(8)
+        TAGI_LAUNCH_STENCIL(16)
+        TAGI_LAUNCH_STENCIL(32)
+    }
+#undef TAGI_LAUNCH_STENCIL
+    return hipErrorInvalidValue;
+}
+
+}  // namespace
+}  // namespace tagi

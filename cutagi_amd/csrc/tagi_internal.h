@@ -131,6 +131,8 @@ hipError_t launch_add_shortcut(const float *mu_s, const float *var_s, const floa
 void conv2d_plan(int M, int N, int R, int *tile, int *splits);
 // 0 switches the sixteen-byte group loads of the conv2d gathers off (tuning knob).
 extern int g_conv2d_group_loads;
+// 0 switches the regular-stencil kernels of the conv2d forward / state backward off.
+extern int g_conv2d_stencil;
 
 hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
                              const float *var_b, const float *mu_a, const float *var_a,

@@ -119,6 +119,39 @@ constexpr int tile_min_waves(int bm, int bn, int waves) {
                : (waves + 3) / 4;
 }
 
+// Writes a workgroup's accumulators: partial sums of a reduction slice go to the
+// workspace, a complete sum to the problem's epilogue. Accumulator register v of
+// lane l is D[8*(v/4) + 4*(l/32) + v%4][l%32]: lanes run along the output columns.
+template <class P, int BM, int BN, int WM, int WN>
+__device__ __forceinline__ void tile_epilogue(const typename P::Params &p,
+                                              floatx16 (&acc0)[BM / WM / 32][BN / WN / 32],
+                                              floatx16 (&acc1)[BM / WM / 32][BN / WN / 32],
+                                              int m0, int n0, int split) {
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wrow = (wave / WN) * (TM * 32), wcol = (wave % WN) * (TN * 32);
+    const bool partial = p.splits > 1;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int col = n0 + wcol + j * 32 + (lane & 31);
+            if (col >= p.N) continue;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = m0 + wrow + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                if (row >= p.M) continue;
+                if (partial) {
+                    const size_t at = ((size_t)split * p.M + row) * p.N + col;
+                    p.ws0[at] = acc0[i][j][v];
+                    p.ws1[at] = acc1[i][j][v];
+                } else {
+                    P::store(p, row, col, acc0[i][j][v], acc1[i][j][v]);
+                }
+            }
+        }
+}
+
 // Everything a workgroup does after its prologue, instantiated once per loader
 // variant V (a problem whose prologue chooses between two ways of loading gets two
 // copies of the loop instead of a branch at every load).
@@ -262,28 +295,7 @@ __device__ __forceinline__ void mfma_tile_body(const typename P::Params &p, type
         }
     }
 
-    // Accumulator register v of lane l is D[8*(v/4) + 4*(l/32) + v%4][l%32]: lanes
-    // run along the output columns.
-    const bool partial = p.splits > 1;
-#pragma unroll
-    for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const int col = n0 + wcol + j * 32 + (lane & 31);
-            if (col >= p.N) continue;
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int row = m0 + wrow + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
-                if (row >= p.M) continue;
-                if (partial) {
-                    const size_t at = ((size_t)split * p.M + row) * p.N + col;
-                    p.ws0[at] = acc0[i][j][v];
-                    p.ws1[at] = acc1[i][j][v];
-                } else {
-                    P::store(p, row, col, acc0[i][j][v], acc1[i][j][v]);
-                }
-            }
-        }
+    tile_epilogue<P, BM, BN, WM, WN>(p, acc0, acc1, m0, n0, split);
 }
 
 

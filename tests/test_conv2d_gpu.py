@@ -23,6 +23,12 @@ GEOMS = [
     (7, 2, 3, 1, 17, 3, 40, 2),  # per-tap table + staged tiles exceed 64 KB of LDS
     (3, 1, 1, 1, 4, 128, 96, 3),  # late-stage shape: few pixels, long reduction (sliced)
     (2, 2, 0, 1, 8, 64, 130, 2),  # projection shortcut, more than 128 output channels
+    # 3x3 s1 p1 on square maps with whole groups of channels: the regular-stencil kernels
+    (3, 1, 1, 1, 32, 16, 64, 2),  # forward only (state backward wants 64 input channels)
+    (3, 1, 1, 1, 32, 64, 64, 1),
+    (3, 1, 1, 1, 16, 64, 128, 3),
+    (3, 1, 1, 1, 8, 128, 64, 3),  # two images per tile, last tile half empty
+    (3, 1, 1, 1, 4, 320, 64, 5),  # eight images per tile, one partial tile, sliced reduction
 ]
 
 
@@ -78,3 +84,89 @@ def test_conv2d_backward(oracle_lib, geom):
                               ref_dw):
         assert_close(got.cpu().numpy(), ref, name)
     assert float(dz[1].max()) <= 0.0 and float(dw[1].max()) <= 0.0
+
+
+def _same_padding_tables(k, wi, hi, pad_idx):
+    """Index tables of a k x k, stride 1, (k-1)/2 padded convolution on a wi x hi map,
+    in the reference's layout (the library's own builder makes square maps only)."""
+    off, k2, n = (k - 1) // 2, k * k, wi * hi
+    fm = np.full((n, k2), -1, np.int32)
+    occ = [[] for _ in range(n)]
+    for oy in range(hi):
+        for ox in range(wi):
+            for ky in range(k):
+                for kx in range(k):
+                    iy, ix = oy + ky - off, ox + kx - off
+                    if 0 <= iy < hi and 0 <= ix < wi:
+                        fm[oy * wi + ox, ky * k + kx] = iy * wi + ix + 1
+                        occ[iy * wi + ix].append((ky * k + kx + 1, oy * wi + ox + 1))
+    h = max(len(o) for o in occ)
+    zw = np.full((n, h), pad_idx, np.int32)
+    zud = np.full((h, n), -1, np.int32)
+    for p, lst in enumerate(occ):
+        for j, (tap, o) in enumerate(lst):
+            zw[p, j], zud[j, p] = tap, o
+    return dict(Fmwa_2=fm.ravel(), FCzwa_1=zw.ravel(), Szz_ud=zud.ravel(), h=h)
+
+
+def test_same_padding_tables_helper_matches_the_builder():
+    from cutagi_amd import capi
+    a = _same_padding_tables(3, 8, 8, 999)
+    b = capi.conv2d_build_idx(3, 1, 8, 8, 1, 1, 999)
+    assert all(np.array_equal(a[k], b[k]) for k in ("Fmwa_2", "FCzwa_1", "Szz_ud")) and a["h"] == b["h"]
+
+
+@pytest.mark.parametrize("wi,hi", [(16, 64), (64, 16)])
+def test_conv2d_tables_of_another_geometry_take_the_table_path(oracle_lib, wi, hi):
+    """1024 pixels per map are taken for a 32 x 32 map by the launcher; the kernels
+    check the tables they are given and fall back to the table-driven loop when
+    these describe something else (here a 16 x 64 / 64 x 16 map)."""
+    import torch
+    import cutagi_amd.functional as F
+    from cutagi_amd import capi
+    k, fi, fo, B = 3, 64, 64, 2
+    idx = _same_padding_tables(k, wi, hi, k * k * fi * fo + 1)
+    assert wi * hi == 1024 and idx["h"] == 9
+    d = conv_inputs(fi, fo, k, 1024, 1024, B, seed=wi, bias=False, jcb_random=True)
+    t = {n: (None if v is None else torch.from_numpy(v).cuda()) for n, v in d.items()}
+    ti = {n: torch.from_numpy(idx[n]).cuda() for n in ("Fmwa_2", "FCzwa_1", "Szz_ud")}
+    mu_z, var_z = F.conv2d_fwd(t["mu_w"], t["var_w"], None, None, t["mu_a"], t["var_a"],
+                               ti["Fmwa_2"], 1024, fo, 1024, fi, k, B)
+    ref = oracle_lib.conv2d_fwd(d["mu_w"], d["var_w"], None, None, d["mu_a"], d["var_a"],
+                                idx["Fmwa_2"], 1024, fo, 1024, fi, k, B, threads=4)
+    assert_close(mu_z.cpu().numpy(), ref[0], "mu_z")
+    assert_close(var_z.cpu().numpy(), ref[1], "var_z")
+    dz = F.conv2d_bwd_dz(t["mu_w"], t["jcb"], t["delta_mu"], t["delta_var"], ti["FCzwa_1"],
+                         ti["Szz_ud"], 1024, fo, 1024, fi, k, idx["h"], B)
+    ref_dz = oracle_lib.conv2d_bwd_dz(d["mu_w"], d["jcb"], d["delta_mu"], d["delta_var"],
+                                      idx["FCzwa_1"], idx["Szz_ud"], 1024, fo, 1024, fi, k,
+                                      idx["h"], B, threads=4)
+    assert_close(dz[0].cpu().numpy(), ref_dz[0], "delta_mu_z")
+    assert_close(dz[1].cpu().numpy(), ref_dz[1], "delta_var_z")
+
+
+def test_conv2d_stencil_kernels_agree_with_the_table_path():
+    """Same inputs through the regular-stencil kernels and, with them switched off,
+    through the table-driven kernels."""
+    import torch
+    import cutagi_amd.functional as F
+    from cutagi_amd import capi
+    k, wi, fi, fo, B = 3, 16, 64, 64, 8
+    idx = capi.conv2d_build_idx(k, 1, wi, wi, 1, 1, k * k * fi * fo + 1)
+    d = conv_inputs(fi, fo, k, wi * wi, wi * wi, B, seed=1, bias=True, jcb_random=True)
+    t = {n: torch.from_numpy(v).cuda() for n, v in d.items()}
+    ti = {n: torch.from_numpy(idx[n]).cuda() for n in ("Fmwa_2", "FCzwa_1", "Szz_ud")}
+    out = {}
+    try:
+        for mode in (1, 0):
+            capi.tune("conv2d.stencil", mode)
+            z = F.conv2d_fwd(t["mu_w"], t["var_w"], t["mu_b"], t["var_b"], t["mu_a"], t["var_a"],
+                             ti["Fmwa_2"], wi * wi, fo, wi * wi, fi, k, B)
+            dz = F.conv2d_bwd_dz(t["mu_w"], t["jcb"], t["delta_mu"], t["delta_var"], ti["FCzwa_1"],
+                                 ti["Szz_ud"], wi * wi, fo, wi * wi, fi, k, idx["h"], B)
+            out[mode] = [x.cpu().numpy() for x in (*z, *dz)]
+    finally:
+        capi.tune("conv2d.stencil", 1)
+    for name, a, b in zip(("mu_z", "var_z", "delta_mu_z", "delta_var_z"), out[1], out[0]):
+        assert_close(a, b, name)
+        assert not np.array_equal(a, b) or name == "", "both modes ran the same kernel?"
