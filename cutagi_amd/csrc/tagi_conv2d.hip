@@ -712,13 +712,21 @@ hipError_t launch_conv2d_bwd_dw(const float *var_w, const float *mu_a, const flo
     p.out0 = dmu_w; p.out1 = dvar_w;
     p.woho = woho; p.fo = fo; p.wihi = wihi; p.fi = fi; p.k2 = ki * ki; p.B = B;
     p.M = fo; p.N = p.k2 * fi; p.R = B * woho;
-    int per = ceil_div(ceil_div(p.R, splits), KT) * KT;
+    const bool vec = (woho % 4 == 0) && aligned16(dmu) && aligned16(dvar);
+    // 3x3, stride 1, "same" padding on a square map (the kernel verifies the table):
+    // 64 x 64 tiles of whole channels, slices of whole 64-pixel k-tiles
+    int stencil = 0;
+    if (g_conv2d_stencil && vec && ki == 3 && woho == wihi && fi % 64 == 0 && fo % 64 == 0 &&
+        p.R % 64 == 0 && tile == TILE_64x64 && aligned16(mu_a))
+        stencil = stencil_width(wihi);
+    const int unit = stencil ? 64 : KT;
+    int per = ceil_div(ceil_div(p.R, splits), unit) * unit;
     p.splits = ceil_div(p.R, per);
     p.r_per_split = per;
     p.ws0 = ws0; p.ws1 = ws1;
-    const bool vec = (woho % 4 == 0) && aligned16(dmu) && aligned16(dvar);
-    hipError_t e = vec ? launch_tiles<ConvDwVecProblem>(tile, p, stream)
-                       : launch_tiles<ConvDwProblem<false>>(tile, p, stream);
+    hipError_t e = stencil ? launch_conv_stencil_dw(stencil, p, stream)
+                   : vec   ? launch_tiles<ConvDwVecProblem>(tile, p, stream)
+                           : launch_tiles<ConvDwProblem<false>>(tile, p, stream);
     if (e != hipSuccess) return e;
     if (p.splits > 1)
         e = launch_reduce_splits(EPI_SCALE, ws0, ws1, p.splits, p.M, p.N, var_w, nullptr, dmu_w,

@@ -173,7 +173,7 @@ __device__ __forceinline__ void stencil_body(const ConvParams &p, float *lds, in
         acc1[0][0][v] = 0.f;
     }
 
-    float4 ra[NA][SLOTS], rp[2];
+    float4 ra[NA][SLOTS], rp0, rp1;
     auto fetch = [&]() {
 #pragma unroll
         for (int i = 0; i < SLOTS; i++) {
@@ -181,8 +181,8 @@ __device__ __forceinline__ void stencil_body(const ConvParams &p, float *lds, in
             if (NA == 2) ra[NA - 1][i] = *reinterpret_cast<const float4 *>(p.w1 + aunit[i]);
             if (a_ok[i]) aunit[i] += astep;
         }
-        rp[0] = *reinterpret_cast<const float4 *>(src0 + punit);
-        rp[1] = *reinterpret_cast<const float4 *>(src1 + punit);
+        rp0 = *reinterpret_cast<const float4 *>(src0 + punit);
+        rp1 = *reinterpret_cast<const float4 *>(src1 + punit);
         punit += pstep;
     };
     auto commit = [&]() {
@@ -198,8 +198,8 @@ __device__ __forceinline__ void stencil_body(const ConvParams &p, float *lds, in
                     dst[adst[i][3]] = ra[a][i].w;
                 }
         if (unit_ok) {
-            *reinterpret_cast<float4 *>(lds_p + pdst) = rp[0];
-            *reinterpret_cast<float4 *>(lds_p + G::PATCH + pdst) = rp[1];
+            *reinterpret_cast<float4 *>(lds_p + pdst) = rp0;
+            *reinterpret_cast<float4 *>(lds_p + G::PATCH + pdst) = rp1;
         }
     };
 
@@ -325,6 +325,230 @@ hipError_t launch_conv_stencil(int width, const ConvParams &p, hipStream_t strea
     }
 #undef TAGI_LAUNCH_STENCIL
     return hipErrorInvalidValue;
+}
+
+// ---- weight backward on the same stencil -------------------------------------------
+//   D[fo][(c,t)] = sum over (b, pixel) of delta[b][fo][pixel] * a[b][c][pixel + tap t]
+// Rows are output channels, the 64 columns of a tile are (channel, tap) pairs of
+// exactly eight channels (fi is a multiple of 64), the reduction runs over pixels,
+// 64 at a time = 64/W whole image rows. Per k-tile the workgroup stages the rows
+// of its eight channels once (zero halo as above; halo ROWS now change from tile
+// to tile, so every cell is rewritten, with zero where the row leaves the image);
+// a lane's column fixes its (channel, tap) and with it one LDS base address, and
+// the pixel of each reduction step is an immediate offset.
+template <int WIDTH>
+struct StencilDwGeom {
+    static constexpr int W = WIDTH, H = WIDTH;
+    static constexpr int KP = 64;                   // pixels per k-tile
+    static constexpr int KC = 8;                    // channels per column tile
+    static constexpr int NR = KP / W;               // image rows per k-tile
+    static constexpr int RPI = NR < H ? NR : H;
+    static constexpr int SEGS = NR / RPI;
+    static constexpr int XO = 4, RS = W + 4;
+    static constexpr int SEG = (RPI + 2) * RS + (W == 4 ? 4 : 0);
+    static constexpr int CS = SEGS * SEG + 4;
+    static constexpr int PATCH = KC * CS;
+    static constexpr int UNITS = KC * SEGS * (RPI + 2) * (W / 4);
+    static constexpr int AS = KP + 4;               // innovation tile [64 rows][64 pixels + 4]
+    static constexpr int LOG_PIX = WIDTH == 4 ? 4 : WIDTH == 8 ? 6 : WIDTH == 16 ? 8 : 10;
+    static_assert(UNITS <= 512 && KP % W == 0 && NR % RPI == 0 && H % RPI == 0, "tile geometry");
+    // LDS offset of pixel k (0..63) of the k-tile relative to its first pixel
+    static constexpr int pixel_offset(int k) {
+        return ((k / W) / RPI) * SEG + ((k / W) % RPI) * RS + k % W;
+    }
+};
+
+template <int WIDTH>
+__device__ __forceinline__ void stencil_dw_body(const ConvParams &p, float *lds, int m0, int n0,
+                                                int split, int r_begin, int r_end) {
+    using G = StencilDwGeom<WIDTH>;
+    constexpr int W = G::W, H = G::H, NT = 512, PIX = W * H, SLOTS = 64 * G::KP / 4 / NT;  // 2
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // eight waves: 2 x 2 sub-tiles of 32 x 32, each held by two waves that take
+    // the first / second 32 pixels of every k-tile and add up at the end
+    const int kgroup = wave >> 2;
+    const int wrow = ((wave & 3) / 2) * 32, wcol = (wave & 1) * 32, half = lane >> 5;
+    float *lds_a = lds;                        // [2][64][AS]
+    float *lds_p = lds + 2 * 64 * G::AS;       // [PATCH]
+    const int c_lo = n0 / 9;                   // first channel of the column tile
+
+    for (int i = tid; i < G::PATCH; i += NT) lds_p[i] = 0.f;
+
+    // patch unit: channel pc, segment, patch row pr, column 4*x4. Rows are counted
+    // over the whole batch (image b, row y <-> b*H + y); `grow` is the first row of
+    // the unit's segment in the current k-tile.
+    int u = tid < G::UNITS ? tid : 0;
+    const int x4 = u % (W / 4);
+    u /= (W / 4);
+    const int pr = u % (G::RPI + 2);
+    u /= (G::RPI + 2);
+    const int seg = u % G::SEGS, pc = u / G::SEGS;
+    const bool has_unit = tid < G::UNITS;
+    int grow = r_begin / W + seg * G::RPI;
+    const int pdst = pc * G::CS + seg * G::SEG + pr * G::RS + G::XO + 4 * x4;
+    const int pchan = (c_lo + pc) * PIX + 4 * x4;
+
+    // innovation pieces: 16 bytes at pixel 4*q of rows tid/16 + 32*i
+    const int q = tid % 16, arow = tid / 16;
+    int gpix = r_begin + 4 * q;  // pixel counted over the whole batch
+
+    floatx16 acc0[1][1], acc1[1][1];
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        acc0[0][0][v] = 0.f;
+        acc1[0][0][v] = 0.f;
+    }
+
+    static_assert(SLOTS == 2, "two innovation pieces per thread and array");
+    float4 ra00, ra01, ra10, ra11, rp;
+    bool rp_ok;
+    auto fetch = [&]() {
+        const int b = gpix >> G::LOG_PIX, o = gpix & (PIX - 1);
+        const size_t at = ((size_t)b * p.fo + m0 + arow) * PIX + o;
+        ra00 = *reinterpret_cast<const float4 *>(p.d0 + at);
+        ra10 = *reinterpret_cast<const float4 *>(p.d1 + at);
+        ra01 = *reinterpret_cast<const float4 *>(p.d0 + at + (size_t)32 * PIX);
+        ra11 = *reinterpret_cast<const float4 *>(p.d1 + at + (size_t)32 * PIX);
+        gpix += G::KP;
+        const int img = grow / H, y = grow - img * H + pr - 1;
+        rp_ok = has_unit && y >= 0 && y < H;
+        rp = *reinterpret_cast<const float4 *>(
+            p.a0 + (rp_ok ? (size_t)img * p.fi * PIX + pchan + y * W : 0));
+        grow += G::NR;
+    };
+    auto commit = [&]() {
+        float *d0 = lds_a + arow * G::AS + 4 * q, *d1 = d0 + 64 * G::AS;
+        *reinterpret_cast<float4 *>(d0) = ra00;
+        *reinterpret_cast<float4 *>(d0 + 32 * G::AS) = ra01;
+        *reinterpret_cast<float4 *>(d1) = ra10;
+        *reinterpret_cast<float4 *>(d1 + 32 * G::AS) = ra11;
+        if (has_unit)
+            *reinterpret_cast<float4 *>(lds_p + pdst) =
+                rp_ok ? rp : make_float4(0.f, 0.f, 0.f, 0.f);
+    };
+
+    // operand addresses of this lane: its column is (channel, tap)
+    const int n = n0 + wcol + (lane & 31);
+    const int ch = n / 9 - c_lo, t = n - (n / 9) * 9, ky = t / 3, kx = t - ky * 3;
+    const float *bp = lds_p + ch * G::CS + ky * G::RS + kx + G::XO - 1 +
+                      (half ? G::pixel_offset(4) : 0) + (kgroup ? G::pixel_offset(32) : 0);
+    const float *a0 = lds_a + (wrow + (lane & 31)) * G::AS + 4 * half + 32 * kgroup;
+    const float *a1 = a0 + 64 * G::AS;
+
+    __syncthreads();  // patch zeroed
+    if (r_begin < r_end) {
+        fetch();
+        commit();
+    }
+    __syncthreads();
+
+    for (int r0 = r_begin; r0 < r_end; r0 += G::KP) {
+        const bool more = r0 + G::KP < r_end;
+        if (more) fetch();
+#pragma unroll
+        for (int kk = 0; kk < G::KP / 2; kk += 8) {
+            const float4 dm = *reinterpret_cast<const float4 *>(a0 + kk);
+            const float4 dv = *reinterpret_cast<const float4 *>(a1 + kk);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float y = bp[G::pixel_offset(kk + e)];
+                acc0[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(comp4(dm, e), y, acc0[0][0], 0, 0, 0);
+                acc1[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(comp4(dv, e), y * y, acc1[0][0], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+        if (more) {
+            commit();
+            __syncthreads();
+        }
+    }
+
+    // the second pixel group hands its sums over through LDS ([value][lane] layout)
+    float *xch = lds;
+    if (kgroup == 1) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            xch[v * 256 + (tid - 256)] = acc0[0][0][v];
+            xch[(16 + v) * 256 + (tid - 256)] = acc1[0][0][v];
+        }
+    }
+    __syncthreads();
+    if (kgroup == 1) return;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        acc0[0][0][v] += xch[v * 256 + tid];
+        acc1[0][0][v] += xch[(16 + v) * 256 + tid];
+    }
+    tile_epilogue<ConvDwVecProblem, 64, 64, 2, 2>(p, acc0, acc1, m0, n0, split);
+}
+
+template <int WIDTH>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4)))
+void conv_stencil_dw_kernel(ConvParams p) {
+    using G = StencilDwGeom<WIDTH>;
+    using P = ConvDwVecProblem;
+    constexpr int XF = TileGeom<P::XK, 64>::floats, YF = TileGeom<P::YK, 64>::floats;
+    constexpr int GENERIC = P::NX * XF + P::NY * YF;
+    constexpr int STENCIL = 2 * 64 * G::AS + G::PATCH;
+    static_assert(2 * 64 * G::AS >= 32 * 256, "the innovation tiles hold the final exchange");
+    __shared__ __attribute__((aligned(16))) float lds[GENERIC > STENCIL ? GENERIC : STENCIL];
+    __shared__ int regular_flag;
+
+    const int tiles_n = (p.N + 63) / 64;
+    int tile = blockIdx.x, split = blockIdx.y;
+    if (gridDim.y % 8 == 0) {
+        // all column tiles of one reduction slice on one XCD (see mfma_tile_kernel)
+        const int id = blockIdx.y * gridDim.x + blockIdx.x;
+        const int qq = id >> 3;
+        tile = qq % gridDim.x;
+        split = (qq / gridDim.x) * 8 + (id & 7);
+    }
+    const int m0 = (tile / tiles_n) * 64, n0 = (tile % tiles_n) * 64;
+    const int r_begin = split * p.r_per_split;
+    const int r_end = min(p.R, r_begin + p.r_per_split);
+
+    // the pixels of this slice, per image position: all of Fmwa_2 once the slice
+    // is as long as a map
+    if (threadIdx.x == 0) regular_flag = 1;
+    __syncthreads();
+    {
+        const int len = min(max(r_end - r_begin, 0), p.woho);
+        bool ok = true;
+        for (int e = threadIdx.x; e < len * 9; e += 512) {
+            const int c = e / 9, t = e - c * 9;
+            const int o = (r_begin + c) & (WIDTH * WIDTH - 1), y = o / WIDTH, x = o - y * WIDTH;
+            const int iy = y + t / 3 - 1, ix = x + t % 3 - 1;
+            const int want =
+                (iy >= 0 && iy < WIDTH && ix >= 0 && ix < WIDTH) ? iy * WIDTH + ix + 1 : -1;
+            ok = ok && p.idx[o * 9 + t] == want;
+        }
+        if (!ok) regular_flag = 0;
+    }
+    __syncthreads();
+    if (__builtin_amdgcn_readfirstlane(regular_flag)) {
+        stencil_dw_body<WIDTH>(p, lds, m0, n0, split, r_begin, r_end);
+        return;
+    }
+    // table-driven loop: written for four waves; the other four leave (a barrier
+    // counts the waves that are still running)
+    if (threadIdx.x >= 256) return;
+    typename P::Ctx ctx;
+    P::prologue(p, ctx, nullptr, threadIdx.x, 256, m0, n0, 64, 64, r_begin, r_end);
+    mfma_tile_body<P, 64, 64, 2, 2, 0>(p, ctx, reinterpret_cast<float (*)[XF]>(lds),
+                                       reinterpret_cast<float (*)[YF]>(lds + P::NX * XF), m0, n0,
+                                       split, r_begin, r_end);
+}
+
+inline hipError_t launch_conv_stencil_dw(int width, const ConvParams &p, hipStream_t stream) {
+    const dim3 grid(((p.M + 63) / 64) * ((p.N + 63) / 64), p.splits);
+    switch (width) {
+        case 4: hipLaunchKernelGGL(conv_stencil_dw_kernel<4>, grid, dim3(512), 0, stream, p); break;
+        case 8: hipLaunchKernelGGL(conv_stencil_dw_kernel<8>, grid, dim3(512), 0, stream, p); break;
+        case 16: hipLaunchKernelGGL(conv_stencil_dw_kernel<16>, grid, dim3(512), 0, stream, p); break;
+        case 32: hipLaunchKernelGGL(conv_stencil_dw_kernel<32>, grid, dim3(512), 0, stream, p); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
 }
 
 }  // namespace
