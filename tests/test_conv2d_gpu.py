@@ -143,6 +143,12 @@ def test_conv2d_tables_of_another_geometry_take_the_table_path(oracle_lib, wi, h
                                       idx["h"], B, threads=4)
     assert_close(dz[0].cpu().numpy(), ref_dz[0], "delta_mu_z")
     assert_close(dz[1].cpu().numpy(), ref_dz[1], "delta_var_z")
+    dw = F.conv2d_bwd_dw(t["var_w"], None, t["mu_a"], t["delta_mu"], t["delta_var"],
+                         ti["Fmwa_2"], B, fo, 1024, 1024, fi, k)
+    ref_dw = oracle_lib.conv2d_bwd_dw(d["var_w"], None, d["mu_a"], d["delta_mu"], d["delta_var"],
+                                      idx["Fmwa_2"], B, fo, 1024, 1024, fi, k, threads=4)
+    assert_close(dw[0].cpu().numpy(), ref_dw[0], "delta_mu_w")
+    assert_close(dw[1].cpu().numpy(), ref_dw[1], "delta_var_w")
 
 
 def test_conv2d_stencil_kernels_agree_with_the_table_path():
@@ -164,9 +170,14 @@ def test_conv2d_stencil_kernels_agree_with_the_table_path():
                              ti["Fmwa_2"], wi * wi, fo, wi * wi, fi, k, B)
             dz = F.conv2d_bwd_dz(t["mu_w"], t["jcb"], t["delta_mu"], t["delta_var"], ti["FCzwa_1"],
                                  ti["Szz_ud"], wi * wi, fo, wi * wi, fi, k, idx["h"], B)
-            out[mode] = [x.cpu().numpy() for x in (*z, *dz)]
+            dw = F.conv2d_bwd_dw(t["var_w"], t["var_b"], t["mu_a"], t["delta_mu"], t["delta_var"],
+                                 ti["Fmwa_2"], B, fo, wi * wi, wi * wi, fi, k)
+            out[mode] = [x.cpu().numpy() for x in (*z, *dz, *dw[:2])]
     finally:
         capi.tune("conv2d.stencil", 1)
-    for name, a, b in zip(("mu_z", "var_z", "delta_mu_z", "delta_var_z"), out[1], out[0]):
+    for name, a, b in zip(("mu_z", "var_z", "delta_mu_z", "delta_var_z", "delta_mu_w",
+                           "delta_var_w"), out[1], out[0]):
         assert_close(a, b, name)
-        assert not np.array_equal(a, b) or name == "", "both modes ran the same kernel?"
+        # the two paths sum in different orders: identical bits would mean that the
+        # switch did not switch
+        assert not np.array_equal(a, b), name
