@@ -183,6 +183,7 @@ int tagi_hip_tune(const char *key, int value) {
     else if (!strcmp(key, "conv2d.tile")) g_tune.conv_tile = value;
     else if (!strcmp(key, "conv2d.group_loads")) g_conv2d_group_loads = value;
     else if (!strcmp(key, "conv2d.stencil")) g_conv2d_stencil = value;
+    else if (!strcmp(key, "conv2d.phase_order")) g_conv2d_phase_order = value;
     else if (!strcmp(key, "linear.tile")) g_tune.tile = value;
     else if (!strcmp(key, "conv2d.dw.splits")) g_tune.conv_dw_splits = value;
     else if (!strcmp(key, "linear.gemv.swizzle")) g_tune.gemv_swz = value;
@@ -393,7 +394,7 @@ int tagi_linear_bwd(const float *mu_w, const float *var_w, const float *var_b, c
 static bool conv_sizes_ok(int B, int fo, int woho, int fi, int wihi, int ki) {
     const long long lim = 0x7fffffffLL;
     return (long long)B * fo * woho < lim && (long long)B * fi * wihi < lim &&
-           (long long)ki * ki * fi * fo < lim && (long long)ki * ki * (128 + 32) * 4 + 16 <= 64 * 1024;
+           (long long)ki * ki * fi * fo < lim && (long long)ki * ki * (128 + 32 + 1) * 4 + 48 <= 64 * 1024;
 }
 
 int tagi_conv2d_out_size(int kernel, int stride, int wi, int hi, int pad, int pad_type, int *wo,

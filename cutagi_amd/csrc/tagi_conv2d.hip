@@ -35,6 +35,9 @@ struct ConvParams {
     int M, N, R, splits, r_per_split;
     float *ws0, *ws1;
     int group_loads;  // 0: never use the sixteen-byte group loads
+    // states: column order. perm_s > 1 numbers the input pixels phase by phase
+    // ((y mod s, x mod s) major, then image, then pixel) on maps of width perm_w.
+    int perm_s, perm_w;
 };
 
 // All operand loads below are unconditional: an element outside the problem (or
@@ -61,6 +64,8 @@ struct GatherCtx {
     int fast;      // wave-uniform: all groups of this tile are consecutive
     int ymask[4];  // per column slot: which of the four loaded values are real
     int xok[2];    // per row slot: the loaded values are real
+    int taps;      // states: taps that reach any column of this tile (rows of tab)
+    const int *act;  // states: their tap numbers
 };
 
 __device__ __forceinline__ float4 keep_masked(const float4 &v, int mask) {
@@ -71,13 +76,14 @@ __device__ __forceinline__ float4 keep_masked(const float4 &v, int mask) {
 typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
 
 // Second half of the prologue: tab[t*bn + c] is complete (a barrier was passed).
-// `pix` = pixels per image of the column index, `src_pix` = elements per channel
+// image_of(n) = image of column n, `src_pix` = elements per channel
 // map of the gathered tensor, B = images. A group whose 16-byte window could leave
 // the tensor (it starts before the first element of image 0 or ends after the
 // last element of image B-1) makes the whole tile gather element by element.
+template <class ImageOf>
 __device__ __forceinline__ void build_group_table(GatherCtx &ctx, int *tab, int k2, int bn, int n0,
-                                                  int N, int pix, int src_pix, int B, int tid,
-                                                  int nthreads, int allow) {
+                                                  int N, ImageOf image_of, int src_pix, int B,
+                                                  int tid, int nthreads, int allow) {
     int *qtab = tab + k2 * bn, *flag = qtab + k2 * (bn / 4);
     if (tid == 0) *flag = (allow && src_pix >= 4) ? 0 : 1;
     __syncthreads();
@@ -97,8 +103,8 @@ __device__ __forceinline__ void build_group_table(GatherCtx &ctx, int *tab, int 
         for (int j = 0; j < 4; j++)
             if (o[j] >= 0 && o[j] != base + j) ok = false;
         if (mask != 0) {
-            const int b = n / pix;
-            if (n + 3 >= N || b != (n + 3) / pix) ok = false;
+            const int b = image_of(n);
+            if (n + 3 >= N || b != image_of(n + 3)) ok = false;
             if (b == 0 && base < 0) ok = false;
             if (b == B - 1 && base + 3 > src_pix - 1) ok = false;
         }
@@ -174,6 +180,7 @@ struct ConvFwdProblem {
     using Ctx = GatherCtx;
     static constexpr bool XK = true, YK = false, PROLOGUE_WRITES_LDS = true, SPLIT_PER_XCD = false;
     static constexpr int VARIANTS = 2;  // 1: sixteen-byte loads of consecutive groups
+    __device__ static __forceinline__ void adjust_range(const Params &, const Ctx &, int &, int &) {}
     // 130 registers without the request: one 64x128 workgroup per CU instead of two
     static constexpr int min_waves_per_simd(int bm, int bn, int waves) {
         return waves == 8 && bm * bn <= 64 * 128 ? 4 : 0;
@@ -202,8 +209,9 @@ struct ConvFwdProblem {
             ctx.img[j] = n0 + row + j < p.N ? ((n0 + row + j) / p.woho) * p.fi * p.wihi : 0;
         ctx.bn = bn;
         ctx.tab = tab;
-        build_group_table(ctx, tab, p.k2, bn, n0, p.N, p.woho, p.wihi, p.B, tid, nthreads,
-                          p.group_loads);
+        build_group_table(
+            ctx, tab, p.k2, bn, n0, p.N, [&](int n) { return n / p.woho; }, p.wihi, p.B, tid,
+            nthreads, p.group_loads);
     }
     __device__ static __forceinline__ void next_tile(const Params &, Ctx &) {}
     __device__ static __forceinline__ float4 fix_x(const Ctx &ctx, int i, const float4 &v) {
@@ -252,6 +260,7 @@ struct ConvDwProblem {
     };
     static constexpr bool XK = true, YK = true, PROLOGUE_WRITES_LDS = false, SPLIT_PER_XCD = true;
     static constexpr int VARIANTS = 1;
+    __device__ static __forceinline__ void adjust_range(const Params &, const Ctx &, int &, int &) {}
     static constexpr int min_waves_per_simd(int, int, int) { return 0; }
     static constexpr int NX = 2, NY = 1, FLAVOR = FLAVOR_DELTA_ROWS;
 
@@ -358,6 +367,7 @@ struct ConvDwVecProblem {
     };
     static constexpr bool XK = true, YK = true, PROLOGUE_WRITES_LDS = false, SPLIT_PER_XCD = true;
     static constexpr int VARIANTS = 1;
+    __device__ static __forceinline__ void adjust_range(const Params &, const Ctx &, int &, int &) {}
     // (asking for four or five 64x64 workgroups per CU instead of three measured
     // no gain)
     static constexpr int min_waves_per_simd(int, int, int) { return 0; }
@@ -453,6 +463,35 @@ struct ConvDwVecProblem {
 // The reference's FCzwa_1 / Szz_ud pair lists, per input pixel, the (tap, output
 // pixel) occurrences; the prologue re-keys the lists of the tile's pixels by tap
 // (each tap meets a pixel at most once), which is the table gather_cols wants.
+//
+// A strided convolution reaches an input pixel through few of its taps, and which
+// ones depends on the pixel's phase (y mod s, x mod s): a 3x3 stride-2 kernel
+// touches a pixel through 4, 2, 2 or 1 of its 9 taps. Summing over all taps would
+// multiply three zeros for every product. So the columns can be numbered phase
+// by phase (ConvParams::perm_s), which makes the pixels of a tile share their
+// taps, and every tile reduces over the taps that reach any of ITS columns only:
+// the prologue finds them in the table, whatever the table holds, and keeps one
+// table row per such tap. The numbering only decides which pixels sit together;
+// results do not depend on it.
+struct DzColumn {
+    int b, px;
+};
+__device__ __forceinline__ DzColumn dz_column(const ConvParams &p, int n) {
+    DzColumn c;
+    if (p.perm_s <= 1) {
+        c.b = n / p.wihi;
+        c.px = n - c.b * p.wihi;
+        return c;
+    }
+    const int s = p.perm_s, W = p.perm_w, ws = W / s;
+    const int per_img = p.wihi / (s * s), per_phase = p.B * per_img;
+    const int phase = n / per_phase, rem = n - phase * per_phase;
+    c.b = rem / per_img;
+    const int l = rem - c.b * per_img, ly = l / ws, lx = l - ly * ws;
+    c.px = (ly * s + phase / s) * W + lx * s + phase % s;
+    return c;
+}
+
 struct ConvDzProblem {
     using Params = ConvParams;
     using Ctx = GatherCtx;
@@ -462,30 +501,68 @@ struct ConvDzProblem {
     __device__ static __forceinline__ bool variant(const Ctx &ctx) { return ctx.fast != 0; }
     static constexpr int NX = 1, NY = 2, FLAVOR = FLAVOR_DELTA_COLS;
 
+    // [k2][bn] offsets, [k2][bn/4] groups + flag, tap mask, [k2] active taps
     static size_t extra_lds_bytes(const Params &p, int, int bn) {
-        return ((size_t)p.k2 * bn + (size_t)p.k2 * (bn / 4) + 4) * sizeof(int);
+        return ((size_t)p.k2 * bn + (size_t)p.k2 * (bn / 4) + 4 + 4 + p.k2) * sizeof(int);
     }
     __device__ static __forceinline__ void prologue(const Params &p, Ctx &ctx, int *tab, int tid,
                                                     int nthreads, int, int n0, int, int bn, int,
                                                     int) {
-        for (int e = tid; e < p.k2 * bn; e += nthreads) tab[e] = -1;
+        int *mask = tab + p.k2 * bn + p.k2 * (bn / 4) + 4, *act = mask + 4;
+        // pass 1: which taps reach a column of this tile (more than 32 taps: all)
+        if (tid == 0) *mask = p.k2 > 32 ? -1 : 0;
         __syncthreads();
+        if (p.k2 <= 32) {
+            int seen = 0;
+            for (int e = tid; e < p.nr * bn; e += nthreads) {
+                const int j = e / bn, c = e - j * bn, n = n0 + c;
+                if (n >= p.N) continue;
+                const int px = dz_column(p, n).px;
+                const int tap = p.idx[px * p.nr + j], o = p.idx2[j * p.wihi + px];
+                if (o > -1 && tap >= 1 && tap <= p.k2) seen |= 1 << (tap - 1);
+            }
+            if (seen) atomicOr(mask, seen);
+        }
+        __syncthreads();
+        const int m = *mask;
+        const int taps = p.k2 > 32 ? p.k2 : __popc(m);
+        for (int t = tid; t < p.k2; t += nthreads) {
+            if (p.k2 > 32)
+                act[t] = t;
+            else if (m >> t & 1)
+                act[__popc(m & ((1 << t) - 1))] = t;
+        }
+        for (int e = tid; e < taps * bn; e += nthreads) tab[e] = -1;
+        __syncthreads();
+        // pass 2: one table row per such tap
         for (int e = tid; e < p.nr * bn; e += nthreads) {
             const int j = e / bn, c = e - j * bn, n = n0 + c;
-            if (n < p.N) {
-                const int px = n % p.wihi;
-                const int tap = p.idx[px * p.nr + j], o = p.idx2[j * p.wihi + px];
-                if (o > -1 && tap >= 1 && tap <= p.k2) tab[(tap - 1) * bn + c] = o - 1;
+            if (n >= p.N) continue;
+            const int px = dz_column(p, n).px;
+            const int tap = p.idx[px * p.nr + j], o = p.idx2[j * p.wihi + px];
+            if (o > -1 && tap >= 1 && tap <= p.k2) {
+                const int row = p.k2 > 32 ? tap - 1 : __popc(m & ((1 << (tap - 1)) - 1));
+                tab[row * bn + c] = o - 1;
             }
         }
         const int row = (tid % (bn / 4)) * 4;
 #pragma unroll
         for (int j = 0; j < 4; j++)
-            ctx.img[j] = n0 + row + j < p.N ? ((n0 + row + j) / p.wihi) * p.fo * p.woho : 0;
+            ctx.img[j] = n0 + row + j < p.N ? dz_column(p, n0 + row + j).b * p.fo * p.woho : 0;
         ctx.bn = bn;
         ctx.tab = tab;
-        build_group_table(ctx, tab, p.k2, bn, n0, p.N, p.wihi, p.woho, p.B, tid, nthreads,
-                          p.group_loads);
+        ctx.taps = taps;
+        ctx.act = act;
+        build_group_table(
+            ctx, tab, taps, bn, n0, p.N, [&](int n) { return dz_column(p, n).b; }, p.woho, p.B, tid,
+            nthreads, p.group_loads);
+    }
+    // The slice [r_begin, r_end) was cut in units of k2 (whole output channels);
+    // with `taps` rows per channel it becomes this.
+    __device__ static __forceinline__ void adjust_range(const Params &p, const Ctx &ctx,
+                                                        int &r_begin, int &r_end) {
+        r_begin = (r_begin / p.k2) * ctx.taps;
+        r_end = (r_end / p.k2) * ctx.taps;
     }
     __device__ static __forceinline__ void next_tile(const Params &, Ctx &) {}
     __device__ static __forceinline__ float4 fix_x(const Ctx &ctx, int i, const float4 &v) {
@@ -498,17 +575,17 @@ struct ConvDzProblem {
                                                     int row, int r, int r_end) {
         const int m = m0 + row;
         const bool row_ok = m < p.M;
-        const int rr = min(r, p.R - 1);
-        int f = rr / p.k2, t = rr - f * p.k2;
+        const int rr = min(r, max(p.fo * ctx.taps - 1, 0));
+        int f = ctx.taps ? rr / ctx.taps : 0, ti = rr - f * ctx.taps;
         float c[4];
         int mask = 0;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const bool ok = row_ok && r + j < r_end;
             mask |= ok ? (1 << j) : 0;
-            c[j] = p.w0[ok ? ((size_t)f * p.fi + m) * p.k2 + t : 0];
-            if (++t == p.k2) {
-                t = 0;
+            c[j] = p.w0[ok ? ((size_t)f * p.fi + m) * p.k2 + ctx.act[ti] : 0];
+            if (++ti >= ctx.taps) {
+                ti = 0;
                 f++;
             }
         }
@@ -517,12 +594,13 @@ struct ConvDzProblem {
     }
     __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &ctx, int V, int arr, int i,
                                                     int, int row, int r, int r_end) {
-        return gather_cols(arr ? p.d1 : p.d0, ctx, V, i, row, r, r_end, p.R, p.k2, p.woho);
+        return gather_cols(arr ? p.d1 : p.d0, ctx, V, i, row, r, r_end,
+                           max(p.fo * ctx.taps, 1), max(ctx.taps, 1), p.woho);
     }
     __device__ static __forceinline__ void store(const Params &p, int m, int n, float a0,
                                                  float a1) {
-        const int b = n / p.wihi, px = n - b * p.wihi;
-        const size_t at = ((size_t)b * p.fi + m) * p.wihi + px;
+        const DzColumn c = dz_column(p, n);
+        const size_t at = ((size_t)c.b * p.fi + m) * p.wihi + c.px;
         const float e = p.e0[at];
         p.out0[at] = a0 * e;
         p.out1[at] = a1 * e * e;
@@ -612,10 +690,21 @@ namespace {
 // `stencil`: map width when the regular-stencil kernel applies (slices are then
 // whole groups of 32 channels: a multiple of its 72-step and of the table-driven
 // loop's 32-step k-tile), 0 otherwise.
+inline int lcm_int(int a, int b) {
+    int x = a, y = b;
+    while (y) {
+        const int t = x % y;
+        x = y;
+        y = t;
+    }
+    return a / x * b;
+}
+
 template <class P, bool DZ>
 hipError_t run_sliced(int tile, int splits, int stencil, float *ws0, float *ws1, ConvParams &p,
                       hipStream_t stream) {
-    const int unit = stencil ? 288 : KT;
+    // the state backward re-states its slices per tile in whole output channels
+    const int unit = stencil ? 288 : DZ ? lcm_int(KT, p.k2) : KT;
     const int per = ceil_div(ceil_div(p.R, splits), unit) * unit;
     p.splits = ceil_div(p.R, per);
     p.r_per_split = per;
@@ -630,6 +719,7 @@ hipError_t run_sliced(int tile, int splits, int stencil, float *ws0, float *ws1,
 
 int g_conv2d_group_loads = 1;
 int g_conv2d_stencil = 1;
+int g_conv2d_phase_order = 1;
 
 hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
                              const float *var_b, const float *mu_a, const float *var_a,
@@ -665,6 +755,18 @@ hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float
     p.woho = woho; p.fo = fo; p.wihi = wihi; p.fi = fi; p.k2 = k2; p.B = B; p.nr = nr;
     p.M = fi; p.N = B * wihi; p.R = k2 * fo;
     p.group_loads = g_conv2d_group_loads;
+    // strided convolution on a square map: number the columns phase by phase
+    p.perm_s = 1;
+    p.perm_w = 0;
+    if (g_conv2d_phase_order && wihi > woho && wihi % woho == 0) {
+        int s = 1, w = 1;
+        while (s * s < wihi / woho) s++;
+        while (w * w < wihi) w++;
+        if (s * s == wihi / woho && w * w == wihi && w % s == 0) {
+            p.perm_s = s;
+            p.perm_w = w;
+        }
+    }
     int stencil = 0;
     if (g_conv2d_stencil && ki == 3 && nr == 9 && woho == wihi && fo % 8 == 0 && fi % 64 == 0 &&
         tile == TILE_64x128 && aligned16(mu_w) && aligned16(dmu) && aligned16(dvar))

@@ -286,9 +286,11 @@ void conv_stencil_kernel(ConvParams p) {
     typename P::Ctx ctx;
     P::prologue(p, ctx, lds_extra, threadIdx.x, 512, m0, n0, 64, 128, r_begin, r_end);
     __syncthreads();
+    int r_lo = r_begin, r_hi = r_end;
+    P::adjust_range(p, ctx, r_lo, r_hi);
     mfma_tile_body<P, 64, 128, 2, 4, 0>(p, ctx, reinterpret_cast<float (*)[XF]>(lds),
                                         reinterpret_cast<float (*)[YF]>(lds + P::NX * XF), m0, n0,
-                                        split, r_begin, r_end);
+                                        split, r_lo, r_hi);
 }
 
 // Map width for which the stencil kernel exists, 0 otherwise (pixels = width^2).

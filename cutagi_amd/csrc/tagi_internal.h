@@ -133,6 +133,8 @@ void conv2d_plan(int M, int N, int R, int *tile, int *splits);
 extern int g_conv2d_group_loads;
 // 0 switches the regular-stencil kernels of the conv2d forward / state backward off.
 extern int g_conv2d_stencil;
+// 0 keeps the natural column order in the conv2d state backward of strided layers.
+extern int g_conv2d_phase_order;
 
 hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
                              const float *var_b, const float *mu_a, const float *var_a,

@@ -29,6 +29,9 @@
 //                               runs once before the first load; a barrier follows
 //   min_waves_per_simd(BM, BN, waves)
 //                               occupancy the register allocation must allow (0: none)
+//   adjust_range(p, ctx, r_begin, r_end)
+//                               after the prologue: a problem whose reduction is shorter
+//                               for this tile than for others re-states its slice
 //   VARIANTS, variant(ctx)      number of loader variants (1 or 2) and, after the
 //                               prologue, which one this workgroup uses (uniform)
 //   load_x(p, ctx, V, arr, i, m0, row, r, r_end)
@@ -334,14 +337,15 @@ void mfma_tile_kernel(typename P::Params p) {
     typename P::Ctx ctx;
     P::prologue(p, ctx, lds_extra, threadIdx.x, NT, m0, n0, BM, BN, r_begin, r_end);
     if (P::PROLOGUE_WRITES_LDS) __syncthreads();
+    int r_lo = r_begin, r_hi = r_end;
+    P::adjust_range(p, ctx, r_lo, r_hi);
     if constexpr (P::VARIANTS > 1) {
         if (P::variant(ctx)) {
-            mfma_tile_body<P, BM, BN, WM, WN, 1>(p, ctx, lds_x, lds_y, m0, n0, split, r_begin,
-                                                 r_end);
+            mfma_tile_body<P, BM, BN, WM, WN, 1>(p, ctx, lds_x, lds_y, m0, n0, split, r_lo, r_hi);
             return;
         }
     }
-    mfma_tile_body<P, BM, BN, WM, WN, 0>(p, ctx, lds_x, lds_y, m0, n0, split, r_begin, r_end);
+    mfma_tile_body<P, BM, BN, WM, WN, 0>(p, ctx, lds_x, lds_y, m0, n0, split, r_lo, r_hi);
 }
 
 

@@ -181,3 +181,27 @@ def test_conv2d_stencil_kernels_agree_with_the_table_path():
         # the two paths sum in different orders: identical bits would mean that the
         # switch did not switch
         assert not np.array_equal(a, b), name
+
+
+@pytest.mark.parametrize("geom", [(3, 2, 1, 2, 16, 16, 64, 4), (2, 2, 0, 1, 8, 64, 32, 3),
+                                  (3, 2, 1, 2, 4, 8, 8, 2)])
+def test_conv2d_state_backward_column_orders_agree(oracle_lib, geom):
+    """Strided layers: columns numbered phase by phase (default) and in natural
+    order give the oracle's result both; the order only decides which taps a tile
+    can skip."""
+    import cutagi_amd.functional as F
+    from cutagi_amd import capi
+    k, s, p, pt, wi, fi, fo, B = geom
+    idx, d, t, ti, wihi, woho = _setup(oracle_lib, geom, False, seed=7)
+    ref = oracle_lib.conv2d_bwd_dz(d["mu_w"], d["jcb"], d["delta_mu"], d["delta_var"],
+                                   idx["FCzwa_1"], idx["Szz_ud"], woho, fo, wihi, fi, k, idx["h"],
+                                   B, threads=4)
+    try:
+        for mode in (1, 0):
+            capi.tune("conv2d.phase_order", mode)
+            dz = F.conv2d_bwd_dz(t["mu_w"], t["jcb"], t["delta_mu"], t["delta_var"], ti["FCzwa_1"],
+                                 ti["Szz_ud"], woho, fo, wihi, fi, k, idx["h"], B)
+            assert_close(dz[0].cpu().numpy(), ref[0], "delta_mu_z order %d" % mode)
+            assert_close(dz[1].cpu().numpy(), ref[1], "delta_var_z order %d" % mode)
+    finally:
+        capi.tune("conv2d.phase_order", 1)
