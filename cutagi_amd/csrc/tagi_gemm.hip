@@ -42,8 +42,22 @@ __device__ __forceinline__ float4 load4(const float *__restrict__ base, int ld, 
     return v;
 }
 
-template <int MODE, bool VEC>
+// The same for a problem whose every k-tile is complete (reduction length and
+// slices are multiples of the k-tile, 16-byte rows): nothing to mask along the
+// reduction, and a row beyond the matrix is read from its last row instead -- its
+// sums land in accumulator rows that the epilogue never stores. No branch and no
+// zero fill around the load.
+template <bool KC>
+__device__ __forceinline__ float4 load4_full(const float *__restrict__ base, int ld, int row,
+                                             int rows, int r) {
+    const int rr = min(row, rows - (KC ? 1 : 4));
+    const float *q = KC ? base + (size_t)rr * ld + r : base + (size_t)r * ld + rr;
+    return *reinterpret_cast<const float4 *>(q);
+}
+
+template <int MODE, bool VEC, bool FULL = false>
 struct LinearProblem {
+    static_assert(VEC || !FULL, "complete k-tiles are a case of the 16-byte path");
     using Params = GemmParams;
     static constexpr bool XK = (MODE != GEMM_DW);
     static constexpr bool YK = (MODE == GEMM_FWD);
@@ -65,10 +79,12 @@ struct LinearProblem {
 
     __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &, int, int arr, int, int m0,
                                                     int row, int r, int r_end) {
+        if (FULL) return load4_full<XK>(arr ? p.x1 : p.x0, p.ldx, m0 + row, p.M, r);
         return load4<XK, VEC>(arr ? p.x1 : p.x0, p.ldx, m0 + row, p.M, r, r_end);
     }
     __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &, int, int arr, int, int n0,
                                                     int row, int r, int r_end) {
+        if (FULL) return load4_full<YK>(arr ? p.y1 : p.y0, p.ldy, n0 + row, p.N, r);
         return load4<YK, VEC>(arr ? p.y1 : p.y0, p.ldy, n0 + row, p.N, r, r_end);
     }
     __device__ static __forceinline__ void store(const Params &p, int m, int n, float a0,
@@ -144,6 +160,9 @@ __global__ __launch_bounds__(64) void reduce_splits_kernel(const float *__restri
 
 template <int MODE>
 hipError_t launch_mode(int tile, bool vec, const GemmParams &p, hipStream_t stream) {
+    const bool full = vec && p.R % KT == 0 && (p.splits == 1 || p.r_per_split % KT == 0) &&
+                      p.M >= 4 && p.N >= 4;
+    if (full) return launch_tiles<LinearProblem<MODE, true, true>>(tile, p, stream);
     if (vec) return launch_tiles<LinearProblem<MODE, true>>(tile, p, stream);
     return launch_tiles<LinearProblem<MODE, false>>(tile, p, stream);
 }
