@@ -220,7 +220,7 @@ struct ConvFwdProblem {
     __device__ static __forceinline__ float4 fix_y(const Ctx &ctx, int i, const float4 &v) {
         return keep_masked(v, ctx.ymask[i]);
     }
-    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &ctx, int V, int arr, int i,
+    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &ctx, int, int arr, int i,
                                                     int m0, int row, int r, int r_end) {
         return load_rows_kc<VEC>(arr ? p.w1 : p.w0, p.R, m0 + row, p.M, r, r_end, &ctx.xok[i]);
     }
@@ -298,7 +298,7 @@ struct ConvDwProblem {
     __device__ static __forceinline__ void next_tile(const Params &, Ctx &) {}
     __device__ static __forceinline__ float4 fix_x(const Ctx &, int, const float4 &v) { return v; }
     __device__ static __forceinline__ float4 fix_y(const Ctx &, int, const float4 &v) { return v; }
-    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &, int V, int arr, int, int m0,
+    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &, int, int arr, int, int m0,
                                                     int row, int r, int r_end) {
         const float *__restrict__ d = arr ? p.d1 : p.d0;
         const int m = m0 + row;
@@ -325,7 +325,7 @@ struct ConvDwProblem {
         }
         return make_float4(c[0], c[1], c[2], c[3]);
     }
-    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &ctx, int V, int, int i, int,
+    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &ctx, int, int, int i, int,
                                                     int, int r, int r_end) {
         float c[4];
 #pragma unroll
@@ -415,7 +415,7 @@ struct ConvDwVecProblem {
             ctx.xoff += (p.fo - 1) * p.woho;
         }
     }
-    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &ctx, int V, int arr, int i, int,
+    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &ctx, int, int arr, int i, int,
                                                     int, int r, int r_end) {
         const bool ok = r < r_end && ctx.xrow[i] >= 0;
         const float *__restrict__ d = arr ? p.d1 : p.d0;
@@ -428,7 +428,7 @@ struct ConvDwVecProblem {
     __device__ static __forceinline__ float4 fix_y(const Ctx &ctx, int i, const float4 &v) {
         return keep_masked(v, ctx.ymask[i]);
     }
-    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &ctx, int V, int, int i, int,
+    __device__ static __forceinline__ float4 load_y(const Params &p, Ctx &ctx, int, int, int i, int,
                                                     int, int r, int r_end) {
         const bool live = r < r_end && ctx.cb[i] >= 0;
         const int base = ctx.img + ctx.cb[i] - 1;
@@ -571,7 +571,7 @@ struct ConvDzProblem {
     __device__ static __forceinline__ float4 fix_y(const Ctx &ctx, int i, const float4 &v) {
         return keep_masked(v, ctx.ymask[i]);
     }
-    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &ctx, int V, int, int i, int m0,
+    __device__ static __forceinline__ float4 load_x(const Params &p, Ctx &ctx, int, int, int i, int m0,
                                                     int row, int r, int r_end) {
         const int m = m0 + row;
         const bool row_ok = m < p.M;

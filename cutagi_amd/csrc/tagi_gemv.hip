@@ -572,10 +572,10 @@ __global__ __launch_bounds__(256) void gemv_dw_kernel(
 
 }  // namespace
 
-// Forward variants (row groups per wave, chunks per stage), by index.
+// Forward variants by index: row groups per wave (their chunks per stage are
+// 1, 2, 2, 4: see the launcher's switch).
 constexpr int FWD_VARIANTS = 4;
 static const int kFwdRG[FWD_VARIANTS] = {2, 2, 1, 1};
-static const int kFwdC[FWD_VARIANTS] = {1, 2, 2, 4};
 
 int gemv_fwd_variants() { return FWD_VARIANTS; }
 int gemv_fwd_rows_per_block(int variant) { return FWD_WAVES * kFwdRG[variant] * 4; }

@@ -307,10 +307,8 @@ __global__ __launch_bounds__(WM *WN * 64)
 __attribute__((amdgpu_waves_per_eu(tile_min_waves<P>(BM, BN, WM * WN))))
 void mfma_tile_kernel(typename P::Params p) {
     constexpr bool XK = P::XK, YK = P::YK;
-    constexpr int NX = P::NX, NY = P::NY, FL = P::FLAVOR;
+    constexpr int NX = P::NX, NY = P::NY;
     constexpr int NT = WM * WN * 64;
-    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
-    constexpr int XS = TileGeom<XK, BM>::stride, YS = TileGeom<YK, BN>::stride;
     constexpr int XF = TileGeom<XK, BM>::floats, YF = TileGeom<YK, BN>::floats;
     constexpr int LX = BM * KT / 4 / NT, LY = BN * KT / 4 / NT;
     static_assert(LX >= 1 && LY >= 1, "tile too small for the thread count");
