@@ -1,0 +1,81 @@
+"""The pytagi.nn-shaped Python layer (cutagi_amd.nn): construction and field
+access without a GPU; on the GPU the README training loop of the reference
+(README.md:28-57, the MLP of config 1) gives exactly what the same calls on the
+C++ module give -- the wrappers add no arithmetic."""
+import numpy as np
+import pytest
+
+
+def test_wrappers_build_and_forward_fields():
+    from cutagi_amd import cutagi
+    from cutagi_amd.nn import (AvgPool2d, BatchNorm2d, Conv2d, LayerBlock, Linear, MixtureReLU,
+                               OutputUpdater, ReLU, ResNetBlock, Sequential, Utils)
+    cutagi.manual_seed(0)
+    lin = Linear(784, 128)
+    assert lin.get_layer_info() == "Linear(784,128)" and lin.input_size == 784
+    assert len(lin.mu_w) == 784 * 128
+    lin.mu_b = [0.0] * 128                       # writes through to the C++ layer
+    assert lin._cpp_backend.mu_b == [0.0] * 128
+    net = Sequential(lin, ReLU(), Linear(128, 128), ReLU(), Linear(128, 11))
+    assert net.get_layer_stack_info().split() == ["Linear(784,128)", "ReLU()", "Linear(128,128)",
+                                                  "ReLU()", "Linear(128,11)"]
+    assert net.device == "cpu" and net.z_buffer_size == 784
+    net.input_state_update = True
+    assert net._cpp_backend.input_state_update is True
+    assert sorted(net.state_dict()) == ["Linear.0", "Linear.2", "Linear.4"]
+    block = ResNetBlock(LayerBlock(Conv2d(4, 8, 3, bias=False, stride=2, padding=1, padding_type=2),
+                                   MixtureReLU(), BatchNorm2d(8)),
+                        LayerBlock(Conv2d(4, 8, 2, bias=False, stride=2)))
+    cnn = Sequential(Conv2d(3, 4, 3, bias=False, padding=1, in_width=8, in_height=8),
+                     BatchNorm2d(4), MixtureReLU(), block, AvgPool2d(4), Linear(8, 5))
+    assert "ResNetBlock" in cnn.get_layer_stack_info()
+    obs, idx, n_obs = Utils().label_to_obs(np.array([3, 0]), 10)
+    assert n_obs == 4 and obs.tolist() == [1, 1, -1, -1, 1, 1, 1, 1]
+    assert idx.tolist() == [1, 2, 4, 8, 1, 2, 4, 7] and idx.dtype == np.int32
+    with pytest.raises(RuntimeError, match="GPU only"):
+        net(np.zeros((2, 784), np.float32))
+    with pytest.raises(NotImplementedError):
+        OutputUpdater("cpu").update_heteros(None, None, None)
+
+
+@pytest.mark.gpu
+def test_readme_training_loop_matches_the_cpp_module():
+    from cutagi_amd import cutagi
+    from cutagi_amd.nn import Linear, OutputUpdater, ReLU, Sequential, Utils
+    batch_size, steps = 32, 3
+    rng = np.random.default_rng(0)
+    xs = rng.normal(0, 1, (steps, batch_size, 784)).astype(np.float32)
+    labels = rng.integers(0, 10, (steps, batch_size))
+    var_y = np.full((batch_size * 4,), 1.0, dtype=np.float32)
+
+    cutagi.manual_seed(0)
+    net = Sequential(Linear(784, 128), ReLU(), Linear(128, 128), ReLU(), Linear(128, 11))
+    net.to_device("cuda")
+    udt = OutputUpdater(net.device)
+    preds = []
+    for i in range(steps):
+        y, idx, _ = Utils().label_to_obs(labels[i], 10)
+        m_pred, v_pred = net(xs[i])
+        udt.update_using_indices(net.output_z_buffer, y, var_y, idx, net.input_delta_z_buffer)
+        net.backward()
+        net.step()
+        preds.append((m_pred, v_pred))
+    assert preds[0][0].shape == (batch_size * 11,) and np.all(preds[-1][1] > 0)
+    assert not np.array_equal(preds[0][0], preds[-1][0])
+
+    cutagi.manual_seed(0)
+    raw = cutagi.Sequential([cutagi.Linear(784, 128), cutagi.ReLU(), cutagi.Linear(128, 128),
+                             cutagi.ReLU(), cutagi.Linear(128, 11)])
+    raw.to_device("cuda")
+    upd = cutagi.OutputUpdater(raw.device)
+    for i in range(steps):
+        y, idx, _ = Utils().label_to_obs(labels[i], 10)
+        raw.forward(xs[i])
+        m, v = raw.get_outputs()
+        assert np.array_equal(m, preds[i][0]) and np.array_equal(v, preds[i][1])
+        upd.update_using_indices(raw.output_z_buffer, y.tolist(), var_y.tolist(), idx.tolist(),
+                                 raw.input_delta_z_buffer)
+        raw.backward()
+        raw.step()
+    a, b = net.state_dict(), raw.state_dict()
+    assert a.keys() == b.keys() and all(a[k] == b[k] for k in a)
