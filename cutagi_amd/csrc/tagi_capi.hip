@@ -491,9 +491,11 @@ int tagi_conv2d_bwd_dw(const float *var_w, const float *var_b, const float *mu_a
         ceil_div(fo, gemm_tile_rows(tile)) * ceil_div(ki * ki * fi, gemm_tile_cols(tile));
     // (three full rounds of resident workgroups: a partly filled last round
     // costs as much time as a full one)
-    int splits = g_tune.conv_dw_splits > 0
-                     ? g_tune.conv_dw_splits
-                     : 3 * conv2d_bwd_dw_blocks_per_cu(tile) * NUM_CU / out_tiles;
+    const bool stencil = conv2d_bwd_dw_stencil(mu_a, delta_mu_out, delta_var_out, B, fo, woho, wihi,
+                                               fi, ki, tile) != 0;
+    int splits = g_tune.conv_dw_splits > 0 ? g_tune.conv_dw_splits
+                 : stencil                 ? conv2d_bwd_dw_stencil_splits(out_tiles)
+                                           : 3 * conv2d_bwd_dw_blocks_per_cu(tile) * NUM_CU / out_tiles;
     const int max_splits = ceil_div(red, 256);
     if (splits > max_splits) splits = max_splits;
     if (splits < 1) splits = 1;

@@ -805,6 +805,38 @@ int conv2d_bwd_dw_blocks_per_cu(int tile) {
     return cached[tile];
 }
 
+// Map width when the weight backward runs on the regular-stencil kernel (3x3,
+// stride 1, "same" padding on a square map -- the kernel verifies the table; 64 x 64
+// tiles of whole channels, slices of whole 64-pixel k-tiles), 0 otherwise.
+int conv2d_bwd_dw_stencil(const float *mu_a, const float *dmu, const float *dvar, int B, int fo,
+                          int woho, int wihi, int fi, int ki, int tile) {
+    if (!g_conv2d_stencil || ki != 3 || woho != wihi || woho % 4 != 0 || fi % 64 != 0 ||
+        fo % 64 != 0 || ((long long)B * woho) % 64 != 0 || tile != TILE_64x64 ||
+        !aligned16(mu_a) || !aligned16(dmu) || !aligned16(dvar))
+        return 0;
+    return stencil_width(wihi);
+}
+
+// Reduction slices for the stencil kernel (two 8-wave workgroups per CU): the
+// fewest rounds of resident workgroups that are at least 95 % full, else the
+// fullest of up to four rounds. A partly filled round costs as much as a full one.
+int conv2d_bwd_dw_stencil_splits(int out_tiles) {
+    const int resident = 2 * NUM_CU;
+    int best = 1;
+    double best_fill = 0.0;
+    for (int rounds = 1; rounds <= 4; rounds++) {
+        const int s = rounds * resident / out_tiles;
+        if (s < 1) continue;
+        const double fill = (double)out_tiles * s / (rounds * resident);
+        if (fill >= 0.95) return s;
+        if (fill > best_fill) {
+            best_fill = fill;
+            best = s;
+        }
+    }
+    return best;
+}
+
 hipError_t launch_conv2d_bwd_dw(const float *var_w, const float *mu_a, const float *dmu,
                                 const float *dvar, const int *aidx, int B, int fo, int woho,
                                 int wihi, int fi, int ki, int tile, int splits, float *ws0, float *ws1,
@@ -815,12 +847,7 @@ hipError_t launch_conv2d_bwd_dw(const float *var_w, const float *mu_a, const flo
     p.woho = woho; p.fo = fo; p.wihi = wihi; p.fi = fi; p.k2 = ki * ki; p.B = B;
     p.M = fo; p.N = p.k2 * fi; p.R = B * woho;
     const bool vec = (woho % 4 == 0) && aligned16(dmu) && aligned16(dvar);
-    // 3x3, stride 1, "same" padding on a square map (the kernel verifies the table):
-    // 64 x 64 tiles of whole channels, slices of whole 64-pixel k-tiles
-    int stencil = 0;
-    if (g_conv2d_stencil && vec && ki == 3 && woho == wihi && fi % 64 == 0 && fo % 64 == 0 &&
-        p.R % 64 == 0 && tile == TILE_64x64 && aligned16(mu_a))
-        stencil = stencil_width(wihi);
+    const int stencil = conv2d_bwd_dw_stencil(mu_a, dmu, dvar, B, fo, woho, wihi, fi, ki, tile);
     const int unit = stencil ? 64 : KT;
     int per = ceil_div(ceil_div(p.R, splits), unit) * unit;
     p.splits = ceil_div(p.R, per);

@@ -48,52 +48,85 @@ struct StencilGeom {
     static_assert(UNITS <= 512 && BN % W == 0 && NR % RPI == 0 && H % RPI == 0, "tile geometry");
 };
 
-// Does the table describe the regular stencil for the pixels n0 .. n0+127? Every
-// thread checks a share and returns its verdict.
+// Expected Fmwa_2 entry (1-based input pixel, -1 = padding) of tap t of output
+// pixel o on a W x W map.
+template <int W>
+__device__ __forceinline__ int stencil_fmwa(int o, int t) {
+    const int y = o / W, x = o - y * W;
+    const int iy = y + t / 3 - 1, ix = x + t % 3 - 1;
+    return (iy >= 0 && iy < W && ix >= 0 && ix < W) ? iy * W + ix + 1 : -1;
+}
+
+// Does the table describe the regular stencil for the pixels n0 .. n0+127? All
+// threads of the workgroup call this; the verdict is uniform. `scratch` holds
+// 130 ints of LDS. Table entries are requested in batches before any is looked
+// at, so that the check costs one memory latency, not one per entry.
 template <bool DZ, int WIDTH>
 __device__ __forceinline__ bool stencil_tables_ok(const ConvParams &p, int n0, int tid,
-                                                  int nthreads) {
-    constexpr int W = WIDTH, H = WIDTH;
+                                                  int nthreads, int *scratch) {
+    constexpr int W = WIDTH, H = WIDTH, PAIRS = 128 * 9;
+    int *flag = scratch, *seen = scratch + 2;
+    if (tid == 0) *flag = 1;
+    if (DZ && tid < 128) seen[tid] = 0;
+    __syncthreads();
     bool ok = true;
     if (!DZ) {
-        // Fmwa_2 [woho][9]: 1-based input pixel under tap t of output pixel o, -1 = padding
-        for (int e = tid; e < 128 * 9; e += nthreads) {
-            const int c = e / 9, t = e - c * 9, n = n0 + c;
-            if (n >= p.N) continue;
-            const int o = n % p.woho, y = o / W, x = o - y * W;
-            const int iy = y + t / 3 - 1, ix = x + t % 3 - 1;
-            const int want = (iy >= 0 && iy < H && ix >= 0 && ix < W) ? iy * W + ix + 1 : -1;
-            ok = ok && p.idx[o * 9 + t] == want;
+        // Fmwa_2 [woho][9]
+        int got[3], want[3];
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+            const int e = tid + i * nthreads, c = e / 9, t = e - c * 9, n = n0 + c;
+            const bool live = e < PAIRS && n < p.N;
+            const int o = live ? n % p.woho : 0;
+            got[i] = p.idx[live ? o * 9 + t : 0];
+            want[i] = live ? stencil_fmwa<W>(o, t) : got[i];
         }
+#pragma unroll
+        for (int i = 0; i < 3; i++) ok = ok && got[i] == want[i];
     } else {
         // FCzwa_1 [wihi][nr] / Szz_ud [nr][wihi]: per input pixel the (tap, output
-        // pixel) pairs that touch it, in any order. Regular stencil: tap t touches
-        // pixel (y, x) from output pixel (y-ky+1, x-kx+1) when that lies in the map.
-        for (int c = tid; c < 128; c += nthreads) {
-            const int n = n0 + c;
-            if (n >= p.N) continue;
-            const int px = n % p.wihi, y = px / W, x = px - y * W;
-            int seen = 0, want = 0;
+        // pixel) pairs that touch it, in any order (nr = 9). Regular stencil: tap t
+        // touches pixel (y, x) from output pixel (y-ky+1, x-kx+1) when that lies in
+        // the map; every such tap must be listed exactly once.
+        int out[3], tap[3], col[3];
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+            const int e = tid + i * nthreads, j = e / 128, c = e - j * 128, n = n0 + c;
+            const bool live = e < PAIRS && n < p.N;
+            const int px = live ? n % p.wihi : 0;
+            out[i] = p.idx2[live ? j * p.wihi + px : 0];
+            tap[i] = p.idx[live ? px * 9 + j : 0];
+            col[i] = live ? c : -1;
+        }
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+            if (col[i] < 0 || out[i] <= -1) continue;
+            const int px = (n0 + col[i]) % p.wihi, y = px / W, x = px - y * W;
+            if (tap[i] < 1 || tap[i] > 9) {
+                ok = false;
+                continue;
+            }
+            const int t = tap[i] - 1, qy = y - t / 3 + 1, qx = x - t % 3 + 1;
+            ok = ok && qy >= 0 && qy < H && qx >= 0 && qx < W && out[i] == qy * W + qx + 1;
+            if (atomicOr(&seen[col[i]], 1 << t) >> t & 1) ok = false;  // listed twice
+        }
+        __syncthreads();
+        if (tid < 128 && n0 + tid < p.N) {
+            const int px = (n0 + tid) % p.wihi, y = px / W, x = px - y * W;
+            int want = 0;
+#pragma unroll
             for (int t = 0; t < 9; t++) {
                 const int qy = y - t / 3 + 1, qx = x - t % 3 + 1;
                 if (qy >= 0 && qy < H && qx >= 0 && qx < W) want |= 1 << t;
             }
-            for (int j = 0; j < p.nr; j++) {
-                const int o = p.idx2[j * p.wihi + px];
-                if (o <= -1) continue;
-                const int tap = p.idx[px * p.nr + j];
-                if (tap < 1 || tap > 9 || (seen >> (tap - 1) & 1)) {
-                    ok = false;
-                    continue;
-                }
-                const int t = tap - 1, qy = y - t / 3 + 1, qx = x - t % 3 + 1;
-                ok = ok && qy >= 0 && qy < H && qx >= 0 && qx < W && o == qy * W + qx + 1;
-                seen |= 1 << t;
-            }
-            ok = ok && seen == want;
+            ok = ok && seen[tid] == want;
         }
     }
-    return ok;
+    if (!ok) *flag = 0;
+    __syncthreads();
+    const bool verdict = __builtin_amdgcn_readfirstlane(*flag) != 0;
+    __syncthreads();  // scratch may be reused
+    return verdict;
 }
 
 // The tile loop on a verified stencil. `lds` holds the weight tile(s) followed by
@@ -273,13 +306,7 @@ void conv_stencil_kernel(ConvParams p) {
     const int r_begin = split * p.r_per_split;
     const int r_end = min(p.R, r_begin + p.r_per_split);
 
-    if (threadIdx.x == 0) lds_extra[0] = 1;
-    __syncthreads();
-    if (!stencil_tables_ok<DZ, WIDTH>(p, n0, threadIdx.x, 512)) lds_extra[0] = 0;
-    __syncthreads();
-    const int regular = __builtin_amdgcn_readfirstlane(lds_extra[0]);
-    __syncthreads();  // the table-driven prologue reuses lds_extra
-    if (regular) {
+    if (stencil_tables_ok<DZ, WIDTH>(p, n0, threadIdx.x, 512, lds_extra)) {
         stencil_body<DZ, WIDTH>(p, lds, m0, n0, split, r_begin, r_end);
         return;
     }
@@ -510,19 +537,25 @@ void conv_stencil_dw_kernel(ConvParams p) {
     const int r_end = min(p.R, r_begin + p.r_per_split);
 
     // the pixels of this slice, per image position: all of Fmwa_2 once the slice
-    // is as long as a map
+    // is as long as a map. Entries are requested six at a time before any is
+    // looked at (one memory latency per batch, not per entry).
     if (threadIdx.x == 0) regular_flag = 1;
     __syncthreads();
     {
-        const int len = min(max(r_end - r_begin, 0), p.woho);
+        const int total = min(max(r_end - r_begin, 0), p.woho) * 9;
         bool ok = true;
-        for (int e = threadIdx.x; e < len * 9; e += 512) {
-            const int c = e / 9, t = e - c * 9;
-            const int o = (r_begin + c) & (WIDTH * WIDTH - 1), y = o / WIDTH, x = o - y * WIDTH;
-            const int iy = y + t / 3 - 1, ix = x + t % 3 - 1;
-            const int want =
-                (iy >= 0 && iy < WIDTH && ix >= 0 && ix < WIDTH) ? iy * WIDTH + ix + 1 : -1;
-            ok = ok && p.idx[o * 9 + t] == want;
+        for (int base = threadIdx.x; base < total; base += 6 * 512) {
+            int got[6], want[6];
+#pragma unroll
+            for (int i = 0; i < 6; i++) {
+                const int e = base + i * 512, c = e / 9, t = e - c * 9;
+                const bool live = e < total;
+                const int o = live ? (r_begin + c) & (WIDTH * WIDTH - 1) : 0;
+                got[i] = p.idx[live ? o * 9 + t : 0];
+                want[i] = live ? stencil_fmwa<WIDTH>(o, t) : got[i];
+            }
+#pragma unroll
+            for (int i = 0; i < 6; i++) ok = ok && got[i] == want[i];
         }
         if (!ok) regular_flag = 0;
     }

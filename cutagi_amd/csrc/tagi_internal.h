@@ -147,6 +147,9 @@ hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float
                                 int tile, int splits, float *ws0, float *ws1, float *out_dmu,
                                 float *out_dvar, hipStream_t stream);
 int conv2d_bwd_dw_blocks_per_cu(int tile);
+int conv2d_bwd_dw_stencil(const float *mu_a, const float *dmu, const float *dvar, int B, int fo,
+                          int woho, int wihi, int fi, int ki, int tile);
+int conv2d_bwd_dw_stencil_splits(int out_tiles);
 hipError_t launch_conv2d_bwd_dw(const float *var_w, const float *mu_a, const float *dmu,
                                 const float *dvar, const int *aidx, int B, int fo, int woho,
                                 int wihi, int fi, int ki, int tile, int splits, float *ws0, float *ws1,
