@@ -142,7 +142,8 @@ __device__ __forceinline__ void stencil_body(const ConvParams &p, float *lds, in
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wrow = (wave / 4) * 32, wcol = (wave % 4) * 32, half = lane >> 5;
     float *lds_a = lds;                       // [NA][64][AS]
-    float *lds_p = lds + NA * 64 * G::AS;     // [2][PATCH]
+    float *lds_p = lds + NA * 64 * G::AS;     // [PATCH][2]: the two gathered arrays interleaved,
+                                              // so that one 8-byte read fetches a lane's pair
     // gathered tensor: activations [B][fi][W*H] (forward), innovations [B][fo][W*H]
     const float *src0 = DZ ? p.d0 : p.a0, *src1 = DZ ? p.d1 : p.a1;
     const int CH = DZ ? p.fo : p.fi;
@@ -231,16 +232,16 @@ __device__ __forceinline__ void stencil_body(const ConvParams &p, float *lds, in
                     dst[adst[i][3]] = ra[a][i].w;
                 }
         if (unit_ok) {
-            *reinterpret_cast<float4 *>(lds_p + pdst) = rp0;
-            *reinterpret_cast<float4 *>(lds_p + G::PATCH + pdst) = rp1;
+            *reinterpret_cast<float4 *>(lds_p + 2 * pdst) = make_float4(rp0.x, rp1.x, rp0.y, rp1.y);
+            *reinterpret_cast<float4 *>(lds_p + 2 * pdst + 4) =
+                make_float4(rp0.z, rp1.z, rp0.w, rp1.w);
         }
     };
 
     // operand addresses of this lane
     const int pix = wcol + (lane & 31), prow = pix / W, px = pix - prow * W;
-    const float *b0 = lds_p + half * G::CS + (prow / G::RPI) * G::SEG + (prow % G::RPI) * G::RS +
-                      G::XO - 1 + px;
-    const float *b1 = b0 + G::PATCH;
+    const float *bp = lds_p + 2 * (half * G::CS + (prow / G::RPI) * G::SEG +
+                                   (prow % G::RPI) * G::RS + G::XO - 1 + px);
     const float *a0 = lds_a + (wrow + (lane & 31)) * G::AS + half * 36;
     const float *a1 = a0 + 64 * G::AS;
 
@@ -264,7 +265,8 @@ __device__ __forceinline__ void stencil_body(const ConvParams &p, float *lds, in
                 const int s = 4 * g + e, pair = s / 9, t = s - pair * 9, ky = t / 3, kx = t - ky * 3;
                 const int off = pair * 2 * G::CS +
                                 (DZ ? (2 - ky) * G::RS + (2 - kx) : ky * G::RS + kx);
-                const float w = comp4(am, e), y0 = b0[off], y1 = b1[off];
+                const float2 y = *reinterpret_cast<const float2 *>(bp + 2 * off);
+                const float w = comp4(am, e), y0 = y.x, y1 = y.y;
                 if (!DZ) {
                     // mean: mu_w mu_a; variance: var_w (var_a + mu_a^2) + mu_w^2 var_a
                     acc0[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(w, y0, acc0[0][0], 0, 0, 0);
