@@ -287,19 +287,28 @@ def cpu_baseline(name):
     jcb = np.ones((B, K), f)
     dmu = (rng.standard_normal((B, N)) * 0.1).astype(f)
     dvar = (-rng.uniform(0, 1e-3, (B, N))).astype(f)
+    def steps(reps, t):
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            lib.linear_fwd(mu_w, var_w, mu_b, var_b, mu_a, var_a, t)
+            lib.linear_bwd_dz(mu_w, jcb, dmu, dvar, t)
+            lib.linear_bwd_dw(var_w, mu_a, dmu, dvar, t)
+            lib.linear_bwd_db(var_b, dmu, dvar, t)
+        return (time.perf_counter() - t0) / reps
+
     reps = 3
-    t0 = time.perf_counter()
-    for _ in range(reps):
-        lib.linear_fwd(mu_w, var_w, mu_b, var_b, mu_a, var_a, threads)
-        lib.linear_bwd_dz(mu_w, jcb, dmu, dvar, threads)
-        lib.linear_bwd_dw(var_w, mu_a, dmu, dvar, threads)
-        lib.linear_bwd_db(var_b, dmu, dvar, threads)
-    dt = (time.perf_counter() - t0) / reps
-    return dict(value=round(14.0 * B * N * K / dt / 1e12, 5), unit="TFLOP/s", cores=threads,
-                kind="port", seconds_per_step=round(dt, 3),
-                sample="%d full forward+backward steps of the %s workload (K=%d, N=%d, B=%d), "
-                       "reference thread fan-out with %d std::threads"
-                       % (reps, name, K, N, B, threads))
+    dt = steps(reps, threads)
+    out = dict(value=round(14.0 * B * N * K / dt / 1e12, 5), unit="TFLOP/s", cores=threads,
+               kind="port", seconds_per_step=round(dt, 3),
+               sample="%d full forward+backward steps of the %s workload (K=%d, N=%d, B=%d), "
+                      "reference thread fan-out with %d std::threads"
+                      % (reps, name, K, N, B, threads))
+    if threads > 4:
+        # the reference's default thread count (include/base_layer.h:60), one step
+        dt4 = steps(1, 4)
+        out["reference_default_threads"] = dict(cores=4, seconds_per_step=round(dt4, 3),
+                                                value=round(14.0 * B * N * K / dt4 / 1e12, 5))
+    return out
 
 
 def main():
