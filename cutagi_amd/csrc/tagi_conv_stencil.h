@@ -41,8 +41,9 @@ struct StencilGeom {
     static constexpr int CS = SEGS * SEG + 4;      // one channel (+ the last row's halo cell)
     static constexpr int PATCH = KC * CS;          // floats per staged array
     static constexpr int UNITS = KC * SEGS * (RPI + 2) * (W / 4);  // 16-byte loads per array
-    // Weight tile [64 rows][2 halves][36 steps], row stride 76: eight consecutive
-    // rows start on eight different groups of four banks.
+    // Weight tile [64 rows][2 k-halves][36 steps], row stride 76: eight consecutive
+    // rows start on eight different groups of four banks. Forward: a half is four
+    // channels in memory order; state backward: the even / odd channels.
     static constexpr int AS = 76;
     static constexpr int A_VEC = BM * KC * 9 / 4;  // 16-byte loads per weight array
     static_assert(UNITS <= 512 && BN % W == 0 && NR % RPI == 0 && H % RPI == 0, "tile geometry");
@@ -181,11 +182,11 @@ __device__ __forceinline__ void stencil_body(const ConvParams &p, float *lds, in
             // rows = output channels, 72 consecutive values of w[row][c*9 + t]
             const int row = id / 18, q = id - row * 18;
             aunit[i] = (size_t)(m0 + row) * p.R + (size_t)c_begin * 9 + 4 * q;
+            // kept in memory order (the 16 bytes stay together): lanes 0-31 of an MFMA
+            // step take channels 0-3 of the k-tile = values 0-35 of the row, lanes
+            // 32-63 channels 4-7
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const int kk = 4 * q + e, c = kk / 9, t = kk - c * 9;
-                adst[i][e] = row * G::AS + (c & 1) * 36 + (c >> 1) * 9 + t;
-            }
+            for (int e = 0; e < 4; e++) adst[i][e] = row * G::AS + 4 * q + e;
         } else {
             // rows = input channels; for one output channel f the values
             // w[f][(m0+row)*9 + t] of the 64 rows are 576 consecutive floats
@@ -207,30 +208,47 @@ __device__ __forceinline__ void stencil_body(const ConvParams &p, float *lds, in
         acc1[0][0][v] = 0.f;
     }
 
-    float4 ra[NA][SLOTS], rp0, rp1;
+    // staging registers, named one by one (an array written in one lambda and read
+    // in another is kept in scratch memory by the compiler)
+    static_assert(SLOTS == 3, "three 16-byte pieces of the weight tile per thread");
+    float4 rm0, rm1, rm2, rv0, rv1, rv2, rp0, rp1;
+    rv0 = rv1 = rv2 = make_float4(0.f, 0.f, 0.f, 0.f);
     auto fetch = [&]() {
-#pragma unroll
-        for (int i = 0; i < SLOTS; i++) {
-            ra[0][i] = *reinterpret_cast<const float4 *>(p.w0 + aunit[i]);
-            if (NA == 2) ra[NA - 1][i] = *reinterpret_cast<const float4 *>(p.w1 + aunit[i]);
-            if (a_ok[i]) aunit[i] += astep;
+        rm0 = *reinterpret_cast<const float4 *>(p.w0 + aunit[0]);
+        rm1 = *reinterpret_cast<const float4 *>(p.w0 + aunit[1]);
+        rm2 = *reinterpret_cast<const float4 *>(p.w0 + aunit[2]);
+        if (NA == 2) {
+            rv0 = *reinterpret_cast<const float4 *>(p.w1 + aunit[0]);
+            rv1 = *reinterpret_cast<const float4 *>(p.w1 + aunit[1]);
+            rv2 = *reinterpret_cast<const float4 *>(p.w1 + aunit[2]);
         }
+#pragma unroll
+        for (int i = 0; i < SLOTS; i++)
+            if (a_ok[i]) aunit[i] += astep;
         rp0 = *reinterpret_cast<const float4 *>(src0 + punit);
         rp1 = *reinterpret_cast<const float4 *>(src1 + punit);
         punit += pstep;
     };
+    auto put = [&](float *dst, int i, const float4 &v) {
+        if (!a_ok[i]) return;
+        if (!DZ) {
+            *reinterpret_cast<float4 *>(dst + adst[i][0]) = v;
+        } else {
+            dst[adst[i][0]] = v.x;
+            dst[adst[i][1]] = v.y;
+            dst[adst[i][2]] = v.z;
+            dst[adst[i][3]] = v.w;
+        }
+    };
     auto commit = [&]() {
-#pragma unroll
-        for (int a = 0; a < NA; a++)
-#pragma unroll
-            for (int i = 0; i < SLOTS; i++)
-                if (a_ok[i]) {
-                    float *dst = lds_a + a * 64 * G::AS;
-                    dst[adst[i][0]] = ra[a][i].x;
-                    dst[adst[i][1]] = ra[a][i].y;
-                    dst[adst[i][2]] = ra[a][i].z;
-                    dst[adst[i][3]] = ra[a][i].w;
-                }
+        put(lds_a, 0, rm0);
+        put(lds_a, 1, rm1);
+        put(lds_a, 2, rm2);
+        if (NA == 2) {
+            put(lds_a + 64 * G::AS, 0, rv0);
+            put(lds_a + 64 * G::AS, 1, rv1);
+            put(lds_a + 64 * G::AS, 2, rv2);
+        }
         if (unit_ok) {
             *reinterpret_cast<float4 *>(lds_p + 2 * pdst) = make_float4(rp0.x, rp1.x, rp0.y, rp1.y);
             *reinterpret_cast<float4 *>(lds_p + 2 * pdst + 4) =
@@ -240,7 +258,10 @@ __device__ __forceinline__ void stencil_body(const ConvParams &p, float *lds, in
 
     // operand addresses of this lane
     const int pix = wcol + (lane & 31), prow = pix / W, px = pix - prow * W;
-    const float *bp = lds_p + 2 * (half * G::CS + (prow / G::RPI) * G::SEG +
+    // k-halves of an MFMA step: forward, channels c and c + 4 (weights stay in memory
+    // order); state backward, channels 2c and 2c + 1
+    constexpr int HALF_CH = DZ ? 1 : 4, STEP_CH = DZ ? 2 : 1;
+    const float *bp = lds_p + 2 * (half * HALF_CH * G::CS + (prow / G::RPI) * G::SEG +
                                    (prow % G::RPI) * G::RS + G::XO - 1 + px);
     const float *a0 = lds_a + (wrow + (lane & 31)) * G::AS + half * 36;
     const float *a1 = a0 + 64 * G::AS;
@@ -263,7 +284,7 @@ __device__ __forceinline__ void stencil_body(const ConvParams &p, float *lds, in
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int s = 4 * g + e, pair = s / 9, t = s - pair * 9, ky = t / 3, kx = t - ky * 3;
-                const int off = pair * 2 * G::CS +
+                const int off = pair * STEP_CH * G::CS +
                                 (DZ ? (2 - ky) * G::RS + (2 - kx) : ky * G::RS + kx);
                 const float2 y = *reinterpret_cast<const float2 *>(bp + 2 * off);
                 const float w = comp4(am, e), y0 = y.x, y1 = y.y;
