@@ -13,9 +13,12 @@
 // nine table lookups per element) the workgroup stages each channel's rows ONCE,
 // with a zero halo, and the nine taps are nine constant offsets into that patch
 // when the MFMA operand is read from LDS. The k-tile is 8 channels x 9 taps = 72
-// reduction steps; MFMA k-halves (lanes 0-31 / 32-63) take an even / odd channel
-// at the same tap, so one LDS address per lane plus an immediate per step reaches
-// every operand.
+// reduction steps; the two MFMA k-halves (lanes 0-31 / 32-63) take two channels a
+// fixed distance apart at the same tap, so one LDS address per lane plus an
+// immediate per step reaches every operand. Weights are staged in the order they
+// have in memory (16-byte commits). What sits between the two barriers of a
+// k-tile is exposed, LDS reads during the MFMAs are not, so layouts favour cheap
+// commits over wide reads.
 //
 // Included by tagi_conv2d.hip after ConvParams, ConvFwdProblem and ConvDzProblem.
 #pragma once
@@ -167,10 +170,9 @@ __device__ __forceinline__ void stencil_body(const ConvParams &p, float *lds, in
     const size_t pstep = unit_ok ? (size_t)G::KC * (W * H) : 0;
     const int pdst = pc * G::CS + seg * G::SEG + pr * G::RS + G::XO + 4 * x4;
 
-    // this thread's 16-byte pieces of the weight tile and where their four values go
-    // in the [row][half][step] layout
+    // this thread's 16-byte pieces of the weight tile and where they go in LDS
     size_t aunit[SLOTS];
-    int adst[SLOTS][4];
+    int adst[SLOTS];
     bool a_ok[SLOTS];
     const size_t astep = DZ ? (size_t)G::KC * p.fi * 9 : (size_t)G::KC * 9;
 #pragma unroll
@@ -185,18 +187,14 @@ __device__ __forceinline__ void stencil_body(const ConvParams &p, float *lds, in
             // kept in memory order (the 16 bytes stay together): lanes 0-31 of an MFMA
             // step take channels 0-3 of the k-tile = values 0-35 of the row, lanes
             // 32-63 channels 4-7
-#pragma unroll
-            for (int e = 0; e < 4; e++) adst[i][e] = row * G::AS + 4 * q + e;
+            adst[i] = row * G::AS + 4 * q;
         } else {
             // rows = input channels; for one output channel f the values
             // w[f][(m0+row)*9 + t] of the 64 rows are 576 consecutive floats
             const int f = id / 144, q = id - f * 144;
             aunit[i] = (size_t)(c_begin + f) * p.fi * 9 + (size_t)m0 * 9 + 4 * q;
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const int flat = 4 * q + e, row = flat / 9, t = flat - row * 9;
-                adst[i][e] = row * G::AS + (f & 1) * 36 + (f >> 1) * 9 + t;
-            }
+            // kept in memory order too: [f][row * 9 + t] (576 values per output channel)
+            adst[i] = f * 576 + 4 * q;
         }
         if (!a_ok[i]) aunit[i] = 0;
     }
@@ -230,15 +228,7 @@ __device__ __forceinline__ void stencil_body(const ConvParams &p, float *lds, in
         punit += pstep;
     };
     auto put = [&](float *dst, int i, const float4 &v) {
-        if (!a_ok[i]) return;
-        if (!DZ) {
-            *reinterpret_cast<float4 *>(dst + adst[i][0]) = v;
-        } else {
-            dst[adst[i][0]] = v.x;
-            dst[adst[i][1]] = v.y;
-            dst[adst[i][2]] = v.z;
-            dst[adst[i][3]] = v.w;
-        }
+        if (a_ok[i]) *reinterpret_cast<float4 *>(dst + adst[i]) = v;
     };
     auto commit = [&]() {
         put(lds_a, 0, rm0);
@@ -263,7 +253,11 @@ __device__ __forceinline__ void stencil_body(const ConvParams &p, float *lds, in
     constexpr int HALF_CH = DZ ? 1 : 4, STEP_CH = DZ ? 2 : 1;
     const float *bp = lds_p + 2 * (half * HALF_CH * G::CS + (prow / G::RPI) * G::SEG +
                                    (prow % G::RPI) * G::RS + G::XO - 1 + px);
-    const float *a0 = lds_a + (wrow + (lane & 31)) * G::AS + half * 36;
+    // weights: forward [row][72] (a lane reads four steps with 16 bytes); state
+    // backward [f][row*9 + t] (one value per step; 32 rows at stride 9 floats fall on
+    // 32 different banks)
+    const float *a0 = DZ ? lds_a + (wrow + (lane & 31)) * 9 + half * 576
+                         : lds_a + (wrow + (lane & 31)) * G::AS + half * 36;
     const float *a1 = a0 + 64 * G::AS;
 
     __syncthreads();  // patch zeroed
@@ -278,16 +272,18 @@ __device__ __forceinline__ void stencil_body(const ConvParams &p, float *lds, in
         if (more) fetch();
 #pragma unroll
         for (int g = 0; g < 9; g++) {
-            const float4 am = *reinterpret_cast<const float4 *>(a0 + 4 * g);
-            float4 av = am;
-            if (NA == 2) av = *reinterpret_cast<const float4 *>(a1 + 4 * g);
+            float4 am = make_float4(0.f, 0.f, 0.f, 0.f), av = am;
+            if (!DZ) {
+                am = *reinterpret_cast<const float4 *>(a0 + 4 * g);
+                av = *reinterpret_cast<const float4 *>(a1 + 4 * g);
+            }
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int s = 4 * g + e, pair = s / 9, t = s - pair * 9, ky = t / 3, kx = t - ky * 3;
                 const int off = pair * STEP_CH * G::CS +
                                 (DZ ? (2 - ky) * G::RS + (2 - kx) : ky * G::RS + kx);
                 const float2 y = *reinterpret_cast<const float2 *>(bp + 2 * off);
-                const float w = comp4(am, e), y0 = y.x, y1 = y.y;
+                const float w = DZ ? a0[pair * 1152 + t] : comp4(am, e), y0 = y.x, y1 = y.y;
                 if (!DZ) {
                     // mean: mu_w mu_a; variance: var_w (var_a + mu_a^2) + mu_w^2 var_a
                     acc0[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(w, y0, acc0[0][0], 0, 0, 0);
