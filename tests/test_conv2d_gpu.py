@@ -21,6 +21,7 @@ GEOMS = [
     (3, 1, 1, 1, 12, 70, 66, 1),
     (4, 2, 1, 1, 10, 3, 5, 2),
     (7, 2, 3, 1, 17, 3, 40, 2),  # per-tap table + staged tiles exceed 64 KB of LDS
+    (10, 1, 0, 1, 12, 2, 3, 2),  # the largest kernel whose per-tap table fits
     (3, 1, 1, 1, 4, 128, 96, 3),  # late-stage shape: few pixels, long reduction (sliced)
     (2, 2, 0, 1, 8, 64, 130, 2),  # projection shortcut, more than 128 output channels
     # 3x3 s1 p1 on square maps with whole groups of channels: the regular-stencil kernels
@@ -205,3 +206,17 @@ def test_conv2d_state_backward_column_orders_agree(oracle_lib, geom):
             assert_close(dz[1].cpu().numpy(), ref[1], "delta_var_z order %d" % mode)
     finally:
         capi.tune("conv2d.phase_order", 1)
+
+
+def test_conv2d_kernel_too_large_for_the_tap_table_is_refused():
+    import torch
+    import cutagi_amd.functional as F
+    from cutagi_amd import capi
+    k, wi, fi, fo, B = 11, 12, 1, 2, 1
+    idx = capi.conv2d_build_idx(k, 1, wi, wi, 0, 1, k * k * fi * fo + 1)
+    woho = idx["wo"] * idx["ho"]
+    z = lambda n: torch.zeros(n, device="cuda")
+    with pytest.raises(capi.TagiHipError):
+        F.conv2d_fwd(z(fo * fi * k * k), z(fo * fi * k * k), None, None, z(B * fi * wi * wi),
+                     z(B * fi * wi * wi), torch.from_numpy(idx["Fmwa_2"]).cuda(), woho, fo,
+                     wi * wi, fi, k, B)
