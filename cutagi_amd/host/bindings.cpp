@@ -270,4 +270,17 @@ PYBIND11_MODULE(cutagi, m) {
     m.def("manual_seed", &manual_seed);
     m.def("is_cuda_available", &is_cuda_available);
     m.def("get_cuda_device_count", &get_cuda_device_count);
+    m.def("get_cuda_current_device", &get_current_cuda_device);
+    m.def("set_cuda_device", &set_cuda_device);
+    m.def("is_cuda_device_available", &is_cuda_device_available);
+    m.def("is_nccl_available", &is_nccl_available);
+    m.def("get_cuda_device_properties", &get_cuda_device_properties);
+    // (free, total) in bytes; the reference's binding of the reference-argument
+    // form is what pytagi.cuda.get_device_memory documents as this pair
+    m.def("get_cuda_device_memory", [](int device_index) {
+        size_t free_memory = 0, total_memory = 0;
+        if (!get_cuda_device_memory(device_index, free_memory, total_memory))
+            throw std::runtime_error("could not query the device memory");
+        return std::make_tuple(free_memory, total_memory);
+    });
 }

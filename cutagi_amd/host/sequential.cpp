@@ -1,6 +1,7 @@
 // Sequential and OutputUpdater: see sequential.h.
 #include "sequential.h"
 
+#include <hip/hip_runtime_api.h>
 #include <sys/stat.h>
 
 #include <fstream>
@@ -19,6 +20,89 @@ int get_cuda_device_count() {
     return n;
 }
 bool is_cuda_available() { return get_cuda_device_count() > 0; }
+
+int get_current_cuda_device() {
+    if (!is_cuda_available()) return -1;
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess) {
+        LOG(LogLevel::ERROR, "Failed to get current CUDA device");
+        return -1;
+    }
+    return device;
+}
+
+bool set_cuda_device(int device_index) {
+    if (!is_cuda_available()) {
+        LOG(LogLevel::ERROR, "CUDA is not available");
+        return false;
+    }
+    if (device_index < 0 || device_index >= get_cuda_device_count()) {
+        LOG(LogLevel::ERROR, "Invalid CUDA device index: " + std::to_string(device_index));
+        return false;
+    }
+    if (hipSetDevice(device_index) != hipSuccess) {
+        LOG(LogLevel::ERROR, "Failed to set CUDA device");
+        return false;
+    }
+    return true;
+}
+
+bool is_cuda_device_available(int device_index) {
+    if (!is_cuda_available()) return false;
+    if (device_index < 0 || device_index >= get_cuda_device_count()) return false;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device_index) != hipSuccess) {
+        LOG(LogLevel::ERROR, "Failed to get CUDA device properties");
+        return false;
+    }
+    return prop.computeMode != hipComputeModeProhibited;
+}
+
+bool is_nccl_available() { return false; }
+
+std::string get_cuda_device_properties(int device_index) {
+    if (!is_cuda_available()) return "CUDA is not available";
+    if (device_index < 0 || device_index >= get_cuda_device_count())
+        return "Invalid CUDA device index: " + std::to_string(device_index);
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device_index) != hipSuccess)
+        return "Failed to get CUDA device properties";
+    std::stringstream ss;
+    ss << "Device " << device_index << ": " << prop.name << " (" << prop.gcnArchName << ")\n";
+    ss << "  Total global memory: " << prop.totalGlobalMem / (1024 * 1024) << " MB\n";
+    ss << "  Compute units: " << prop.multiProcessorCount << "\n";
+    ss << "  Max threads per block: " << prop.maxThreadsPerBlock << "\n";
+    ss << "  Shared memory (LDS) per block: " << prop.sharedMemPerBlock / 1024 << " KB\n";
+    ss << "  Wavefront size: " << prop.warpSize << "\n";
+    ss << "  Clock rate: " << prop.clockRate / 1000 << " MHz\n";
+    ss << "  Memory clock rate: " << prop.memoryClockRate / 1000 << " MHz\n";
+    ss << "  Memory bus width: " << prop.memoryBusWidth << " bits\n";
+    ss << "  L2 cache size: " << prop.l2CacheSize / 1024 << " KB\n";
+    return ss.str();
+}
+
+bool get_cuda_device_memory(int device_index, size_t &free_memory, size_t &total_memory) {
+    if (!is_cuda_available()) {
+        LOG(LogLevel::ERROR, "CUDA is not available");
+        return false;
+    }
+    if (device_index < 0 || device_index >= get_cuda_device_count()) {
+        LOG(LogLevel::ERROR, "Invalid CUDA device index: " + std::to_string(device_index));
+        return false;
+    }
+    int current = 0;
+    if (hipGetDevice(&current) != hipSuccess || hipSetDevice(device_index) != hipSuccess) {
+        LOG(LogLevel::ERROR, "Failed to set CUDA device");
+        return false;
+    }
+    const hipError_t e = hipMemGetInfo(&free_memory, &total_memory);
+    (void)hipSetDevice(current);
+    if (e != hipSuccess) {
+        LOG(LogLevel::ERROR, "Failed to get CUDA memory info");
+        return false;
+    }
+    return true;
+}
 
 // ---- OutputUpdater ------------------------------------------------------------------
 OutputUpdater::OutputUpdater(const std::string model_device) : device(model_device) {

@@ -12,8 +12,16 @@
 
 namespace tagi_host {
 
+// Device queries under the reference's names (src/cuda_utils.cpp:11-230); "cuda"
+// means the HIP device here, as everywhere in this API.
 bool is_cuda_available();
 int get_cuda_device_count();
+int get_current_cuda_device();                 // -1 without a device
+bool set_cuda_device(int device_index);        // logs and throws on an invalid index
+bool is_cuda_device_available(int device_index);
+bool is_nccl_available();                      // always false: one GPU, no collectives
+std::string get_cuda_device_properties(int device_index);
+bool get_cuda_device_memory(int device_index, size_t &free_memory, size_t &total_memory);
 
 class OutputUpdater {
    public:

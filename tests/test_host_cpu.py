@@ -84,3 +84,20 @@ def test_resnet18_builds_on_the_host():
     assert info[-2] == "AvgPool2d(512,512,1,1,4)"
     assert net.z_buffer_size == 64 * 32 * 32
     assert len(net.layers) == 13
+
+
+def test_device_queries_without_a_device():
+    """The reference's module-level device queries exist; without a GPU they answer
+    as the reference's CPU-only build does (src/cuda_utils.cpp)."""
+    from cutagi_amd import cutagi
+    if cutagi.is_cuda_available():
+        pytest.skip("a GPU is present")
+    assert cutagi.get_cuda_device_count() == 0
+    assert cutagi.get_cuda_current_device() == -1
+    assert cutagi.is_cuda_device_available(0) is False
+    assert cutagi.is_nccl_available() is False
+    assert cutagi.get_cuda_device_properties(0) == "CUDA is not available"
+    with pytest.raises(RuntimeError):
+        cutagi.set_cuda_device(0)
+    with pytest.raises(RuntimeError):
+        cutagi.get_cuda_device_memory(0)

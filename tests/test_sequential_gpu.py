@@ -233,3 +233,15 @@ def test_output_updater_reads_numpy_arrays_in_place():
     bad[5] = 0
     with pytest.raises(RuntimeError):
         upd.update_using_indices(net.output_z_buffer, ys, vs, bad, d)
+
+
+def test_device_queries():
+    from cutagi_amd import cutagi
+    assert cutagi.is_cuda_available() and cutagi.get_cuda_device_count() >= 1
+    assert cutagi.get_cuda_current_device() == 0 and cutagi.set_cuda_device(0) is True
+    assert cutagi.is_cuda_device_available(0) and not cutagi.is_cuda_device_available(99)
+    assert "gfx950" in cutagi.get_cuda_device_properties(0)
+    free, total = cutagi.get_cuda_device_memory(0)
+    assert 0 < free <= total and total > 100 * 2 ** 30
+    with pytest.raises(RuntimeError):
+        cutagi.set_cuda_device(99)
