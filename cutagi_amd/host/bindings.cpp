@@ -105,12 +105,19 @@ PYBIND11_MODULE(cutagi, m) {
         .def("preinit_layer", &BaseLayer::preinit_layer)
         .def("params_to_host", &BaseLayer::params_to_host)
         .def("params_to_device", &BaseLayer::params_to_device)
-        .def("delta_params_to_host", &BaseLayer::delta_params_to_host);
+        .def("delta_params_to_host", &BaseLayer::delta_params_to_host)
+        .def("get_norm_mean_var", &BaseLayer::get_norm_mean_var)
+        .def("to_cuda", [](BaseLayer &self, int device_idx) {
+                 return std::shared_ptr<BaseLayer>(self.to_cuda(device_idx));
+             }, py::arg("device_idx") = 0);
 
     py::class_<Linear, BaseLayer, std::shared_ptr<Linear>>(m, "Linear")
         .def(py::init<size_t, size_t, bool, float, float, std::string, int>(), py::arg("ip_size"),
              py::arg("op_size"), py::arg("bias") = true, py::arg("gain_weight") = 1.0f,
              py::arg("gain_bias") = 1.0f, py::arg("method") = "He", py::arg("device_idx") = 0)
+        .def_readwrite("gain_w", &Linear::gain_w)
+        .def_readwrite("gain_b", &Linear::gain_b)
+        .def_readwrite("init_method", &Linear::init_method)
         .def("init_weight_bias", &Linear::init_weight_bias);
     py::class_<Conv2d, BaseLayer, std::shared_ptr<Conv2d>>(m, "Conv2d")
         .def(py::init<size_t, size_t, size_t, bool, int, int, int, size_t, size_t, float, float,
@@ -120,6 +127,9 @@ PYBIND11_MODULE(cutagi, m) {
              py::arg("padding_type") = 1, py::arg("in_width") = 0, py::arg("in_height") = 0,
              py::arg("gain_weight") = 1.0f, py::arg("gain_bias") = 1.0f,
              py::arg("init_method") = "He", py::arg("device_idx") = 0)
+        .def_readwrite("gain_w", &Conv2d::gain_w)
+        .def_readwrite("gain_b", &Conv2d::gain_b)
+        .def_readwrite("init_method", &Conv2d::init_method)
         .def("init_weight_bias", &Conv2d::init_weight_bias);
     py::class_<ReLU, BaseLayer, std::shared_ptr<ReLU>>(m, "ReLU").def(py::init<>());
     py::class_<MixtureReLU, BaseLayer, std::shared_ptr<MixtureReLU>>(m, "MixtureReLU")
@@ -252,6 +262,7 @@ PYBIND11_MODULE(cutagi, m) {
         .def("save", &Sequential::save)
         .def("load", &Sequential::load)
         .def("save_csv", &Sequential::save_csv)
+        .def("get_norm_mean_var", &Sequential::get_norm_mean_var)
         .def("load_csv", &Sequential::load_csv)
         .def("params_from", &Sequential::params_from)
         .def("parameters", &Sequential::parameters)

@@ -168,10 +168,20 @@ void BatchNorm2dHip::running_mean_var_to_host() {
     d2h(var_norm_batch, d_var_norm_batch, num_features);
 }
 
-std::tuple<std::vector<float>, std::vector<float>, std::vector<float>, std::vector<float>>
-BatchNorm2dHip::get_norm_mean_var() {
+BaseLayer::NormStats BatchNorm2dHip::get_norm_mean_var() {
     this->running_mean_var_to_host();
-    return {mu_ra, var_ra, mu_norm_batch, var_norm_batch};
+    return NormStats({mu_ra}, {var_ra}, {mu_norm_batch}, {var_norm_batch});
+}
+
+// appends the entries of `from` to `to`
+static void append_norm_stats(BaseLayer::NormStats &to, const BaseLayer::NormStats &from) {
+    auto add = [](std::vector<std::vector<float>> &a, const std::vector<std::vector<float>> &b) {
+        a.insert(a.end(), b.begin(), b.end());
+    };
+    add(std::get<0>(to), std::get<0>(from));
+    add(std::get<1>(to), std::get<1>(from));
+    add(std::get<2>(to), std::get<2>(from));
+    add(std::get<3>(to), std::get<3>(from));
 }
 
 // reference: BatchNorm2dCuda::forward, src/batchnorm_layer_cuda.cu:832-967. After a
@@ -570,6 +580,11 @@ int LayerBlock::get_neg_var_w_counter() {
     for (auto &layer : layers) total += layer->get_neg_var_w_counter();
     return total;
 }
+BaseLayer::NormStats LayerBlock::get_norm_mean_var() {
+    NormStats all;
+    for (auto &layer : layers) append_norm_stats(all, layer->get_norm_mean_var());
+    return all;
+}
 void LayerBlock::params_to_device() {
     for (auto &layer : layers) layer->params_to_device();
 }
@@ -789,6 +804,12 @@ void ResNetBlock::preinit_layer() {
 
 int ResNetBlock::get_neg_var_w_counter() {
     return main_block->get_neg_var_w_counter() + (shortcut ? shortcut->get_neg_var_w_counter() : 0);
+}
+
+BaseLayer::NormStats ResNetBlock::get_norm_mean_var() {
+    NormStats all = main_block->get_norm_mean_var();
+    if (shortcut) append_norm_stats(all, shortcut->get_norm_mean_var());
+    return all;
 }
 
 void ResNetBlock::params_to_device() {

@@ -51,6 +51,9 @@ class BatchNorm2d : public BaseLayer {
    public:
     int num_features;
     std::vector<float> mu_ra, var_ra, mu_norm_batch, var_norm_batch;
+    NormStats get_norm_mean_var() override {
+        return NormStats({mu_ra}, {var_ra}, {mu_norm_batch}, {var_norm_batch});
+    }
     float epsilon, momentum, gain_w, gain_b;
 
     BatchNorm2d(int num_features, float eps = 1e-5f, float momentum = 0.9f, bool bias = true,
@@ -87,9 +90,8 @@ class BatchNorm2dHip : public BaseLayerHip {
     void load(std::ifstream &file) override;
     void running_mean_var_to_host();
     void running_mean_var_to_device();
-    // (mu_ra, var_ra, mu_norm_batch, var_norm_batch), refreshed from the device
-    std::tuple<std::vector<float>, std::vector<float>, std::vector<float>, std::vector<float>>
-    get_norm_mean_var();
+    // refreshed from the device
+    NormStats get_norm_mean_var() override;
 
    private:
     void allocate_running_mean_var();
@@ -180,6 +182,7 @@ class LayerBlock : public BaseLayer {
     std::unique_ptr<BaseLayer> to_cuda(int device_idx = 0) override;
     void preinit_layer() override;
     int get_neg_var_w_counter() override;
+    NormStats get_norm_mean_var() override;
     void params_to_device() override;
     void params_to_host() override;
     void delta_params_to_host() override;
@@ -221,6 +224,7 @@ class ResNetBlock : public BaseLayer {
     std::unique_ptr<BaseLayer> to_cuda(int device_idx = 0) override;
     void preinit_layer() override;
     int get_neg_var_w_counter() override;
+    NormStats get_norm_mean_var() override;
     void params_to_device() override;
     void params_to_host() override;
     void delta_params_to_host() override;

@@ -10,6 +10,7 @@
 #include <memory>
 #include <random>
 #include <string>
+#include <tuple>
 #include <vector>
 
 #include "states.h"
@@ -105,6 +106,13 @@ class BaseLayer {
     virtual std::vector<ParameterTuple> parameters();
     virtual void preinit_layer() {}
     virtual int get_neg_var_w_counter() { return neg_var_w_counter; }
+    // Running averages and last batch statistics of the normalisation layers inside
+    // this layer, one entry per such layer: (mu_ra, var_ra, mu_norm_batch,
+    // var_norm_batch). Empty for everything else (reference: include/base_layer.h,
+    // BaseLayer::get_norm_mean_var).
+    using NormStats = std::tuple<std::vector<std::vector<float>>, std::vector<std::vector<float>>,
+                                 std::vector<std::vector<float>>, std::vector<std::vector<float>>>;
+    virtual NormStats get_norm_mean_var() { return NormStats(); }
     // host <-> device copies of the parameters; layers without device storage
     // have nothing to move, blocks pass the call on to their members
     virtual void params_to_device() {}

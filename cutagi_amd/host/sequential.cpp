@@ -495,6 +495,17 @@ void Sequential::load_csv(const std::string &filename) {
     }
 }
 
+// reference: Sequential::get_norm_mean_var, src/sequential.cpp:521-553
+std::unordered_map<std::string, BaseLayer::NormStats> Sequential::get_norm_mean_var() {
+    std::unordered_map<std::string, BaseLayer::NormStats> all;
+    for (size_t i = 0; i < layers.size(); i++) {
+        auto stats = layers[i]->get_norm_mean_var();
+        if (std::get<0>(stats).empty()) continue;
+        all[layers[i]->get_layer_info() + "_" + std::to_string(i)] = stats;
+    }
+    return all;
+}
+
 std::vector<ParameterTuple> Sequential::parameters() {
     std::vector<ParameterTuple> params;
     for (auto &layer : layers) {

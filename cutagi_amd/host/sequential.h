@@ -90,6 +90,8 @@ class Sequential {
     void save(const std::string &filename);
     void load(const std::string &filename);
     void save_csv(const std::string &filename);
+    // per normalisation-carrying layer, keyed `<layer info>_<index>`
+    std::unordered_map<std::string, BaseLayer::NormStats> get_norm_mean_var();
     void load_csv(const std::string &filename);
     std::vector<ParameterTuple> parameters();
     ParameterMap state_dict();

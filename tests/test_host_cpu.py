@@ -101,3 +101,25 @@ def test_device_queries_without_a_device():
         cutagi.set_cuda_device(0)
     with pytest.raises(RuntimeError):
         cutagi.get_cuda_device_memory(0)
+
+
+def test_layer_fields_and_norm_statistics_on_the_host():
+    from cutagi_amd import cutagi as ct
+    lin = ct.Linear(6, 4, True, 0.5, 2.0, "Xavier")
+    assert (lin.gain_w, lin.gain_b, lin.init_method) == (0.5, 2.0, "Xavier")
+    conv = ct.Conv2d(3, 4, 3, False, 1, 1, 1, 8, 8, 0.25, 1.0, "He")
+    assert conv.gain_w == 0.25 and conv.init_method == "He"
+    assert lin.get_norm_mean_var() == ([], [], [], [])
+    main = ct.LayerBlock([ct.Conv2d(4, 8, 3, False, 2, 1, 2), ct.ReLU(), ct.BatchNorm2d(8)])
+    net = ct.Sequential([conv, ct.BatchNorm2d(4), ct.MixtureReLU(),
+                         ct.ResNetBlock(main, ct.LayerBlock([ct.Conv2d(4, 8, 2, False, 2),
+                                                             ct.BatchNorm2d(8)])),
+                         ct.AvgPool2d(4), ct.Linear(8, 5)])
+    stats = net.get_norm_mean_var()
+    assert sorted(stats) == ["BatchNorm2d()_1", "ResNetBlock(256,128)_3"]
+    mu_ra, var_ra, mu_nb, var_nb = stats["ResNetBlock(256,128)_3"]
+    assert [len(v) for v in mu_ra] == [8, 8] and [len(v) for v in var_nb] == [8, 8]
+    assert [len(v) for v in stats["BatchNorm2d()_1"][1]] == [4]
+    if not ct.is_cuda_available():
+        with pytest.raises(RuntimeError):
+            lin.to_cuda()

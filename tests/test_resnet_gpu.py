@@ -178,4 +178,4 @@ def test_resnet18_full_size_step():
         assert np.all(np.isfinite(mu_w)) and min(var_w) > 0, key
         if len(var_b):
             assert np.all(np.isfinite(mu_b)) and min(var_b) > 0, key
-    assert min(net.layers[2].get_norm_mean_var()[1]) > 0
+    assert min(net.layers[2].get_norm_mean_var()[1][0]) > 0  # one entry per norm layer
