@@ -8,11 +8,16 @@ sequential.py, linear.py, conv2d.py, activation.py, batch_norm.py, pooling.py,
 layer_block.py, resnet_block.py, output_updater.py). The wrappers add no
 arithmetic; every call goes to the C++ host classes, which call the HIP library.
 
+``Utils`` and ``HRCSoftmaxMetric`` are the label helpers of the reference's
+``pytagi`` package that the README classification example uses (hierarchical
+softmax encoding, class probabilities, error rate).
+
 Not here, because they are outside the Linear / Conv2d path: the other layer
 families of pytagi.nn (LSTM, attention, normalisations other than BatchNorm2d,
-max pooling, further activations), DDP, ``OutputUpdater.update_heteros`` and the
-metric helpers.
+max pooling, further activations), DDP and ``OutputUpdater.update_heteros``.
 """
+import math
+
 import numpy as np
 
 from . import cutagi
@@ -189,6 +194,9 @@ class Sequential:
     def get_neg_var_w_counter(self):
         return self._cpp_backend.get_neg_var_w_counter()
 
+    def get_norm_mean_var(self):
+        return self._cpp_backend.get_norm_mean_var()
+
     def save(self, filename):
         self._cpp_backend.save(filename)
 
@@ -250,18 +258,67 @@ class OutputUpdater:
         self._cpp_backend.device = value
 
 
+class HRCSoftmax:
+    """Binary-tree encoding of the class labels: ``obs`` (+-1 per level), ``idx``
+    (1-based output unit per level), ``num_obs`` levels, ``len`` output units."""
+
+    def __init__(self, num_classes):
+        obs, idx, self.num_obs, self.len = hrc_softmax(num_classes)
+        self.obs, self.idx = obs, idx       # [classes][num_obs]
+
+
 class Utils:
-    """The two label helpers of the reference's ``pytagi.Utils`` that a
-    classification step needs (pytagi/tagi_utils.py:24-48,181-191)."""
+    """Label helpers of the reference's ``pytagi.Utils`` for hierarchical-softmax
+    classification (pytagi/tagi_utils.py:24-48,108-215 over src/cost.cpp:76-246)."""
 
     def get_hierarchical_softmax(self, num_classes):
-        """(obs [classes][n_obs], idx [classes][n_obs] 1-based, n_obs, n_outputs)."""
-        return hrc_softmax(num_classes)
+        return HRCSoftmax(num_classes)
 
     def label_to_obs(self, labels, num_classes):
         """Observations (+-1) and 1-based output indices of each label's path in the
         binary tree, flattened sample by sample, and the path length."""
-        obs, idx, n_obs, _ = hrc_softmax(num_classes)
+        hs = HRCSoftmax(num_classes)
         labels = np.asarray(labels, dtype=np.int64).ravel()
-        return (np.ascontiguousarray(obs[labels].ravel(), np.float32),
-                np.ascontiguousarray(idx[labels].ravel(), np.int32), n_obs)
+        return (np.ascontiguousarray(hs.obs[labels].ravel(), np.float32),
+                np.ascontiguousarray(hs.idx[labels].ravel(), np.int32), hs.num_obs)
+
+    def obs_to_label_prob(self, ma, Sa, hr_softmax, num_classes):
+        """Class probabilities [samples][classes] from the output layer's means and
+        variances: every tree node is a probit with scale 1/3, a class multiplies
+        the branch probabilities along its path (reference: obs_to_class)."""
+        ma = np.asarray(ma, np.float64).reshape(-1, hr_softmax.len)
+        Sa = np.asarray(Sa, np.float64).reshape(-1, hr_softmax.len)
+        z = ma / np.sqrt((1.0 / 3.0) ** 2 + Sa)
+        p_node = 0.5 * np.vectorize(math.erfc)(-z / math.sqrt(2.0))
+        picked = p_node[:, hr_softmax.idx - 1]                      # [samples][classes][levels]
+        branch = np.where(hr_softmax.obs[None] == -1.0, np.abs(picked - 1.0), picked)
+        return branch.prod(axis=2)[:, :num_classes].astype(np.float32)
+
+    def get_labels(self, ma, Sa, hr_softmax, num_classes, batch_size):
+        """Predicted labels and the class probabilities they come from."""
+        prob = self.obs_to_label_prob(ma, Sa, hr_softmax, num_classes)
+        assert prob.shape[0] == batch_size
+        return prob.argmax(axis=1), prob
+
+    def get_errors(self, ma, Sa, labels, hr_softmax, num_classes, batch_size):
+        pred, prob = self.get_labels(ma, Sa, hr_softmax, num_classes, batch_size)
+        return (pred != np.asarray(labels).ravel()).astype(np.int32), prob
+
+
+class HRCSoftmaxMetric:
+    """``metric = HRCSoftmaxMetric(10); metric.error_rate(m_pred, v_pred, label)``
+    (reference: pytagi/metric.py:7-60)."""
+
+    def __init__(self, num_classes):
+        self.num_classes = num_classes
+        self.utils = Utils()
+        self.hrc_softmax = self.utils.get_hierarchical_softmax(num_classes)
+
+    def get_predicted_labels(self, m_pred, v_pred):
+        batch_size = np.asarray(m_pred).size // self.hrc_softmax.len
+        return self.utils.get_labels(m_pred, v_pred, self.hrc_softmax, self.num_classes,
+                                     batch_size)[0]
+
+    def error_rate(self, m_pred, v_pred, label):
+        pred = self.get_predicted_labels(m_pred, v_pred)
+        return float(np.mean(pred != np.asarray(label).ravel()))

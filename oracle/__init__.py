@@ -299,6 +299,18 @@ class Oracle:
         self._fn("class_to_obs")(n_classes, _fp(obs), _ip(idx), ctypes.byref(a), ctypes.byref(b))
         return obs.reshape(n_classes, n_obs), idx.reshape(n_classes, n_obs), a.value, b.value
 
+    def get_error(self, mz, Sz, labels, n_classes):
+        """(errors [B], class probabilities [B][n_classes]) as the reference computes
+        them from the output moments [B][len] (reference build only)."""
+        mz, Sz = f32(mz), f32(Sz)
+        labels = np.ascontiguousarray(labels, np.int32)
+        B, length = labels.size, mz.size // labels.size
+        er = np.zeros(B, np.int32)
+        prob = np.zeros(B * n_classes, np.float32)
+        self._fn("get_error")(_fp(mz), _fp(Sz), _ip(labels), n_classes, B, length, _ip(er),
+                              _fp(prob))
+        return er, prob.reshape(B, n_classes)
+
     # ---- checkpoint files (reference build only) -----------------------------------
     def checkpoint_save(self, model, path):
         """Writes the reference's binary checkpoint of zoo model `model` with the

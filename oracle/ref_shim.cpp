@@ -9,6 +9,7 @@
 #include <fstream>
 #include <memory>
 #include <stdexcept>
+#include <tuple>
 #include <vector>
 
 #include "activation.h"
@@ -633,6 +634,19 @@ int ref_checkpoint_load(int model, const char *path, float *out, int capacity) {
     } catch (const std::exception &) {
         return -1;
     }
+}
+
+// Classification error and class probabilities from the output layer's moments
+// (src/cost.cpp:195-246 over obs_to_class, 150-190). er: [B], prob: [B][n_classes].
+void ref_get_error(const float *mz, const float *Sz, const int *labels, int n_classes, int B,
+                   int len, int *er, float *prob) {
+    std::vector<float> m(mz, mz + (size_t)B * len), S(Sz, Sz + (size_t)B * len);
+    std::vector<int> l(labels, labels + B);
+    std::vector<int> e;
+    std::vector<float> P;
+    std::tie(e, P) = get_error(m, S, l, n_classes, B);
+    std::memcpy(er, e.data(), e.size() * sizeof(int));
+    std::memcpy(prob, P.data(), P.size() * sizeof(float));
 }
 
 // The text format of Sequential::save_csv / load_csv (src/sequential.cpp:612-709):

@@ -38,11 +38,33 @@ def test_wrappers_build_and_forward_fields():
         OutputUpdater("cpu").update_heteros(None, None, None)
 
 
+def test_label_helpers_match_the_reference_cost_functions(ref_lib):
+    """Class probabilities and errors of the hierarchical softmax against the
+    compiled reference (get_error over obs_to_class, src/cost.cpp:150-246)."""
+    if ref_lib is None or not hasattr(ref_lib.lib, "ref_get_error"):
+        pytest.skip("compiled reference not available")
+    from cutagi_amd.nn import HRCSoftmaxMetric, Utils
+    rng = np.random.default_rng(0)
+    for n_classes, n_out in ((10, 11), (4, 3), (7, 7)):
+        B = 50
+        hs = Utils().get_hierarchical_softmax(n_classes)
+        assert hs.len == n_out
+        mz = rng.normal(0, 1, (B, hs.len)).astype(np.float32)
+        Sz = rng.uniform(0.01, 2, (B, hs.len)).astype(np.float32)
+        labels = rng.integers(0, n_classes, B)
+        er, prob = ref_lib.get_error(mz, Sz, labels, n_classes)
+        e2, p2 = Utils().get_errors(mz.ravel(), Sz.ravel(), labels, hs, n_classes, B)
+        assert np.allclose(p2, prob, rtol=1e-5, atol=1e-7) and np.array_equal(e2, er)
+        rate = HRCSoftmaxMetric(n_classes).error_rate(mz.ravel(), Sz.ravel(), labels)
+        assert rate == pytest.approx(er.mean())
+
+
 @pytest.mark.gpu
 def test_readme_training_loop_matches_the_cpp_module():
     from cutagi_amd import cutagi
-    from cutagi_amd.nn import Linear, OutputUpdater, ReLU, Sequential, Utils
+    from cutagi_amd.nn import HRCSoftmaxMetric, Linear, OutputUpdater, ReLU, Sequential, Utils
     batch_size, steps = 32, 3
+    metric = HRCSoftmaxMetric(num_classes=10)
     rng = np.random.default_rng(0)
     xs = rng.normal(0, 1, (steps, batch_size, 784)).astype(np.float32)
     labels = rng.integers(0, 10, (steps, batch_size))
@@ -60,6 +82,7 @@ def test_readme_training_loop_matches_the_cpp_module():
         net.backward()
         net.step()
         preds.append((m_pred, v_pred))
+        assert 0.0 <= metric.error_rate(m_pred, v_pred, labels[i]) <= 1.0
     assert preds[0][0].shape == (batch_size * 11,) and np.all(preds[-1][1] > 0)
     assert not np.array_equal(preds[0][0], preds[-1][0])
 
