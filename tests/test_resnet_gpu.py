@@ -179,3 +179,34 @@ def test_resnet18_full_size_step():
         if len(var_b):
             assert np.all(np.isfinite(mu_b)) and min(var_b) > 0, key
     assert min(net.layers[2].get_norm_mean_var()[1][0]) > 0  # one entry per norm layer
+
+
+def test_resnet18_learns_a_synthetic_classification_task():
+    """The reference's accuracy gate for this model (test/cpp_unit/test_resnet.cpp:
+    267-270: CIFAR error rate below 0.8 after 100 batches of 64), on synthetic images
+    since no dataset travels: noisy copies of ten random prototypes; chance is 0.9."""
+    from cutagi_amd import cutagi
+    from cutagi_amd.nn import HRCSoftmaxMetric, Utils
+    from cutagi_amd.resnet import resnet18_cifar10
+    cutagi.manual_seed(2)
+    rng = np.random.default_rng(2)
+    protos = rng.normal(0, 1, (10, 3 * 32 * 32)).astype(np.float32)
+    net = resnet18_cifar10(cutagi, gain_w=0.1, gain_b=0.1)
+    net.to_device("cuda")
+    updater = cutagi.OutputUpdater(net.device)
+    metric = HRCSoftmaxMetric(10)
+    batch = 64
+    var_y = np.full(batch * 4, 1.0, np.float32)
+    errors = []
+    for _ in range(100):
+        label = rng.integers(0, 10, batch)
+        x = protos[label] + rng.normal(0, 0.5, (batch, 3072)).astype(np.float32)
+        y, idx, _ = Utils().label_to_obs(label, 10)
+        net.forward(x)
+        m_pred, v_pred = net.get_outputs()
+        errors.append(metric.error_rate(m_pred, v_pred, label))
+        updater.update_using_indices(net.output_z_buffer, y, var_y, idx, net.input_delta_z_buffer)
+        net.backward()
+        net.step()
+    assert np.all(np.isfinite(m_pred)) and v_pred.min() >= 0
+    assert np.mean(errors[-20:]) < 0.8, errors[-20:]
