@@ -181,6 +181,7 @@ struct ConvFwdProblem {
     static constexpr bool XK = true, YK = false, PROLOGUE_WRITES_LDS = true, SPLIT_PER_XCD = false;
     static constexpr int VARIANTS = 2;  // 1: sixteen-byte loads of consecutive groups
     __device__ static __forceinline__ void adjust_range(const Params &, const Ctx &, int &, int &) {}
+    __device__ static __forceinline__ int place_tile(const Params &, int tile, int, int) { return tile; }
     // 130 registers without the request: one 64x128 workgroup per CU instead of two
     static constexpr int min_waves_per_simd(int bm, int bn, int waves) {
         return waves == 8 && bm * bn <= 64 * 128 ? 4 : 0;
@@ -261,6 +262,7 @@ struct ConvDwProblem {
     static constexpr bool XK = true, YK = true, PROLOGUE_WRITES_LDS = false, SPLIT_PER_XCD = true;
     static constexpr int VARIANTS = 1;
     __device__ static __forceinline__ void adjust_range(const Params &, const Ctx &, int &, int &) {}
+    __device__ static __forceinline__ int place_tile(const Params &, int tile, int, int) { return tile; }
     static constexpr int min_waves_per_simd(int, int, int) { return 0; }
     static constexpr int NX = 2, NY = 1, FLAVOR = FLAVOR_DELTA_ROWS;
 
@@ -368,6 +370,7 @@ struct ConvDwVecProblem {
     static constexpr bool XK = true, YK = true, PROLOGUE_WRITES_LDS = false, SPLIT_PER_XCD = true;
     static constexpr int VARIANTS = 1;
     __device__ static __forceinline__ void adjust_range(const Params &, const Ctx &, int &, int &) {}
+    __device__ static __forceinline__ int place_tile(const Params &, int tile, int, int) { return tile; }
     // (asking for four or five 64x64 workgroups per CU instead of three measured
     // no gain)
     static constexpr int min_waves_per_simd(int, int, int) { return 0; }
@@ -556,6 +559,13 @@ struct ConvDzProblem {
         build_group_table(
             ctx, tab, taps, bn, n0, p.N, [&](int n) { return dz_column(p, n).b; }, p.woho, p.B, tid,
             nthreads, p.group_loads);
+    }
+    // Tiles of different phases differ in length (4, 2, 2, 1 taps for 3x3 stride 2)
+    // and lie phase by phase. The two slices of a tile tend to land on the same CU;
+    // odd slices walk the tiles backwards, so a CU gets a long and a short one.
+    __device__ static __forceinline__ int place_tile(const Params &p, int tile, int split,
+                                                     int tiles) {
+        return (p.perm_s > 1 && (split & 1)) ? tiles - 1 - tile : tile;
     }
     // The slice [r_begin, r_end) was cut in units of k2 (whole output channels);
     // with `taps` rows per channel it becomes this.

@@ -69,6 +69,7 @@ struct LinearProblem {
     static constexpr bool PROLOGUE_WRITES_LDS = false, SPLIT_PER_XCD = false;
     static constexpr int VARIANTS = 1;
     __device__ static __forceinline__ void adjust_range(const Params &, const Ctx &, int &, int &) {}
+    __device__ static __forceinline__ int place_tile(const Params &, int tile, int, int) { return tile; }
     static constexpr int min_waves_per_simd(int, int, int) { return 0; }
     static size_t extra_lds_bytes(const Params &, int, int) { return 0; }
     __device__ static __forceinline__ void prologue(const Params &, Ctx &, int *, int, int, int,

@@ -29,6 +29,9 @@
 //                               runs once before the first load; a barrier follows
 //   min_waves_per_simd(BM, BN, waves)
 //                               occupancy the register allocation must allow (0: none)
+//   place_tile(p, tile, split, tiles)
+//                               which tile the workgroup (tile, split) of the grid takes
+//                               (a permutation of the tiles for every split)
 //   adjust_range(p, ctx, r_begin, r_end)
 //                               after the prologue: a problem whose reduction is shorter
 //                               for this tile than for others re-states its slice
@@ -328,6 +331,7 @@ void mfma_tile_kernel(typename P::Params p) {
         tile = q % gridDim.x;
         split = (q / gridDim.x) * 8 + (id & 7);
     }
+    tile = P::place_tile(p, tile, split, (int)gridDim.x);
     const int m0 = (tile / tiles_n) * BM, n0 = (tile % tiles_n) * BN;
     const int r_begin = split * p.r_per_split;
     const int r_end = min(p.R, r_begin + p.r_per_split);
