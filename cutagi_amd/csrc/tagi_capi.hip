@@ -271,7 +271,7 @@ static int linear_bwd_dz_impl(const float *mu_w, const float *jcb, const float *
         int rc = workspace_get(2 * part * sizeof(float), &ws);
         if (rc != TAGI_OK) return rc;
         TAGI_TRY(launch_gemv_dz(mu_w, delta_mu, delta_var, K, N, B, splits,
-                                (g_tune.gemv_rev >= 0 ? g_tune.gemv_rev : 8) & 3, ws, ws + part,
+                                (g_tune.gemv_rev >= 0 ? g_tune.gemv_rev : 0) & 3, ws, ws + part,
                                 stream));
         if (defer != nullptr && aligned16(jcb) && aligned16(delta_mu_z) && aligned16(delta_var_z)) {
             defer->ws0 = ws; defer->ws1 = ws + part; defer->jcb = jcb;
@@ -315,7 +315,7 @@ static int linear_bwd_dw_impl(const float *var_w, const float *mu_a, const float
 
     if (B <= gemv_max_batch() && k_vec) {
         TAGI_TRY(launch_gemv_dw(var_w, mu_a, delta_mu, delta_var, K, N, B,
-                                ((g_tune.gemv_rev >= 0 ? g_tune.gemv_rev : 8) >> 2) & 3,
+                                ((g_tune.gemv_rev >= 0 ? g_tune.gemv_rev : 0) >> 2) & 3,
                                 delta_mu_w, delta_var_w, var_b, delta_mu_b, delta_var_b, fold,
                                 stream));
         if (bias_done) *bias_done = var_b != nullptr;

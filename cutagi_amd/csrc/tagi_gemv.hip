@@ -266,8 +266,7 @@ __global__ __launch_bounds__(DZ_WAVES * 64) void gemv_dz_kernel(
     constexpr int STAGE = H <= 2 ? DZ_STAGE : DZ_STAGE / 2;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int j = lane & 3;
-    // Row slices are walked from the end of the matrix: a forward pass that just
-    // ran left the last weight rows in the memory-side cache.
+    // (rev bit 0 walks the row slices from the end of the matrix; no gain measured)
     // Workgroup -> (column slab, row slice). Consecutive workgroup ids go to the 8
     // XCDs round-robin; mode 1 gives each XCD runs of 4 adjacent column slabs (4 KB
     // of every row, i.e. all of its L2 channels) instead of every 8th slab.
@@ -422,14 +421,19 @@ __global__ __launch_bounds__(DZ_WAVES * 64) void gemv_dz_kernel(
 // broadcast reads. Per row a wave reads 1 KB of var_w and writes 2 KB
 // (non-temporal: the results are not read again by this kernel).
 //
-// EXACT (K % 256 == 0 and N % rows-per-block == 0): no predicate anywhere, and
-// the var_w rows move through two register stages of DW_STAGE rows used in turn,
-// so a stage's loads are in flight while the other stage is multiplied and
-// stored. The general variant guards every row and column.
+// Workgroups are small (16 rows x 256 columns, a wave loads its 4 rows at once,
+// then multiplies and stores them) and are numbered along the rows of the matrix
+// first: the workgroups resident at any time then sweep a narrow band of rows
+// through var_w and the two results in address order. Measured at 8192 x 8192,
+// batch 8, forward + backward step: 128 rows per workgroup 283 us, 32 rows 274 us,
+// 16 rows 268 us, 8 rows 279 us.
+//
+// EXACT (K % 256 == 0 and N % 16 == 0): no predicate anywhere. The general
+// variant guards every row and column.
 // ---------------------------------------------------------------------------
 constexpr int DW_COLS_PER_BLOCK = 256;  // 64 lanes x 4 columns, shared by the 4 waves
-constexpr int DW_ROWS_PER_BLOCK = 128;  // 32 rows per wave
-constexpr int DW_STAGE = 4;
+constexpr int DW_ROWS_PER_BLOCK = 16;   // 4 rows per wave
+constexpr int DW_STAGE = 4;             // rows a wave has in flight per register stage
 
 template <int BMAX>
 __device__ __forceinline__ void dw_row(const float4 &vw, const float (*s_dm)[BMAX],
@@ -454,21 +458,37 @@ __global__ __launch_bounds__(256) void gemv_dw_kernel(
     const float *__restrict__ var_w, const float *__restrict__ mu_a,
     const float *__restrict__ dmu, const float *__restrict__ dvar, int K, int N, int B, int rev,
     float *__restrict__ dmu_w, float *__restrict__ dvar_w, const float *__restrict__ var_b,
-    float *__restrict__ dmu_b, float *__restrict__ dvar_b, DzFold fold) {
-    __shared__ __attribute__((aligned(16))) float s_dm[DW_ROWS_PER_BLOCK][BMAX];
+    float *__restrict__ dmu_b, float *__restrict__ dvar_b, DzFold fold, int fold_rows) {
+    constexpr int ROWS = DW_ROWS_PER_BLOCK;
+    __shared__ __attribute__((aligned(16))) float s_dm[ROWS][BMAX];
+    __shared__ __attribute__((aligned(16))) float s_dv[ROWS][BMAX];
     // The state backward that ran before this kernel may have left its slices
-    // unfolded: every workgroup folds its share of them first (a few float4 each),
-    // which saves a launch of its own for that.
-    if (fold.ws0 != nullptr) {
+    // unfolded. The first fold_rows rows of the grid (the first workgroups to be
+    // dispatched) do nothing but fold them, one float4 of the result per thread
+    // and round, while the other workgroups already stream; that saves a launch,
+    // and no streaming workgroup waits for the fold's dependent loads.
+    int id = blockIdx.y * gridDim.x + blockIdx.x;
+    const int nfold = fold_rows * gridDim.x;
+    if (id < nfold) {
         const size_t items = fold.total / 4;
-        const size_t nwg = (size_t)gridDim.x * gridDim.y;
-        const size_t per = (items + nwg - 1) / nwg;
-        const size_t wg = (size_t)blockIdx.y * gridDim.x + blockIdx.x;
-        for (size_t it = threadIdx.x; it < per; it += 256) {
-            const size_t at = (wg * per + it) * 4;
-            if (at >= fold.total) break;
+        for (size_t it = (size_t)id * 256 + threadIdx.x; it < items; it += (size_t)nfold * 256) {
+            const size_t at = it * 4;
             float4 m = zero4(), v = zero4();
-            for (int sl = 0; sl < fold.splits; sl++) {
+            int sl = 0;
+            for (; sl + 4 <= fold.splits; sl += 4) {
+                float4 x[4], y[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    x[u] = ld4(fold.ws0 + (sl + u) * fold.total + at);
+                    y[u] = ld4(fold.ws1 + (sl + u) * fold.total + at);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++) {  // slices are added in index order
+                    m.x += x[u].x; m.y += x[u].y; m.z += x[u].z; m.w += x[u].w;
+                    v.x += y[u].x; v.y += y[u].y; v.z += y[u].z; v.w += y[u].w;
+                }
+            }
+            for (; sl < fold.splits; sl++) {
                 const float4 a = ld4(fold.ws0 + sl * fold.total + at);
                 const float4 b = ld4(fold.ws1 + sl * fold.total + at);
                 m.x += a.x; m.y += a.y; m.z += a.z; m.w += a.w;
@@ -480,13 +500,14 @@ __global__ __launch_bounds__(256) void gemv_dw_kernel(
             *reinterpret_cast<float4 *>(fold.out1 + at) = make_float4(
                 v.x * j.x * j.x, v.y * j.y * j.y, v.z * j.z * j.z, v.w * j.w * j.w);
         }
+        return;
     }
-    __shared__ __attribute__((aligned(16))) float s_dv[DW_ROWS_PER_BLOCK][BMAX];
+    id -= nfold;  // a multiple of gridDim.x: the id's XCD (id % 8) stays when gridDim.x % 8 == 0
+    const int grid_rows = gridDim.y - fold_rows;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     // same XCD-aware choice of the column block as in the state backward
-    int cblock = blockIdx.x, rblock = blockIdx.y;
+    int cblock = id % gridDim.x, rblock = id / gridDim.x;
     if ((rev & 2) && gridDim.x % 32 == 0) {
-        const int id = blockIdx.y * gridDim.x + blockIdx.x;
         const int xcd = id & 7, local = id >> 3;
         const int groups = gridDim.x / 32;
         const int g = local % groups, rest = local / groups;
@@ -494,18 +515,19 @@ __global__ __launch_bounds__(256) void gemv_dw_kernel(
         rblock = rest >> 2;
     }
     const int col = cblock * DW_COLS_PER_BLOCK + lane * 4;
-    const int n0 = ((rev & 1) ? gridDim.y - 1 - rblock : rblock) * DW_ROWS_PER_BLOCK;
+    const int n0 = ((rev & 1) ? grid_rows - 1 - rblock : rblock) * ROWS;
 
-    constexpr int RPW = DW_ROWS_PER_BLOCK / 4;
+    constexpr int RPW = ROWS / 4;  // rows per wave
+    constexpr int STAGE = RPW < DW_STAGE ? RPW : DW_STAGE;
     const int r0 = wave * RPW;
     const float *src = var_w + (size_t)(n0 + r0) * K + col;
-    float4 st[2][DW_STAGE];
-    auto load = [&](float4(&x)[DW_STAGE], int rr) {
+    float4 st[2][STAGE];
+    auto load = [&](float4(&x)[STAGE], int rr) {
 #pragma unroll
-        for (int u = 0; u < DW_STAGE; u++) x[u] = ldw_dw(src + (size_t)(rr + u) * K);
+        for (int u = 0; u < STAGE; u++) x[u] = ldw_dw(src + (size_t)(rr + u) * K);
     };
-    for (int e = threadIdx.x; e < DW_ROWS_PER_BLOCK * BMAX; e += 256) {
-        const int b = e / DW_ROWS_PER_BLOCK, r = e % DW_ROWS_PER_BLOCK;
+    for (int e = threadIdx.x; e < ROWS * BMAX; e += 256) {
+        const int b = e / ROWS, r = e % ROWS;
         const bool ok = b < B && n0 + r < N;
         s_dm[r][b] = ok ? dmu[(size_t)b * N + n0 + r] : 0.f;
         s_dv[r][b] = ok ? dvar[(size_t)b * N + n0 + r] : 0.f;
@@ -522,40 +544,41 @@ __global__ __launch_bounds__(256) void gemv_dw_kernel(
 
     // Bias innovations ride along: the staged innovations of this row block are
     // all that delta_b needs, so the first column block folds them over the batch.
-    if (var_b != nullptr && cblock == 0 && threadIdx.x < DW_ROWS_PER_BLOCK &&
-        n0 + (int)threadIdx.x < N) {
-        const int r = threadIdx.x;
-        float sm = 0.f, sv = 0.f;
+    if (var_b != nullptr && cblock == 0) {
+        for (int r = threadIdx.x; r < ROWS && n0 + r < N; r += 256) {
+            float sm = 0.f, sv = 0.f;
 #pragma unroll
-        for (int b = 0; b < BMAX; b++) {
-            sm += s_dm[r][b];
-            sv += s_dv[r][b];
+            for (int b = 0; b < BMAX; b++) {
+                sm += s_dm[r][b];
+                sv += s_dv[r][b];
+            }
+            const float vb = var_b[n0 + r];
+            dmu_b[n0 + r] = sm * vb;
+            dvar_b[n0 + r] = sv * vb * vb;
         }
-        const float vb = var_b[n0 + r];
-        dmu_b[n0 + r] = sm * vb;
-        dvar_b[n0 + r] = sv * vb * vb;
     }
 
     if (EXACT) {
         float *dm = dmu_w + (size_t)(n0 + r0) * K + col;
         float *dv = dvar_w + (size_t)(n0 + r0) * K + col;
-        auto flush = [&](const float4(&x)[DW_STAGE], int rr) {
+        auto flush = [&](const float4(&x)[STAGE], int rr) {
 #pragma unroll
-            for (int u = 0; u < DW_STAGE; u++)
+            for (int u = 0; u < STAGE; u++)
                 dw_row<BMAX>(x[u], s_dm, s_dv, r0 + rr + u, a, a2, dm + (size_t)(rr + u) * K,
                              dv + (size_t)(rr + u) * K);
         };
+        static_assert(RPW % STAGE == 0, "whole stages per wave");
         load(st[0], 0);
 #pragma unroll 1
-        for (int rr = 0; rr < RPW; rr += 2 * DW_STAGE) {
-            load(st[1], rr + DW_STAGE);
+        for (int rr = 0; rr < RPW; rr += 2 * STAGE) {
+            const bool second = rr + STAGE < RPW;
+            if (second) load(st[1], rr + STAGE);
             __builtin_amdgcn_sched_barrier(0);
             flush(st[0], rr);
             __builtin_amdgcn_sched_barrier(0);
-            // the last pair prefetches nothing new: re-reads its own first rows
-            load(st[0], rr + 2 * DW_STAGE < RPW ? rr + 2 * DW_STAGE : rr);
+            if (rr + 2 * STAGE < RPW) load(st[0], rr + 2 * STAGE);
             __builtin_amdgcn_sched_barrier(0);
-            flush(st[1], rr + DW_STAGE);
+            if (second) flush(st[1], rr + STAGE);
             __builtin_amdgcn_sched_barrier(0);
         }
     } else {
@@ -678,16 +701,31 @@ hipError_t launch_gemv_dz(const float *mu_w, const float *dmu, const float *dvar
 }
 
 template <int BMAX>
-static void dw_launch(bool exact, dim3 grid, hipStream_t stream, const float *var_w,
-                      const float *mu_a, const float *dmu, const float *dvar, int K, int N, int B,
-                      int rev, float *dmu_w, float *dvar_w, const float *var_b, float *dmu_b,
-                      float *dvar_b, const DzFold &fold) {
+static void dw_launch(const float *var_w, const float *mu_a, const float *dmu, const float *dvar,
+                      int K, int N, int B, int rev, float *dmu_w, float *dvar_w,
+                      const float *var_b, float *dmu_b, float *dvar_b, const DzFold &fold,
+                      hipStream_t stream) {
+    dim3 grid((K + DW_COLS_PER_BLOCK - 1) / DW_COLS_PER_BLOCK,
+              (N + DW_ROWS_PER_BLOCK - 1) / DW_ROWS_PER_BLOCK);
+    const bool exact = (K % DW_COLS_PER_BLOCK == 0) && (N % DW_ROWS_PER_BLOCK == 0);
+    // grid rows that only fold the state backward's slices: about 64 workgroups,
+    // not more than one float4 of the result per thread asks for
+    int fold_rows = 0;
+    if (fold.ws0 != nullptr) {
+        const size_t wgs = (fold.total / 4 + 255) / 256;
+        const size_t want = wgs < 64 ? wgs : 64;
+        fold_rows = (int)((want + grid.x - 1) / grid.x);
+        if (fold_rows < 1) fold_rows = 1;
+        grid.y += fold_rows;
+    }
     if (exact)
         hipLaunchKernelGGL((gemv_dw_kernel<BMAX, true>), grid, dim3(256), 0, stream, var_w, mu_a,
-                           dmu, dvar, K, N, B, rev, dmu_w, dvar_w, var_b, dmu_b, dvar_b, fold);
+                           dmu, dvar, K, N, B, rev, dmu_w, dvar_w, var_b, dmu_b, dvar_b, fold,
+                           fold_rows);
     else
         hipLaunchKernelGGL((gemv_dw_kernel<BMAX, false>), grid, dim3(256), 0, stream, var_w, mu_a,
-                           dmu, dvar, K, N, B, rev, dmu_w, dvar_w, var_b, dmu_b, dvar_b, fold);
+                           dmu, dvar, K, N, B, rev, dmu_w, dvar_w, var_b, dmu_b, dvar_b, fold,
+                           fold_rows);
 }
 
 hipError_t launch_gemv_dw(const float *var_w, const float *mu_a, const float *dmu,
@@ -695,18 +733,15 @@ hipError_t launch_gemv_dw(const float *var_w, const float *mu_a, const float *dm
                           float *dvar_w, const float *var_b, float *dmu_b, float *dvar_b,
                           const DzFold *fold_in, hipStream_t stream) {
     const DzFold fold = fold_in ? *fold_in : DzFold();
-    dim3 grid((K + DW_COLS_PER_BLOCK - 1) / DW_COLS_PER_BLOCK,
-              (N + DW_ROWS_PER_BLOCK - 1) / DW_ROWS_PER_BLOCK);
-    const bool exact = (K % DW_COLS_PER_BLOCK == 0) && (N % DW_ROWS_PER_BLOCK == 0);
     if (B <= 4)
-        dw_launch<4>(exact, grid, stream, var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w,
-                      var_b, dmu_b, dvar_b, fold);
+        dw_launch<4>(var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w, var_b, dmu_b, dvar_b,
+                     fold, stream);
     else if (B <= 8)
-        dw_launch<8>(exact, grid, stream, var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w,
-                      var_b, dmu_b, dvar_b, fold);
+        dw_launch<8>(var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w, var_b, dmu_b, dvar_b,
+                     fold, stream);
     else
-        dw_launch<16>(exact, grid, stream, var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w,
-                      var_b, dmu_b, dvar_b, fold);
+        dw_launch<16>(var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w, var_b, dmu_b, dvar_b,
+                      fold, stream);
     return hipGetLastError();
 }
 
