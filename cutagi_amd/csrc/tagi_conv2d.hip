@@ -179,6 +179,7 @@ struct ConvFwdProblem {
     using Params = ConvParams;
     using Ctx = GatherCtx;
     static constexpr bool XK = true, YK = false, PROLOGUE_WRITES_LDS = true, SPLIT_PER_XCD = false;
+    static constexpr bool EPI_PREFETCH = false;
     static constexpr int VARIANTS = 2;  // 1: sixteen-byte loads of consecutive groups
     __device__ static __forceinline__ void adjust_range(const Params &, const Ctx &, int &, int &) {}
     __device__ static __forceinline__ int place_tile(const Params &, int tile, int, int) { return tile; }
@@ -260,6 +261,7 @@ struct ConvDwProblem {
         int nimg[DW_SLOTS][4];  // image offsets b*fi*wihi of the next visit
     };
     static constexpr bool XK = true, YK = true, PROLOGUE_WRITES_LDS = false, SPLIT_PER_XCD = true;
+    static constexpr bool EPI_PREFETCH = true;
     static constexpr int VARIANTS = 1;
     __device__ static __forceinline__ void adjust_range(const Params &, const Ctx &, int &, int &) {}
     __device__ static __forceinline__ int place_tile(const Params &, int tile, int, int) { return tile; }
@@ -340,12 +342,18 @@ struct ConvDwProblem {
         lookup(p, ctx, i, r + KT);
         return make_float4(c[0], c[1], c[2], c[3]);
     }
-    __device__ static __forceinline__ void store(const Params &p, int m, int n, float a0,
-                                                 float a1) {
+    __device__ static __forceinline__ float epi_load(const Params &p, int m, int n) {
+        return p.e0[(size_t)m * p.N + n];
+    }
+    __device__ static __forceinline__ void store_with(const Params &p, int m, int n, float a0,
+                                                      float a1, float e) {
         const size_t at = (size_t)m * p.N + n;
-        const float e = p.e0[at];
         p.out0[at] = a0 * e;
         p.out1[at] = a1 * e * e;
+    }
+    __device__ static __forceinline__ void store(const Params &p, int m, int n, float a0,
+                                                 float a1) {
+        store_with(p, m, n, a0, a1, epi_load(p, m, n));
     }
 };
 
@@ -368,6 +376,7 @@ struct ConvDwVecProblem {
         int ymask[DW_SLOTS];
     };
     static constexpr bool XK = true, YK = true, PROLOGUE_WRITES_LDS = false, SPLIT_PER_XCD = true;
+    static constexpr bool EPI_PREFETCH = true;
     static constexpr int VARIANTS = 1;
     __device__ static __forceinline__ void adjust_range(const Params &, const Ctx &, int &, int &) {}
     __device__ static __forceinline__ int place_tile(const Params &, int tile, int, int) { return tile; }
@@ -452,12 +461,18 @@ struct ConvDwVecProblem {
         lookup(p, ctx, i, o);
         return make_float4(c[0], c[1], c[2], c[3]);
     }
-    __device__ static __forceinline__ void store(const Params &p, int m, int n, float a0,
-                                                 float a1) {
+    __device__ static __forceinline__ float epi_load(const Params &p, int m, int n) {
+        return p.e0[(size_t)m * p.N + n];
+    }
+    __device__ static __forceinline__ void store_with(const Params &p, int m, int n, float a0,
+                                                      float a1, float e) {
         const size_t at = (size_t)m * p.N + n;
-        const float e = p.e0[at];
         p.out0[at] = a0 * e;
         p.out1[at] = a1 * e * e;
+    }
+    __device__ static __forceinline__ void store(const Params &p, int m, int n, float a0,
+                                                 float a1) {
+        store_with(p, m, n, a0, a1, epi_load(p, m, n));
     }
 };
 
@@ -499,6 +514,7 @@ struct ConvDzProblem {
     using Params = ConvParams;
     using Ctx = GatherCtx;
     static constexpr bool XK = true, YK = false, PROLOGUE_WRITES_LDS = true, SPLIT_PER_XCD = false;
+    static constexpr bool EPI_PREFETCH = true;
     static constexpr int VARIANTS = 2;  // 1: sixteen-byte loads of consecutive groups
     static constexpr int min_waves_per_simd(int, int, int) { return 0; }
     __device__ static __forceinline__ bool variant(const Ctx &ctx) { return ctx.fast != 0; }
@@ -607,13 +623,22 @@ struct ConvDzProblem {
         return gather_cols(arr ? p.d1 : p.d0, ctx, V, i, row, r, r_end,
                            max(p.fo * ctx.taps, 1), max(ctx.taps, 1), p.woho);
     }
-    __device__ static __forceinline__ void store(const Params &p, int m, int n, float a0,
-                                                 float a1) {
+    __device__ static __forceinline__ size_t out_index(const Params &p, int m, int n) {
         const DzColumn c = dz_column(p, n);
-        const size_t at = ((size_t)c.b * p.fi + m) * p.wihi + c.px;
-        const float e = p.e0[at];
+        return ((size_t)c.b * p.fi + m) * p.wihi + c.px;
+    }
+    __device__ static __forceinline__ float epi_load(const Params &p, int m, int n) {
+        return p.e0[out_index(p, m, n)];
+    }
+    __device__ static __forceinline__ void store_with(const Params &p, int m, int n, float a0,
+                                                      float a1, float e) {
+        const size_t at = out_index(p, m, n);
         p.out0[at] = a0 * e;
         p.out1[at] = a1 * e * e;
+    }
+    __device__ static __forceinline__ void store(const Params &p, int m, int n, float a0,
+                                                 float a1) {
+        store_with(p, m, n, a0, a1, epi_load(p, m, n));
     }
 };
 

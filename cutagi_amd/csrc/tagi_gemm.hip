@@ -88,6 +88,17 @@ struct LinearProblem {
         if (FULL) return load4_full<YK>(arr ? p.y1 : p.y0, p.ldy, n0 + row, p.N, r);
         return load4<YK, VEC>(arr ? p.y1 : p.y0, p.ldy, n0 + row, p.N, r, r_end);
     }
+    // delta_z / delta_w: the Jacobian / var_w element that scales an output
+    static constexpr bool EPI_PREFETCH = (MODE != GEMM_FWD);
+    __device__ static __forceinline__ float epi_load(const Params &p, int m, int n) {
+        return p.e0[(size_t)m * p.ldo + n];
+    }
+    __device__ static __forceinline__ void store_with(const Params &p, int m, int n, float a0,
+                                                      float a1, float e) {
+        const size_t at = (size_t)m * p.ldo + n;
+        p.out0[at] = a0 * e;
+        p.out1[at] = a1 * (e * e);
+    }
     __device__ static __forceinline__ void store(const Params &p, int m, int n, float a0,
                                                  float a1) {
         const size_t at = (size_t)m * p.ldo + n;

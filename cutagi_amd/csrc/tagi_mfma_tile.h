@@ -29,6 +29,9 @@
 //                               runs once before the first load; a barrier follows
 //   min_waves_per_simd(BM, BN, waves)
 //                               occupancy the register allocation must allow (0: none)
+//   EPI_PREFETCH, epi_load(p, row, col), store_with(p, row, col, a0, a1, e)
+//                               optional: the epilogue's per-element operand, loaded
+//                               for a whole fragment before its stores
 //   place_tile(p, tile, split, tiles)
 //                               which tile the workgroup (tile, split) of the grid takes
 //                               (a permutation of the tiles for every split)
@@ -137,15 +140,47 @@ __device__ __forceinline__ void tile_epilogue(const typename P::Params &p,
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wrow = (wave / WN) * (TM * 32), wcol = (wave % WN) * (TN * 32);
     const bool partial = p.splits > 1;
+    // a tile inside the matrix needs no per-element bounds checks
+    const bool inside = m0 + BM <= p.M && n0 + BN <= p.N;
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const int col = n0 + wcol + j * 32 + (lane & 31);
+            const int row0 = m0 + wrow + i * 32 + 4 * (lane >> 5);  // + 8*(v/4) + v%4
+            if (inside) {
+                if (partial) {
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        const int row = row0 + 8 * (v / 4) + (v % 4);
+                        const size_t at = ((size_t)split * p.M + row) * p.N + col;
+                        p.ws0[at] = acc0[i][j][v];
+                        p.ws1[at] = acc1[i][j][v];
+                    }
+                    continue;
+                }
+                if constexpr (P::EPI_PREFETCH) {
+                    // the epilogue operands of the fragment are all requested before the
+                    // stores that use them: a load that follows a store waits for it
+                    constexpr int EPI_BATCH = 16;
+#pragma unroll
+                    for (int h = 0; h < 16; h += EPI_BATCH) {
+                        float e[EPI_BATCH];
+#pragma unroll
+                        for (int v = h; v < h + EPI_BATCH; v++)
+                            e[v - h] = P::epi_load(p, row0 + 8 * (v / 4) + (v % 4), col);
+#pragma unroll
+                        for (int v = h; v < h + EPI_BATCH; v++)
+                            P::store_with(p, row0 + 8 * (v / 4) + (v % 4), col, acc0[i][j][v],
+                                          acc1[i][j][v], e[v - h]);
+                    }
+                    continue;
+                }
+            }
             if (col >= p.N) continue;
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int row = m0 + wrow + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v % 4);
+                const int row = row0 + 8 * (v / 4) + (v % 4);
                 if (row >= p.M) continue;
                 if (partial) {
                     const size_t at = ((size_t)split * p.M + row) * p.N + col;
