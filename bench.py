@@ -41,11 +41,11 @@ WORKLOADS = {
 # profiles/.
 MEASURED_TRAFFIC_BYTES = {
     ("gemm", "fwd"): 235.0e6,      # algorithmic 151.0e6
-    ("gemm", "bwd_dw"): 284.0e6,   # algorithmic 213.9e6
-    ("gemm", "bwd_dz"): 168.0e6,   # algorithmic 88.1e6
-    ("skinny", "fwd"): 562.5e6,    # algorithmic 536.9e6
-    ("skinny", "bwd_dz"): 286.5e6, # algorithmic 268.4e6
-    ("skinny", "bwd_dw"): 820.7e6, # algorithmic 805.3e6
+    ("gemm", "bwd_dw"): 285.8e6,   # algorithmic 213.9e6
+    ("gemm", "bwd_dz"): 167.9e6,   # algorithmic 88.1e6
+    ("skinny", "fwd"): 562.2e6,    # algorithmic 536.9e6
+    ("skinny", "bwd_dz"): 286.3e6, # algorithmic 268.4e6
+    ("skinny", "bwd_dw"): 815.3e6, # algorithmic 805.3e6
 }
 
 # Conv2d 3x3, stride 1, pad 1, 64 -> 64 channels on 32x32 maps, batch 128, no bias
