@@ -583,12 +583,20 @@ __global__ __launch_bounds__(256) void gemv_dw_kernel(
         }
     } else {
         if (!col_ok) return;
+        // all rows of the wave are requested before the first store (a load that
+        // follows a store would wait for it)
+        float4 vw[RPW];
+#pragma unroll
         for (int rr = 0; rr < RPW; rr++) {
             const int n = n0 + r0 + rr;
-            if (n >= N) break;
-            const float4 vw = ld4(var_w + (size_t)n * K + col);
-            dw_row<BMAX>(vw, s_dm, s_dv, r0 + rr, a, a2, dmu_w + (size_t)n * K + col,
-                         dvar_w + (size_t)n * K + col);
+            vw[rr] = n < N ? ld4(var_w + (size_t)n * K + col) : zero4();
+        }
+#pragma unroll
+        for (int rr = 0; rr < RPW; rr++) {
+            const int n = n0 + r0 + rr;
+            if (n < N)
+                dw_row<BMAX>(vw[rr], s_dm, s_dv, r0 + rr, a, a2, dmu_w + (size_t)n * K + col,
+                             dvar_w + (size_t)n * K + col);
         }
     }
 }
