@@ -13,6 +13,8 @@ SHAPES = [
     (256, 256, 128), (512, 384, 256), (100, 36, 40), (785, 600, 16), (784, 128, 32),
     (128, 128, 32), (128, 11, 32), (64, 32, 1), (256, 512, 8), (1024, 256, 5),
     (516, 260, 16), (130, 70, 17), (5, 3, 2), (4, 4, 4), (333, 129, 77),
+    # skinny path: several grid rows of fold workgroups, ragged row blocks, one row block
+    (2048, 48, 7), (768, 1000, 3), (4096, 16, 16), (260, 20, 9),
 ]
 
 
