@@ -84,7 +84,13 @@ int pick_splits(int tiles, int reduction, int forced, int min_tiles = 8) {
     const int kt = gemm_k_tile();
     const int k_tiles = ceil_div(reduction, kt);
     int s = forced > 0 ? forced : ceil_div(2 * NUM_CU, tiles);
-    const int cap = k_tiles / min_tiles > 0 ? k_tiles / min_tiles : 1;
+    int cap = k_tiles / min_tiles > 0 ? k_tiles / min_tiles : 1;
+    // A launch that leaves most of the chip empty is bound by the latency of its
+    // k-tile loop (one memory round trip per k-tile, nothing else on the CU to hide
+    // it), not by throughput: such a launch is cut into single k-tiles when its
+    // reduction is long enough to pay for the fold (784 -> 128, batch 32: forward
+    // 31 -> 12 us).
+    if (tiles * 8 <= NUM_CU && k_tiles >= 8) cap = k_tiles < 32 ? k_tiles : 32;
     if (forced <= 0 && s > cap) s = cap;
     if (s > k_tiles) s = k_tiles;
     if (s < 1) s = 1;
