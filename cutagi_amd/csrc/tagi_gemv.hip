@@ -458,17 +458,17 @@ __global__ __launch_bounds__(256) void gemv_dw_kernel(
     const float *__restrict__ var_w, const float *__restrict__ mu_a,
     const float *__restrict__ dmu, const float *__restrict__ dvar, int K, int N, int B, int rev,
     float *__restrict__ dmu_w, float *__restrict__ dvar_w, const float *__restrict__ var_b,
-    float *__restrict__ dmu_b, float *__restrict__ dvar_b, DzFold fold, int fold_rows) {
+    float *__restrict__ dmu_b, float *__restrict__ dvar_b, DzFold fold, int col_blocks,
+    int nfold) {
     constexpr int ROWS = DW_ROWS_PER_BLOCK;
     __shared__ __attribute__((aligned(16))) float s_dm[ROWS][BMAX];
     __shared__ __attribute__((aligned(16))) float s_dv[ROWS][BMAX];
     // The state backward that ran before this kernel may have left its slices
-    // unfolded. The first fold_rows rows of the grid (the first workgroups to be
-    // dispatched) do nothing but fold them, one float4 of the result per thread
-    // and round, while the other workgroups already stream; that saves a launch,
-    // and no streaming workgroup waits for the fold's dependent loads.
-    int id = blockIdx.y * gridDim.x + blockIdx.x;
-    const int nfold = fold_rows * gridDim.x;
+    // unfolded. The first nfold workgroups of the (one-dimensional) grid, the first
+    // to be dispatched, do nothing but fold them, one float4 of the result per
+    // thread and round, while the other workgroups already stream; that saves a
+    // launch, and no streaming workgroup waits for the fold's dependent loads.
+    int id = blockIdx.x;
     if (id < nfold) {
         const size_t items = fold.total / 4;
         for (size_t it = (size_t)id * 256 + threadIdx.x; it < items; it += (size_t)nfold * 256) {
@@ -502,14 +502,14 @@ __global__ __launch_bounds__(256) void gemv_dw_kernel(
         }
         return;
     }
-    id -= nfold;  // a multiple of gridDim.x: the id's XCD (id % 8) stays when gridDim.x % 8 == 0
-    const int grid_rows = gridDim.y - fold_rows;
+    id -= nfold;  // a multiple of 8 (launcher): the id's XCD (id % 8) stays
+    const int grid_rows = ((int)gridDim.x - nfold) / col_blocks;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     // same XCD-aware choice of the column block as in the state backward
-    int cblock = id % gridDim.x, rblock = id / gridDim.x;
-    if ((rev & 2) && gridDim.x % 32 == 0) {
+    int cblock = id % col_blocks, rblock = id / col_blocks;
+    if ((rev & 2) && col_blocks % 32 == 0) {
         const int xcd = id & 7, local = id >> 3;
-        const int groups = gridDim.x / 32;
+        const int groups = col_blocks / 32;
         const int g = local % groups, rest = local / groups;
         cblock = g * 32 + xcd * 4 + (rest & 3);
         rblock = rest >> 2;
@@ -713,27 +713,25 @@ static void dw_launch(const float *var_w, const float *mu_a, const float *dmu, c
                       int K, int N, int B, int rev, float *dmu_w, float *dvar_w,
                       const float *var_b, float *dmu_b, float *dvar_b, const DzFold &fold,
                       hipStream_t stream) {
-    dim3 grid((K + DW_COLS_PER_BLOCK - 1) / DW_COLS_PER_BLOCK,
-              (N + DW_ROWS_PER_BLOCK - 1) / DW_ROWS_PER_BLOCK);
+    const int col_blocks = (K + DW_COLS_PER_BLOCK - 1) / DW_COLS_PER_BLOCK;
+    const int row_blocks = (N + DW_ROWS_PER_BLOCK - 1) / DW_ROWS_PER_BLOCK;
     const bool exact = (K % DW_COLS_PER_BLOCK == 0) && (N % DW_ROWS_PER_BLOCK == 0);
-    // grid rows that only fold the state backward's slices: about 64 workgroups,
-    // not more than one float4 of the result per thread asks for
-    int fold_rows = 0;
+    // workgroups that only fold the state backward's slices: 64, or as many as one
+    // float4 of the result per thread asks for
+    int nfold = 0;
     if (fold.ws0 != nullptr) {
         const size_t wgs = (fold.total / 4 + 255) / 256;
-        const size_t want = wgs < 64 ? wgs : 64;
-        fold_rows = (int)((want + grid.x - 1) / grid.x);
-        if (fold_rows < 1) fold_rows = 1;
-        grid.y += fold_rows;
+        nfold = wgs < 64 ? (int)((wgs + 7) / 8 * 8) : 64;
     }
+    const dim3 grid((unsigned)((size_t)col_blocks * row_blocks + nfold));
     if (exact)
         hipLaunchKernelGGL((gemv_dw_kernel<BMAX, true>), grid, dim3(256), 0, stream, var_w, mu_a,
                            dmu, dvar, K, N, B, rev, dmu_w, dvar_w, var_b, dmu_b, dvar_b, fold,
-                           fold_rows);
+                           col_blocks, nfold);
     else
         hipLaunchKernelGGL((gemv_dw_kernel<BMAX, false>), grid, dim3(256), 0, stream, var_w, mu_a,
                            dmu, dvar, K, N, B, rev, dmu_w, dvar_w, var_b, dmu_b, dvar_b, fold,
-                           fold_rows);
+                           col_blocks, nfold);
 }
 
 hipError_t launch_gemv_dw(const float *var_w, const float *mu_a, const float *dmu,
