@@ -63,6 +63,7 @@ struct Tuning {
     // bits 0-1: state backward, bits 2-3: weight backward; low bit of each pair:
     // walk rows from the end, high bit: XCD-aware column mapping
     int gemv_rev = -1;
+    int dw_side = -1;   // 0: bias innovations and the state-backward fold as launches of their own
 };
 Tuning g_tune;
 
@@ -99,17 +100,27 @@ int pick_splits(int tiles, int reduction, int forced, int min_tiles = 8) {
 
 int gemv_max_batch() { return g_tune.gemv_max_batch >= 0 ? g_tune.gemv_max_batch : 16; }
 
-// Tiled MFMA launch + (when sliced) the fold of the partial sums.
-int run_gemm(GemmMode mode, GemmParams p, bool vec, int forced_splits, hipStream_t stream) {
+// Tile shape and reduction slices of a tiled launch.
+void plan_gemm(GemmMode mode, GemmParams &p, int forced_splits, int *tile_out) {
     const int tile = pick_tile(p.M);
     const int tiles = ceil_div(p.M, gemm_tile_rows(tile)) * ceil_div(p.N, gemm_tile_cols(tile));
     const int kt = gemm_k_tile();
     int splits = (mode == GEMM_DW && forced_splits <= 0) ? 1
                                                           : pick_splits(tiles, p.R, forced_splits);
-    int per = ceil_div(ceil_div(p.R, splits), kt) * kt;
-    splits = ceil_div(p.R, per);
-    p.splits = splits;
+    const int per = ceil_div(ceil_div(p.R, splits), kt) * kt;
+    p.splits = ceil_div(p.R, per);
     p.r_per_split = per;
+    *tile_out = tile;
+}
+
+// Tiled MFMA launch + (when sliced) the fold of the partial sums. With `defer`
+// given (state backward), a fold that the 16-byte path can do is left to a later
+// kernel and described in *defer instead.
+int run_gemm(GemmMode mode, GemmParams p, bool vec, int forced_splits, hipStream_t stream,
+             DzFold *defer = nullptr) {
+    int tile = 0;
+    plan_gemm(mode, p, forced_splits, &tile);
+    const int splits = p.splits;
     if (splits > 1) {
         float *ws = nullptr;
         const size_t part = (size_t)splits * p.M * p.N;
@@ -120,6 +131,14 @@ int run_gemm(GemmMode mode, GemmParams p, bool vec, int forced_splits, hipStream
     }
     TAGI_TRY(launch_gemm(mode, tile, vec, p, stream));
     if (splits > 1) {
+        const size_t total = (size_t)p.M * p.N;
+        if (defer != nullptr && mode == GEMM_DZ && p.ldo == p.N && total % 4 == 0 &&
+            aligned16(p.e0) && aligned16(p.out0) && aligned16(p.out1)) {
+            defer->ws0 = p.ws0; defer->ws1 = p.ws1; defer->jcb = p.e0;
+            defer->out0 = p.out0; defer->out1 = p.out1;
+            defer->splits = splits; defer->total = total;
+            return TAGI_OK;
+        }
         TAGI_TRY(launch_reduce_splits(mode == GEMM_FWD ? EPI_BIAS : EPI_SCALE, p.ws0, p.ws1,
                                       splits, p.M, p.N, p.e0, p.e1, p.out0, p.out1, p.ldo,
                                       stream));
@@ -195,6 +214,7 @@ int tagi_hip_tune(const char *key, int value) {
     else if (!strcmp(key, "linear.gemv.swizzle")) g_tune.gemv_swz = value;
     else if (!strcmp(key, "linear.gemv.fwd_variant")) g_tune.gemv_fwd_variant = value;
     else if (!strcmp(key, "linear.gemv.reverse")) g_tune.gemv_rev = value;
+    else if (!strcmp(key, "linear.dw_side")) g_tune.dw_side = value;
     else return TAGI_ERR_INVALID_ARG;
     return TAGI_OK;
 }
@@ -295,7 +315,7 @@ static int linear_bwd_dz_impl(const float *mu_w, const float *jcb, const float *
     p.M = B; p.N = K; p.R = N; p.ldx = N; p.ldy = K;
     p.out0 = delta_mu_z; p.out1 = delta_var_z; p.ldo = K;
     p.e0 = jcb; p.e1 = nullptr;
-    return run_gemm(GEMM_DZ, p, vec, g_tune.dz_splits, stream);
+    return run_gemm(GEMM_DZ, p, vec, g_tune.dz_splits, stream, defer);
 }
 
 int tagi_linear_bwd_dz(const float *mu_w, const float *jcb, const float *delta_mu,
@@ -335,6 +355,37 @@ static int linear_bwd_dw_impl(const float *var_w, const float *mu_a, const float
     p.M = N; p.N = K; p.R = B; p.ldx = N; p.ldy = K;
     p.out0 = delta_mu_w; p.out1 = delta_var_w; p.ldo = K;
     p.e0 = var_w; p.e1 = nullptr;
+    // The bias innovations and a pending fold of the state backward ride along
+    // with an unsliced tile launch (its first workgroups do them).
+    GemmParams q = p;
+    int tile = 0;
+    plan_gemm(GEMM_DW, q, g_tune.dw_splits, &tile);
+    const bool want_bias = var_b != nullptr && bias_done != nullptr;
+    const bool want_fold = fold != nullptr && fold_done != nullptr;
+    if (want_fold && q.splits > 1) {
+        // a sliced weight backward takes the workspace the pending slices lie in
+        TAGI_TRY(launch_reduce_splits(EPI_SCALE, fold->ws0, fold->ws1, fold->splits,
+                                      (int)(fold->total / K), K, fold->jcb, nullptr, fold->out0,
+                                      fold->out1, K, stream));
+        *fold_done = true;
+    } else if ((want_bias || want_fold) && g_tune.dw_side != 0 &&
+               gemm_dw_side_supported(tile, vec, q)) {
+        LinearSideWork w;
+        if (want_fold) {
+            w.ws0 = fold->ws0; w.ws1 = fold->ws1; w.jcb = fold->jcb;
+            w.out0 = fold->out0; w.out1 = fold->out1;
+            w.fold_splits = fold->splits; w.fold_total = fold->total;
+        }
+        if (want_bias) {
+            w.var_b = var_b; w.dmu = delta_mu; w.dvar = delta_var;
+            w.dmu_b = delta_mu_b; w.dvar_b = delta_var_b;
+            w.bias_n = N; w.bias_b = B;
+        }
+        TAGI_TRY(launch_gemm_dw_side(q, w, stream));
+        if (want_bias) *bias_done = true;
+        if (want_fold) *fold_done = true;
+        return TAGI_OK;
+    }
     return run_gemm(GEMM_DW, p, vec, g_tune.dw_splits, stream);
 }
 

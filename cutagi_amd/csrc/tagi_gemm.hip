@@ -179,6 +179,103 @@ hipError_t launch_mode(int tile, bool vec, const GemmParams &p, hipStream_t stre
     return launch_tiles<LinearProblem<MODE, false>>(tile, p, stream);
 }
 
+
+// ---------------------------------------------------------------------------
+// Weight backward with the small jobs of the backward call riding along: the
+// first workgroups of the launch (the first to be dispatched) fold the slices a
+// sliced state backward left in the workspace, and sum the bias innovations over
+// the batch, while the others already multiply tiles. That saves two dependent
+// launches per layer (the weight backward needs neither result).
+// ---------------------------------------------------------------------------
+constexpr int SIDE_BIAS_COLS = 64;  // bias columns per side workgroup (8 batch slices each)
+
+template <int NT>
+__device__ __forceinline__ void side_workgroup(const LinearSideWork &w, int id) {
+    if (id < w.bias_wgs) {
+        // delta_b[n] = var_b[n] * sum_b delta[b][n]: NT/64 batch slices of 64 columns,
+        // folded through LDS in slice order
+        constexpr int SL = NT / 64;
+        __shared__ float s0[SL][64], s1[SL][64];
+        const int c = threadIdx.x & 63, slice = threadIdx.x >> 6;
+        const int n = id * SIDE_BIAS_COLS + c;
+        float a0 = 0.f, a1 = 0.f;
+        if (n < w.bias_n) {
+#pragma unroll 4
+            for (int b = slice; b < w.bias_b; b += SL) {
+                a0 += w.dmu[(size_t)b * w.bias_n + n];
+                a1 += w.dvar[(size_t)b * w.bias_n + n];
+            }
+        }
+        s0[slice][c] = a0;
+        s1[slice][c] = a1;
+        __syncthreads();
+        if (slice == 0 && n < w.bias_n) {
+            float m = 0.f, v = 0.f;
+#pragma unroll
+            for (int sl = 0; sl < SL; sl++) {
+                m += s0[sl][c];
+                v += s1[sl][c];
+            }
+            const float vb = w.var_b[n];
+            w.dmu_b[n] = m * vb;
+            w.dvar_b[n] = v * vb * vb;
+        }
+        return;
+    }
+    // fold: out = (sum over slices, in slice order) * jcb, * jcb^2; float4 items
+    const int fid = id - w.bias_wgs, fold_wgs = w.side_wgs - w.bias_wgs;
+    const size_t items = w.fold_total / 4;
+    for (size_t it = (size_t)fid * NT + threadIdx.x; it < items; it += (size_t)fold_wgs * NT) {
+        const size_t at = it * 4;
+        float4 m = make_float4(0.f, 0.f, 0.f, 0.f), v = m;
+        int sl = 0;
+        for (; sl + 4 <= w.fold_splits; sl += 4) {
+            float4 x[4], y[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                x[u] = *reinterpret_cast<const float4 *>(w.ws0 + (sl + u) * w.fold_total + at);
+                y[u] = *reinterpret_cast<const float4 *>(w.ws1 + (sl + u) * w.fold_total + at);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                m.x += x[u].x; m.y += x[u].y; m.z += x[u].z; m.w += x[u].w;
+                v.x += y[u].x; v.y += y[u].y; v.z += y[u].z; v.w += y[u].w;
+            }
+        }
+        for (; sl < w.fold_splits; sl++) {
+            const float4 x = *reinterpret_cast<const float4 *>(w.ws0 + sl * w.fold_total + at);
+            const float4 y = *reinterpret_cast<const float4 *>(w.ws1 + sl * w.fold_total + at);
+            m.x += x.x; m.y += x.y; m.z += x.z; m.w += x.w;
+            v.x += y.x; v.y += y.y; v.z += y.z; v.w += y.w;
+        }
+        const float4 j = *reinterpret_cast<const float4 *>(w.jcb + at);
+        *reinterpret_cast<float4 *>(w.out0 + at) =
+            make_float4(m.x * j.x, m.y * j.y, m.z * j.z, m.w * j.w);
+        *reinterpret_cast<float4 *>(w.out1 + at) =
+            make_float4(v.x * (j.x * j.x), v.y * (j.y * j.y), v.z * (j.z * j.z), v.w * (j.w * j.w));
+    }
+}
+
+template <class P, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM *WN * 64) void linear_dw_side_kernel(GemmParams p,
+                                                                      LinearSideWork w) {
+    const int id = blockIdx.x;
+    if (id < w.side_wgs) {
+        side_workgroup<WM * WN * 64>(w, id);
+        return;
+    }
+    // (side_wgs is a multiple of 8: a tile's workgroup keeps its XCD)
+    tile_workgroup<P, BM, BN, WM, WN>(p, id - w.side_wgs, 0, (int)gridDim.x - w.side_wgs, 1);
+}
+
+template <bool FULL>
+hipError_t launch_dw_side(const GemmParams &p, const LinearSideWork &w, hipStream_t stream) {
+    using P = LinearProblem<GEMM_DW, true, FULL>;
+    const int tiles = ((p.M + 63) / 64) * ((p.N + 127) / 128);
+    hipLaunchKernelGGL((linear_dw_side_kernel<P, 64, 128, 2, 4>), dim3(tiles + w.side_wgs),
+                       dim3(512), 0, stream, p, w);
+    return hipGetLastError();
+}
 }  // namespace
 
 int gemm_tile_rows(int tile) { return tile_rows(tile); }
@@ -194,6 +291,26 @@ hipError_t launch_gemm(GemmMode mode, int tile, bool vec, const GemmParams &p,
         case GEMM_DW: return launch_mode<GEMM_DW>(tile, vec, p, stream);
     }
     return hipErrorInvalidValue;
+}
+
+bool gemm_dw_side_supported(int tile, bool vec, const GemmParams &p) {
+    return tile == TILE_64x128 && vec && p.splits == 1;
+}
+
+hipError_t launch_gemm_dw_side(const GemmParams &p, LinearSideWork w, hipStream_t stream) {
+    // side workgroups: one per 64 bias columns, then up to 64 for the fold (one
+    // float4 of its result per thread and round); padded to a multiple of 8
+    w.bias_wgs = w.var_b != nullptr ? (w.bias_n + SIDE_BIAS_COLS - 1) / SIDE_BIAS_COLS : 0;
+    int fold_wgs = 0;
+    if (w.ws0 != nullptr) {
+        const size_t want = (w.fold_total / 4 + 511) / 512;
+        fold_wgs = want < 64 ? (int)want : 64;
+        if (fold_wgs < 1) fold_wgs = 1;
+    }
+    w.side_wgs = (w.bias_wgs + fold_wgs + 7) / 8 * 8;
+    if (w.ws0 == nullptr) w.fold_total = 0;  // the padding workgroups find nothing to fold
+    const bool full = p.R % KT == 0 && p.M >= 4 && p.N >= 4;
+    return full ? launch_dw_side<true>(p, w, stream) : launch_dw_side<false>(p, w, stream);
 }
 
 hipError_t launch_reduce_splits(Epilogue epi, const float *ws0, const float *ws1, int splits,

@@ -498,7 +498,7 @@ __global__ __launch_bounds__(256) void gemv_dw_kernel(
             *reinterpret_cast<float4 *>(fold.out0 + at) =
                 make_float4(m.x * j.x, m.y * j.y, m.z * j.z, m.w * j.w);
             *reinterpret_cast<float4 *>(fold.out1 + at) = make_float4(
-                v.x * j.x * j.x, v.y * j.y * j.y, v.z * j.z * j.z, v.w * j.w * j.w);
+                v.x * (j.x * j.x), v.y * (j.y * j.y), v.z * (j.z * j.z), v.w * (j.w * j.w));
         }
         return;
     }

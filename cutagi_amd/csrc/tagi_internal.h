@@ -44,6 +44,24 @@ int gemm_k_tile();
 hipError_t launch_gemm(GemmMode mode, int tile, bool vec, const GemmParams &p,
                        hipStream_t stream);
 
+// Small jobs of a Linear backward call that ride along with the tiled weight
+// backward (first workgroups of its launch): the fold of a sliced state backward
+// (out = sum over slices of ws, times jcb / jcb^2; total a multiple of 4, all
+// pointers 16-byte aligned) and the bias innovations. A null ws0 / var_b leaves
+// the job out.
+struct LinearSideWork {
+    const float *ws0 = nullptr, *ws1 = nullptr, *jcb = nullptr;
+    float *out0 = nullptr, *out1 = nullptr;
+    int fold_splits = 0;
+    size_t fold_total = 0;
+    const float *var_b = nullptr, *dmu = nullptr, *dvar = nullptr;
+    float *dmu_b = nullptr, *dvar_b = nullptr;
+    int bias_n = 0, bias_b = 0;
+    int bias_wgs = 0, side_wgs = 0;  // set by the launcher
+};
+bool gemm_dw_side_supported(int tile, bool vec, const GemmParams &p);
+hipError_t launch_gemm_dw_side(const GemmParams &p, LinearSideWork w, hipStream_t stream);
+
 // out = epilogue(sum over splits of ws[s]) for the two accumulators.
 hipError_t launch_reduce_splits(Epilogue epi, const float *ws0, const float *ws1,
                                 int splits, int M, int N, const float *e0,

@@ -340,10 +340,10 @@ __device__ __forceinline__ void mfma_tile_body(const typename P::Params &p, type
 }
 
 
+// What the workgroup (bx, by) of a gx x gy grid of (tiles, reduction slices) does.
 template <class P, int BM, int BN, int WM, int WN>
-__global__ __launch_bounds__(WM *WN * 64)
-__attribute__((amdgpu_waves_per_eu(tile_min_waves<P>(BM, BN, WM * WN))))
-void mfma_tile_kernel(typename P::Params p) {
+__device__ __forceinline__ void tile_workgroup(const typename P::Params &p, int bx, int by, int gx,
+                                               int gy) {
     constexpr bool XK = P::XK, YK = P::YK;
     constexpr int NX = P::NX, NY = P::NY;
     constexpr int NT = WM * WN * 64;
@@ -356,17 +356,17 @@ void mfma_tile_kernel(typename P::Params p) {
     extern __shared__ __attribute__((aligned(16))) int lds_extra[];
 
     const int tiles_n = (p.N + BN - 1) / BN;
-    int tile = blockIdx.x, split = blockIdx.y;
-    if (P::SPLIT_PER_XCD && gridDim.y % 8 == 0) {
+    int tile = bx, split = by;
+    if (P::SPLIT_PER_XCD && gy % 8 == 0) {
         // Workgroups are handed to the 8 XCDs round-robin in launch order. Give all
         // tiles of one reduction slice to one XCD, so that the operands they share
         // are fetched into one L2 instead of eight.
-        const int id = blockIdx.y * gridDim.x + blockIdx.x;
+        const int id = by * gx + bx;
         const int q = id >> 3;
-        tile = q % gridDim.x;
-        split = (q / gridDim.x) * 8 + (id & 7);
+        tile = q % gx;
+        split = (q / gx) * 8 + (id & 7);
     }
-    tile = P::place_tile(p, tile, split, (int)gridDim.x);
+    tile = P::place_tile(p, tile, split, gx);
     const int m0 = (tile / tiles_n) * BM, n0 = (tile % tiles_n) * BN;
     const int r_begin = split * p.r_per_split;
     const int r_end = min(p.R, r_begin + p.r_per_split);
@@ -385,7 +385,12 @@ void mfma_tile_kernel(typename P::Params p) {
     mfma_tile_body<P, BM, BN, WM, WN, 0>(p, ctx, lds_x, lds_y, m0, n0, split, r_lo, r_hi);
 }
 
-
+template <class P, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM *WN * 64)
+__attribute__((amdgpu_waves_per_eu(tile_min_waves<P>(BM, BN, WM * WN))))
+void mfma_tile_kernel(typename P::Params p) {
+    tile_workgroup<P, BM, BN, WM, WN>(p, blockIdx.x, blockIdx.y, gridDim.x, gridDim.y);
+}
 
 // Folds the partial sums of a sliced reduction (ws0/ws1 [split][M][N]) in slice
 // order and hands every output element to the problem's epilogue.

@@ -54,6 +54,32 @@ def test_linear_backward(oracle_lib, K, N, B):
     assert float(out[1].max()) <= 0.0 and float(out[3].max()) <= 0.0 and float(out[5].max()) <= 0.0
 
 
+@pytest.mark.parametrize("K,N,B", [(512, 384, 256), (100, 36, 40), (784, 128, 32)])
+def test_linear_backward_separate_launches(oracle_lib, K, N, B):
+    """The tiled backward with the bias innovations and the state-backward fold as
+    launches of their own (tuning switch) instead of riding along with the weight
+    backward: same results."""
+    import cutagi_amd.functional as F
+    from cutagi_amd import capi
+    d = linear_inputs(K, N, B, seed=K + 3 * N + B, bias=True, jcb_random=True)
+    t = _dev(d)
+    capi.tune("linear.dw_side", 0)
+    try:
+        out = F.linear_bwd(t["mu_w"], t["var_w"], t["var_b"], t["mu_a"], t["jcb"], t["delta_mu"],
+                           t["delta_var"])
+    finally:
+        capi.tune("linear.dw_side", -1)
+    ref = (oracle_lib.linear_bwd_dz(d["mu_w"], d["jcb"], d["delta_mu"], d["delta_var"], threads=4)
+           + oracle_lib.linear_bwd_dw(d["var_w"], d["mu_a"], d["delta_mu"], d["delta_var"], threads=4)
+           + oracle_lib.linear_bwd_db(d["var_b"], d["delta_mu"], d["delta_var"]))
+    for i, (got, want) in enumerate(zip(out, ref)):
+        assert_close(got.cpu().numpy(), want, "output %d" % i)
+    riding = F.linear_bwd(t["mu_w"], t["var_w"], t["var_b"], t["mu_a"], t["jcb"], t["delta_mu"],
+                          t["delta_var"])
+    for a, b in zip(out[:4], riding[:4]):   # same arithmetic, same order: same bits
+        assert bool((a == b).all())
+
+
 def test_linear_backward_skips(oracle_lib):
     """state_update / param_update switches of LinearCuda::backward."""
     import torch
