@@ -48,8 +48,16 @@ const char *tagi_hip_error_string(int code);
 int tagi_hip_workspace_reserve(size_t bytes);
 /* Free the workspaces of all devices. */
 int tagi_hip_shutdown(void);
-/* Kernel-selection knobs for experiments ("linear.splitk", "linear.path", ...);
- * value < 0 restores the built-in heuristic. Unknown keys are an error. */
+/* Kernel-selection knobs for experiments and tests; value < 0 restores the
+ * built-in heuristic, unknown keys are an error. Linear: "linear.tile",
+ * "linear.fwd.splits", "linear.dz.splits", "linear.dw.splits",
+ * "linear.gemv_max_batch" (largest batch of the streaming kernels),
+ * "linear.gemv.swizzle", "linear.gemv.fwd_variant", "linear.gemv.reverse",
+ * "linear.dw_side" (0: bias innovations and the state-backward fold as launches
+ * of their own instead of inside the weight-backward launch). Conv2d:
+ * "conv2d.tile", "conv2d.splits", "conv2d.dw.tile", "conv2d.dw.splits",
+ * "conv2d.group_loads", "conv2d.stencil", "conv2d.phase_order" (0 switches the
+ * named path off). */
 int tagi_hip_tune(const char *key /* host */, int value);
 
 /* ---- Linear -------------------------------------------------------------- */
