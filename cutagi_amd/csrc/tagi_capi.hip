@@ -63,6 +63,7 @@ struct Tuning {
     // bits 0-1: state backward, bits 2-3: weight backward; low bit of each pair:
     // walk rows from the end, high bit: XCD-aware column mapping
     int gemv_rev = -1;
+    int gemv16 = -1;    // 0: 9..16 samples on the 4x4x1 kernels too
     int dw_side = -1;   // 0: bias innovations and the state-backward fold as launches of their own
 };
 Tuning g_tune;
@@ -215,6 +216,7 @@ int tagi_hip_tune(const char *key, int value) {
     else if (!strcmp(key, "linear.gemv.fwd_variant")) g_tune.gemv_fwd_variant = value;
     else if (!strcmp(key, "linear.gemv.reverse")) g_tune.gemv_rev = value;
     else if (!strcmp(key, "linear.dw_side")) g_tune.dw_side = value;
+    else if (!strcmp(key, "linear.gemv16")) g_tune.gemv16 = value;
     else return TAGI_ERR_INVALID_ARG;
     return TAGI_OK;
 }
@@ -233,6 +235,28 @@ int tagi_linear_fwd(const float *mu_w, const float *var_w, const float *mu_b, co
     const float *e0 = bias ? mu_b : nullptr, *e1 = bias ? var_b : nullptr;
     const bool vec = (K % 4 == 0) && aligned16(mu_w) && aligned16(var_w) && aligned16(mu_a) &&
                      aligned16(var_a);
+
+    if (B > 8 && B <= gemv_max_batch() && B <= 16 && vec && g_tune.gemv16 != 0) {
+        // 9..16 samples: the 16-wide streaming kernel
+        const int blocks = ceil_div(N, gemv16_fwd_rows_per_block());
+        const int step = gemv16_fwd_k_step();
+        int splits = g_tune.fwd_splits > 0 ? g_tune.fwd_splits : ceil_div(2 * NUM_CU, blocks);
+        const int max_splits = ceil_div(K, 4 * step);
+        if (splits > max_splits) splits = max_splits;
+        const int min_splits = ceil_div(K, gemv16_fwd_max_slice());
+        if (splits < min_splits) splits = min_splits;
+        const int per = ceil_div(ceil_div(K, splits), step) * step;
+        splits = ceil_div(K, per);
+        float *ws = nullptr;
+        const size_t part = (size_t)splits * B * N;
+        int rc = workspace_get(2 * part * sizeof(float), &ws);
+        if (rc != TAGI_OK) return rc;
+        TAGI_TRY(launch_gemv16_fwd(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, ws, ws + part,
+                                   stream));
+        TAGI_TRY(launch_reduce_splits(EPI_BIAS, ws, ws + part, splits, B, N, e0, e1, mu_z, var_z, N,
+                                      stream));
+        return TAGI_OK;
+    }
 
     if (B <= gemv_max_batch() && vec) {
         // slices: short enough for the LDS-resident activations, and enough of
@@ -282,13 +306,14 @@ static int linear_bwd_dz_impl(const float *mu_w, const float *jcb, const float *
     const bool vec = (K % 4 == 0) && (N % 4 == 0) && aligned16(mu_w) && aligned16(delta_mu) &&
                      aligned16(delta_var);
 
+    const bool wide16 = B > 8 && B <= 16 && g_tune.gemv16 != 0;
     if (B <= gemv_max_batch() && vec) {
-        const int blocks = ceil_div(K, gemv_dz_cols_per_block());
-        const int step = gemv_dz_n_step();
+        const int blocks = ceil_div(K, wide16 ? gemv16_dz_cols_per_block() : gemv_dz_cols_per_block());
+        const int step = wide16 ? gemv16_dz_n_step() : gemv_dz_n_step();
         int splits = g_tune.dz_splits > 0 ? g_tune.dz_splits : ceil_div(NUM_CU, blocks);
         const int max_splits = ceil_div(N, 2 * step);
         if (splits > max_splits) splits = max_splits;
-        const int min_splits = ceil_div(N, gemv_dz_max_slice(B));
+        const int min_splits = ceil_div(N, wide16 ? gemv16_dz_max_slice() : gemv_dz_max_slice(B));
         if (splits < min_splits) splits = min_splits;
         int per = ceil_div(ceil_div(N, splits), step) * step;
         splits = ceil_div(N, per);
@@ -296,9 +321,13 @@ static int linear_bwd_dz_impl(const float *mu_w, const float *jcb, const float *
         const size_t part = (size_t)splits * B * K;
         int rc = workspace_get(2 * part * sizeof(float), &ws);
         if (rc != TAGI_OK) return rc;
-        TAGI_TRY(launch_gemv_dz(mu_w, delta_mu, delta_var, K, N, B, splits,
-                                (g_tune.gemv_rev >= 0 ? g_tune.gemv_rev : 0) & 3, ws, ws + part,
-                                stream));
+        if (wide16)
+            TAGI_TRY(launch_gemv16_dz(mu_w, delta_mu, delta_var, K, N, B, per, splits, ws,
+                                      ws + part, stream));
+        else
+            TAGI_TRY(launch_gemv_dz(mu_w, delta_mu, delta_var, K, N, B, splits,
+                                    (g_tune.gemv_rev >= 0 ? g_tune.gemv_rev : 0) & 3, ws,
+                                    ws + part, stream));
         if (defer != nullptr && aligned16(jcb) && aligned16(delta_mu_z) && aligned16(delta_var_z)) {
             defer->ws0 = ws; defer->ws1 = ws + part; defer->jcb = jcb;
             defer->out0 = delta_mu_z; defer->out1 = delta_var_z;

@@ -605,8 +605,8 @@ __global__ __launch_bounds__(256) void gemv_dw_kernel(
 
 // Forward variants by index: row groups per wave (their chunks per stage are
 // 1, 2, 2, 4: see the launcher's switch).
-constexpr int FWD_VARIANTS = 4;
-static const int kFwdRG[FWD_VARIANTS] = {2, 2, 1, 1};
+constexpr int FWD_VARIANTS = 5;
+static const int kFwdRG[FWD_VARIANTS] = {2, 2, 1, 1, 1};
 
 int gemv_fwd_variants() { return FWD_VARIANTS; }
 int gemv_fwd_rows_per_block(int variant) { return FWD_WAVES * kFwdRG[variant] * 4; }
@@ -653,6 +653,7 @@ static hipError_t fwd_variant(int variant, const float *mu_w, const float *var_w
         case 1: return fwd_launch<H, 2, 2>(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1, stream);
         case 2: return fwd_launch<H, 1, 2>(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1, stream);
         case 3: return fwd_launch<H, 1, 4>(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1, stream);
+        case 4: return fwd_launch<H, 1, 1>(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, swz, ws0, ws1, stream);
     }
     return hipErrorInvalidValue;
 }

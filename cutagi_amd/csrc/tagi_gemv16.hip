@@ -1,0 +1,374 @@
+// Skinny-batch kernels of the TAGI Linear layer for 9 <= B <= 16, gfx950.
+//
+// Same plan as tagi_gemv.hip (the weight matrices stream from HBM once, straight
+// into MFMA operand layout; the few activations / innovations sit in LDS), but on
+// v_mfma_f32_16x16x4_f32: one instruction multiplies a 16 x 4 weight fragment by
+// all (up to) 16 samples, so a wave needs a quarter of the instructions, LDS
+// reads and accumulator registers that sixteen 4x4 blocks of four samples need.
+// Operand layout of the instruction: A[i][k] from lane 16*k + i, B[k][j] from
+// lane 16*k + j, D[4*(l/16) + v][l%16] in register v of lane l.
+//
+// The weight backward of tagi_gemv.hip serves every B <= 16 and is not repeated.
+#include "tagi_internal.h"
+
+namespace tagi {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+namespace {
+
+__device__ __forceinline__ float4 ld4(const float *p) {
+    return *reinterpret_cast<const float4 *>(p);
+}
+__device__ __forceinline__ float4 zero4() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+__device__ __forceinline__ float comp(const float4 &v, int t) {
+    return t == 0 ? v.x : t == 1 ? v.y : t == 2 ? v.z : v.w;
+}
+__device__ __forceinline__ float4 sq4(const float4 &v) {
+    return make_float4(v.x * v.x, v.y * v.y, v.z * v.z, v.w * v.w);
+}
+__device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
+constexpr int W16_WAVES = 8;
+constexpr int W16_SAMPLES = 16;
+
+// ---------------------------------------------------------------------------
+// Forward. Lane (i = l%16, kk = l/16) streams weight row n0 + 16*rg + i and
+// holds the float4 at k = kb + 4*kk: one load instruction covers 16 rows x 64
+// bytes, two of them a full 128-byte line of each row (plain loads: with
+// streaming loads the second half of a line was fetched from memory again, 1.5x
+// the traffic). Component t of that
+// float4 is A[i][kk] of MFMA t, which multiplies reduction elements
+// kb + 4*kk + t against B[kk][j] = the same elements of sample j = l%16, read
+// from LDS as one float4 per lane. The sums over k are complete inside the
+// accumulators: D[row][sample], no cross-lane reduction at the end.
+// ---------------------------------------------------------------------------
+// (measured at 8192 x 8192, batch 16, forward call: RG x C = 1x2 118 us, 2x2 120,
+// 1x4 121, 2x4 124, 4x1 136, 1x8 138)
+constexpr int F16_RG = 1;        // groups of 16 rows per wave
+constexpr int F16_C = 2;         // 16-element chunks per row and register stage
+constexpr int F16_KSTEP = 16 * F16_C;
+constexpr int F16_PAD = 4;       // LDS row stride % 32 == 4
+
+__global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_kernel(
+    const float *__restrict__ mu_w, const float *__restrict__ var_w,
+    const float *__restrict__ mu_a, const float *__restrict__ var_a, int K, int N, int B,
+    int k_per_split, int splits, float *__restrict__ ws0, float *__restrict__ ws1) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    constexpr int RG = F16_RG, C = F16_C, KSTEP = F16_KSTEP;
+    constexpr int ROWS_PER_BLOCK = W16_WAVES * RG * 16;
+    const int S = k_per_split + F16_PAD;
+    float *s_mu = lds, *s_var = lds + W16_SAMPLES * S;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int i = lane & 15, kk = lane >> 4;
+    // consecutive workgroup ids go to the 8 XCDs round-robin: the slice is the fast
+    // index inside an XCD, so an XCD's workgroups cover all windows of a weight row
+    int row_block, split;
+    const int id = blockIdx.x, row_blocks = gridDim.x / splits;
+    if (row_blocks % 8 == 0) {
+        const int xcd = id & 7, local = id >> 3;
+        split = local % splits;
+        row_block = (local / splits) * 8 + xcd;
+    } else {
+        row_block = id % row_blocks;
+        split = id / row_blocks;
+    }
+    const int k_begin = split * k_per_split;
+    const int kr = min(K, k_begin + k_per_split) - k_begin;
+    // each wave walks its slice from a different starting point (sums commute)
+    const int rot = ((row_block * W16_WAVES + wave) * 2 * KSTEP) % k_per_split;
+
+    // stage the slice of the activations: [sample][k], zero beyond B and kr
+    const int k4s = k_per_split / 4;
+    for (int e = tid; e < W16_SAMPLES * k4s; e += W16_WAVES * 64) {
+        const int b = e / k4s, k = (e - b * k4s) * 4;
+        float4 m = zero4(), v = zero4();
+        if (b < B && k < kr) {
+            m = ld4(mu_a + (size_t)b * K + k_begin + k);
+            v = ld4(var_a + (size_t)b * K + k_begin + k);
+        }
+        *reinterpret_cast<float4 *>(s_mu + b * S + k) = m;
+        *reinterpret_cast<float4 *>(s_var + b * S + k) = v;
+    }
+
+    // Weight loads are never predicated: rows beyond N read row N-1 and are
+    // dropped at the end, reduction elements beyond the slice read the last float4
+    // of the row and meet zero activations.
+    const int n0 = row_block * ROWS_PER_BLOCK + wave * (RG * 16);
+    const float *wm[RG], *wv[RG];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) {
+        const int row = min(n0 + 16 * rg + i, N - 1);
+        wm[rg] = mu_w + (size_t)row * K;
+        wv[rg] = var_w + (size_t)row * K;
+    }
+    const int k_lane = k_begin + 4 * kk, k_last = K - 4;
+
+    // the two variance terms have accumulators of their own, so that no MFMA waits
+    // for the one issued just before it
+    floatx4 acc0[RG], acc1[RG], acc2[RG];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) {
+        acc0[rg] = (floatx4){0.f, 0.f, 0.f, 0.f};
+        acc1[rg] = acc0[rg];
+        acc2[rg] = acc0[rg];
+    }
+
+    float4 sm[2][RG][C], sv[2][RG][C];
+    auto load = [&](float4(&m)[RG][C], float4(&v)[RG][C], int kb) {
+#pragma unroll
+        for (int c = 0; c < C; c++) {
+            const int k = min(k_lane + kb + 16 * c, k_last);
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) {
+                m[rg][c] = ld4(wm[rg] + k);
+                v[rg][c] = ld4(wv[rg] + k);
+            }
+        }
+    };
+    auto multiply = [&](const float4(&cm)[RG][C], const float4(&cv)[RG][C], int kb) {
+#pragma unroll
+        for (int c = 0; c < C; c++) {
+            const int at = kb + 16 * c + 4 * kk;
+            const float4 am = *reinterpret_cast<const float4 *>(s_mu + i * S + at);
+            const float4 av = *reinterpret_cast<const float4 *>(s_var + i * S + at);
+            const float4 as = make_float4(av.x + am.x * am.x, av.y + am.y * am.y,
+                                          av.z + am.z * am.z, av.w + am.w * am.w);
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) {
+                const float4 w = cm[rg][c], u = cv[rg][c];
+                const float4 q = sq4(w);
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    acc0[rg] = mfma16(comp(w, t), comp(am, t), acc0[rg]);
+                    acc1[rg] = mfma16(comp(u, t), comp(as, t), acc1[rg]);
+                    acc2[rg] = mfma16(comp(q, t), comp(av, t), acc2[rg]);
+                }
+            }
+        }
+    };
+
+    // k_per_split is a multiple of two stages; positions are inside the slice,
+    // rotated by `rot`
+    auto wrap = [&](int p) { return p >= k_per_split ? p - k_per_split : p; };
+    load(sm[0], sv[0], rot);
+    __syncthreads();
+    for (int kb = 0; kb < k_per_split; kb += 2 * KSTEP) {
+        const int p0 = wrap(rot + kb), p1 = p0 + KSTEP;
+        // (the last pair has nothing left to prefetch: it re-reads a cached stage)
+        const int p2 = kb + 2 * KSTEP < k_per_split ? wrap(p0 + 2 * KSTEP) : p1;
+        load(sm[1], sv[1], p1);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(sm[0], sv[0], p0);
+        __builtin_amdgcn_sched_barrier(0);
+        load(sm[0], sv[0], p2);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(sm[1], sv[1], p1);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // register v of lane l: row n0 + 16*rg + 4*(l/16) + v, sample l%16
+    const int b = lane & 15;
+    if (b < B) {
+        const bool vec = (N & 3) == 0;
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            const int n = n0 + 16 * rg + 4 * (lane >> 4);
+            const size_t at = ((size_t)split * B + b) * N + n;
+            const floatx4 m = acc0[rg], v = acc1[rg] + acc2[rg];
+            if (vec && n + 3 < N) {
+                *reinterpret_cast<float4 *>(ws0 + at) = make_float4(m[0], m[1], m[2], m[3]);
+                *reinterpret_cast<float4 *>(ws1 + at) = make_float4(v[0], v[1], v[2], v[3]);
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                    if (n + c < N) {
+                        ws0[at + c] = m[c];
+                        ws1[at + c] = v[c];
+                    }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// State backward. A wave owns 64 consecutive input columns; the eight waves of a
+// workgroup sit side by side (512 columns) and walk the same slice of output
+// rows, so the staged innovations of the slice serve all of them and no wave
+// shares an output with another. Lane (i = l%16, kk = l/16) holds the float4 at
+// row n + kk, columns c0 + 4*i ..: one load instruction covers 4 rows x 256
+// bytes. MFMA t takes A[i][kk] = w[n+kk][c0 + 4*i + t] and B[kk][j] =
+// delta[j][n+kk] and accumulates over the rows in place; register v of lane l of
+// accumulator t is column c0 + 16*(l/16) + 4*v + t of sample l%16. The
+// innovations are staged as [sample][kk][step] (step = row/4), so that a lane
+// reads four steps' worth of its B operands as one float4.
+// ---------------------------------------------------------------------------
+constexpr int Z16_ST = 4;      // 4-row steps per register stage (= steps per LDS float4)
+constexpr int Z16_PADQ = 1;    // plane stride per/4 + 4: spreads the kk planes over the banks
+constexpr int Z16_WAVES = 8;   // side by side, 64 columns each (4 measured slower)
+constexpr int Z16_COLS = Z16_WAVES * 64;
+
+__global__ __launch_bounds__(Z16_WAVES * 64) void gemv16_dz_kernel(
+    const float *__restrict__ mu_w, const float *__restrict__ dmu,
+    const float *__restrict__ dvar, int K, int N, int B, int n_per_split,
+    float *__restrict__ ws0, float *__restrict__ ws1) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    constexpr int ST = Z16_ST;
+    // the float4 of B operands must start at a multiple of 4 steps: Q % 4 == 0
+    const int Q = n_per_split / 4 + 4 * Z16_PADQ;  // steps per (sample, kk) plane
+    const int S = 4 * Q;                           // floats per sample
+    float *s_dm = lds, *s_dv = lds + W16_SAMPLES * S;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int i = lane & 15, kk = lane >> 4;
+    const int slab = blockIdx.x, split = blockIdx.y;
+    const int n_begin = split * n_per_split;
+    const int n_last = N - 1;
+
+    // columns beyond K read column K-4 and are dropped at the end; rows beyond N
+    // read row N-1 and meet zero innovations
+    const int c0 = slab * Z16_COLS + wave * 64;
+    const float *w = mu_w + min(c0 + 4 * i, K - 4);
+
+    const int steps = n_per_split / 4;  // multiple of 2*ST
+    float4 st[2][ST];
+    auto load = [&](float4(&x)[ST], int s) {
+#pragma unroll
+        for (int u = 0; u < ST; u++)
+            x[u] = ld4(w + (size_t)min(n_begin + 4 * (s + u) + kk, n_last) * K);
+    };
+    load(st[0], 0);
+    // stage the innovations: global [sample][n] -> LDS [sample][n % 4][n / 4]
+    for (int e = tid; e < W16_SAMPLES * steps; e += Z16_WAVES * 64) {
+        const int b = e / steps, step = e - b * steps;
+        float4 m = zero4(), v = zero4();
+        if (b < B && n_begin + 4 * step < N) {  // N % 4 == 0 on this path
+            m = ld4(dmu + (size_t)b * N + n_begin + 4 * step);
+            v = ld4(dvar + (size_t)b * N + n_begin + 4 * step);
+        }
+        float *pm = s_dm + b * S + step, *pv = s_dv + b * S + step;
+        pm[0] = m.x; pm[Q] = m.y; pm[2 * Q] = m.z; pm[3 * Q] = m.w;
+        pv[0] = v.x; pv[Q] = v.y; pv[2 * Q] = v.z; pv[3 * Q] = v.w;
+    }
+
+    floatx4 acc0[4], acc1[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        acc0[t] = (floatx4){0.f, 0.f, 0.f, 0.f};
+        acc1[t] = acc0[t];
+    }
+
+    auto multiply = [&](const float4(&cur)[ST], int s) {  // s: multiple of ST = 4
+        const float4 dm = *reinterpret_cast<const float4 *>(s_dm + i * S + kk * Q + s);
+        const float4 dv = *reinterpret_cast<const float4 *>(s_dv + i * S + kk * Q + s);
+#pragma unroll
+        for (int u = 0; u < ST; u++) {
+            const float4 x = cur[u];
+            const float4 q = sq4(x);
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                acc0[t] = mfma16(comp(x, t), comp(dm, u), acc0[t]);
+                acc1[t] = mfma16(comp(q, t), comp(dv, u), acc1[t]);
+            }
+        }
+    };
+
+    __syncthreads();
+    for (int s = 0; s < steps; s += 2 * ST) {
+        load(st[1], s + ST);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(st[0], s);
+        __builtin_amdgcn_sched_barrier(0);
+        // (nothing left to prefetch in the last pair: re-read the cached stage)
+        load(st[0], s + 2 * ST < steps ? s + 2 * ST : s + ST);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(st[1], s + ST);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // register v of accumulator t of lane l: column c0 + 16*(l/16) + 4*v + t, sample l%16
+    if (i < B) {
+        const int c = c0 + 16 * (lane >> 4);
+        const size_t base = ((size_t)split * B + i) * K + c;
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            if (c + 4 * v < K) {  // K % 4 == 0 on this path
+                *reinterpret_cast<float4 *>(ws0 + base + 4 * v) =
+                    make_float4(acc0[0][v], acc0[1][v], acc0[2][v], acc0[3][v]);
+                *reinterpret_cast<float4 *>(ws1 + base + 4 * v) =
+                    make_float4(acc1[0][v], acc1[1][v], acc1[2][v], acc1[3][v]);
+            }
+        }
+    }
+}
+
+constexpr int F16_KROUND = 2 * F16_KSTEP;                     // slices: whole pairs of stages
+constexpr int Z16_NSTEP = 2 * Z16_ST * 4;                     // rows: whole pairs of stages
+constexpr size_t W16_LDS_BUDGET = 72 * 1024;                  // two workgroups per CU
+
+}  // namespace
+
+int gemv16_fwd_rows_per_block() { return W16_WAVES * F16_RG * 16; }
+int gemv16_fwd_k_step() { return F16_KROUND; }
+int gemv16_fwd_max_slice() {
+    return (int)(W16_LDS_BUDGET / (2 * W16_SAMPLES * sizeof(float)) - F16_PAD) / F16_KROUND *
+           F16_KROUND;
+}
+int gemv16_dz_cols_per_block() { return Z16_COLS; }
+int gemv16_dz_n_step() { return Z16_NSTEP; }
+int gemv16_dz_max_slice() {
+    return (int)(W16_LDS_BUDGET / (2 * W16_SAMPLES * sizeof(float)) - 16 * Z16_PADQ) / Z16_NSTEP *
+           Z16_NSTEP;
+}
+
+// k_per_split: a multiple of gemv16_fwd_k_step(), at most gemv16_fwd_max_slice();
+// ws0/ws1: [splits][B][N] partial sums for the caller to fold.
+hipError_t launch_gemv16_fwd(const float *mu_w, const float *var_w, const float *mu_a,
+                             const float *var_a, int K, int N, int B, int k_per_split,
+                             int splits, float *ws0, float *ws1, hipStream_t stream) {
+    if (B < 1 || B > W16_SAMPLES || K % 4 != 0 || k_per_split % F16_KROUND != 0 ||
+        k_per_split > gemv16_fwd_max_slice() || (long long)k_per_split * splits < K)
+        return hipErrorInvalidValue;
+    const size_t lds = (size_t)2 * W16_SAMPLES * (k_per_split + F16_PAD) * sizeof(float);
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemv16_fwd_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    const int rows = gemv16_fwd_rows_per_block();
+    dim3 grid(((N + rows - 1) / rows) * splits), block(W16_WAVES * 64);
+    hipLaunchKernelGGL(gemv16_fwd_kernel, grid, block, lds, stream, mu_w, var_w, mu_a, var_a, K,
+                       N, B, k_per_split, splits, ws0, ws1);
+    return hipGetLastError();
+}
+
+// n_per_split: a multiple of gemv16_dz_n_step(), at most gemv16_dz_max_slice();
+// ws0/ws1: [splits][B][K] partial sums for the caller to fold.
+hipError_t launch_gemv16_dz(const float *mu_w, const float *dmu, const float *dvar, int K, int N,
+                            int B, int n_per_split, int splits, float *ws0, float *ws1,
+                            hipStream_t stream) {
+    if (B < 1 || B > W16_SAMPLES || K % 4 != 0 || N % 4 != 0 || n_per_split % Z16_NSTEP != 0 ||
+        n_per_split > gemv16_dz_max_slice() || (long long)n_per_split * splits < N ||
+        splits > 65535)
+        return hipErrorInvalidValue;
+    const size_t lds = (size_t)2 * W16_SAMPLES * (n_per_split + 16 * Z16_PADQ) * sizeof(float);
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemv16_dz_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    const int cols = gemv16_dz_cols_per_block();
+    dim3 grid((K + cols - 1) / cols, splits), block(Z16_WAVES * 64);
+    hipLaunchKernelGGL(gemv16_dz_kernel, grid, block, lds, stream, mu_w, dmu, dvar, K, N, B,
+                       n_per_split, ws0, ws1);
+    return hipGetLastError();
+}
+
+}  // namespace tagi

@@ -53,6 +53,7 @@ int tagi_hip_shutdown(void);
  * "linear.fwd.splits", "linear.dz.splits", "linear.dw.splits",
  * "linear.gemv_max_batch" (largest batch of the streaming kernels),
  * "linear.gemv.swizzle", "linear.gemv.fwd_variant", "linear.gemv.reverse",
+ * "linear.gemv16" (0: 9..16 samples on the kernels for up to 8),
  * "linear.dw_side" (0: bias innovations and the state-backward fold as launches
  * of their own instead of inside the weight-backward launch). Conv2d:
  * "conv2d.tile", "conv2d.splits", "conv2d.dw.tile", "conv2d.dw.splits",

@@ -15,6 +15,8 @@ SHAPES = [
     (516, 260, 16), (130, 70, 17), (5, 3, 2), (4, 4, 4), (333, 129, 77),
     # skinny path: several grid rows of fold workgroups, ragged row blocks, one row block
     (2048, 48, 7), (768, 1000, 3), (4096, 16, 16), (260, 20, 9),
+    # 9..16 samples: the 16-wide streaming kernels (several slices, ragged rows and columns)
+    (1024, 512, 16), (1536, 260, 12), (72, 1028, 10), (2052, 300, 13), (512, 2048, 9),
 ]
 
 
