@@ -10,6 +10,10 @@
 // weight backward has no reduction worth an MFMA (length B) and is a pure VALU
 // streaming kernel.
 //
+// The forward and state-backward kernels here are instantiated for up to 16
+// samples but dispatched for B <= 8; 9..16 samples take the 16x16x4 kernels of
+// tagi_gemv16.hip. The weight backward serves every B <= 16.
+//
 // Reduction slices (gridDim.y) write partial sums [slice][B][cols]; the caller
 // folds them, together with the bias or Jacobian epilogue, in reduce_splits.
 #include "tagi_internal.h"
