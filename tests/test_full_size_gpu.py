@@ -41,7 +41,8 @@ def _linear_inputs(K, N, B, seed):
                 jcb=u(B, K), delta_mu=0.1 * r(B, N), delta_var=-1e-3 * u(B, N))
 
 
-@pytest.mark.parametrize("K,N,B", [(4096, 4096, 256), (8192, 8192, 8)])
+# (the third shape: the 16-wide streaming kernels at the full weight size)
+@pytest.mark.parametrize("K,N,B", [(4096, 4096, 256), (8192, 8192, 8), (8192, 8192, 16)])
 def test_linear_full_size_against_float64_closed_forms(K, N, B):
     import torch
     import cutagi_amd.functional as F
