@@ -1,12 +1,17 @@
 // Host and device state containers: see states.h. Device buffers are plain
-// hipMalloc allocations owned by the object that made them; copies are
-// synchronous hipMemcpy on the null stream, which also orders them after every
-// kernel the layers queued there.
+// hipMalloc allocations owned by the object that made them. Everything runs on
+// the null stream, which orders copies and kernels. The per-batch transfers
+// (inputs, observations) go through a small ring of pinned staging buffers and do
+// not block the host, so the host can queue a step's launches while the GPU still
+// works on the previous ones; whole-buffer transfers (to_device / to_host) and
+// device-to-device copies are plain synchronous copies (an asynchronous
+// device-to-device copy measured slower: ResNet-18 step 13.2 -> 13.8 ms).
 #include "states.h"
 
 #include "../../include/tagi_hip.h"
 
 #include <algorithm>
+#include <cstring>
 
 #include "logger.h"
 
@@ -32,6 +37,48 @@ void d2h(float *dst, const float *src, size_t n) {
 }
 void d2d(float *dst, const float *src, size_t n) {
     if (n) HIP_OK(hipMemcpy(dst, src, n * sizeof(float), hipMemcpyDeviceToDevice));
+}
+
+// Pinned staging for the small host-to-device transfers of every batch. A copy
+// from pageable memory blocks the host until the stream has drained; a copy from
+// pinned memory does not. The caller's data is copied into the next slot of a
+// ring, the transfer is queued from there, and an event marks when the slot may
+// be written again (waited for only when the ring comes round to it).
+class StagingRing {
+   public:
+    static constexpr int SLOTS = 8;
+    // queues dst[0..bytes) = src[0..bytes) on the null stream of the current device
+    void upload(void *dst, const void *src, size_t bytes) {
+        if (bytes == 0) return;
+        Slot &s = slots_[next_];
+        next_ = (next_ + 1) % SLOTS;
+        if (s.event == nullptr) HIP_OK(hipEventCreateWithFlags(&s.event, hipEventDisableTiming));
+        if (s.used) HIP_OK(hipEventSynchronize(s.event));
+        if (s.cap < bytes) {
+            if (s.host != nullptr) HIP_OK(hipHostFree(s.host));
+            s.cap = std::max(bytes, (size_t)1 << 16);
+            HIP_OK(hipHostMalloc(&s.host, s.cap, hipHostMallocDefault));
+        }
+        std::memcpy(s.host, src, bytes);
+        HIP_OK(hipMemcpyAsync(dst, s.host, bytes, hipMemcpyHostToDevice, nullptr));
+        HIP_OK(hipEventRecord(s.event, nullptr));
+        s.used = true;
+    }
+
+   private:
+    struct Slot {
+        void *host = nullptr;
+        size_t cap = 0;
+        hipEvent_t event = nullptr;
+        bool used = false;
+    };
+    Slot slots_[SLOTS];
+    int next_ = 0;
+};
+// one ring per device, created on first use and kept until the process ends
+StagingRing &staging_ring(int device_idx) {
+    static StagingRing rings[16];
+    return rings[device_idx >= 0 && device_idx < 16 ? device_idx : 0];
 }
 }  // namespace
 
@@ -210,9 +257,10 @@ void HiddenStateHip::set_input_raw(const float *mu_x, const float *var_x, size_t
     this->actual_size = n / new_block_size;
     this->block_size = new_block_size;
     HIP_OK(hipSetDevice(device_idx));
-    HIP_OK(hipMemcpy(d_mu_a, mu_x, n * sizeof(float), hipMemcpyHostToDevice));
+    StagingRing &ring = staging_ring(device_idx);
+    ring.upload(d_mu_a, mu_x, n * sizeof(float));
     if (var_x != nullptr)
-        HIP_OK(hipMemcpy(d_var_a, var_x, n * sizeof(float), hipMemcpyHostToDevice));
+        ring.upload(d_var_a, var_x, n * sizeof(float));
     else
         HIP_OK(hipMemsetAsync(d_var_a, 0, n * sizeof(float), nullptr));
     if (tagi_store_states(nullptr, nullptr, 0, nullptr, nullptr, d_jcb, n, nullptr) != TAGI_OK)
@@ -378,9 +426,10 @@ void ObservationHip::reserve(size_t n, size_t ni) {
 void ObservationHip::upload(const float *mu, const float *var, size_t n, const int *idx,
                             size_t ni) {
     this->reserve(n, ni);
-    h2d(d_mu_obs, mu, n);
-    h2d(d_var_obs, var, n);
-    if (ni) HIP_OK(hipMemcpy(d_selected_idx, idx, ni * sizeof(int), hipMemcpyHostToDevice));
+    StagingRing &ring = staging_ring(device_idx);
+    ring.upload(d_mu_obs, mu, n * sizeof(float));
+    ring.upload(d_var_obs, var, n * sizeof(float));
+    if (ni) ring.upload(d_selected_idx, idx, ni * sizeof(int));
 }
 void ObservationHip::to_device() {
     this->upload(mu_obs.data(), var_obs.data(), mu_obs.size(), selected_idx.data(),
