@@ -377,7 +377,7 @@ def main():
     if "conv" in extras:
         line["extra"]["conv"] = run_conv(max(5, args.steps // 2), args.warmup)
     if "resnet18" in extras:
-        line["extra"]["resnet18"] = run_resnet(max(5, args.steps // 5), 3)
+        line["extra"]["resnet18"] = run_resnet(max(20, args.steps // 2), 5)
     if args.calibrate:
         calibrate_copy()
     if not args.no_cpu:

@@ -689,16 +689,9 @@ void ResNetBlock::forward(BaseHiddenStates &input_states, BaseHiddenStates &outp
         this->init_buffers();
     }
     if (training && shortcut && !shortcut_output_delta_z) this->init_buffers();
-    const size_t act_size = input_states.actual_size * batch_size;
-    if (training) {
-        // the identity shortcut needs the Jacobian of the block's input later
-        auto *bwd = dynamic_cast<BackwardStateHip *>(this->bwd_states.get());
-        if (bwd->size < act_size) bwd->set_size(act_size);
-        HIP_OK(hipMemcpyAsync(bwd->d_mu_a, in->d_mu_a, act_size * sizeof(float),
-                              hipMemcpyDeviceToDevice, nullptr));
-        HIP_OK(hipMemcpyAsync(bwd->d_jcb, in->d_jcb, act_size * sizeof(float),
-                              hipMemcpyDeviceToDevice, nullptr));
-    }
+    // input_z keeps the block's input for the shortcut; its Jacobian is also what
+    // the identity shortcut's backward needs (the reference copies mu_a and jcb
+    // once more into the block's bwd_states: two transfers per block saved here)
     input_z->copy_from(input_states, (int)(this->input_size * batch_size));
     main_block->forward(input_states, output_states, temp_states);
 
@@ -741,8 +734,8 @@ void ResNetBlock::backward(BaseDeltaStates &input_delta_states,
     } else {
         if (!state_update) return;
         auto *sc = as<DeltaStateHip>(*input_delta_z);
-        auto *bwd = dynamic_cast<BackwardStateHip *>(this->bwd_states.get());
-        TAGI_OK_OR_THROW(tagi_add_shortcut_delta(sc->d_delta_mu, sc->d_delta_var, bwd->d_jcb,
+        auto *kept = as<HiddenStateHip>(*input_z);
+        TAGI_OK_OR_THROW(tagi_add_shortcut_delta(sc->d_delta_mu, sc->d_delta_var, kept->d_jcb,
                                                  num_states, dout->d_delta_mu, dout->d_delta_var,
                                                  nullptr));
     }
