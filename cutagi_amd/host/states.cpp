@@ -425,6 +425,7 @@ void ObservationHip::reserve(size_t n, size_t ni) {
 }
 void ObservationHip::upload(const float *mu, const float *var, size_t n, const int *idx,
                             size_t ni) {
+    HIP_OK(hipSetDevice(device_idx));
     this->reserve(n, ni);
     StagingRing &ring = staging_ring(device_idx);
     ring.upload(d_mu_obs, mu, n * sizeof(float));
