@@ -621,6 +621,21 @@ int tagi_param_update(const float *delta_mu, const float *delta_var, float cap_f
     return TAGI_OK;
 }
 
+int tagi_layer_update(const float *delta_mu_w, const float *delta_var_w, size_t num_weights,
+                      float *mu_w, float *var_w, const float *delta_mu_b,
+                      const float *delta_var_b, size_t num_biases, float *mu_b, float *var_b,
+                      float cap_factor, int *neg_var_count, int slot, void *stream_) {
+    if (num_weights > 0 && (!delta_mu_w || !delta_var_w || !mu_w || !var_w))
+        return TAGI_ERR_INVALID_ARG;
+    if (num_biases > 0 && (!delta_mu_b || !delta_var_b || !mu_b || !var_b))
+        return TAGI_ERR_INVALID_ARG;
+    if (!(cap_factor > 0.0f) || (slot != 0 && slot != 1)) return TAGI_ERR_INVALID_ARG;
+    TAGI_TRY(launch_layer_update(delta_mu_w, delta_var_w, num_weights, mu_w, var_w, delta_mu_b,
+                                 delta_var_b, num_biases, mu_b, var_b, cap_factor, neg_var_count,
+                                 slot, static_cast<hipStream_t>(stream_)));
+    return TAGI_OK;
+}
+
 float tagi_cap_factor(int batch_size, float prev) {
     if (batch_size == 1) return 0.1f;
     if (batch_size > 1 && batch_size < 256) return 2.0f;

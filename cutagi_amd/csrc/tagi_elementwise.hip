@@ -83,6 +83,47 @@ __global__ __launch_bounds__(TPB) void param_update_kernel(
     }
 }
 
+// Both parameter sets of a layer in one launch: threads [0, nw) take the weights,
+// [nw, nw + nb) the biases. Clamped weight variances are counted in count[slot];
+// count[1 - slot], which this launch does not touch otherwise, is set to zero for
+// the next step, so no launch is spent on resetting a counter.
+__device__ __forceinline__ bool capped_step(float dm, float dv, float cap, float &m, float &v) {
+    const float sm = (float)((dm > 0.f) - (dm < 0.f));
+    const float sv = (float)((dv > 0.f) - (dv < 0.f));
+    const float bar = sqrtf(v) / cap;
+    m += sm * fminf(fabsf(dm), bar);
+    float nv = v + sv * fminf(fabsf(dv), bar);
+    const bool clamped = nv <= 0.0f;
+    if (clamped) nv = 1E-5f;
+    v = nv;
+    return clamped;
+}
+__global__ __launch_bounds__(TPB) void layer_update_kernel(
+    const float *__restrict__ dmu_w, const float *__restrict__ dvar_w, size_t nw,
+    float *__restrict__ mu_w, float *__restrict__ var_w, const float *__restrict__ dmu_b,
+    const float *__restrict__ dvar_b, size_t nb, float *__restrict__ mu_b,
+    float *__restrict__ var_b, float cap, int *__restrict__ count, int slot) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i == 0 && count != nullptr) count[1 - slot] = 0;
+    bool clamped = false;
+    if (i < nw) {
+        float m = mu_w[i], v = var_w[i];
+        clamped = capped_step(dmu_w[i], dvar_w[i], cap, m, v);
+        mu_w[i] = m;
+        var_w[i] = v;
+    } else if (i < nw + nb) {
+        const size_t j = i - nw;
+        float m = mu_b[j], v = var_b[j];
+        capped_step(dmu_b[j], dvar_b[j], cap, m, v);
+        mu_b[j] = m;
+        var_b[j] = v;
+    }
+    if (count != nullptr) {
+        const unsigned long long mask = __ballot(clamped);
+        if (mask != 0ull && (threadIdx.x & 63) == 0) atomicAdd(count + slot, __popcll(mask));
+    }
+}
+
 __global__ __launch_bounds__(TPB) void out_update_dense_kernel(
     const float *__restrict__ mu_a, const float *__restrict__ var_a,
     const float *__restrict__ jcb, const float *__restrict__ obs,
@@ -154,6 +195,17 @@ hipError_t launch_param_update(const float *dmu, const float *dvar, float cap, s
     if (n == 0) return hipSuccess;
     hipLaunchKernelGGL(param_update_kernel, dim3(blocks_for(n, TPB)), dim3(TPB), 0, stream, dmu,
                        dvar, cap, n, mu, var, neg_count);
+    return hipGetLastError();
+}
+
+hipError_t launch_layer_update(const float *dmu_w, const float *dvar_w, size_t nw, float *mu_w,
+                               float *var_w, const float *dmu_b, const float *dvar_b, size_t nb,
+                               float *mu_b, float *var_b, float cap, int *count, int slot,
+                               hipStream_t stream) {
+    if (nw + nb == 0) return hipSuccess;
+    hipLaunchKernelGGL(layer_update_kernel, dim3(blocks_for(nw + nb, TPB)), dim3(TPB), 0, stream,
+                       dmu_w, dvar_w, nw, mu_w, var_w, dmu_b, dvar_b, nb, mu_b, var_b, cap, count,
+                       slot);
     return hipGetLastError();
 }
 

@@ -148,6 +148,19 @@ def param_update(delta_mu, delta_var, cap_factor, mu, var, neg_var_count=None):
                                           capi.ptr(neg_var_count), _stream()))
 
 
+
+def layer_update(delta_mu_w, delta_var_w, mu_w, var_w, delta_mu_b, delta_var_b, mu_b, var_b,
+                 cap_factor, neg_var_count=None, slot=0):
+    """Weights and biases of a layer in one launch, in place. Bias tensors may be
+    None. neg_var_count: int32 device tensor of two elements (counts go to [slot],
+    [1 - slot] is zeroed)."""
+    _chk(delta_mu_w, delta_var_w, mu_w, var_w, delta_mu_b, delta_var_b, mu_b, var_b, neg_var_count)
+    nb = 0 if mu_b is None else mu_b.numel()
+    capi.check(capi.lib.tagi_layer_update(
+        capi.ptr(delta_mu_w), capi.ptr(delta_var_w), mu_w.numel(), capi.ptr(mu_w), capi.ptr(var_w),
+        capi.ptr(delta_mu_b), capi.ptr(delta_var_b), nb, capi.ptr(mu_b), capi.ptr(var_b),
+        cap_factor, capi.ptr(neg_var_count), int(slot), _stream()))
+
 def out_update_dense(mu_a, var_a, jcb, obs, var_obs, delta_mu, delta_var):
     _chk(mu_a, var_a, jcb, obs, var_obs, delta_mu, delta_var)
     capi.check(capi.lib.tagi_out_update_dense(capi.ptr(mu_a), capi.ptr(var_a), capi.ptr(jcb),

@@ -502,6 +502,11 @@ void LayerBlock::update_biases() {
         if (layer->get_layer_type() != LayerType::Activation) layer->update_biases();
 }
 
+void LayerBlock::update_params() {
+    for (auto &layer : layers)
+        if (layer->get_layer_type() != LayerType::Activation) layer->update_params();
+}
+
 void LayerBlock::compute_input_output_size(const InitArgs &args) {
     in_channels = args.depth;
     in_height = args.height;
@@ -748,6 +753,10 @@ void ResNetBlock::update_weights() {
 void ResNetBlock::update_biases() {
     main_block->update_biases();
     if (shortcut) shortcut->update_biases();
+}
+void ResNetBlock::update_params() {
+    main_block->update_params();
+    if (shortcut) shortcut->update_params();
 }
 void ResNetBlock::save(std::ofstream &file) {
     main_block->save(file);

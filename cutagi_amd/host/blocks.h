@@ -43,6 +43,7 @@ class MixtureReLUHip : public BaseLayer {
     void backward(BaseDeltaStates &, BaseDeltaStates &, BaseTempStates &, bool = true) override {}
     void update_weights() override {}
     void update_biases() override {}
+    void update_params() override {}
     std::unique_ptr<BaseLayer> to_cuda(int device_idx = 0) override;
 };
 
@@ -136,6 +137,7 @@ class AvgPool2dHip : public BaseLayerHip {
     void allocate_param_delta() override {}
     void update_weights() override {}
     void update_biases() override {}
+    void update_params() override {}
     void preinit_layer() override;
     void params_to_device() override {}
     void params_to_host() override {}
@@ -172,6 +174,7 @@ class LayerBlock : public BaseLayer {
                   BaseTempStates &temp_states, bool state_update = true) override;
     void update_weights() override;
     void update_biases() override;
+    void update_params() override;
     void compute_input_output_size(const InitArgs &args) override;
     void save(std::ofstream &file) override;
     void load(std::ifstream &file) override;
@@ -215,6 +218,7 @@ class ResNetBlock : public BaseLayer {
                   BaseTempStates &temp_states, bool state_update = true) override;
     void update_weights() override;
     void update_biases() override;
+    void update_params() override;
     void save(std::ofstream &file) override;
     void load(std::ifstream &file) override;
     ParameterMap get_parameters_as_map(std::string suffix = "") override;

@@ -162,8 +162,8 @@ void BaseLayerHip::allocate_param_memory() {
     d_mu_b = dev_alloc_t<float>(num_biases, device_idx);
     d_var_b = dev_alloc_t<float>(num_biases, device_idx);
     if (d_neg_var_count == nullptr) {
-        d_neg_var_count = dev_alloc_t<int>(1, device_idx);
-        HIP_OK(hipMemset(d_neg_var_count, 0, sizeof(int)));
+        d_neg_var_count = dev_alloc_t<int>(2, device_idx);
+        HIP_OK(hipMemset(d_neg_var_count, 0, 2 * sizeof(int)));
     }
 }
 
@@ -211,9 +211,11 @@ void BaseLayerHip::copy_params_from(const BaseLayer &source) {
 
 // The clamped-variance counter stays on the device; it is read back only when
 // somebody asks for it (the reference copies it in both directions every step,
-// src/base_layer_cuda.cu:170-185).
+// src/base_layer_cuda.cu:170-185). There are two counters used in turn: the
+// update that counts into one zeroes the other for the next update.
 void BaseLayerHip::update_weights() {
-    HIP_OK(hipMemsetAsync(d_neg_var_count, 0, sizeof(int), nullptr));
+    HIP_OK(hipMemsetAsync(d_neg_var_count, 0, 2 * sizeof(int), nullptr));
+    neg_var_slot = 0;
     TAGI_OK_OR_THROW(tagi_param_update(d_delta_mu_w, d_delta_var_w, cap_factor_update, num_weights,
                                        d_mu_w, d_var_w, d_neg_var_count, nullptr));
     neg_var_dirty = true;
@@ -225,9 +227,20 @@ void BaseLayerHip::update_biases() {
                                        d_mu_b, d_var_b, nullptr, nullptr));
 }
 
+// Weights and biases in one launch, no launch for the counter.
+void BaseLayerHip::update_params() {
+    neg_var_slot = 1 - neg_var_slot;
+    TAGI_OK_OR_THROW(tagi_layer_update(d_delta_mu_w, d_delta_var_w, num_weights, d_mu_w, d_var_w,
+                                       d_delta_mu_b, d_delta_var_b, bias ? num_biases : 0, d_mu_b,
+                                       d_var_b, cap_factor_update, d_neg_var_count, neg_var_slot,
+                                       nullptr));
+    neg_var_dirty = true;
+}
+
 int BaseLayerHip::get_neg_var_w_counter() {
     if (neg_var_dirty) {
-        HIP_OK(hipMemcpy(&neg_var_w_counter, d_neg_var_count, sizeof(int), hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(&neg_var_w_counter, d_neg_var_count + neg_var_slot, sizeof(int),
+                         hipMemcpyDeviceToHost));
         neg_var_dirty = false;
     }
     return neg_var_w_counter;

@@ -91,6 +91,11 @@ class BaseLayer {
     virtual void allocate_param_delta();
     virtual void update_weights();
     virtual void update_biases();
+    // Both of them, as Sequential::step issues them (one launch on the device).
+    virtual void update_params() {
+        this->update_weights();
+        this->update_biases();
+    }
     virtual void set_cap_factor_udapte(int batch_size);
     virtual void set_threads(int num) { num_threads = num; }
     virtual void compute_input_output_size(const InitArgs &args);
@@ -138,6 +143,7 @@ class BaseLayerHip : public BaseLayer {
     void allocate_param_delta() override;
     void update_weights() override;
     void update_biases() override;
+    void update_params() override;
     void save(std::ofstream &file) override;
     void load(std::ifstream &file) override;
     ParameterMap get_parameters_as_map(std::string suffix = "") override;
@@ -156,6 +162,7 @@ class BaseLayerHip : public BaseLayer {
     void release_param_memory();
     void store_states_for_training_hip(HiddenStateHip &input_states, HiddenStateHip &output_states);
     bool neg_var_dirty = false;
+    int neg_var_slot = 0;  // which of the two device counters holds the last update's count
 };
 
 // ---- Linear -----------------------------------------------------------------------
@@ -272,6 +279,7 @@ class ReLUHip : public BaseLayer {
     void backward(BaseDeltaStates &, BaseDeltaStates &, BaseTempStates &, bool = true) override {}
     void update_weights() override {}
     void update_biases() override {}
+    void update_params() override {}
     std::unique_ptr<BaseLayer> to_cuda(int = 0) override;
 };
 

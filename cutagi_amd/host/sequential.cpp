@@ -380,8 +380,7 @@ void Sequential::step() {
     this->require_device("step");
     for (auto &layer : layers) {
         if (layer->get_layer_type() == LayerType::Activation) continue;
-        layer->update_weights();
-        layer->update_biases();
+        layer->update_params();  // update_weights + update_biases, one launch on the device
     }
 }
 

@@ -171,6 +171,21 @@ int tagi_param_update(const float *delta_mu, const float *delta_var,
                       float cap_factor, size_t n, float *mu, float *var,
                       int *neg_var_count, void *stream);
 
+/* The two calls above for one layer in a single launch, as Sequential::step
+ * issues them back to back (src/sequential.cpp:444-447: update_weights, then
+ * update_biases of every layer): the capped step of the num_weights weights and
+ * the num_biases biases (num_biases may be 0). neg_var_count (device int[2], may
+ * be NULL): the clamped weight variances of this call are added to
+ * neg_var_count[slot], and neg_var_count[1 - slot] is set to zero; a caller that
+ * zeroes both once and alternates slot 0, 1, 0, ... reads each call's count from
+ * its slot without ever resetting anything. */
+int tagi_layer_update(const float *delta_mu_w, const float *delta_var_w,
+                      size_t num_weights, float *mu_w, float *var_w,
+                      const float *delta_mu_b, const float *delta_var_b,
+                      size_t num_biases, float *mu_b, float *var_b,
+                      float cap_factor, int *neg_var_count, int slot,
+                      void *stream);
+
 /* Cap factor for a batch size (src/base_layer.cpp:164-187); `prev` is returned
  * for batch sizes below 1. Host only. */
 float tagi_cap_factor(int batch_size, float prev);

@@ -44,6 +44,10 @@ def test_null_and_bad_sizes_are_rejected_before_any_launch():
     assert L.tagi_linear_bwd_dz(one, one, one, one, 4, -1, 4, one, one, None) == capi.ERR_INVALID_ARG
     assert L.tagi_linear_bwd_dw(one, one, one, None, 4, 4, 4, one, one, None) == capi.ERR_INVALID_ARG
     assert L.tagi_param_update(one, one, 0.0, 4, one, one, None, None) == capi.ERR_INVALID_ARG
+    assert L.tagi_layer_update(one, one, 4, one, one, None, None, 0, None, None, 2.0, None, 2,
+                               None) == capi.ERR_INVALID_ARG      # slot is 0 or 1
+    assert L.tagi_layer_update(one, one, 4, one, one, None, None, 3, None, None, 2.0, None, 0,
+                               None) == capi.ERR_INVALID_ARG      # biases announced, none given
     assert L.tagi_hip_tune(b"no.such.key", 1) == capi.ERR_INVALID_ARG
     with pytest.raises(capi.TagiHipError):
         capi.check(capi.ERR_INVALID_ARG)

@@ -34,6 +34,41 @@ def test_param_update(oracle_lib, cap):
     assert float(t_var.min()) > 0.0
 
 
+@pytest.mark.parametrize("nw,nb", [(100003, 257), (4096, 0), (5, 3)])
+def test_layer_update_one_launch(oracle_lib, nw, nb):
+    """Weights and biases in one launch: the same numbers as the two separate
+    updates of the oracle; the counter of the call's slot holds the clamped weight
+    variances, the other slot is reset."""
+    import torch
+    import cutagi_amd.functional as F
+    rng = np.random.default_rng(nw + nb)
+    cap = 2.0
+    def params(n):
+        return (rng.normal(0, 1, n).astype(np.float32), rng.uniform(1e-4, 1, n).astype(np.float32),
+                rng.normal(0, 1, n).astype(np.float32), rng.normal(0, 0.5, n).astype(np.float32))
+    mu_w, var_w, dmu_w, dvar_w = params(nw)
+    mu_b, var_b, dmu_b, dvar_b = params(nb)
+    ref_mw, ref_vw, ref_cnt = oracle_lib.param_update(mu_w, var_w, dmu_w, dvar_w, cap)
+    t_mw, t_vw = _t(mu_w), _t(var_w)
+    cnt = torch.tensor([7, 9], dtype=torch.int32, device="cuda")   # stale values in both slots
+    if nb:
+        ref_mb, ref_vb, _ = oracle_lib.param_update(mu_b, var_b, dmu_b, dvar_b, cap)
+        t_mb, t_vb = _t(mu_b), _t(var_b)
+        cnt[1] = 0                                                  # what the previous call left
+        F.layer_update(_t(dmu_w), _t(dvar_w), t_mw, t_vw, _t(dmu_b), _t(dvar_b), t_mb, t_vb, cap,
+                       cnt, slot=1)
+        np.testing.assert_allclose(t_mb.cpu().numpy(), ref_mb, rtol=1e-6, atol=1e-7)
+        np.testing.assert_allclose(t_vb.cpu().numpy(), ref_vb, rtol=1e-6, atol=1e-7)
+        assert cnt.tolist() == [0, ref_cnt]
+    else:
+        cnt[0] = 0
+        F.layer_update(_t(dmu_w), _t(dvar_w), t_mw, t_vw, None, None, None, None, cap, cnt, slot=0)
+        assert cnt.tolist() == [ref_cnt, 0]
+    np.testing.assert_allclose(t_mw.cpu().numpy(), ref_mw, rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(t_vw.cpu().numpy(), ref_vw, rtol=1e-6, atol=1e-7)
+    assert float(t_vw.min()) > 0.0
+
+
 def test_out_update_dense_and_indexed(oracle_lib):
     import torch
     import cutagi_amd.functional as F
