@@ -67,3 +67,17 @@ def test_host_only_entry_points(oracle_lib):
     for key in ("Fmwa_2", "FCzwa_1", "Szz_ud", "w", "h"):
         assert np.array_equal(a[key], b[key])
     assert (a["w"], a["h"]) == (1024, 9)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asking for more ends with a message and a non-zero
+    status before anything touches a device."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"],
+                         capture_output=True, text=True, timeout=120)
+    assert res.returncode != 0
+    assert "one GPU" in res.stderr
+    assert res.stdout.strip() == ""
