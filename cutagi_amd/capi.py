@@ -32,6 +32,7 @@ SIGNATURES = {
     "tagi_hip_shutdown": (_i, []),
     "tagi_hip_tune": (_i, [ctypes.c_char_p, _i]),
     "tagi_linear_fwd": (_i, [_vp] * 6 + [_i] * 4 + [_vp] * 3),
+    "tagi_linear_fwd_static": (_i, [_vp] * 6 + [_i] * 4 + [_vp] * 3),
     "tagi_linear_bwd_dz": (_i, [_vp] * 4 + [_i] * 3 + [_vp] * 3),
     "tagi_linear_bwd_dw": (_i, [_vp] * 4 + [_i] * 3 + [_vp] * 3),
     "tagi_linear_bwd_db": (_i, [_vp] * 3 + [_i] * 2 + [_vp] * 3),

@@ -9,6 +9,13 @@
 
 using namespace tagi;
 
+// Device memory that exists from module load on, for tagi_linear_fwd_static. In
+// host code the name is only a handle: the address that kernels, copies and
+// memsets can use comes from hipGetSymbolAddress, once per device (every GPU
+// holds its own copy of the array at its own address).
+constexpr size_t STATIC_SCRATCH_BYTES = TAGI_LINEAR_FWD_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) float scratch[STATIC_SCRATCH_BYTES / sizeof(float)];
+
 namespace {
 
 constexpr int ABI_VERSION = 100;
@@ -45,6 +52,29 @@ int workspace_get(size_t bytes, float **out) {
         w.bytes = want;
     }
     *out = w.ptr;
+    return TAGI_OK;
+}
+
+// Where a call's partial sums go: the grow-only workspace above, or the static
+// array of the entry point that allocates nothing.
+typedef int (*ScratchSource)(size_t bytes, float **out);
+
+float *g_scratch_ptr[MAX_DEVICES];
+std::mutex g_scratch_mutex;
+
+int static_scratch_get(size_t bytes, float **out) {
+    if (bytes > STATIC_SCRATCH_BYTES) return TAGI_ERR_UNSUPPORTED;
+    int dev = 0;
+    TAGI_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) return TAGI_ERR_NO_DEVICE;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        float *p = nullptr;
+        TAGI_TRY(hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch)));
+        if (p == nullptr) return TAGI_ERR_NO_DEVICE;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
     return TAGI_OK;
 }
 
@@ -118,14 +148,14 @@ void plan_gemm(GemmMode mode, GemmParams &p, int forced_splits, int *tile_out) {
 // given (state backward), a fold that the 16-byte path can do is left to a later
 // kernel and described in *defer instead.
 int run_gemm(GemmMode mode, GemmParams p, bool vec, int forced_splits, hipStream_t stream,
-             DzFold *defer = nullptr) {
+             DzFold *defer = nullptr, ScratchSource scratch_get = workspace_get) {
     int tile = 0;
     plan_gemm(mode, p, forced_splits, &tile);
     const int splits = p.splits;
     if (splits > 1) {
         float *ws = nullptr;
         const size_t part = (size_t)splits * p.M * p.N;
-        int rc = workspace_get(2 * part * sizeof(float), &ws);
+        int rc = scratch_get(2 * part * sizeof(float), &ws);
         if (rc != TAGI_OK) return rc;
         p.ws0 = ws;
         p.ws1 = ws + part;
@@ -225,9 +255,10 @@ int tagi_hip_tune(const char *key, int value) {
 // Linear
 // ---------------------------------------------------------------------------
 
-int tagi_linear_fwd(const float *mu_w, const float *var_w, const float *mu_b, const float *var_b,
-                    const float *mu_a, const float *var_a, int K, int N, int B, int bias,
-                    float *mu_z, float *var_z, void *stream_) {
+static int linear_fwd_impl(const float *mu_w, const float *var_w, const float *mu_b,
+                           const float *var_b, const float *mu_a, const float *var_a, int K, int N,
+                           int B, int bias, float *mu_z, float *var_z, void *stream_,
+                           ScratchSource scratch_get) {
     if (!mu_w || !var_w || !mu_a || !var_a || !mu_z || !var_z) return TAGI_ERR_INVALID_ARG;
     if (K <= 0 || N <= 0 || B <= 0) return TAGI_ERR_INVALID_ARG;
     if (bias && (!mu_b || !var_b)) return TAGI_ERR_INVALID_ARG;
@@ -249,7 +280,7 @@ int tagi_linear_fwd(const float *mu_w, const float *var_w, const float *mu_b, co
         splits = ceil_div(K, per);
         float *ws = nullptr;
         const size_t part = (size_t)splits * B * N;
-        int rc = workspace_get(2 * part * sizeof(float), &ws);
+        int rc = scratch_get(2 * part * sizeof(float), &ws);
         if (rc != TAGI_OK) return rc;
         TAGI_TRY(launch_gemv16_fwd(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, ws, ws + part,
                                    stream));
@@ -276,7 +307,7 @@ int tagi_linear_fwd(const float *mu_w, const float *var_w, const float *mu_b, co
         splits = ceil_div(K, per);
         float *ws = nullptr;
         const size_t part = (size_t)splits * B * N;
-        int rc = workspace_get(2 * part * sizeof(float), &ws);
+        int rc = scratch_get(2 * part * sizeof(float), &ws);
         if (rc != TAGI_OK) return rc;
         TAGI_TRY(launch_gemv_fwd(mu_w, var_w, mu_a, var_a, K, N, B, splits,
                                  g_tune.gemv_swz >= 0 ? g_tune.gemv_swz : 3, variant, ws,
@@ -291,7 +322,21 @@ int tagi_linear_fwd(const float *mu_w, const float *var_w, const float *mu_b, co
     p.M = B; p.N = N; p.R = K; p.ldx = K; p.ldy = K;
     p.out0 = mu_z; p.out1 = var_z; p.ldo = N;
     p.e0 = e0; p.e1 = e1;
-    return run_gemm(GEMM_FWD, p, vec, g_tune.fwd_splits, stream);
+    return run_gemm(GEMM_FWD, p, vec, g_tune.fwd_splits, stream, nullptr, scratch_get);
+}
+
+int tagi_linear_fwd(const float *mu_w, const float *var_w, const float *mu_b, const float *var_b,
+                    const float *mu_a, const float *var_a, int K, int N, int B, int bias,
+                    float *mu_z, float *var_z, void *stream) {
+    return linear_fwd_impl(mu_w, var_w, mu_b, var_b, mu_a, var_a, K, N, B, bias, mu_z, var_z,
+                           stream, workspace_get);
+}
+
+int tagi_linear_fwd_static(const float *mu_w, const float *var_w, const float *mu_b,
+                           const float *var_b, const float *mu_a, const float *var_a, int K,
+                           int N, int B, int bias, float *mu_z, float *var_z, void *stream) {
+    return linear_fwd_impl(mu_w, var_w, mu_b, var_b, mu_a, var_a, K, N, B, bias, mu_z, var_z,
+                           stream, static_scratch_get);
 }
 
 // State backward; with `defer` given and the skinny-batch kernel running, the

@@ -73,6 +73,25 @@ int tagi_linear_fwd(const float *mu_w, const float *var_w, const float *mu_b,
                     int K, int N, int B, int bias, float *mu_z, float *var_z,
                     void *stream);
 
+/* tagi_linear_fwd for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc). It has no
+ * counterpart in the reference. Same arguments, same kernels and bit-identical
+ * results; the partial sums of a sliced reduction go to a fixed array of
+ * TAGI_LINEAR_FWD_STATIC_SCRATCH_BYTES that every GPU holds from the moment the
+ * library is loaded until the process ends, so the call never reaches hipMalloc,
+ * hipFree or the grow-only workspace. A shape whose partial sums need more than
+ * that returns TAGI_ERR_UNSUPPORTED and launches nothing (2 * slices * B * N * 4
+ * bytes; 32 MiB at K = N = 4096, B = 256). All calls on one GPU share the array:
+ * calls that overlap on one GPU (two streams, two host threads) race. The first
+ * call on a device looks the array's address up once; make that call outside a
+ * graph capture. */
+#define TAGI_LINEAR_FWD_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
+int tagi_linear_fwd_static(const float *mu_w, const float *var_w,
+                           const float *mu_b, const float *var_b,
+                           const float *mu_a, const float *var_a, int K, int N,
+                           int B, int bias, float *mu_z, float *var_z,
+                           void *stream);
+
 /* delta_mu_z = (delta_mu * mu_w) .* jcb ; delta_var_z = (delta_var * mu_w^2) .* jcb^2
  * replaces linear_state_backward_cuda (src/linear_layer_cuda.cu:75-121). */
 int tagi_linear_bwd_dz(const float *mu_w, const float *jcb,
