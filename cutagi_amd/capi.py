@@ -44,9 +44,11 @@ SIGNATURES = {
     "tagi_conv2d_bwd_dw": (_i, [_vp] * 6 + [_i] * 7 + [_vp] * 5),
     "tagi_store_states": (_i, [_vp, _vp, _sz, _vp, _vp, _vp, _sz, _vp]),
     "tagi_param_update": (_i, [_vp, _vp, _f, _sz, _vp, _vp, _vp, _vp]),
+    "tagi_param_raw_update": (_i, [_vp, _vp, _sz, _vp, _vp, _vp]),
     "tagi_layer_update": (_i, [_vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _f, _vp, _i, _vp]),
     "tagi_cap_factor": (_f, [_i, _f]),
     "tagi_out_update_dense": (_i, [_vp] * 5 + [_i] + [_vp] * 3),
+    "tagi_out_update_heteros": (_i, [_vp] * 4 + [_i] + [_vp] * 3),
     "tagi_out_update_indexed": (_i, [_vp] * 6 + [_i] * 3 + [_vp] * 3),
     "tagi_relu_fwd": (_i, [_vp, _vp, _sz, _vp, _vp, _vp, _vp]),
     "tagi_mixture_relu_fwd": (_i, [_vp, _vp, _sz, _vp, _vp, _vp, _vp]),

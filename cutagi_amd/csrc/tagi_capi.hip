@@ -666,6 +666,14 @@ int tagi_param_update(const float *delta_mu, const float *delta_var, float cap_f
     return TAGI_OK;
 }
 
+int tagi_param_raw_update(const float *delta_mu, const float *delta_var, size_t n, float *mu,
+                          float *var, void *stream_) {
+    if (n > 0 && (!delta_mu || !delta_var || !mu || !var)) return TAGI_ERR_INVALID_ARG;
+    TAGI_TRY(launch_param_raw_update(delta_mu, delta_var, n, mu, var,
+                                     static_cast<hipStream_t>(stream_)));
+    return TAGI_OK;
+}
+
 int tagi_layer_update(const float *delta_mu_w, const float *delta_var_w, size_t num_weights,
                       float *mu_w, float *var_w, const float *delta_mu_b,
                       const float *delta_var_b, size_t num_biases, float *mu_b, float *var_b,
@@ -696,6 +704,21 @@ int tagi_out_update_dense(const float *mu_a, const float *var_a, const float *jc
         return TAGI_ERR_INVALID_ARG;
     TAGI_TRY(launch_out_update_dense(mu_a, var_a, jcb, obs, var_obs, n, delta_mu, delta_var,
                                      static_cast<hipStream_t>(stream_)));
+    return TAGI_OK;
+}
+
+int tagi_out_update_heteros(const float *mu_a, const float *var_a, const float *jcb,
+                            const float *obs, int n, float *delta_mu, float *delta_var,
+                            void *stream_) {
+    if (n < 0) return TAGI_ERR_INVALID_ARG;
+    if (n > 0 && (!mu_a || !var_a || !jcb || !obs || !delta_mu || !delta_var))
+        return TAGI_ERR_INVALID_ARG;
+    // pairs are read and written as 8-byte elements
+    if (n > 0 && (((uintptr_t)mu_a | (uintptr_t)var_a | (uintptr_t)jcb | (uintptr_t)delta_mu |
+                   (uintptr_t)delta_var) & 7u))
+        return TAGI_ERR_INVALID_ARG;
+    TAGI_TRY(launch_out_update_heteros(mu_a, var_a, jcb, obs, n, delta_mu, delta_var,
+                                       static_cast<hipStream_t>(stream_)));
     return TAGI_OK;
 }
 

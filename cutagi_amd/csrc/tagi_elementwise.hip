@@ -83,6 +83,16 @@ __global__ __launch_bounds__(TPB) void param_update_kernel(
     }
 }
 
+// p += d without a cap or a floor.
+__global__ __launch_bounds__(TPB) void param_raw_update_kernel(
+    const float *__restrict__ dmu, const float *__restrict__ dvar, size_t n,
+    float *__restrict__ mu, float *__restrict__ var) {
+    const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n) return;
+    mu[i] += dmu[i];
+    var[i] += dvar[i];
+}
+
 // Both parameter sets of a layer in one launch: threads [0, nw) take the weights,
 // [nw, nw + nb) the biases. Clamped weight variances are counted in count[slot];
 // count[1 - slot], which this launch does not touch otherwise, is set to zero for
@@ -139,6 +149,48 @@ __global__ __launch_bounds__(TPB) void out_update_dense_kernel(
         dmu[col] = t * (obs[col] - mu_a[col]);
         dvar[col] = -t * jcb[col];
     }
+}
+
+// Output layer with a learned error variance: unit 2i is the mean output, unit
+// 2i+1 the expected squared error (positive). One thread per observation.
+__global__ __launch_bounds__(TPB) void out_update_heteros_kernel(
+    const float2 *__restrict__ mu_a, const float2 *__restrict__ var_a,
+    const float2 *__restrict__ jcb, const float *__restrict__ obs, int n,
+    float2 *__restrict__ dmu, float2 *__restrict__ dvar) {
+// differences of nearly equal moments: keep the reference's roundings (no fused
+// multiply-adds), so that the cancellations lose the same digits on both sides
+#pragma clang fp contract(off)
+    const int i = blockIdx.x * TPB + threadIdx.x;
+    if (i >= n) return;
+    const float2 m = mu_a[i], v = var_a[i], j = jcb[i];
+    const float y = obs[i];
+    const float mu_v2 = m.y;                               // prior mean of V^2
+    const float var_v2 = 3.0f * v.y + 2.0f * m.y * m.y;    // prior variance of V^2
+    const float var_sum = v.x + mu_v2;                     // predictive variance of y
+    const float t = j.x / var_sum;
+    const bool bad_obs = isinf(y) || isnan(y);
+    float2 om = make_float2(0.f, 0.f), ov = make_float2(0.f, 0.f);
+    if (!(isinf(t) || isnan(t) || bad_obs)) {
+        om.x = t * (y - m.x);
+        ov.x = -t * j.x;
+    }
+    if (!bad_obs) {
+        const float gain = mu_v2 / var_sum;                // cov(y, V) / var(y)
+        const float mu_v_pos = gain * (y - m.x);
+        const float var_v_pos = mu_v2 - gain * mu_v2;
+        const float mu_v2_pos = mu_v_pos * mu_v_pos + var_v_pos;
+        const float var_v2_pos =
+            2.0f * var_v_pos * var_v_pos + 4.0f * var_v_pos * mu_v_pos * mu_v_pos;
+        const float k = v.y / var_v2;
+        const float mu_pos = m.y + k * (mu_v2_pos - mu_v2);
+        const float var_pos = v.y + k * k * (var_v2_pos - var_v2);
+        float jv = j.y / v.y;
+        if (isinf(jv) || isnan(jv)) jv = 0.0f;
+        om.y = jv * (mu_pos - m.y);
+        ov.y = jv * jv * (var_pos - v.y);
+    }
+    dmu[i] = om;
+    dvar[i] = ov;
 }
 
 __global__ __launch_bounds__(TPB) void out_update_indexed_kernel(
@@ -198,6 +250,14 @@ hipError_t launch_param_update(const float *dmu, const float *dvar, float cap, s
     return hipGetLastError();
 }
 
+hipError_t launch_param_raw_update(const float *dmu, const float *dvar, size_t n, float *mu,
+                                   float *var, hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(param_raw_update_kernel, dim3(blocks_for(n, TPB)), dim3(TPB), 0, stream,
+                       dmu, dvar, n, mu, var);
+    return hipGetLastError();
+}
+
 hipError_t launch_layer_update(const float *dmu_w, const float *dvar_w, size_t nw, float *mu_w,
                                float *var_w, const float *dmu_b, const float *dvar_b, size_t nb,
                                float *mu_b, float *var_b, float cap, int *count, int slot,
@@ -215,6 +275,18 @@ hipError_t launch_out_update_dense(const float *mu_a, const float *var_a, const 
     if (n == 0) return hipSuccess;
     hipLaunchKernelGGL(out_update_dense_kernel, dim3(blocks_for(n, TPB)), dim3(TPB), 0, stream,
                        mu_a, var_a, jcb, obs, var_obs, n, dmu, dvar);
+    return hipGetLastError();
+}
+
+hipError_t launch_out_update_heteros(const float *mu_a, const float *var_a, const float *jcb,
+                                     const float *obs, int n, float *dmu, float *dvar,
+                                     hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(out_update_heteros_kernel, dim3(blocks_for(n, TPB)), dim3(TPB), 0, stream,
+                       reinterpret_cast<const float2 *>(mu_a),
+                       reinterpret_cast<const float2 *>(var_a),
+                       reinterpret_cast<const float2 *>(jcb), obs, n,
+                       reinterpret_cast<float2 *>(dmu), reinterpret_cast<float2 *>(dvar));
     return hipGetLastError();
 }
 

@@ -119,6 +119,8 @@ hipError_t launch_store_states(const float *mu_a, const float *jcb, size_t n_in,
                                hipStream_t stream);
 hipError_t launch_param_update(const float *dmu, const float *dvar, float cap, size_t n,
                                float *mu, float *var, int *neg_count, hipStream_t stream);
+hipError_t launch_param_raw_update(const float *dmu, const float *dvar, size_t n, float *mu,
+                                   float *var, hipStream_t stream);
 hipError_t launch_layer_update(const float *dmu_w, const float *dvar_w, size_t nw, float *mu_w,
                                float *var_w, const float *dmu_b, const float *dvar_b, size_t nb,
                                float *mu_b, float *var_b, float cap, int *count, int slot,
@@ -126,6 +128,9 @@ hipError_t launch_layer_update(const float *dmu_w, const float *dvar_w, size_t n
 hipError_t launch_out_update_dense(const float *mu_a, const float *var_a, const float *jcb,
                                    const float *obs, const float *var_obs, int n, float *dmu,
                                    float *dvar, hipStream_t stream);
+hipError_t launch_out_update_heteros(const float *mu_a, const float *var_a, const float *jcb,
+                                     const float *obs, int n, float *dmu, float *dvar,
+                                     hipStream_t stream);
 hipError_t launch_out_update_indexed(const float *mu_a, const float *var_a, const float *jcb,
                                      const float *obs, const float *var_obs, const int *sel,
                                      int n_obs, int n_enc, int n, float *dmu, float *dvar,

@@ -168,6 +168,14 @@ def out_update_dense(mu_a, var_a, jcb, obs, var_obs, delta_mu, delta_var):
                                               capi.ptr(delta_mu), capi.ptr(delta_var), _stream()))
 
 
+def out_update_heteros(mu_a, var_a, jcb, obs, delta_mu, delta_var):
+    """obs.numel() observations against 2 * obs.numel() output units."""
+    _chk(mu_a, var_a, jcb, obs, delta_mu, delta_var)
+    capi.check(capi.lib.tagi_out_update_heteros(capi.ptr(mu_a), capi.ptr(var_a), capi.ptr(jcb),
+                                                capi.ptr(obs), obs.numel(), capi.ptr(delta_mu),
+                                                capi.ptr(delta_var), _stream()))
+
+
 def out_update_indexed(mu_a, var_a, jcb, obs, var_obs, selected_idx, n_obs, n_enc, delta_mu,
                        delta_var):
     _chk(mu_a, var_a, jcb, obs, var_obs, selected_idx, delta_mu, delta_var)

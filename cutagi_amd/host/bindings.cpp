@@ -106,6 +106,16 @@ PYBIND11_MODULE(cutagi, m) {
         .def("params_to_host", &BaseLayer::params_to_host)
         .def("params_to_device", &BaseLayer::params_to_device)
         .def("delta_params_to_host", &BaseLayer::delta_params_to_host)
+        .def("delta_params_to_device", &BaseLayer::delta_params_to_device)
+        .def("update_weights", &BaseLayer::update_weights)
+        .def("update_biases", &BaseLayer::update_biases)
+        .def("raw_update_weights", &BaseLayer::raw_update_weights)
+        .def("raw_update_biases", &BaseLayer::raw_update_biases)
+        .def("set_cuda_threads", [](BaseLayer &self, int num) {
+                 // launch shapes are chosen by the kernels here; the value is kept for
+                 // code written for the reference's device layers
+                 if (auto *d = dynamic_cast<BaseLayerHip *>(&self)) d->set_cuda_threads(num);
+             })
         .def("get_norm_mean_var", &BaseLayer::get_norm_mean_var)
         .def("to_cuda", [](BaseLayer &self, int device_idx) {
                  return std::shared_ptr<BaseLayer>(self.to_cuda(device_idx));
@@ -197,6 +207,14 @@ PYBIND11_MODULE(cutagi, m) {
         .def("update_using_indices", &OutputUpdater::update_using_indices,
              py::arg("output_states"), py::arg("mu_obs"), py::arg("var_obs"),
              py::arg("selected_idx"), py::arg("delta_states"))
+        .def("update_heteros",
+             [](OutputUpdater &self, BaseHiddenStates &out, const FloatArray &mu,
+                BaseDeltaStates &delta) {
+                 self.update_heteros_raw(out, mu.data(), (size_t)mu.size(), delta);
+             },
+             py::arg("output_states"), py::arg("mu_obs").noconvert(), py::arg("delta_states"))
+        .def("update_heteros", &OutputUpdater::update_heteros, py::arg("output_states"),
+             py::arg("mu_obs"), py::arg("delta_states"))
         .def_readwrite("device", &OutputUpdater::device);
 
     py::class_<Sequential, std::shared_ptr<Sequential>>(m, "Sequential")

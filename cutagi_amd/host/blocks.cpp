@@ -563,6 +563,14 @@ std::vector<ParameterTuple> LayerBlock::parameters() {
     return params;
 }
 
+// Input / output image sizes a caller may have set on a block before it is moved to
+// the device (a network that starts with a block has nothing else to take them from).
+static void copy_geometry(const BaseLayer &from, BaseLayer &to) {
+    to.in_width = from.in_width; to.in_height = from.in_height; to.in_channels = from.in_channels;
+    to.out_width = from.out_width; to.out_height = from.out_height;
+    to.out_channels = from.out_channels;
+}
+
 std::unique_ptr<BaseLayer> LayerBlock::to_cuda(int device_idx) {
     auto block = std::make_unique<LayerBlock>();
     block->device = "cuda";
@@ -571,6 +579,7 @@ std::unique_ptr<BaseLayer> LayerBlock::to_cuda(int device_idx) {
     block->input_size = input_size;
     block->output_size = output_size;
     block->training = training;
+    copy_geometry(*this, *block);
     this->device = "cuda";
     this->device_idx = device_idx;
     return block;
@@ -796,7 +805,9 @@ std::unique_ptr<BaseLayer> ResNetBlock::to_cuda(int device_idx) {
     this->device_idx = device_idx;
     std::shared_ptr<BaseLayer> m = main_block->to_cuda(device_idx);
     std::shared_ptr<BaseLayer> s = shortcut ? shortcut->to_cuda(device_idx) : nullptr;
-    return std::make_unique<ResNetBlockHip>(std::move(m), std::move(s), device_idx);
+    auto block = std::make_unique<ResNetBlockHip>(std::move(m), std::move(s), device_idx);
+    copy_geometry(*this, *block);
+    return block;
 }
 
 void ResNetBlock::preinit_layer() {

@@ -67,6 +67,8 @@ void BaseLayer::backward(BaseDeltaStates &, BaseDeltaStates &, BaseTempStates &,
 }
 void BaseLayer::update_weights() { no_cpu_path("update_weights"); }
 void BaseLayer::update_biases() { no_cpu_path("update_biases"); }
+void BaseLayer::raw_update_weights() { no_cpu_path("raw_update_weights"); }
+void BaseLayer::raw_update_biases() { no_cpu_path("raw_update_biases"); }
 
 void BaseLayer::allocate_param_delta() {
     delta_mu_w.assign(num_weights, 0.0f);
@@ -161,6 +163,8 @@ void BaseLayerHip::allocate_param_memory() {
     d_var_w = dev_alloc_t<float>(num_weights, device_idx);
     d_mu_b = dev_alloc_t<float>(num_biases, device_idx);
     d_var_b = dev_alloc_t<float>(num_biases, device_idx);
+    alloc_w = num_weights;
+    alloc_b = num_biases;
     if (d_neg_var_count == nullptr) {
         d_neg_var_count = dev_alloc_t<int>(2, device_idx);
         HIP_OK(hipMemset(d_neg_var_count, 0, 2 * sizeof(int)));
@@ -199,6 +203,34 @@ void BaseLayerHip::params_to_host() {
 void BaseLayerHip::delta_params_to_host() {
     d2h(delta_mu_w, d_delta_mu_w, num_weights); d2h(delta_var_w, d_delta_var_w, num_weights);
     d2h(delta_mu_b, d_delta_mu_b, num_biases); d2h(delta_var_b, d_delta_var_b, num_biases);
+}
+
+// reference: BaseLayerCuda::delta_params_to_device, src/base_layer_cuda.cu:313-332
+void BaseLayerHip::delta_params_to_device() {
+    if (delta_mu_w.size() != num_weights || delta_var_w.size() != num_weights ||
+        (bias && (delta_mu_b.size() != num_biases || delta_var_b.size() != num_biases)))
+        LOG(LogLevel::ERROR, "Host parameter innovations do not have the layer's sizes");
+    if (d_delta_mu_w == nullptr) {  // allocation zeroes the host vectors: keep them
+        auto keep = std::make_tuple(delta_mu_w, delta_var_w, delta_mu_b, delta_var_b);
+        this->allocate_param_delta();
+        std::tie(delta_mu_w, delta_var_w, delta_mu_b, delta_var_b) = keep;
+    }
+    h2d(d_delta_mu_w, delta_mu_w); h2d(d_delta_var_w, delta_var_w);
+    if (bias) {
+        h2d(d_delta_mu_b, delta_mu_b); h2d(d_delta_var_b, delta_var_b);
+    }
+}
+
+// reference: BaseLayerCuda::raw_update_weights / raw_update_biases,
+// src/base_layer_cuda.cu:127-159
+void BaseLayerHip::raw_update_weights() {
+    TAGI_OK_OR_THROW(tagi_param_raw_update(d_delta_mu_w, d_delta_var_w, num_weights, d_mu_w,
+                                           d_var_w, nullptr));
+}
+void BaseLayerHip::raw_update_biases() {
+    if (!bias) return;
+    TAGI_OK_OR_THROW(tagi_param_raw_update(d_delta_mu_b, d_delta_var_b, num_biases, d_mu_b,
+                                           d_var_b, nullptr));
 }
 
 void BaseLayerHip::copy_params_from(const BaseLayer &source) {
@@ -261,9 +293,22 @@ ParameterMap BaseLayerHip::get_parameters_as_map(std::string suffix) {
     return BaseLayer::get_parameters_as_map(suffix);
 }
 
+void BaseLayerHip::adopt_host_params() {
+    if (var_w.size() != mu_w.size() || var_b.size() != mu_b.size())
+        LOG(LogLevel::ERROR, "Parameter means and variances differ in size");
+    num_weights = mu_w.size();
+    num_biases = mu_b.size();
+    if (d_mu_w == nullptr || alloc_w != num_weights || alloc_b != num_biases)
+        this->allocate_param_memory();
+    if (training && (d_delta_mu_w == nullptr || delta_mu_w.size() != num_weights ||
+                     delta_mu_b.size() != num_biases))
+        this->allocate_param_delta();
+    this->params_to_device();
+}
+
 void BaseLayerHip::load_parameters_from_map(const ParameterMap &param_map, const std::string &suffix) {
     BaseLayer::load_parameters_from_map(param_map, suffix);
-    this->params_to_device();
+    this->adopt_host_params();
 }
 
 std::vector<ParameterTuple> BaseLayerHip::parameters() {

@@ -91,6 +91,10 @@ class BaseLayer {
     virtual void allocate_param_delta();
     virtual void update_weights();
     virtual void update_biases();
+    // the same steps without the cap and the variance floor
+    // (reference: BaseLayer::raw_update_weights / raw_update_biases)
+    virtual void raw_update_weights();
+    virtual void raw_update_biases();
     // Both of them, as Sequential::step issues them (one launch on the device).
     virtual void update_params() {
         this->update_weights();
@@ -123,6 +127,7 @@ class BaseLayer {
     virtual void params_to_device() {}
     virtual void params_to_host() {}
     virtual void delta_params_to_host() {}
+    virtual void delta_params_to_device() {}
 
    protected:
     [[noreturn]] void no_cpu_path(const char *what) const;
@@ -136,6 +141,9 @@ class BaseLayerHip : public BaseLayer {
     float *d_delta_mu_w = nullptr, *d_delta_var_w = nullptr;
     float *d_delta_mu_b = nullptr, *d_delta_var_b = nullptr;
     int *d_neg_var_count = nullptr;
+    // Threads per block of the reference's elementwise launches. Kept so that code
+    // written for the reference runs; the kernels here choose their own launch shape.
+    unsigned int num_cuda_threads = 16;
 
     BaseLayerHip();
     ~BaseLayerHip() override;
@@ -144,6 +152,9 @@ class BaseLayerHip : public BaseLayer {
     void update_weights() override;
     void update_biases() override;
     void update_params() override;
+    void raw_update_weights() override;
+    void raw_update_biases() override;
+    void set_cuda_threads(int num) { num_cuda_threads = (unsigned int)num; }
     void save(std::ofstream &file) override;
     void load(std::ifstream &file) override;
     ParameterMap get_parameters_as_map(std::string suffix = "") override;
@@ -155,12 +166,18 @@ class BaseLayerHip : public BaseLayer {
     void params_to_device() override;
     void params_to_host() override;
     void delta_params_to_host() override;
+    void delta_params_to_device() override;
     void copy_params_from(const BaseLayer &source);
+    // The host vectors were replaced from outside (state dict, another model): take
+    // the layer's sizes from them, make the device storage fit - also on a layer that
+    // has not allocated anything yet - and upload.
+    void adopt_host_params();
 
    protected:
     void allocate_param_memory();
     void release_param_memory();
     void store_states_for_training_hip(HiddenStateHip &input_states, HiddenStateHip &output_states);
+    size_t alloc_w = 0, alloc_b = 0;  // sizes the device parameter arrays were allocated for
     bool neg_var_dirty = false;
     int neg_var_slot = 0;  // which of the two device counters holds the last update's count
 };

@@ -194,6 +194,30 @@ void OutputUpdater::update_using_indices_raw(BaseHiddenStates &output_states,
                                              nullptr));
 }
 
+void OutputUpdater::update_heteros(BaseHiddenStates &output_states, std::vector<float> &mu_obs,
+                                   BaseDeltaStates &delta_states) {
+    this->update_heteros_raw(output_states, mu_obs.data(), mu_obs.size(), delta_states);
+}
+
+void OutputUpdater::update_heteros_raw(BaseHiddenStates &output_states, const float *mu_obs,
+                                       size_t n, BaseDeltaStates &delta_states) {
+    ObservationHip *o = this->device_obs();
+    auto *out = dynamic_cast<HiddenStateHip *>(&output_states);
+    auto *delta = dynamic_cast<DeltaStateHip *>(&delta_states);
+    if (out == nullptr || delta == nullptr)
+        LOG(LogLevel::ERROR, "OutputUpdater needs device state buffers");
+    if (2 * n > out->size || 2 * n > delta->size)
+        LOG(LogLevel::ERROR, "Observation size does not fit the output buffers");
+    o->block_size = output_states.block_size;
+    o->size = n;
+    o->actual_size = output_states.block_size ? n / output_states.block_size : 0;
+    o->upload(mu_obs, nullptr, n, nullptr, 0);
+    delta->reset_zeros();
+    TAGI_OK_OR_THROW(tagi_out_update_heteros(out->d_mu_a, out->d_var_a, out->d_jcb, o->d_mu_obs,
+                                             (int)o->size, delta->d_delta_mu, delta->d_delta_var,
+                                             nullptr));
+}
+
 // ---- Sequential -----------------------------------------------------------------------
 void Sequential::add_layer(std::shared_ptr<BaseLayer> layer) {
     if (this->device == "cpu")
@@ -306,7 +330,9 @@ void Sequential::prepare_buffers(int batch_size) {
         this->z_buffer_block_size = batch_size;
         this->input_z_buffer->set_size(this->z_buffer_size, batch_size);
         this->output_z_buffer->set_size(this->z_buffer_size, batch_size);
-        if (this->training) {
+        // a model first run in eval mode has no delta buffers yet: they are created
+        // below at the new size
+        if (this->training && this->input_delta_z_buffer) {
             this->input_delta_z_buffer->set_size(this->z_buffer_size, batch_size);
             this->output_delta_z_buffer->set_size(this->z_buffer_size, batch_size);
         }
@@ -549,8 +575,7 @@ void Sequential::params_from(const Sequential &ref) {
         layers[i]->var_w = src->var_w;
         layers[i]->mu_b = src->mu_b;
         layers[i]->var_b = src->var_b;
-        if (auto *d = dynamic_cast<BaseLayerHip *>(layers[i].get()))
-            if (d->d_mu_w != nullptr) d->params_to_device();
+        if (auto *d = dynamic_cast<BaseLayerHip *>(layers[i].get())) d->adopt_host_params();
     }
 }
 

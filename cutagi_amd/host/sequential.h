@@ -42,6 +42,13 @@ class OutputUpdater {
     void update_using_indices_raw(BaseHiddenStates &output_states, const float *mu_obs,
                                   const float *var_obs, const int *selected_idx, size_t n,
                                   BaseDeltaStates &delta_states);
+    // Output layer with a learned error variance (twice as many output units as
+    // observations); reference: OutputUpdater::update_heteros,
+    // src/base_output_updater.cpp:391-408.
+    void update_heteros(BaseHiddenStates &output_states, std::vector<float> &mu_obs,
+                        BaseDeltaStates &delta_states);
+    void update_heteros_raw(BaseHiddenStates &output_states, const float *mu_obs, size_t n,
+                            BaseDeltaStates &delta_states);
 
    private:
     ObservationHip *device_obs();

@@ -429,7 +429,7 @@ void ObservationHip::upload(const float *mu, const float *var, size_t n, const i
     this->reserve(n, ni);
     StagingRing &ring = staging_ring(device_idx);
     ring.upload(d_mu_obs, mu, n * sizeof(float));
-    ring.upload(d_var_obs, var, n * sizeof(float));
+    if (var != nullptr) ring.upload(d_var_obs, var, n * sizeof(float));
     if (ni) ring.upload(d_selected_idx, idx, ni * sizeof(int));
 }
 void ObservationHip::to_device() {

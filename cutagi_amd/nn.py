@@ -229,8 +229,9 @@ class Sequential:
 
 
 class OutputUpdater:
-    """Innovations of the output layer from observations (dense) or from a few
-    observed output units per sample (``update_using_indices``, 1-based indices).
+    """Innovations of the output layer from observations (dense), from a few
+    observed output units per sample (``update_using_indices``, 1-based indices) or
+    for an output layer that learns its own error variance (``update_heteros``).
     float32 / int32 numpy arrays are handed to the C++ side in place."""
 
     def __init__(self, model_device):
@@ -246,8 +247,9 @@ class OutputUpdater:
                                                _f32(var_obs).ravel(), idx, delta_states)
 
     def update_heteros(self, output_states, mu_obs, delta_states):
-        raise NotImplementedError("heteroscedastic output update is outside the Linear / Conv2d "
-                                  "path this package covers")
+        """Output layer with a learned error variance: twice as many output units
+        (mean, expected squared error) as observations."""
+        self._cpp_backend.update_heteros(output_states, _f32(mu_obs).ravel(), delta_states)
 
     @property
     def device(self):

@@ -190,7 +190,13 @@ int tagi_param_update(const float *delta_mu, const float *delta_var,
                       float cap_factor, size_t n, float *mu, float *var,
                       int *neg_var_count, void *stream);
 
-/* The two calls above for one layer in a single launch, as Sequential::step
+/* Uncapped step, mu += delta_mu, var += delta_var; replaces device_raw_weight_update
+ * / device_raw_bias_update (src/base_layer_cuda.cu:28-54) as
+ * BaseLayerCuda::raw_update_weights / raw_update_biases launch them (127-159). */
+int tagi_param_raw_update(const float *delta_mu, const float *delta_var, size_t n,
+                          float *mu, float *var, void *stream);
+
+/* tagi_param_update for the weights and the biases of one layer in a single launch, as Sequential::step
  * issues them back to back (src/sequential.cpp:444-447: update_weights, then
  * update_biases of every layer): the capped step of the num_weights weights and
  * the num_biases biases (num_biases may be 0). neg_var_count (device int[2], may
@@ -226,6 +232,17 @@ int tagi_out_update_indexed(const float *mu_a, const float *var_a,
                             const float *var_obs, const int *selected_idx,
                             int n_obs, int n_enc, int n, float *delta_mu,
                             float *delta_var, void *stream);
+
+/* Output layer with a learned (heteroscedastic) error variance: the 2n output
+ * units are pairs, unit 2i the mean output and unit 2i+1 the expected squared error,
+ * and obs holds n observations. Unit 2i is updated as in the dense form with the
+ * expected squared error as observation noise; unit 2i+1 through the posterior
+ * moments of the error and of its square. inf/nan observations give zeros. Replaces
+ * update_delta_z_cuda_heteros (src/output_updater_cuda.cu:46-135, launched at
+ * 225-269); CPU form src/base_output_updater.cpp:131-226. Arrays 8-byte aligned. */
+int tagi_out_update_heteros(const float *mu_a, const float *var_a,
+                            const float *jcb, const float *obs, int n,
+                            float *delta_mu, float *delta_var, void *stream);
 
 /* ---- ReLU -------------------------------------------------------------------- */
 

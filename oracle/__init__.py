@@ -180,6 +180,13 @@ class Oracle:
                                      _fp(dvar))
         return dmu, dvar
 
+    def out_update_heteros(self, mu_a, var_a, jcb, obs, dmu, dvar):
+        """obs.size observations against 2*obs.size output units (mean, error variance)."""
+        dmu, dvar = dmu.copy(), dvar.copy()
+        self._fn("out_update_heteros")(_fp(mu_a), _fp(var_a), _fp(jcb), _fp(obs), obs.size,
+                                       _fp(dmu), _fp(dvar))
+        return dmu, dvar
+
     def out_update_indexed(self, mu_a, var_a, jcb, obs, var_obs, sel, n_obs,
                            n_enc, dmu, dvar):
         dmu, dvar = dmu.copy(), dvar.copy()
@@ -328,6 +335,51 @@ class Oracle:
         n = fn(int(model), os.fsencode(path), _fp(out), capacity)
         return None if n < 0 else out[:n].copy()
 
+    # ---- whole models through the reference's own drivers (reference build only) ---
+    def model_param_sizes(self, spec):
+        """Sizes of the parameter arrays of a network description in leaf order
+        (oracle/ref_model.cpp), or None if the description does not parse."""
+        fn = self._fn("model_param_sizes")
+        fn.restype = ctypes.c_int
+        sizes = np.zeros(4096, np.int32)
+        n = fn(spec.encode(), _ip(sizes), sizes.size)
+        return None if n < 0 else sizes[:n].tolist()
+
+    def model_run(self, spec, params, mu_x, var_x, y, var_y, sel, B, update, n_enc=0,
+                  input_state_update=False, eval_forward=False, threads=2):
+        """Training steps of the reference's Sequential on the CPU: forward, output
+        update (0 dense, 1 selected indices, 2 heteroscedastic), backward, step.
+        mu_x [steps][B*n_in] etc. Returns a dict of per-step outputs."""
+        fn = self._fn("model_run")
+        fn.restype = ctypes.c_int
+        params = f32(np.concatenate([np.ravel(p) for p in params]))
+        mu_x = f32(mu_x)
+        steps, nx = mu_x.shape
+        n_in = nx // B
+        var_x = None if var_x is None else f32(var_x)
+        y, var_y = f32(y), f32(var_y)
+        sel = np.zeros(1, np.int32) if sel is None else np.ascontiguousarray(sel, np.int32)
+        cap = 1 << 22
+        out_mu = np.zeros(cap, np.float32)
+        out_var = np.zeros(cap, np.float32)
+        in_dmu = np.zeros((steps, nx), np.float32)
+        in_dvar = np.zeros((steps, nx), np.float32)
+        params_out = np.zeros((steps, params.size), np.float32)
+        neg = np.zeros((steps, 256), np.int32)
+        top = len(_top_level(spec))
+        neg = np.zeros((steps, top), np.int32)
+        n_out = fn(spec.encode(), int(threads), int(input_state_update), _fp(params), steps, B,
+                   n_in, _fp(mu_x), _fp(var_x), int(update), int(n_enc), _fp(y), _fp(var_y),
+                   _ip(sel), int(eval_forward), _fp(out_mu), _fp(out_var), _fp(in_dmu),
+                   _fp(in_dvar), _fp(params_out), _ip(neg))
+        if n_out < 0:
+            raise RuntimeError("the reference threw while running: " + spec)
+        rows = steps + (1 if eval_forward else 0)
+        no = B * n_out
+        return dict(n_out=n_out, out_mu=out_mu[:rows * no].reshape(rows, no).copy(),
+                    out_var=out_var[:rows * no].reshape(rows, no).copy(), in_dmu=in_dmu,
+                    in_dvar=in_dvar, params=params_out, neg=neg)
+
     def write_csv(self, path, data):
         fn = self._fn("write_csv")
         fn.restype = ctypes.c_int
@@ -339,6 +391,21 @@ class Oracle:
         fn.restype = ctypes.c_int
         out = np.zeros(n, np.float32)
         return out if fn(os.fsencode(path), _fp(out), n) == 0 else None
+
+
+def _top_level(spec):
+    """Top-level layer names of a network description (brackets skipped)."""
+    names, depth = [], 0
+    tok = spec.split()
+    i = 4 if tok and tok[0] == "input" else 0
+    for t in tok[i:]:
+        if t == "[":
+            depth += 1
+        elif t == "]":
+            depth -= 1
+        elif depth == 0 and t[0].isalpha():
+            names.append(t)
+    return names
 
 
 def load():

@@ -310,6 +310,16 @@ void ref_out_update_dense(const float *mu_a, const float *var_a, const float *jc
     put(dv, delta_var);
 }
 
+// n observations, 2n output units
+void ref_out_update_heteros(const float *mu_a, const float *var_a, const float *jcb,
+                            const float *obs, int n, float *delta_mu, float *delta_var) {
+    auto ma = vec(mu_a, 2 * n), va = vec(var_a, 2 * n), jc = vec(jcb, 2 * n), ob = vec(obs, n);
+    auto dm = vec(delta_mu, 2 * n), dv = vec(delta_var, 2 * n);
+    compute_delta_z_heteros(ma, va, jc, ob, 0, 2 * n, dm, dv);
+    put(dm, delta_mu);
+    put(dv, delta_var);
+}
+
 // n_states = block_size * n_obs floats in the state / delta arrays
 void ref_out_update_indexed(const float *mu_a, const float *var_a, const float *jcb,
                             const float *obs, const float *var_obs, const int *selected_idx,

@@ -496,6 +496,51 @@ void oracle_out_update_dense(const float *mu_a, const float *var_a,
     }
 }
 
+// src/base_output_updater.cpp:131-226. The output layer holds pairs: the mean
+// output at 2i and the (positive) error variance V2_bar_tilde at 2i+1; n counts
+// observations. The observation updates the mean output with the expected error
+// variance as observation noise, and the error-variance unit through the Gaussian
+// moments of V (posterior of the error) and V^2.
+void oracle_out_update_heteros(const float *mu_a, const float *var_a, const float *jcb,
+                               const float *obs, int n, float *delta_mu, float *delta_var) {
+    for (int i = 0; i < n; i++) {
+        const int col = 2 * i;
+        const float var_y = var_a[col], mu_y = mu_a[col], jcb_y = jcb[col];
+        const float mu_v2b = mu_a[col + 1], var_v2b = var_a[col + 1], cov_v2b = jcb[col + 1];
+        const float mu_v2 = mu_v2b;
+        const float var_v2 = 3.0f * var_v2b + 2.0f * mu_v2b * mu_v2b;
+        const float cov_y_v = mu_v2;
+        const float var_sum = var_y + mu_v2;
+        const float t = jcb_y / var_sum;
+        const float y = obs[i];
+        const bool bad_obs = std::isinf(y) || std::isnan(y);
+        if (std::isinf(t) || std::isnan(t) || bad_obs) {
+            delta_mu[col] = 0.0f;
+            delta_var[col] = 0.0f;
+        } else {
+            delta_mu[col] = t * (y - mu_y);
+            delta_var[col] = -t * jcb_y;
+        }
+        if (bad_obs) {
+            delta_mu[col + 1] = 0.0f;
+            delta_var[col + 1] = 0.0f;
+        } else {
+            const float mu_v_pos = cov_y_v / var_sum * (y - mu_y);
+            const float var_v_pos = mu_v2 - cov_y_v / var_sum * cov_y_v;
+            const float mu_v2_pos = mu_v_pos * mu_v_pos + var_v_pos;
+            const float var_v2_pos =
+                2.0f * var_v_pos * var_v_pos + 4.0f * var_v_pos * mu_v_pos * mu_v_pos;
+            const float k = var_v2b / var_v2;
+            const float mu_v2b_pos = mu_v2b + k * (mu_v2_pos - mu_v2);
+            const float var_v2b_pos = var_v2b + k * k * (var_v2_pos - var_v2);
+            float jv = cov_v2b / var_v2b;
+            if (std::isinf(jv) || std::isnan(jv)) jv = 0.0f;
+            delta_mu[col + 1] = jv * (mu_v2b_pos - mu_v2b);
+            delta_var[col + 1] = jv * jv * (var_v2b_pos - var_v2b);
+        }
+    }
+}
+
 // src/base_output_updater.cpp:67-93
 void oracle_out_update_indexed(const float *mu_a, const float *var_a,
                                const float *jcb, const float *obs,

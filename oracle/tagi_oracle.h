@@ -109,6 +109,11 @@ void oracle_out_update_dense(const float *mu_a, const float *var_a,
                              const float *jcb, const float *obs,
                              const float *var_obs, int n, float *delta_mu,
                              float *delta_var);
+/* reference: src/base_output_updater.cpp:131-226; n observations, 2n output units
+ * (mean at 2i, learned error variance at 2i+1) */
+void oracle_out_update_heteros(const float *mu_a, const float *var_a,
+                               const float *jcb, const float *obs, int n,
+                               float *delta_mu, float *delta_var);
 /* reference: src/base_output_updater.cpp:67-93; selected_idx is 1-based */
 void oracle_out_update_indexed(const float *mu_a, const float *var_a,
                                const float *jcb, const float *obs,

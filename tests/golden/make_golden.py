@@ -15,7 +15,9 @@ sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 sys.path.insert(0, os.path.dirname(HERE))
 
 import oracle  # noqa: E402
-from util import batchnorm_inputs, conv_inputs, linear_inputs, pool_inputs  # noqa: E402
+from model_cases import CASES, REF_THREADS, case_inputs, sample_index  # noqa: E402
+from util import (batchnorm_inputs, conv_inputs, heteros_inputs, linear_inputs,  # noqa: E402
+                  pool_inputs)
 
 # (kernel, stride, pad, pad_type, wi): every geometry of the Conv2d and ResNet-18
 # configurations plus a few odd ones
@@ -84,6 +86,30 @@ def layer_vectors(lib):
         out["sc_in%d" % i] = a
     out["sc_mu"], out["sc_var"] = lib.add_shortcut(v[0], v[1], v[2], v[3])
     out["scd_mu"], out["scd_var"] = lib.add_shortcut_delta(v[0], v[1], v[4], v[2], v[3])
+    return out
+
+
+def model_vectors(ref):
+    """Training steps of whole networks through the reference's own Sequential,
+    LayerBlock, ResNetBlock and OutputUpdater (oracle/ref_model.cpp): outputs of every
+    forward, input innovations where asked for, every parameter after every step (a
+    strided sample plus float64 sums for the large MLP) and the clamped-variance
+    counters. Inputs are regenerated from the seeds in tests/model_cases.py."""
+    out = {}
+    for name, c in CASES.items():
+        inp = case_inputs(name)
+        r = ref.model_run(c["spec"], inp["params"], inp["mu_x"], inp["var_x"], inp["y"],
+                          inp["var_y"], inp["sel"], c["B"], c["update"], c.get("n_enc", 0),
+                          c.get("input_state_update", False), c.get("eval_forward", False),
+                          REF_THREADS)
+        assert r["n_out"] == inp["n_out"]
+        out[name + "_out_mu"], out[name + "_out_var"] = r["out_mu"], r["out_var"]
+        if c.get("input_state_update", False):
+            out[name + "_in_dmu"], out[name + "_in_dvar"] = r["in_dmu"], r["in_dvar"]
+        idx = sample_index(r["params"].shape[1])
+        out[name + "_params"] = r["params"][:, idx]
+        out[name + "_params_sum"] = r["params"].astype(np.float64).sum(axis=1)
+        out[name + "_neg"] = r["neg"]
     return out
 
 
@@ -173,6 +199,10 @@ def main():
                                                                       var_obs, z, z)
     out["out_idx_dmu"], out["out_idx_dvar"] = ref.out_update_indexed(mu_a, var_a, jcb, y, vy, sel,
                                                                     n_obs, n_enc, z, z)
+    d = heteros_inputs(257, seed=13)
+    zz = np.zeros(2 * 257, np.float32)
+    out["out_het_dmu"], out["out_het_dvar"] = ref.out_update_heteros(d["mu_a"], d["var_a"],
+                                                                    d["jcb"], d["obs"], zz, zz)
     mz = rng.normal(0, 1, 512).astype(np.float32)
     mz[::9] = 0
     vz = rng.uniform(0.1, 1, 512).astype(np.float32)
@@ -180,7 +210,8 @@ def main():
     out["relu_mu_a"], out["relu_var_a"], out["relu_jcb"] = ref.relu_fwd(mz, vz)
     np.savez_compressed(os.path.join(HERE, "misc.npz"), **out)
     np.savez_compressed(os.path.join(HERE, "layers.npz"), **layer_vectors(ref))
-    for f in ("conv_idx.npz", "linear.npz", "conv.npz", "misc.npz", "layers.npz"):
+    np.savez_compressed(os.path.join(HERE, "models.npz"), **model_vectors(ref))
+    for f in ("conv_idx.npz", "linear.npz", "conv.npz", "misc.npz", "layers.npz", "models.npz"):
         print(f, os.path.getsize(os.path.join(HERE, f)))
 
 

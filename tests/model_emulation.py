@@ -140,22 +140,33 @@ class Emulator:
         z = np.zeros_like(mu)
         self.delta = self.o.out_update_dense(mu, var, jcb, y, var_y, z, z)
 
+    def update_heteros(self, y):
+        mu, var, jcb = self.out
+        z = np.zeros_like(mu)
+        self.delta = self.o.out_update_heteros(mu, var, jcb, y, z, z)
+
     # ---- backward --------------------------------------------------------------
-    def _bwd_list(self, layers, dmu, dvar, state):
-        """Layers in reverse; only the first non-activation layer of the list may
-        skip its state update."""
-        first = next(i for i, L in enumerate(layers) if not isinstance(L, ACTIVATIONS))
-        for i in range(len(layers) - 1, -1, -1):
-            L = layers[i]
-            if isinstance(L, ACTIVATIONS):
-                continue
-            dmu, dvar = self._bwd(L, dmu, dvar, state if i == first else True)
-        return dmu, dvar
+    def _bwd_list(self, layers, dmu, dvar, state, block):
+        """Layers in reverse. All but the first run with their state update. The
+        first one: in a Sequential (src/sequential.cpp:392-410) it runs and only its
+        state update depends on `state`; in a LayerBlock (src/layer_block.cpp:208-213)
+        it runs only when `state` is set and the block has more than one layer -
+        otherwise it gets no backward pass at all, so its parameters see no
+        innovation either."""
+        for i in range(len(layers) - 1, 0, -1):
+            if not isinstance(layers[i], ACTIVATIONS):
+                dmu, dvar = self._bwd(layers[i], dmu, dvar, True)
+        first = layers[0]
+        if isinstance(first, ACTIVATIONS):
+            return dmu, dvar
+        if block and not (state and len(layers) > 1):
+            return dmu, dvar
+        return self._bwd(first, dmu, dvar, state)
 
     def _bwd(self, L, dmu, dvar, state):
         o, B = self.o, self.B
         if isinstance(L, Block):
-            return self._bwd_list(L.layers, dmu, dvar, state)
+            return self._bwd_list(L.layers, dmu, dvar, state, True)
         if isinstance(L, Res):
             m = self._bwd(L.main, dmu, dvar, state)
             if L.shortcut is not None:
@@ -201,7 +212,7 @@ class Emulator:
 
     def backward(self, input_state_update=False):
         dmu, dvar = self.delta
-        self.input_delta = self._bwd_list(self.layers, dmu, dvar, input_state_update)
+        self.input_delta = self._bwd_list(self.layers, dmu, dvar, input_state_update, False)
 
     # ---- step -------------------------------------------------------------------
     def step(self):
@@ -210,6 +221,10 @@ class Emulator:
         self.neg = {}
         for sfx, L in param_layers(self.layers):
             shape = L.mu_w.shape
+            if not hasattr(L, "dw"):  # no backward pass yet: innovations are still zero
+                L.dw = (np.zeros(L.mu_w.size, np.float32), np.zeros(L.mu_w.size, np.float32))
+                if L.mu_b is not None:
+                    L.db = (np.zeros_like(L.mu_b), np.zeros_like(L.mu_b))
             m, v, c = o.param_update(L.mu_w.ravel(), L.var_w.ravel(), L.dw[0].ravel(),
                                      L.dw[1].ravel(), cap, True)
             L.mu_w, L.var_w = m.reshape(shape), v.reshape(shape)

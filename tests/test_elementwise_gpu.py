@@ -101,6 +101,36 @@ def test_out_update_dense_and_indexed(oracle_lib):
     assert np.count_nonzero(ref[0]) == B * n_enc
 
 
+def test_out_update_heteros(oracle_lib):
+    """Learned error variance: pairs (mean, expected squared error), with nan / inf
+    observations and zero denominators among the inputs."""
+    import cutagi_amd.functional as F
+    from util import heteros_inputs
+    for n in (40, 3001):
+        d = heteros_inputs(n, seed=n)
+        z = np.full(2 * n, 7.0, np.float32)
+        ref = oracle_lib.out_update_heteros(d["mu_a"], d["var_a"], d["jcb"], d["obs"], z, z)
+        dm, dv = _t(z), _t(z)
+        F.out_update_heteros(_t(d["mu_a"]), _t(d["var_a"]), _t(d["jcb"]), _t(d["obs"]), dm, dv)
+        np.testing.assert_allclose(dm.cpu().numpy(), ref[0], rtol=1e-5, atol=1e-7)
+        np.testing.assert_allclose(dv.cpu().numpy(), ref[1], rtol=1e-5, atol=1e-7)
+        assert ref[0][6] == 0 and ref[0][16] == 0 and ref[0][10] == 0 and ref[1][23] == 0
+
+
+def test_param_raw_update():
+    import torch
+    from cutagi_amd import capi
+    rng = np.random.default_rng(8)
+    n = 70001
+    mu, var, dmu, dvar = (rng.normal(0, 1, n).astype(np.float32) for _ in range(4))
+    t_mu, t_var, t_dmu, t_dvar = _t(mu), _t(var), _t(dmu), _t(dvar)
+    capi.check(capi.lib.tagi_param_raw_update(capi.ptr(t_dmu), capi.ptr(t_dvar), n,
+                                              capi.ptr(t_mu), capi.ptr(t_var), None))
+    torch.cuda.synchronize()
+    assert np.array_equal(t_mu.cpu().numpy(), mu + dmu)      # one fp32 addition: exact
+    assert np.array_equal(t_var.cpu().numpy(), var + dvar)   # no floor: may be negative
+
+
 def test_relu_and_store_states(oracle_lib):
     import torch
     import cutagi_amd.functional as F

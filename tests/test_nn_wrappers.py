@@ -34,8 +34,7 @@ def test_wrappers_build_and_forward_fields():
     assert idx.tolist() == [1, 2, 4, 8, 1, 2, 4, 7] and idx.dtype == np.int32
     with pytest.raises(RuntimeError, match="GPU only"):
         net(np.zeros((2, 784), np.float32))
-    with pytest.raises(NotImplementedError):
-        OutputUpdater("cpu").update_heteros(None, None, None)
+    assert callable(OutputUpdater("cpu").update_heteros)
 
 
 def test_label_helpers_match_the_reference_cost_functions(ref_lib):

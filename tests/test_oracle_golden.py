@@ -105,6 +105,11 @@ def test_update_output_relu(oracle_lib):
     r = oracle_lib.out_update_indexed(g["out_mu_a"], g["out_var_a"], g["out_jcb"], g["out_y"],
                                       g["out_vy"], g["out_sel"], 11, 4, z, z)
     _same(r[0], g["out_idx_dmu"], "idx dmu"); _same(r[1], g["out_idx_dvar"], "idx dvar")
+    from util import heteros_inputs
+    d = heteros_inputs(257, seed=13)
+    zz = np.zeros(2 * 257, np.float32)
+    r = oracle_lib.out_update_heteros(d["mu_a"], d["var_a"], d["jcb"], d["obs"], zz, zz)
+    _same(r[0], g["out_het_dmu"], "heteros dmu"); _same(r[1], g["out_het_dvar"], "heteros dvar")
     r = oracle_lib.relu_fwd(g["relu_mu_z"], g["relu_var_z"])
     _same(r[0], g["relu_mu_a"], "relu mu"); _same(r[1], g["relu_var_a"], "relu var")
     _same(r[2], g["relu_jcb"], "relu jcb")

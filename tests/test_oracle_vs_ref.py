@@ -103,6 +103,17 @@ def test_update_output_relu(oracle_lib, ref):
     assert _eq(oracle_lib.relu_fwd(m, v), ref.relu_fwd(m, v))
 
 
+def test_out_update_heteros(oracle_lib, ref):
+    from util import heteros_inputs
+    for n, seed in ((64, 1), (1001, 2)):
+        d = heteros_inputs(n, seed)
+        z = np.full(2 * n, 7.0, np.float32)   # every entry is written
+        a = oracle_lib.out_update_heteros(d["mu_a"], d["var_a"], d["jcb"], d["obs"], z, z)
+        b = ref.out_update_heteros(d["mu_a"], d["var_a"], d["jcb"], d["obs"], z, z)
+        assert np.array_equal(a[0], b[0], equal_nan=True) and np.array_equal(a[1], b[1], equal_nan=True)
+        assert a[0][6] == 0 and a[0][7] == 0 and a[0][16] == 0 and a[0][10] == 0
+
+
 # ---- layers around the hot path: MixtureReLU, BatchNorm2d, AvgPool2d, residual adds ----
 
 @pytest.mark.parametrize("threads", [1, 4])

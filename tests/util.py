@@ -94,3 +94,21 @@ def pool_inputs(wihi, woho, fo, B, seed=0):
         jcb=rng.uniform(0, 1, B * fo * wihi).astype(f),
         dmu=rng.standard_normal(B * fo * woho).astype(f),
         dvar=(-rng.uniform(0, 1e-2, B * fo * woho)).astype(f))
+
+
+def heteros_inputs(n, seed=0):
+    """Output layer with a learned error variance: 2n units (mean at 2i, expected
+    squared error at 2i+1, kept positive as the exponential activation in front of it
+    would) and n observations, with the special cases the reference guards: a nan and
+    an inf observation, a zero predictive variance, a zero variance of the error unit."""
+    rng = np.random.default_rng(seed)
+    f = np.float32
+    mu_a = rng.normal(0, 1, 2 * n).astype(f)
+    mu_a[1::2] = rng.uniform(0.05, 2.0, n)
+    var_a = rng.uniform(0.01, 0.5, 2 * n).astype(f)
+    jcb = rng.uniform(0.2, 1.0, 2 * n).astype(f)
+    obs = rng.normal(0, 1.5, n).astype(f)
+    obs[3], obs[8] = np.nan, np.inf
+    var_a[2 * 5], mu_a[2 * 5 + 1] = 0.25, -0.25     # var_sum == 0 -> inf -> zeros
+    var_a[2 * 11 + 1], jcb[2 * 11 + 1] = 0.0, 0.0   # 0/0 Jacobian ratio -> 0
+    return dict(mu_a=mu_a, var_a=var_a, jcb=jcb, obs=obs)
