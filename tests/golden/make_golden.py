@@ -15,6 +15,7 @@ sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 sys.path.insert(0, os.path.dirname(HERE))
 
 import oracle  # noqa: E402
+import full_size_cases as fs  # noqa: E402
 from model_cases import CASES, REF_THREADS, case_inputs, sample_index  # noqa: E402
 from util import (batchnorm_inputs, conv_inputs, heteros_inputs, linear_inputs,  # noqa: E402
                   pool_inputs)
@@ -101,7 +102,7 @@ def model_vectors(ref):
         r = ref.model_run(c["spec"], inp["params"], inp["mu_x"], inp["var_x"], inp["y"],
                           inp["var_y"], inp["sel"], c["B"], c["update"], c.get("n_enc", 0),
                           c.get("input_state_update", False), c.get("eval_forward", False),
-                          REF_THREADS)
+                          8 if c.get("big") else REF_THREADS)
         assert r["n_out"] == inp["n_out"]
         out[name + "_out_mu"], out[name + "_out_var"] = r["out_mu"], r["out_var"]
         if c.get("input_state_update", False):
@@ -110,6 +111,35 @@ def model_vectors(ref):
         out[name + "_params"] = r["params"][:, idx]
         out[name + "_params_sum"] = r["params"].astype(np.float64).sum(axis=1)
         out[name + "_neg"] = r["neg"]
+    return out
+
+
+def full_size_vectors(ref, threads=8):
+    """The benchmark configurations at their full sizes through the reference's CPU
+    kernels (seconds each with 8 threads): sampled entries and sums of every output."""
+    out = {}
+    for name in fs.LINEAR:
+        d = fs.linear_inputs(name)
+        r = ref.linear_fwd(d["mu_w"], d["var_w"], d["mu_b"], d["var_b"], d["mu_a"], d["var_a"],
+                           threads)
+        r += ref.linear_bwd_dz(d["mu_w"], d["jcb"], d["delta_mu"], d["delta_var"], threads)
+        r += ref.linear_bwd_dw(d["var_w"], d["mu_a"], d["delta_mu"], d["delta_var"], threads)
+        r += ref.linear_bwd_db(d["var_b"], d["delta_mu"], d["delta_var"], threads)
+        out.update(fs.summarize(name, dict(zip(fs.LINEAR_OUTPUTS, r))))
+        print(name, "done", flush=True)
+    for name, g in fs.CONV.items():
+        fi, fo, k, wi, B = g["fi"], g["fo"], g["k"], g["wi"], g["B"]
+        pix = wi * wi
+        idx = ref.conv2d_build_idx(k, 1, wi, wi, 1, 1, k * k * fi * fo + 1)
+        d = fs.conv_inputs(name)
+        r = ref.conv2d_fwd(d["mu_w"], d["var_w"], None, None, d["mu_a"], d["var_a"],
+                           idx["Fmwa_2"], pix, fo, pix, fi, k, B, threads)
+        r += ref.conv2d_bwd_dz(d["mu_w"], d["jcb"], d["delta_mu"], d["delta_var"], idx["FCzwa_1"],
+                               idx["Szz_ud"], pix, fo, pix, fi, k, idx["h"], B, threads)
+        r += ref.conv2d_bwd_dw(d["var_w"], None, d["mu_a"], d["delta_mu"], d["delta_var"],
+                               idx["Fmwa_2"], B, fo, pix, pix, fi, k, threads)[:2]
+        out.update(fs.summarize(name, dict(zip(fs.CONV_OUTPUTS, r))))
+        print(name, "done", flush=True)
     return out
 
 
@@ -211,7 +241,9 @@ def main():
     np.savez_compressed(os.path.join(HERE, "misc.npz"), **out)
     np.savez_compressed(os.path.join(HERE, "layers.npz"), **layer_vectors(ref))
     np.savez_compressed(os.path.join(HERE, "models.npz"), **model_vectors(ref))
-    for f in ("conv_idx.npz", "linear.npz", "conv.npz", "misc.npz", "layers.npz", "models.npz"):
+    np.savez_compressed(os.path.join(HERE, "full_size.npz"), **full_size_vectors(ref))
+    for f in ("conv_idx.npz", "linear.npz", "conv.npz", "misc.npz", "layers.npz", "models.npz",
+              "full_size.npz"):
         print(f, os.path.getsize(os.path.join(HERE, f)))
 
 

@@ -347,3 +347,33 @@ def sample_index(n, limit=40000):
     if n <= limit:
         return np.arange(n)
     return np.arange(0, n, -(-n // limit))
+
+
+def resnet18_spec():
+    """The CIFAR ResNet-18 of the reference's examples (examples/tagi_resnet_model.py:
+    56-147) as a description: stem, eight residual blocks (three of them strided with a
+    2x2 projection shortcut), global average pooling, an 11-unit head."""
+    bn = "BatchNorm2d {c} 1e-5 0.9 1"
+
+    def main(i, o, s, pt):
+        return ("Conv2d {i} {o} 3 0 {s} 1 {pt} 0 0 MixtureReLU " + bn.format(c=o) +
+                " Conv2d {o} {o} 3 0 1 1 1 0 0 MixtureReLU " + bn.format(c=o)).format(
+                    i=i, o=o, s=s, pt=pt)
+
+    def same(c):
+        return "ResNetBlock [ " + main(c, c, 1, 1) + " ] [ ]"
+
+    def down(i, o):
+        return ("ResNetBlock [ " + main(i, o, 2, 2) + " ] [ Conv2d {i} {o} 2 0 2 0 1 0 0 MixtureReLU "
+                .format(i=i, o=o) + bn.format(c=o) + " ]")
+
+    return " ".join(["Conv2d 3 64 3 0 1 1 1 32 32 MixtureReLU " + bn.format(c=64),
+                     same(64), same(64), down(64, 128), same(128), down(128, 256), same(256),
+                     down(256, 512), same(512), "AvgPool2d 4 -1 0 0 Linear 512 11 1"])
+
+
+# The ResNet-18 configuration at a batch the CPU reference finishes in seconds: one
+# training step with the hierarchical-softmax update. `big`: left out of the CPU
+# tests that re-run a case through the emulator (tens of seconds there).
+CASES["resnet18_cifar_batch8"] = dict(spec=resnet18_spec(), B=8, steps=1, update=1, n_enc=4,
+                                      var_x=False, seed=18, big=True)

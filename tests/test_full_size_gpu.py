@@ -131,3 +131,77 @@ def test_conv2d_full_size_against_float64_closed_forms():
     _check(dw[0], sum_mu * V, "delta_mu_w")
     _check(dw[1], sum_var * V ** 2, "delta_var_w")
     assert float(dw[1].max()) <= 0.0
+
+
+# ---- against the reference's own fp32 CPU results at the full sizes ---------------------
+# tests/golden/full_size.npz holds, for every output tensor of the three Linear shapes
+# and the Conv2d configuration, the values the compiled reference produced at a seeded
+# sample of entries plus float64 sums over the whole tensor (tests/golden/make_golden.py;
+# the inputs regenerate from tests/full_size_cases.py on any machine). Three checks per
+# tensor: the 1e-4 gate against the reference's values (elementwise as well for the
+# same-signed tensors), the whole-tensor sum, and the distance to the float64 closed
+# form, which may not exceed twice the reference's own distance to it.
+
+def _against_reference(name, outputs, truth, gold):
+    import full_size_cases as fs
+    from util import SAME_SIGN, assert_close, rel_err
+    report = []
+    for tensor, got in outputs.items():
+        flat = got.reshape(-1)
+        idx = fs.sample_of(name, tensor, flat.numel())
+        import torch
+        sample = flat[torch.from_numpy(idx).cuda()].cpu().numpy()
+        ref = gold["%s_%s" % (name, tensor)]
+        assert_close(sample, ref, "%s %s vs reference CPU" % (name, tensor),
+                     same_sign=tensor in SAME_SIGN)
+        ref_sum, ref_abs = gold["%s_%s_sums" % (name, tensor)]
+        got_sum = float(flat.double().sum())
+        assert abs(got_sum - ref_sum) <= 1e-4 * ref_abs, (name, tensor, got_sum, ref_sum)
+        e_gpu, e_ref = rel_err(sample, truth[tensor]), rel_err(ref, truth[tensor])
+        report.append("%-12s gpu-vs-f64 %.2e  reference-vs-f64 %.2e" % (tensor, e_gpu, e_ref))
+        assert e_gpu <= max(2 * e_ref, 2e-6), "%s %s: %.3e from float64, the reference %.3e" % (
+            name, tensor, e_gpu, e_ref)
+    print("\n" + name + "\n  " + "\n  ".join(report))
+
+
+@pytest.mark.parametrize("name", ["linear_4096_b256", "linear_8192_b8", "linear_8192_b16"])
+def test_linear_full_size_against_reference_cpu(name):
+    import os
+    import torch
+    import cutagi_amd.functional as F
+    import full_size_cases as fs
+    gold = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                                "full_size.npz"), allow_pickle=False)
+    d = fs.linear_inputs(name)
+    t = {k: torch.from_numpy(v).cuda() for k, v in d.items()}
+    out = list(F.linear_fwd(t["mu_w"], t["var_w"], t["mu_b"], t["var_b"], t["mu_a"], t["var_a"]))
+    out += list(F.linear_bwd(t["mu_w"], t["var_w"], t["var_b"], t["mu_a"], t["jcb"],
+                             t["delta_mu"], t["delta_var"]))
+    torch.cuda.synchronize()
+    _against_reference(name, dict(zip(fs.LINEAR_OUTPUTS, out)), fs.linear_float64(name, d), gold)
+
+
+def test_conv2d_full_size_against_reference_cpu():
+    import os
+    import torch
+    import cutagi_amd.functional as F
+    import full_size_cases as fs
+    from cutagi_amd import capi
+    name = "conv_3x3_64_32_b128"
+    gold = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                                "full_size.npz"), allow_pickle=False)
+    g = fs.CONV[name]
+    fi, fo, k, wi, B = g["fi"], g["fo"], g["k"], g["wi"], g["B"]
+    pix = wi * wi
+    idx = capi.conv2d_build_idx(k, 1, wi, wi, 1, 1, k * k * fi * fo + 1)
+    ti = {n: torch.from_numpy(idx[n]).cuda() for n in ("Fmwa_2", "FCzwa_1", "Szz_ud")}
+    d = fs.conv_inputs(name)
+    t = {key: torch.from_numpy(v).cuda() for key, v in d.items()}
+    out = list(F.conv2d_fwd(t["mu_w"], t["var_w"], None, None, t["mu_a"], t["var_a"],
+                            ti["Fmwa_2"], pix, fo, pix, fi, k, B))
+    out += list(F.conv2d_bwd_dz(t["mu_w"], t["jcb"], t["delta_mu"], t["delta_var"], ti["FCzwa_1"],
+                                ti["Szz_ud"], pix, fo, pix, fi, k, idx["h"], B))
+    out += list(F.conv2d_bwd_dw(t["var_w"], None, t["mu_a"], t["delta_mu"], t["delta_var"],
+                                ti["Fmwa_2"], B, fo, pix, pix, fi, k))[:2]
+    torch.cuda.synchronize()
+    _against_reference(name, dict(zip(fs.CONV_OUTPUTS, out)), fs.conv_float64(name, d), gold)

@@ -57,7 +57,8 @@ def test_description_parser_and_sizes(ref_lib):
             assert ref_lib.model_param_sizes(c["spec"]) == sizes, name
 
 
-@pytest.mark.parametrize("name", [n for n in CASES if not CASES[n].get("eval_forward")])
+@pytest.mark.parametrize("name", [n for n in CASES if not CASES[n].get("eval_forward")
+                                  and not CASES[n].get("big")])
 def test_emulation_matches_reference_drivers(oracle_lib, name):
     c = CASES[name]
     r = run_emulation(oracle_lib, name)
@@ -110,11 +111,13 @@ def test_vectors_regenerate_from_the_reference(ref_lib, name):
     if ref_lib is None:
         pytest.skip("the reference library is not built here")
     c = CASES[name]
+    if c.get("big") and not os.environ.get("TAGI_SLOW_TESTS"):
+        pytest.skip("ten seconds of CPU: runs with TAGI_SLOW_TESTS=1")
     inp = case_inputs(name)
     r = ref_lib.model_run(c["spec"], inp["params"], inp["mu_x"], inp["var_x"], inp["y"],
                           inp["var_y"], inp["sel"], c["B"], c["update"], c.get("n_enc", 0),
                           c.get("input_state_update", False), c.get("eval_forward", False),
-                          REF_THREADS)
+                          8 if c.get("big") else REF_THREADS)
     assert np.array_equal(r["out_mu"], GOLD[name + "_out_mu"])
     assert np.array_equal(r["out_var"], GOLD[name + "_out_var"])
     idx = sample_index(r["params"].shape[1])

@@ -18,11 +18,31 @@ def rel_err(x, ref):
     return float(np.max(np.abs(x - ref) / denom))
 
 
-def assert_close(x, ref, what, tol=TOL):
+def max_rel(x, ref):
+    """Plain elementwise max |x - ref| / |ref| (entries where both are zero count 0)."""
+    x = np.asarray(x, dtype=np.float64).ravel()
+    ref = np.asarray(ref, dtype=np.float64).ravel()
+    if ref.size == 0:
+        return 0.0
+    diff = np.abs(x - ref)
+    return float(np.max(np.where(diff == 0, 0.0, diff / np.maximum(np.abs(ref), 1e-300))))
+
+
+def assert_close(x, ref, what, tol=TOL, same_sign=False):
+    """The parity gate. same_sign: the tensor is a sum of terms of one sign (var_z,
+    the variance innovations), so nothing cancels and the plain elementwise relative
+    error is held to the same tolerance as well."""
     e = rel_err(x, ref)
     assert np.all(np.isfinite(np.asarray(x))), what + ": non-finite values"
     assert e <= tol, "%s: rel err %.3e > %.1e" % (what, e, tol)
+    if same_sign:
+        m = max_rel(x, ref)
+        assert m <= tol, "%s: elementwise rel err %.3e > %.1e" % (what, m, tol)
     return e
+
+
+# outputs of the Linear / Conv2d path that are sums of terms of one sign
+SAME_SIGN = ("var_z", "delta_var_z", "delta_var_w", "delta_var_b")
 
 
 def linear_inputs(K, N, B, seed=0, bias=True, jcb_random=False):
