@@ -28,7 +28,8 @@ SIGNATURES = {
     "tagi_hip_version": (_i, []),
     "tagi_hip_device_count": (_i, [_ip]),
     "tagi_hip_error_string": (ctypes.c_char_p, [_i]),
-    "tagi_hip_workspace_reserve": (_i, [_sz]),
+    "tagi_hip_workspace_reserve": (_i, [_sz, _vp]),
+    "tagi_hip_device_info": (_i, [_ip, _ip, ctypes.c_char_p, _sz]),
     "tagi_hip_shutdown": (_i, []),
     "tagi_hip_tune": (_i, [ctypes.c_char_p, _i]),
     "tagi_linear_fwd": (_i, [_vp] * 6 + [_i] * 4 + [_vp] * 3),
@@ -108,6 +109,14 @@ def device_count():
     n = ctypes.c_int(0)
     check(lib.tagi_hip_device_count(ctypes.byref(n)))
     return n.value
+
+
+def device_info():
+    """(compute units, clock in MHz, name) of the current device."""
+    cus, mhz = ctypes.c_int(0), ctypes.c_int(0)
+    name = ctypes.create_string_buffer(256)
+    check(lib.tagi_hip_device_info(ctypes.byref(cus), ctypes.byref(mhz), name, 256))
+    return cus.value, mhz.value, name.value.decode()
 
 
 def tune(key, value):

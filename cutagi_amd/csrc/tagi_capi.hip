@@ -3,6 +3,8 @@
 #include <cstdint>
 #include <cstring>
 #include <mutex>
+#include <utility>
+#include <vector>
 
 #include "../../include/tagi_hip.h"
 #include "tagi_internal.h"
@@ -18,8 +20,7 @@ static __device__ __align__(256) float scratch[STATIC_SCRATCH_BYTES / sizeof(flo
 
 namespace {
 
-constexpr int ABI_VERSION = 100;
-constexpr int MAX_DEVICES = 16;
+constexpr int ABI_VERSION = 101;
 
 #define TAGI_TRY(expr)                          \
     do {                                        \
@@ -31,38 +32,51 @@ struct Workspace {
     float *ptr = nullptr;
     size_t bytes = 0;
 };
-Workspace g_ws[MAX_DEVICES];
+// One grow-only workspace per (device, stream): partial sums stay in it between the
+// launches of a call, so calls on different streams of a device must not share one.
+// Calls on one stream are ordered by the stream and share theirs.
+struct DeviceWorkspaces {
+    std::vector<std::pair<hipStream_t, Workspace>> by_stream;
+};
+DeviceWorkspaces g_ws[MAX_DEVICES];
 std::mutex g_ws_mutex;
+int g_num_cu[MAX_DEVICES];
 
 // Grow-only. Reallocation waits for the device, so buffers still in use by
 // queued kernels are never freed under them.
-int workspace_get(size_t bytes, float **out) {
+int workspace_get(size_t bytes, hipStream_t stream, float **out) {
     int dev = 0;
     TAGI_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= MAX_DEVICES) return TAGI_ERR_NO_DEVICE;
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    Workspace &w = g_ws[dev];
-    if (w.bytes < bytes) {
-        TAGI_TRY(hipDeviceSynchronize());
-        if (w.ptr != nullptr) TAGI_TRY(hipFree(w.ptr));
-        w.ptr = nullptr;
-        w.bytes = 0;
-        const size_t want = (bytes + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
-        TAGI_TRY(hipMalloc(reinterpret_cast<void **>(&w.ptr), want));
-        w.bytes = want;
+    Workspace *w = nullptr;
+    for (auto &entry : g_ws[dev].by_stream)
+        if (entry.first == stream) w = &entry.second;
+    if (w == nullptr) {
+        g_ws[dev].by_stream.emplace_back(stream, Workspace());
+        w = &g_ws[dev].by_stream.back().second;
     }
-    *out = w.ptr;
+    if (w->bytes < bytes) {
+        TAGI_TRY(hipDeviceSynchronize());
+        if (w->ptr != nullptr) TAGI_TRY(hipFree(w->ptr));
+        w->ptr = nullptr;
+        w->bytes = 0;
+        const size_t want = (bytes + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
+        TAGI_TRY(hipMalloc(reinterpret_cast<void **>(&w->ptr), want));
+        w->bytes = want;
+    }
+    *out = w->ptr;
     return TAGI_OK;
 }
 
 // Where a call's partial sums go: the grow-only workspace above, or the static
 // array of the entry point that allocates nothing.
-typedef int (*ScratchSource)(size_t bytes, float **out);
+typedef int (*ScratchSource)(size_t bytes, hipStream_t stream, float **out);
 
 float *g_scratch_ptr[MAX_DEVICES];
 std::mutex g_scratch_mutex;
 
-int static_scratch_get(size_t bytes, float **out) {
+int static_scratch_get(size_t bytes, hipStream_t, float **out) {
     if (bytes > STATIC_SCRATCH_BYTES) return TAGI_ERR_UNSUPPORTED;
     int dev = 0;
     TAGI_TRY(hipGetDevice(&dev));
@@ -115,21 +129,24 @@ int pick_tile(int rows) {
 int pick_splits(int tiles, int reduction, int forced, int min_tiles = 8) {
     const int kt = gemm_k_tile();
     const int k_tiles = ceil_div(reduction, kt);
-    int s = forced > 0 ? forced : ceil_div(2 * NUM_CU, tiles);
+    int s = forced > 0 ? forced : ceil_div(2 * num_cu(), tiles);
     int cap = k_tiles / min_tiles > 0 ? k_tiles / min_tiles : 1;
     // A launch that leaves most of the chip empty is bound by the latency of its
     // k-tile loop (one memory round trip per k-tile, nothing else on the CU to hide
     // it), not by throughput: such a launch is cut into single k-tiles when its
     // reduction is long enough to pay for the fold (784 -> 128, batch 32: forward
     // 31 -> 12 us).
-    if (tiles * 8 <= NUM_CU && k_tiles >= 8) cap = k_tiles < 32 ? k_tiles : 32;
+    if (tiles * 8 <= num_cu() && k_tiles >= 8) cap = k_tiles < 32 ? k_tiles : 32;
     if (forced <= 0 && s > cap) s = cap;
     if (s > k_tiles) s = k_tiles;
     if (s < 1) s = 1;
     return s;
 }
 
-int gemv_max_batch() { return g_tune.gemv_max_batch >= 0 ? g_tune.gemv_max_batch : 16; }
+// the streaming kernels hold at most 16 samples
+int gemv_max_batch() {
+    return g_tune.gemv_max_batch >= 0 && g_tune.gemv_max_batch < 16 ? g_tune.gemv_max_batch : 16;
+}
 
 // Tile shape and reduction slices of a tiled launch.
 void plan_gemm(GemmMode mode, GemmParams &p, int forced_splits, int *tile_out) {
@@ -155,7 +172,7 @@ int run_gemm(GemmMode mode, GemmParams p, bool vec, int forced_splits, hipStream
     if (splits > 1) {
         float *ws = nullptr;
         const size_t part = (size_t)splits * p.M * p.N;
-        int rc = scratch_get(2 * part * sizeof(float), &ws);
+        int rc = scratch_get(2 * part * sizeof(float), stream, &ws);
         if (rc != TAGI_OK) return rc;
         p.ws0 = ws;
         p.ws1 = ws + part;
@@ -178,6 +195,23 @@ int run_gemm(GemmMode mode, GemmParams p, bool vec, int forced_splits, hipStream
 }
 
 }  // namespace
+
+namespace tagi {
+int num_cu() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return 256;
+    if (g_num_cu[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+            n <= 0) {
+            (void)hipGetLastError();
+            n = 256;
+        }
+        g_num_cu[dev] = n;
+    }
+    return g_num_cu[dev];
+}
+}  // namespace tagi
 
 extern "C" {
 
@@ -208,9 +242,23 @@ const char *tagi_hip_error_string(int code) {
     return "tagi: unknown error";
 }
 
-int tagi_hip_workspace_reserve(size_t bytes) {
+int tagi_hip_workspace_reserve(size_t bytes, void *stream) {
     float *p = nullptr;
-    return workspace_get(bytes, &p);
+    return workspace_get(bytes, static_cast<hipStream_t>(stream), &p);
+}
+
+int tagi_hip_device_info(int *compute_units, int *clock_mhz, char *name, size_t name_capacity) {
+    int dev = 0;
+    TAGI_TRY(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    TAGI_TRY(hipGetDeviceProperties(&prop, dev));
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    if (clock_mhz) *clock_mhz = prop.clockRate / 1000;
+    if (name && name_capacity > 0) {
+        strncpy(name, prop.name, name_capacity - 1);
+        name[name_capacity - 1] = '\0';
+    }
+    return TAGI_OK;
 }
 
 int tagi_hip_shutdown(void) {
@@ -218,11 +266,12 @@ int tagi_hip_shutdown(void) {
     int cur = 0;
     if (hipGetDevice(&cur) != hipSuccess) return TAGI_OK;
     for (int d = 0; d < MAX_DEVICES; d++) {
-        if (g_ws[d].ptr == nullptr) continue;
+        if (g_ws[d].by_stream.empty()) continue;
         TAGI_TRY(hipSetDevice(d));
         TAGI_TRY(hipDeviceSynchronize());
-        TAGI_TRY(hipFree(g_ws[d].ptr));
-        g_ws[d] = Workspace();
+        for (auto &entry : g_ws[d].by_stream)
+            if (entry.second.ptr != nullptr) TAGI_TRY(hipFree(entry.second.ptr));
+        g_ws[d].by_stream.clear();
     }
     TAGI_TRY(hipSetDevice(cur));
     return TAGI_OK;
@@ -271,7 +320,7 @@ static int linear_fwd_impl(const float *mu_w, const float *var_w, const float *m
         // 9..16 samples: the 16-wide streaming kernel
         const int blocks = ceil_div(N, gemv16_fwd_rows_per_block());
         const int step = gemv16_fwd_k_step();
-        int splits = g_tune.fwd_splits > 0 ? g_tune.fwd_splits : ceil_div(2 * NUM_CU, blocks);
+        int splits = g_tune.fwd_splits > 0 ? g_tune.fwd_splits : ceil_div(2 * num_cu(), blocks);
         const int max_splits = ceil_div(K, 4 * step);
         if (splits > max_splits) splits = max_splits;
         const int min_splits = ceil_div(K, gemv16_fwd_max_slice());
@@ -280,7 +329,7 @@ static int linear_fwd_impl(const float *mu_w, const float *var_w, const float *m
         splits = ceil_div(K, per);
         float *ws = nullptr;
         const size_t part = (size_t)splits * B * N;
-        int rc = scratch_get(2 * part * sizeof(float), &ws);
+        int rc = scratch_get(2 * part * sizeof(float), stream, &ws);
         if (rc != TAGI_OK) return rc;
         TAGI_TRY(launch_gemv16_fwd(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, ws, ws + part,
                                    stream));
@@ -298,7 +347,7 @@ static int linear_fwd_impl(const float *mu_w, const float *var_w, const float *m
                                 : 0;
         const int blocks = ceil_div(N, gemv_fwd_rows_per_block(variant));
         const int step = gemv_fwd_k_step();
-        int splits = g_tune.fwd_splits > 0 ? g_tune.fwd_splits : ceil_div(2 * NUM_CU, blocks);
+        int splits = g_tune.fwd_splits > 0 ? g_tune.fwd_splits : ceil_div(2 * num_cu(), blocks);
         const int max_splits = ceil_div(K, 4 * step);
         if (splits > max_splits) splits = max_splits;
         const int min_splits = ceil_div(K, gemv_fwd_max_slice(B));
@@ -307,7 +356,7 @@ static int linear_fwd_impl(const float *mu_w, const float *var_w, const float *m
         splits = ceil_div(K, per);
         float *ws = nullptr;
         const size_t part = (size_t)splits * B * N;
-        int rc = scratch_get(2 * part * sizeof(float), &ws);
+        int rc = scratch_get(2 * part * sizeof(float), stream, &ws);
         if (rc != TAGI_OK) return rc;
         TAGI_TRY(launch_gemv_fwd(mu_w, var_w, mu_a, var_a, K, N, B, splits,
                                  g_tune.gemv_swz >= 0 ? g_tune.gemv_swz : 3, variant, ws,
@@ -355,7 +404,7 @@ static int linear_bwd_dz_impl(const float *mu_w, const float *jcb, const float *
     if (B <= gemv_max_batch() && vec) {
         const int blocks = ceil_div(K, wide16 ? gemv16_dz_cols_per_block() : gemv_dz_cols_per_block());
         const int step = wide16 ? gemv16_dz_n_step() : gemv_dz_n_step();
-        int splits = g_tune.dz_splits > 0 ? g_tune.dz_splits : ceil_div(NUM_CU, blocks);
+        int splits = g_tune.dz_splits > 0 ? g_tune.dz_splits : ceil_div(num_cu(), blocks);
         const int max_splits = ceil_div(N, 2 * step);
         if (splits > max_splits) splits = max_splits;
         const int min_splits = ceil_div(N, wide16 ? gemv16_dz_max_slice() : gemv_dz_max_slice(B));
@@ -364,7 +413,7 @@ static int linear_bwd_dz_impl(const float *mu_w, const float *jcb, const float *
         splits = ceil_div(N, per);
         float *ws = nullptr;
         const size_t part = (size_t)splits * B * K;
-        int rc = workspace_get(2 * part * sizeof(float), &ws);
+        int rc = workspace_get(2 * part * sizeof(float), stream, &ws);
         if (rc != TAGI_OK) return rc;
         if (wide16)
             TAGI_TRY(launch_gemv16_dz(mu_w, delta_mu, delta_var, K, N, B, per, splits, ws,
@@ -556,6 +605,7 @@ int tagi_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b, co
         return TAGI_ERR_INVALID_ARG;
     if (bias && (!mu_b || !var_b)) return TAGI_ERR_INVALID_ARG;
     if (!conv_sizes_ok(B, fo, woho, fi, wihi, ki)) return TAGI_ERR_UNSUPPORTED;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
     int tile = 0, splits = 1;
     conv2d_plan(fo, B * woho, ki * ki * fi, &tile, &splits);
     if (g_tune.conv_splits > 0) splits = g_tune.conv_splits;
@@ -563,12 +613,11 @@ int tagi_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b, co
     float *ws = nullptr;
     const size_t part = splits > 1 ? (size_t)splits * fo * B * woho : 0;
     if (part) {
-        int rc = workspace_get(2 * part * sizeof(float), &ws);
+        int rc = workspace_get(2 * part * sizeof(float), stream, &ws);
         if (rc != TAGI_OK) return rc;
     }
     TAGI_TRY(launch_conv2d_fwd(mu_w, var_w, mu_b, var_b, mu_a, var_a, aidx, woho, fo, wihi, fi, ki,
-                               B, bias, tile, splits, ws, ws + part, mu_z, var_z,
-                               static_cast<hipStream_t>(stream_)));
+                               B, bias, tile, splits, ws, ws + part, mu_z, var_z, stream));
     return TAGI_OK;
 }
 
@@ -582,6 +631,7 @@ int tagi_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *delta_m
     if (woho <= 0 || fo <= 0 || wihi <= 0 || fi <= 0 || ki <= 0 || nr <= 0 || B <= 0)
         return TAGI_ERR_INVALID_ARG;
     if (!conv_sizes_ok(B, fo, woho, fi, wihi, ki)) return TAGI_ERR_UNSUPPORTED;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
     int tile = 0, splits = 1;
     conv2d_plan(fi, B * wihi, ki * ki * fo, &tile, &splits);
     if (g_tune.conv_splits > 0) splits = g_tune.conv_splits;
@@ -589,12 +639,12 @@ int tagi_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *delta_m
     float *ws = nullptr;
     const size_t part = splits > 1 ? (size_t)splits * fi * B * wihi : 0;
     if (part) {
-        int rc = workspace_get(2 * part * sizeof(float), &ws);
+        int rc = workspace_get(2 * part * sizeof(float), stream, &ws);
         if (rc != TAGI_OK) return rc;
     }
     TAGI_TRY(launch_conv2d_bwd_dz(mu_w, jcb, delta_mu_out, delta_var_out, zw_idx, zud_idx, woho,
                                   fo, wihi, fi, ki, nr, B, tile, splits, ws, ws + part, delta_mu,
-                                  delta_var, static_cast<hipStream_t>(stream_)));
+                                  delta_var, stream));
     return TAGI_OK;
 }
 
@@ -626,14 +676,14 @@ int tagi_conv2d_bwd_dw(const float *var_w, const float *var_b, const float *mu_a
                                                fi, ki, tile) != 0;
     int splits = g_tune.conv_dw_splits > 0 ? g_tune.conv_dw_splits
                  : stencil                 ? conv2d_bwd_dw_stencil_splits(out_tiles)
-                                           : 3 * conv2d_bwd_dw_blocks_per_cu(tile) * NUM_CU / out_tiles;
+                                           : 3 * conv2d_bwd_dw_blocks_per_cu(tile) * num_cu() / out_tiles;
     const int max_splits = ceil_div(red, 256);
     if (splits > max_splits) splits = max_splits;
     if (splits < 1) splits = 1;
     float *ws = nullptr;
     const size_t part = (size_t)splits * fo * ki * ki * fi;
     const int chunks = 64;  // slices of the (b, o) range in the bias reduction
-    int rc = workspace_get((2 * part + 2 * (size_t)chunks * fo) * sizeof(float), &ws);
+    int rc = workspace_get((2 * part + 2 * (size_t)chunks * fo) * sizeof(float), stream, &ws);
     if (rc != TAGI_OK) return rc;
     TAGI_TRY(launch_conv2d_bwd_dw(var_w, mu_a, delta_mu_out, delta_var_out, aidx, B, fo, woho, wihi,
                                   fi, ki, tile, splits, ws, ws + part, delta_mu_w, delta_var_w, stream));
@@ -766,7 +816,8 @@ int tagi_batchnorm2d_stats(const float *mu_a, const float *var_a, int wihi, int 
     if (!mu_a || !var_a || !mu_s || !var_s || !mu_ra || !var_ra) return TAGI_ERR_INVALID_ARG;
     if (!bn_sizes_ok(wihi, fi, B)) return TAGI_ERR_INVALID_ARG;
     float *ws = nullptr;
-    int rc = workspace_get(batchnorm2d_scratch_floats(fi, B) * sizeof(float), &ws);
+    int rc = workspace_get(batchnorm2d_scratch_floats(fi, B) * sizeof(float),
+                           static_cast<hipStream_t>(stream), &ws);
     if (rc != TAGI_OK) return rc;
     TAGI_TRY(launch_batchnorm2d_stats(mu_a, var_a, wihi, fi, B, momentum, ws, mu_s, var_s, mu_ra,
                                       var_ra, static_cast<hipStream_t>(stream)));
@@ -803,7 +854,8 @@ int tagi_batchnorm2d_bwd(const float *mu_w, const float *var_w, const float *var
     if (!bn_sizes_ok(wihi, fi, B)) return TAGI_ERR_INVALID_ARG;
     if (!state_update && !param_update) return TAGI_OK;
     float *ws = nullptr;
-    int rc = workspace_get(batchnorm2d_scratch_floats(fi, B) * sizeof(float), &ws);
+    int rc = workspace_get(batchnorm2d_scratch_floats(fi, B) * sizeof(float),
+                           static_cast<hipStream_t>(stream), &ws);
     if (rc != TAGI_OK) return rc;
     TAGI_TRY(launch_batchnorm2d_bwd(mu_w, var_w, bias ? var_b : nullptr, mu_a, jcb, mu_norm,
                                     var_norm, delta_mu_out, delta_var_out, epsilon, wihi, fi, B,

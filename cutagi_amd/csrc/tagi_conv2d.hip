@@ -713,7 +713,7 @@ void conv2d_plan(int M, int N, int R, int *tile, int *splits) {
     *tile = M > 32 ? TILE_64x128 : TILE_32x128;
     const int tiles = ceil_div(M, tile_rows(*tile)) * ceil_div(N, tile_cols(*tile));
     const int k_tiles = ceil_div(R, KT);
-    int s = ceil_div(2 * NUM_CU, tiles);
+    int s = ceil_div(2 * num_cu(), tiles);
     const int cap = k_tiles / 8 > 0 ? k_tiles / 8 : 1;  // at least 8 k-tiles per slice
     if (s > cap) s = cap;
     if (s < 1) s = 1;
@@ -856,7 +856,7 @@ int conv2d_bwd_dw_stencil(const float *mu_a, const float *dmu, const float *dvar
 // fewest rounds of resident workgroups that are at least 95 % full, else the
 // fullest of up to four rounds. A partly filled round costs as much as a full one.
 int conv2d_bwd_dw_stencil_splits(int out_tiles) {
-    const int resident = 2 * NUM_CU;
+    const int resident = 2 * num_cu();
     int best = 1;
     double best_fill = 0.0;
     for (int rounds = 1; rounds <= 4; rounds++) {

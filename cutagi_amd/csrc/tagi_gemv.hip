@@ -744,6 +744,7 @@ hipError_t launch_gemv_dw(const float *var_w, const float *mu_a, const float *dm
                           float *dvar_w, const float *var_b, float *dmu_b, float *dvar_b,
                           const DzFold *fold_in, hipStream_t stream) {
     const DzFold fold = fold_in ? *fold_in : DzFold();
+    if (B > 16) return hipErrorInvalidValue;  // the kernels hold at most 16 samples
     if (B <= 4)
         dw_launch<4>(var_w, mu_a, dmu, dvar, K, N, B, rev, dmu_w, dvar_w, var_b, dmu_b, dvar_b,
                      fold, stream);

@@ -6,7 +6,10 @@
 
 namespace tagi {
 
-constexpr int NUM_CU = 256;  // MI355X
+// Compute units of the current device (256 on an MI355X), asked of the runtime once
+// per device; launch shapes that aim at "workgroups per CU" are derived from it.
+int num_cu();
+constexpr int MAX_DEVICES = 16;
 
 // Which contraction of the layer a tiled GEMM launch computes.
 //   FWD: D[b][n]  = sum_k  act[b][k] * w[n][k]      (mean; variance with 2 terms)

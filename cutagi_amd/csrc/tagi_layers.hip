@@ -298,7 +298,7 @@ __global__ __launch_bounds__(TPB) void add_shortcut_kernel(const float *__restri
 
 // Samples per chunk so that a channel-major grid has about 4 workgroups per CU.
 int bn_chunks(int fi, int B, int *b_per_chunk) {
-    int chunks = (4 * NUM_CU + fi - 1) / fi;
+    int chunks = (4 * num_cu() + fi - 1) / fi;
     if (chunks > B) chunks = B;
     if (chunks < 1) chunks = 1;
     *b_per_chunk = (B + chunks - 1) / chunks;

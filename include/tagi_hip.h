@@ -19,7 +19,10 @@
  *     positive hipError_t when the HIP runtime failed; nothing throws;
  *     tagi_hip_error_string() describes any of them;
  *   - the library owns no user buffer. It keeps one grow-only device workspace
- *     per GPU for split-reduction partial sums (see tagi_hip_workspace_reserve).
+ *     per (GPU, stream) for split-reduction partial sums (see
+ *     tagi_hip_workspace_reserve), so calls on different streams never share
+ *     scratch memory; calls issued to ONE stream from several host threads must be
+ *     serialised by the caller, as with any stream-ordered API.
  */
 #ifndef TAGI_HIP_H
 #define TAGI_HIP_H
@@ -43,15 +46,24 @@ int tagi_hip_version(void);
  * Sequential::to_device (src/sequential.cpp:32-73). */
 int tagi_hip_device_count(int *count /* host, out */);
 const char *tagi_hip_error_string(int code);
-/* Grow the current device's workspace to at least `bytes` now (synchronises the
- * device if it has to reallocate). Optional: entry points grow it on demand. */
-int tagi_hip_workspace_reserve(size_t bytes);
+/* Grow the workspace of `stream` on the current device to at least `bytes` now
+ * (synchronises the device if it has to reallocate). Optional: entry points grow it
+ * on demand. */
+int tagi_hip_workspace_reserve(size_t bytes, void *stream);
 /* Free the workspaces of all devices. */
 int tagi_hip_shutdown(void);
-/* Kernel-selection knobs for experiments and tests; value < 0 restores the
- * built-in heuristic, unknown keys are an error. Linear: "linear.tile",
+/* Compute units, peak engine clock (MHz) and name of the current device, as the
+ * runtime reports them (hipGetDeviceProperties); any pointer may be NULL. The
+ * reference's counterpart is get_cuda_device_properties (src/cuda_utils.cpp). */
+int tagi_hip_device_info(int *compute_units /* host */, int *clock_mhz /* host */,
+                         char *name /* host */, size_t name_capacity);
+/* TEST AND EXPERIMENT HOOK, not part of the drop-in surface: a caller of the
+ * reference has no reason to touch it, and every knob is process-wide (set it only
+ * while no other thread is inside the library). Kernel-selection switches used by
+ * the parity tests to force each code path and by the tuning sweeps; value < 0
+ * restores the built-in heuristic, unknown keys are an error. Linear: "linear.tile",
  * "linear.fwd.splits", "linear.dz.splits", "linear.dw.splits",
- * "linear.gemv_max_batch" (largest batch of the streaming kernels),
+ * "linear.gemv_max_batch" (largest batch of the streaming kernels, at most 16),
  * "linear.gemv.swizzle", "linear.gemv.fwd_variant", "linear.gemv.reverse",
  * "linear.gemv16" (0: 9..16 samples on the kernels for up to 8),
  * "linear.dw_side" (0: bias innovations and the state-backward fold as launches
