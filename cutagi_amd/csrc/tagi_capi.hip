@@ -290,6 +290,7 @@ int tagi_hip_tune(const char *key, int value) {
     else if (!strcmp(key, "conv2d.stencil")) g_conv2d_stencil = value;
     else if (!strcmp(key, "conv2d.phase_order")) g_conv2d_phase_order = value;
     else if (!strcmp(key, "linear.tile")) g_tune.tile = value;
+    else if (!strcmp(key, "linear.double_buffer")) g_gemm_double_buffer = value < 0 ? 1 : value;
     else if (!strcmp(key, "conv2d.dw.splits")) g_tune.conv_dw_splits = value;
     else if (!strcmp(key, "linear.gemv.swizzle")) g_tune.gemv_swz = value;
     else if (!strcmp(key, "linear.gemv.fwd_variant")) g_tune.gemv_fwd_variant = value;

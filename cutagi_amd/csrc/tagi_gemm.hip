@@ -13,6 +13,7 @@
 #include "tagi_mfma_tile.h"
 
 namespace tagi {
+extern int g_gemm_double_buffer;
 namespace {
 
 // Four elements of a row-major matrix `base` (leading dimension ld): along the
@@ -55,10 +56,12 @@ __device__ __forceinline__ float4 load4_full(const float *__restrict__ base, int
     return *reinterpret_cast<const float4 *>(q);
 }
 
-template <int MODE, bool VEC, bool FULL = false>
+template <int MODE, bool VEC, bool FULL = false, bool DB = false>
 struct LinearProblem {
     static_assert(VEC || !FULL, "complete k-tiles are a case of the 16-byte path");
+    static_assert(FULL || !DB, "the double-buffered loop is built for complete k-tiles");
     using Params = GemmParams;
+    static constexpr bool DOUBLE_BUFFER = DB;
     static constexpr bool XK = (MODE != GEMM_DW);
     static constexpr bool YK = (MODE == GEMM_FWD);
     static constexpr int NX = 2;
@@ -174,6 +177,8 @@ template <int MODE>
 hipError_t launch_mode(int tile, bool vec, const GemmParams &p, hipStream_t stream) {
     const bool full = vec && p.R % KT == 0 && (p.splits == 1 || p.r_per_split % KT == 0) &&
                       p.M >= 4 && p.N >= 4;
+    if (full && g_gemm_double_buffer != 0)
+        return launch_tiles<LinearProblem<MODE, true, true, true>>(tile, p, stream);
     if (full) return launch_tiles<LinearProblem<MODE, true, true>>(tile, p, stream);
     if (vec) return launch_tiles<LinearProblem<MODE, true>>(tile, p, stream);
     return launch_tiles<LinearProblem<MODE, false>>(tile, p, stream);
@@ -268,15 +273,17 @@ __global__ __launch_bounds__(WM *WN * 64) void linear_dw_side_kernel(GemmParams 
     tile_workgroup<P, BM, BN, WM, WN>(p, id - w.side_wgs, 0, (int)gridDim.x - w.side_wgs, 1);
 }
 
-template <bool FULL>
+template <bool FULL, bool DB = false>
 hipError_t launch_dw_side(const GemmParams &p, const LinearSideWork &w, hipStream_t stream) {
-    using P = LinearProblem<GEMM_DW, true, FULL>;
+    using P = LinearProblem<GEMM_DW, true, FULL, DB>;
     const int tiles = ((p.M + 63) / 64) * ((p.N + 127) / 128);
     hipLaunchKernelGGL((linear_dw_side_kernel<P, 64, 128, 2, 4>), dim3(tiles + w.side_wgs),
                        dim3(512), 0, stream, p, w);
     return hipGetLastError();
 }
 }  // namespace
+
+int g_gemm_double_buffer = 1;
 
 int gemm_tile_rows(int tile) { return tile_rows(tile); }
 int gemm_tile_cols(int tile) { return tile_cols(tile); }
@@ -310,6 +317,7 @@ hipError_t launch_gemm_dw_side(const GemmParams &p, LinearSideWork w, hipStream_
     w.side_wgs = (w.bias_wgs + fold_wgs + 7) / 8 * 8;
     if (w.ws0 == nullptr) w.fold_total = 0;  // the padding workgroups find nothing to fold
     const bool full = p.R % KT == 0 && p.M >= 4 && p.N >= 4;
+    if (full && g_gemm_double_buffer != 0) return launch_dw_side<true, true>(p, w, stream);
     return full ? launch_dw_side<true>(p, w, stream) : launch_dw_side<false>(p, w, stream);
 }
 

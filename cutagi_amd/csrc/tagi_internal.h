@@ -41,6 +41,9 @@ int gemm_tile_rows(int tile);
 int gemm_tile_cols(int tile);
 int gemm_k_tile();
 
+// 0 keeps the Linear tile kernels on the single-stage k-loop (tuning knob).
+extern int g_gemm_double_buffer;
+
 // Launches the tiled MFMA kernel. `vec` selects 16-byte global loads (the caller
 // guarantees the alignment rules); partial sums go to ws0/ws1 when splits > 1
 // and the caller then runs reduce_splits.

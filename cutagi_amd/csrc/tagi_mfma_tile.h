@@ -77,10 +77,10 @@ constexpr int KT = 32;  // reduction elements per LDS stage
 
 struct TileNoCtx {};
 
-template <bool KC, int ROWS>
+template <bool KC, int ROWS, int KTILE = KT>
 struct TileGeom {
-    static constexpr int stride = KC ? KT + 4 : ROWS + 4;
-    static constexpr int floats = KC ? ROWS * stride : KT * stride;
+    static constexpr int stride = KC ? KTILE + 4 : ROWS + 4;
+    static constexpr int floats = KC ? ROWS * stride : KTILE * stride;
 };
 
 __device__ __forceinline__ float comp4(const float4 &v, int t) {
@@ -94,20 +94,20 @@ __device__ __forceinline__ float4 add_sq4(const float4 &v, const float4 &m) {
 }
 
 // Position of the f-th float4 of a staged tile: (row, k) of its first element.
-template <bool KC, int ROWS>
+template <bool KC, int ROWS, int KTILE = KT>
 __device__ __forceinline__ void tile_pos(int f, int &row, int &k) {
     if (KC) {
-        row = f / (KT / 4);
-        k = (f % (KT / 4)) * 4;
+        row = f / (KTILE / 4);
+        k = (f % (KTILE / 4)) * 4;
     } else {
         k = f / (ROWS / 4);
         row = (f % (ROWS / 4)) * 4;
     }
 }
 
-template <bool KC, int ROWS>
+template <bool KC, int ROWS, int KTILE = KT>
 __device__ __forceinline__ float4 read_frag(const float *lds, int row, int kk, int lane) {
-    constexpr int S = TileGeom<KC, ROWS>::stride;
+    constexpr int S = TileGeom<KC, ROWS, KTILE>::stride;
     const int k = kk + 4 * (lane >> 5);
     if (KC) {
         return *reinterpret_cast<const float4 *>(lds + (row + (lane & 31)) * S + k);
@@ -340,6 +340,178 @@ __device__ __forceinline__ void mfma_tile_body(const typename P::Params &p, type
 }
 
 
+// Does the problem ask for the double-buffered loop below? (A problem opts in with
+// `static constexpr bool DOUBLE_BUFFER = true`; it must not depend on the slot index
+// of its loaders, because slots are dealt to the threads differently there.)
+template <class P, class = void>
+struct tile_double_buffer { static constexpr bool value = false; };
+template <class P>
+struct tile_double_buffer<P, decltype((void)P::DOUBLE_BUFFER)> {
+    static constexpr bool value = P::DOUBLE_BUFFER;
+};
+
+constexpr int KT_DB = 16;  // reduction elements per stage of the double-buffered loop
+
+// One multiply step on the staged tiles of one LDS stage (KTILE reduction elements).
+template <class P, int BM, int BN, int WM, int WN, int KTILE>
+__device__ __forceinline__ void tile_multiply(const float (*lx)[TileGeom<P::XK, BM, KTILE>::floats],
+                                              const float (*ly)[TileGeom<P::YK, BN, KTILE>::floats],
+                                              floatx16 (&acc0)[BM / WM / 32][BN / WN / 32],
+                                              floatx16 (&acc1)[BM / WM / 32][BN / WN / 32],
+                                              int wrow, int wcol, int lane) {
+    constexpr bool XK = P::XK, YK = P::YK;
+    constexpr int NX = P::NX, NY = P::NY, FL = P::FLAVOR;
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+#pragma unroll
+    for (int kk = 0; kk < KTILE; kk += 8) {
+        float4 A0[TM], A1[TM], A2[TM], B0[TN], B1[TN], B2[TN];
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            const float4 x0 = read_frag<XK, BM, KTILE>(lx[0], wrow + i * 32, kk, lane);
+            float4 x1 = x0;
+            if (NX == 2) x1 = read_frag<XK, BM, KTILE>(lx[NX - 1], wrow + i * 32, kk, lane);
+            A0[i] = x0;
+            if (FL == FLAVOR_FWD_ACT_ROWS) {
+                A1[i] = add_sq4(x1, x0);
+                A2[i] = x1;
+            } else if (FL == FLAVOR_FWD_W_ROWS) {
+                A1[i] = x1;
+                A2[i] = sq4(x0);
+            } else if (FL == FLAVOR_DELTA_ROWS) {
+                A1[i] = x1;
+            } else {
+                A1[i] = sq4(x0);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const float4 y0 = read_frag<YK, BN, KTILE>(ly[0], wcol + j * 32, kk, lane);
+            float4 y1 = y0;
+            if (NY == 2) y1 = read_frag<YK, BN, KTILE>(ly[NY - 1], wcol + j * 32, kk, lane);
+            B0[j] = y0;
+            if (FL == FLAVOR_FWD_ACT_ROWS) {
+                B1[j] = y1;
+                B2[j] = sq4(y0);
+            } else if (FL == FLAVOR_FWD_W_ROWS) {
+                B1[j] = add_sq4(y1, y0);
+                B2[j] = y1;
+            } else if (FL == FLAVOR_DELTA_ROWS) {
+                B1[j] = sq4(y0);
+            } else {
+                B1[j] = y1;
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    acc0[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                        comp4(A0[i], t), comp4(B0[j], t), acc0[i][j], 0, 0, 0);
+                    acc1[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                        comp4(A1[i], t), comp4(B1[j], t), acc1[i][j], 0, 0, 0);
+                    if (FL == FLAVOR_FWD_ACT_ROWS || FL == FLAVOR_FWD_W_ROWS)
+                        acc1[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                            comp4(A2[i], t), comp4(B2[j], t), acc1[i][j], 0, 0, 0);
+                }
+    }
+}
+
+// The k-loop with two LDS stages of KT_DB reduction elements each (the same LDS
+// footprint as one stage of KT): while a stage is multiplied, the registers that hold
+// the next k-tile are written to the other stage, so a k-tile costs one barrier and no
+// wave waits between its multiplies and its LDS writes for the others to finish
+// reading. The float4 slots of a stage are dealt to the threads across the arrays of a
+// side (slot g of NX*BM*KT_DB/4: array g / (BM*KT_DB/4)).
+template <class P, int BM, int BN, int WM, int WN>
+__device__ __forceinline__ void mfma_tile_body_db(
+    const typename P::Params &p, typename P::Ctx &ctx,
+    float (*lds_x)[P::NX][TileGeom<P::XK, BM, KT_DB>::floats],
+    float (*lds_y)[P::NY][TileGeom<P::YK, BN, KT_DB>::floats], int m0, int n0, int split,
+    int r_begin, int r_end) {
+    constexpr bool XK = P::XK, YK = P::YK;
+    constexpr int NX = P::NX, NY = P::NY;
+    constexpr int NT = WM * WN * 64;
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int XS = TileGeom<XK, BM, KT_DB>::stride, YS = TileGeom<YK, BN, KT_DB>::stride;
+    constexpr int FX = BM * KT_DB / 4, FY = BN * KT_DB / 4;  // float4 per array and stage
+    static_assert((NX * FX) % NT == 0 && (NY * FY) % NT == 0, "slots must divide evenly");
+    constexpr int SX = NX * FX / NT, SY = NY * FY / NT;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wrow = (wave / WN) * (TM * 32), wcol = (wave % WN) * (TN * 32);
+
+    floatx16 acc0[TM][TN], acc1[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                acc0[i][j][v] = 0.f;
+                acc1[i][j][v] = 0.f;
+            }
+
+    float4 rx[SX], ry[SY];
+    auto fetch = [&](int r0) {
+#pragma unroll
+        for (int s = 0; s < SX; s++) {
+            const int g = tid + s * NT;
+            int row, k;
+            tile_pos<XK, BM, KT_DB>(g % FX, row, k);
+            rx[s] = P::load_x(p, ctx, 0, g / FX, s, m0, row, r0 + k, r_end);
+        }
+#pragma unroll
+        for (int s = 0; s < SY; s++) {
+            const int g = tid + s * NT;
+            int row, k;
+            tile_pos<YK, BN, KT_DB>(g % FY, row, k);
+            ry[s] = P::load_y(p, ctx, 0, g / FY, s, n0, row, r0 + k, r_end);
+        }
+    };
+    auto commit = [&](int stage) {
+#pragma unroll
+        for (int s = 0; s < SX; s++) {
+            const int g = tid + s * NT;
+            int row, k;
+            tile_pos<XK, BM, KT_DB>(g % FX, row, k);
+            *reinterpret_cast<float4 *>(&lds_x[stage][g / FX][XK ? row * XS + k : k * XS + row]) =
+                rx[s];
+        }
+#pragma unroll
+        for (int s = 0; s < SY; s++) {
+            const int g = tid + s * NT;
+            int row, k;
+            tile_pos<YK, BN, KT_DB>(g % FY, row, k);
+            *reinterpret_cast<float4 *>(&lds_y[stage][g / FY][YK ? row * YS + k : k * YS + row]) =
+                ry[s];
+        }
+    };
+
+    if (r_begin < r_end) {
+        fetch(r_begin);
+        commit(0);
+    }
+    __syncthreads();
+    // two k-tiles per trip, so that the stage is a constant in every LDS address
+    for (int r0 = r_begin; r0 < r_end; r0 += 2 * KT_DB) {
+#pragma unroll
+        for (int stage = 0; stage < 2; stage++) {
+            const int r = r0 + stage * KT_DB;
+            if (r < r_end) {
+                const bool more = r + KT_DB < r_end;
+                if (more) fetch(r + KT_DB);
+                tile_multiply<P, BM, BN, WM, WN, KT_DB>(lds_x[stage], lds_y[stage], acc0, acc1,
+                                                        wrow, wcol, lane);
+                if (more) commit(stage ^ 1);
+                __syncthreads();
+            }
+        }
+    }
+    tile_epilogue<P, BM, BN, WM, WN>(p, acc0, acc1, m0, n0, split);
+}
+
+
 // What the workgroup (bx, by) of a gx x gy grid of (tiles, reduction slices) does.
 template <class P, int BM, int BN, int WM, int WN>
 __device__ __forceinline__ void tile_workgroup(const typename P::Params &p, int bx, int by, int gx,
@@ -351,8 +523,6 @@ __device__ __forceinline__ void tile_workgroup(const typename P::Params &p, int 
     constexpr int LX = BM * KT / 4 / NT, LY = BN * KT / 4 / NT;
     static_assert(LX >= 1 && LY >= 1, "tile too small for the thread count");
 
-    __shared__ __attribute__((aligned(16))) float lds_x[NX][XF];
-    __shared__ __attribute__((aligned(16))) float lds_y[NY][YF];
     extern __shared__ __attribute__((aligned(16))) int lds_extra[];
 
     const int tiles_n = (p.N + BN - 1) / BN;
@@ -376,6 +546,14 @@ __device__ __forceinline__ void tile_workgroup(const typename P::Params &p, int 
     if (P::PROLOGUE_WRITES_LDS) __syncthreads();
     int r_lo = r_begin, r_hi = r_end;
     P::adjust_range(p, ctx, r_lo, r_hi);
+    if constexpr (tile_double_buffer<P>::value) {
+        __shared__ __attribute__((aligned(16))) float
+            dbx[2][NX][TileGeom<XK, BM, KT_DB>::floats], dby[2][NY][TileGeom<YK, BN, KT_DB>::floats];
+        mfma_tile_body_db<P, BM, BN, WM, WN>(p, ctx, dbx, dby, m0, n0, split, r_lo, r_hi);
+        return;
+    }
+    __shared__ __attribute__((aligned(16))) float lds_x[NX][XF];
+    __shared__ __attribute__((aligned(16))) float lds_y[NY][YF];
     if constexpr (P::VARIANTS > 1) {
         if (P::variant(ctx)) {
             mfma_tile_body<P, BM, BN, WM, WN, 1>(p, ctx, lds_x, lds_y, m0, n0, split, r_lo, r_hi);
@@ -418,7 +596,9 @@ hipError_t launch_reduce_store(const typename P::Params &p, hipStream_t stream) 
 
 // Launch over a (tiles, splits) grid for one of the instantiated tile shapes.
 // (A 64x128 tile held by four waves of 32 x 64 instead of eight of 32 x 32 needs
-// 250 VGPRs and measured slower on every shape.)
+// 250 VGPRs and measured slower on every shape; so did a 128x128 tile held by four
+// waves of 64 x 64 with the double-buffered loop, which halves the LDS reads and
+// operand arithmetic per MFMA: 4096^2 at batch 1024, weight backward 528 -> 537 us.)
 enum TileShape { TILE_128x128 = 0, TILE_64x128 = 1, TILE_32x128 = 2, TILE_64x64 = 3, TILE_COUNT = 4 };
 
 inline int tile_rows(int t) { return t == TILE_128x128 ? 128 : t == TILE_32x128 ? 32 : 64; }
