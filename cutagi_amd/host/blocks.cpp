@@ -42,6 +42,7 @@ void MixtureReLUHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &o
     if (n > out->size) LOG(LogLevel::ERROR, "Output state buffer too small for MixtureReLU");
     TAGI_OK_OR_THROW(tagi_mixture_relu_fwd(in->d_mu_a, in->d_var_a, n, out->d_mu_a, out->d_jcb,
                                            out->d_var_a, nullptr));
+    out->jcb_ones = false;
     this->input_size = input_states.actual_size;
     this->output_size = input_states.actual_size;
     output_states.block_size = input_states.block_size;
@@ -229,6 +230,7 @@ void BatchNorm2dHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &o
     TAGI_OK_OR_THROW(tagi_batchnorm2d_fwd(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a, in->d_var_a,
                                           mu_target, var_target, bias ? 1 : 0, epsilon, wihi, fi,
                                           batch_size, out->d_mu_a, out->d_var_a, nullptr));
+    out->jcb_ones = true;
     if (this->training) this->store_states_for_training_hip(*in, *out);
 }
 
@@ -246,7 +248,7 @@ void BatchNorm2dHip::backward(BaseDeltaStates &input_delta_states,
     if (state_udapte && (size_t)wihi * fi * batch_size > dout->size)
         LOG(LogLevel::ERROR, "Delta state buffer too small for " + this->get_layer_info());
     TAGI_OK_OR_THROW(tagi_batchnorm2d_bwd(
-        d_mu_w, d_var_w, d_var_b, bwd->d_mu_a, bwd->d_jcb, d_mu_norm_batch, d_var_norm_batch,
+        d_mu_w, d_var_w, d_var_b, bwd->d_mu_a, bwd->jcb_ptr(), d_mu_norm_batch, d_var_norm_batch,
         din->d_delta_mu, din->d_delta_var, epsilon, wihi, fi, batch_size, bias ? 1 : 0,
         state_udapte ? 1 : 0, param_update ? 1 : 0, dout->d_delta_mu, dout->d_delta_var,
         d_delta_mu_w, d_delta_var_w, d_delta_mu_b, d_delta_var_b, nullptr));
@@ -370,6 +372,7 @@ void AvgPool2dHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &out
     TAGI_OK_OR_THROW(tagi_avgpool2d_fwd(in->d_mu_a, in->d_var_a, d_pool_idx, woho, wihi,
                                         (int)kernel_size, woho * (int)out_channels * batch_size,
                                         out->d_mu_a, out->d_var_a, nullptr));
+    out->jcb_ones = true;
     if (this->training) this->store_states_for_training_hip(*in, *out);
 }
 
@@ -386,7 +389,7 @@ void AvgPool2dHip::backward(BaseDeltaStates &input_delta_states,
     const int n_in = wihi * (int)in_channels * batch_size;
     if ((size_t)n_in > dout->size)
         LOG(LogLevel::ERROR, "Delta state buffer too small for " + this->get_layer_info());
-    TAGI_OK_OR_THROW(tagi_avgpool2d_bwd_dz(bwd->d_jcb, din->d_delta_mu, din->d_delta_var,
+    TAGI_OK_OR_THROW(tagi_avgpool2d_bwd_dz(bwd->jcb_ptr(), din->d_delta_mu, din->d_delta_var,
                                            d_z_ud_idx, woho, wihi, (int)kernel_size,
                                            (int)col_z_ud, (int)out_width, n_in, overlap ? 1 : 0,
                                            dout->d_delta_mu, dout->d_delta_var, nullptr));
@@ -687,6 +690,10 @@ void ResNetBlock::init_buffers() {
     input_delta_z = std::make_shared<DeltaStateHip>(size, batch_size_, device_idx);
     if (shortcut) {
         shortcut_output_z = std::make_shared<HiddenStateHip>(size, batch_size_, device_idx);
+        // the shortcut's layers ping-pong between these two; nothing else reads them
+        // once the shortcut has run, so its layers may keep their arrays
+        as<HiddenStateHip>(*input_z)->transient = true;
+        as<HiddenStateHip>(*shortcut_output_z)->transient = true;
         if (training)
             shortcut_output_delta_z = std::make_shared<DeltaStateHip>(size, batch_size_, device_idx);
     }
@@ -721,11 +728,7 @@ void ResNetBlock::forward(BaseHiddenStates &input_states, BaseHiddenStates &outp
     TAGI_OK_OR_THROW(tagi_add_shortcut(sc->d_mu_a, sc->d_var_a, num_states, out->d_mu_a,
                                        out->d_var_a, nullptr));
     set_output_dims(output_states, *this, batch_size);
-    if (training) {
-        // the block's output Jacobian is one (store_states with nothing to store)
-        TAGI_OK_OR_THROW(tagi_store_states(nullptr, nullptr, 0, nullptr, nullptr, out->d_jcb,
-                                           num_states, nullptr));
-    }
+    out->jcb_ones = true;  // the block's output Jacobian is one: marked, not written
 }
 
 // reference: ResNetBlockCuda::backward, src/resnet_block_cuda.cu:301-347
@@ -749,7 +752,7 @@ void ResNetBlock::backward(BaseDeltaStates &input_delta_states,
         if (!state_update) return;
         auto *sc = as<DeltaStateHip>(*input_delta_z);
         auto *kept = as<HiddenStateHip>(*input_z);
-        TAGI_OK_OR_THROW(tagi_add_shortcut_delta(sc->d_delta_mu, sc->d_delta_var, kept->d_jcb,
+        TAGI_OK_OR_THROW(tagi_add_shortcut_delta(sc->d_delta_mu, sc->d_delta_var, kept->jcb_ptr(),
                                                  num_states, dout->d_delta_mu, dout->d_delta_var,
                                                  nullptr));
     }

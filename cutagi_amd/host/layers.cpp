@@ -316,13 +316,36 @@ std::vector<ParameterTuple> BaseLayerHip::parameters() {
     return BaseLayer::parameters();
 }
 
+// What the backward pass needs from the input (its mean and its Jacobian), and the
+// output's Jacobian of one; reference: store_states_for_training_cuda,
+// src/base_layer_cuda.cu:464-486 (two device copies and a fill kernel per layer).
+// Here the output is only marked (HiddenStateHip::jcb_ones); an input Jacobian that is
+// marked is not copied either; and where the input is one of its owner's ping-pong
+// buffers, whose contents are dead once this layer has read them, the layer keeps the
+// input's arrays and leaves its own arrays of the previous step in their place: no
+// copy and no launch at all. Called after the layer's own kernels were queued (they
+// hold the old addresses).
 void BaseLayerHip::store_states_for_training_hip(HiddenStateHip &in, HiddenStateHip &out) {
     auto *bwd = dynamic_cast<BackwardStateHip *>(this->bwd_states.get());
     const size_t n_in = in.actual_size * in.block_size;
-    const size_t n_out = out.actual_size * out.block_size;
+    bwd->device_idx = in.device_idx;
+    out.jcb_ones = true;
+    if (in.transient) {
+        bwd->resize_exact(in.size);
+        std::swap(bwd->d_mu_a, in.d_mu_a);
+        bwd->jcb_ones = in.jcb_ones;
+        if (!in.jcb_ones) std::swap(bwd->d_jcb, in.d_jcb);
+        return;
+    }
     if (bwd->size < n_in) bwd->set_size(n_in);
-    TAGI_OK_OR_THROW(tagi_store_states(in.d_mu_a, in.d_jcb, n_in, bwd->d_mu_a, bwd->d_jcb, out.d_jcb,
-                                       n_out, nullptr));
+    bwd->jcb_ones = in.jcb_ones;
+    if (in.jcb_ones) {
+        HIP_OK(hipMemcpyAsync(bwd->d_mu_a, in.d_mu_a, n_in * sizeof(float),
+                              hipMemcpyDeviceToDevice, nullptr));
+        return;
+    }
+    TAGI_OK_OR_THROW(tagi_store_states(in.d_mu_a, in.d_jcb, n_in, bwd->d_mu_a, bwd->d_jcb, nullptr,
+                                       0, nullptr));
 }
 
 // ---- Linear -----------------------------------------------------------------------------
@@ -402,6 +425,7 @@ void LinearHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &output
     output_states.depth = this->out_channels;
     output_states.block_size = batch_size;
     output_states.actual_size = this->output_size;
+    out->jcb_ones = true;
     if (this->training) this->store_states_for_training_hip(*in, *out);
 }
 
@@ -414,7 +438,7 @@ void LinearHip::backward(BaseDeltaStates &input_delta_states, BaseDeltaStates &o
     const int batch_size = (int)input_delta_states.block_size;
     if (state_udapte && input_size * batch_size > dout->size)
         LOG(LogLevel::ERROR, "Delta state buffer too small for " + this->get_layer_info());
-    TAGI_OK_OR_THROW(tagi_linear_bwd(d_mu_w, d_var_w, d_var_b, bwd->d_mu_a, bwd->d_jcb,
+    TAGI_OK_OR_THROW(tagi_linear_bwd(d_mu_w, d_var_w, d_var_b, bwd->d_mu_a, bwd->jcb_ptr(),
                                      din->d_delta_mu, din->d_delta_var, (int)input_size,
                                      (int)output_size, batch_size, bias ? 1 : 0, state_udapte ? 1 : 0,
                                      param_update ? 1 : 0, dout->d_delta_mu, dout->d_delta_var,
@@ -597,6 +621,7 @@ void Conv2dHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &output
                                      d_idx_mwa_2, woho, (int)out_channels, wihi, (int)in_channels,
                                      (int)kernel_size, batch_size, bias ? 1 : 0, out->d_mu_a,
                                      out->d_var_a, nullptr));
+    out->jcb_ones = true;
     if (training) this->store_states_for_training_hip(*in, *out);
 }
 
@@ -618,7 +643,7 @@ void Conv2dHip::backward(BaseDeltaStates &input_delta_states, BaseDeltaStates &o
     if (state_udapte) {
         if (input_size * batch_size > dout->size)
             LOG(LogLevel::ERROR, "Delta state buffer too small for " + this->get_layer_info());
-        TAGI_OK_OR_THROW(tagi_conv2d_bwd_dz(d_mu_w, bwd->d_jcb, din->d_delta_mu, din->d_delta_var,
+        TAGI_OK_OR_THROW(tagi_conv2d_bwd_dz(d_mu_w, bwd->jcb_ptr(), din->d_delta_mu, din->d_delta_var,
                                             d_idx_cov_zwa_1, d_idx_var_z_ud, woho, (int)out_channels,
                                             wihi, (int)in_channels, (int)kernel_size, row_zw,
                                             batch_size, dout->d_delta_mu, dout->d_delta_var,
@@ -649,6 +674,7 @@ void ReLUHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &output_s
     if (n > out->size) LOG(LogLevel::ERROR, "Output state buffer too small for ReLU");
     TAGI_OK_OR_THROW(tagi_relu_fwd(in->d_mu_a, in->d_var_a, n, out->d_mu_a, out->d_jcb, out->d_var_a,
                                    nullptr));
+    out->jcb_ones = false;
     this->input_size = input_states.actual_size;
     this->output_size = input_states.actual_size;
     output_states.block_size = input_states.block_size;

@@ -148,7 +148,7 @@ void OutputUpdater::update_raw(BaseHiddenStates &output_states, const float *mu_
     o->actual_size = output_states.block_size ? n / output_states.block_size : 0;
     o->upload(mu_obs, var_obs, n, nullptr, 0);
     delta->reset_zeros();
-    TAGI_OK_OR_THROW(tagi_out_update_dense(out->d_mu_a, out->d_var_a, out->d_jcb, o->d_mu_obs,
+    TAGI_OK_OR_THROW(tagi_out_update_dense(out->d_mu_a, out->d_var_a, out->jcb_ptr(), o->d_mu_obs,
                                            o->d_var_obs, (int)o->size, delta->d_delta_mu,
                                            delta->d_delta_var, nullptr));
 }
@@ -188,7 +188,7 @@ void OutputUpdater::update_using_indices_raw(BaseHiddenStates &output_states,
     o->upload(mu_obs, var_obs, n, selected_idx, n);
     const int n_enc = (int)(o->idx_size / output_states.block_size);
     delta->reset_zeros();
-    TAGI_OK_OR_THROW(tagi_out_update_indexed(out->d_mu_a, out->d_var_a, out->d_jcb, o->d_mu_obs,
+    TAGI_OK_OR_THROW(tagi_out_update_indexed(out->d_mu_a, out->d_var_a, out->jcb_ptr(), o->d_mu_obs,
                                              o->d_var_obs, o->d_selected_idx, n_obs, n_enc,
                                              (int)o->size, delta->d_delta_mu, delta->d_delta_var,
                                              nullptr));
@@ -213,7 +213,7 @@ void OutputUpdater::update_heteros_raw(BaseHiddenStates &output_states, const fl
     o->actual_size = output_states.block_size ? n / output_states.block_size : 0;
     o->upload(mu_obs, nullptr, n, nullptr, 0);
     delta->reset_zeros();
-    TAGI_OK_OR_THROW(tagi_out_update_heteros(out->d_mu_a, out->d_var_a, out->d_jcb, o->d_mu_obs,
+    TAGI_OK_OR_THROW(tagi_out_update_heteros(out->d_mu_a, out->d_var_a, out->jcb_ptr(), o->d_mu_obs,
                                              (int)o->size, delta->d_delta_mu, delta->d_delta_var,
                                              nullptr));
 }
@@ -306,6 +306,9 @@ void Sequential::require_device(const char *what) const {
 void Sequential::init_output_state_buffer() {
     output_z_buffer = std::make_shared<HiddenStateHip>(z_buffer_size, z_buffer_block_size, device_idx);
     input_z_buffer = std::make_shared<HiddenStateHip>(z_buffer_size, z_buffer_block_size, device_idx);
+    // ping-pong buffers: what a layer has read is dead, so it may keep the arrays
+    for (auto *b : {output_z_buffer.get(), input_z_buffer.get()})
+        dynamic_cast<HiddenStateHip *>(b)->transient = true;
     temp_states = std::make_shared<TempStateHip>(0, z_buffer_block_size, device_idx);
 }
 

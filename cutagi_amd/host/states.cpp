@@ -82,6 +82,23 @@ StagingRing &staging_ring(int device_idx) {
 }
 }  // namespace
 
+const float *device_ones(size_t n, int device_idx) {
+    static float *ones[16] = {};
+    static size_t cap[16] = {};
+    if (device_idx < 0 || device_idx >= 16) LOG(LogLevel::ERROR, "Invalid device index");
+    if (n > cap[device_idx]) {
+        HIP_OK(hipSetDevice(device_idx));
+        HIP_OK(hipDeviceSynchronize());  // kernels in flight may still read the old array
+        dev_free(ones[device_idx]);
+        ones[device_idx] = dev_alloc(n, device_idx);
+        cap[device_idx] = n;
+        if (tagi_store_states(nullptr, nullptr, 0, nullptr, nullptr, ones[device_idx], n,
+                              nullptr) != TAGI_OK)
+            LOG(LogLevel::ERROR, "Cannot fill the array of ones");
+    }
+    return ones[device_idx];
+}
+
 // ---- BaseHiddenStates (reference: src/data_struct.cpp:6-95) ---------------------
 BaseHiddenStates::BaseHiddenStates(size_t n, size_t m, int device_idx)
     : mu_a(n, 0.0f), var_a(n, 0.0f), jcb(n, 1.0f), size(n), block_size(m), device_idx(device_idx) {
@@ -229,13 +246,17 @@ void HiddenStateHip::chunks_to_device(size_t n) {
     h2d(d_mu_a, mu_a.data(), n);
     h2d(d_var_a, var_a.data(), n);
     h2d(d_jcb, jcb.data(), n);
+    jcb_ones = false;
 }
 void HiddenStateHip::to_host() { this->to_host(this->size); }
 void HiddenStateHip::to_host(size_t n) {
     n = std::min(n, this->size);
     d2h(mu_a.data(), d_mu_a, n);
     d2h(var_a.data(), d_var_a, n);
-    d2h(jcb.data(), d_jcb, n);
+    if (jcb_ones)
+        std::fill(jcb.begin(), jcb.begin() + n, 1.0f);
+    else
+        d2h(jcb.data(), d_jcb, n);
 }
 void HiddenStateHip::set_input_x(const std::vector<float> &mu_x, const std::vector<float> &var_x,
                                  size_t block_size) {
@@ -263,8 +284,7 @@ void HiddenStateHip::set_input_raw(const float *mu_x, const float *var_x, size_t
         ring.upload(d_var_a, var_x, n * sizeof(float));
     else
         HIP_OK(hipMemsetAsync(d_var_a, 0, n * sizeof(float), nullptr));
-    if (tagi_store_states(nullptr, nullptr, 0, nullptr, nullptr, d_jcb, n, nullptr) != TAGI_OK)
-        LOG(LogLevel::ERROR, "Cannot initialise the input Jacobian");
+    jcb_ones = true;  // the input's Jacobian is one: marked, not written
 }
 void HiddenStateHip::set_size(size_t new_size, size_t new_block_size) {
     if (new_size > this->size) {
@@ -283,6 +303,8 @@ void HiddenStateHip::swap(BaseHiddenStates &other) {
     std::swap(d_mu_a, o->d_mu_a);
     std::swap(d_var_a, o->d_var_a);
     std::swap(d_jcb, o->d_jcb);
+    std::swap(jcb_ones, o->jcb_ones);
+    std::swap(transient, o->transient);
 }
 void HiddenStateHip::copy_from(const BaseHiddenStates &source, int num_data) {
     auto *s = dynamic_cast<const HiddenStateHip *>(&source);
@@ -290,7 +312,8 @@ void HiddenStateHip::copy_from(const BaseHiddenStates &source, int num_data) {
     if (num_data == -1) num_data = (int)std::min(source.size, this->size);
     d2d(d_mu_a, s->d_mu_a, num_data);
     d2d(d_var_a, s->d_var_a, num_data);
-    d2d(d_jcb, s->d_jcb, num_data);
+    if (!s->jcb_ones) d2d(d_jcb, s->d_jcb, num_data);
+    this->jcb_ones = s->jcb_ones;
     this->block_size = source.block_size;
     this->actual_size = source.actual_size;
     this->width = source.width;
@@ -392,7 +415,16 @@ void BackwardStateHip::to_host() {
     mu_a.resize(size);
     jcb.resize(size);
     d2h(mu_a.data(), d_mu_a, size);
-    d2h(jcb.data(), d_jcb, size);
+    if (jcb_ones)
+        std::fill(jcb.begin(), jcb.end(), 1.0f);
+    else
+        d2h(jcb.data(), d_jcb, size);
+}
+void BackwardStateHip::resize_exact(size_t new_size) {
+    if (new_size == this->size && d_mu_a != nullptr) return;
+    this->size = new_size;
+    HIP_OK(hipDeviceSynchronize());
+    this->allocate_memory();
 }
 void BackwardStateHip::set_size(size_t new_size) {
     if (new_size > this->size) {

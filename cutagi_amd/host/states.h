@@ -95,9 +95,23 @@ class BaseObservation {
 
 // ---- device side ---------------------------------------------------------------
 
+// A device array of ones, at least n long, on the given device (grow-only, shared):
+// what a consumer reads for a Jacobian that is known to be one everywhere.
+const float *device_ones(size_t n, int device_idx);
+
 class HiddenStateHip : public BaseHiddenStates {
    public:
     float *d_mu_a = nullptr, *d_var_a = nullptr, *d_jcb = nullptr;
+    // The Jacobian is one everywhere and d_jcb was NOT written: Linear, Conv2d,
+    // BatchNorm2d, AvgPool2d and the residual add produce such outputs, and marking
+    // them costs nothing where the reference runs a fill kernel per layer
+    // (src/base_layer_cuda.cu:464-486). Readers go through jcb_ptr().
+    bool jcb_ones = false;
+    // Set by the owner of a ping-pong buffer (Sequential, ResNetBlock): after a layer
+    // has read it, its contents are dead, so the layer may keep its arrays for the
+    // backward pass and leave its own old ones in their place instead of copying.
+    bool transient = false;
+    const float *jcb_ptr() const { return jcb_ones ? device_ones(size, device_idx) : d_jcb; }
 
     HiddenStateHip(size_t n, size_t m, int device_idx = 0);
     HiddenStateHip() = default;
@@ -154,6 +168,10 @@ class TempStateHip : public BaseTempStates {
 class BackwardStateHip : public BaseBackwardStates {
    public:
     float *d_mu_a = nullptr, *d_jcb = nullptr;
+    bool jcb_ones = false;  // as HiddenStateHip::jcb_ones
+    const float *jcb_ptr() const { return jcb_ones ? device_ones(size, device_idx) : d_jcb; }
+    // exactly new_size floats per array (reallocates when the size differs)
+    void resize_exact(size_t new_size);
 
     BackwardStateHip() = default;
     ~BackwardStateHip() override;
