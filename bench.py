@@ -8,8 +8,10 @@ Linear layer on synthetic inputs that are resident in HBM before the timed
 region starts. The default workload is the dense one the headline metric is
 quoted on (4096 -> 4096, batch 256, fp32); `--workload skinny` times the
 HBM-bound one (8192 -> 8192, batch 8) and reports GB/s. The default run also
-times the skinny workload, the Conv2d workload, one training step of the CIFAR
-ResNet-18 and the CPU baseline, and attaches them to the same JSON line.
+times the skinny workload (and its 12- and 16-sample variants), the Conv2d
+workload, one training step of the MLP configuration and of the CIFAR ResNet-18,
+and the CPU baseline, and attaches them to the same JSON line, together with what
+the runtime reports for the device and the wall time of the GPU legs.
 
 Prints ONE JSON line. `roofline` is computed for the dominant kernel from its
 algorithmic work and its average duration measured with HIP events on the
@@ -25,27 +27,33 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak
-HBM_PEAK_GBS = 8000.0          # MI355X HBM3E peak
+FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak (published)
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E peak (published)
+FP32_MFMA_FLOP_PER_CLK_PER_CU = 256  # v_mfma_f32_32x32x2_f32: 4096 flop in 64 cycles on each of 4 SIMDs
 
 WORKLOADS = {
     # name: (K, N, B, bound)
     "gemm": (4096, 4096, 256, "mfma"),
     "skinny": (8192, 8192, 8, "hbm"),
+    # the 16-wide streaming kernels (9..16 samples), reported in `extra` only
+    "skinny12": (8192, 8192, 12, "hbm"),
+    "skinny16": (8192, 8192, 16, "hbm"),
 }
-# HBM bytes per launch of the dominant kernel of each workload: FETCH_SIZE and
-# WRITE_SIZE of two `rocprofv3 --pmc` runs of this script, each scaled by what the
-# same counter reads for a plain 1 GiB copy (x2.000 and x1.000; `--calibrate` adds
-# that copy to a run). Counters cannot be read from inside this process, so the
-# figures of the last profiled build are carried here; the summaries are under
-# profiles/.
+# HBM bytes per launch of the kernel that dominates each phase of a step, keyed by
+# the kernel that runs there: FETCH_SIZE and WRITE_SIZE of two `rocprofv3 --pmc`
+# runs of this script, each scaled by what the same counter reads for a plain 1 GiB
+# copy (`--calibrate` adds that copy to a run). Counters cannot be read from inside
+# this process, so the figures of the last profiled build are carried here; the
+# summaries, with their commands, are profiles/linear_and_conv2d_hbm_traffic_counters.md.
 MEASURED_TRAFFIC_BYTES = {
-    ("gemm", "fwd"): 235.0e6,      # algorithmic 151.0e6
-    ("gemm", "bwd_dw"): 285.8e6,   # algorithmic 213.9e6
-    ("gemm", "bwd_dz"): 167.9e6,   # algorithmic 88.1e6
-    ("skinny", "fwd"): 562.2e6,    # algorithmic 536.9e6
-    ("skinny", "bwd_dz"): 286.3e6, # algorithmic 268.4e6
-    ("skinny", "bwd_dw"): 815.3e6, # algorithmic 805.3e6
+    # (workload, phase): (kernel, bytes)
+    ("gemm", "fwd"): ("mfma_tile_kernel<LinearProblem<0,...>, 64, 128, 2, 4>", 235.0e6),      # algorithmic 151.0e6
+    ("gemm", "bwd_dw"): ("linear_dw_side_kernel<LinearProblem<2,...>, 64, 128, 2, 4>", 334.0e6),  # algorithmic 213.9e6
+    ("gemm", "bwd_dz"): ("mfma_tile_kernel<LinearProblem<1,...>, 64, 128, 2, 4>", 167.9e6),   # algorithmic 88.1e6
+    ("skinny", "fwd"): ("gemv_fwd_kernel<2, 2, 1>", 562.2e6),       # algorithmic 536.9e6
+    ("skinny", "bwd_dz"): ("gemv_dz_kernel<2>", 286.3e6),           # algorithmic 268.4e6
+    ("skinny", "bwd_dw"): ("gemv_dw_kernel<8, true>", 815.3e6),     # algorithmic 805.3e6
+    ("conv", "fwd"): ("conv_stencil_kernel<false, 32>", None),
 }
 
 # Conv2d 3x3, stride 1, pad 1, 64 -> 64 channels on 32x32 maps, batch 128, no bias
@@ -167,7 +175,9 @@ def run_workload(name, steps, warmup):
         # the timed call launches the tile kernel and, after it, the fold of its
         # reduction slices (about 9 of the 211 us); a kernel trace lists them apart
         roof["covers"] = "forward call = tile kernel + fold of its four reduction slices"
-    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get((name, dominant))
+    kernel, traffic = MEASURED_TRAFFIC_BYTES.get((name, dominant), (None, None))
+    roof["traffic"] = traffic
+    roof["traffic_kernel"] = kernel
     roof["kernel_ms"] = round(phase_ms[dominant], 5)
     return dict(name=name, K=K, N=N, B=B, value=value, unit=unit, frac_of_peak=value / peak,
                 ms_per_step=ms_per_step, wall_ms=wall_ms, phase_ms=phase_ms, roofline=roof)
@@ -210,9 +220,67 @@ def run_conv(steps, warmup):
     torch.cuda.synchronize()
     ms = e0.elapsed_time(e1) / steps
     tflops = 14.0 * fo * (B * woho) * R / (ms * 1e-3) / 1e12
+    # the forward kernel alone, for the roofline of the dominant kernel
+    f0, f1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    f0.record()
+    for _ in range(steps):
+        F.conv2d_fwd(mu_w, var_w, None, None, mu_a, var_a, t["Fmwa_2"], woho, fo, wihi, fi, k, B)
+    f1.record()
+    torch.cuda.synchronize()
+    fwd_ms = f0.elapsed_time(f1) / steps
+    fwd_tflops = 6.0 * fo * (B * woho) * R / (fwd_ms * 1e-3) / 1e12
     return dict(workload="TAGI Conv2d 3x3 s1 p1, 64->64 channels, 32x32 maps, batch 128, no bias, "
                          "forward + backward", value=round(tflops, 3), unit="TFLOP/s",
-                frac_of_peak=round(tflops / FP32_MFMA_PEAK_TFLOPS, 4), ms_per_step=round(ms, 5))
+                frac_of_peak=round(tflops / FP32_MFMA_PEAK_TFLOPS, 4), ms_per_step=round(ms, 5),
+                roofline=dict(bound="mfma", kernel="fwd", achieved=round(fwd_tflops, 2),
+                              peak=FP32_MFMA_PEAK_TFLOPS, unit="TFLOP/s",
+                              frac=round(fwd_tflops / FP32_MFMA_PEAK_TFLOPS, 4), traffic=None,
+                              traffic_kernel=MEASURED_TRAFFIC_BYTES[("conv", "fwd")][0],
+                              kernel_ms=round(fwd_ms, 5)))
+
+
+def run_mlp(steps, warmup, B=32):
+    """One training step of the MLP configuration (784 -> 128 -> 128 -> 11 with ReLU,
+    batch 32: forward, output update on 4 selected units per sample, backward, step)
+    through the host classes with host input arrays, outputs fetched: wall time per
+    step. Latency-bound (a few dozen small launches), so no throughput is quoted."""
+    import numpy as np
+    import torch
+    from cutagi_amd import cutagi
+
+    cutagi.manual_seed(0)
+    net = cutagi.Sequential([cutagi.Linear(784, 128), cutagi.ReLU(), cutagi.Linear(128, 128),
+                             cutagi.ReLU(), cutagi.Linear(128, 11)])
+    net.to_device("cuda")
+    updater = cutagi.OutputUpdater(net.device)
+    rng = np.random.default_rng(0)
+    x = rng.normal(0, 1, (B, 784)).astype(np.float32)
+    sel = np.concatenate([rng.choice(11, 4, replace=False) + 1 for _ in range(B)]).astype(np.int32)
+    y = rng.normal(0, 1, B * 4).astype(np.float32)
+    var_y = np.ones(B * 4, np.float32)
+
+    def step():
+        net.forward(x)
+        mu, var = net.get_outputs()
+        updater.update_using_indices(net.output_z_buffer, y, var_y, sel, net.input_delta_z_buffer)
+        net.backward()
+        net.step()
+        return mu, var
+
+    for _ in range(max(warmup, 20)):
+        step()
+    torch.cuda.synchronize()
+    n = max(steps, 200)
+    t0 = time.perf_counter()
+    for _ in range(n):
+        mu, var = step()
+    torch.cuda.synchronize()
+    us = (time.perf_counter() - t0) * 1e6 / n
+    return dict(workload="TAGI MLP 784->128->128->11 (ReLU), batch %d, one training step through "
+                         "the host classes, outputs fetched" % B,
+                value=round(us, 1), unit="us/step", higher_is_better=False, steps=n,
+                outputs_finite_and_variances_nonnegative=bool(np.all(np.isfinite(mu))
+                                                              and var.min() >= 0))
 
 
 def run_resnet(steps, warmup, B=128):
@@ -323,12 +391,14 @@ def main():
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="gemm")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
-    ap.add_argument("--extra", default="linear,conv,resnet18",
-                    help="comma-separated secondary workloads to run (linear, conv, resnet18)")
+    ap.add_argument("--extra", default="linear,conv,resnet18,mlp",
+                    help="comma-separated secondary workloads to run (linear, conv, resnet18, mlp)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain 1 GiB device copy (reference for byte counters)")
     args = ap.parse_args()
 
+    if args.workload not in ("gemm", "skinny"):
+        ap.error("--workload is gemm or skinny")
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path "
               "(run with --gpus 1)", file=sys.stderr)
@@ -339,6 +409,9 @@ def main():
         print("bench.py needs a GPU (torch.cuda.is_available() is False)", file=sys.stderr)
         sys.exit(1)
 
+    gpu_t0 = time.perf_counter()
+    from cutagi_amd import capi
+    cus, clock_mhz, dev_name = capi.device_info()
     main_res = run_workload(args.workload, args.steps, args.warmup)
     line = {
         "metric": "TAGI Linear fwd+bwd TFLOP/s (% fp32 MFMA peak) 4096^2,B=256; GB/s at B=8",
@@ -360,6 +433,12 @@ def main():
         "frac_of_peak": round(main_res["frac_of_peak"], 4),
         "phase_ms": {k: round(v, 5) for k, v in main_res["phase_ms"].items()},
         "roofline": main_res["roofline"],
+        # what the runtime reports for the part, and the fp32 matrix peak that follows
+        # from it (compute units x 256 flop per clock x clock); `roofline.peak` is the
+        # published figure
+        "device": {"name": dev_name, "cus": cus, "sclk_mhz": clock_mhz,
+                   "fp32_mfma_peak_from_device_tflops": round(
+                       cus * FP32_MFMA_FLOP_PER_CLK_PER_CU * clock_mhz * 1e6 / 1e12, 1)},
     }
     extras = [] if args.no_extra else [e for e in args.extra.split(",") if e]
     if extras:
@@ -374,12 +453,27 @@ def main():
             "ms_per_step": round(r["ms_per_step"], 5),
             "phase_ms": {k: round(v, 5) for k, v in r["phase_ms"].items()},
             "roofline": r["roofline"]}
+        if args.workload == "gemm":
+            for wide in ("skinny12", "skinny16"):
+                r = run_workload(wide, args.steps, args.warmup)
+                line["extra"][wide] = {
+                    "workload": "TAGI Linear %d->%d, batch %d" % (r["K"], r["N"], r["B"]),
+                    "value": round(r["value"], 3), "unit": r["unit"],
+                    "frac_of_peak": round(r["frac_of_peak"], 4),
+                    "ms_per_step": round(r["ms_per_step"], 5),
+                    "phase_ms": {k: round(v, 5) for k, v in r["phase_ms"].items()},
+                    "roofline": r["roofline"]}
+    if "mlp" in extras:
+        line["extra"]["mlp"] = run_mlp(args.steps, args.warmup)
     if "conv" in extras:
         line["extra"]["conv"] = run_conv(max(5, args.steps // 2), args.warmup)
     if "resnet18" in extras:
         line["extra"]["resnet18"] = run_resnet(max(20, args.steps // 2), 5)
     if args.calibrate:
         calibrate_copy()
+    # wall time of everything that ran on the GPU, so that the short timed regions can
+    # be placed inside the whole run (the CPU baseline below takes most of it)
+    line["gpu_wall_s"] = round(time.perf_counter() - gpu_t0, 2)
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(args.workload)
     print(json.dumps(line))
