@@ -33,6 +33,7 @@ SIGNATURES = {
     "tagi_hip_shutdown": (_i, []),
     "tagi_hip_tune": (_i, [ctypes.c_char_p, _i]),
     "tagi_linear_fwd": (_i, [_vp] * 6 + [_i] * 4 + [_vp] * 3),
+    "tagi_linear_fwd_act": (_i, [_vp] * 6 + [_i] * 5 + [_vp] * 4),
     "tagi_linear_fwd_static": (_i, [_vp] * 6 + [_i] * 4 + [_vp] * 3),
     "tagi_linear_bwd_dz": (_i, [_vp] * 4 + [_i] * 3 + [_vp] * 3),
     "tagi_linear_bwd_dw": (_i, [_vp] * 4 + [_i] * 3 + [_vp] * 3),
@@ -41,6 +42,7 @@ SIGNATURES = {
     "tagi_conv2d_out_size": (_i, [_i] * 6 + [_ip, _ip]),
     "tagi_conv2d_build_idx": (_i, [_i] * 7 + [_ip] * 5),
     "tagi_conv2d_fwd": (_i, [_vp] * 7 + [_i] * 7 + [_vp] * 3),
+    "tagi_conv2d_fwd_act": (_i, [_vp] * 7 + [_i] * 8 + [_vp] * 4),
     "tagi_conv2d_bwd_dz": (_i, [_vp] * 6 + [_i] * 7 + [_vp] * 3),
     "tagi_conv2d_bwd_dw": (_i, [_vp] * 6 + [_i] * 7 + [_vp] * 5),
     "tagi_store_states": (_i, [_vp, _vp, _sz, _vp, _vp, _vp, _sz, _vp]),

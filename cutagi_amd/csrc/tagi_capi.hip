@@ -189,7 +189,7 @@ int run_gemm(GemmMode mode, GemmParams p, bool vec, int forced_splits, hipStream
         }
         TAGI_TRY(launch_reduce_splits(mode == GEMM_FWD ? EPI_BIAS : EPI_SCALE, p.ws0, p.ws1,
                                       splits, p.M, p.N, p.e0, p.e1, p.out0, p.out1, p.ldo,
-                                      stream));
+                                      stream, p.act, p.out2));
     }
     return TAGI_OK;
 }
@@ -308,7 +308,8 @@ int tagi_hip_tune(const char *key, int value) {
 static int linear_fwd_impl(const float *mu_w, const float *var_w, const float *mu_b,
                            const float *var_b, const float *mu_a, const float *var_a, int K, int N,
                            int B, int bias, float *mu_z, float *var_z, void *stream_,
-                           ScratchSource scratch_get) {
+                           ScratchSource scratch_get, int act = 0, float *jcb = nullptr) {
+    if (act < 0 || act > 2 || (act != 0 && jcb == nullptr)) return TAGI_ERR_INVALID_ARG;
     if (!mu_w || !var_w || !mu_a || !var_a || !mu_z || !var_z) return TAGI_ERR_INVALID_ARG;
     if (K <= 0 || N <= 0 || B <= 0) return TAGI_ERR_INVALID_ARG;
     if (bias && (!mu_b || !var_b)) return TAGI_ERR_INVALID_ARG;
@@ -335,7 +336,7 @@ static int linear_fwd_impl(const float *mu_w, const float *var_w, const float *m
         TAGI_TRY(launch_gemv16_fwd(mu_w, var_w, mu_a, var_a, K, N, B, per, splits, ws, ws + part,
                                    stream));
         TAGI_TRY(launch_reduce_splits(EPI_BIAS, ws, ws + part, splits, B, N, e0, e1, mu_z, var_z, N,
-                                      stream));
+                                      stream, act, jcb));
         return TAGI_OK;
     }
 
@@ -363,7 +364,7 @@ static int linear_fwd_impl(const float *mu_w, const float *var_w, const float *m
                                  g_tune.gemv_swz >= 0 ? g_tune.gemv_swz : 3, variant, ws,
                                  ws + part, stream));
         TAGI_TRY(launch_reduce_splits(EPI_BIAS, ws, ws + part, splits, B, N, e0, e1, mu_z, var_z, N,
-                                      stream));
+                                      stream, act, jcb));
         return TAGI_OK;
     }
 
@@ -372,6 +373,7 @@ static int linear_fwd_impl(const float *mu_w, const float *var_w, const float *m
     p.M = B; p.N = N; p.R = K; p.ldx = K; p.ldy = K;
     p.out0 = mu_z; p.out1 = var_z; p.ldo = N;
     p.e0 = e0; p.e1 = e1;
+    p.act = act; p.out2 = jcb;
     return run_gemm(GEMM_FWD, p, vec, g_tune.fwd_splits, stream, nullptr, scratch_get);
 }
 
@@ -380,6 +382,16 @@ int tagi_linear_fwd(const float *mu_w, const float *var_w, const float *mu_b, co
                     float *mu_z, float *var_z, void *stream) {
     return linear_fwd_impl(mu_w, var_w, mu_b, var_b, mu_a, var_a, K, N, B, bias, mu_z, var_z,
                            stream, workspace_get);
+}
+
+int tagi_linear_fwd_act(const float *mu_w, const float *var_w, const float *mu_b,
+                        const float *var_b, const float *mu_a, const float *var_a, int K, int N,
+                        int B, int bias, int activation, float *mu_out, float *var_out,
+                        float *jcb_out, void *stream) {
+    if (activation != TAGI_ACT_RELU && activation != TAGI_ACT_MIXTURE_RELU)
+        return TAGI_ERR_INVALID_ARG;
+    return linear_fwd_impl(mu_w, var_w, mu_b, var_b, mu_a, var_a, K, N, B, bias, mu_out, var_out,
+                           stream, workspace_get, activation, jcb_out);
 }
 
 int tagi_linear_fwd_static(const float *mu_w, const float *var_w, const float *mu_b,
@@ -596,10 +608,12 @@ int tagi_conv2d_build_idx(int kernel, int stride, int wi, int hi, int pad, int p
                : TAGI_ERR_INVALID_ARG;
 }
 
-int tagi_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b, const float *var_b,
-                    const float *mu_a, const float *var_a, const int *aidx, int woho, int fo,
-                    int wihi, int fi, int ki, int B, int bias, float *mu_z, float *var_z,
-                    void *stream_) {
+static int conv2d_fwd_impl(const float *mu_w, const float *var_w, const float *mu_b,
+                           const float *var_b, const float *mu_a, const float *var_a,
+                           const int *aidx, int woho, int fo, int wihi, int fi, int ki, int B,
+                           int bias, float *mu_z, float *var_z, void *stream_, int act,
+                           float *jcb) {
+    if (act < 0 || act > 2 || (act != 0 && jcb == nullptr)) return TAGI_ERR_INVALID_ARG;
     if (!mu_w || !var_w || !mu_a || !var_a || !aidx || !mu_z || !var_z)
         return TAGI_ERR_INVALID_ARG;
     if (woho <= 0 || fo <= 0 || wihi <= 0 || fi <= 0 || ki <= 0 || B <= 0)
@@ -618,8 +632,28 @@ int tagi_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b, co
         if (rc != TAGI_OK) return rc;
     }
     TAGI_TRY(launch_conv2d_fwd(mu_w, var_w, mu_b, var_b, mu_a, var_a, aidx, woho, fo, wihi, fi, ki,
-                               B, bias, tile, splits, ws, ws + part, mu_z, var_z, stream));
+                               B, bias, tile, splits, ws, ws + part, mu_z, var_z, stream, act,
+                               jcb));
     return TAGI_OK;
+}
+
+int tagi_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b, const float *var_b,
+                    const float *mu_a, const float *var_a, const int *aidx, int woho, int fo,
+                    int wihi, int fi, int ki, int B, int bias, float *mu_z, float *var_z,
+                    void *stream) {
+    return conv2d_fwd_impl(mu_w, var_w, mu_b, var_b, mu_a, var_a, aidx, woho, fo, wihi, fi, ki, B,
+                           bias, mu_z, var_z, stream, 0, nullptr);
+}
+
+int tagi_conv2d_fwd_act(const float *mu_w, const float *var_w, const float *mu_b,
+                        const float *var_b, const float *mu_a, const float *var_a,
+                        const int *aidx, int woho, int fo, int wihi, int fi, int ki, int B,
+                        int bias, int activation, float *mu_out, float *var_out, float *jcb_out,
+                        void *stream) {
+    if (activation != TAGI_ACT_RELU && activation != TAGI_ACT_MIXTURE_RELU)
+        return TAGI_ERR_INVALID_ARG;
+    return conv2d_fwd_impl(mu_w, var_w, mu_b, var_b, mu_a, var_a, aidx, woho, fo, wihi, fi, ki, B,
+                           bias, mu_out, var_out, stream, activation, jcb_out);
 }
 
 int tagi_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *delta_mu_out,

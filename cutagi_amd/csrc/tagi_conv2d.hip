@@ -18,6 +18,7 @@
 #include <type_traits>
 
 #include "tagi_internal.h"
+#include "tagi_activation.h"
 #include "tagi_mfma_tile.h"
 
 namespace tagi {
@@ -38,6 +39,10 @@ struct ConvParams {
     // states: column order. perm_s > 1 numbers the input pixels phase by phase
     // ((y mod s, x mod s) major, then image, then pixel) on maps of width perm_w.
     int perm_s, perm_w;
+    // forward only: activation applied to the sums before they are stored
+    // (tagi_activation.h); out2 then receives its Jacobian
+    int act;
+    float *out2;
 };
 
 // All operand loads below are unconditional: an element outside the problem (or
@@ -238,8 +243,7 @@ struct ConvFwdProblem {
             a0 += p.e0[m];
             a1 += p.e1[m];
         }
-        p.out0[at] = a0;
-        p.out1[at] = a1;
+        store_activated(p.act, a0, a1, at, p.out0, p.out1, p.out2);
     }
 };
 
@@ -760,8 +764,9 @@ hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float 
                              const float *var_b, const float *mu_a, const float *var_a,
                              const int *aidx, int woho, int fo, int wihi, int fi, int ki, int B,
                              int bias, int tile, int splits, float *ws0, float *ws1, float *mu_z,
-                             float *var_z, hipStream_t stream) {
+                             float *var_z, hipStream_t stream, int act, float *jcb) {
     ConvParams p = {};
+    p.act = act; p.out2 = jcb;
     p.w0 = mu_w; p.w1 = var_w; p.a0 = mu_a; p.a1 = var_a;
     p.e0 = bias ? mu_b : nullptr; p.e1 = bias ? var_b : nullptr;
     p.idx = aidx; p.out0 = mu_z; p.out1 = var_z;

@@ -1,6 +1,7 @@
 // Small bandwidth-bound kernels around the TAGI layers: bias innovation, state
 // bookkeeping, capped parameter step, output innovation and ReLU. gfx950.
 #include "tagi_internal.h"
+#include "tagi_activation.h"
 
 namespace tagi {
 namespace {
@@ -217,11 +218,11 @@ __global__ __launch_bounds__(TPB) void relu_kernel(const float *mu_z, const floa
                                                    float *var_a) {
     const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
     if (i >= n) return;
-    const float m = fmaxf(mu_z[i], 0.f);
-    const float v = var_z[i];
+    float m, v, j;
+    relu_moments(mu_z[i], var_z[i], m, v, j);
     mu_a[i] = m;
-    jcb[i] = (m == 0.f) ? 0.f : 1.f;
-    var_a[i] = (m == 0.f) ? 0.f : v;
+    jcb[i] = j;
+    var_a[i] = v;
 }
 
 }  // namespace

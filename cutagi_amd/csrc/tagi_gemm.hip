@@ -10,6 +10,7 @@
 //   DW : D[n][k'] = sum_b delta[b][n] * act[b][k'] (variance with act^2); both
 //        operands are staged [b][...] as they lie in memory.
 #include "tagi_internal.h"
+#include "tagi_activation.h"
 #include "tagi_mfma_tile.h"
 
 namespace tagi {
@@ -110,6 +111,8 @@ struct LinearProblem {
                 a0 += p.e0[n];
                 a1 += p.e1[n];
             }
+            store_activated(p.act, a0, a1, at, p.out0, p.out1, p.out2);
+            return;
         } else {
             const float e = p.e0[at];
             a0 *= e;
@@ -127,7 +130,8 @@ __global__ __launch_bounds__(64) void reduce_splits_kernel(const float *__restri
                                                             const float *__restrict__ e0,
                                                             const float *__restrict__ e1,
                                                             float *__restrict__ out0,
-                                                            float *__restrict__ out1, int ldo) {
+                                                            float *__restrict__ out1, int ldo,
+                                                            int act, float *__restrict__ out2) {
     const size_t total = (size_t)M * N;
     constexpr int W = VEC ? 4 : 1;
     const size_t idx = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * W;
@@ -163,6 +167,21 @@ __global__ __launch_bounds__(64) void reduce_splits_kernel(const float *__restri
             s0[c] *= e;
             s1[c] *= e * e;
         }
+    }
+    float s2[W];
+    if (EPI == EPI_BIAS && act != ACT_NONE) {
+#pragma unroll
+        for (int c = 0; c < W; c++) {
+            const float m = s0[c], v = s1[c];
+            if (act == ACT_RELU)
+                relu_moments(m, v, s0[c], s1[c], s2[c]);
+            else
+                mixture_relu_moments(m, v, s0[c], s1[c], s2[c]);
+        }
+        if constexpr (VEC)
+            *reinterpret_cast<float4 *>(out2 + at) = make_float4(s2[0], s2[1], s2[2], s2[3]);
+        else
+            out2[at] = s2[0];
     }
     if constexpr (VEC) {
         *reinterpret_cast<float4 *>(out0 + at) = make_float4(s0[0], s0[1], s0[2], s0[3]);
@@ -323,27 +342,28 @@ hipError_t launch_gemm_dw_side(const GemmParams &p, LinearSideWork w, hipStream_
 
 hipError_t launch_reduce_splits(Epilogue epi, const float *ws0, const float *ws1, int splits,
                                 int M, int N, const float *e0, const float *e1, float *out0,
-                                float *out1, int ldo, hipStream_t stream) {
+                                float *out1, int ldo, hipStream_t stream, int act, float *out2) {
     const size_t total = (size_t)M * N;
     auto al = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; };
     const bool vec = (N % 4 == 0) && (ldo % 4 == 0) && al(ws0) && al(ws1) && al(out0) &&
-                     al(out1) && (epi == EPI_BIAS || al(e0));
+                     al(out1) && (epi == EPI_BIAS || al(e0)) && (act == ACT_NONE || al(out2));
+    if (epi != EPI_BIAS) act = ACT_NONE;
     const size_t items = vec ? total / 4 : total;
     dim3 grid((unsigned)((items + 63) / 64)), block(64);
     if (epi == EPI_BIAS) {
         if (vec)
             hipLaunchKernelGGL((reduce_splits_kernel<EPI_BIAS, true>), grid, block, 0, stream, ws0,
-                               ws1, splits, M, N, e0, e1, out0, out1, ldo);
+                               ws1, splits, M, N, e0, e1, out0, out1, ldo, act, out2);
         else
             hipLaunchKernelGGL((reduce_splits_kernel<EPI_BIAS, false>), grid, block, 0, stream,
-                               ws0, ws1, splits, M, N, e0, e1, out0, out1, ldo);
+                               ws0, ws1, splits, M, N, e0, e1, out0, out1, ldo, act, out2);
     } else {
         if (vec)
             hipLaunchKernelGGL((reduce_splits_kernel<EPI_SCALE, true>), grid, block, 0, stream,
-                               ws0, ws1, splits, M, N, e0, e1, out0, out1, ldo);
+                               ws0, ws1, splits, M, N, e0, e1, out0, out1, ldo, act, out2);
         else
             hipLaunchKernelGGL((reduce_splits_kernel<EPI_SCALE, false>), grid, block, 0, stream,
-                               ws0, ws1, splits, M, N, e0, e1, out0, out1, ldo);
+                               ws0, ws1, splits, M, N, e0, e1, out0, out1, ldo, act, out2);
     }
     return hipGetLastError();
 }

@@ -33,6 +33,10 @@ struct GemmParams {
     int splits;            // number of reduction slices (gridDim.y)
     int r_per_split;       // reduction elements per slice, multiple of the k-tile
     float *ws0, *ws1;      // [splits][M][N] partial sums when splits > 1
+    // FWD only: activation applied to the sums before they are stored (tagi_activation.h);
+    // then out0/out1 receive its mean / variance and out2 its Jacobian
+    int act;
+    float *out2;
 };
 
 // Tile shapes the tiled kernels are instantiated for (indices 0..count-1).
@@ -69,10 +73,11 @@ bool gemm_dw_side_supported(int tile, bool vec, const GemmParams &p);
 hipError_t launch_gemm_dw_side(const GemmParams &p, LinearSideWork w, hipStream_t stream);
 
 // out = epilogue(sum over splits of ws[s]) for the two accumulators.
+// (EPI_BIAS only: `act` / `out2` as in GemmParams.)
 hipError_t launch_reduce_splits(Epilogue epi, const float *ws0, const float *ws1,
                                 int splits, int M, int N, const float *e0,
                                 const float *e1, float *out0, float *out1, int ldo,
-                                hipStream_t stream);
+                                hipStream_t stream, int act = 0, float *out2 = nullptr);
 
 // Skinny-batch (B <= 16) streaming kernels: weights are read once from HBM
 // straight into MFMA operand layout, nothing is staged in LDS.
@@ -187,7 +192,7 @@ hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float 
                              const float *var_b, const float *mu_a, const float *var_a,
                              const int *aidx, int woho, int fo, int wihi, int fi, int ki, int B,
                              int bias, int tile, int splits, float *ws0, float *ws1, float *mu_z,
-                             float *var_z, hipStream_t stream);
+                             float *var_z, hipStream_t stream, int act = 0, float *jcb = nullptr);
 hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *dmu,
                                 const float *dvar, const int *zw_idx, const int *zud_idx,
                                 int woho, int fo, int wihi, int fi, int ki, int nr, int B,

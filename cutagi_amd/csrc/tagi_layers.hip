@@ -3,6 +3,7 @@
 // AvgPool2d and the residual adds. All of them are bandwidth-bound passes over
 // [B][channels][pixels] tensors; gfx950.
 #include "tagi_internal.h"
+#include "tagi_activation.h"
 
 namespace tagi {
 namespace {
@@ -24,16 +25,11 @@ __global__ __launch_bounds__(TPB) void mixture_relu_kernel(const float *__restri
                                                            float *__restrict__ var_a) {
     const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
     if (i >= n) return;
-    constexpr float INV_SQRT_2PI = 1.0f / 2.5066282746310002f;
-    const float m = mu_z[i], v = var_z[i];
-    const float sd = sqrtf(v);
-    const float alpha = m / sd;
-    const float pdf = INV_SQRT_2PI * expf(-0.5f * alpha * alpha);
-    const float cdf = 0.5f * erfcf(-alpha * 0.7071067811865475f);
-    const float t = m * cdf + sd * pdf;
-    mu_a[i] = fmaxf(0.000001f, t);
-    var_a[i] = fmaxf(0.000001f, -t * t + 2.f * t * m - m * sd * pdf + (v - m * m) * cdf);
-    jcb[i] = cdf;
+    float m, v, j;
+    mixture_relu_moments(mu_z[i], var_z[i], m, v, j);
+    mu_a[i] = m;
+    var_a[i] = v;
+    jcb[i] = j;
 }
 
 // ---------------------------------------------------------------------------

@@ -37,6 +37,24 @@ def linear_fwd(mu_w, var_w, mu_b, var_b, mu_a, var_a, out=None):
     return mu_z, var_z
 
 
+ACTIVATIONS = {"relu": 1, "mixture_relu": 2}
+
+
+def linear_fwd_act(mu_w, var_w, mu_b, var_b, mu_a, var_a, activation):
+    """Linear forward with the following activation ("relu" / "mixture_relu") applied
+    in the kernel's epilogue: returns the activation's (mu_a, var_a, jcb)."""
+    _chk(mu_w, var_w, mu_b, var_b, mu_a, var_a)
+    N, K = mu_w.shape
+    B = mu_a.shape[0]
+    out = [torch.empty((B, N), device=mu_w.device) for _ in range(3)]
+    capi.check(capi.lib.tagi_linear_fwd_act(capi.ptr(mu_w), capi.ptr(var_w), capi.ptr(mu_b),
+                                            capi.ptr(var_b), capi.ptr(mu_a), capi.ptr(var_a), K, N,
+                                            B, int(mu_b is not None), ACTIVATIONS[activation],
+                                            capi.ptr(out[0]), capi.ptr(out[1]), capi.ptr(out[2]),
+                                            _stream()))
+    return tuple(out)
+
+
 def linear_bwd_dz(mu_w, jcb, delta_mu, delta_var, out=None):
     _chk(mu_w, jcb, delta_mu, delta_var)
     N, K = mu_w.shape
@@ -106,6 +124,21 @@ def conv2d_fwd(mu_w, var_w, mu_b, var_b, mu_a, var_a, aidx, woho, fo, wihi, fi, 
                                         capi.ptr(aidx), woho, fo, wihi, fi, ki, B, int(bias),
                                         capi.ptr(mu_z), capi.ptr(var_z), _stream()))
     return mu_z, var_z
+
+
+def conv2d_fwd_act(mu_w, var_w, mu_b, var_b, mu_a, var_a, aidx, woho, fo, wihi, fi, ki, B,
+                   activation):
+    """Conv2d forward with the following activation applied in the kernel's epilogue:
+    returns the activation's (mu_a, var_a, jcb), each [B][fo][woho] flattened."""
+    _chk(mu_w, var_w, mu_b, var_b, mu_a, var_a, aidx)
+    out = [torch.empty(B * fo * woho, device=mu_w.device) for _ in range(3)]
+    capi.check(capi.lib.tagi_conv2d_fwd_act(capi.ptr(mu_w), capi.ptr(var_w), capi.ptr(mu_b),
+                                            capi.ptr(var_b), capi.ptr(mu_a), capi.ptr(var_a),
+                                            capi.ptr(aidx), woho, fo, wihi, fi, ki, B,
+                                            int(mu_b is not None), ACTIVATIONS[activation],
+                                            capi.ptr(out[0]), capi.ptr(out[1]), capi.ptr(out[2]),
+                                            _stream()))
+    return tuple(out)
 
 
 def conv2d_bwd_dz(mu_w, jcb, delta_mu, delta_var, zw_idx, zud_idx, woho, fo, wihi, fi, ki, nr, B):

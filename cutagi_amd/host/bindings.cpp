@@ -297,6 +297,9 @@ PYBIND11_MODULE(cutagi, m) {
         });
 
     m.def("manual_seed", &manual_seed);
+    // not in the reference: ReLU / MixtureReLU after a Linear / Conv2d layer run in that
+    // layer's kernel by default; False gives every layer its own launch again
+    m.def("set_fused_activations", &set_fused_activations, py::arg("on"));
     m.def("is_cuda_available", &is_cuda_available);
     m.def("get_cuda_device_count", &get_cuda_device_count);
     m.def("get_cuda_current_device", &get_current_cuda_device);

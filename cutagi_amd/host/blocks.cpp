@@ -33,6 +33,23 @@ std::unique_ptr<BaseLayer> MixtureReLUHip::to_cuda(int device_idx) {
     return layer;
 }
 
+// ---- activation fusion --------------------------------------------------------------------
+static bool g_fused_activations = true;
+void set_fused_activations(bool on) { g_fused_activations = on; }
+
+int fusable_activation(const BaseLayer *layer, const BaseLayer *next) {
+    if (!g_fused_activations || layer == nullptr || next == nullptr) return 0;
+    if (!layer->can_fuse_activation()) return 0;
+    if (dynamic_cast<const ReLUHip *>(next) != nullptr) return TAGI_ACT_RELU;
+    if (dynamic_cast<const MixtureReLUHip *>(next) != nullptr) return TAGI_ACT_MIXTURE_RELU;
+    return 0;
+}
+
+void activation_absorbed(BaseLayer *activation, const BaseHiddenStates &output_states) {
+    activation->input_size = output_states.actual_size;
+    activation->output_size = output_states.actual_size;
+}
+
 // reference: MixtureReLUCuda::forward, src/activation_cuda.cu:726-760
 void MixtureReLUHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &output_states,
                              BaseTempStates &) {
@@ -471,11 +488,18 @@ void LayerBlock::forward(BaseHiddenStates &input_states, BaseHiddenStates &outpu
                          BaseTempStates &temp_states) {
     BaseHiddenStates *in = &input_states, *out = &output_states;
     const size_t batch_size = input_states.block_size;
-    for (auto &layer : layers) {
-        layer->forward(*in, *out, temp_states);
+    size_t passes = 0;
+    for (size_t i = 0; i < layers.size(); i++, passes++) {
+        // an activation that follows a Linear / Conv2d layer runs in that layer's epilogue
+        const int act = i + 1 < layers.size()
+                            ? fusable_activation(layers[i].get(), layers[i + 1].get())
+                            : 0;
+        layers[i]->fused_activation = act;
+        layers[i]->forward(*in, *out, temp_states);
+        if (act != 0) activation_absorbed(layers[++i].get(), *out);
         std::swap(in, out);
     }
-    if (layers.size() % 2 == 0) output_states.swap(input_states);
+    if (passes % 2 == 0) output_states.swap(input_states);
     set_output_dims(output_states, *this, batch_size);
 }
 

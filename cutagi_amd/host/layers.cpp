@@ -417,9 +417,18 @@ void LinearHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &output
         LOG(LogLevel::ERROR, "Output state buffer too small for " + this->get_layer_info());
     if (d_mu_w == nullptr) LOG(LogLevel::ERROR, "Parameters of " + get_layer_info() + " are not on the device");
 
-    TAGI_OK_OR_THROW(tagi_linear_fwd(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a, in->d_var_a,
-                                     (int)input_size, (int)output_size, batch_size, bias ? 1 : 0,
-                                     out->d_mu_a, out->d_var_a, nullptr));
+    const int act = this->fused_activation;
+    this->fused_activation = 0;
+    if (act != 0)
+        TAGI_OK_OR_THROW(tagi_linear_fwd_act(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a,
+                                             in->d_var_a, (int)input_size, (int)output_size,
+                                             batch_size, bias ? 1 : 0, act, out->d_mu_a,
+                                             out->d_var_a, out->d_jcb, nullptr));
+    else
+        TAGI_OK_OR_THROW(tagi_linear_fwd(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a,
+                                         in->d_var_a, (int)input_size, (int)output_size,
+                                         batch_size, bias ? 1 : 0, out->d_mu_a, out->d_var_a,
+                                         nullptr));
     output_states.width = this->out_width;
     output_states.height = this->out_height;
     output_states.depth = this->out_channels;
@@ -427,6 +436,7 @@ void LinearHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &output
     output_states.actual_size = this->output_size;
     out->jcb_ones = true;
     if (this->training) this->store_states_for_training_hip(*in, *out);
+    if (act != 0) out->jcb_ones = false;  // the activation's Jacobian was written
 }
 
 // reference: LinearCuda::backward, src/linear_layer_cuda.cu:273-323
@@ -617,12 +627,22 @@ void Conv2dHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &output
     output_states.actual_size = output_size;
 
     const int woho = (int)(out_width * out_height), wihi = (int)(in_width * in_height);
-    TAGI_OK_OR_THROW(tagi_conv2d_fwd(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a, in->d_var_a,
-                                     d_idx_mwa_2, woho, (int)out_channels, wihi, (int)in_channels,
-                                     (int)kernel_size, batch_size, bias ? 1 : 0, out->d_mu_a,
-                                     out->d_var_a, nullptr));
+    const int act = this->fused_activation;
+    this->fused_activation = 0;
+    if (act != 0)
+        TAGI_OK_OR_THROW(tagi_conv2d_fwd_act(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a,
+                                             in->d_var_a, d_idx_mwa_2, woho, (int)out_channels,
+                                             wihi, (int)in_channels, (int)kernel_size, batch_size,
+                                             bias ? 1 : 0, act, out->d_mu_a, out->d_var_a,
+                                             out->d_jcb, nullptr));
+    else
+        TAGI_OK_OR_THROW(tagi_conv2d_fwd(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a,
+                                         in->d_var_a, d_idx_mwa_2, woho, (int)out_channels, wihi,
+                                         (int)in_channels, (int)kernel_size, batch_size,
+                                         bias ? 1 : 0, out->d_mu_a, out->d_var_a, nullptr));
     out->jcb_ones = true;
     if (training) this->store_states_for_training_hip(*in, *out);
+    if (act != 0) out->jcb_ones = false;  // the activation's Jacobian was written
 }
 
 // reference: Conv2dCuda::backward, src/conv2d_layer_cuda.cu:453-519. No temporary

@@ -65,6 +65,12 @@ class BaseLayer {
     std::vector<float> mu_w, var_w, mu_b, var_b;
     std::vector<float> delta_mu_w, delta_var_w, delta_mu_b, delta_var_b;
     std::unique_ptr<BaseBackwardStates> bwd_states;
+    // One-shot request to the next forward() of a layer that can_fuse_activation():
+    // apply this activation (TAGI_ACT_*) in the kernel's epilogue and write its
+    // moments and Jacobian instead of the layer's own output. Set by the owner of the
+    // layer list when the next layer is that activation; forward() clears it.
+    int fused_activation = 0;
+    virtual bool can_fuse_activation() const { return false; }
 
     unsigned int num_threads = 4;
     bool training = true;
@@ -208,6 +214,7 @@ class LinearHip : public BaseLayerHip {
     // the reference names its device layers *Cuda; state_dict keys derive from this
     std::string get_layer_name() const override { return "LinearCuda"; }
     LayerType get_layer_type() const override { return LayerType::Linear; }
+    bool can_fuse_activation() const override { return true; }
     void init_weight_bias() override;
     void forward(BaseHiddenStates &input_states, BaseHiddenStates &output_states,
                  BaseTempStates &temp_states) override;
@@ -254,6 +261,7 @@ class Conv2dHip : public BaseLayerHip {
     std::string get_layer_info() const override;
     std::string get_layer_name() const override { return "Conv2dCuda"; }
     LayerType get_layer_type() const override { return LayerType::Conv2d; }
+    bool can_fuse_activation() const override { return true; }
     void compute_input_output_size(const InitArgs &args) override;
     void get_number_param();
     void init_weight_bias() override;
@@ -299,6 +307,16 @@ class ReLUHip : public BaseLayer {
     void update_params() override {}
     std::unique_ptr<BaseLayer> to_cuda(int = 0) override;
 };
+
+// Fusion of an activation layer into the forward of the layer before it (the
+// reference runs them as two launches with a round trip through memory between
+// them). fusable_activation: TAGI_ACT_* when `next` is a device ReLU / MixtureReLU
+// that `layer` can absorb and fusion is switched on, else 0. After the fused forward
+// the owner calls activation_absorbed so that the skipped layer's sizes read as if it
+// had run. set_fused_activations(false) switches the fusion off (tests, comparisons).
+int fusable_activation(const BaseLayer *layer, const BaseLayer *next);
+void activation_absorbed(BaseLayer *activation, const BaseHiddenStates &output_states);
+void set_fused_activations(bool on);
 
 std::tuple<int, int> compute_downsample_img_size_v2(int kernel, int stride, int wi, int hi, int pad,
                                                     int pad_type);

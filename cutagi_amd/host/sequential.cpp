@@ -373,8 +373,20 @@ void Sequential::forward(const float *mu_x, const float *var_x, size_t n) {
     this->prepare_buffers(batch_size);
     auto *in = dynamic_cast<HiddenStateHip *>(this->input_z_buffer.get());
     in->set_input_raw(mu_x, var_x, n, batch_size);
-    for (auto &layer : layers) {
-        layer->forward(*input_z_buffer, *output_z_buffer, *temp_states);
+    this->forward_layers(0);
+}
+
+// Layers from `first` on, reading input_z_buffer; the network's output ends up in
+// output_z_buffer. An activation that follows a Linear / Conv2d layer runs in that
+// layer's epilogue (one launch and one pass over the tensor instead of two).
+void Sequential::forward_layers(size_t first) {
+    for (size_t i = first; i < layers.size(); i++) {
+        const int act = i + 1 < layers.size()
+                            ? fusable_activation(layers[i].get(), layers[i + 1].get())
+                            : 0;
+        layers[i]->fused_activation = act;
+        layers[i]->forward(*input_z_buffer, *output_z_buffer, *temp_states);
+        if (act != 0) activation_absorbed(layers[++i].get(), *output_z_buffer);
         std::swap(input_z_buffer, output_z_buffer);
     }
     std::swap(output_z_buffer, input_z_buffer);
@@ -384,11 +396,7 @@ void Sequential::forward(BaseHiddenStates &input_states) {
     this->require_device("forward");
     this->prepare_buffers((int)input_states.block_size);
     layers.front()->forward(input_states, *input_z_buffer, *temp_states);
-    for (size_t i = 1; i < layers.size(); i++) {
-        layers[i]->forward(*input_z_buffer, *output_z_buffer, *temp_states);
-        std::swap(input_z_buffer, output_z_buffer);
-    }
-    std::swap(output_z_buffer, input_z_buffer);
+    this->forward_layers(1);
 }
 
 // reference: src/sequential.cpp:387-411. Activations do not consume a delta

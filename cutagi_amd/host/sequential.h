@@ -120,6 +120,7 @@ class Sequential {
     void init_output_state_buffer();
     void init_delta_state_buffer();
     void prepare_buffers(int batch_size);
+    void forward_layers(size_t first);
     void require_device(const char *what) const;
 };
 

@@ -85,6 +85,19 @@ int tagi_linear_fwd(const float *mu_w, const float *var_w, const float *mu_b,
                     int K, int N, int B, int bias, float *mu_z, float *var_z,
                     void *stream);
 
+/* tagi_linear_fwd with the activation that follows the layer applied to its sums
+ * before anything is stored: mu_out / var_out / jcb_out [B][N] receive what
+ * relu_mean_var_cuda or mixture_relu_mean_var_cuda (src/activation_cuda.cu:130-150,
+ * 726-760) would write from this layer's output; the pre-activation moments are never
+ * written. Replaces the LinearCuda::forward + ReLUCuda / MixtureReLUCuda::forward
+ * pair of a Sequential (src/sequential.cpp:323-331 runs them back to back). */
+#define TAGI_ACT_RELU 1
+#define TAGI_ACT_MIXTURE_RELU 2
+int tagi_linear_fwd_act(const float *mu_w, const float *var_w, const float *mu_b,
+                        const float *var_b, const float *mu_a, const float *var_a,
+                        int K, int N, int B, int bias, int activation,
+                        float *mu_out, float *var_out, float *jcb_out, void *stream);
+
 /* tagi_linear_fwd for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc). It has no
  * counterpart in the reference. Same arguments, same kernels and bit-identical
@@ -161,6 +174,14 @@ int tagi_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
                     const int *aidx, int woho, int fo, int wihi, int fi,
                     int ki, int B, int bias, float *mu_z, float *var_z,
                     void *stream);
+
+/* tagi_conv2d_fwd with the activation that follows the layer (TAGI_ACT_*) applied
+ * before anything is stored, as tagi_linear_fwd_act: outputs [B][fo][woho]. */
+int tagi_conv2d_fwd_act(const float *mu_w, const float *var_w, const float *mu_b,
+                        const float *var_b, const float *mu_a, const float *var_a,
+                        const int *aidx, int woho, int fo, int wihi, int fi,
+                        int ki, int B, int bias, int activation, float *mu_out,
+                        float *var_out, float *jcb_out, void *stream);
 
 /* State backward through FCzwa_1 (`zw_idx`, [wihi][nr]) and Szz_ud (`zud_idx`,
  * [nr][wihi]); replaces conv2d_state_backward_cuda
