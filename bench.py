@@ -47,13 +47,19 @@ WORKLOADS = {
 # summaries, with their commands, are profiles/linear_and_conv2d_hbm_traffic_counters.md.
 MEASURED_TRAFFIC_BYTES = {
     # (workload, phase): (kernel, bytes)
-    ("gemm", "fwd"): ("mfma_tile_kernel<LinearProblem<0,...>, 64, 128, 2, 4>", 235.0e6),      # algorithmic 151.0e6
-    ("gemm", "bwd_dw"): ("linear_dw_side_kernel<LinearProblem<2,...>, 64, 128, 2, 4>", 334.0e6),  # algorithmic 213.9e6
+    ("gemm", "fwd"): ("mfma_tile_kernel<LinearProblem<0,...>, 64, 128, 2, 4>", 235.6e6),      # algorithmic 151.0e6
+    ("gemm", "bwd_dw"): ("linear_dw_side_kernel<LinearProblem<2,...>, 64, 128, 2, 4>", 333.6e6),  # algorithmic 213.9e6
     ("gemm", "bwd_dz"): ("mfma_tile_kernel<LinearProblem<1,...>, 64, 128, 2, 4>", 167.9e6),   # algorithmic 88.1e6
-    ("skinny", "fwd"): ("gemv_fwd_kernel<2, 2, 1>", 562.2e6),       # algorithmic 536.9e6
+    ("skinny", "fwd"): ("gemv_fwd_kernel<2, 2, 1>", 562.3e6),       # algorithmic 536.9e6
     ("skinny", "bwd_dz"): ("gemv_dz_kernel<2>", 286.3e6),           # algorithmic 268.4e6
     ("skinny", "bwd_dw"): ("gemv_dw_kernel<8, true>", 815.3e6),     # algorithmic 805.3e6
-    ("conv", "fwd"): ("conv_stencil_kernel<false, 32>", None),
+    ("skinny12", "bwd_dw"): ("gemv_dw_kernel<16, true>", 829.0e6),  # algorithmic 805.3e6
+    ("skinny16", "bwd_dw"): ("gemv_dw_kernel<16, true>", 829.0e6),
+    ("skinny12", "fwd"): ("gemv16_fwd_kernel", 582.1e6),            # algorithmic 536.9e6
+    ("skinny16", "fwd"): ("gemv16_fwd_kernel", 582.1e6),
+    ("skinny12", "bwd_dz"): ("gemv16_dz_kernel", 291.6e6),          # algorithmic 268.4e6
+    ("skinny16", "bwd_dz"): ("gemv16_dz_kernel", 291.6e6),
+    ("conv", "fwd"): ("conv_stencil_kernel<false, 32>", 169.2e6),   # algorithmic 134.2e6
 }
 
 # Conv2d 3x3, stride 1, pad 1, 64 -> 64 channels on 32x32 maps, batch 128, no bias
@@ -234,7 +240,8 @@ def run_conv(steps, warmup):
                 frac_of_peak=round(tflops / FP32_MFMA_PEAK_TFLOPS, 4), ms_per_step=round(ms, 5),
                 roofline=dict(bound="mfma", kernel="fwd", achieved=round(fwd_tflops, 2),
                               peak=FP32_MFMA_PEAK_TFLOPS, unit="TFLOP/s",
-                              frac=round(fwd_tflops / FP32_MFMA_PEAK_TFLOPS, 4), traffic=None,
+                              frac=round(fwd_tflops / FP32_MFMA_PEAK_TFLOPS, 4),
+                              traffic=MEASURED_TRAFFIC_BYTES[("conv", "fwd")][1],
                               traffic_kernel=MEASURED_TRAFFIC_BYTES[("conv", "fwd")][0],
                               kernel_ms=round(fwd_ms, 5)))
 
