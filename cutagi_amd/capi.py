@@ -48,6 +48,7 @@ SIGNATURES = {
     "tagi_store_states": (_i, [_vp, _vp, _sz, _vp, _vp, _vp, _sz, _vp]),
     "tagi_param_update": (_i, [_vp, _vp, _f, _sz, _vp, _vp, _vp, _vp]),
     "tagi_param_raw_update": (_i, [_vp, _vp, _sz, _vp, _vp, _vp]),
+    "tagi_model_update": (_i, [_vp, _i, _vp]),
     "tagi_layer_update": (_i, [_vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _f, _vp, _i, _vp]),
     "tagi_cap_factor": (_f, [_i, _f]),
     "tagi_out_update_dense": (_i, [_vp] * 5 + [_i] + [_vp] * 3),
@@ -64,6 +65,14 @@ SIGNATURES = {
     "tagi_add_shortcut": (_i, [_vp, _vp, _sz, _vp, _vp, _vp]),
     "tagi_add_shortcut_delta": (_i, [_vp, _vp, _vp, _sz, _vp, _vp, _vp]),
 }
+
+
+class UpdateItem(ctypes.Structure):
+    """tagi_update_item of include/tagi_hip.h."""
+    _fields_ = [("delta_mu_w", _vp), ("delta_var_w", _vp), ("mu_w", _vp), ("var_w", _vp),
+                ("num_weights", _sz), ("delta_mu_b", _vp), ("delta_var_b", _vp), ("mu_b", _vp),
+                ("var_b", _vp), ("num_biases", _sz), ("cap_factor", _f),
+                ("neg_var_count", _vp), ("slot", _i)]
 
 
 class TagiHipError(RuntimeError):

@@ -774,6 +774,42 @@ int tagi_layer_update(const float *delta_mu_w, const float *delta_var_w, size_t 
     return TAGI_OK;
 }
 
+int tagi_model_update(const tagi_update_item *items, int n_items, void *stream_) {
+    if (n_items < 0 || (n_items > 0 && items == nullptr)) return TAGI_ERR_INVALID_ARG;
+    for (int i = 0; i < n_items; i++) {
+        const tagi_update_item &t = items[i];
+        if (t.num_weights > 0 && (!t.delta_mu_w || !t.delta_var_w || !t.mu_w || !t.var_w))
+            return TAGI_ERR_INVALID_ARG;
+        if (t.num_biases > 0 && (!t.delta_mu_b || !t.delta_var_b || !t.mu_b || !t.var_b))
+            return TAGI_ERR_INVALID_ARG;
+        if (!(t.cap_factor > 0.0f) || (t.slot != 0 && t.slot != 1)) return TAGI_ERR_INVALID_ARG;
+        if ((t.num_weights + t.num_biases + 255) / 256 > 0x3fffffffu) return TAGI_ERR_UNSUPPORTED;
+    }
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    int i = 0;
+    while (i < n_items) {
+        ModelUpdateArgs a = {};
+        unsigned long long blocks = 0;
+        for (; i < n_items && a.n < MODEL_UPDATE_MAX; i++) {
+            const tagi_update_item &t = items[i];
+            const unsigned long long b = (t.num_weights + t.num_biases + 255) / 256;
+            if (b == 0) continue;
+            if (a.n > 0 && blocks + b > 0x7fffffffULL) break;  // the rest: next launch
+            const int k = a.n++;
+            a.dmu_w[k] = t.delta_mu_w; a.dvar_w[k] = t.delta_var_w;
+            a.mu_w[k] = t.mu_w; a.var_w[k] = t.var_w; a.nw[k] = t.num_weights;
+            a.dmu_b[k] = t.delta_mu_b; a.dvar_b[k] = t.delta_var_b;
+            a.mu_b[k] = t.mu_b; a.var_b[k] = t.var_b; a.nb[k] = t.num_biases;
+            a.cap[k] = t.cap_factor; a.count[k] = t.neg_var_count; a.slot[k] = t.slot;
+            a.first_block[k] = (unsigned)blocks;
+            blocks += b;
+        }
+        a.first_block[a.n] = (unsigned)blocks;
+        TAGI_TRY(launch_model_update(a, stream));
+    }
+    return TAGI_OK;
+}
+
 float tagi_cap_factor(int batch_size, float prev) {
     if (batch_size == 1) return 0.1f;
     if (batch_size > 1 && batch_size < 256) return 2.0f;

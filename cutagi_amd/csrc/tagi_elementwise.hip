@@ -135,6 +135,36 @@ __global__ __launch_bounds__(TPB) void layer_update_kernel(
     }
 }
 
+// layer_update_kernel for several layers at once: the block finds its layer in the
+// table of first blocks (uniform over the block), then does that layer's step.
+__global__ __launch_bounds__(TPB) void model_update_kernel(ModelUpdateArgs a) {
+    int it = 0;
+    while (it + 1 < a.n && blockIdx.x >= a.first_block[it + 1]) it++;
+    const size_t i = (size_t)(blockIdx.x - a.first_block[it]) * TPB + threadIdx.x;
+    const size_t nw = a.nw[it], nb = a.nb[it];
+    int *count = a.count[it];
+    const int slot = a.slot[it];
+    const float cap = a.cap[it];
+    if (i == 0 && count != nullptr) count[1 - slot] = 0;
+    bool clamped = false;
+    if (i < nw) {
+        float m = a.mu_w[it][i], v = a.var_w[it][i];
+        clamped = capped_step(a.dmu_w[it][i], a.dvar_w[it][i], cap, m, v);
+        a.mu_w[it][i] = m;
+        a.var_w[it][i] = v;
+    } else if (i < nw + nb) {
+        const size_t j = i - nw;
+        float m = a.mu_b[it][j], v = a.var_b[it][j];
+        capped_step(a.dmu_b[it][j], a.dvar_b[it][j], cap, m, v);
+        a.mu_b[it][j] = m;
+        a.var_b[it][j] = v;
+    }
+    if (count != nullptr) {
+        const unsigned long long mask = __ballot(clamped);
+        if (mask != 0ull && (threadIdx.x & 63) == 0) atomicAdd(count + slot, __popcll(mask));
+    }
+}
+
 __global__ __launch_bounds__(TPB) void out_update_dense_kernel(
     const float *__restrict__ mu_a, const float *__restrict__ var_a,
     const float *__restrict__ jcb, const float *__restrict__ obs,
@@ -267,6 +297,13 @@ hipError_t launch_layer_update(const float *dmu_w, const float *dvar_w, size_t n
     hipLaunchKernelGGL(layer_update_kernel, dim3(blocks_for(nw + nb, TPB)), dim3(TPB), 0, stream,
                        dmu_w, dvar_w, nw, mu_w, var_w, dmu_b, dvar_b, nb, mu_b, var_b, cap, count,
                        slot);
+    return hipGetLastError();
+}
+
+hipError_t launch_model_update(const ModelUpdateArgs &args, hipStream_t stream) {
+    const unsigned blocks = args.first_block[args.n];
+    if (args.n == 0 || blocks == 0) return hipSuccess;
+    hipLaunchKernelGGL(model_update_kernel, dim3(blocks), dim3(TPB), 0, stream, args);
     return hipGetLastError();
 }
 

@@ -136,6 +136,22 @@ hipError_t launch_layer_update(const float *dmu_w, const float *dvar_w, size_t n
                                float *var_w, const float *dmu_b, const float *dvar_b, size_t nb,
                                float *mu_b, float *var_b, float cap, int *count, int slot,
                                hipStream_t stream);
+// Up to MODEL_UPDATE_MAX layers per launch; block b belongs to the item whose
+// [first_block, first_block of the next) range holds it.
+constexpr int MODEL_UPDATE_MAX = 24;
+struct ModelUpdateArgs {
+    const float *dmu_w[MODEL_UPDATE_MAX], *dvar_w[MODEL_UPDATE_MAX];
+    float *mu_w[MODEL_UPDATE_MAX], *var_w[MODEL_UPDATE_MAX];
+    const float *dmu_b[MODEL_UPDATE_MAX], *dvar_b[MODEL_UPDATE_MAX];
+    float *mu_b[MODEL_UPDATE_MAX], *var_b[MODEL_UPDATE_MAX];
+    int *count[MODEL_UPDATE_MAX];
+    unsigned long long nw[MODEL_UPDATE_MAX], nb[MODEL_UPDATE_MAX];
+    float cap[MODEL_UPDATE_MAX];
+    int slot[MODEL_UPDATE_MAX];
+    unsigned first_block[MODEL_UPDATE_MAX + 1];
+    int n;
+};
+hipError_t launch_model_update(const ModelUpdateArgs &args, hipStream_t stream);
 hipError_t launch_out_update_dense(const float *mu_a, const float *var_a, const float *jcb,
                                    const float *obs, const float *var_obs, int n, float *dmu,
                                    float *dvar, hipStream_t stream);

@@ -790,6 +790,14 @@ void ResNetBlock::update_biases() {
     main_block->update_biases();
     if (shortcut) shortcut->update_biases();
 }
+void LayerBlock::collect_update_items(std::vector<tagi_update_item> &items) {
+    for (auto &layer : layers)
+        if (layer->get_layer_type() != LayerType::Activation) layer->collect_update_items(items);
+}
+void ResNetBlock::collect_update_items(std::vector<tagi_update_item> &items) {
+    main_block->collect_update_items(items);
+    if (shortcut) shortcut->collect_update_items(items);
+}
 void ResNetBlock::update_params() {
     main_block->update_params();
     if (shortcut) shortcut->update_params();

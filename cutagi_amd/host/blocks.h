@@ -175,6 +175,7 @@ class LayerBlock : public BaseLayer {
     void update_weights() override;
     void update_biases() override;
     void update_params() override;
+    void collect_update_items(std::vector<tagi_update_item> &items) override;
     void compute_input_output_size(const InitArgs &args) override;
     void save(std::ofstream &file) override;
     void load(std::ifstream &file) override;
@@ -219,6 +220,7 @@ class ResNetBlock : public BaseLayer {
     void update_weights() override;
     void update_biases() override;
     void update_params() override;
+    void collect_update_items(std::vector<tagi_update_item> &items) override;
     void save(std::ofstream &file) override;
     void load(std::ifstream &file) override;
     ParameterMap get_parameters_as_map(std::string suffix = "") override;

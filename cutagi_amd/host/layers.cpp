@@ -269,6 +269,21 @@ void BaseLayerHip::update_params() {
     neg_var_dirty = true;
 }
 
+void BaseLayerHip::collect_update_items(std::vector<tagi_update_item> &items) {
+    if (num_weights == 0 || d_mu_w == nullptr || d_delta_mu_w == nullptr) return;  // nothing to update
+    neg_var_slot = 1 - neg_var_slot;
+    tagi_update_item t = {};
+    t.delta_mu_w = d_delta_mu_w; t.delta_var_w = d_delta_var_w;
+    t.mu_w = d_mu_w; t.var_w = d_var_w; t.num_weights = num_weights;
+    t.delta_mu_b = d_delta_mu_b; t.delta_var_b = d_delta_var_b;
+    t.mu_b = d_mu_b; t.var_b = d_var_b; t.num_biases = bias ? num_biases : 0;
+    t.cap_factor = cap_factor_update;
+    t.neg_var_count = d_neg_var_count;
+    t.slot = neg_var_slot;
+    items.push_back(t);
+    neg_var_dirty = true;
+}
+
 int BaseLayerHip::get_neg_var_w_counter() {
     if (neg_var_dirty) {
         HIP_OK(hipMemcpy(&neg_var_w_counter, d_neg_var_count + neg_var_slot, sizeof(int),

@@ -13,6 +13,7 @@
 #include <tuple>
 #include <vector>
 
+#include "../../include/tagi_hip.h"
 #include "states.h"
 
 namespace tagi_host {
@@ -106,6 +107,10 @@ class BaseLayer {
         this->update_weights();
         this->update_biases();
     }
+    // For Sequential::step: a device layer appends what one tagi_layer_update call
+    // would take, so that the whole model is updated in one launch; a layer that
+    // cannot describe its update that way performs it on the spot.
+    virtual void collect_update_items(std::vector<tagi_update_item> &) { this->update_params(); }
     virtual void set_cap_factor_udapte(int batch_size);
     virtual void set_threads(int num) { num_threads = num; }
     virtual void compute_input_output_size(const InitArgs &args);
@@ -158,6 +163,7 @@ class BaseLayerHip : public BaseLayer {
     void update_weights() override;
     void update_biases() override;
     void update_params() override;
+    void collect_update_items(std::vector<tagi_update_item> &items) override;
     void raw_update_weights() override;
     void raw_update_biases() override;
     void set_cuda_threads(int num) { num_cuda_threads = (unsigned int)num; }

@@ -415,10 +415,15 @@ void Sequential::backward() {
 
 void Sequential::step() {
     this->require_device("step");
+    // update_weights + update_biases of every layer (reference: src/sequential.cpp:
+    // 440-448), gathered into one launch per 24 layers
+    std::vector<tagi_update_item> items;
     for (auto &layer : layers) {
         if (layer->get_layer_type() == LayerType::Activation) continue;
-        layer->update_params();  // update_weights + update_biases, one launch on the device
+        layer->collect_update_items(items);
     }
+    if (!items.empty())
+        TAGI_OK_OR_THROW(tagi_model_update(items.data(), (int)items.size(), nullptr));
 }
 
 std::string Sequential::get_layer_stack_info() const {

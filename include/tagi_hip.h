@@ -244,6 +244,24 @@ int tagi_layer_update(const float *delta_mu_w, const float *delta_var_w,
                       float cap_factor, int *neg_var_count, int slot,
                       void *stream);
 
+/* tagi_layer_update for every layer of a model in as few launches as the kernel
+ * argument space allows (24 layers per launch), as Sequential::step walks its layers
+ * (src/sequential.cpp:440-448): item i carries the arguments of one
+ * tagi_layer_update call. `items` is a host array, read before the call returns. */
+typedef struct tagi_update_item {
+    const float *delta_mu_w, *delta_var_w;
+    float *mu_w, *var_w;
+    size_t num_weights;
+    const float *delta_mu_b, *delta_var_b;
+    float *mu_b, *var_b;
+    size_t num_biases;
+    float cap_factor;
+    int *neg_var_count;
+    int slot;
+} tagi_update_item;
+int tagi_model_update(const tagi_update_item *items /* host */, int n_items,
+                      void *stream);
+
 /* Cap factor for a batch size (src/base_layer.cpp:164-187); `prev` is returned
  * for batch sizes below 1. Host only. */
 float tagi_cap_factor(int batch_size, float prev);

@@ -156,3 +156,48 @@ def test_relu_and_store_states(oracle_lib):
     assert torch.equal(bm[:3000], mu_a[:3000]) and float(bm[3000:].abs().max()) == 0.0
     assert torch.equal(bj[:3000], jcb[:3000])
     assert float(oj[:7000].min()) == 1.0 and float(oj[7000:].max()) == 0.0
+
+
+def test_model_update_matches_layer_updates(oracle_lib):
+    """tagi_model_update (all layers of a model in one launch per 24) against the
+    oracle's capped step, layer by layer, counters included; 30 layers make two
+    launches, one layer has no biases and one is empty."""
+    import ctypes
+    import torch
+    from cutagi_amd import capi
+    rng = np.random.default_rng(21)
+    sizes = [(int(rng.integers(1, 5000)), int(rng.integers(0, 200))) for _ in range(30)]
+    sizes[3] = (70000, 0)
+    sizes[7] = (0, 0)
+    items = (capi.UpdateItem * len(sizes))()
+    keep, want = [], []
+    for i, (nw, nb) in enumerate(sizes):
+        cap = [0.1, 2.0, 3.0][i % 3]
+        host = [rng.normal(0, 1, nw).astype(np.float32), rng.uniform(1e-4, 1, nw).astype(np.float32),
+                rng.normal(0, 1, nw).astype(np.float32), rng.normal(0, 0.5, nw).astype(np.float32),
+                rng.normal(0, 1, nb).astype(np.float32), rng.uniform(1e-4, 1, nb).astype(np.float32),
+                rng.normal(0, 1, nb).astype(np.float32), rng.normal(0, 0.5, nb).astype(np.float32)]
+        dev = [_t(a) for a in host]
+        cnt = torch.tensor([5, 7], dtype=torch.int32, device="cuda")   # what earlier steps left
+        slot = i % 2
+        keep.append((dev, cnt, slot))
+        mw, vw, c = oracle_lib.param_update(host[0], host[1], host[2], host[3], cap, True)
+        mb, vb, _ = oracle_lib.param_update(host[4], host[5], host[6], host[7], cap, False)
+        want.append((mw, vw, mb, vb, c))
+        it = items[i]
+        it.mu_w, it.var_w, it.delta_mu_w, it.delta_var_w = (capi.ptr(dev[k]) if nw else None for k in range(4))
+        it.mu_b, it.var_b, it.delta_mu_b, it.delta_var_b = (capi.ptr(dev[k]) if nb else None for k in range(4, 8))
+        it.num_weights, it.num_biases, it.cap_factor = nw, nb, cap
+        it.neg_var_count, it.slot = capi.ptr(cnt), slot
+    capi.check(capi.lib.tagi_model_update(ctypes.cast(items, ctypes.c_void_p), len(sizes), None))
+    torch.cuda.synchronize()
+    for i, ((dev, cnt, slot), (mw, vw, mb, vb, c)) in enumerate(zip(keep, want)):
+        np.testing.assert_allclose(dev[0].cpu().numpy(), mw, rtol=1e-6, atol=1e-7)
+        np.testing.assert_allclose(dev[1].cpu().numpy(), vw, rtol=1e-6, atol=1e-7)
+        np.testing.assert_allclose(dev[4].cpu().numpy(), mb, rtol=1e-6, atol=1e-7)
+        np.testing.assert_allclose(dev[5].cpu().numpy(), vb, rtol=1e-6, atol=1e-7)
+        got = cnt.tolist()
+        if sizes[i] == (0, 0):
+            assert got == [5, 7]                       # an empty layer launches nothing
+        else:
+            assert got[slot] == [5, 7][slot] + c and got[1 - slot] == 0, (i, got, c)
