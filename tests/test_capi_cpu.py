@@ -53,6 +53,40 @@ def test_null_and_bad_sizes_are_rejected_before_any_launch():
         capi.check(capi.ERR_INVALID_ARG)
 
 
+def test_newer_entry_points_reject_bad_arguments_before_any_launch():
+    import ctypes
+    from cutagi_amd import capi
+    L = capi.lib
+    one = ctypes.c_void_p(16)  # never dereferenced: the checks fire first
+    # fused activation: only ReLU (1) and MixtureReLU (2); the Jacobian output is required
+    assert L.tagi_linear_fwd_act(one, one, one, one, one, one, 4, 4, 4, 1, 0, one, one, one,
+                                 None) == capi.ERR_INVALID_ARG
+    assert L.tagi_linear_fwd_act(one, one, one, one, one, one, 4, 4, 4, 1, 3, one, one, one,
+                                 None) == capi.ERR_INVALID_ARG
+    assert L.tagi_linear_fwd_act(one, one, one, one, one, one, 4, 4, 4, 1, 1, one, one, None,
+                                 None) == capi.ERR_INVALID_ARG
+    assert L.tagi_conv2d_fwd_act(one, one, one, one, one, one, one, 4, 4, 4, 4, 3, 2, 1, 7, one,
+                                 one, one, None) == capi.ERR_INVALID_ARG
+    # heteroscedastic update: negative count, null arrays, arrays that are not 8-byte aligned
+    assert L.tagi_out_update_heteros(one, one, one, one, -1, one, one, None) == capi.ERR_INVALID_ARG
+    assert L.tagi_out_update_heteros(None, one, one, one, 4, one, one, None) == capi.ERR_INVALID_ARG
+    odd = ctypes.c_void_p(20)
+    assert L.tagi_out_update_heteros(odd, one, one, one, 4, one, one, None) == capi.ERR_INVALID_ARG
+    assert L.tagi_param_raw_update(None, one, 4, one, one, None) == capi.ERR_INVALID_ARG
+    # model update: a null table, a layer with weights announced and none given, a bad slot
+    assert L.tagi_model_update(None, 2, None) == capi.ERR_INVALID_ARG
+    assert L.tagi_model_update(None, 0, None) == capi.OK
+    items = (capi.UpdateItem * 1)()
+    items[0].num_weights, items[0].cap_factor, items[0].slot = 8, 2.0, 0
+    assert L.tagi_model_update(ctypes.cast(items, ctypes.c_void_p), 1, None) == capi.ERR_INVALID_ARG
+    for name in ("delta_mu_w", "delta_var_w", "mu_w", "var_w"):
+        setattr(items[0], name, 16)
+    items[0].slot = 2
+    assert L.tagi_model_update(ctypes.cast(items, ctypes.c_void_p), 1, None) == capi.ERR_INVALID_ARG
+    items[0].slot, items[0].cap_factor = 0, 0.0
+    assert L.tagi_model_update(ctypes.cast(items, ctypes.c_void_p), 1, None) == capi.ERR_INVALID_ARG
+
+
 def test_host_only_entry_points(oracle_lib):
     from cutagi_amd import capi
     for b in (-1, 0, 1, 2, 255, 256, 5000):
