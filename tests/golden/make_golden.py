@@ -104,6 +104,7 @@ def model_vectors(ref):
                           c.get("input_state_update", False), c.get("eval_forward", False),
                           8 if c.get("big") else REF_THREADS)
         assert r["n_out"] == inp["n_out"]
+        assert np.all(np.isfinite(r["params"])) and np.all(np.isfinite(r["out_mu"])), name
         out[name + "_out_mu"], out[name + "_out_var"] = r["out_mu"], r["out_var"]
         if c.get("input_state_update", False):
             out[name + "_in_dmu"], out[name + "_in_dvar"] = r["in_dmu"], r["in_dvar"]

@@ -377,3 +377,94 @@ def resnet18_spec():
 # tests that re-run a case through the emulator (tens of seconds there).
 CASES["resnet18_cifar_batch8"] = dict(spec=resnet18_spec(), B=8, steps=1, update=1, n_enc=4,
                                       var_x=False, seed=18, big=True)
+
+
+def random_spec(rng):
+    """A random small convolutional network as a description, with the image size
+    and channel count tracked so that every layer fits: convolutions (3x3 same, 3x3
+    stride 2 with one-sided padding, 2x2 stride 2, 1x1), activations, BatchNorm2d,
+    identity and projection ResNetBlocks, LayerBlocks, average pooling, a Linear head.
+    Returns (description, number of outputs)."""
+    w = int(rng.choice([6, 8, 10, 12]))
+    c = int(rng.integers(1, 4))
+    first_w, first_c = w, c
+    act = lambda: str(rng.choice(["ReLU", "MixtureReLU"]))
+    bn = lambda ch: "BatchNorm2d %d 1e-5 0.9 %d" % (ch, int(rng.integers(0, 2)))
+
+    def conv(ci, co, kind, size=0):
+        k, s, p, pt = {"same": (3, 1, 1, 1), "down3": (3, 2, 1, 2), "down2": (2, 2, 0, 1),
+                       "one": (1, 1, 0, 1)}[kind]
+        return "Conv2d %d %d %d %d %d %d %d %d %d" % (ci, co, k, int(rng.integers(0, 2)), s, p, pt,
+                                                     size, size)
+
+    parts = []
+    n_units = int(rng.integers(2, 5))
+    for u in range(n_units):
+        size = first_w if u == 0 else 0       # only the first convolution names its input size
+        kinds = ["conv", "conv", "identity", "layerblock"]
+        if w % 2 == 0 and w >= 4:
+            kinds += ["projection", "pool", "convdown"]
+        kind = str(rng.choice(kinds))
+        if kind == "conv":
+            co = int(rng.integers(2, 9))
+            parts.append(conv(c, co, str(rng.choice(["same", "one"])), size))
+            if rng.random() < 0.8:
+                parts.append(act())
+            if rng.random() < 0.5:
+                parts.append(bn(co))
+            c = co
+        elif kind == "convdown":
+            co = int(rng.integers(2, 9))
+            parts.append(conv(c, co, str(rng.choice(["down3", "down2"])), size))
+            parts.append(act())
+            c, w = co, w // 2
+        elif kind == "identity":
+            main = [conv(c, c, "same", size), act(), bn(c), conv(c, c, "same")]
+            if rng.random() < 0.5:
+                main += [act(), bn(c)]
+            parts.append("ResNetBlock [ " + " ".join(main) + " ] [ ]")
+        elif kind == "projection":
+            co = int(rng.integers(2, 9))
+            main = [conv(c, co, "down3", size), act(), bn(co), conv(co, co, "same"), act(), bn(co)]
+            short = [conv(c, co, "down2", size), act(), bn(co)]
+            parts.append("ResNetBlock [ " + " ".join(main) + " ] [ " + " ".join(short) + " ]")
+            c, w = co, w // 2
+        elif kind == "layerblock":
+            co = int(rng.integers(2, 7))
+            parts.append("LayerBlock [ " + " ".join([conv(c, co, "same", size), act(),
+                                                     conv(co, co, "one")]) + " ]")
+            c = co
+        else:  # pool
+            if u == 0:      # a pooling layer cannot open the network: put a convolution first
+                parts.append(conv(c, c, "same", size))
+            parts.append("AvgPool2d 2 2 0 0")
+            w //= 2
+    if rng.random() < 0.5 and w > 1:
+        parts.append("AvgPool2d %d -1 0 0" % w)
+        w = 1
+    if rng.random() < 0.5 and not parts[-1].endswith("ReLU"):   # (never two activations in a row:
+        parts.append(act())                                      # MixtureReLU of a zero variance is 0/0)
+    n_out = int(rng.integers(2, 8))
+    parts.append("Linear %d %d 1" % (c * w * w, n_out))
+    spec = " ".join(parts)
+    if spec.startswith(("ResNetBlock", "LayerBlock")):
+        spec = "input %d %d %d " % (first_w, first_w, first_c) + spec
+    return spec, n_out
+
+
+def _random_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    out = {}
+    for i in range(n):
+        spec, n_out = random_spec(rng)
+        indexed = n_out >= 3 and rng.random() < 0.4
+        out["random_%02d" % i] = dict(spec=spec, B=int(rng.integers(2, 6)), steps=2,
+                                      update=1 if indexed else 0, n_enc=min(3, n_out),
+                                      var_x=bool(rng.random() < 0.5),
+                                      input_state_update=bool(rng.random() < 0.5),
+                                      seed=300 + i)
+    return out
+
+
+# sixteen networks nobody designed by hand
+CASES.update(_random_cases(16, seed=4242))
