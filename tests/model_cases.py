@@ -466,5 +466,9 @@ def _random_cases(n, seed):
     return out
 
 
+# BatchNorm2d behind a fully-connected layer (one "pixel" per feature)
+CASES["mlp_batchnorm"] = dict(spec="Linear 10 8 1 BatchNorm2d 8 1e-5 0.9 1 ReLU Linear 8 3 1", B=5,
+                              steps=2, update=0, var_x=True, input_state_update=True, seed=19)
+
 # sixteen networks nobody designed by hand
 CASES.update(_random_cases(16, seed=4242))
