@@ -196,7 +196,12 @@ template <int MODE>
 hipError_t launch_mode(int tile, bool vec, const GemmParams &p, hipStream_t stream) {
     const bool full = vec && p.R % KT == 0 && (p.splits == 1 || p.r_per_split % KT == 0) &&
                       p.M >= 4 && p.N >= 4;
-    if (full && g_gemm_double_buffer != 0)
+    // The two-stage loop pays one memory round trip per 16 reduction elements when
+    // nothing else runs on the CU to hide it: launches that leave most of the chip
+    // empty (the layers of a small MLP) keep the single stage of 32.
+    const int tiles = ((p.M + tile_rows(tile) - 1) / tile_rows(tile)) *
+                      ((p.N + tile_cols(tile) - 1) / tile_cols(tile));
+    if (full && g_gemm_double_buffer != 0 && tiles * p.splits >= num_cu())
         return launch_tiles<LinearProblem<MODE, true, true, true>>(tile, p, stream);
     if (full) return launch_tiles<LinearProblem<MODE, true, true>>(tile, p, stream);
     if (vec) return launch_tiles<LinearProblem<MODE, true>>(tile, p, stream);
@@ -336,7 +341,9 @@ hipError_t launch_gemm_dw_side(const GemmParams &p, LinearSideWork w, hipStream_
     w.side_wgs = (w.bias_wgs + fold_wgs + 7) / 8 * 8;
     if (w.ws0 == nullptr) w.fold_total = 0;  // the padding workgroups find nothing to fold
     const bool full = p.R % KT == 0 && p.M >= 4 && p.N >= 4;
-    if (full && g_gemm_double_buffer != 0) return launch_dw_side<true, true>(p, w, stream);
+    const int tiles = ((p.M + 63) / 64) * ((p.N + 127) / 128);
+    if (full && g_gemm_double_buffer != 0 && tiles >= num_cu())
+        return launch_dw_side<true, true>(p, w, stream);
     return full ? launch_dw_side<true>(p, w, stream) : launch_dw_side<false>(p, w, stream);
 }
 
