@@ -49,6 +49,14 @@ class StagingRing {
     static constexpr int SLOTS = 8;
     // queues dst[0..bytes) = src[0..bytes) on the null stream of the current device
     void upload(void *dst, const void *src, size_t bytes) {
+        const void *parts[1] = {src};
+        const size_t sizes[1] = {bytes};
+        this->upload_parts(dst, parts, sizes, 1);
+    }
+    // the same for several host pieces that lie back to back on the device: one transfer
+    void upload_parts(void *dst, const void *const *parts, const size_t *sizes, int n) {
+        size_t bytes = 0;
+        for (int i = 0; i < n; i++) bytes += sizes[i];
         if (bytes == 0) return;
         Slot &s = slots_[next_];
         next_ = (next_ + 1) % SLOTS;
@@ -59,7 +67,11 @@ class StagingRing {
             s.cap = std::max(bytes, (size_t)1 << 16);
             HIP_OK(hipHostMalloc(&s.host, s.cap, hipHostMallocDefault));
         }
-        std::memcpy(s.host, src, bytes);
+        size_t at = 0;
+        for (int i = 0; i < n; i++) {
+            if (sizes[i]) std::memcpy(static_cast<char *>(s.host) + at, parts[i], sizes[i]);
+            at += sizes[i];
+        }
         HIP_OK(hipMemcpyAsync(dst, s.host, bytes, hipMemcpyHostToDevice, nullptr));
         HIP_OK(hipEventRecord(s.event, nullptr));
         s.used = true;
@@ -326,15 +338,17 @@ DeltaStateHip::DeltaStateHip(size_t n, size_t m, int device_idx) : BaseDeltaStat
     this->allocate_memory();
 }
 DeltaStateHip::~DeltaStateHip() { this->deallocate_memory(); }
+// The two arrays are one allocation (variance right after the mean), so that
+// reset_zeros is one launch; swap() exchanges both pointers, which keeps pairs together.
 void DeltaStateHip::allocate_memory() {
     this->deallocate_memory();
-    d_delta_mu = dev_alloc(size, device_idx);
-    d_delta_var = dev_alloc(size, device_idx);
+    d_delta_mu = dev_alloc(2 * size, device_idx);
+    d_delta_var = d_delta_mu != nullptr ? d_delta_mu + size : nullptr;
     this->to_device();
 }
 void DeltaStateHip::deallocate_memory() {
     dev_free(d_delta_mu);
-    dev_free(d_delta_var);
+    d_delta_var = nullptr;
 }
 void DeltaStateHip::to_device() {
     h2d(d_delta_mu, delta_mu.data(), size);
@@ -346,8 +360,7 @@ void DeltaStateHip::to_host() {
 }
 void DeltaStateHip::reset_zeros() {
     if (size == 0) return;
-    HIP_OK(hipMemsetAsync(d_delta_mu, 0, size * sizeof(float), nullptr));
-    HIP_OK(hipMemsetAsync(d_delta_var, 0, size * sizeof(float), nullptr));
+    HIP_OK(hipMemsetAsync(d_delta_mu, 0, 2 * size * sizeof(float), nullptr));
 }
 void DeltaStateHip::copy_from(const BaseDeltaStates &source, int num_data) {
     auto *s = dynamic_cast<const DeltaStateHip *>(&source);
@@ -434,35 +447,34 @@ void BackwardStateHip::set_size(size_t new_size) {
     }
 }
 
-ObservationHip::~ObservationHip() {
-    dev_free(d_mu_obs);
-    dev_free(d_var_obs);
-    if (d_selected_idx != nullptr) (void)hipFree(d_selected_idx);
-}
+// Observations, their variances and the selected indices live in one device block,
+// back to back in that order, so that a batch's observations are one transfer.
+ObservationHip::~ObservationHip() { dev_free(d_mu_obs); }
 void ObservationHip::reserve(size_t n, size_t ni) {
-    if (n > cap_obs) {
+    const size_t words = 2 * n + ni;  // floats and ints are both four bytes
+    if (words > cap_obs) {
         HIP_OK(hipDeviceSynchronize());
         dev_free(d_mu_obs);
-        dev_free(d_var_obs);
-        d_mu_obs = dev_alloc(n, device_idx);
-        d_var_obs = dev_alloc(n, device_idx);
-        cap_obs = n;
+        d_mu_obs = dev_alloc(words, device_idx);
+        cap_obs = words;
     }
-    if (ni > cap_idx) {
-        HIP_OK(hipDeviceSynchronize());
-        if (d_selected_idx != nullptr) (void)hipFree(d_selected_idx);
-        HIP_OK(hipMalloc(reinterpret_cast<void **>(&d_selected_idx), ni * sizeof(int)));
-        cap_idx = ni;
-    }
+    cap_idx = ni;
+    d_var_obs = d_mu_obs + n;
+    d_selected_idx = reinterpret_cast<int *>(d_mu_obs + 2 * n);
 }
 void ObservationHip::upload(const float *mu, const float *var, size_t n, const int *idx,
                             size_t ni) {
     HIP_OK(hipSetDevice(device_idx));
     this->reserve(n, ni);
     StagingRing &ring = staging_ring(device_idx);
-    ring.upload(d_mu_obs, mu, n * sizeof(float));
-    if (var != nullptr) ring.upload(d_var_obs, var, n * sizeof(float));
-    if (ni) ring.upload(d_selected_idx, idx, ni * sizeof(int));
+    if (var != nullptr) {
+        const void *parts[3] = {mu, var, idx};
+        const size_t sizes[3] = {n * sizeof(float), n * sizeof(float), ni * sizeof(int)};
+        ring.upload_parts(d_mu_obs, parts, sizes, 3);
+    } else {
+        ring.upload(d_mu_obs, mu, n * sizeof(float));
+        if (ni) ring.upload(d_selected_idx, idx, ni * sizeof(int));
+    }
 }
 void ObservationHip::to_device() {
     this->upload(mu_obs.data(), var_obs.data(), mu_obs.size(), selected_idx.data(),
