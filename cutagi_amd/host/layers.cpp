@@ -421,6 +421,9 @@ void LinearHip::init_weight_bias() {
 // reference: LinearCuda::forward, src/linear_layer_cuda.cu:231-271
 void LinearHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &output_states,
                         BaseTempStates &) {
+    // (the one-shot request is taken before anything can throw)
+    const int act = this->fused_activation;
+    this->fused_activation = 0;
     auto *in = as<HiddenStateHip>(input_states);
     auto *out = as<HiddenStateHip>(output_states);
     const int batch_size = (int)input_states.block_size;
@@ -432,8 +435,6 @@ void LinearHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &output
         LOG(LogLevel::ERROR, "Output state buffer too small for " + this->get_layer_info());
     if (d_mu_w == nullptr) LOG(LogLevel::ERROR, "Parameters of " + get_layer_info() + " are not on the device");
 
-    const int act = this->fused_activation;
-    this->fused_activation = 0;
     if (act != 0)
         TAGI_OK_OR_THROW(tagi_linear_fwd_act(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a,
                                              in->d_var_a, (int)input_size, (int)output_size,
@@ -619,6 +620,8 @@ void Conv2dHip::preinit_layer() {
 // reference: Conv2dCuda::forward, src/conv2d_layer_cuda.cu:387-451
 void Conv2dHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &output_states,
                         BaseTempStates &) {
+    const int act = this->fused_activation;  // one-shot: taken before anything can throw
+    this->fused_activation = 0;
     auto *in = as<HiddenStateHip>(input_states);
     auto *out = as<HiddenStateHip>(output_states);
     if (this->input_size != input_states.actual_size)
@@ -642,8 +645,6 @@ void Conv2dHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &output
     output_states.actual_size = output_size;
 
     const int woho = (int)(out_width * out_height), wihi = (int)(in_width * in_height);
-    const int act = this->fused_activation;
-    this->fused_activation = 0;
     if (act != 0)
         TAGI_OK_OR_THROW(tagi_conv2d_fwd_act(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a,
                                              in->d_var_a, d_idx_mwa_2, woho, (int)out_channels,
