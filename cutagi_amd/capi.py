@@ -58,6 +58,7 @@ SIGNATURES = {
     "tagi_mixture_relu_fwd": (_i, [_vp, _vp, _sz, _vp, _vp, _vp, _vp]),
     "tagi_batchnorm2d_stats": (_i, [_vp, _vp, _i, _i, _i, _f] + [_vp] * 5),
     "tagi_batchnorm2d_fwd": (_i, [_vp] * 8 + [_i, _f, _i, _i, _i] + [_vp] * 3),
+    "tagi_batchnorm2d_fwd_res": (_i, [_vp] * 10 + [_i, _f, _i, _i, _i] + [_vp] * 3),
     "tagi_batchnorm2d_bwd": (_i, [_vp] * 9 + [_f] + [_i] * 6 + [_vp] * 7),
     "tagi_avgpool2d_build_idx": (_i, [_i] * 6 + [_ip] * 5),
     "tagi_avgpool2d_fwd": (_i, [_vp] * 3 + [_i] * 4 + [_vp] * 3),

@@ -905,18 +905,37 @@ int tagi_batchnorm2d_stats(const float *mu_a, const float *var_a, int wihi, int 
     return TAGI_OK;
 }
 
-int tagi_batchnorm2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
+static int batchnorm2d_fwd_impl(const float *mu_w, const float *var_w, const float *mu_b,
                          const float *var_b, const float *mu_a, const float *var_a,
                          const float *mu_norm, const float *var_norm, int bias, float epsilon,
-                         int wihi, int fi, int B, float *mu_z, float *var_z, void *stream) {
+                         int wihi, int fi, int B, float *mu_z, float *var_z, void *stream,
+                               const float *mu_res, const float *var_res) {
     if (!mu_w || !var_w || !mu_a || !var_a || !mu_norm || !var_norm || !mu_z || !var_z)
         return TAGI_ERR_INVALID_ARG;
     if (bias && (!mu_b || !var_b)) return TAGI_ERR_INVALID_ARG;
     if (!bn_sizes_ok(wihi, fi, B)) return TAGI_ERR_INVALID_ARG;
     TAGI_TRY(launch_batchnorm2d_fwd(mu_w, var_w, bias ? mu_b : nullptr, bias ? var_b : nullptr,
                                     mu_a, var_a, mu_norm, var_norm, epsilon, wihi, fi, B, mu_z,
-                                    var_z, static_cast<hipStream_t>(stream)));
+                                    var_z, static_cast<hipStream_t>(stream), mu_res, var_res));
     return TAGI_OK;
+}
+
+int tagi_batchnorm2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
+                         const float *var_b, const float *mu_a, const float *var_a,
+                         const float *mu_norm, const float *var_norm, int bias, float epsilon,
+                         int wihi, int fi, int B, float *mu_z, float *var_z, void *stream) {
+    return batchnorm2d_fwd_impl(mu_w, var_w, mu_b, var_b, mu_a, var_a, mu_norm, var_norm, bias,
+                                epsilon, wihi, fi, B, mu_z, var_z, stream, nullptr, nullptr);
+}
+
+int tagi_batchnorm2d_fwd_res(const float *mu_w, const float *var_w, const float *mu_b,
+                             const float *var_b, const float *mu_a, const float *var_a,
+                             const float *mu_norm, const float *var_norm, const float *mu_res,
+                             const float *var_res, int bias, float epsilon, int wihi, int fi,
+                             int B, float *mu_z, float *var_z, void *stream) {
+    if (!mu_res || !var_res) return TAGI_ERR_INVALID_ARG;
+    return batchnorm2d_fwd_impl(mu_w, var_w, mu_b, var_b, mu_a, var_a, mu_norm, var_norm, bias,
+                                epsilon, wihi, fi, B, mu_z, var_z, stream, mu_res, var_res);
 }
 
 int tagi_batchnorm2d_bwd(const float *mu_w, const float *var_w, const float *var_b,

@@ -177,7 +177,8 @@ hipError_t launch_batchnorm2d_fwd(const float *mu_w, const float *var_w, const f
                                   const float *var_b, const float *mu_a, const float *var_a,
                                   const float *mu_norm, const float *var_norm, float epsilon,
                                   int wihi, int fi, int B, float *mu_z, float *var_z,
-                                  hipStream_t stream);
+                                  hipStream_t stream, const float *mu_res = nullptr,
+                                  const float *var_res = nullptr);
 hipError_t launch_batchnorm2d_bwd(const float *mu_w, const float *var_w, const float *var_b,
                                   const float *mu_a, const float *jcb, const float *mu_norm,
                                   const float *var_norm, const float *dmu_out,

@@ -129,7 +129,8 @@ __global__ __launch_bounds__(TPB) void bn_fwd_kernel(
     const float *__restrict__ mu_b, const float *__restrict__ var_b,
     const float *__restrict__ mu_a, const float *__restrict__ var_a,
     const float *__restrict__ mu_norm, const float *__restrict__ var_norm, float epsilon,
-    int wihi, int fi, size_t n, float *__restrict__ mu_z, float *__restrict__ var_z) {
+    int wihi, int fi, size_t n, const float *__restrict__ mu_res,
+    const float *__restrict__ var_res, float *__restrict__ mu_z, float *__restrict__ var_z) {
     const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
     if (i >= n) return;
     const int c = (int)((i / wihi) % fi);
@@ -141,6 +142,10 @@ __global__ __launch_bounds__(TPB) void bn_fwd_kernel(
     if (mu_b != nullptr) {
         mz += mu_b[c];
         vz += var_b[c];
+    }
+    if (mu_res != nullptr) {  // the residual connection that ends on this layer
+        mz += mu_res[i];
+        vz += var_res[i];
     }
     mu_z[i] = mz;
     var_z[i] = vz;
@@ -332,11 +337,11 @@ hipError_t launch_batchnorm2d_fwd(const float *mu_w, const float *var_w, const f
                                   const float *var_b, const float *mu_a, const float *var_a,
                                   const float *mu_norm, const float *var_norm, float epsilon,
                                   int wihi, int fi, int B, float *mu_z, float *var_z,
-                                  hipStream_t stream) {
+                                  hipStream_t stream, const float *mu_res, const float *var_res) {
     const size_t n = (size_t)B * fi * wihi;
     hipLaunchKernelGGL(bn_fwd_kernel, dim3(blocks_for(n, TPB)), dim3(TPB), 0, stream, mu_w, var_w,
-                       mu_b, var_b, mu_a, var_a, mu_norm, var_norm, epsilon, wihi, fi, n, mu_z,
-                       var_z);
+                       mu_b, var_b, mu_a, var_a, mu_norm, var_norm, epsilon, wihi, fi, n, mu_res,
+                       var_res, mu_z, var_z);
     return hipGetLastError();
 }
 

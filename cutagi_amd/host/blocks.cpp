@@ -209,6 +209,9 @@ static void append_norm_stats(BaseLayer::NormStats &to, const BaseLayer::NormSta
 // device path and its default (multi-threaded) host path.
 void BatchNorm2dHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &output_states,
                              BaseTempStates &) {
+    // (the one-shot residual request is taken before anything can throw)
+    const float *res_mu = this->residual_mu, *res_var = this->residual_var;
+    this->residual_mu = this->residual_var = nullptr;
     auto *in = as<HiddenStateHip>(input_states);
     auto *out = as<HiddenStateHip>(output_states);
     const int batch_size = (int)input_states.block_size;
@@ -244,9 +247,16 @@ void BatchNorm2dHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &o
     }
     const float *mu_target = this->training ? d_mu_norm_batch : d_mu_ra;
     const float *var_target = this->training ? d_var_norm_batch : d_var_ra;
-    TAGI_OK_OR_THROW(tagi_batchnorm2d_fwd(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a, in->d_var_a,
-                                          mu_target, var_target, bias ? 1 : 0, epsilon, wihi, fi,
-                                          batch_size, out->d_mu_a, out->d_var_a, nullptr));
+    if (res_mu != nullptr)
+        TAGI_OK_OR_THROW(tagi_batchnorm2d_fwd_res(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a,
+                                                  in->d_var_a, mu_target, var_target, res_mu,
+                                                  res_var, bias ? 1 : 0, epsilon, wihi, fi,
+                                                  batch_size, out->d_mu_a, out->d_var_a, nullptr));
+    else
+        TAGI_OK_OR_THROW(tagi_batchnorm2d_fwd(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a,
+                                              in->d_var_a, mu_target, var_target, bias ? 1 : 0,
+                                              epsilon, wihi, fi, batch_size, out->d_mu_a,
+                                              out->d_var_a, nullptr));
     out->jcb_ones = true;
     if (this->training) this->store_states_for_training_hip(*in, *out);
 }
@@ -738,10 +748,9 @@ void ResNetBlock::forward(BaseHiddenStates &input_states, BaseHiddenStates &outp
     // the identity shortcut's backward needs (the reference copies mu_a and jcb
     // once more into the block's bwd_states: two transfers per block saved here)
     input_z->copy_from(input_states, (int)(this->input_size * batch_size));
-    main_block->forward(input_states, output_states, temp_states);
-
-    auto *out = as<HiddenStateHip>(output_states);
-    const size_t num_states = output_states.block_size * this->output_size;
+    // The shortcut runs first (it reads the copy), so that a main block that ends on a
+    // BatchNorm2d layer can add the shortcut's output in that layer's pass instead of
+    // in a pass of its own.
     HiddenStateHip *sc = nullptr;
     if (shortcut) {
         shortcut->forward(*input_z, *shortcut_output_z, temp_states);
@@ -749,8 +758,21 @@ void ResNetBlock::forward(BaseHiddenStates &input_states, BaseHiddenStates &outp
     } else {
         sc = as<HiddenStateHip>(*input_z);
     }
-    TAGI_OK_OR_THROW(tagi_add_shortcut(sc->d_mu_a, sc->d_var_a, num_states, out->d_mu_a,
-                                       out->d_var_a, nullptr));
+    BatchNorm2dHip *closing = nullptr;
+    if (auto *block = dynamic_cast<LayerBlock *>(main_block.get()))
+        if (!block->layers.empty())
+            closing = dynamic_cast<BatchNorm2dHip *>(block->layers.back().get());
+    if (closing != nullptr) {
+        closing->residual_mu = sc->d_mu_a;
+        closing->residual_var = sc->d_var_a;
+    }
+    main_block->forward(input_states, output_states, temp_states);
+
+    auto *out = as<HiddenStateHip>(output_states);
+    const size_t num_states = output_states.block_size * this->output_size;
+    if (closing == nullptr)
+        TAGI_OK_OR_THROW(tagi_add_shortcut(sc->d_mu_a, sc->d_var_a, num_states, out->d_mu_a,
+                                           out->d_var_a, nullptr));
     set_output_dims(output_states, *this, batch_size);
     out->jcb_ones = true;  // the block's output Jacobian is one: marked, not written
 }

@@ -75,6 +75,9 @@ class BatchNorm2dHip : public BaseLayerHip {
     float *d_mu_ra = nullptr, *d_var_ra = nullptr;
     float *d_mu_norm_batch = nullptr, *d_var_norm_batch = nullptr;
     float epsilon, momentum, gain_w, gain_b;
+    // One-shot, set by a ResNetBlock whose main block ends on this layer: the next
+    // forward() adds these arrays (the shortcut's output) to its own output.
+    const float *residual_mu = nullptr, *residual_var = nullptr;
 
     BatchNorm2dHip(int num_features, float eps = 1e-5f, float momentum = 0.9f, bool bias = true,
                    float gain_weight = 1.0f, float gain_bias = 1.0f, int device_idx = 0);

@@ -338,6 +338,19 @@ int tagi_batchnorm2d_fwd(const float *mu_w, const float *var_w,
                          float epsilon, int wihi, int fi, int B, float *mu_z,
                          float *var_z, void *stream);
 
+/* tagi_batchnorm2d_fwd followed by the residual add that ends on this layer, in one
+ * pass: mu_z += mu_res, var_z += var_res ([B][fi][wihi] like the output). Replaces a
+ * BatchNorm2dCuda::forward that closes the main block of a ResNetBlock together with
+ * the add_shortcut_mean_var_cuda launch of ResNetBlockCuda::forward
+ * (src/resnet_block_cuda.cu:7-18, 262-287). */
+int tagi_batchnorm2d_fwd_res(const float *mu_w, const float *var_w,
+                             const float *mu_b, const float *var_b,
+                             const float *mu_a, const float *var_a,
+                             const float *mu_norm, const float *var_norm,
+                             const float *mu_res, const float *var_res, int bias,
+                             float epsilon, int wihi, int fi, int B, float *mu_z,
+                             float *var_z, void *stream);
+
 /* All of BatchNorm2dCuda::backward (src/batchnorm_layer_cuda.cu:969-1102) in one
  * call: state innovations (state_update) and the per-channel weight / bias
  * innovations (param_update; bias ones only when bias != 0). mu_a and jcb are the

@@ -145,3 +145,36 @@ def test_shortcut_adds(oracle_lib):
     ref = oracle_lib.add_shortcut_delta(v[0], v[1], v[4], v[2], v[3])
     assert_close(mu.cpu().numpy(), ref[0], "mu", tol=1e-6)
     assert_close(var.cpu().numpy(), ref[1], "var", tol=1e-6)
+
+
+def test_batchnorm2d_forward_with_residual(oracle_lib):
+    """tagi_batchnorm2d_fwd_res = the layer's forward followed by the residual add."""
+    import torch
+    from cutagi_amd import capi
+    from util import assert_close, batchnorm_inputs
+    for (wihi, fi, B, bias) in [(16, 8, 4, True), (64, 3, 5, False), (1, 37, 6, True)]:
+        d = batchnorm_inputs(wihi, fi, B, seed=wihi + fi + B)
+        rng = np.random.default_rng(wihi * 7 + fi)
+        n = B * fi * wihi
+        res_mu = rng.standard_normal(n).astype(np.float32)
+        res_var = rng.uniform(0.01, 0.5, n).astype(np.float32)
+        mu_s = rng.standard_normal(fi).astype(np.float32)
+        var_s = rng.uniform(0.5, 2.0, fi).astype(np.float32)
+        mb, vb = (d["mu_b"], d["var_b"]) if bias else (None, None)
+        z = oracle_lib.batchnorm2d_fwd(d["mu_w"], d["var_w"], mb, vb, d["mu_a"], d["var_a"], mu_s,
+                                       var_s, 1e-5, wihi, fi, B, 2)
+        want = oracle_lib.add_shortcut(res_mu, res_var, z[0].ravel(), z[1].ravel())
+        t = lambda a: None if a is None else torch.from_numpy(a).cuda()
+        dev = {k: t(v) for k, v in dict(mu_w=d["mu_w"], var_w=d["var_w"], mu_b=mb, var_b=vb,
+                                        mu_a=d["mu_a"], var_a=d["var_a"], mu_s=mu_s, var_s=var_s,
+                                        res_mu=res_mu, res_var=res_var).items()}
+        mu_z, var_z = torch.empty(n, device="cuda"), torch.empty(n, device="cuda")
+        capi.check(capi.lib.tagi_batchnorm2d_fwd_res(
+            capi.ptr(dev["mu_w"]), capi.ptr(dev["var_w"]), capi.ptr(dev["mu_b"]),
+            capi.ptr(dev["var_b"]), capi.ptr(dev["mu_a"]), capi.ptr(dev["var_a"]),
+            capi.ptr(dev["mu_s"]), capi.ptr(dev["var_s"]), capi.ptr(dev["res_mu"]),
+            capi.ptr(dev["res_var"]), int(bias), 1e-5, wihi, fi, B, capi.ptr(mu_z),
+            capi.ptr(var_z), None))
+        torch.cuda.synchronize()
+        assert_close(mu_z.cpu().numpy(), want[0], "mu_z + residual")
+        assert_close(var_z.cpu().numpy(), want[1], "var_z + residual", same_sign=True)
