@@ -44,6 +44,7 @@ SIGNATURES = {
     "tagi_conv2d_fwd": (_i, [_vp] * 7 + [_i] * 7 + [_vp] * 3),
     "tagi_conv2d_fwd_act": (_i, [_vp] * 7 + [_i] * 8 + [_vp] * 4),
     "tagi_conv2d_bwd_dz": (_i, [_vp] * 6 + [_i] * 7 + [_vp] * 3),
+    "tagi_conv2d_bwd_dz_res": (_i, [_vp] * 6 + [_i] * 7 + [_vp, _vp, _i] + [_vp] * 3),
     "tagi_conv2d_bwd_dw": (_i, [_vp] * 6 + [_i] * 7 + [_vp] * 5),
     "tagi_store_states": (_i, [_vp, _vp, _sz, _vp, _vp, _vp, _sz, _vp]),
     "tagi_param_update": (_i, [_vp, _vp, _f, _sz, _vp, _vp, _vp, _vp]),

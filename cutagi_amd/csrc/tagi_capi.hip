@@ -656,10 +656,11 @@ int tagi_conv2d_fwd_act(const float *mu_w, const float *var_w, const float *mu_b
                            bias, mu_out, var_out, stream, activation, jcb_out);
 }
 
-int tagi_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *delta_mu_out,
+static int conv2d_bwd_dz_impl(const float *mu_w, const float *jcb, const float *delta_mu_out,
                        const float *delta_var_out, const int *zw_idx, const int *zud_idx, int woho,
                        int fo, int wihi, int fi, int ki, int nr, int B, float *delta_mu,
-                       float *delta_var, void *stream_) {
+                       float *delta_var, void *stream_, const float *res_mu,
+                              const float *res_var, int res_mode) {
     if (!mu_w || !jcb || !delta_mu_out || !delta_var_out || !zw_idx || !zud_idx || !delta_mu ||
         !delta_var)
         return TAGI_ERR_INVALID_ARG;
@@ -689,8 +690,27 @@ int tagi_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *delta_m
     }
     TAGI_TRY(launch_conv2d_bwd_dz(mu_w, jcb, delta_mu_out, delta_var_out, zw_idx, zud_idx, woho,
                                   fo, wihi, fi, ki, nr, B, tile, splits, ws, ws + part, delta_mu,
-                                  delta_var, stream));
+                                  delta_var, stream, res_mu, res_var, res_mode));
     return TAGI_OK;
+}
+
+int tagi_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *delta_mu_out,
+                       const float *delta_var_out, const int *zw_idx, const int *zud_idx, int woho,
+                       int fo, int wihi, int fi, int ki, int nr, int B, float *delta_mu,
+                       float *delta_var, void *stream) {
+    return conv2d_bwd_dz_impl(mu_w, jcb, delta_mu_out, delta_var_out, zw_idx, zud_idx, woho, fo,
+                              wihi, fi, ki, nr, B, delta_mu, delta_var, stream, nullptr, nullptr, 0);
+}
+
+int tagi_conv2d_bwd_dz_res(const float *mu_w, const float *jcb, const float *delta_mu_out,
+                           const float *delta_var_out, const int *zw_idx, const int *zud_idx,
+                           int woho, int fo, int wihi, int fi, int ki, int nr, int B,
+                           const float *res_mu, const float *res_var, int res_mode,
+                           float *delta_mu, float *delta_var, void *stream) {
+    if (!res_mu || !res_var || (res_mode != 1 && res_mode != 2)) return TAGI_ERR_INVALID_ARG;
+    return conv2d_bwd_dz_impl(mu_w, jcb, delta_mu_out, delta_var_out, zw_idx, zud_idx, woho, fo,
+                              wihi, fi, ki, nr, B, delta_mu, delta_var, stream, res_mu, res_var,
+                              res_mode);
 }
 
 int tagi_conv2d_bwd_dw(const float *var_w, const float *var_b, const float *mu_a,

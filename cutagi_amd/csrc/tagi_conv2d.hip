@@ -43,6 +43,12 @@ struct ConvParams {
     // (tagi_activation.h); out2 then receives its Jacobian
     int act;
     float *out2;
+    // states only: innovations of a residual connection added to the result, laid out
+    // like the output. res_mode 1: added before the Jacobian scaling (identity
+    // shortcut: (sum + res) * jcb), 2: added after it (a shortcut branch's finished
+    // innovations), 0: none.
+    const float *res0, *res1;
+    int res_mode;
 };
 
 // All operand loads below are unconditional: an element outside the problem (or
@@ -637,8 +643,18 @@ struct ConvDzProblem {
     __device__ static __forceinline__ void store_with(const Params &p, int m, int n, float a0,
                                                       float a1, float e) {
         const size_t at = out_index(p, m, n);
-        p.out0[at] = a0 * e;
-        p.out1[at] = a1 * e * e;
+        if (p.res_mode == 1) {
+            a0 += p.res0[at];
+            a1 += p.res1[at];
+        }
+        a0 *= e;
+        a1 *= e * e;
+        if (p.res_mode == 2) {
+            a0 += p.res0[at];
+            a1 += p.res1[at];
+        }
+        p.out0[at] = a0;
+        p.out1[at] = a1;
     }
     __device__ static __forceinline__ void store(const Params &p, int m, int n, float a0,
                                                  float a1) {
@@ -787,9 +803,11 @@ hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float
                                 const float *dvar, const int *zw_idx, const int *zud_idx,
                                 int woho, int fo, int wihi, int fi, int ki, int nr, int B,
                                 int tile, int splits, float *ws0, float *ws1, float *out_dmu,
-                                float *out_dvar, hipStream_t stream) {
+                                float *out_dvar, hipStream_t stream, const float *res_mu,
+                                const float *res_var, int res_mode) {
     const int k2 = ki * ki;
     ConvParams p = {};
+    p.res0 = res_mu; p.res1 = res_var; p.res_mode = res_mu != nullptr ? res_mode : 0;
     p.w0 = mu_w; p.d0 = dmu; p.d1 = dvar; p.e0 = jcb; p.idx = zw_idx; p.idx2 = zud_idx;
     p.out0 = out_dmu; p.out1 = out_dvar;
     p.woho = woho; p.fo = fo; p.wihi = wihi; p.fi = fi; p.k2 = k2; p.B = B; p.nr = nr;

@@ -214,7 +214,8 @@ hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float
                                 const float *dvar, const int *zw_idx, const int *zud_idx,
                                 int woho, int fo, int wihi, int fi, int ki, int nr, int B,
                                 int tile, int splits, float *ws0, float *ws1, float *out_dmu,
-                                float *out_dvar, hipStream_t stream);
+                                float *out_dvar, hipStream_t stream, const float *res_mu = nullptr,
+                                const float *res_var = nullptr, int res_mode = 0);
 int conv2d_bwd_dw_blocks_per_cu(int tile);
 int conv2d_bwd_dw_stencil(const float *mu_a, const float *dmu, const float *dvar, int B, int fo,
                           int woho, int wihi, int fi, int ki, int tile);

@@ -784,19 +784,38 @@ void ResNetBlock::backward(BaseDeltaStates &input_delta_states,
     if (!on_device) no_cpu_path("backward");
     const int batch_size = (int)input_delta_states.block_size;
     input_delta_z->copy_from(input_delta_states, (int)(this->output_size * batch_size));
-    main_block->backward(input_delta_states, output_delta_states, temp_states, state_update);
-
+    // The residual's innovations are added by the state backward of the main block's
+    // first layer where that is a convolution (one pass less per block); the shortcut
+    // branch then runs first, so that its result is there to be added.
+    Conv2dHip *opening = nullptr;
+    if (state_update)
+        if (auto *block = dynamic_cast<LayerBlock *>(main_block.get()))
+            if (block->layers.size() > 1)
+                opening = dynamic_cast<Conv2dHip *>(block->layers.front().get());
     auto *dout = as<DeltaStateHip>(output_delta_states);
     const size_t num_states = (size_t)batch_size * this->input_size;
     if (shortcut) {
         shortcut->backward(*input_delta_z, *shortcut_output_delta_z, temp_states, state_update);
-        if (!state_update) return;
         auto *sc = as<DeltaStateHip>(*shortcut_output_delta_z);
+        if (opening != nullptr) {
+            opening->bwd_residual_mu = sc->d_delta_mu;
+            opening->bwd_residual_var = sc->d_delta_var;
+            opening->bwd_residual_mode = 2;
+        }
+        main_block->backward(input_delta_states, output_delta_states, temp_states, state_update);
+        if (!state_update || opening != nullptr) return;
         TAGI_OK_OR_THROW(tagi_add_shortcut(sc->d_delta_mu, sc->d_delta_var, num_states,
                                            dout->d_delta_mu, dout->d_delta_var, nullptr));
     } else {
-        if (!state_update) return;
         auto *sc = as<DeltaStateHip>(*input_delta_z);
+        if (opening != nullptr) {
+            // (the opening layer's stored Jacobian is the block input's)
+            opening->bwd_residual_mu = sc->d_delta_mu;
+            opening->bwd_residual_var = sc->d_delta_var;
+            opening->bwd_residual_mode = 1;
+        }
+        main_block->backward(input_delta_states, output_delta_states, temp_states, state_update);
+        if (!state_update || opening != nullptr) return;
         auto *kept = as<HiddenStateHip>(*input_z);
         TAGI_OK_OR_THROW(tagi_add_shortcut_delta(sc->d_delta_mu, sc->d_delta_var, kept->jcb_ptr(),
                                                  num_states, dout->d_delta_mu, dout->d_delta_var,

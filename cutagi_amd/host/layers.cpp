@@ -665,6 +665,10 @@ void Conv2dHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &output
 // buffers are needed: the permutations are folded into the kernels' addressing.
 void Conv2dHip::backward(BaseDeltaStates &input_delta_states, BaseDeltaStates &output_delta_states,
                          BaseTempStates &, bool state_udapte) {
+    const float *res_mu = bwd_residual_mu, *res_var = bwd_residual_var;
+    const int res_mode = bwd_residual_mode;
+    bwd_residual_mu = bwd_residual_var = nullptr;
+    bwd_residual_mode = 0;
     auto *din = as<DeltaStateHip>(input_delta_states);
     auto *dout = as<DeltaStateHip>(output_delta_states);
     auto *bwd = dynamic_cast<BackwardStateHip *>(this->bwd_states.get());
@@ -679,11 +683,20 @@ void Conv2dHip::backward(BaseDeltaStates &input_delta_states, BaseDeltaStates &o
     if (state_udapte) {
         if (input_size * batch_size > dout->size)
             LOG(LogLevel::ERROR, "Delta state buffer too small for " + this->get_layer_info());
-        TAGI_OK_OR_THROW(tagi_conv2d_bwd_dz(d_mu_w, bwd->jcb_ptr(), din->d_delta_mu, din->d_delta_var,
-                                            d_idx_cov_zwa_1, d_idx_var_z_ud, woho, (int)out_channels,
-                                            wihi, (int)in_channels, (int)kernel_size, row_zw,
-                                            batch_size, dout->d_delta_mu, dout->d_delta_var,
-                                            nullptr));
+        if (res_mu != nullptr)
+            TAGI_OK_OR_THROW(tagi_conv2d_bwd_dz_res(
+                d_mu_w, bwd->jcb_ptr(), din->d_delta_mu, din->d_delta_var, d_idx_cov_zwa_1,
+                d_idx_var_z_ud, woho, (int)out_channels, wihi, (int)in_channels, (int)kernel_size,
+                row_zw, batch_size, res_mu, res_var, res_mode, dout->d_delta_mu,
+                dout->d_delta_var, nullptr));
+        else
+            TAGI_OK_OR_THROW(tagi_conv2d_bwd_dz(d_mu_w, bwd->jcb_ptr(), din->d_delta_mu,
+                                                din->d_delta_var, d_idx_cov_zwa_1, d_idx_var_z_ud,
+                                                woho, (int)out_channels, wihi, (int)in_channels,
+                                                (int)kernel_size, row_zw, batch_size,
+                                                dout->d_delta_mu, dout->d_delta_var, nullptr));
+    } else if (res_mu != nullptr) {
+        LOG(LogLevel::ERROR, "Residual innovations handed to a layer that skips its state update");
     }
 }
 

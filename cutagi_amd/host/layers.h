@@ -256,6 +256,12 @@ class Conv2dHip : public BaseLayerHip {
     float gain_w, gain_b;
     std::string init_method;
     std::vector<int> idx_mwa_2, idx_cov_zwa_1, idx_var_z_ud;
+    // One-shot, set by a ResNetBlock whose main block starts with this layer: the next
+    // backward() adds the block's residual innovations to its state innovations in the
+    // same pass (mode 1: identity shortcut, scaled by this layer's Jacobian like its own
+    // sum; mode 2: a shortcut branch's finished innovations). Cleared by backward().
+    const float *bwd_residual_mu = nullptr, *bwd_residual_var = nullptr;
+    int bwd_residual_mode = 0;
     int row_zw = 0, col_z_ud = 0;
     int *d_idx_mwa_2 = nullptr, *d_idx_cov_zwa_1 = nullptr, *d_idx_var_z_ud = nullptr;
 

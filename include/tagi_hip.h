@@ -195,6 +195,20 @@ int tagi_conv2d_bwd_dz(const float *mu_w, const float *jcb,
                        int wihi, int fi, int ki, int nr, int B,
                        float *delta_mu, float *delta_var, void *stream);
 
+/* tagi_conv2d_bwd_dz for the first layer of a ResNetBlock's main block, with the
+ * block's residual innovations added in the same pass (res_* laid out like the
+ * output, [B][fi][wihi]). res_mode 1, identity shortcut: (sum + res) .* jcb, which is
+ * the layer's result plus add_shortcut_delta_cuda (src/resnet_block_cuda.cu:20-33) on
+ * the block's incoming innovations; res_mode 2, shortcut branch: the layer's result
+ * plus add_shortcut_mean_var_cuda (7-18) on the branch's finished innovations, as
+ * ResNetBlockCuda::backward runs them (301-347). */
+int tagi_conv2d_bwd_dz_res(const float *mu_w, const float *jcb,
+                           const float *delta_mu_out, const float *delta_var_out,
+                           const int *zw_idx, const int *zud_idx, int woho, int fo,
+                           int wihi, int fi, int ki, int nr, int B,
+                           const float *res_mu, const float *res_var, int res_mode,
+                           float *delta_mu, float *delta_var, void *stream);
+
 /* Weight (and, with bias != 0, bias) backward through Fmwa_2; replaces
  * conv2d_param_backward_cuda (src/conv2d_layer_cuda.cu:149-227) including its
  * delta permutation, and the bias reduction of Conv2dCuda::backward (478-498): delta_*_out are the un-permuted [B][fo][woho] deltas. */

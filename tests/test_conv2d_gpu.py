@@ -220,3 +220,39 @@ def test_conv2d_kernel_too_large_for_the_tap_table_is_refused():
         F.conv2d_fwd(z(fo * fi * k * k), z(fo * fi * k * k), None, None, z(B * fi * wi * wi),
                      z(B * fi * wi * wi), torch.from_numpy(idx["Fmwa_2"]).cuda(), woho, fo,
                      wi * wi, fi, k, B)
+
+
+# stencil kernel, table-driven strided kernel (phase order), sliced reduction
+RES_GEOMS = [(3, 1, 1, 1, 8, 64, 64, 3), (3, 2, 1, 2, 8, 8, 16, 4), (3, 1, 1, 1, 4, 128, 96, 3),
+             (3, 1, 1, 1, 6, 5, 7, 2)]
+
+
+@pytest.mark.parametrize("geom", RES_GEOMS)
+@pytest.mark.parametrize("mode", [1, 2])
+def test_conv2d_state_backward_with_residual(oracle_lib, geom, mode):
+    """tagi_conv2d_bwd_dz_res: mode 1 = (sum + res) .* jcb (identity shortcut), mode 2 =
+    sum .* jcb + res (a shortcut branch's finished innovations)."""
+    import torch
+    from cutagi_amd import capi
+    k, s, p, pt, wi, fi, fo, B = geom
+    idx, d, t, ti, wihi, woho = _setup(oracle_lib, geom, False, seed=sum(geom) + mode)
+    rng = np.random.default_rng(sum(geom))
+    n_in = B * fi * wihi
+    res_mu = rng.normal(0, 0.1, n_in).astype(np.float32)
+    res_var = (-rng.uniform(0, 1e-3, n_in)).astype(np.float32)
+    ref = oracle_lib.conv2d_bwd_dz(d["mu_w"], d["jcb"], d["delta_mu"], d["delta_var"],
+                                   idx["FCzwa_1"], idx["Szz_ud"], woho, fo, wihi, fi, k, idx["h"],
+                                   B, 4)
+    if mode == 1:
+        want = oracle_lib.add_shortcut_delta(res_mu, res_var, d["jcb"], ref[0].ravel(), ref[1].ravel())
+    else:
+        want = oracle_lib.add_shortcut(res_mu, res_var, ref[0].ravel(), ref[1].ravel())
+    r_mu, r_var = torch.from_numpy(res_mu).cuda(), torch.from_numpy(res_var).cuda()
+    om, ov = torch.empty(n_in, device="cuda"), torch.empty(n_in, device="cuda")
+    capi.check(capi.lib.tagi_conv2d_bwd_dz_res(
+        capi.ptr(t["mu_w"]), capi.ptr(t["jcb"]), capi.ptr(t["delta_mu"]), capi.ptr(t["delta_var"]),
+        capi.ptr(ti["FCzwa_1"]), capi.ptr(ti["Szz_ud"]), woho, fo, wihi, fi, k, idx["h"], B,
+        capi.ptr(r_mu), capi.ptr(r_var), mode, capi.ptr(om), capi.ptr(ov), None))
+    torch.cuda.synchronize()
+    assert_close(om.cpu().numpy(), want[0], "delta_mu_z + residual")
+    assert_close(ov.cpu().numpy(), want[1], "delta_var_z + residual", same_sign=True)
