@@ -466,6 +466,11 @@ def _random_cases(n, seed):
     return out
 
 
+# ... and at the batch size the benchmark quotes (minutes of CPU for the reference: the
+# fixture is written once; the GPU test regenerates the inputs from the seed)
+CASES["resnet18_cifar_batch128"] = dict(spec=resnet18_spec(), B=128, steps=1, update=1, n_enc=4,
+                                        var_x=False, seed=28, big=True)
+
 # BatchNorm2d behind a fully-connected layer (one "pixel" per feature)
 CASES["mlp_batchnorm"] = dict(spec="Linear 10 8 1 BatchNorm2d 8 1e-5 0.9 1 ReLU Linear 8 3 1", B=5,
                               steps=2, update=0, var_x=True, input_state_update=True, seed=19)
