@@ -15,8 +15,9 @@ the runtime reports for the device and the wall time of the GPU legs.
 
 Prints ONE JSON line. `roofline` is computed for the dominant kernel from its
 algorithmic work and its average duration measured with HIP events on the
-stream the kernels run on; `cpu_baseline` is the CPU oracle (a bit-identical
-restatement of the reference's multithreaded CPU path) timed on this host.
+stream the kernels run on; `cpu_baseline` is the reference's multithreaded CPU path
+timed on this host: its own sources compiled in place where that library is present
+(kind "reference"), otherwise the bit-identical restatement (kind "port").
 """
 import argparse
 import json
@@ -353,7 +354,17 @@ def cpu_baseline(name):
     import oracle
 
     K, N, B, _ = WORKLOADS[name]
-    lib = oracle.load()
+    # the reference's own CPU kernels where their compiled library travelled with the
+    # tree, otherwise this repository's bit-identical restatement of them
+    kind, lib = "port", None
+    try:
+        lib = oracle.load_ref()
+        if lib is not None:
+            kind = "reference"
+    except OSError:
+        lib = None
+    if lib is None:
+        lib = oracle.load()
     threads = max(1, min(16, os.cpu_count() or 1))
     rng = np.random.default_rng(0)
     f = np.float32
@@ -378,7 +389,7 @@ def cpu_baseline(name):
     reps = 3
     dt = steps(reps, threads)
     out = dict(value=round(14.0 * B * N * K / dt / 1e12, 5), unit="TFLOP/s", cores=threads,
-               kind="port", seconds_per_step=round(dt, 3),
+               kind=kind, seconds_per_step=round(dt, 3),
                sample="%d full forward+backward steps of the %s workload (K=%d, N=%d, B=%d), "
                       "reference thread fan-out with %d std::threads"
                       % (reps, name, K, N, B, threads))
