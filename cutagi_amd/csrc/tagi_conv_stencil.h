@@ -354,14 +354,11 @@ hipError_t launch_conv_stencil(int width, const ConvParams &p, hipStream_t strea
     if (extra > kTileExtraLdsMax) return hipErrorInvalidValue;
 #define TAGI_LAUNCH_STENCIL(WD)                                                                  \
     case WD: {                                                                                   \
-        static bool allowed = false;                                                             \
-        if (!allowed) {                                                                          \
-            hipError_t e = hipFuncSetAttribute(                                                  \
-                reinterpret_cast<const void *>(conv_stencil_kernel<DZ, WD>),                     \
-                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTileExtraLdsMax);              \
-            if (e != hipSuccess) return e;                                                       \
-            allowed = true;                                                                      \
-        }                                                                                        \
+        static PerDeviceOnce once;                                                               \
+        hipError_t e = allow_dynamic_lds(                                                        \
+            once, reinterpret_cast<const void *>(conv_stencil_kernel<DZ, WD>),                   \
+            (int)kTileExtraLdsMax);                                                              \
+        if (e != hipSuccess) return e;                                                           \
         hipLaunchKernelGGL((conv_stencil_kernel<DZ, WD>), grid, dim3(512), extra, stream, p);    \
         return hipGetLastError();                                                                \
     }

@@ -633,14 +633,9 @@ static hipError_t fwd_launch(const float *mu_w, const float *var_w, const float 
                              const float *var_a, int K, int N, int B, int per, int splits,
                              int swz, float *ws0, float *ws1, hipStream_t stream) {
     const size_t lds = (size_t)2 * 4 * H * (per + FWD_LDS_PAD) * sizeof(float);
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e =
-            hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_fwd_kernel<H, RG, C>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return e;
-        configured = true;
-    }
+    static PerDeviceOnce once;
+    hipError_t e = allow_dynamic_lds(once, reinterpret_cast<const void *>(gemv_fwd_kernel<H, RG, C>), 160 * 1024);
+    if (e != hipSuccess) return e;
     constexpr int rows = FWD_WAVES * RG * 4;
     dim3 grid(((N + rows - 1) / rows) * splits), block(FWD_WAVES * 64);
     hipLaunchKernelGGL((gemv_fwd_kernel<H, RG, C>), grid, block, lds, stream, mu_w, var_w, mu_a,
@@ -685,13 +680,9 @@ static hipError_t dz_launch(const float *mu_w, const float *dmu, const float *dv
     size_t lds = (size_t)2 * 4 * H * (per + 4) * sizeof(float);
     const size_t red = (size_t)(DZ_WAVES / 2) * (4 * H * 4 * 2) * 64 * sizeof(float);
     if (red > lds) lds = red;
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_dz_kernel<H>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return e;
-        configured = true;
-    }
+    static PerDeviceOnce once;
+    hipError_t e = allow_dynamic_lds(once, reinterpret_cast<const void *>(gemv_dz_kernel<H>), 160 * 1024);
+    if (e != hipSuccess) return e;
     dim3 grid((K + DZ_COLS_PER_BLOCK - 1) / DZ_COLS_PER_BLOCK, splits), block(DZ_WAVES * 64);
     hipLaunchKernelGGL(gemv_dz_kernel<H>, grid, block, lds, stream, mu_w, dmu, dvar, K, N, B, per,
                        rev, ws0, ws1);

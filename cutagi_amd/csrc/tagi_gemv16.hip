@@ -333,13 +333,9 @@ hipError_t launch_gemv16_fwd(const float *mu_w, const float *var_w, const float 
         k_per_split > gemv16_fwd_max_slice() || (long long)k_per_split * splits < K)
         return hipErrorInvalidValue;
     const size_t lds = (size_t)2 * W16_SAMPLES * (k_per_split + F16_PAD) * sizeof(float);
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemv16_fwd_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return e;
-        configured = true;
-    }
+    static PerDeviceOnce once;
+    hipError_t e = allow_dynamic_lds(once, reinterpret_cast<const void *>(gemv16_fwd_kernel), 160 * 1024);
+    if (e != hipSuccess) return e;
     const int rows = gemv16_fwd_rows_per_block();
     dim3 grid(((N + rows - 1) / rows) * splits), block(W16_WAVES * 64);
     hipLaunchKernelGGL(gemv16_fwd_kernel, grid, block, lds, stream, mu_w, var_w, mu_a, var_a, K,
@@ -357,13 +353,9 @@ hipError_t launch_gemv16_dz(const float *mu_w, const float *dmu, const float *dv
         splits > 65535)
         return hipErrorInvalidValue;
     const size_t lds = (size_t)2 * W16_SAMPLES * (n_per_split + 16 * Z16_PADQ) * sizeof(float);
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemv16_dz_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return e;
-        configured = true;
-    }
+    static PerDeviceOnce once;
+    hipError_t e = allow_dynamic_lds(once, reinterpret_cast<const void *>(gemv16_dz_kernel), 160 * 1024);
+    if (e != hipSuccess) return e;
     const int cols = gemv16_dz_cols_per_block();
     dim3 grid((K + cols - 1) / cols, splits), block(Z16_WAVES * 64);
     hipLaunchKernelGGL(gemv16_dz_kernel, grid, block, lds, stream, mu_w, dmu, dvar, K, N, B,

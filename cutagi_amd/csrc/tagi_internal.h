@@ -11,6 +11,22 @@ namespace tagi {
 int num_cu();
 constexpr int MAX_DEVICES = 16;
 
+// Raises a kernel's dynamic-LDS limit, once per device: the attribute belongs to the
+// kernel's code object on the device that is current when it is set.
+struct PerDeviceOnce {
+    bool done[MAX_DEVICES] = {};
+};
+inline hipError_t allow_dynamic_lds(PerDeviceOnce &once, const void *kernel, int bytes) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= MAX_DEVICES) return hipErrorInvalidDevice;
+    if (once.done[dev]) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) once.done[dev] = true;
+    return e;
+}
+
 // Which contraction of the layer a tiled GEMM launch computes.
 //   FWD: D[b][n]  = sum_k  act[b][k] * w[n][k]      (mean; variance with 2 terms)
 //   DZ : D[b][k'] = sum_n  delta[b][n] * w[n][k']   (variance with w^2)

@@ -611,18 +611,11 @@ template <class P, int BM, int BN, int WM, int WN>
 hipError_t launch_tile(dim3 grid, size_t extra, const typename P::Params &p, hipStream_t stream) {
     if (extra > 0) {
         // static + dynamic LDS beyond 64 KB has to be allowed once per kernel and device
-        static bool allowed[MAX_DEVICES] = {};
-        int dev = 0;
-        hipError_t e = hipGetDevice(&dev);
+        static PerDeviceOnce once;
+        hipError_t e = allow_dynamic_lds(
+            once, reinterpret_cast<const void *>(mfma_tile_kernel<P, BM, BN, WM, WN>),
+            (int)kTileExtraLdsMax);
         if (e != hipSuccess) return e;
-        if (dev < 0 || dev >= MAX_DEVICES) return hipErrorInvalidDevice;
-        if (!allowed[dev]) {
-            e = hipFuncSetAttribute(
-                reinterpret_cast<const void *>(mfma_tile_kernel<P, BM, BN, WM, WN>),
-                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTileExtraLdsMax);
-            if (e != hipSuccess) return e;
-            allowed[dev] = true;
-        }
     }
     hipLaunchKernelGGL((mfma_tile_kernel<P, BM, BN, WM, WN>), grid, dim3(WM * WN * 64), extra,
                        stream, p);
