@@ -17,7 +17,11 @@ Prints ONE JSON line. `roofline` is computed for the dominant kernel from its
 algorithmic work and its average duration measured with HIP events on the
 stream the kernels run on; `cpu_baseline` is the reference's multithreaded CPU path
 timed on this host: its own sources compiled in place where that library is present
-(kind "reference"), otherwise the bit-identical restatement (kind "port").
+(kind "reference"), otherwise the bit-identical restatement (kind "port"). Every
+secondary workload in `extra` carries its own `cpu_baseline` beside its GPU figure
+(a bounded sample of the same workload, stated in `sample`), and its own `roofline`.
+`warmup_effective_steps` / `warmup_seconds` say how long the GPU really worked before
+the timed region: `--warmup` steps plus as many more as it takes to reach 0.3 s.
 """
 import argparse
 import json
@@ -39,13 +43,19 @@ WORKLOADS = {
     # the 16-wide streaming kernels (9..16 samples), reported in `extra` only
     "skinny12": (8192, 8192, 12, "hbm"),
     "skinny16": (8192, 8192, 16, "hbm"),
+    # between the two regimes: the tiled kernels on few rows, reported in `extra.mid`
+    "mid32": (4096, 4096, 32, "mfma"),
+    "mid64": (4096, 4096, 64, "mfma"),
 }
 # HBM bytes per launch of the kernel that dominates each phase of a step, keyed by
 # the kernel that runs there: FETCH_SIZE and WRITE_SIZE of two `rocprofv3 --pmc`
 # runs of this script, each scaled by what the same counter reads for a plain 1 GiB
 # copy (`--calibrate` adds that copy to a run). Counters cannot be read from inside
 # this process, so the figures of the last profiled build are carried here; the
-# summaries, with their commands, are profiles/linear_and_conv2d_hbm_traffic_counters.md.
+# summaries, with their commands, are profiles/linear_and_conv2d_hbm_traffic_counters.md,
+# written by bench_profile.py; TRAFFIC_MEASURED_AT is the commit whose kernels they
+# were measured on and is reported next to every figure taken from the table.
+TRAFFIC_MEASURED_AT = "3c80e14"
 MEASURED_TRAFFIC_BYTES = {
     # (workload, phase): (kernel, bytes)
     ("gemm", "fwd"): ("mfma_tile_kernel<LinearProblem<0,...>, 64, 128, 2, 4>", 235.6e6),      # algorithmic 151.0e6
@@ -92,14 +102,20 @@ def warm_up(step, warmup, min_seconds=0.3):
     `min_seconds`: a handful of sub-millisecond steps right after start-up would
     otherwise be timed on clocks that are still ramping."""
     import torch
+    t_start = time.perf_counter()
+    done = 0
     for _ in range(warmup):
         step()
+    done += warmup
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     while time.perf_counter() - t0 < min_seconds:
         for _ in range(10):
             step()
+        done += 10
         torch.cuda.synchronize()
+    return dict(warmup_effective_steps=done,
+                warmup_seconds=round(time.perf_counter() - t_start, 3))
 
 
 def run_workload(name, steps, warmup):
@@ -134,7 +150,7 @@ def run_workload(name, steps, warmup):
         F.linear_bwd(t["mu_w"], t["var_w"], t["var_b"], t["mu_a"], t["jcb"], t["delta_mu"],
                      t["delta_var"], out=out_bwd)
 
-    warm_up(step, warmup)
+    warm = warm_up(step, warmup)
 
     # timed region: exactly `steps` steps between two synchronisations
     t0 = time.perf_counter()
@@ -185,9 +201,20 @@ def run_workload(name, steps, warmup):
     kernel, traffic = MEASURED_TRAFFIC_BYTES.get((name, dominant), (None, None))
     roof["traffic"] = traffic
     roof["traffic_kernel"] = kernel
+    roof["traffic_measured_at"] = TRAFFIC_MEASURED_AT if traffic is not None else None
     roof["kernel_ms"] = round(phase_ms[dominant], 5)
+    if name.startswith("mid"):
+        # both bounds are close at these batches: the step cannot be faster than the
+        # slower of "all flops at the matrix peak" and "all weight bytes at the HBM peak"
+        t_mfma = 14.0 * B * N * K / (FP32_MFMA_PEAK_TFLOPS * 1e12)
+        t_hbm = 6.0 * N * K * 4 / (HBM_PEAK_GBS * 1e9)
+        roof = dict(bound="mfma" if t_mfma >= t_hbm else "hbm", covers="whole step",
+                    t_mfma_us=round(t_mfma * 1e6, 2), t_hbm_us=round(t_hbm * 1e6, 2),
+                    achieved_us=round(ms_per_step * 1e3, 2),
+                    frac=round(max(t_mfma, t_hbm) / (ms_per_step * 1e-3), 4), traffic=None)
     return dict(name=name, K=K, N=N, B=B, value=value, unit=unit, frac_of_peak=value / peak,
-                ms_per_step=ms_per_step, wall_ms=wall_ms, phase_ms=phase_ms, roofline=roof)
+                ms_per_step=ms_per_step, wall_ms=wall_ms, phase_ms=phase_ms, roofline=roof,
+                warm=warm)
 
 
 def run_conv(steps, warmup):
@@ -218,7 +245,7 @@ def run_conv(steps, warmup):
         F.conv2d_bwd_dz(mu_w, jcb, dmu, dvar, t["FCzwa_1"], t["Szz_ud"], woho, fo, wihi, fi, k,
                         idx["h"], B)
 
-    warm_up(step, warmup)
+    warm = warm_up(step, warmup)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(steps):
@@ -244,7 +271,11 @@ def run_conv(steps, warmup):
                               frac=round(fwd_tflops / FP32_MFMA_PEAK_TFLOPS, 4),
                               traffic=MEASURED_TRAFFIC_BYTES[("conv", "fwd")][1],
                               traffic_kernel=MEASURED_TRAFFIC_BYTES[("conv", "fwd")][0],
-                              kernel_ms=round(fwd_ms, 5)))
+                              traffic_measured_at=TRAFFIC_MEASURED_AT,
+                              kernel_ms=round(fwd_ms, 5)), steps=steps, **warm)
+
+
+MLP_SPEC = "Linear 784 128 1 ReLU Linear 128 128 1 ReLU Linear 128 11 1"
 
 
 def run_mlp(steps, warmup, B=32):
@@ -275,9 +306,7 @@ def run_mlp(steps, warmup, B=32):
         net.step()
         return mu, var
 
-    for _ in range(max(warmup, 20)):
-        step()
-    torch.cuda.synchronize()
+    warm = warm_up(lambda: step(), warmup)
     n = max(steps, 200)
     t0 = time.perf_counter()
     for _ in range(n):
@@ -286,7 +315,7 @@ def run_mlp(steps, warmup, B=32):
     us = (time.perf_counter() - t0) * 1e6 / n
     return dict(workload="TAGI MLP 784->128->128->11 (ReLU), batch %d, one training step through "
                          "the host classes, outputs fetched" % B,
-                value=round(us, 1), unit="us/step", higher_is_better=False, steps=n,
+                value=round(us, 1), unit="us/step", higher_is_better=False, steps=n, **warm,
                 outputs_finite_and_variances_nonnegative=bool(np.all(np.isfinite(mu))
                                                               and var.min() >= 0))
 
@@ -319,9 +348,7 @@ def run_resnet(steps, warmup, B=128):
         net.backward()
         net.step()
 
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
+    warm = warm_up(step, warmup)
     t0 = time.perf_counter()
     for _ in range(steps):
         step()
@@ -329,10 +356,25 @@ def run_resnet(steps, warmup, B=128):
     ms = (time.perf_counter() - t0) * 1e3 / steps
     mu, var = net.get_outputs()
     ok = bool(np.all(np.isfinite(mu)) and var.min() >= 0)
+    # Algorithmic work of the contractions only (Conv2d and Linear layers; BatchNorm,
+    # activations, pooling and the update are not counted): per multiply-accumulate of a
+    # layer 6 flop forward, 4 for the weight innovations and 4 for the state innovations;
+    # the first layer propagates nothing to the input image (10 instead of 14).
+    from cutagi_amd.resnet import resnet18_cifar10_macs
+    macs = resnet18_cifar10_macs()
+    flop = B * sum((14.0 if needs_dz else 10.0) * m for m, needs_dz in macs)
+    tflops = flop / (ms * 1e-3) / 1e12
     return dict(workload="TAGI ResNet-18 (CIFAR: 3x32x32 input, BatchNorm, MixtureReLU, 11 "
                          "hierarchical-softmax outputs), batch %d, one training step" % B,
                 value=round(B / (ms * 1e-3), 1), unit="images/s", ms_per_step=round(ms, 3),
-                outputs_finite_and_variances_nonnegative=ok)
+                steps=steps,
+                roofline=dict(bound="mfma", covers="whole training step (wall clock, host "
+                              "input arrays): flop of the Conv2d / Linear contractions only",
+                              mac_per_image=int(sum(m for m, _ in macs)), flop=flop,
+                              achieved=round(tflops, 2), peak=FP32_MFMA_PEAK_TFLOPS,
+                              unit="TFLOP/s", frac=round(tflops / FP32_MFMA_PEAK_TFLOPS, 4),
+                              traffic=None),
+                outputs_finite_and_variances_nonnegative=ok, **warm)
 
 
 def calibrate_copy():
@@ -348,24 +390,32 @@ def calibrate_copy():
     torch.cuda.synchronize()
 
 
-def cpu_baseline(name):
-    """Full steps of the same workload on the host cores, through the oracle."""
-    import numpy as np
+def _cpu_lib():
+    """The reference's own CPU kernels where their compiled library travelled with the
+    tree (kind "reference"), otherwise this repository's bit-identical restatement of
+    them (kind "port")."""
     import oracle
-
-    K, N, B, _ = WORKLOADS[name]
-    # the reference's own CPU kernels where their compiled library travelled with the
-    # tree, otherwise this repository's bit-identical restatement of them
-    kind, lib = "port", None
     try:
         lib = oracle.load_ref()
         if lib is not None:
-            kind = "reference"
+            return lib, "reference"
     except OSError:
-        lib = None
-    if lib is None:
-        lib = oracle.load()
-    threads = max(1, min(16, os.cpu_count() or 1))
+        pass
+    return oracle.load(), "port"
+
+
+def _cpu_threads():
+    return max(1, min(16, os.cpu_count() or 1))
+
+
+def cpu_baseline(name, reps=2):
+    """Full steps of a Linear workload on the host cores: the reference's thread
+    fan-out with 16 std::threads, and one step with its default of 4."""
+    import numpy as np
+
+    K, N, B, bound = WORKLOADS[name]
+    lib, kind = _cpu_lib()
+    threads = _cpu_threads()
     rng = np.random.default_rng(0)
     f = np.float32
     mu_w = (rng.standard_normal((N, K)) * K ** -0.5).astype(f)
@@ -377,19 +427,22 @@ def cpu_baseline(name):
     jcb = np.ones((B, K), f)
     dmu = (rng.standard_normal((B, N)) * 0.1).astype(f)
     dvar = (-rng.uniform(0, 1e-3, (B, N))).astype(f)
-    def steps(reps, t):
+
+    def steps(n, t):
         t0 = time.perf_counter()
-        for _ in range(reps):
+        for _ in range(n):
             lib.linear_fwd(mu_w, var_w, mu_b, var_b, mu_a, var_a, t)
             lib.linear_bwd_dz(mu_w, jcb, dmu, dvar, t)
             lib.linear_bwd_dw(var_w, mu_a, dmu, dvar, t)
             lib.linear_bwd_db(var_b, dmu, dvar, t)
-        return (time.perf_counter() - t0) / reps
+        return (time.perf_counter() - t0) / n
 
-    reps = 3
+    if bound == "hbm":
+        figure, unit = lambda dt: round(6.0 * N * K * 4 / dt / 1e9, 3), "GB/s"
+    else:
+        figure, unit = lambda dt: round(14.0 * B * N * K / dt / 1e12, 5), "TFLOP/s"
     dt = steps(reps, threads)
-    out = dict(value=round(14.0 * B * N * K / dt / 1e12, 5), unit="TFLOP/s", cores=threads,
-               kind=kind, seconds_per_step=round(dt, 3),
+    out = dict(value=figure(dt), unit=unit, cores=threads, kind=kind, seconds_per_step=round(dt, 3),
                sample="%d full forward+backward steps of the %s workload (K=%d, N=%d, B=%d), "
                       "reference thread fan-out with %d std::threads"
                       % (reps, name, K, N, B, threads))
@@ -397,8 +450,127 @@ def cpu_baseline(name):
         # the reference's default thread count (include/base_layer.h:60), one step
         dt4 = steps(1, 4)
         out["reference_default_threads"] = dict(cores=4, seconds_per_step=round(dt4, 3),
-                                                value=round(14.0 * B * N * K / dt4 / 1e12, 5))
+                                                value=figure(dt4))
     return out
+
+
+def cpu_baseline_conv():
+    """One full forward + backward step of the Conv2d workload on the host cores, and
+    one step at a quarter of the batch with the reference's default of 4 threads."""
+    import numpy as np
+    from cutagi_amd import capi
+
+    lib, kind = _cpu_lib()
+    threads = _cpu_threads()
+    c = CONV
+    fi, fo, k, wi = c["fi"], c["fo"], c["k"], c["wi"]
+    idx = capi.conv2d_build_idx(k, c["stride"], wi, wi, c["pad"], c["pad_type"], k * k * fi * fo + 1)
+    wihi, woho = wi * wi, idx["wo"] * idx["ho"]
+    R = k * k * fi
+    f = np.float32
+
+    def one_step(B, t):
+        rng = np.random.default_rng(0)
+        mu_w = (rng.standard_normal(fo * R) * R ** -0.5).astype(f)
+        var_w = np.full(fo * R, 1.0 / R, f)
+        mu_a = rng.standard_normal(B * fi * wihi).astype(f)
+        var_a = rng.uniform(0.01, 0.1, B * fi * wihi).astype(f)
+        jcb = np.ones(B * fi * wihi, f)
+        dmu = (rng.standard_normal(B * fo * woho) * 0.1).astype(f)
+        dvar = (-rng.uniform(0, 1e-3, B * fo * woho)).astype(f)
+        t0 = time.perf_counter()
+        lib.conv2d_fwd(mu_w, var_w, None, None, mu_a, var_a, idx["Fmwa_2"], woho, fo, wihi, fi, k,
+                       B, t)
+        lib.conv2d_bwd_dw(var_w, None, mu_a, dmu, dvar, idx["Fmwa_2"], B, fo, woho, wihi, fi, k, t)
+        lib.conv2d_bwd_dz(mu_w, jcb, dmu, dvar, idx["FCzwa_1"], idx["Szz_ud"], woho, fo, wihi, fi,
+                          k, idx["h"], B, t)
+        return time.perf_counter() - t0
+
+    tf = lambda B, dt: round(14.0 * fo * (B * woho) * R / dt / 1e12, 5)
+    B = c["B"]
+    dt = one_step(B, threads)
+    out = dict(value=tf(B, dt), unit="TFLOP/s", cores=threads, kind=kind,
+               seconds_per_step=round(dt, 3),
+               sample="1 full forward+backward step of the Conv2d workload (batch %d), reference "
+                      "thread fan-out with %d std::threads" % (B, threads))
+    if threads > 4:
+        Bq = B // 4
+        dt4 = one_step(Bq, 4)
+        out["reference_default_threads"] = dict(
+            cores=4, value=tf(Bq, dt4), seconds_per_step_at_full_batch=round(dt4 * B / Bq, 3),
+            sample="1 step at batch %d (a quarter of the workload; the work is linear in the "
+                   "batch)" % Bq)
+    return out
+
+
+def _ref_model_seconds_per_step(ref, spec, B, n_in, n_obs, n_out, steps_a, steps_b, threads):
+    """Seconds per training step of the reference's own Sequential on the CPU
+    (oracle/ref_model.cpp): two runs that differ in their number of steps, so that
+    building the network and loading its parameters cancel."""
+    import numpy as np
+    rng = np.random.default_rng(0)
+    sizes = ref.model_param_sizes(spec)
+    params = [np.abs(rng.standard_normal(n)).astype(np.float32) * 0.05 + 1e-3 for n in sizes]
+
+    def run(steps):
+        x = rng.standard_normal((steps, B * n_in)).astype(np.float32)
+        y = rng.standard_normal((steps, B * n_obs)).astype(np.float32)
+        var_y = np.ones((steps, B * n_obs), np.float32)
+        sel = np.stack([np.concatenate([rng.choice(n_out, n_obs, replace=False) + 1
+                                        for _ in range(B)]) for _ in range(steps)]).astype(np.int32)
+        t0 = time.perf_counter()
+        ref.model_run(spec, params, x, None, y, var_y, sel, B, 1, n_enc=n_obs, threads=threads)
+        return time.perf_counter() - t0
+
+    ta, tb = run(steps_a), run(steps_b)
+    return (tb - ta) / (steps_b - steps_a)
+
+
+def cpu_baseline_mlp(B=32):
+    import oracle
+    ref = oracle.load_ref()
+    if ref is None:
+        return dict(value=None, reason="the compiled reference (oracle/_ref) is not present; "
+                                       "its Sequential is what this baseline runs")
+    threads = 4  # the reference's default (include/base_layer.h:60)
+    dt = _ref_model_seconds_per_step(ref, MLP_SPEC, B, 784, 4, 11, 20, 120, threads)
+    return dict(value=round(dt * 1e6, 1), unit="us/step", cores=threads, kind="reference",
+                sample="100 training steps of the same network and batch through the reference's "
+                       "Sequential / OutputUpdater on the CPU (difference of a 120- and a 20-step "
+                       "run), %d std::threads" % threads)
+
+
+def resnet18_spec():
+    """The CIFAR ResNet-18 as the text description oracle/ref_model.cpp builds the
+    reference's layers from (same architecture as cutagi_amd/resnet.py)."""
+    bn = "BatchNorm2d %d 1e-5 0.9 1"
+
+    def main(i, o, s, pt):
+        return ("Conv2d %d %d 3 0 %d 1 %d 0 0 MixtureReLU " % (i, o, s, pt) + bn % o +
+                " Conv2d %d %d 3 0 1 1 1 0 0 MixtureReLU " % (o, o) + bn % o)
+
+    same = lambda c: "ResNetBlock [ " + main(c, c, 1, 1) + " ] [ ]"
+    down = lambda i, o: ("ResNetBlock [ " + main(i, o, 2, 2) + " ] [ Conv2d %d %d 2 0 2 0 1 0 0 "
+                         "MixtureReLU " % (i, o) + bn % o + " ]")
+    return " ".join(["Conv2d 3 64 3 0 1 1 1 32 32 MixtureReLU " + bn % 64, same(64), same(64),
+                     down(64, 128), same(128), down(128, 256), same(256), down(256, 512),
+                     same(512), "AvgPool2d 4 -1 0 0 Linear 512 11 1"])
+
+
+def cpu_baseline_resnet(B=16, full_batch=128):
+    import oracle
+    ref = oracle.load_ref()
+    if ref is None:
+        return dict(value=None, reason="the compiled reference (oracle/_ref) is not present; "
+                                       "its Sequential is what this baseline runs")
+    threads = _cpu_threads()
+    dt = _ref_model_seconds_per_step(ref, resnet18_spec(), B, 3 * 32 * 32, 4, 11, 1, 2, threads)
+    return dict(value=round(B / dt, 2), unit="images/s", cores=threads, kind="reference",
+                seconds_per_step=round(dt, 3), batch=B,
+                sample="1 training step of the same network at batch %d (1/%d of the workload's "
+                       "%d: a full-batch step takes minutes on the CPU) through the reference's "
+                       "Sequential / OutputUpdater (difference of a 2- and a 1-step run), %d "
+                       "std::threads" % (B, full_batch // B, full_batch, threads))
 
 
 def main():
@@ -438,6 +610,9 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        # what really ran before the timed region (see warm_up)
+        "warmup_effective_steps": main_res["warm"]["warmup_effective_steps"],
+        "warmup_seconds": main_res["warm"]["warmup_seconds"],
         "ms_per_step": round(main_res["ms_per_step"], 5),
         "higher_is_better": True,
         "scaling": "weak",
@@ -461,26 +636,24 @@ def main():
     extras = [] if args.no_extra else [e for e in args.extra.split(",") if e]
     if extras:
         line["extra"] = {}
+
+    def linear_entry(r):
+        return {"workload": "TAGI Linear %d->%d, batch %d" % (r["K"], r["N"], r["B"]),
+                "value": round(r["value"], 3), "unit": r["unit"],
+                "frac_of_peak": round(r["frac_of_peak"], 4),
+                "ms_per_step": round(r["ms_per_step"], 5), "steps": args.steps,
+                "phase_ms": {k: round(v, 5) for k, v in r["phase_ms"].items()},
+                "roofline": r["roofline"], **r["warm"]}
+
     if "linear" in extras:
         other = "skinny" if args.workload == "gemm" else "gemm"
-        r = run_workload(other, args.steps, args.warmup)
-        line["extra"][other] = {
-            "workload": "TAGI Linear %d->%d, batch %d" % (r["K"], r["N"], r["B"]),
-            "value": round(r["value"], 3), "unit": r["unit"],
-            "frac_of_peak": round(r["frac_of_peak"], 4),
-            "ms_per_step": round(r["ms_per_step"], 5),
-            "phase_ms": {k: round(v, 5) for k, v in r["phase_ms"].items()},
-            "roofline": r["roofline"]}
+        line["extra"][other] = linear_entry(run_workload(other, args.steps, args.warmup))
         if args.workload == "gemm":
             for wide in ("skinny12", "skinny16"):
-                r = run_workload(wide, args.steps, args.warmup)
-                line["extra"][wide] = {
-                    "workload": "TAGI Linear %d->%d, batch %d" % (r["K"], r["N"], r["B"]),
-                    "value": round(r["value"], 3), "unit": r["unit"],
-                    "frac_of_peak": round(r["frac_of_peak"], 4),
-                    "ms_per_step": round(r["ms_per_step"], 5),
-                    "phase_ms": {k: round(v, 5) for k, v in r["phase_ms"].items()},
-                    "roofline": r["roofline"]}
+                line["extra"][wide] = linear_entry(run_workload(wide, args.steps, args.warmup))
+            # Linear 4096^2 at batch 32 and 64, where the matrix and the memory bound meet
+            line["extra"]["mid"] = {name: linear_entry(run_workload(name, args.steps, args.warmup))
+                                    for name in ("mid32", "mid64")}
     if "mlp" in extras:
         line["extra"]["mlp"] = run_mlp(args.steps, args.warmup)
     if "conv" in extras:
@@ -490,10 +663,22 @@ def main():
     if args.calibrate:
         calibrate_copy()
     # wall time of everything that ran on the GPU, so that the short timed regions can
-    # be placed inside the whole run (the CPU baseline below takes most of it)
+    # be placed inside the whole run (the CPU baselines below take most of it)
     line["gpu_wall_s"] = round(time.perf_counter() - gpu_t0, 2)
     if not args.no_cpu:
+        cpu_t0 = time.perf_counter()
         line["cpu_baseline"] = cpu_baseline(args.workload)
+        ex = line.get("extra", {})
+        other = "skinny" if args.workload == "gemm" else "gemm"
+        if other in ex:
+            ex[other]["cpu_baseline"] = cpu_baseline(other)
+        if "mlp" in ex:
+            ex["mlp"]["cpu_baseline"] = cpu_baseline_mlp()
+        if "conv" in ex:
+            ex["conv"]["cpu_baseline"] = cpu_baseline_conv()
+        if "resnet18" in ex:
+            ex["resnet18"]["cpu_baseline"] = cpu_baseline_resnet()
+        line["cpu_wall_s"] = round(time.perf_counter() - cpu_t0, 2)
     print(json.dumps(line))
 
 

@@ -7,6 +7,7 @@
 #include <vector>
 
 #include "../../include/tagi_hip.h"
+#include "../../include/tagi_hip_test_hooks.h"
 #include "tagi_internal.h"
 
 using namespace tagi;

@@ -346,7 +346,7 @@ void BaseLayerHip::store_states_for_training_hip(HiddenStateHip &in, HiddenState
     bwd->device_idx = in.device_idx;
     out.jcb_ones = true;
     if (in.transient) {
-        bwd->resize_exact(in.size);
+        bwd->resize_exact(in.size, !in.jcb_ones);
         std::swap(bwd->d_mu_a, in.d_mu_a);
         bwd->jcb_ones = in.jcb_ones;
         if (!in.jcb_ones) std::swap(bwd->d_jcb, in.d_jcb);

@@ -316,7 +316,9 @@ void HiddenStateHip::swap(BaseHiddenStates &other) {
     std::swap(d_var_a, o->d_var_a);
     std::swap(d_jcb, o->d_jcb);
     std::swap(jcb_ones, o->jcb_ones);
-    std::swap(transient, o->transient);
+    // `transient` stays: it says what role the OBJECT plays for its owner (a ping-pong
+    // buffer whose contents are dead once read), not what the arrays hold. A caller's
+    // input state that trades arrays with such a buffer remains the caller's.
 }
 void HiddenStateHip::copy_from(const BaseHiddenStates &source, int num_data) {
     auto *s = dynamic_cast<const HiddenStateHip *>(&source);
@@ -338,12 +340,15 @@ DeltaStateHip::DeltaStateHip(size_t n, size_t m, int device_idx) : BaseDeltaStat
     this->allocate_memory();
 }
 DeltaStateHip::~DeltaStateHip() { this->deallocate_memory(); }
-// The two arrays are one allocation (variance right after the mean), so that
-// reset_zeros is one launch; swap() exchanges both pointers, which keeps pairs together.
+// The two arrays are one allocation, so that reset_zeros is one launch; swap() exchanges
+// both pointers, which keeps pairs together. The variance starts at the next multiple of
+// 64 floats after the mean, so that both arrays are 256-byte aligned for any size (the
+// kernels choose their 16-byte paths by pointer alignment).
+static size_t delta_var_offset(size_t size) { return (size + 63) / 64 * 64; }
 void DeltaStateHip::allocate_memory() {
     this->deallocate_memory();
-    d_delta_mu = dev_alloc(2 * size, device_idx);
-    d_delta_var = d_delta_mu != nullptr ? d_delta_mu + size : nullptr;
+    d_delta_mu = dev_alloc(delta_var_offset(size) + size, device_idx);
+    d_delta_var = d_delta_mu != nullptr ? d_delta_mu + delta_var_offset(size) : nullptr;
     this->to_device();
 }
 void DeltaStateHip::deallocate_memory() {
@@ -360,7 +365,7 @@ void DeltaStateHip::to_host() {
 }
 void DeltaStateHip::reset_zeros() {
     if (size == 0) return;
-    HIP_OK(hipMemsetAsync(d_delta_mu, 0, 2 * size * sizeof(float), nullptr));
+    HIP_OK(hipMemsetAsync(d_delta_mu, 0, (delta_var_offset(size) + size) * sizeof(float), nullptr));
 }
 void DeltaStateHip::copy_from(const BaseDeltaStates &source, int num_data) {
     auto *s = dynamic_cast<const DeltaStateHip *>(&source);
@@ -433,11 +438,16 @@ void BackwardStateHip::to_host() {
     else
         d2h(jcb.data(), d_jcb, size);
 }
-void BackwardStateHip::resize_exact(size_t new_size) {
-    if (new_size == this->size && d_mu_a != nullptr) return;
-    this->size = new_size;
-    HIP_OK(hipDeviceSynchronize());
-    this->allocate_memory();
+// Exactly `new_size` elements (the arrays are traded with a buffer of that size). The
+// Jacobian array is only allocated once a Jacobian that is not all ones has to be kept.
+void BackwardStateHip::resize_exact(size_t new_size, bool need_jcb) {
+    if (new_size != this->size || d_mu_a == nullptr) {
+        this->size = new_size;
+        HIP_OK(hipDeviceSynchronize());
+        this->deallocate_memory();
+        d_mu_a = dev_alloc(size, device_idx);
+    }
+    if (need_jcb && d_jcb == nullptr) d_jcb = dev_alloc(size, device_idx);
 }
 void BackwardStateHip::set_size(size_t new_size) {
     if (new_size > this->size) {

@@ -171,7 +171,7 @@ class BackwardStateHip : public BaseBackwardStates {
     bool jcb_ones = false;  // as HiddenStateHip::jcb_ones
     const float *jcb_ptr() const { return jcb_ones ? device_ones(size, device_idx) : d_jcb; }
     // exactly new_size floats per array (reallocates when the size differs)
-    void resize_exact(size_t new_size);
+    void resize_exact(size_t new_size, bool need_jcb);
 
     BackwardStateHip() = default;
     ~BackwardStateHip() override;

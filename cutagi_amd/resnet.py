@@ -59,3 +59,25 @@ def hrc_softmax(num_classes):
             obs[cls, level] = -1.0 if bit else 1.0
             idx[cls, level] = nodes[(level, cls >> (n_obs - level))]
     return obs, idx, n_obs, unit
+
+
+def resnet18_cifar10_macs():
+    """(multiply-accumulates per image, propagates innovations to its input) of every
+    Conv2d / Linear layer of resnet18_cifar10, in network order: output channels x
+    output pixels x kernel taps x input channels. The stem is the network's first
+    layer and propagates nothing to the image."""
+    out = [(64 * 32 * 32 * 9 * 3, False)]
+
+    def main(i, o, w_out):
+        return [(o * w_out * w_out * 9 * i, True), (o * w_out * w_out * 9 * o, True)]
+
+    w, c = 32, 64
+    for stage, o in enumerate((64, 128, 256, 512)):
+        if stage == 0:
+            out += main(c, o, w) + main(o, o, w)
+        else:
+            w //= 2
+            out += main(c, o, w) + [(o * w * w * 4 * c, True)] + main(o, o, w)   # + 2x2 projection
+        c = o
+    out.append((512 * 11, True))
+    return out

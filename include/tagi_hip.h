@@ -57,21 +57,6 @@ int tagi_hip_shutdown(void);
  * reference's counterpart is get_cuda_device_properties (src/cuda_utils.cpp). */
 int tagi_hip_device_info(int *compute_units /* host */, int *clock_mhz /* host */,
                          char *name /* host */, size_t name_capacity);
-/* TEST AND EXPERIMENT HOOK, not part of the drop-in surface: a caller of the
- * reference has no reason to touch it, and every knob is process-wide (set it only
- * while no other thread is inside the library). Kernel-selection switches used by
- * the parity tests to force each code path and by the tuning sweeps; value < 0
- * restores the built-in heuristic, unknown keys are an error. Linear: "linear.tile",
- * "linear.fwd.splits", "linear.dz.splits", "linear.dw.splits",
- * "linear.gemv_max_batch" (largest batch of the streaming kernels, at most 16),
- * "linear.gemv.swizzle", "linear.gemv.fwd_variant", "linear.gemv.reverse",
- * "linear.gemv16" (0: 9..16 samples on the kernels for up to 8),
- * "linear.dw_side" (0: bias innovations and the state-backward fold as launches
- * of their own instead of inside the weight-backward launch). Conv2d:
- * "conv2d.tile", "conv2d.splits", "conv2d.dw.tile", "conv2d.dw.splits",
- * "conv2d.group_loads", "conv2d.stencil", "conv2d.phase_order" (0 switches the
- * named path off). */
-int tagi_hip_tune(const char *key /* host */, int value);
 
 /* ---- Linear -------------------------------------------------------------- */
 
@@ -109,7 +94,9 @@ int tagi_linear_fwd_act(const float *mu_w, const float *var_w, const float *mu_b
  * bytes; 32 MiB at K = N = 4096, B = 256). All calls on one GPU share the array:
  * calls that overlap on one GPU (two streams, two host threads) race. The first
  * call on a device looks the array's address up once; make that call outside a
- * graph capture. */
+ * graph capture. The array is part of the library's device image: every process
+ * that loads the library holds these 64 MiB on every GPU it touches, whether or
+ * not it ever calls this entry point. */
 #define TAGI_LINEAR_FWD_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
 int tagi_linear_fwd_static(const float *mu_w, const float *var_w,
                            const float *mu_b, const float *var_b,

@@ -1,0 +1,31 @@
+/*
+ * tagi_hip_test_hooks.h - kernel-selection switches of libtagi_hip.so for its own
+ * parity tests and tuning sweeps. NOT part of the drop-in boundary (tagi_hip.h): a
+ * binding of the reference never includes this file, and nothing a caller of the
+ * reference does maps to it. It has no counterpart in the reference.
+ */
+#ifndef TAGI_HIP_TEST_HOOKS_H
+#define TAGI_HIP_TEST_HOOKS_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Every knob is process-wide (set it only while no other thread is inside the
+ * library). The parity tests use them to force each code path, the tuning sweeps
+ * to compare them; value < 0 restores the built-in heuristic, unknown keys return
+ * TAGI_ERR_INVALID_ARG. Linear: "linear.tile", "linear.fwd.splits",
+ * "linear.dz.splits", "linear.dw.splits", "linear.gemv_max_batch" (largest batch of
+ * the streaming kernels, at most 16), "linear.gemv.swizzle",
+ * "linear.gemv.fwd_variant", "linear.gemv.reverse", "linear.gemv16" (0: 9..16
+ * samples on the kernels for up to 8), "linear.dw_side" (0: bias innovations and
+ * the state-backward fold as launches of their own instead of inside the
+ * weight-backward launch), "linear.double_buffer". Conv2d: "conv2d.tile",
+ * "conv2d.splits", "conv2d.dw.tile", "conv2d.dw.splits", "conv2d.group_loads",
+ * "conv2d.stencil", "conv2d.phase_order" (0 switches the named path off). */
+int tagi_hip_tune(const char *key /* host */, int value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TAGI_HIP_TEST_HOOKS_H */

@@ -11,7 +11,10 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def _declared():
-    text = open(os.path.join(ROOT, "include", "tagi_hip.h")).read()
+    import glob
+    headers = sorted(glob.glob(os.path.join(ROOT, "include", "*.h")))
+    assert [os.path.basename(h) for h in headers] == ["tagi_hip.h", "tagi_hip_test_hooks.h"]
+    text = "".join(open(h).read() for h in headers)
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(tagi_[a-z0-9_]+)\s*\(", text)))
 
@@ -115,3 +118,11 @@ def test_bench_refuses_more_than_one_gpu():
     assert res.returncode != 0
     assert "one GPU" in res.stderr
     assert res.stdout.strip() == ""
+
+
+def test_tuning_switches_are_not_part_of_the_boundary_header():
+    """The drop-in boundary (tagi_hip.h) offers no kernel-selection switch; the test
+    hook lives in a header of its own that a binding of the reference never includes."""
+    text = open(os.path.join(ROOT, "include", "tagi_hip.h")).read()
+    assert "tagi_hip_tune" not in text
+    assert "tagi_hip_tune" in open(os.path.join(ROOT, "include", "tagi_hip_test_hooks.h")).read()

@@ -77,6 +77,57 @@ def test_linear_full_size_against_float64_closed_forms(K, N, B):
         assert torch.equal(2 * a, b)
 
 
+# Large batches (the tiled kernels far above the 256 rows of the benchmark shape; the
+# second shape also has a ragged reduction): float64 closed forms for every entry, and
+# the CPU oracle on a sample -- whole batch rows for the forward and the state backward
+# (rows of a batch do not interact), whole output units for the weight / bias backward
+# (a unit's innovations depend on its own column of the incoming innovations only).
+@pytest.mark.parametrize("K,N,B", [(2048, 1024, 1024), (1000, 512, 4096)])
+def test_linear_large_batch_against_float64_and_sampled_oracle(oracle_lib, K, N, B):
+    import torch
+    import cutagi_amd.functional as F
+    from util import SAME_SIGN, assert_close
+    t = _linear_inputs(K, N, B, seed=K + B)
+    d = {k: v.double() for k, v in t.items()}
+    mu_z, var_z = F.linear_fwd(t["mu_w"], t["var_w"], t["mu_b"], t["var_b"], t["mu_a"], t["var_a"])
+    _check(mu_z, d["mu_a"] @ d["mu_w"].T + d["mu_b"], "mu_z")
+    _check(var_z, (d["mu_a"] ** 2 + d["var_a"]) @ d["var_w"].T + d["var_a"] @ (d["mu_w"] ** 2).T
+           + d["var_b"], "var_z")
+    assert float(var_z.min()) >= 0.0
+    out = F.linear_bwd(t["mu_w"], t["var_w"], t["var_b"], t["mu_a"], t["jcb"], t["delta_mu"],
+                       t["delta_var"])
+    _check(out[0], (d["delta_mu"] @ d["mu_w"]) * d["jcb"], "delta_mu_z")
+    _check(out[1], (d["delta_var"] @ d["mu_w"] ** 2) * d["jcb"] ** 2, "delta_var_z")
+    _check(out[2], (d["delta_mu"].T @ d["mu_a"]) * d["var_w"], "delta_mu_w")
+    _check(out[3], (d["delta_var"].T @ d["mu_a"] ** 2) * d["var_w"] ** 2, "delta_var_w")
+    _check(out[4], d["delta_mu"].sum(0) * d["var_b"], "delta_mu_b")
+    _check(out[5], d["delta_var"].sum(0) * d["var_b"] ** 2, "delta_var_b")
+
+    h = {k: v.cpu().numpy() for k, v in t.items()}
+    rng = np.random.default_rng(B)
+    rows = np.sort(rng.choice(B, 6, replace=False))       # batch rows
+    units = np.sort(rng.choice(N, 6, replace=False))      # output units
+    ref = oracle_lib.linear_fwd(h["mu_w"], h["var_w"], h["mu_b"], h["var_b"],
+                                np.ascontiguousarray(h["mu_a"][rows]),
+                                np.ascontiguousarray(h["var_a"][rows]), threads=4)
+    assert_close(mu_z.cpu().numpy()[rows], ref[0], "mu_z rows vs oracle")
+    assert_close(var_z.cpu().numpy()[rows], ref[1], "var_z rows vs oracle", same_sign=True)
+    ref = oracle_lib.linear_bwd_dz(h["mu_w"], np.ascontiguousarray(h["jcb"][rows]),
+                                   np.ascontiguousarray(h["delta_mu"][rows]),
+                                   np.ascontiguousarray(h["delta_var"][rows]), threads=4)
+    assert_close(out[0].cpu().numpy()[rows], ref[0], "delta_mu_z rows vs oracle")
+    assert_close(out[1].cpu().numpy()[rows], ref[1], "delta_var_z rows vs oracle", same_sign=True)
+    dmu_u = np.ascontiguousarray(h["delta_mu"][:, units])
+    dvar_u = np.ascontiguousarray(h["delta_var"][:, units])
+    ref = oracle_lib.linear_bwd_dw(np.ascontiguousarray(h["var_w"][units]), h["mu_a"], dmu_u,
+                                   dvar_u, threads=4)
+    assert_close(out[2].cpu().numpy()[units], ref[0], "delta_mu_w units vs oracle")
+    assert_close(out[3].cpu().numpy()[units], ref[1], "delta_var_w units vs oracle", same_sign=True)
+    ref = oracle_lib.linear_bwd_db(np.ascontiguousarray(h["var_b"][units]), dmu_u, dvar_u)
+    assert_close(out[4].cpu().numpy()[units], ref[0], "delta_mu_b units vs oracle")
+    assert_close(out[5].cpu().numpy()[units], ref[1], "delta_var_b units vs oracle", same_sign=True)
+
+
 def test_conv2d_full_size_against_float64_closed_forms():
     """Config 4 through the regular-stencil kernels (the library's own tables)."""
     import torch

@@ -1,7 +1,14 @@
 """Linear / Conv2d forward with the following activation applied in the kernel's
-epilogue (tagi_linear_fwd_act, tagi_conv2d_fwd_act) against the oracle's layer
-followed by the oracle's activation; and the host classes with the fusion switched
-off against the same reference vectors as with it on."""
+epilogue (tagi_linear_fwd_act, tagi_conv2d_fwd_act); and the host classes with the
+fusion switched off against the same reference vectors as with it on.
+
+The fused call is checked in two separate steps, so that neither hides the other:
+the layer's sums (the unfused call on the same inputs, which runs the same kernel
+without the epilogue) against the oracle's layer at the 1e-4 parity tolerance, and
+the epilogue alone - the fused outputs against the oracle's activation applied to
+the GPU's OWN sums - at 1e-5 (ReLU: exactly). A non-linearity amplifies the 1e-4
+reordering error of its input, which is why the fused outputs are not compared with
+oracle-layer-then-oracle-activation at one tolerance."""
 import os
 
 import numpy as np
@@ -10,6 +17,10 @@ import pytest
 from util import assert_close, conv_inputs, linear_inputs
 
 pytestmark = pytest.mark.gpu
+
+# fused epilogue against the oracle's activation of the same fp32 sums: what is left
+# is the difference between the device's and the host's erfc / exp
+EPILOGUE_TOL = 1e-5
 
 # tiled unsliced / sliced reductions, ragged shapes, the streaming kernels (B <= 8, 9..16)
 LINEAR = [(256, 256, 128), (1024, 512, 64), (100, 36, 40), (785, 600, 16), (784, 128, 32),
@@ -38,7 +49,6 @@ def test_linear_forward_with_activation(oracle_lib, K, N, B, act, bias):
     plain = F.linear_fwd(t["mu_w"], t["var_w"], t["mu_b"], t["var_b"], t["mu_a"], t["var_a"])
     z = oracle_lib.linear_fwd(d["mu_w"], d["var_w"], d["mu_b"], d["var_b"], d["mu_a"], d["var_a"],
                               threads=4)
-    ref = _activate(oracle_lib, act, z[0], z[1])
     if act == "relu":
         # ReLU is a selection: exactly the unfused kernel's sums, gated by their sign
         m = plain[0].cpu().numpy().ravel()
@@ -47,8 +57,13 @@ def test_linear_forward_with_activation(oracle_lib, K, N, B, act, bias):
         assert np.array_equal(got[1].cpu().numpy().ravel(), np.where(keep, plain[1].cpu().numpy().ravel(), 0))
         assert np.array_equal(got[2].cpu().numpy().ravel(), keep.astype(np.float32))
         return
-    for name, g, r in zip(("mu_a", "var_a", "jcb"), got, ref):
-        assert_close(g.cpu().numpy().ravel(), r, name, tol=2e-4)
+    # the sums, against the oracle's layer
+    assert_close(plain[0].cpu().numpy().ravel(), z[0].ravel(), "mu_z")
+    assert_close(plain[1].cpu().numpy().ravel(), z[1].ravel(), "var_z", same_sign=True)
+    # the epilogue, against the oracle's activation of those very sums
+    own = _activate(oracle_lib, act, plain[0].cpu().numpy(), plain[1].cpu().numpy())
+    for name, g, r in zip(("mu_a", "var_a", "jcb"), got, own):
+        assert_close(g.cpu().numpy().ravel(), r, name, tol=EPILOGUE_TOL)
     assert float(got[1].min()) > 0 and 0 <= float(got[2].min()) and float(got[2].max()) <= 1
 
 
@@ -73,16 +88,18 @@ def test_conv2d_forward_with_activation(oracle_lib, geom, act):
                            aidx, woho, fo, wihi, fi, k, B, act)
     z = oracle_lib.conv2d_fwd(d["mu_w"], d["var_w"], d["mu_b"], d["var_b"], d["mu_a"], d["var_a"],
                               idx["Fmwa_2"], woho, fo, wihi, fi, k, B, 2)
-    ref = _activate(oracle_lib, act, z[0], z[1])
+    plain = F.conv2d_fwd(t["mu_w"], t["var_w"], t["mu_b"], t["var_b"], t["mu_a"], t["var_a"],
+                         aidx, woho, fo, wihi, fi, k, B)
     if act == "relu":
-        plain = F.conv2d_fwd(t["mu_w"], t["var_w"], t["mu_b"], t["var_b"], t["mu_a"], t["var_a"],
-                             aidx, woho, fo, wihi, fi, k, B)
         m = plain[0].cpu().numpy()
         assert np.array_equal(got[0].cpu().numpy(), np.maximum(m, 0))
         assert np.array_equal(got[2].cpu().numpy(), (np.maximum(m, 0) != 0).astype(np.float32))
         return
-    for name, g, r in zip(("mu_a", "var_a", "jcb"), got, ref):
-        assert_close(g.cpu().numpy(), r, name, tol=2e-4)
+    assert_close(plain[0].cpu().numpy().ravel(), z[0].ravel(), "mu_z")
+    assert_close(plain[1].cpu().numpy().ravel(), z[1].ravel(), "var_z", same_sign=True)
+    own = _activate(oracle_lib, act, plain[0].cpu().numpy(), plain[1].cpu().numpy())
+    for name, g, r in zip(("mu_a", "var_a", "jcb"), got, own):
+        assert_close(g.cpu().numpy().ravel(), r, name, tol=EPILOGUE_TOL)
 
 
 @pytest.mark.parametrize("name", ["mlp_config1", "conv_relu_linear", "small_resnet",

@@ -8,7 +8,7 @@ pytestmark = pytest.mark.gpu
 
 # (K, N, B): tiled path (aligned / ragged / odd), skinny path, layer shapes of
 # the MLP configuration, and the reference's odd-size smoke shape (785 -> 6000)
-# scaled down.
+# scaled down (its real size: test_pack_size_network_at_its_real_size below).
 SHAPES = [
     (256, 256, 128), (512, 384, 256), (100, 36, 40), (785, 600, 16), (784, 128, 32),
     (128, 128, 32), (128, 11, 32), (64, 32, 1), (256, 512, 8), (1024, 256, 5),
@@ -105,3 +105,56 @@ def test_size_mismatch_raises():
     with pytest.raises(ValueError):
         F.linear_fwd(t["mu_w"], t["var_w"], t["mu_b"], t["var_b"], t["mu_a"][:, :32].contiguous(),
                      t["var_a"][:, :32].contiguous())
+
+
+# The reference's odd-size survival test at its real size: Linear(785, 6000) - ReLU -
+# Linear(6000, 784), batch 16, one forward / dense output update / backward / step
+# (test/cpp_unit/test_pack_size.cpp:26-62; it only asserts that the run survives).
+# Here each layer at that size is also held against the oracle.
+@pytest.mark.parametrize("K,N", [(785, 6000), (6000, 784)])
+def test_pack_size_layers_at_their_real_size(oracle_lib, K, N):
+    import cutagi_amd.functional as F
+    B = 16
+    d = linear_inputs(K, N, B, seed=K + N, bias=True, jcb_random=True)
+    t = _dev(d)
+    z = F.linear_fwd(t["mu_w"], t["var_w"], t["mu_b"], t["var_b"], t["mu_a"], t["var_a"])
+    ref = oracle_lib.linear_fwd(d["mu_w"], d["var_w"], d["mu_b"], d["var_b"], d["mu_a"],
+                                d["var_a"], threads=8)
+    assert_close(z[0].cpu().numpy(), ref[0], "mu_z")
+    assert_close(z[1].cpu().numpy(), ref[1], "var_z", same_sign=True)
+    out = F.linear_bwd(t["mu_w"], t["var_w"], t["var_b"], t["mu_a"], t["jcb"], t["delta_mu"],
+                       t["delta_var"])
+    want = (oracle_lib.linear_bwd_dz(d["mu_w"], d["jcb"], d["delta_mu"], d["delta_var"], threads=8)
+            + oracle_lib.linear_bwd_dw(d["var_w"], d["mu_a"], d["delta_mu"], d["delta_var"], threads=8)
+            + oracle_lib.linear_bwd_db(d["var_b"], d["delta_mu"], d["delta_var"]))
+    names = ["delta_mu_z", "delta_var_z", "delta_mu_w", "delta_var_w", "delta_mu_b", "delta_var_b"]
+    for name, got, r in zip(names, out, want):
+        assert_close(got.cpu().numpy(), r, name, same_sign=name in SAME_SIGN)
+
+
+def test_pack_size_network_at_its_real_size():
+    from cutagi_amd import cutagi
+    cutagi.manual_seed(0)
+    net = cutagi.Sequential([cutagi.Linear(785, 6000), cutagi.ReLU(), cutagi.Linear(6000, 784)])
+    net.to_device("cuda")
+    updater = cutagi.OutputUpdater(net.device)
+    rng = np.random.default_rng(0)
+    B = 16
+    x = rng.uniform(0, 1, (B, 785)).astype(np.float32)
+    y = rng.uniform(0, 1, B * 784).astype(np.float32)
+    var_y = np.ones(B * 784, np.float32)
+    before = {k: [np.array(a) for a in v] for k, v in net.state_dict().items()}
+    net.forward(x)
+    mu, var = net.get_outputs()
+    updater.update(net.output_z_buffer, y, var_y, net.input_delta_z_buffer)
+    net.backward()
+    net.step()
+    assert mu.size == B * 784 and np.all(np.isfinite(mu)) and var.min() >= 0
+    after = net.state_dict()
+    for key, arrays in after.items():
+        for a, b in zip(arrays, before[key]):
+            a = np.asarray(a)
+            assert np.all(np.isfinite(a))
+        # the step moved the weight means and shrank no variance below zero
+        assert not np.array_equal(np.asarray(arrays[0]), before[key][0])
+        assert np.asarray(arrays[1]).min() >= 0

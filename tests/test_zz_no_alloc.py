@@ -83,3 +83,43 @@ def test_static_forward_rejects_what_does_not_fit():
     torch.cuda.synchronize()
     assert rc == capi.ERR_UNSUPPORTED
     assert float(mu_z.min()) == 7.0 and float(var_z.max()) == 7.0
+
+
+def test_static_forward_allocates_no_device_memory():
+    """The property the entry point exists for. On a stream that has never been used
+    with the library (so it owns no workspace), a sliced shape runs through the static
+    entry point without the free device memory moving; the regular entry point, called
+    on such a stream, does grow a workspace - which shows that the probe would see an
+    allocation."""
+    import torch
+    from cutagi_amd import capi
+    K, N, B = 4096, 2048, 256        # eight reduction slices: 32 MiB of partial sums
+    d = linear_inputs(K, N, B, seed=5, bias=True)
+    t = {k: torch.from_numpy(v).cuda() for k, v in d.items()}
+    mu_z, var_z = torch.empty((B, N), device="cuda"), torch.empty((B, N), device="cuda")
+    want_mu, want_var = torch.empty_like(mu_z), torch.empty_like(var_z)
+    args = [capi.ptr(t[k]) for k in ("mu_w", "var_w", "mu_b", "var_b", "mu_a", "var_a")] + [K, N, B, 1]
+    # first use of the static array on this device (address look-up) happens here
+    capi.check(capi.lib.tagi_linear_fwd_static(*args, capi.ptr(want_mu), capi.ptr(want_var), None))
+    torch.cuda.synchronize()
+
+    # a stream's first launch makes the runtime set up its queue (device memory of its
+    # own): let both streams run something that is not this library first
+    fresh, other = torch.cuda.Stream(), torch.cuda.Stream()
+    dummy = torch.zeros(1024, device="cuda")
+    for s in (fresh, other):
+        with torch.cuda.stream(s):
+            dummy.add_(1.0)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    capi.check(capi.lib.tagi_linear_fwd_static(*args, capi.ptr(mu_z), capi.ptr(var_z),
+                                               fresh.cuda_stream))
+    fresh.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "the static entry point allocated"
+    assert torch.equal(mu_z, want_mu) and torch.equal(var_z, want_var)
+
+    free_before = torch.cuda.mem_get_info()[0]
+    capi.check(capi.lib.tagi_linear_fwd(*args, capi.ptr(mu_z), capi.ptr(var_z), other.cuda_stream))
+    other.synchronize()
+    assert torch.cuda.mem_get_info()[0] < free_before, "probe insensitive: no workspace grew"
+    assert torch.equal(mu_z, want_mu)
