@@ -2,6 +2,8 @@
 // network: MixtureReLU, BatchNorm2d (statistics, normalisation, backward),
 // AvgPool2d and the residual adds. All of them are bandwidth-bound passes over
 // [B][channels][pixels] tensors; gfx950.
+#include <cstdint>
+
 #include "tagi_internal.h"
 #include "tagi_activation.h"
 
@@ -13,6 +15,8 @@ constexpr int TPB = 256;
 inline unsigned blocks_for(size_t n, int per_block) {
     return (unsigned)((n + per_block - 1) / per_block);
 }
+// (a null pointer counts as aligned: optional operands)
+inline bool aligned16(const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; }
 
 // ---------------------------------------------------------------------------
 // MixtureReLU: moments of max(z, 0) for z ~ N(mu, var), floored at 1e-6; the
@@ -62,6 +66,9 @@ __device__ __forceinline__ void block_sum(float (&v)[NV], float (*s)[TPB / 64]) 
 // channel are merged pairwise in index order (Chan et al.), which keeps the
 // two-pass accuracy of the reference's "mean first, then deviations".
 // ---------------------------------------------------------------------------
+// (VEC: wihi % 4 == 0 and 16-byte aligned arrays: four pixels of one channel map per
+// load, two loads in flight per array)
+template <bool VEC>
 __global__ __launch_bounds__(TPB) void bn_stats_partial_kernel(
     const float *__restrict__ mu_a, const float *__restrict__ var_a, int wihi, int fi, int B,
     int b_per_chunk, float *__restrict__ part) {
@@ -71,21 +78,43 @@ __global__ __launch_bounds__(TPB) void bn_stats_partial_kernel(
     const int count = max(0, b_hi - b_lo) * wihi;
 
     float v[2] = {0.f, 0.f};
-    for (int i = threadIdx.x; i < count; i += TPB) {
-        const int b = b_lo + i / wihi, p = i % wihi;
-        const size_t at = ((size_t)b * fi + c) * wihi + p;
-        v[0] += mu_a[at];
-        v[1] += var_a[at];
+    if (VEC) {
+        const int w4 = wihi >> 2, n4 = count >> 2;
+        for (int i = threadIdx.x; i < n4; i += TPB) {
+            const int b = b_lo + i / w4, p = (i % w4) * 4;
+            const size_t at = ((size_t)b * fi + c) * wihi + p;
+            const float4 m = *reinterpret_cast<const float4 *>(mu_a + at);
+            const float4 q = *reinterpret_cast<const float4 *>(var_a + at);
+            v[0] += (m.x + m.y) + (m.z + m.w);
+            v[1] += (q.x + q.y) + (q.z + q.w);
+        }
+    } else {
+        for (int i = threadIdx.x; i < count; i += TPB) {
+            const int b = b_lo + i / wihi, p = i % wihi;
+            const size_t at = ((size_t)b * fi + c) * wihi + p;
+            v[0] += mu_a[at];
+            v[1] += var_a[at];
+        }
     }
     block_sum<2>(v, s);
     const float mean = count > 0 ? v[0] / count : 0.f;
     const float sum_var = v[1];
 
     float d[1] = {0.f};
-    for (int i = threadIdx.x; i < count; i += TPB) {
-        const int b = b_lo + i / wihi, p = i % wihi;
-        const float x = mu_a[((size_t)b * fi + c) * wihi + p] - mean;
-        d[0] += x * x;
+    if (VEC) {
+        const int w4 = wihi >> 2, n4 = count >> 2;
+        for (int i = threadIdx.x; i < n4; i += TPB) {
+            const int b = b_lo + i / w4, p = (i % w4) * 4;
+            const float4 m = *reinterpret_cast<const float4 *>(mu_a + ((size_t)b * fi + c) * wihi + p);
+            const float x0 = m.x - mean, x1 = m.y - mean, x2 = m.z - mean, x3 = m.w - mean;
+            d[0] += (x0 * x0 + x1 * x1) + (x2 * x2 + x3 * x3);
+        }
+    } else {
+        for (int i = threadIdx.x; i < count; i += TPB) {
+            const int b = b_lo + i / wihi, p = i % wihi;
+            const float x = mu_a[((size_t)b * fi + c) * wihi + p] - mean;
+            d[0] += x * x;
+        }
     }
     block_sum<1>(d, s);
     if (threadIdx.x == 0) {
@@ -151,8 +180,55 @@ __global__ __launch_bounds__(TPB) void bn_fwd_kernel(
     var_z[i] = vz;
 }
 
+// The same for four consecutive pixels of one channel map per thread (wihi % 4 == 0,
+// 16-byte aligned arrays).
+__global__ __launch_bounds__(TPB) void bn_fwd_vec_kernel(
+    const float *__restrict__ mu_w, const float *__restrict__ var_w,
+    const float *__restrict__ mu_b, const float *__restrict__ var_b,
+    const float *__restrict__ mu_a, const float *__restrict__ var_a,
+    const float *__restrict__ mu_norm, const float *__restrict__ var_norm, float epsilon,
+    int wihi, int fi, size_t n4, const float *__restrict__ mu_res,
+    const float *__restrict__ var_res, float *__restrict__ mu_z, float *__restrict__ var_z) {
+    const size_t i4 = (size_t)blockIdx.x * TPB + threadIdx.x;
+    if (i4 >= n4) return;
+    const size_t i = i4 * 4;
+    const int c = (int)((i / wihi) % fi);
+    const float4 ma = *reinterpret_cast<const float4 *>(mu_a + i);
+    const float4 va = *reinterpret_cast<const float4 *>(var_a + i);
+    float4 rm = make_float4(0.f, 0.f, 0.f, 0.f), rv = rm;
+    if (mu_res != nullptr) {
+        rm = *reinterpret_cast<const float4 *>(mu_res + i);
+        rv = *reinterpret_cast<const float4 *>(var_res + i);
+    }
+    const float inv = 1.0f / sqrtf(var_norm[c] + epsilon);
+    const float mw = mu_w[c], vw = var_w[c], mean = mu_norm[c];
+    const float bm = mu_b != nullptr ? mu_b[c] : 0.f, bv = mu_b != nullptr ? var_b[c] : 0.f;
+    const bool has_b = mu_b != nullptr, has_r = mu_res != nullptr;
+    auto one = [&](float a, float v, float r0, float r1, float &mz, float &vz) {
+        const float d = a - mean;
+        mz = inv * d * mw;
+        vz = inv * inv * (v * (mw * mw + vw) + vw * d * d);
+        if (has_b) {
+            mz += bm;
+            vz += bv;
+        }
+        if (has_r) {
+            mz += r0;
+            vz += r1;
+        }
+    };
+    float4 om, ov;
+    one(ma.x, va.x, rm.x, rv.x, om.x, ov.x);
+    one(ma.y, va.y, rm.y, rv.y, om.y, ov.y);
+    one(ma.z, va.z, rm.z, rv.z, om.z, ov.z);
+    one(ma.w, va.w, rm.w, rv.w, om.w, ov.w);
+    *reinterpret_cast<float4 *>(mu_z + i) = om;
+    *reinterpret_cast<float4 *>(var_z + i) = ov;
+}
+
 // Backward of one (chunk, channel): the state innovations element by element,
 // and partial sums of the four parameter innovations of the channel.
+template <bool VEC>
 __global__ __launch_bounds__(TPB) void bn_bwd_partial_kernel(
     const float *__restrict__ mu_w, const float *__restrict__ var_w,
     const float *__restrict__ mu_a, const float *__restrict__ jcb,
@@ -168,21 +244,49 @@ __global__ __launch_bounds__(TPB) void bn_bwd_partial_kernel(
     const float mean = mu_norm[c], mw = mu_w[c], vw = var_w[c];
 
     float v[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int i = threadIdx.x; i < count; i += TPB) {
-        const int b = b_lo + i / wihi, p = i % wihi;
-        const size_t at = ((size_t)b * fi + c) * wihi + p;
-        const float dm = dmu_out[at], dv = dvar_out[at];
-        if (state_update) {
-            const float t = inv * mw * jcb[at];
-            dmu[at] = t * dm;
-            dvar[at] = t * dv * t;
+    if (VEC) {
+        const int w4 = wihi >> 2, n4 = count >> 2;
+        const float sj = inv * mw, sp = inv * vw;
+        for (int i = threadIdx.x; i < n4; i += TPB) {
+            const int b = b_lo + i / w4, p = (i % w4) * 4;
+            const size_t at = ((size_t)b * fi + c) * wihi + p;
+            const float4 dm = *reinterpret_cast<const float4 *>(dmu_out + at);
+            const float4 dv = *reinterpret_cast<const float4 *>(dvar_out + at);
+            if (state_update) {
+                const float4 j = *reinterpret_cast<const float4 *>(jcb + at);
+                const float t0 = sj * j.x, t1 = sj * j.y, t2 = sj * j.z, t3 = sj * j.w;
+                *reinterpret_cast<float4 *>(dmu + at) =
+                    make_float4(t0 * dm.x, t1 * dm.y, t2 * dm.z, t3 * dm.w);
+                *reinterpret_cast<float4 *>(dvar + at) =
+                    make_float4(t0 * dv.x * t0, t1 * dv.y * t1, t2 * dv.z * t2, t3 * dv.w * t3);
+            }
+            if (param_update) {
+                const float4 a = *reinterpret_cast<const float4 *>(mu_a + at);
+                const float t0 = sp * (a.x - mean), t1 = sp * (a.y - mean), t2 = sp * (a.z - mean),
+                            t3 = sp * (a.w - mean);
+                v[0] += (t0 * dm.x + t1 * dm.y) + (t2 * dm.z + t3 * dm.w);
+                v[1] += (t0 * dv.x * t0 + t1 * dv.y * t1) + (t2 * dv.z * t2 + t3 * dv.w * t3);
+                v[2] += (dm.x + dm.y) + (dm.z + dm.w);
+                v[3] += (dv.x + dv.y) + (dv.z + dv.w);
+            }
         }
-        if (param_update) {
-            const float t = inv * (mu_a[at] - mean) * vw;
-            v[0] += t * dm;
-            v[1] += t * dv * t;
-            v[2] += dm;
-            v[3] += dv;
+    } else {
+        for (int i = threadIdx.x; i < count; i += TPB) {
+            const int b = b_lo + i / wihi, p = i % wihi;
+            const size_t at = ((size_t)b * fi + c) * wihi + p;
+            const float dm = dmu_out[at], dv = dvar_out[at];
+            if (state_update) {
+                const float t = inv * mw * jcb[at];
+                dmu[at] = t * dm;
+                dvar[at] = t * dv * t;
+            }
+            if (param_update) {
+                const float t = inv * (mu_a[at] - mean) * vw;
+                v[0] += t * dm;
+                v[1] += t * dv * t;
+                v[2] += dm;
+                v[3] += dv;
+            }
         }
     }
     if (!param_update) return;
@@ -326,8 +430,12 @@ hipError_t launch_batchnorm2d_stats(const float *mu_a, const float *var_a, int w
                                     hipStream_t stream) {
     int per = 0;
     const int chunks = bn_chunks(fi, B, &per);
-    hipLaunchKernelGGL(bn_stats_partial_kernel, dim3(chunks, fi), dim3(TPB), 0, stream, mu_a,
-                       var_a, wihi, fi, B, per, scratch);
+    if (wihi % 4 == 0 && aligned16(mu_a) && aligned16(var_a))
+        hipLaunchKernelGGL(bn_stats_partial_kernel<true>, dim3(chunks, fi), dim3(TPB), 0, stream,
+                           mu_a, var_a, wihi, fi, B, per, scratch);
+    else
+        hipLaunchKernelGGL(bn_stats_partial_kernel<false>, dim3(chunks, fi), dim3(TPB), 0, stream,
+                           mu_a, var_a, wihi, fi, B, per, scratch);
     hipLaunchKernelGGL(bn_stats_final_kernel, dim3((fi + 63) / 64), dim3(64), 0, stream, scratch,
                        fi, chunks, momentum, mu_s, var_s, mu_ra, var_ra);
     return hipGetLastError();
@@ -339,6 +447,13 @@ hipError_t launch_batchnorm2d_fwd(const float *mu_w, const float *var_w, const f
                                   int wihi, int fi, int B, float *mu_z, float *var_z,
                                   hipStream_t stream, const float *mu_res, const float *var_res) {
     const size_t n = (size_t)B * fi * wihi;
+    if (wihi % 4 == 0 && aligned16(mu_a) && aligned16(var_a) && aligned16(mu_z) && aligned16(var_z) &&
+        aligned16(mu_res) && aligned16(var_res)) {
+        hipLaunchKernelGGL(bn_fwd_vec_kernel, dim3(blocks_for(n / 4, TPB)), dim3(TPB), 0, stream,
+                           mu_w, var_w, mu_b, var_b, mu_a, var_a, mu_norm, var_norm, epsilon, wihi,
+                           fi, n / 4, mu_res, var_res, mu_z, var_z);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(bn_fwd_kernel, dim3(blocks_for(n, TPB)), dim3(TPB), 0, stream, mu_w, var_w,
                        mu_b, var_b, mu_a, var_a, mu_norm, var_norm, epsilon, wihi, fi, n, mu_res,
                        var_res, mu_z, var_z);
@@ -354,9 +469,17 @@ hipError_t launch_batchnorm2d_bwd(const float *mu_w, const float *var_w, const f
                                   float *dvar_b, hipStream_t stream) {
     int per = 0;
     const int chunks = bn_chunks(fi, B, &per);
-    hipLaunchKernelGGL(bn_bwd_partial_kernel, dim3(chunks, fi), dim3(TPB), 0, stream, mu_w, var_w,
-                       mu_a, jcb, mu_norm, var_norm, dmu_out, dvar_out, epsilon, wihi, fi, B, per,
-                       state_update, param_update, dmu, dvar, scratch);
+    const bool vec = wihi % 4 == 0 && aligned16(dmu_out) && aligned16(dvar_out) &&
+                     (!state_update || (aligned16(jcb) && aligned16(dmu) && aligned16(dvar))) &&
+                     (!param_update || aligned16(mu_a));
+    if (vec)
+        hipLaunchKernelGGL(bn_bwd_partial_kernel<true>, dim3(chunks, fi), dim3(TPB), 0, stream, mu_w,
+                           var_w, mu_a, jcb, mu_norm, var_norm, dmu_out, dvar_out, epsilon, wihi,
+                           fi, B, per, state_update, param_update, dmu, dvar, scratch);
+    else
+        hipLaunchKernelGGL(bn_bwd_partial_kernel<false>, dim3(chunks, fi), dim3(TPB), 0, stream,
+                           mu_w, var_w, mu_a, jcb, mu_norm, var_norm, dmu_out, dvar_out, epsilon,
+                           wihi, fi, B, per, state_update, param_update, dmu, dvar, scratch);
     if (param_update)
         hipLaunchKernelGGL(bn_bwd_final_kernel, dim3((fi + 63) / 64), dim3(64), 0, stream, scratch,
                            var_b, fi, chunks, dmu_w, dvar_w, dmu_b, dvar_b);
