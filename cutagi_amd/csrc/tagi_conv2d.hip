@@ -666,6 +666,7 @@ struct ConvDzProblem {
 }  // namespace tagi
 
 #include "tagi_conv_stencil.h"
+#include "tagi_conv_stencil_s2.h"
 
 namespace tagi {
 namespace {
@@ -755,18 +756,20 @@ inline int lcm_int(int a, int b) {
     return a / x * b;
 }
 
+// `stencil_s2`: output map width when the strided state-backward stencil kernel applies.
 template <class P, bool DZ>
 hipError_t run_sliced(int tile, int splits, int stencil, float *ws0, float *ws1, ConvParams &p,
-                      hipStream_t stream) {
+                      hipStream_t stream, int stencil_s2 = 0) {
     // the state backward re-states its slices per tile in whole output channels
-    const int unit = stencil ? 288 : DZ ? lcm_int(KT, p.k2) : KT;
+    const int unit = (stencil || stencil_s2) ? 288 : DZ ? lcm_int(KT, p.k2) : KT;
     const int per = ceil_div(ceil_div(p.R, splits), unit) * unit;
     p.splits = ceil_div(p.R, per);
     p.r_per_split = per;
     p.ws0 = ws0;
     p.ws1 = ws1;
-    hipError_t e = stencil ? launch_conv_stencil<DZ>(stencil, p, stream)
-                           : launch_tiles<P>(tile, p, stream);
+    hipError_t e = stencil_s2 ? launch_conv_stencil_s2_dz(stencil_s2, p, stream)
+                   : stencil  ? launch_conv_stencil<DZ>(stencil, p, stream)
+                              : launch_tiles<P>(tile, p, stream);
     if (e != hipSuccess || p.splits == 1) return e;
     return launch_reduce_store<P>(p, stream);
 }
@@ -829,7 +832,13 @@ hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float
     if (g_conv2d_stencil && ki == 3 && nr == 9 && woho == wihi && fo % 8 == 0 && fi % 64 == 0 &&
         tile == TILE_64x128 && aligned16(mu_w) && aligned16(dmu) && aligned16(dvar))
         stencil = stencil_width(wihi);
-    return run_sliced<ConvDzProblem, true>(tile, splits, stencil, ws0, ws1, p, stream);
+    // 3x3, stride 2, padding on the right and bottom (the kernel verifies the tables)
+    int stencil_s2 = 0;
+    if (g_conv2d_stencil && ki == 3 && nr == 4 && wihi == 4 * woho && p.perm_s == 2 &&
+        fo % 32 == 0 && fi % 64 == 0 && tile == TILE_64x128 && ((long long)B * woho) % 128 == 0 &&
+        aligned16(dmu) && aligned16(dvar))
+        stencil_s2 = s2_out_width(woho);
+    return run_sliced<ConvDzProblem, true>(tile, splits, stencil, ws0, ws1, p, stream, stencil_s2);
 }
 
 // Workgroups of the weight-backward kernel that one CU holds at a time.

@@ -30,6 +30,11 @@ GEOMS = [
     (3, 1, 1, 1, 16, 64, 128, 3),
     (3, 1, 1, 1, 8, 128, 64, 3),  # two images per tile, last tile half empty
     (3, 1, 1, 1, 4, 320, 64, 5),  # eight images per tile, one partial tile, sliced reduction
+    # 3x3 s2 with right/bottom padding and whole groups of channels: the strided stencil kernels
+    (3, 2, 1, 2, 32, 64, 64, 1),   # 16x16 output maps, half an image per tile
+    (3, 2, 1, 2, 16, 128, 96, 2),  # 8x8 output maps, two images per tile
+    (3, 2, 1, 2, 8, 64, 160, 8),   # 4x4 output maps, eight images per tile
+    (3, 2, 1, 2, 16, 64, 640, 2),  # long reduction: sliced
 ]
 
 
@@ -184,8 +189,83 @@ def test_conv2d_stencil_kernels_agree_with_the_table_path():
         assert not np.array_equal(a, b), name
 
 
+def test_conv2d_strided_stencil_kernels_agree_with_the_table_path():
+    """3x3 stride 2: the same inputs through the strided stencil kernels and, with the
+    stencil kernels switched off, through the table-driven ones."""
+    import torch
+    import cutagi_amd.functional as F
+    from cutagi_amd import capi
+    k, wi, fi, fo, B = 3, 16, 64, 64, 4
+    idx = capi.conv2d_build_idx(k, 2, wi, wi, 1, 2, k * k * fi * fo + 1)
+    wihi, woho = wi * wi, idx["wo"] * idx["ho"]
+    d = conv_inputs(fi, fo, k, wihi, woho, B, seed=2, bias=True, jcb_random=True)
+    t = {n: torch.from_numpy(v).cuda() for n, v in d.items()}
+    ti = {n: torch.from_numpy(idx[n]).cuda() for n in ("Fmwa_2", "FCzwa_1", "Szz_ud")}
+    out = {}
+    try:
+        for mode in (1, 0):
+            capi.tune("conv2d.stencil", mode)
+            z = F.conv2d_fwd(t["mu_w"], t["var_w"], t["mu_b"], t["var_b"], t["mu_a"], t["var_a"],
+                             ti["Fmwa_2"], woho, fo, wihi, fi, k, B)
+            dz = F.conv2d_bwd_dz(t["mu_w"], t["jcb"], t["delta_mu"], t["delta_var"], ti["FCzwa_1"],
+                                 ti["Szz_ud"], woho, fo, wihi, fi, k, idx["h"], B)
+            dw = F.conv2d_bwd_dw(t["var_w"], t["var_b"], t["mu_a"], t["delta_mu"], t["delta_var"],
+                                 ti["Fmwa_2"], B, fo, woho, wihi, fi, k)
+            out[mode] = [x.cpu().numpy() for x in (*z, *dz, *dw[:2])]
+    finally:
+        capi.tune("conv2d.stencil", 1)
+    switched = []
+    for name, a, b in zip(("mu_z", "var_z", "delta_mu_z", "delta_var_z", "delta_mu_w",
+                           "delta_var_w"), out[1], out[0]):
+        assert_close(a, b, name, same_sign=name in SAME_SIGN)
+        if not np.array_equal(a, b):
+            switched.append(name)
+    # a different summation order shows that the switch switched the state backward
+    assert "delta_mu_z" in switched
+
+
+def test_conv2d_strided_tables_of_another_geometry_take_the_table_path(oracle_lib):
+    """The strided stencil kernel is chosen by sizes (3x3, four input pixels per output
+    pixel, lists of four occurrences) and checks the tables it is given. Here the
+    tables of the right geometry are altered: the first two occurrences of every
+    pixel's list trade places (still the same contraction, which the check accepts in
+    any order) and one pixel's list names a wrong output pixel (a different
+    contraction, which sends that tile to the table-driven loop). The result must be
+    what the tables say."""
+    import torch
+    import cutagi_amd.functional as F
+    from cutagi_amd import capi
+    k, wi, fi, fo, B = 3, 16, 64, 32, 2
+    idx = capi.conv2d_build_idx(k, 2, wi, wi, 1, 2, k * k * fi * fo + 1)
+    wihi, woho, h = wi * wi, idx["wo"] * idx["ho"], idx["h"]
+    assert h == 4
+    zw = idx["FCzwa_1"].reshape(wihi, h).copy()
+    zud = idx["Szz_ud"].reshape(h, wihi).copy()
+    # (a) reorder: swap the first two occurrences of every pixel that has two
+    two = zud[1] > -1
+    zw[two, 0], zw[two, 1] = zw[two, 1].copy(), zw[two, 0].copy()
+    zud[0, two], zud[1, two] = zud[1, two].copy(), zud[0, two].copy()
+    # (b) one wrong entry: pixel 37 takes its first tap from another output pixel
+    zud[0, 37] = (zud[0, 37] % woho) + 1
+    d = conv_inputs(fi, fo, k, wihi, woho, B, seed=9, bias=False, jcb_random=True)
+    t = {n: (None if v is None else torch.from_numpy(v).cuda()) for n, v in d.items()}
+    zw_f, zud_f = np.ascontiguousarray(zw.ravel()), np.ascontiguousarray(zud.ravel())
+    dz = F.conv2d_bwd_dz(t["mu_w"], t["jcb"], t["delta_mu"], t["delta_var"],
+                         torch.from_numpy(zw_f).cuda(), torch.from_numpy(zud_f).cuda(), woho, fo,
+                         wihi, fi, k, h, B)
+    ref = oracle_lib.conv2d_bwd_dz(d["mu_w"], d["jcb"], d["delta_mu"], d["delta_var"], zw_f, zud_f,
+                                   woho, fo, wihi, fi, k, h, B, threads=4)
+    assert_close(dz[0].cpu().numpy(), ref[0], "delta_mu_z")
+    assert_close(dz[1].cpu().numpy(), ref[1], "delta_var_z", same_sign=True)
+    # and the corruption did change the contraction
+    clean = oracle_lib.conv2d_bwd_dz(d["mu_w"], d["jcb"], d["delta_mu"], d["delta_var"],
+                                     idx["FCzwa_1"], idx["Szz_ud"], woho, fo, wihi, fi, k, h, B,
+                                     threads=4)
+    assert not np.array_equal(clean[0], ref[0])
+
+
 @pytest.mark.parametrize("geom", [(3, 2, 1, 2, 16, 16, 64, 4), (2, 2, 0, 1, 8, 64, 32, 3),
-                                  (3, 2, 1, 2, 4, 8, 8, 2)])
+                                  (3, 2, 1, 2, 4, 8, 8, 2), (3, 2, 1, 2, 16, 64, 64, 2)])
 def test_conv2d_state_backward_column_orders_agree(oracle_lib, geom):
     """Strided layers: columns numbered phase by phase (default) and in natural
     order give the oracle's result both; the order only decides which taps a tile
@@ -224,7 +304,7 @@ def test_conv2d_kernel_too_large_for_the_tap_table_is_refused():
 
 # stencil kernel, table-driven strided kernel (phase order), sliced reduction
 RES_GEOMS = [(3, 1, 1, 1, 8, 64, 64, 3), (3, 2, 1, 2, 8, 8, 16, 4), (3, 1, 1, 1, 4, 128, 96, 3),
-             (3, 1, 1, 1, 6, 5, 7, 2)]
+             (3, 1, 1, 1, 6, 5, 7, 2), (3, 2, 1, 2, 16, 64, 64, 2)]
 
 
 @pytest.mark.parametrize("geom", RES_GEOMS)
