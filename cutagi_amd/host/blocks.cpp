@@ -496,8 +496,10 @@ void LayerBlock::eval() {
 // two objects trade contents.
 void LayerBlock::forward(BaseHiddenStates &input_states, BaseHiddenStates &output_states,
                          BaseTempStates &temp_states) {
+    BaseHiddenStates *first = this->first_input;  // one-shot: taken before anything can throw
+    this->first_input = nullptr;
     BaseHiddenStates *in = &input_states, *out = &output_states;
-    const size_t batch_size = input_states.block_size;
+    const size_t batch_size = first != nullptr ? first->block_size : input_states.block_size;
     size_t passes = 0;
     for (size_t i = 0; i < layers.size(); i++, passes++) {
         // an activation that follows a Linear / Conv2d layer runs in that layer's epilogue
@@ -505,7 +507,7 @@ void LayerBlock::forward(BaseHiddenStates &input_states, BaseHiddenStates &outpu
                             ? fusable_activation(layers[i].get(), layers[i + 1].get())
                             : 0;
         layers[i]->fused_activation = act;
-        layers[i]->forward(*in, *out, temp_states);
+        layers[i]->forward(i == 0 && first != nullptr ? *first : *in, *out, temp_states);
         if (act != 0) activation_absorbed(layers[++i].get(), *out);
         std::swap(in, out);
     }
@@ -517,14 +519,20 @@ void LayerBlock::forward(BaseHiddenStates &input_states, BaseHiddenStates &outpu
 void LayerBlock::backward(BaseDeltaStates &input_delta_states,
                           BaseDeltaStates &output_delta_states, BaseTempStates &temp_states,
                           bool state_update) {
+    // (one-shot request: the innovations arrive in another object than the first buffer)
+    BaseDeltaStates *src = this->first_delta_input != nullptr ? this->first_delta_input
+                                                              : &input_delta_states;
+    this->first_delta_input = nullptr;
     for (auto it = layers.rbegin(); it != layers.rend() - 1; ++it) {
         BaseLayer *layer = it->get();
-        layer->backward(input_delta_states, output_delta_states, temp_states);
-        if (layer->get_layer_type() != LayerType::Activation)
+        layer->backward(*src, output_delta_states, temp_states);
+        if (layer->get_layer_type() != LayerType::Activation) {
             input_delta_states.swap(output_delta_states);
+            src = &input_delta_states;
+        }
     }
     if (state_update && layers.size() > 1)
-        layers[0]->backward(input_delta_states, output_delta_states, temp_states, state_update);
+        layers[0]->backward(*src, output_delta_states, temp_states, state_update);
     if (layers[0]->get_layer_type() == LayerType::Activation || !state_update ||
         layers.size() == 1)
         output_delta_states.swap(input_delta_states);
@@ -715,22 +723,32 @@ void ResNetBlock::eval() {
 
 // reference: init_input_buffer / init_shortcut_state / init_shortcut_delta_state,
 // src/resnet_block_cuda.cu:106-139
-void ResNetBlock::init_buffers() {
-    int states = (int)this->input_size;
-    if (shortcut) states = std::max(states, shortcut->get_max_num_states());
-    states = std::max(states, (int)this->output_size);
-    const size_t size = (size_t)states * batch_size_;
+void ResNetBlock::init_buffers(size_t size) {
+    if (size == 0) {
+        int states = (int)this->input_size;
+        if (shortcut) states = std::max(states, shortcut->get_max_num_states());
+        states = std::max(states, (int)this->output_size);
+        size = (size_t)states * batch_size_;
+    }
+    buffer_size_ = size;
     input_z = std::make_shared<HiddenStateHip>(size, batch_size_, device_idx);
     input_delta_z = std::make_shared<DeltaStateHip>(size, batch_size_, device_idx);
     if (shortcut) {
         shortcut_output_z = std::make_shared<HiddenStateHip>(size, batch_size_, device_idx);
-        // the shortcut's layers ping-pong between these two; nothing else reads them
-        // once the shortcut has run, so its layers may keep their arrays
-        as<HiddenStateHip>(*input_z)->transient = true;
+        // the shortcut's layers ping-pong between this buffer and another one that nothing
+        // else reads once the shortcut has run, so its layers may keep their arrays
         as<HiddenStateHip>(*shortcut_output_z)->transient = true;
         if (training)
             shortcut_output_delta_z = std::make_shared<DeltaStateHip>(size, batch_size_, device_idx);
     }
+}
+
+bool ResNetBlock::can_trade() const {
+    auto *m = dynamic_cast<LayerBlock *>(main_block.get());
+    if (m == nullptr || m->layers.size() < 2) return false;
+    if (!shortcut) return true;
+    auto *sc = dynamic_cast<LayerBlock *>(shortcut.get());
+    return sc != nullptr && sc->layers.size() >= 2;
 }
 
 // reference: ResNetBlockCuda::forward, src/resnet_block_cuda.cu:211-299
@@ -739,33 +757,54 @@ void ResNetBlock::forward(BaseHiddenStates &input_states, BaseHiddenStates &outp
     if (!on_device) no_cpu_path("forward");
     auto *in = as<HiddenStateHip>(input_states);
     const int batch_size = (int)input_states.block_size;
-    if (batch_size != batch_size_) {
+    // The block keeps its input for the shortcut (the reference copies it: mu_a, var_a,
+    // jcb, and once more into the block's bwd_states). Where the input arrives in a
+    // ping-pong buffer of the enclosing network, and both branches can be told where to
+    // read (LayerBlocks), the block TRADES arrays with that buffer instead: its own
+    // state object (as large as the buffer) takes the input, the buffer takes the
+    // block's arrays of the previous step and serves on as scratch. Nothing is copied,
+    // and the first layers of both branches borrow the kept arrays for their backward.
+    const bool trade = in->transient && this->can_trade();
+    const size_t want = trade ? in->size : 0;
+    if (batch_size != batch_size_ || !input_z || (trade && buffer_size_ != want) ||
+        (training && shortcut && !shortcut_output_delta_z)) {
         batch_size_ = batch_size;
-        this->init_buffers();
+        this->init_buffers(want);
     }
-    if (training && shortcut && !shortcut_output_delta_z) this->init_buffers();
-    // input_z keeps the block's input for the shortcut; its Jacobian is also what
-    // the identity shortcut's backward needs (the reference copies mu_a and jcb
-    // once more into the block's bwd_states: two transfers per block saved here)
-    input_z->copy_from(input_states, (int)(this->input_size * batch_size));
-    // The shortcut runs first (it reads the copy), so that a main block that ends on a
-    // BatchNorm2d layer can add the shortcut's output in that layer's pass instead of
-    // in a pass of its own.
+    auto *kept = as<HiddenStateHip>(*input_z);
+    auto *main_lb = dynamic_cast<LayerBlock *>(main_block.get());
+    if (trade) {
+        kept->swap(input_states);
+        kept->stable = true;
+        kept->transient = false;
+    } else {
+        kept->stable = false;
+        kept->transient = shortcut != nullptr;  // read by the shortcut only, then dead
+        input_z->copy_from(input_states, (int)(this->input_size * batch_size));
+    }
+    // The shortcut runs first, so that a main block that ends on a BatchNorm2d layer can
+    // add the shortcut's output in that layer's pass instead of in a pass of its own.
     HiddenStateHip *sc = nullptr;
     if (shortcut) {
-        shortcut->forward(*input_z, *shortcut_output_z, temp_states);
+        if (trade) {
+            // first layer reads the kept input; the traded-away buffer is its scratch
+            dynamic_cast<LayerBlock *>(shortcut.get())->first_input = input_z.get();
+            shortcut->forward(input_states, *shortcut_output_z, temp_states);
+        } else {
+            shortcut->forward(*input_z, *shortcut_output_z, temp_states);
+        }
         sc = as<HiddenStateHip>(*shortcut_output_z);
     } else {
-        sc = as<HiddenStateHip>(*input_z);
+        sc = kept;
     }
     BatchNorm2dHip *closing = nullptr;
-    if (auto *block = dynamic_cast<LayerBlock *>(main_block.get()))
-        if (!block->layers.empty())
-            closing = dynamic_cast<BatchNorm2dHip *>(block->layers.back().get());
+    if (main_lb != nullptr && !main_lb->layers.empty())
+        closing = dynamic_cast<BatchNorm2dHip *>(main_lb->layers.back().get());
     if (closing != nullptr) {
         closing->residual_mu = sc->d_mu_a;
         closing->residual_var = sc->d_var_a;
     }
+    if (trade) main_lb->first_input = input_z.get();
     main_block->forward(input_states, output_states, temp_states);
 
     auto *out = as<HiddenStateHip>(output_states);
@@ -783,24 +822,40 @@ void ResNetBlock::backward(BaseDeltaStates &input_delta_states,
                            bool state_update) {
     if (!on_device) no_cpu_path("backward");
     const int batch_size = (int)input_delta_states.block_size;
-    input_delta_z->copy_from(input_delta_states, (int)(this->output_size * batch_size));
+    // As in forward(): the incoming innovations are needed by both branches; trade arrays
+    // with the buffer they arrive in where both branches can be told where to read.
+    auto *din = as<DeltaStateHip>(input_delta_states);
+    auto *main_lb = dynamic_cast<LayerBlock *>(main_block.get());
+    const bool trade = this->can_trade() && din->size == as<DeltaStateHip>(*input_delta_z)->size &&
+                       (!shortcut || as<DeltaStateHip>(*shortcut_output_delta_z)->size == din->size);
+    if (trade)
+        input_delta_z->swap(input_delta_states);
+    else
+        input_delta_z->copy_from(input_delta_states, (int)(this->output_size * batch_size));
     // The residual's innovations are added by the state backward of the main block's
     // first layer where that is a convolution (one pass less per block); the shortcut
     // branch then runs first, so that its result is there to be added.
     Conv2dHip *opening = nullptr;
-    if (state_update)
-        if (auto *block = dynamic_cast<LayerBlock *>(main_block.get()))
-            if (block->layers.size() > 1)
-                opening = dynamic_cast<Conv2dHip *>(block->layers.front().get());
+    if (state_update && main_lb != nullptr && main_lb->layers.size() > 1)
+        opening = dynamic_cast<Conv2dHip *>(main_lb->layers.front().get());
     auto *dout = as<DeltaStateHip>(output_delta_states);
     const size_t num_states = (size_t)batch_size * this->input_size;
     if (shortcut) {
-        shortcut->backward(*input_delta_z, *shortcut_output_delta_z, temp_states, state_update);
+        if (trade) {
+            dynamic_cast<LayerBlock *>(shortcut.get())->first_delta_input = input_delta_z.get();
+            shortcut->backward(input_delta_states, *shortcut_output_delta_z, temp_states, state_update);
+        } else {
+            shortcut->backward(*input_delta_z, *shortcut_output_delta_z, temp_states, state_update);
+        }
         auto *sc = as<DeltaStateHip>(*shortcut_output_delta_z);
         if (opening != nullptr) {
             opening->bwd_residual_mu = sc->d_delta_mu;
             opening->bwd_residual_var = sc->d_delta_var;
             opening->bwd_residual_mode = 2;
+        }
+        if (trade) {
+            main_lb->first_delta_input = input_delta_z.get();
+            input_delta_states.block_size = batch_size;
         }
         main_block->backward(input_delta_states, output_delta_states, temp_states, state_update);
         if (!state_update || opening != nullptr) return;
@@ -813,6 +868,10 @@ void ResNetBlock::backward(BaseDeltaStates &input_delta_states,
             opening->bwd_residual_mu = sc->d_delta_mu;
             opening->bwd_residual_var = sc->d_delta_var;
             opening->bwd_residual_mode = 1;
+        }
+        if (trade) {
+            main_lb->first_delta_input = input_delta_z.get();
+            input_delta_states.block_size = batch_size;
         }
         main_block->backward(input_delta_states, output_delta_states, temp_states, state_update);
         if (!state_update || opening != nullptr) return;

@@ -155,6 +155,13 @@ class AvgPool2dHip : public BaseLayerHip {
 class LayerBlock : public BaseLayer {
    public:
     std::vector<std::shared_ptr<BaseLayer>> layers;
+    // One-shot requests of an enclosing ResNetBlock: the next forward() lets its first
+    // layer read this state, the next backward() lets its last layer read these
+    // innovations, instead of the first argument - which then only serves as the second
+    // ping-pong buffer. The enclosing block keeps the named object unchanged, so nothing
+    // has to be copied to protect it from the block's own passes.
+    BaseHiddenStates *first_input = nullptr;
+    BaseDeltaStates *first_delta_input = nullptr;
 
     LayerBlock() = default;
     explicit LayerBlock(const std::vector<std::shared_ptr<BaseLayer>> &layers);
@@ -241,7 +248,12 @@ class ResNetBlock : public BaseLayer {
    protected:
     bool on_device = false;
     int batch_size_ = 0;
-    void init_buffers();
+    size_t buffer_size_ = 0;
+    // buffers of `size` floats per array (0: what the block's own layers need)
+    void init_buffers(size_t size = 0);
+    // both branches are LayerBlocks (or the shortcut is the identity): they can be told to
+    // read the block's own copy of its input, so that copy can be a trade of arrays
+    bool can_trade() const;
 };
 
 // Device form: same object layout, device state buffers, residual adds on the GPU.

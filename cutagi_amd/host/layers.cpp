@@ -345,6 +345,11 @@ void BaseLayerHip::store_states_for_training_hip(HiddenStateHip &in, HiddenState
     const size_t n_in = in.actual_size * in.block_size;
     bwd->device_idx = in.device_idx;
     out.jcb_ones = true;
+    if (in.stable) {
+        // the owner keeps these arrays as they are until the backward pass is over
+        bwd->borrow(in.d_mu_a, in.d_jcb, in.jcb_ones, in.size);
+        return;
+    }
     if (in.transient) {
         bwd->resize_exact(in.size, !in.jcb_ones);
         std::swap(bwd->d_mu_a, in.d_mu_a);

@@ -426,8 +426,25 @@ void BackwardStateHip::allocate_memory() {
     d_jcb = dev_alloc(size, device_idx);
 }
 void BackwardStateHip::deallocate_memory() {
+    if (borrowed) {
+        d_mu_a = d_jcb = nullptr;
+        borrowed = false;
+        size = 0;
+        return;
+    }
     dev_free(d_mu_a);
     dev_free(d_jcb);
+}
+void BackwardStateHip::borrow(float *mu, float *jac, bool ones, size_t n) {
+    if (!borrowed) {
+        HIP_OK(hipDeviceSynchronize());
+        this->deallocate_memory();
+    }
+    borrowed = true;
+    d_mu_a = mu;
+    d_jcb = ones ? nullptr : jac;
+    jcb_ones = ones;
+    size = n;
 }
 void BackwardStateHip::to_host() {
     mu_a.resize(size);
@@ -441,6 +458,7 @@ void BackwardStateHip::to_host() {
 // Exactly `new_size` elements (the arrays are traded with a buffer of that size). The
 // Jacobian array is only allocated once a Jacobian that is not all ones has to be kept.
 void BackwardStateHip::resize_exact(size_t new_size, bool need_jcb) {
+    if (borrowed) this->deallocate_memory();
     if (new_size != this->size || d_mu_a == nullptr) {
         this->size = new_size;
         HIP_OK(hipDeviceSynchronize());
@@ -450,6 +468,7 @@ void BackwardStateHip::resize_exact(size_t new_size, bool need_jcb) {
     if (need_jcb && d_jcb == nullptr) d_jcb = dev_alloc(size, device_idx);
 }
 void BackwardStateHip::set_size(size_t new_size) {
+    if (borrowed) this->deallocate_memory();
     if (new_size > this->size) {
         this->size = new_size;
         HIP_OK(hipDeviceSynchronize());

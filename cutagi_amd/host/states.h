@@ -111,6 +111,10 @@ class HiddenStateHip : public BaseHiddenStates {
     // has read it, its contents are dead, so the layer may keep its arrays for the
     // backward pass and leave its own old ones in their place instead of copying.
     bool transient = false;
+    // Set by an owner that keeps the contents unchanged until its backward pass has run
+    // (a ResNetBlock's copy of its input): a layer that reads it may borrow the arrays for
+    // its own backward pass instead of copying them.
+    bool stable = false;
     const float *jcb_ptr() const { return jcb_ones ? device_ones(size, device_idx) : d_jcb; }
 
     HiddenStateHip(size_t n, size_t m, int device_idx = 0);
@@ -169,9 +173,13 @@ class BackwardStateHip : public BaseBackwardStates {
    public:
     float *d_mu_a = nullptr, *d_jcb = nullptr;
     bool jcb_ones = false;  // as HiddenStateHip::jcb_ones
+    // The arrays belong to a HiddenStateHip marked `stable` (nothing is freed here).
+    bool borrowed = false;
     const float *jcb_ptr() const { return jcb_ones ? device_ones(size, device_idx) : d_jcb; }
     // exactly new_size floats per array (reallocates when the size differs)
     void resize_exact(size_t new_size, bool need_jcb);
+    // points at the arrays of a stable state instead of owning any
+    void borrow(float *mu_a, float *jcb, bool ones, size_t n);
 
     BackwardStateHip() = default;
     ~BackwardStateHip() override;
