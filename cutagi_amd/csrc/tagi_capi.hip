@@ -298,6 +298,7 @@ int tagi_hip_tune(const char *key, int value) {
     else if (!strcmp(key, "linear.gemv.reverse")) g_tune.gemv_rev = value;
     else if (!strcmp(key, "linear.dw_side")) g_tune.dw_side = value;
     else if (!strcmp(key, "linear.gemv16")) g_tune.gemv16 = value;
+    else if (!strcmp(key, "linear.gemv16.fwd_lines")) g_gemv16_fwd_lines = value < 0 ? 0 : value;
     else return TAGI_ERR_INVALID_ARG;
     return TAGI_OK;
 }

@@ -195,6 +195,157 @@ __global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// Forward, loading whole cache lines (not the default: it measures the same as the
+// kernel above, which says that half-line requests are not what holds that one at
+// 5 TB/s). The MFMA wants lane (i, kk) to hold row i,
+// which makes a load instruction of the kernel above touch sixteen rows, half a
+// 128-byte line each. Here a load instruction covers 4 rows x 256 bytes instead
+// (lane (r = l/16, q = l%16): row 4*j + r of the wave's sixteen, reduction elements
+// 4*q .. 4*q+3 of a 64-element stage, j = 0..3), and the wave turns the stage into
+// the operand layout through a small LDS tile of its own, [16 rows][64 + 4]: four
+// 16-byte writes and four 16-byte reads per lane and array, no barrier (the tile
+// belongs to the wave; LDS operations of a wave complete in order). Component t of
+// the float4 a lane reads back is A[i][kk] of MFMA t as before.
+// ---------------------------------------------------------------------------
+constexpr int T16_STAGE = 64;             // reduction elements per stage
+constexpr int T16_TS = T16_STAGE + 4;     // row stride of the transposition tile
+constexpr int T16_TILE = 16 * T16_TS;     // floats per array and wave
+constexpr int T16_DEPTH = 2;              // register stages (4 measured slower: 131 vs 114 us at 8192^2, batch 16)
+
+__global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_lines_kernel(
+    const float *__restrict__ mu_w, const float *__restrict__ var_w,
+    const float *__restrict__ mu_a, const float *__restrict__ var_a, int K, int N, int B,
+    int k_per_split, int splits, float *__restrict__ ws0, float *__restrict__ ws1) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    constexpr int ROWS_PER_BLOCK = W16_WAVES * 16;
+    const int S = k_per_split + F16_PAD;
+    float *s_mu = lds, *s_var = lds + W16_SAMPLES * S;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int i = lane & 15, kk = lane >> 4;  // operand layout: row i, reduction slot kk
+    float *t_mu = lds + 2 * W16_SAMPLES * S + wave * 2 * T16_TILE, *t_var = t_mu + T16_TILE;
+    int row_block, split;
+    const int id = blockIdx.x, row_blocks = gridDim.x / splits;
+    if (row_blocks % 8 == 0) {
+        const int xcd = id & 7, local = id >> 3;
+        split = local % splits;
+        row_block = (local / splits) * 8 + xcd;
+    } else {
+        row_block = id % row_blocks;
+        split = id / row_blocks;
+    }
+    const int k_begin = split * k_per_split;
+    const int kr = min(K, k_begin + k_per_split) - k_begin;
+    const int rot = ((row_block * W16_WAVES + wave) * 2 * T16_STAGE) % k_per_split;
+
+    const int k4s = k_per_split / 4;
+    for (int e = tid; e < W16_SAMPLES * k4s; e += W16_WAVES * 64) {
+        const int b = e / k4s, k = (e - b * k4s) * 4;
+        float4 m = zero4(), v = zero4();
+        if (b < B && k < kr) {
+            m = ld4(mu_a + (size_t)b * K + k_begin + k);
+            v = ld4(var_a + (size_t)b * K + k_begin + k);
+        }
+        *reinterpret_cast<float4 *>(s_mu + b * S + k) = m;
+        *reinterpret_cast<float4 *>(s_var + b * S + k) = v;
+    }
+
+    // load layout: lane (r = kk, q = i) -> rows 4*j + r, elements 4*q ..; rows beyond N
+    // read row N-1 and are dropped at the end, elements beyond the slice read the last
+    // float4 of the row and meet zero activations
+    const int n0 = row_block * ROWS_PER_BLOCK + wave * 16;
+    const float *wm[4], *wv[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int row = min(n0 + 4 * j + kk, N - 1);
+        wm[j] = mu_w + (size_t)row * K;
+        wv[j] = var_w + (size_t)row * K;
+    }
+    const int k_lane = k_begin + 4 * i, k_last = K - 4;
+
+    floatx4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0;
+
+    float4 gm[T16_DEPTH][4], gv[T16_DEPTH][4];
+#define TAGI_T16_LOAD(buf, kb)                                      \
+    do {                                                            \
+        const int k_ = min(k_lane + (kb), k_last);                  \
+        _Pragma("unroll") for (int j = 0; j < 4; j++) {             \
+            gm[buf][j] = ld4(wm[j] + k_);                           \
+            gv[buf][j] = ld4(wv[j] + k_);                           \
+        }                                                           \
+    } while (0)
+    // registers -> the wave's tile -> operand layout -> MFMAs, one stage
+#define TAGI_T16_MULTIPLY(buf, kb)                                                               \
+    do {                                                                                         \
+        _Pragma("unroll") for (int j = 0; j < 4; j++) {                                          \
+            *reinterpret_cast<float4 *>(t_mu + (4 * j + kk) * T16_TS + 4 * i) = gm[buf][j];      \
+            *reinterpret_cast<float4 *>(t_var + (4 * j + kk) * T16_TS + 4 * i) = gv[buf][j];     \
+        }                                                                                        \
+        __builtin_amdgcn_wave_barrier(); /* other lanes' writes are read below */                \
+        _Pragma("unroll") for (int c = 0; c < 4; c++) {                                          \
+            const int at = (kb) + 16 * c + 4 * kk;                                               \
+            const float4 w = *reinterpret_cast<const float4 *>(t_mu + i * T16_TS + 16 * c + 4 * kk);  \
+            const float4 u = *reinterpret_cast<const float4 *>(t_var + i * T16_TS + 16 * c + 4 * kk); \
+            const float4 am = *reinterpret_cast<const float4 *>(s_mu + i * S + at);              \
+            const float4 av = *reinterpret_cast<const float4 *>(s_var + i * S + at);             \
+            const float4 as = make_float4(av.x + am.x * am.x, av.y + am.y * am.y,                \
+                                          av.z + am.z * am.z, av.w + am.w * am.w);               \
+            const float4 q = sq4(w);                                                             \
+            _Pragma("unroll") for (int t = 0; t < 4; t++) {                                      \
+                acc0 = mfma16(comp(w, t), comp(am, t), acc0);                                    \
+                acc1 = mfma16(comp(u, t), comp(as, t), acc1);                                    \
+                acc2 = mfma16(comp(q, t), comp(av, t), acc2);                                    \
+            }                                                                                    \
+        }                                                                                        \
+        __builtin_amdgcn_wave_barrier(); /* the tile is rewritten by the next stage */           \
+    } while (0)
+
+    // T16_DEPTH register stages in turn: while stage s is multiplied, the loads of the
+    // next T16_DEPTH - 1 stages are in flight (one workgroup per CU: the registers are
+    // there, and it is what keeps enough bytes on their way). Positions are inside the
+    // slice, rotated by `rot`; the last stages prefetch positions that wrap around
+    // (cached, never multiplied).
+    auto pos = [&](int p) {
+        p += rot;
+        while (p >= k_per_split) p -= k_per_split;
+        return p;
+    };
+#pragma unroll
+    for (int u = 0; u < T16_DEPTH - 1; u++) TAGI_T16_LOAD(u, pos(u * T16_STAGE));
+    __syncthreads();
+    for (int kb = 0; kb < k_per_split; kb += T16_DEPTH * T16_STAGE) {
+#pragma unroll
+        for (int u = 0; u < T16_DEPTH; u++) {
+            TAGI_T16_LOAD((u + T16_DEPTH - 1) % T16_DEPTH, pos(kb + (u + T16_DEPTH - 1) * T16_STAGE));
+            __builtin_amdgcn_sched_barrier(0);
+            TAGI_T16_MULTIPLY(u, pos(kb + u * T16_STAGE));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+#undef TAGI_T16_LOAD
+#undef TAGI_T16_MULTIPLY
+
+    // register v of lane l: row n0 + 4*(l/16) + v, sample l%16
+    const int b = lane & 15;
+    if (b < B) {
+        const int n = n0 + 4 * (lane >> 4);
+        const size_t at = ((size_t)split * B + b) * N + n;
+        const floatx4 m = acc0, v = acc1 + acc2;
+        if ((N & 3) == 0 && n + 3 < N) {
+            *reinterpret_cast<float4 *>(ws0 + at) = make_float4(m[0], m[1], m[2], m[3]);
+            *reinterpret_cast<float4 *>(ws1 + at) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+                if (n + c < N) {
+                    ws0[at + c] = m[c];
+                    ws1[at + c] = v[c];
+                }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // State backward. A wave owns 64 consecutive input columns; the eight waves of a
 // workgroup sit side by side (512 columns) and walk the same slice of output
 // rows, so the staged innovations of the slice serve all of them and no wave
@@ -311,9 +462,21 @@ constexpr size_t W16_LDS_BUDGET = 72 * 1024;                  // two workgroups 
 
 }  // namespace
 
+// 1: the forward that loads whole cache lines and transposes them in LDS. Measured equal
+// to the direct kernel (8192^2, batch 16: 113.6 vs 113.9 us per call), so the simpler one
+// stays the default.
+int g_gemv16_fwd_lines = 0;
+
 int gemv16_fwd_rows_per_block() { return W16_WAVES * F16_RG * 16; }
-int gemv16_fwd_k_step() { return F16_KROUND; }
+int gemv16_fwd_k_step() { return g_gemv16_fwd_lines ? T16_DEPTH * T16_STAGE : F16_KROUND; }
 int gemv16_fwd_max_slice() {
+    if (g_gemv16_fwd_lines) {
+        // one workgroup per CU: the activations of a slice plus the waves' tiles
+        const size_t budget = 150 * 1024 - (size_t)W16_WAVES * 2 * T16_TILE * sizeof(float);
+        int s = (int)(budget / (2 * W16_SAMPLES * sizeof(float)) - F16_PAD) /
+                (T16_DEPTH * T16_STAGE) * (T16_DEPTH * T16_STAGE);
+        return s > 512 ? 512 : s;
+    }
     return (int)(W16_LDS_BUDGET / (2 * W16_SAMPLES * sizeof(float)) - F16_PAD) / F16_KROUND *
            F16_KROUND;
 }
@@ -329,15 +492,25 @@ int gemv16_dz_max_slice() {
 hipError_t launch_gemv16_fwd(const float *mu_w, const float *var_w, const float *mu_a,
                              const float *var_a, int K, int N, int B, int k_per_split,
                              int splits, float *ws0, float *ws1, hipStream_t stream) {
-    if (B < 1 || B > W16_SAMPLES || K % 4 != 0 || k_per_split % F16_KROUND != 0 ||
+    if (B < 1 || B > W16_SAMPLES || K % 4 != 0 || k_per_split % gemv16_fwd_k_step() != 0 ||
         k_per_split > gemv16_fwd_max_slice() || (long long)k_per_split * splits < K)
         return hipErrorInvalidValue;
-    const size_t lds = (size_t)2 * W16_SAMPLES * (k_per_split + F16_PAD) * sizeof(float);
+    size_t lds = (size_t)2 * W16_SAMPLES * (k_per_split + F16_PAD) * sizeof(float);
+    const int rows = gemv16_fwd_rows_per_block();
+    dim3 grid(((N + rows - 1) / rows) * splits), block(W16_WAVES * 64);
+    if (g_gemv16_fwd_lines) {
+        lds += (size_t)W16_WAVES * 2 * T16_TILE * sizeof(float);
+        static PerDeviceOnce once_lines;
+        hipError_t e = allow_dynamic_lds(
+            once_lines, reinterpret_cast<const void *>(gemv16_fwd_lines_kernel), 160 * 1024);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(gemv16_fwd_lines_kernel, grid, block, lds, stream, mu_w, var_w, mu_a,
+                           var_a, K, N, B, k_per_split, splits, ws0, ws1);
+        return hipGetLastError();
+    }
     static PerDeviceOnce once;
     hipError_t e = allow_dynamic_lds(once, reinterpret_cast<const void *>(gemv16_fwd_kernel), 160 * 1024);
     if (e != hipSuccess) return e;
-    const int rows = gemv16_fwd_rows_per_block();
-    dim3 grid(((N + rows - 1) / rows) * splits), block(W16_WAVES * 64);
     hipLaunchKernelGGL(gemv16_fwd_kernel, grid, block, lds, stream, mu_w, var_w, mu_a, var_a, K,
                        N, B, k_per_split, splits, ws0, ws1);
     return hipGetLastError();

@@ -124,6 +124,8 @@ hipError_t launch_gemv16_fwd(const float *mu_w, const float *var_w, const float 
 hipError_t launch_gemv16_dz(const float *mu_w, const float *dmu, const float *dvar, int K, int N,
                             int B, int n_per_split, int splits, float *ws0, float *ws1,
                             hipStream_t stream);
+// 1: the 9..16-sample forward kernel that loads whole cache lines (default 0)
+extern int g_gemv16_fwd_lines;
 int gemv16_fwd_rows_per_block();
 int gemv16_fwd_k_step();
 int gemv16_fwd_max_slice();

@@ -18,7 +18,8 @@ extern "C" {
  * "linear.dz.splits", "linear.dw.splits", "linear.gemv_max_batch" (largest batch of
  * the streaming kernels, at most 16), "linear.gemv.swizzle",
  * "linear.gemv.fwd_variant", "linear.gemv.reverse", "linear.gemv16" (0: 9..16
- * samples on the kernels for up to 8), "linear.dw_side" (0: bias innovations and
+ * samples on the kernels for up to 8), "linear.gemv16.fwd_lines" (1: the 9..16-sample
+ * forward that loads whole cache lines and transposes them in LDS), "linear.dw_side" (0: bias innovations and
  * the state-backward fold as launches of their own instead of inside the
  * weight-backward launch), "linear.double_buffer". Conv2d: "conv2d.tile",
  * "conv2d.splits", "conv2d.dw.tile", "conv2d.dw.splits", "conv2d.group_loads",

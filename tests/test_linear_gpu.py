@@ -158,3 +158,28 @@ def test_pack_size_network_at_its_real_size():
         # the step moved the weight means and shrank no variance below zero
         assert not np.array_equal(np.asarray(arrays[0]), before[key][0])
         assert np.asarray(arrays[1]).min() >= 0
+
+
+@pytest.mark.parametrize("K,N,B", [(1024, 512, 16), (1536, 260, 12), (72, 1028, 10),
+                                   (2052, 300, 13), (4096, 256, 9)])
+def test_both_forward_kernels_for_9_to_16_samples(oracle_lib, K, N, B):
+    """The 16-wide streaming forward exists twice: loading the MFMA operand layout
+    directly (16 rows x 64 bytes per instruction, the default), and loading whole cache
+    lines that a wave-private LDS tile turns into that layout (same speed, kept as a
+    switch)."""
+    import cutagi_amd.functional as F
+    from cutagi_amd import capi
+    d = linear_inputs(K, N, B, seed=K + N + B, bias=True)
+    t = _dev(d)
+    ref = oracle_lib.linear_fwd(d["mu_w"], d["var_w"], d["mu_b"], d["var_b"], d["mu_a"],
+                                d["var_a"], threads=4)
+    got = {}
+    try:
+        for lines in (1, 0):
+            capi.tune("linear.gemv16.fwd_lines", lines)
+            z = F.linear_fwd(t["mu_w"], t["var_w"], t["mu_b"], t["var_b"], t["mu_a"], t["var_a"])
+            got[lines] = (z[0].cpu().numpy(), z[1].cpu().numpy())
+            assert_close(got[lines][0], ref[0], "mu_z (lines=%d)" % lines)
+            assert_close(got[lines][1], ref[1], "var_z (lines=%d)" % lines, same_sign=True)
+    finally:
+        capi.tune("linear.gemv16.fwd_lines", -1)
