@@ -308,14 +308,29 @@ def run_mlp(steps, warmup, B=32):
 
     warm = warm_up(lambda: step(), warmup)
     n = max(steps, 200)
-    t0 = time.perf_counter()
-    for _ in range(n):
-        mu, var = step()
+
+    def timed():
+        t0 = time.perf_counter()
+        for _ in range(n):
+            out = step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e6 / n, out
+
+    us, (mu, var) = timed()
+    # the same step with the forward and backward launches replayed from HIP graphs
+    # (Sequential.enable_graphs): reported beside the default, which is the eager path
+    net.enable_graphs(True)
+    for _ in range(20):
+        step()
     torch.cuda.synchronize()
-    us = (time.perf_counter() - t0) * 1e6 / n
+    us_graphs, _ = timed()
+    graphs = net.graphs_captured()
+    net.enable_graphs(False)
     return dict(workload="TAGI MLP 784->128->128->11 (ReLU), batch %d, one training step through "
                          "the host classes, outputs fetched" % B,
                 value=round(us, 1), unit="us/step", higher_is_better=False, steps=n, **warm,
+                with_hip_graph_replay=dict(value=round(us_graphs, 1), unit="us/step",
+                                           graphs_replayed_per_step=graphs),
                 outputs_finite_and_variances_nonnegative=bool(np.all(np.isfinite(mu))
                                                               and var.min() >= 0))
 

@@ -767,7 +767,8 @@ int tagi_conv2d_bwd_dw(const float *var_w, const float *var_b, const float *mu_a
 
 int tagi_store_states(const float *mu_a, const float *jcb, size_t n_in, float *bwd_mu_a,
                       float *bwd_jcb, float *out_jcb, size_t n_out, void *stream_) {
-    if (n_in > 0 && (!mu_a || !jcb || !bwd_mu_a || !bwd_jcb)) return TAGI_ERR_INVALID_ARG;
+    if (n_in > 0 && (!mu_a || !bwd_mu_a || (jcb != nullptr) != (bwd_jcb != nullptr)))
+        return TAGI_ERR_INVALID_ARG;
     if (n_out > 0 && !out_jcb) return TAGI_ERR_INVALID_ARG;
     TAGI_TRY(launch_store_states(mu_a, jcb, n_in, bwd_mu_a, bwd_jcb, out_jcb, n_out,
                                  static_cast<hipStream_t>(stream_)));

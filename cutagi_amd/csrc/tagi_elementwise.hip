@@ -53,7 +53,7 @@ __global__ __launch_bounds__(TPB) void store_states_kernel(
     const size_t i = (size_t)blockIdx.x * TPB + threadIdx.x;
     if (i < n_in) {
         bwd_mu_a[i] = mu_a[i];
-        bwd_jcb[i] = jcb[i];
+        if (jcb != nullptr) bwd_jcb[i] = jcb[i];  // (null: a Jacobian of one, only marked)
     }
     if (i < n_out) out_jcb[i] = 1.0f;
 }

@@ -265,6 +265,11 @@ PYBIND11_MODULE(cutagi, m) {
              py::arg("mu_x"), py::arg("var_x") = py::none())
         .def("backward", &Sequential::backward)
         .def("step", &Sequential::step)
+        // not in the reference: record the launches of a forward / backward pass into HIP
+        // graphs and replay them (see Sequential::enable_graphs)
+        .def("enable_graphs", &Sequential::enable_graphs, py::arg("on") = true)
+        .def("graphs_enabled", &Sequential::graphs_enabled)
+        .def("graphs_captured", &Sequential::graphs_captured)
         .def("output_to_host", &Sequential::output_to_host)
         .def("delta_z_to_host", &Sequential::delta_z_to_host)
         .def("set_delta_z",

@@ -58,7 +58,7 @@ void MixtureReLUHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &o
     const size_t n = input_states.actual_size * input_states.block_size;
     if (n > out->size) LOG(LogLevel::ERROR, "Output state buffer too small for MixtureReLU");
     TAGI_OK_OR_THROW(tagi_mixture_relu_fwd(in->d_mu_a, in->d_var_a, n, out->d_mu_a, out->d_jcb,
-                                           out->d_var_a, nullptr));
+                                           out->d_var_a, host_stream()));
     out->jcb_ones = false;
     this->input_size = input_states.actual_size;
     this->output_size = input_states.actual_size;
@@ -243,7 +243,7 @@ void BatchNorm2dHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &o
             LOG(LogLevel::ERROR, "BatchNorm2d needs more than one value per feature in training");
         TAGI_OK_OR_THROW(tagi_batchnorm2d_stats(in->d_mu_a, in->d_var_a, wihi, fi, batch_size,
                                                 momentum, d_mu_norm_batch, d_var_norm_batch,
-                                                d_mu_ra, d_var_ra, nullptr));
+                                                d_mu_ra, d_var_ra, host_stream()));
     }
     const float *mu_target = this->training ? d_mu_norm_batch : d_mu_ra;
     const float *var_target = this->training ? d_var_norm_batch : d_var_ra;
@@ -251,12 +251,12 @@ void BatchNorm2dHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &o
         TAGI_OK_OR_THROW(tagi_batchnorm2d_fwd_res(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a,
                                                   in->d_var_a, mu_target, var_target, res_mu,
                                                   res_var, bias ? 1 : 0, epsilon, wihi, fi,
-                                                  batch_size, out->d_mu_a, out->d_var_a, nullptr));
+                                                  batch_size, out->d_mu_a, out->d_var_a, host_stream()));
     else
         TAGI_OK_OR_THROW(tagi_batchnorm2d_fwd(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a,
                                               in->d_var_a, mu_target, var_target, bias ? 1 : 0,
                                               epsilon, wihi, fi, batch_size, out->d_mu_a,
-                                              out->d_var_a, nullptr));
+                                              out->d_var_a, host_stream()));
     out->jcb_ones = true;
     if (this->training) this->store_states_for_training_hip(*in, *out);
 }
@@ -278,7 +278,7 @@ void BatchNorm2dHip::backward(BaseDeltaStates &input_delta_states,
         d_mu_w, d_var_w, d_var_b, bwd->d_mu_a, bwd->jcb_ptr(), d_mu_norm_batch, d_var_norm_batch,
         din->d_delta_mu, din->d_delta_var, epsilon, wihi, fi, batch_size, bias ? 1 : 0,
         state_udapte ? 1 : 0, param_update ? 1 : 0, dout->d_delta_mu, dout->d_delta_var,
-        d_delta_mu_w, d_delta_var_w, d_delta_mu_b, d_delta_var_b, nullptr));
+        d_delta_mu_w, d_delta_var_w, d_delta_mu_b, d_delta_var_b, host_stream()));
 }
 
 void BatchNorm2dHip::save(std::ofstream &file) {
@@ -398,7 +398,7 @@ void AvgPool2dHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &out
     const int woho = (int)(out_width * out_height), wihi = (int)(in_width * in_height);
     TAGI_OK_OR_THROW(tagi_avgpool2d_fwd(in->d_mu_a, in->d_var_a, d_pool_idx, woho, wihi,
                                         (int)kernel_size, woho * (int)out_channels * batch_size,
-                                        out->d_mu_a, out->d_var_a, nullptr));
+                                        out->d_mu_a, out->d_var_a, host_stream()));
     out->jcb_ones = true;
     if (this->training) this->store_states_for_training_hip(*in, *out);
 }
@@ -419,7 +419,7 @@ void AvgPool2dHip::backward(BaseDeltaStates &input_delta_states,
     TAGI_OK_OR_THROW(tagi_avgpool2d_bwd_dz(bwd->jcb_ptr(), din->d_delta_mu, din->d_delta_var,
                                            d_z_ud_idx, woho, wihi, (int)kernel_size,
                                            (int)col_z_ud, (int)out_width, n_in, overlap ? 1 : 0,
-                                           dout->d_delta_mu, dout->d_delta_var, nullptr));
+                                           dout->d_delta_mu, dout->d_delta_var, host_stream()));
 }
 
 // ---- LayerBlock --------------------------------------------------------------------------
@@ -811,7 +811,7 @@ void ResNetBlock::forward(BaseHiddenStates &input_states, BaseHiddenStates &outp
     const size_t num_states = output_states.block_size * this->output_size;
     if (closing == nullptr)
         TAGI_OK_OR_THROW(tagi_add_shortcut(sc->d_mu_a, sc->d_var_a, num_states, out->d_mu_a,
-                                           out->d_var_a, nullptr));
+                                           out->d_var_a, host_stream()));
     set_output_dims(output_states, *this, batch_size);
     out->jcb_ones = true;  // the block's output Jacobian is one: marked, not written
 }
@@ -860,7 +860,7 @@ void ResNetBlock::backward(BaseDeltaStates &input_delta_states,
         main_block->backward(input_delta_states, output_delta_states, temp_states, state_update);
         if (!state_update || opening != nullptr) return;
         TAGI_OK_OR_THROW(tagi_add_shortcut(sc->d_delta_mu, sc->d_delta_var, num_states,
-                                           dout->d_delta_mu, dout->d_delta_var, nullptr));
+                                           dout->d_delta_mu, dout->d_delta_var, host_stream()));
     } else {
         auto *sc = as<DeltaStateHip>(*input_delta_z);
         if (opening != nullptr) {
@@ -878,7 +878,7 @@ void ResNetBlock::backward(BaseDeltaStates &input_delta_states,
         auto *kept = as<HiddenStateHip>(*input_z);
         TAGI_OK_OR_THROW(tagi_add_shortcut_delta(sc->d_delta_mu, sc->d_delta_var, kept->jcb_ptr(),
                                                  num_states, dout->d_delta_mu, dout->d_delta_var,
-                                                 nullptr));
+                                                 host_stream()));
     }
 }
 

@@ -12,6 +12,13 @@
 
 namespace tagi_host {
 
+// The stream every host class queues its device work on: the null stream, or - once a
+// model has switched graph replay on - one ordinary (blocking) stream of its own,
+// because work on the null stream cannot be captured into a HIP graph. A blocking
+// stream still orders with the synchronous copies that go through the null stream.
+hipStream_t host_stream();
+void set_host_stream(hipStream_t stream);
+
 template <typename T>
 T *dev_alloc_t(size_t n, int device_idx) {
     T *p = nullptr;

@@ -225,12 +225,12 @@ void BaseLayerHip::delta_params_to_device() {
 // src/base_layer_cuda.cu:127-159
 void BaseLayerHip::raw_update_weights() {
     TAGI_OK_OR_THROW(tagi_param_raw_update(d_delta_mu_w, d_delta_var_w, num_weights, d_mu_w,
-                                           d_var_w, nullptr));
+                                           d_var_w, host_stream()));
 }
 void BaseLayerHip::raw_update_biases() {
     if (!bias) return;
     TAGI_OK_OR_THROW(tagi_param_raw_update(d_delta_mu_b, d_delta_var_b, num_biases, d_mu_b,
-                                           d_var_b, nullptr));
+                                           d_var_b, host_stream()));
 }
 
 void BaseLayerHip::copy_params_from(const BaseLayer &source) {
@@ -246,17 +246,17 @@ void BaseLayerHip::copy_params_from(const BaseLayer &source) {
 // src/base_layer_cuda.cu:170-185). There are two counters used in turn: the
 // update that counts into one zeroes the other for the next update.
 void BaseLayerHip::update_weights() {
-    HIP_OK(hipMemsetAsync(d_neg_var_count, 0, 2 * sizeof(int), nullptr));
+    HIP_OK(hipMemsetAsync(d_neg_var_count, 0, 2 * sizeof(int), host_stream()));
     neg_var_slot = 0;
     TAGI_OK_OR_THROW(tagi_param_update(d_delta_mu_w, d_delta_var_w, cap_factor_update, num_weights,
-                                       d_mu_w, d_var_w, d_neg_var_count, nullptr));
+                                       d_mu_w, d_var_w, d_neg_var_count, host_stream()));
     neg_var_dirty = true;
 }
 
 void BaseLayerHip::update_biases() {
     if (!bias) return;
     TAGI_OK_OR_THROW(tagi_param_update(d_delta_mu_b, d_delta_var_b, cap_factor_update, num_biases,
-                                       d_mu_b, d_var_b, nullptr, nullptr));
+                                       d_mu_b, d_var_b, nullptr, host_stream()));
 }
 
 // Weights and biases in one launch, no launch for the counter.
@@ -265,7 +265,7 @@ void BaseLayerHip::update_params() {
     TAGI_OK_OR_THROW(tagi_layer_update(d_delta_mu_w, d_delta_var_w, num_weights, d_mu_w, d_var_w,
                                        d_delta_mu_b, d_delta_var_b, bias ? num_biases : 0, d_mu_b,
                                        d_var_b, cap_factor_update, d_neg_var_count, neg_var_slot,
-                                       nullptr));
+                                       host_stream()));
     neg_var_dirty = true;
 }
 
@@ -360,12 +360,18 @@ void BaseLayerHip::store_states_for_training_hip(HiddenStateHip &in, HiddenState
     if (bwd->size < n_in) bwd->set_size(n_in);
     bwd->jcb_ones = in.jcb_ones;
     if (in.jcb_ones) {
-        HIP_OK(hipMemcpyAsync(bwd->d_mu_a, in.d_mu_a, n_in * sizeof(float),
-                              hipMemcpyDeviceToDevice, nullptr));
+        // (a kernel rather than a copy command where the work may be recorded into a
+        // graph: copy nodes make a graph launch far more expensive than its kernels)
+        if (host_stream() != nullptr)
+            TAGI_OK_OR_THROW(tagi_store_states(in.d_mu_a, nullptr, n_in, bwd->d_mu_a, nullptr,
+                                               nullptr, 0, host_stream()));
+        else
+            HIP_OK(hipMemcpyAsync(bwd->d_mu_a, in.d_mu_a, n_in * sizeof(float),
+                                  hipMemcpyDeviceToDevice, host_stream()));
         return;
     }
     TAGI_OK_OR_THROW(tagi_store_states(in.d_mu_a, in.d_jcb, n_in, bwd->d_mu_a, bwd->d_jcb, nullptr,
-                                       0, nullptr));
+                                       0, host_stream()));
 }
 
 // ---- Linear -----------------------------------------------------------------------------
@@ -444,12 +450,12 @@ void LinearHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &output
         TAGI_OK_OR_THROW(tagi_linear_fwd_act(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a,
                                              in->d_var_a, (int)input_size, (int)output_size,
                                              batch_size, bias ? 1 : 0, act, out->d_mu_a,
-                                             out->d_var_a, out->d_jcb, nullptr));
+                                             out->d_var_a, out->d_jcb, host_stream()));
     else
         TAGI_OK_OR_THROW(tagi_linear_fwd(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a,
                                          in->d_var_a, (int)input_size, (int)output_size,
                                          batch_size, bias ? 1 : 0, out->d_mu_a, out->d_var_a,
-                                         nullptr));
+                                         host_stream()));
     output_states.width = this->out_width;
     output_states.height = this->out_height;
     output_states.depth = this->out_channels;
@@ -474,7 +480,7 @@ void LinearHip::backward(BaseDeltaStates &input_delta_states, BaseDeltaStates &o
                                      (int)output_size, batch_size, bias ? 1 : 0, state_udapte ? 1 : 0,
                                      param_update ? 1 : 0, dout->d_delta_mu, dout->d_delta_var,
                                      d_delta_mu_w, d_delta_var_w, d_delta_mu_b, d_delta_var_b,
-                                     nullptr));
+                                     host_stream()));
 }
 
 // ---- Conv2d -----------------------------------------------------------------------------
@@ -655,12 +661,12 @@ void Conv2dHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &output
                                              in->d_var_a, d_idx_mwa_2, woho, (int)out_channels,
                                              wihi, (int)in_channels, (int)kernel_size, batch_size,
                                              bias ? 1 : 0, act, out->d_mu_a, out->d_var_a,
-                                             out->d_jcb, nullptr));
+                                             out->d_jcb, host_stream()));
     else
         TAGI_OK_OR_THROW(tagi_conv2d_fwd(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a,
                                          in->d_var_a, d_idx_mwa_2, woho, (int)out_channels, wihi,
                                          (int)in_channels, (int)kernel_size, batch_size,
-                                         bias ? 1 : 0, out->d_mu_a, out->d_var_a, nullptr));
+                                         bias ? 1 : 0, out->d_mu_a, out->d_var_a, host_stream()));
     out->jcb_ones = true;
     if (training) this->store_states_for_training_hip(*in, *out);
     if (act != 0) out->jcb_ones = false;  // the activation's Jacobian was written
@@ -684,7 +690,7 @@ void Conv2dHip::backward(BaseDeltaStates &input_delta_states, BaseDeltaStates &o
                                             din->d_delta_var, d_idx_mwa_2, batch_size,
                                             (int)out_channels, woho, wihi, (int)in_channels,
                                             (int)kernel_size, bias ? 1 : 0, d_delta_mu_w,
-                                            d_delta_var_w, d_delta_mu_b, d_delta_var_b, nullptr));
+                                            d_delta_var_w, d_delta_mu_b, d_delta_var_b, host_stream()));
     if (state_udapte) {
         if (input_size * batch_size > dout->size)
             LOG(LogLevel::ERROR, "Delta state buffer too small for " + this->get_layer_info());
@@ -693,13 +699,13 @@ void Conv2dHip::backward(BaseDeltaStates &input_delta_states, BaseDeltaStates &o
                 d_mu_w, bwd->jcb_ptr(), din->d_delta_mu, din->d_delta_var, d_idx_cov_zwa_1,
                 d_idx_var_z_ud, woho, (int)out_channels, wihi, (int)in_channels, (int)kernel_size,
                 row_zw, batch_size, res_mu, res_var, res_mode, dout->d_delta_mu,
-                dout->d_delta_var, nullptr));
+                dout->d_delta_var, host_stream()));
         else
             TAGI_OK_OR_THROW(tagi_conv2d_bwd_dz(d_mu_w, bwd->jcb_ptr(), din->d_delta_mu,
                                                 din->d_delta_var, d_idx_cov_zwa_1, d_idx_var_z_ud,
                                                 woho, (int)out_channels, wihi, (int)in_channels,
                                                 (int)kernel_size, row_zw, batch_size,
-                                                dout->d_delta_mu, dout->d_delta_var, nullptr));
+                                                dout->d_delta_mu, dout->d_delta_var, host_stream()));
     } else if (res_mu != nullptr) {
         LOG(LogLevel::ERROR, "Residual innovations handed to a layer that skips its state update");
     }
@@ -727,7 +733,7 @@ void ReLUHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &output_s
     const size_t n = input_states.actual_size * input_states.block_size;
     if (n > out->size) LOG(LogLevel::ERROR, "Output state buffer too small for ReLU");
     TAGI_OK_OR_THROW(tagi_relu_fwd(in->d_mu_a, in->d_var_a, n, out->d_mu_a, out->d_jcb, out->d_var_a,
-                                   nullptr));
+                                   host_stream()));
     out->jcb_ones = false;
     this->input_size = input_states.actual_size;
     this->output_size = input_states.actual_size;

@@ -1,6 +1,8 @@
 // Sequential and OutputUpdater: see sequential.h.
 #include "sequential.h"
 
+#include "host_util.h"
+
 #include <hip/hip_runtime_api.h>
 #include <sys/stat.h>
 
@@ -150,7 +152,7 @@ void OutputUpdater::update_raw(BaseHiddenStates &output_states, const float *mu_
     delta->reset_zeros();
     TAGI_OK_OR_THROW(tagi_out_update_dense(out->d_mu_a, out->d_var_a, out->jcb_ptr(), o->d_mu_obs,
                                            o->d_var_obs, (int)o->size, delta->d_delta_mu,
-                                           delta->d_delta_var, nullptr));
+                                           delta->d_delta_var, host_stream()));
 }
 
 void OutputUpdater::update_using_indices(BaseHiddenStates &output_states,
@@ -191,7 +193,7 @@ void OutputUpdater::update_using_indices_raw(BaseHiddenStates &output_states,
     TAGI_OK_OR_THROW(tagi_out_update_indexed(out->d_mu_a, out->d_var_a, out->jcb_ptr(), o->d_mu_obs,
                                              o->d_var_obs, o->d_selected_idx, n_obs, n_enc,
                                              (int)o->size, delta->d_delta_mu, delta->d_delta_var,
-                                             nullptr));
+                                             host_stream()));
 }
 
 void OutputUpdater::update_heteros(BaseHiddenStates &output_states, std::vector<float> &mu_obs,
@@ -215,7 +217,7 @@ void OutputUpdater::update_heteros_raw(BaseHiddenStates &output_states, const fl
     delta->reset_zeros();
     TAGI_OK_OR_THROW(tagi_out_update_heteros(out->d_mu_a, out->d_var_a, out->jcb_ptr(), o->d_mu_obs,
                                              (int)o->size, delta->d_delta_mu, delta->d_delta_var,
-                                             nullptr));
+                                             host_stream()));
 }
 
 // ---- Sequential -----------------------------------------------------------------------
@@ -240,6 +242,7 @@ void Sequential::switch_to_cuda() {
 
 // reference: src/sequential.cpp:32-73. "hip" is accepted as a synonym of "cuda".
 void Sequential::to_device(const std::string &new_device) {
+    this->clear_graphs();  // what a recorded graph refers to may change here
     if (new_device == "cpu") {
         this->device = "cpu";
         return;
@@ -308,7 +311,7 @@ void Sequential::init_output_state_buffer() {
     input_z_buffer = std::make_shared<HiddenStateHip>(z_buffer_size, z_buffer_block_size, device_idx);
     // ping-pong buffers: what a layer has read is dead, so it may keep the arrays
     for (auto *b : {output_z_buffer.get(), input_z_buffer.get()})
-        dynamic_cast<HiddenStateHip *>(b)->transient = true;
+        dynamic_cast<HiddenStateHip *>(b)->transient = !graphs_on_;
     temp_states = std::make_shared<TempStateHip>(0, z_buffer_block_size, device_idx);
 }
 
@@ -348,10 +351,12 @@ void Sequential::set_threads(unsigned n) {
     for (auto &layer : layers) layer->set_threads(n);
 }
 void Sequential::train() {
+    this->clear_graphs();  // what a recorded graph refers to may change here
     this->training = true;
     for (auto &layer : layers) layer->train();
 }
 void Sequential::eval() {
+    this->clear_graphs();  // what a recorded graph refers to may change here
     this->training = false;
     for (auto &layer : layers) layer->eval();
 }
@@ -373,7 +378,9 @@ void Sequential::forward(const float *mu_x, const float *var_x, size_t n) {
     this->prepare_buffers(batch_size);
     auto *in = dynamic_cast<HiddenStateHip *>(this->input_z_buffer.get());
     in->set_input_raw(mu_x, var_x, n, batch_size);
-    this->forward_layers(0);
+    auto *out = dynamic_cast<HiddenStateHip *>(this->output_z_buffer.get());
+    this->run_or_replay(GraphKey(0, in->d_mu_a, out->d_mu_a, batch_size, training ? 1 : 0),
+                        [this] { this->forward_layers(0); });
 }
 
 // Layers from `first` on, reading input_z_buffer; the network's output ends up in
@@ -403,6 +410,16 @@ void Sequential::forward(BaseHiddenStates &input_states) {
 // buffer; the first layer propagates to its input only on request.
 void Sequential::backward() {
     this->require_device("backward");
+    auto *din = dynamic_cast<DeltaStateHip *>(this->input_delta_z_buffer.get());
+    auto *dout = dynamic_cast<DeltaStateHip *>(this->output_delta_z_buffer.get());
+    if (din == nullptr || dout == nullptr)
+        LOG(LogLevel::ERROR, "backward needs a forward pass in training mode first");
+    this->run_or_replay(GraphKey(1, din->d_delta_mu, dout->d_delta_mu, (int)din->block_size,
+                                 (input_state_update ? 1 : 0) | (param_update ? 2 : 0)),
+                        [this] { this->backward_layers(); });
+}
+
+void Sequential::backward_layers() {
     for (size_t i = layers.size() - 1; i >= 1; i--) {
         BaseLayer *layer = layers[i].get();
         layer->backward(*input_delta_z_buffer, *output_delta_z_buffer, *temp_states);
@@ -411,6 +428,113 @@ void Sequential::backward() {
     }
     layers.front()->backward(*input_delta_z_buffer, *output_delta_z_buffer, *temp_states,
                              this->input_state_update);
+}
+
+// ---- HIP graph replay -------------------------------------------------------------------
+static hipStream_t graph_stream() {
+    static hipStream_t stream = nullptr;
+    // an ordinary (blocking) stream at the default priority: synchronous copies on the
+    // null stream still order with it
+    if (stream == nullptr) HIP_OK(hipStreamCreateWithFlags(&stream, hipStreamDefault));
+    return stream;
+}
+
+void Sequential::enable_graphs(bool on) {
+    this->require_device("enable_graphs");
+    if (on == graphs_on_) return;
+    HIP_OK(hipDeviceSynchronize());
+    this->clear_graphs();
+    graphs_on_ = on;
+    if (on) set_host_stream(graph_stream());
+    // replayed work must meet the same arrays every step: no trading with the buffers
+    for (auto *b : {output_z_buffer.get(), input_z_buffer.get()})
+        if (auto *h = dynamic_cast<HiddenStateHip *>(b)) h->transient = !on;
+}
+
+int Sequential::graphs_captured() const {
+    int n = 0;
+    for (const auto &kv : graphs_) n += kv.second.exec != nullptr ? 1 : 0;
+    return n;
+}
+
+void Sequential::clear_graphs() {
+    for (auto &kv : graphs_)
+        if (kv.second.exec != nullptr)
+            (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(kv.second.exec));
+    graphs_.clear();
+}
+
+bool Sequential::only_plain_layers() const {
+    for (const auto &layer : layers) {
+        const LayerType t = layer->get_layer_type();
+        if (t == LayerType::LayerBlock || t == LayerType::ResNetBlock) return false;
+    }
+    return true;
+}
+
+// `body` queues device work on host_stream() and moves the buffer pointers around; it
+// is run as it is, or recorded into a graph, or skipped in favour of the recorded graph
+// (whose effect on the buffer pointers is then repeated by hand).
+void Sequential::run_or_replay(const GraphKey &key, const std::function<void()> &body) {
+    if (!graphs_on_ || host_stream() == nullptr || !this->only_plain_layers()) {
+        body();
+        return;
+    }
+    GraphEntry &e = graphs_[key];
+    hipStream_t stream = host_stream();
+    if (e.exec != nullptr) {
+        HIP_OK(hipGraphLaunch(static_cast<hipGraphExec_t>(e.exec), stream));
+        if (e.swaps_state) std::swap(input_z_buffer, output_z_buffer);
+        if (e.swaps_delta) std::swap(input_delta_z_buffer, output_delta_z_buffer);
+        return;
+    }
+    // the first runs allocate (workspaces, what layers keep for the backward pass):
+    // they stay eager
+    if (e.unusable || e.warm_runs < 2) {
+        e.warm_runs++;
+        body();
+        return;
+    }
+    const auto state_before = input_z_buffer, out_before = output_z_buffer;
+    const auto delta_before = input_delta_z_buffer, dout_before = output_delta_z_buffer;
+    auto restore = [&] {
+        input_z_buffer = state_before;
+        output_z_buffer = out_before;
+        input_delta_z_buffer = delta_before;
+        output_delta_z_buffer = dout_before;
+    };
+    if (hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed) != hipSuccess) {
+        (void)hipGetLastError();
+        e.unusable = true;
+        body();
+        return;
+    }
+    hipGraph_t graph = nullptr;
+    try {
+        body();
+    } catch (...) {
+        (void)hipStreamEndCapture(stream, &graph);
+        if (graph != nullptr) (void)hipGraphDestroy(graph);
+        (void)hipGetLastError();
+        e.unusable = true;
+        throw;
+    }
+    hipGraphExec_t exec = nullptr;
+    hipError_t rc = hipStreamEndCapture(stream, &graph);
+    if (rc == hipSuccess && graph != nullptr) rc = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    if (graph != nullptr) (void)hipGraphDestroy(graph);
+    if (rc != hipSuccess || exec == nullptr) {
+        // something in the body cannot be recorded: nothing has run yet, so run it now
+        (void)hipGetLastError();
+        e.unusable = true;
+        restore();
+        body();
+        return;
+    }
+    e.exec = exec;
+    e.swaps_state = input_z_buffer != state_before;
+    e.swaps_delta = input_delta_z_buffer != delta_before;
+    HIP_OK(hipGraphLaunch(exec, stream));
 }
 
 void Sequential::step() {
@@ -423,7 +547,7 @@ void Sequential::step() {
         layer->collect_update_items(items);
     }
     if (!items.empty())
-        TAGI_OK_OR_THROW(tagi_model_update(items.data(), (int)items.size(), nullptr));
+        TAGI_OK_OR_THROW(tagi_model_update(items.data(), (int)items.size(), host_stream()));
 }
 
 std::string Sequential::get_layer_stack_info() const {
@@ -456,6 +580,7 @@ void Sequential::save(const std::string &filename) {
 }
 
 void Sequential::load(const std::string &filename) {
+    this->clear_graphs();  // what a recorded graph refers to may change here
     this->preinit_layer();
     std::ifstream file(filename, std::ios::binary);
     if (!file.is_open()) LOG(LogLevel::ERROR, "Failed to open file for loading");
@@ -512,6 +637,7 @@ void Sequential::save_csv(const std::string &filename) {
 }
 
 void Sequential::load_csv(const std::string &filename) {
+    this->clear_graphs();  // what a recorded graph refers to may change here
     size_t num_weights = 0, num_biases = 0;
     for (auto &layer : layers) {
         num_weights += layer->mu_w.size();
@@ -572,6 +698,7 @@ ParameterMap Sequential::state_dict() {
 }
 
 void Sequential::load_state_dict(const ParameterMap &sd) {
+    this->clear_graphs();  // what a recorded graph refers to may change here
     for (size_t i = 0; i < layers.size(); i++) {
         if (layers[i]->get_layer_type() == LayerType::Activation ||
             layers[i]->get_layer_type() == LayerType::Pool2d)
@@ -581,6 +708,7 @@ void Sequential::load_state_dict(const ParameterMap &sd) {
 }
 
 void Sequential::params_from(const Sequential &ref) {
+    this->clear_graphs();  // what a recorded graph refers to may change here
     if (layers.size() != ref.layers.size()) LOG(LogLevel::ERROR, "Model architecture is different.");
     for (size_t i = 0; i < layers.size(); i++) {
         BaseLayer *src = ref.layers[i].get();

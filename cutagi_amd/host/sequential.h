@@ -3,8 +3,11 @@
 // OutputUpdater (include/base_output_updater.h, src/base_output_updater.cpp:269-386,
 // src/output_updater_cuda.cu:146-223).
 #pragma once
+#include <functional>
+#include <map>
 #include <memory>
 #include <string>
+#include <tuple>
 #include <unordered_map>
 #include <vector>
 
@@ -73,6 +76,9 @@ class Sequential {
     std::vector<std::shared_ptr<BaseLayer>> layers;
 
     Sequential() = default;
+    ~Sequential() { this->clear_graphs(); }
+    Sequential(const Sequential &) = delete;
+    Sequential &operator=(const Sequential &) = delete;
     void add_layer(std::shared_ptr<BaseLayer> layer);
     void add_layers();  // call once after the last add_layer
 
@@ -91,6 +97,21 @@ class Sequential {
     void forward(BaseHiddenStates &input_states);
     void backward();
     void step();
+
+    // Not in the reference. A small network's training step is a chain of a dozen short
+    // launches, and the host needs longer to queue them than the GPU to run them. With
+    // graphs on, the launches of a forward pass (and of a backward pass) are recorded into
+    // a HIP graph the third time they run with the same buffers and batch size, and
+    // replayed as one submission from then on. What is replayed must not change between
+    // steps, so in this mode layers copy what they keep for the backward pass instead of
+    // trading arrays with the buffers, all device work of the host classes moves to one
+    // ordinary stream (the null stream cannot be captured), and only networks of plain
+    // layers (no LayerBlock / ResNetBlock, whose buffers trade contents) are replayed;
+    // others run as before. Input transfers, the output update and step() are not part
+    // of a graph. Results are the same kernels' results either way.
+    void enable_graphs(bool on);
+    bool graphs_enabled() const { return graphs_on_; }
+    int graphs_captured() const;  // graphs held at the moment (for tests)
 
     std::string get_layer_stack_info() const;
     void preinit_layer();
@@ -121,7 +142,22 @@ class Sequential {
     void init_delta_state_buffer();
     void prepare_buffers(int batch_size);
     void forward_layers(size_t first);
+    void backward_layers();
     void require_device(const char *what) const;
+
+    struct GraphEntry {
+        void *exec = nullptr;    // hipGraphExec_t
+        int warm_runs = 0;       // eager runs seen with this key (allocations happen in them)
+        bool unusable = false;   // capture failed: stay eager
+        bool swaps_state = false, swaps_delta = false;  // net effect on the buffer pointers
+    };
+    // (kind, first buffer's arrays, second buffer's arrays, batch size, flags)
+    using GraphKey = std::tuple<int, const void *, const void *, int, int>;
+    std::map<GraphKey, GraphEntry> graphs_;
+    bool graphs_on_ = false;
+    void clear_graphs();
+    bool only_plain_layers() const;
+    void run_or_replay(const GraphKey &key, const std::function<void()> &body);
 };
 
 }  // namespace tagi_host

@@ -16,6 +16,11 @@
 
 namespace tagi_host {
 
+// (declared in host_util.h) the stream the host classes queue their device work on
+static hipStream_t g_host_stream = nullptr;
+hipStream_t host_stream() { return g_host_stream; }
+void set_host_stream(hipStream_t stream) { g_host_stream = stream; }
+
 namespace {
 float *dev_alloc(size_t n, int device_idx) {
     float *p = nullptr;
@@ -36,7 +41,7 @@ void d2h(float *dst, const float *src, size_t n) {
 }
 void d2d(float *dst, const float *src, size_t n) {
     if (n)
-        HIP_OK(hipMemcpyAsync(dst, src, n * sizeof(float), hipMemcpyDeviceToDevice, nullptr));
+        HIP_OK(hipMemcpyAsync(dst, src, n * sizeof(float), hipMemcpyDeviceToDevice, host_stream()));
 }
 
 // Pinned staging for the small host-to-device transfers of every batch. A copy
@@ -72,8 +77,8 @@ class StagingRing {
             if (sizes[i]) std::memcpy(static_cast<char *>(s.host) + at, parts[i], sizes[i]);
             at += sizes[i];
         }
-        HIP_OK(hipMemcpyAsync(dst, s.host, bytes, hipMemcpyHostToDevice, nullptr));
-        HIP_OK(hipEventRecord(s.event, nullptr));
+        HIP_OK(hipMemcpyAsync(dst, s.host, bytes, hipMemcpyHostToDevice, host_stream()));
+        HIP_OK(hipEventRecord(s.event, host_stream()));
         s.used = true;
     }
 
@@ -295,7 +300,7 @@ void HiddenStateHip::set_input_raw(const float *mu_x, const float *var_x, size_t
     if (var_x != nullptr)
         ring.upload(d_var_a, var_x, n * sizeof(float));
     else
-        HIP_OK(hipMemsetAsync(d_var_a, 0, n * sizeof(float), nullptr));
+        HIP_OK(hipMemsetAsync(d_var_a, 0, n * sizeof(float), host_stream()));
     jcb_ones = true;  // the input's Jacobian is one: marked, not written
 }
 void HiddenStateHip::set_size(size_t new_size, size_t new_block_size) {
@@ -365,7 +370,7 @@ void DeltaStateHip::to_host() {
 }
 void DeltaStateHip::reset_zeros() {
     if (size == 0) return;
-    HIP_OK(hipMemsetAsync(d_delta_mu, 0, (delta_var_offset(size) + size) * sizeof(float), nullptr));
+    HIP_OK(hipMemsetAsync(d_delta_mu, 0, (delta_var_offset(size) + size) * sizeof(float), host_stream()));
 }
 void DeltaStateHip::copy_from(const BaseDeltaStates &source, int num_data) {
     auto *s = dynamic_cast<const DeltaStateHip *>(&source);

@@ -211,7 +211,9 @@ int tagi_conv2d_bwd_dw(const float *var_w, const float *var_b,
 /* Keep what the backward pass needs and reset the output Jacobian; replaces
  * BaseLayerCuda::store_states_for_training_cuda
  * (src/base_layer_cuda.cu:464-486): bwd_mu_a/bwd_jcb <- first n_in entries of
- * mu_a/jcb, out_jcb[0..n_out) <- 1. */
+ * mu_a/jcb, out_jcb[0..n_out) <- 1. jcb and bwd_jcb may both be NULL (an input
+ * Jacobian that is known to be one everywhere: only the mean is kept); out_jcb may
+ * be NULL with n_out == 0. */
 int tagi_store_states(const float *mu_a, const float *jcb, size_t n_in,
                       float *bwd_mu_a, float *bwd_jcb, float *out_jcb,
                       size_t n_out, void *stream);
