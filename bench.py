@@ -669,12 +669,12 @@ def main():
             # Linear 4096^2 at batch 32 and 64, where the matrix and the memory bound meet
             line["extra"]["mid"] = {name: linear_entry(run_workload(name, args.steps, args.warmup))
                                     for name in ("mid32", "mid64")}
-    if "mlp" in extras:
-        line["extra"]["mlp"] = run_mlp(args.steps, args.warmup)
     if "conv" in extras:
         line["extra"]["conv"] = run_conv(max(5, args.steps // 2), args.warmup)
     if "resnet18" in extras:
         line["extra"]["resnet18"] = run_resnet(max(20, args.steps // 2), 5)
+    if "mlp" in extras:
+        line["extra"]["mlp"] = run_mlp(args.steps, args.warmup)
     if args.calibrate:
         calibrate_copy()
     # wall time of everything that ran on the GPU, so that the short timed regions can

@@ -109,6 +109,7 @@ struct Tuning {
     // walk rows from the end, high bit: XCD-aware column mapping
     int gemv_rev = -1;
     int gemv16 = -1;    // 0: 9..16 samples on the 4x4x1 kernels too
+    int wide32 = -1;    // 0: 17..32 samples on the tiled kernels; 2: state backward streams too
     int dw_side = -1;   // 0: bias innovations and the state-backward fold as launches of their own
 };
 Tuning g_tune;
@@ -147,6 +148,16 @@ int pick_splits(int tiles, int reduction, int forced, int min_tiles = 8) {
 // the streaming kernels hold at most 16 samples
 int gemv_max_batch() {
     return g_tune.gemv_max_batch >= 0 && g_tune.gemv_max_batch < 16 ? g_tune.gemv_max_batch : 16;
+}
+// ... except the 16x16x4 forward, which also takes two groups of 16 (17..32 samples:
+// twice the MFMA work per weight byte, still one pass over the weights). Measured against
+// the tiled kernel at 4096^2: forward 35-37 us instead of 40-41 us for 17..32 samples. The
+// state backward has the same two-group form but measured slower than the tiled kernel
+// there (39 against 30 us at batch 32) and keeps to 16 samples. The knob that limits the
+// streaming kernels limits these too.
+int wide_max_batch() {
+    if (g_tune.gemv_max_batch >= 0 && g_tune.gemv_max_batch < 16) return g_tune.gemv_max_batch;
+    return g_tune.wide32 == 0 ? 16 : gemv16_max_batch();
 }
 
 // Tile shape and reduction slices of a tiled launch.
@@ -298,6 +309,7 @@ int tagi_hip_tune(const char *key, int value) {
     else if (!strcmp(key, "linear.gemv.reverse")) g_tune.gemv_rev = value;
     else if (!strcmp(key, "linear.dw_side")) g_tune.dw_side = value;
     else if (!strcmp(key, "linear.gemv16")) g_tune.gemv16 = value;
+    else if (!strcmp(key, "linear.gemv32")) g_tune.wide32 = value;
     else if (!strcmp(key, "linear.gemv16.fwd_lines")) g_gemv16_fwd_lines = value < 0 ? 0 : value;
     else return TAGI_ERR_INVALID_ARG;
     return TAGI_OK;
@@ -320,14 +332,14 @@ static int linear_fwd_impl(const float *mu_w, const float *var_w, const float *m
     const bool vec = (K % 4 == 0) && aligned16(mu_w) && aligned16(var_w) && aligned16(mu_a) &&
                      aligned16(var_a);
 
-    if (B > 8 && B <= gemv_max_batch() && B <= 16 && vec && g_tune.gemv16 != 0) {
-        // 9..16 samples: the 16-wide streaming kernel
+    if (B > 8 && B <= wide_max_batch() && vec && g_tune.gemv16 != 0) {
+        // 9..32 samples: the 16-wide streaming kernel (two sample groups beyond 16)
         const int blocks = ceil_div(N, gemv16_fwd_rows_per_block());
         const int step = gemv16_fwd_k_step();
         int splits = g_tune.fwd_splits > 0 ? g_tune.fwd_splits : ceil_div(2 * num_cu(), blocks);
         const int max_splits = ceil_div(K, 4 * step);
         if (splits > max_splits) splits = max_splits;
-        const int min_splits = ceil_div(K, gemv16_fwd_max_slice());
+        const int min_splits = ceil_div(K, gemv16_fwd_max_slice(B));
         if (splits < min_splits) splits = min_splits;
         const int per = ceil_div(ceil_div(K, splits), step) * step;
         splits = ceil_div(K, per);
@@ -415,14 +427,15 @@ static int linear_bwd_dz_impl(const float *mu_w, const float *jcb, const float *
     const bool vec = (K % 4 == 0) && (N % 4 == 0) && aligned16(mu_w) && aligned16(delta_mu) &&
                      aligned16(delta_var);
 
-    const bool wide16 = B > 8 && B <= 16 && g_tune.gemv16 != 0;
-    if (B <= gemv_max_batch() && vec) {
+    const bool wide16 = B > 8 && B <= (g_tune.wide32 == 2 ? wide_max_batch() : gemv_max_batch()) &&
+                        g_tune.gemv16 != 0;
+    if ((B <= gemv_max_batch() || wide16) && vec) {
         const int blocks = ceil_div(K, wide16 ? gemv16_dz_cols_per_block() : gemv_dz_cols_per_block());
         const int step = wide16 ? gemv16_dz_n_step() : gemv_dz_n_step();
         int splits = g_tune.dz_splits > 0 ? g_tune.dz_splits : ceil_div(num_cu(), blocks);
         const int max_splits = ceil_div(N, 2 * step);
         if (splits > max_splits) splits = max_splits;
-        const int min_splits = ceil_div(N, wide16 ? gemv16_dz_max_slice() : gemv_dz_max_slice(B));
+        const int min_splits = ceil_div(N, wide16 ? gemv16_dz_max_slice(B) : gemv_dz_max_slice(B));
         if (splits < min_splits) splits = min_splits;
         int per = ceil_div(ceil_div(N, splits), step) * step;
         splits = ceil_div(N, per);

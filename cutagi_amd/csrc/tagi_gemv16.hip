@@ -52,6 +52,9 @@ constexpr int F16_C = 2;         // 16-element chunks per row and register stage
 constexpr int F16_KSTEP = 16 * F16_C;
 constexpr int F16_PAD = 4;       // LDS row stride % 32 == 4
 
+// NG: groups of 16 samples (1: up to 16 samples, 2: up to 32 - every weight fragment
+// then feeds two MFMAs, one per group, from the same registers).
+template <int NG>
 __global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_kernel(
     const float *__restrict__ mu_w, const float *__restrict__ var_w,
     const float *__restrict__ mu_a, const float *__restrict__ var_a, int K, int N, int B,
@@ -59,8 +62,9 @@ __global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_kernel(
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int RG = F16_RG, C = F16_C, KSTEP = F16_KSTEP;
     constexpr int ROWS_PER_BLOCK = W16_WAVES * RG * 16;
+    constexpr int NS = NG * W16_SAMPLES;
     const int S = k_per_split + F16_PAD;
-    float *s_mu = lds, *s_var = lds + W16_SAMPLES * S;
+    float *s_mu = lds, *s_var = lds + NS * S;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int i = lane & 15, kk = lane >> 4;
@@ -83,7 +87,7 @@ __global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_kernel(
 
     // stage the slice of the activations: [sample][k], zero beyond B and kr
     const int k4s = k_per_split / 4;
-    for (int e = tid; e < W16_SAMPLES * k4s; e += W16_WAVES * 64) {
+    for (int e = tid; e < NS * k4s; e += W16_WAVES * 64) {
         const int b = e / k4s, k = (e - b * k4s) * 4;
         float4 m = zero4(), v = zero4();
         if (b < B && k < kr) {
@@ -109,13 +113,15 @@ __global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_kernel(
 
     // the two variance terms have accumulators of their own, so that no MFMA waits
     // for the one issued just before it
-    floatx4 acc0[RG], acc1[RG], acc2[RG];
+    floatx4 acc0[NG][RG], acc1[NG][RG], acc2[NG][RG];
 #pragma unroll
-    for (int rg = 0; rg < RG; rg++) {
-        acc0[rg] = (floatx4){0.f, 0.f, 0.f, 0.f};
-        acc1[rg] = acc0[rg];
-        acc2[rg] = acc0[rg];
-    }
+    for (int g = 0; g < NG; g++)
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            acc0[g][rg] = (floatx4){0.f, 0.f, 0.f, 0.f};
+            acc1[g][rg] = acc0[g][rg];
+            acc2[g][rg] = acc0[g][rg];
+        }
 
     float4 sm[2][RG][C], sv[2][RG][C];
     auto load = [&](float4(&m)[RG][C], float4(&v)[RG][C], int kb) {
@@ -133,20 +139,26 @@ __global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_kernel(
 #pragma unroll
         for (int c = 0; c < C; c++) {
             const int at = kb + 16 * c + 4 * kk;
-            const float4 am = *reinterpret_cast<const float4 *>(s_mu + i * S + at);
-            const float4 av = *reinterpret_cast<const float4 *>(s_var + i * S + at);
-            const float4 as = make_float4(av.x + am.x * am.x, av.y + am.y * am.y,
-                                          av.z + am.z * am.z, av.w + am.w * am.w);
+            float4 am[NG], av[NG], as[NG];
+#pragma unroll
+            for (int g = 0; g < NG; g++) {
+                am[g] = *reinterpret_cast<const float4 *>(s_mu + (16 * g + i) * S + at);
+                av[g] = *reinterpret_cast<const float4 *>(s_var + (16 * g + i) * S + at);
+                as[g] = make_float4(av[g].x + am[g].x * am[g].x, av[g].y + am[g].y * am[g].y,
+                                    av[g].z + am[g].z * am[g].z, av[g].w + am[g].w * am[g].w);
+            }
 #pragma unroll
             for (int rg = 0; rg < RG; rg++) {
                 const float4 w = cm[rg][c], u = cv[rg][c];
                 const float4 q = sq4(w);
 #pragma unroll
-                for (int t = 0; t < 4; t++) {
-                    acc0[rg] = mfma16(comp(w, t), comp(am, t), acc0[rg]);
-                    acc1[rg] = mfma16(comp(u, t), comp(as, t), acc1[rg]);
-                    acc2[rg] = mfma16(comp(q, t), comp(av, t), acc2[rg]);
-                }
+                for (int t = 0; t < 4; t++)
+#pragma unroll
+                    for (int g = 0; g < NG; g++) {
+                        acc0[g][rg] = mfma16(comp(w, t), comp(am[g], t), acc0[g][rg]);
+                        acc1[g][rg] = mfma16(comp(u, t), comp(as[g], t), acc1[g][rg]);
+                        acc2[g][rg] = mfma16(comp(q, t), comp(av[g], t), acc2[g][rg]);
+                    }
             }
         }
     };
@@ -170,15 +182,17 @@ __global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_kernel(
         __builtin_amdgcn_sched_barrier(0);
     }
 
-    // register v of lane l: row n0 + 16*rg + 4*(l/16) + v, sample l%16
-    const int b = lane & 15;
-    if (b < B) {
+    // register v of lane l: row n0 + 16*rg + 4*(l/16) + v, sample 16*g + l%16
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+        const int b = 16 * g + (lane & 15);
+        if (b >= B) continue;
         const bool vec = (N & 3) == 0;
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) {
             const int n = n0 + 16 * rg + 4 * (lane >> 4);
             const size_t at = ((size_t)split * B + b) * N + n;
-            const floatx4 m = acc0[rg], v = acc1[rg] + acc2[rg];
+            const floatx4 m = acc0[g][rg], v = acc1[g][rg] + acc2[g][rg];
             if (vec && n + 3 < N) {
                 *reinterpret_cast<float4 *>(ws0 + at) = make_float4(m[0], m[1], m[2], m[3]);
                 *reinterpret_cast<float4 *>(ws1 + at) = make_float4(v[0], v[1], v[2], v[3]);
@@ -362,16 +376,18 @@ constexpr int Z16_PADQ = 1;    // plane stride per/4 + 4: spreads the kk planes 
 constexpr int Z16_WAVES = 8;   // side by side, 64 columns each (4 measured slower)
 constexpr int Z16_COLS = Z16_WAVES * 64;
 
+template <int NG>
 __global__ __launch_bounds__(Z16_WAVES * 64) void gemv16_dz_kernel(
     const float *__restrict__ mu_w, const float *__restrict__ dmu,
     const float *__restrict__ dvar, int K, int N, int B, int n_per_split,
     float *__restrict__ ws0, float *__restrict__ ws1) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int ST = Z16_ST;
+    constexpr int NS = NG * W16_SAMPLES;
     // the float4 of B operands must start at a multiple of 4 steps: Q % 4 == 0
     const int Q = n_per_split / 4 + 4 * Z16_PADQ;  // steps per (sample, kk) plane
     const int S = 4 * Q;                           // floats per sample
-    float *s_dm = lds, *s_dv = lds + W16_SAMPLES * S;
+    float *s_dm = lds, *s_dv = lds + NS * S;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int i = lane & 15, kk = lane >> 4;
@@ -393,7 +409,7 @@ __global__ __launch_bounds__(Z16_WAVES * 64) void gemv16_dz_kernel(
     };
     load(st[0], 0);
     // stage the innovations: global [sample][n] -> LDS [sample][n % 4][n / 4]
-    for (int e = tid; e < W16_SAMPLES * steps; e += Z16_WAVES * 64) {
+    for (int e = tid; e < NS * steps; e += Z16_WAVES * 64) {
         const int b = e / steps, step = e - b * steps;
         float4 m = zero4(), v = zero4();
         if (b < B && n_begin + 4 * step < N) {  // N % 4 == 0 on this path
@@ -405,25 +421,33 @@ __global__ __launch_bounds__(Z16_WAVES * 64) void gemv16_dz_kernel(
         pv[0] = v.x; pv[Q] = v.y; pv[2 * Q] = v.z; pv[3 * Q] = v.w;
     }
 
-    floatx4 acc0[4], acc1[4];
+    floatx4 acc0[NG][4], acc1[NG][4];
 #pragma unroll
-    for (int t = 0; t < 4; t++) {
-        acc0[t] = (floatx4){0.f, 0.f, 0.f, 0.f};
-        acc1[t] = acc0[t];
-    }
+    for (int g = 0; g < NG; g++)
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            acc0[g][t] = (floatx4){0.f, 0.f, 0.f, 0.f};
+            acc1[g][t] = acc0[g][t];
+        }
 
     auto multiply = [&](const float4(&cur)[ST], int s) {  // s: multiple of ST = 4
-        const float4 dm = *reinterpret_cast<const float4 *>(s_dm + i * S + kk * Q + s);
-        const float4 dv = *reinterpret_cast<const float4 *>(s_dv + i * S + kk * Q + s);
+        float4 dm[NG], dv[NG];
+#pragma unroll
+        for (int g = 0; g < NG; g++) {
+            dm[g] = *reinterpret_cast<const float4 *>(s_dm + (16 * g + i) * S + kk * Q + s);
+            dv[g] = *reinterpret_cast<const float4 *>(s_dv + (16 * g + i) * S + kk * Q + s);
+        }
 #pragma unroll
         for (int u = 0; u < ST; u++) {
             const float4 x = cur[u];
             const float4 q = sq4(x);
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
-                acc0[t] = mfma16(comp(x, t), comp(dm, u), acc0[t]);
-                acc1[t] = mfma16(comp(q, t), comp(dv, u), acc1[t]);
-            }
+            for (int t = 0; t < 4; t++)
+#pragma unroll
+                for (int g = 0; g < NG; g++) {
+                    acc0[g][t] = mfma16(comp(x, t), comp(dm[g], u), acc0[g][t]);
+                    acc1[g][t] = mfma16(comp(q, t), comp(dv[g], u), acc1[g][t]);
+                }
         }
     };
 
@@ -440,17 +464,21 @@ __global__ __launch_bounds__(Z16_WAVES * 64) void gemv16_dz_kernel(
         __builtin_amdgcn_sched_barrier(0);
     }
 
-    // register v of accumulator t of lane l: column c0 + 16*(l/16) + 4*v + t, sample l%16
-    if (i < B) {
+    // register v of accumulator t of lane l: column c0 + 16*(l/16) + 4*v + t, sample
+    // 16*g + l%16
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+        const int b = 16 * g + i;
+        if (b >= B) continue;
         const int c = c0 + 16 * (lane >> 4);
-        const size_t base = ((size_t)split * B + i) * K + c;
+        const size_t base = ((size_t)split * B + b) * K + c;
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             if (c + 4 * v < K) {  // K % 4 == 0 on this path
                 *reinterpret_cast<float4 *>(ws0 + base + 4 * v) =
-                    make_float4(acc0[0][v], acc0[1][v], acc0[2][v], acc0[3][v]);
+                    make_float4(acc0[g][0][v], acc0[g][1][v], acc0[g][2][v], acc0[g][3][v]);
                 *reinterpret_cast<float4 *>(ws1 + base + 4 * v) =
-                    make_float4(acc1[0][v], acc1[1][v], acc1[2][v], acc1[3][v]);
+                    make_float4(acc1[g][0][v], acc1[g][1][v], acc1[g][2][v], acc1[g][3][v]);
             }
         }
     }
@@ -469,36 +497,39 @@ int g_gemv16_fwd_lines = 0;
 
 int gemv16_fwd_rows_per_block() { return W16_WAVES * F16_RG * 16; }
 int gemv16_fwd_k_step() { return g_gemv16_fwd_lines ? T16_DEPTH * T16_STAGE : F16_KROUND; }
-int gemv16_fwd_max_slice() {
-    if (g_gemv16_fwd_lines) {
+// sample slots the kernels stage for a batch of B: 16 up to 16 samples, 32 beyond
+static int sample_slots(int B) { return B <= W16_SAMPLES ? W16_SAMPLES : 2 * W16_SAMPLES; }
+int gemv16_max_batch() { return 2 * W16_SAMPLES; }
+int gemv16_fwd_max_slice(int B) {
+    if (g_gemv16_fwd_lines && B <= W16_SAMPLES) {
         // one workgroup per CU: the activations of a slice plus the waves' tiles
         const size_t budget = 150 * 1024 - (size_t)W16_WAVES * 2 * T16_TILE * sizeof(float);
         int s = (int)(budget / (2 * W16_SAMPLES * sizeof(float)) - F16_PAD) /
                 (T16_DEPTH * T16_STAGE) * (T16_DEPTH * T16_STAGE);
         return s > 512 ? 512 : s;
     }
-    return (int)(W16_LDS_BUDGET / (2 * W16_SAMPLES * sizeof(float)) - F16_PAD) / F16_KROUND *
+    return (int)(W16_LDS_BUDGET / (2 * sample_slots(B) * sizeof(float)) - F16_PAD) / F16_KROUND *
            F16_KROUND;
 }
 int gemv16_dz_cols_per_block() { return Z16_COLS; }
 int gemv16_dz_n_step() { return Z16_NSTEP; }
-int gemv16_dz_max_slice() {
-    return (int)(W16_LDS_BUDGET / (2 * W16_SAMPLES * sizeof(float)) - 16 * Z16_PADQ) / Z16_NSTEP *
-           Z16_NSTEP;
+int gemv16_dz_max_slice(int B) {
+    return (int)(W16_LDS_BUDGET / (2 * sample_slots(B) * sizeof(float)) - 16 * Z16_PADQ) /
+           Z16_NSTEP * Z16_NSTEP;
 }
 
-// k_per_split: a multiple of gemv16_fwd_k_step(), at most gemv16_fwd_max_slice();
+// k_per_split: a multiple of gemv16_fwd_k_step(), at most gemv16_fwd_max_slice(B);
 // ws0/ws1: [splits][B][N] partial sums for the caller to fold.
 hipError_t launch_gemv16_fwd(const float *mu_w, const float *var_w, const float *mu_a,
                              const float *var_a, int K, int N, int B, int k_per_split,
                              int splits, float *ws0, float *ws1, hipStream_t stream) {
-    if (B < 1 || B > W16_SAMPLES || K % 4 != 0 || k_per_split % gemv16_fwd_k_step() != 0 ||
-        k_per_split > gemv16_fwd_max_slice() || (long long)k_per_split * splits < K)
+    if (B < 1 || B > gemv16_max_batch() || K % 4 != 0 || k_per_split % gemv16_fwd_k_step() != 0 ||
+        k_per_split > gemv16_fwd_max_slice(B) || (long long)k_per_split * splits < K)
         return hipErrorInvalidValue;
-    size_t lds = (size_t)2 * W16_SAMPLES * (k_per_split + F16_PAD) * sizeof(float);
+    size_t lds = (size_t)2 * sample_slots(B) * (k_per_split + F16_PAD) * sizeof(float);
     const int rows = gemv16_fwd_rows_per_block();
     dim3 grid(((N + rows - 1) / rows) * splits), block(W16_WAVES * 64);
-    if (g_gemv16_fwd_lines) {
+    if (g_gemv16_fwd_lines && B <= W16_SAMPLES) {
         lds += (size_t)W16_WAVES * 2 * T16_TILE * sizeof(float);
         static PerDeviceOnce once_lines;
         hipError_t e = allow_dynamic_lds(
@@ -508,31 +539,51 @@ hipError_t launch_gemv16_fwd(const float *mu_w, const float *var_w, const float 
                            var_a, K, N, B, k_per_split, splits, ws0, ws1);
         return hipGetLastError();
     }
-    static PerDeviceOnce once;
-    hipError_t e = allow_dynamic_lds(once, reinterpret_cast<const void *>(gemv16_fwd_kernel), 160 * 1024);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(gemv16_fwd_kernel, grid, block, lds, stream, mu_w, var_w, mu_a, var_a, K,
-                       N, B, k_per_split, splits, ws0, ws1);
+    if (B <= W16_SAMPLES) {
+        static PerDeviceOnce once;
+        hipError_t e = allow_dynamic_lds(
+            once, reinterpret_cast<const void *>(gemv16_fwd_kernel<1>), 160 * 1024);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(gemv16_fwd_kernel<1>, grid, block, lds, stream, mu_w, var_w, mu_a, var_a,
+                           K, N, B, k_per_split, splits, ws0, ws1);
+    } else {
+        static PerDeviceOnce once2;
+        hipError_t e = allow_dynamic_lds(
+            once2, reinterpret_cast<const void *>(gemv16_fwd_kernel<2>), 160 * 1024);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(gemv16_fwd_kernel<2>, grid, block, lds, stream, mu_w, var_w, mu_a, var_a,
+                           K, N, B, k_per_split, splits, ws0, ws1);
+    }
     return hipGetLastError();
 }
 
-// n_per_split: a multiple of gemv16_dz_n_step(), at most gemv16_dz_max_slice();
+// n_per_split: a multiple of gemv16_dz_n_step(), at most gemv16_dz_max_slice(B);
 // ws0/ws1: [splits][B][K] partial sums for the caller to fold.
 hipError_t launch_gemv16_dz(const float *mu_w, const float *dmu, const float *dvar, int K, int N,
                             int B, int n_per_split, int splits, float *ws0, float *ws1,
                             hipStream_t stream) {
-    if (B < 1 || B > W16_SAMPLES || K % 4 != 0 || N % 4 != 0 || n_per_split % Z16_NSTEP != 0 ||
-        n_per_split > gemv16_dz_max_slice() || (long long)n_per_split * splits < N ||
-        splits > 65535)
+    if (B < 1 || B > gemv16_max_batch() || K % 4 != 0 || N % 4 != 0 ||
+        n_per_split % Z16_NSTEP != 0 || n_per_split > gemv16_dz_max_slice(B) ||
+        (long long)n_per_split * splits < N || splits > 65535)
         return hipErrorInvalidValue;
-    const size_t lds = (size_t)2 * W16_SAMPLES * (n_per_split + 16 * Z16_PADQ) * sizeof(float);
-    static PerDeviceOnce once;
-    hipError_t e = allow_dynamic_lds(once, reinterpret_cast<const void *>(gemv16_dz_kernel), 160 * 1024);
-    if (e != hipSuccess) return e;
+    const size_t lds = (size_t)2 * sample_slots(B) * (n_per_split + 16 * Z16_PADQ) * sizeof(float);
     const int cols = gemv16_dz_cols_per_block();
     dim3 grid((K + cols - 1) / cols, splits), block(Z16_WAVES * 64);
-    hipLaunchKernelGGL(gemv16_dz_kernel, grid, block, lds, stream, mu_w, dmu, dvar, K, N, B,
-                       n_per_split, ws0, ws1);
+    if (B <= W16_SAMPLES) {
+        static PerDeviceOnce once;
+        hipError_t e = allow_dynamic_lds(
+            once, reinterpret_cast<const void *>(gemv16_dz_kernel<1>), 160 * 1024);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(gemv16_dz_kernel<1>, grid, block, lds, stream, mu_w, dmu, dvar, K, N, B,
+                           n_per_split, ws0, ws1);
+    } else {
+        static PerDeviceOnce once2;
+        hipError_t e = allow_dynamic_lds(
+            once2, reinterpret_cast<const void *>(gemv16_dz_kernel<2>), 160 * 1024);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(gemv16_dz_kernel<2>, grid, block, lds, stream, mu_w, dmu, dvar, K, N, B,
+                           n_per_split, ws0, ws1);
+    }
     return hipGetLastError();
 }
 

@@ -116,7 +116,8 @@ hipError_t launch_gemv_dw(const float *var_w, const float *mu_a, const float *dm
                           const float *dvar, int K, int N, int B, int rev, float *dmu_w,
                           float *dvar_w, const float *var_b, float *dmu_b, float *dvar_b,
                           const DzFold *fold, hipStream_t stream);
-// The same for 9 <= B <= 16 on the 16x16x4 MFMA (tagi_gemv16.hip); slices are
+// The same for 9 <= B <= 32 on the 16x16x4 MFMA (tagi_gemv16.hip; beyond 16 samples every
+// weight fragment feeds two MFMAs); slices are
 // multiples of the *_step() and at most the *_max_slice().
 hipError_t launch_gemv16_fwd(const float *mu_w, const float *var_w, const float *mu_a,
                              const float *var_a, int K, int N, int B, int k_per_split,
@@ -128,10 +129,11 @@ hipError_t launch_gemv16_dz(const float *mu_w, const float *dmu, const float *dv
 extern int g_gemv16_fwd_lines;
 int gemv16_fwd_rows_per_block();
 int gemv16_fwd_k_step();
-int gemv16_fwd_max_slice();
+int gemv16_fwd_max_slice(int B);
+int gemv16_max_batch();  // 32: two groups of sixteen samples
 int gemv16_dz_cols_per_block();
 int gemv16_dz_n_step();
-int gemv16_dz_max_slice();
+int gemv16_dz_max_slice(int B);
 int gemv_fwd_variants();
 int gemv_fwd_rows_per_block(int variant);
 int gemv_fwd_k_step();

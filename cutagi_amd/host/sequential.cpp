@@ -445,10 +445,25 @@ void Sequential::enable_graphs(bool on) {
     HIP_OK(hipDeviceSynchronize());
     this->clear_graphs();
     graphs_on_ = on;
-    if (on) set_host_stream(graph_stream());
+    // the host classes share one stream: it is the recording stream while any model has
+    // graphs on, the null stream otherwise
+    static int models_with_graphs = 0;
+    models_with_graphs += on ? 1 : -1;
+    set_host_stream(models_with_graphs > 0 ? graph_stream() : nullptr);
     // replayed work must meet the same arrays every step: no trading with the buffers
     for (auto *b : {output_z_buffer.get(), input_z_buffer.get()})
         if (auto *h = dynamic_cast<HiddenStateHip *>(b)) h->transient = !on;
+}
+
+Sequential::~Sequential() {
+    // (a model destroyed with graphs on hands the stream back like one that switches off)
+    if (graphs_on_ && this->device == "cuda") {
+        try {
+            this->enable_graphs(false);
+        } catch (...) {
+        }
+    }
+    this->clear_graphs();
 }
 
 int Sequential::graphs_captured() const {

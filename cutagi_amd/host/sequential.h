@@ -76,7 +76,7 @@ class Sequential {
     std::vector<std::shared_ptr<BaseLayer>> layers;
 
     Sequential() = default;
-    ~Sequential() { this->clear_graphs(); }
+    ~Sequential();
     Sequential(const Sequential &) = delete;
     Sequential &operator=(const Sequential &) = delete;
     void add_layer(std::shared_ptr<BaseLayer> layer);

@@ -18,7 +18,9 @@ extern "C" {
  * "linear.dz.splits", "linear.dw.splits", "linear.gemv_max_batch" (largest batch of
  * the streaming kernels, at most 16), "linear.gemv.swizzle",
  * "linear.gemv.fwd_variant", "linear.gemv.reverse", "linear.gemv16" (0: 9..16
- * samples on the kernels for up to 8), "linear.gemv16.fwd_lines" (1: the 9..16-sample
+ * samples on the kernels for up to 8), "linear.gemv32" (0: the forward of 17..32
+ * samples on the tiled kernel instead of the 16-wide streaming one; 2: their state
+ * backward on the streaming kernel too), "linear.gemv16.fwd_lines" (1: the 9..16-sample
  * forward that loads whole cache lines and transposes them in LDS), "linear.dw_side" (0: bias innovations and
  * the state-backward fold as launches of their own instead of inside the
  * weight-backward launch), "linear.double_buffer". Conv2d: "conv2d.tile",

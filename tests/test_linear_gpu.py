@@ -17,6 +17,8 @@ SHAPES = [
     (2048, 48, 7), (768, 1000, 3), (4096, 16, 16), (260, 20, 9),
     # 9..16 samples: the 16-wide streaming kernels (several slices, ragged rows and columns)
     (1024, 512, 16), (1536, 260, 12), (72, 1028, 10), (2052, 300, 13), (512, 2048, 9),
+    # 17..32 samples: the same kernels with two groups of sixteen samples
+    (1024, 512, 32), (1536, 260, 24), (72, 1028, 17), (516, 300, 31), (4096, 256, 20),
 ]
 
 
@@ -183,3 +185,24 @@ def test_both_forward_kernels_for_9_to_16_samples(oracle_lib, K, N, B):
             assert_close(got[lines][1], ref[1], "var_z (lines=%d)" % lines, same_sign=True)
     finally:
         capi.tune("linear.gemv16.fwd_lines", -1)
+
+
+@pytest.mark.parametrize("K,N,B", [(1024, 512, 32), (1536, 260, 24), (516, 300, 31)])
+def test_state_backward_streaming_kernel_for_17_to_32_samples(oracle_lib, K, N, B):
+    """The two-group form of the 16-wide state backward (not the default above 16
+    samples: the tiled kernel measures faster there) still gives the oracle's result."""
+    import cutagi_amd.functional as F
+    from cutagi_amd import capi
+    d = linear_inputs(K, N, B, seed=K + N + B, bias=True, jcb_random=True)
+    t = _dev(d)
+    ref = oracle_lib.linear_bwd_dz(d["mu_w"], d["jcb"], d["delta_mu"], d["delta_var"], threads=4)
+    capi.tune("linear.gemv32", 2)
+    try:
+        dz = F.linear_bwd_dz(t["mu_w"], t["jcb"], t["delta_mu"], t["delta_var"])
+        out = F.linear_bwd(t["mu_w"], t["var_w"], t["var_b"], t["mu_a"], t["jcb"], t["delta_mu"],
+                           t["delta_var"])
+    finally:
+        capi.tune("linear.gemv32", -1)
+    for got in (dz, out[:2]):
+        assert_close(got[0].cpu().numpy(), ref[0], "delta_mu_z")
+        assert_close(got[1].cpu().numpy(), ref[1], "delta_var_z", same_sign=True)
