@@ -13,7 +13,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtagi_hip.so")
-SOURCES = ["tagi_gemm.hip", "tagi_gemv.hip", "tagi_gemv16.hip", "tagi_elementwise.hip",
+SOURCES = ["tagi_gemm.hip", "tagi_gemv.hip", "tagi_gemv16.hip", "tagi_small.hip", "tagi_elementwise.hip",
            "tagi_conv2d.hip", "tagi_layers.hip", "tagi_conv_idx.cpp", "tagi_capi.hip"]
 # packed fp32 VALU ops are kept off for gfx950 (device pass only; the host pass
 # does not know the feature and says so)

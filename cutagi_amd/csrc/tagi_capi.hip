@@ -21,7 +21,7 @@ static __device__ __align__(256) float scratch[STATIC_SCRATCH_BYTES / sizeof(flo
 
 namespace {
 
-constexpr int ABI_VERSION = 101;
+constexpr int ABI_VERSION = 103;
 
 #define TAGI_TRY(expr)                          \
     do {                                        \
@@ -111,6 +111,10 @@ struct Tuning {
     int gemv16 = -1;    // 0: 9..16 samples on the 4x4x1 kernels too
     int wide32 = -1;    // 0: 17..32 samples on the tiled kernels; 2: state backward streams too
     int dw_side = -1;   // 0: bias innovations and the state-backward fold as launches of their own
+    // >= 0: the smallest weight matrix (elements) the streaming kernels take, whatever the
+    // batch; -1: the measured thresholds of streams_weights()
+    long long stream_min_weights = -1;
+    int small = -1;     // 0: small layers on the tiled / streaming kernels too
 };
 Tuning g_tune;
 
@@ -158,6 +162,25 @@ int gemv_max_batch() {
 int wide_max_batch() {
     if (g_tune.gemv_max_batch >= 0 && g_tune.gemv_max_batch < 16) return g_tune.gemv_max_batch;
     return g_tune.wide32 == 0 ? 16 : gemv16_max_batch();
+}
+
+// Whether a layer of n x k weights goes to the streaming kernels (one pass over the
+// weights, activations resident in LDS) or to the tiled kernel. The streaming kernels win
+// where reading the weights is what takes the time; on smaller layers a launch is bound by
+// latency and the tiled kernel's many short slices finish sooner. Thresholds from kernel
+// times at 128^2 .. 4096^2 (weights in elements):
+//   forward        <= 8 samples: 8M (4096^2: 29 against 39 us; 2048^2: 25 against 19 us)
+//                  9..16: 2M (2048^2: 15.6 against 19.7 us; 1024^2: 15.3 against 13.3 us)
+//                  17..32: 8M (4096^2: 36 against 41 us; 2048^2: 22.4 against 21.3 us)
+//   state backward <= 8 samples: 4M (4096^2: 19-22 against 28 us; 1024^2: 13-16 against 11 us)
+//                  9..16: 2M (2048x1024: 13.5 against 14.4 us; 1024^2: 12.7 against 12.2 us)
+enum StreamOp { STREAM_FWD, STREAM_DZ };
+bool streams_weights(StreamOp op, int n, int k, int batch) {
+    const long long weights = (long long)n * k;
+    if (g_tune.stream_min_weights >= 0) return weights >= g_tune.stream_min_weights;
+    const long long M = 1ll << 20;
+    if (op == STREAM_FWD) return weights >= (batch <= 8 ? 8 * M : batch <= 16 ? 2 * M : 8 * M);
+    return weights >= (batch <= 8 ? 4 * M : 2 * M);
 }
 
 // Tile shape and reduction slices of a tiled launch.
@@ -311,6 +334,8 @@ int tagi_hip_tune(const char *key, int value) {
     else if (!strcmp(key, "linear.gemv16")) g_tune.gemv16 = value;
     else if (!strcmp(key, "linear.gemv32")) g_tune.wide32 = value;
     else if (!strcmp(key, "linear.gemv16.fwd_lines")) g_gemv16_fwd_lines = value < 0 ? 0 : value;
+    else if (!strcmp(key, "linear.stream_min_weights")) g_tune.stream_min_weights = value;
+    else if (!strcmp(key, "linear.small")) g_tune.small = value;
     else return TAGI_ERR_INVALID_ARG;
     return TAGI_OK;
 }
@@ -332,7 +357,14 @@ static int linear_fwd_impl(const float *mu_w, const float *var_w, const float *m
     const bool vec = (K % 4 == 0) && aligned16(mu_w) && aligned16(var_w) && aligned16(mu_a) &&
                      aligned16(var_a);
 
-    if (B > 8 && B <= wide_max_batch() && vec && g_tune.gemv16 != 0) {
+    if (vec && g_tune.small != 0 && g_tune.stream_min_weights < 0 && small_fwd_supported(K, N, B)) {
+        // small layers: one launch, bias and activation included
+        TAGI_TRY(launch_small_fwd(mu_w, var_w, e0, e1, mu_a, var_a, K, N, B, act, mu_z, var_z, jcb,
+                                  stream));
+        return TAGI_OK;
+    }
+    const bool streams = streams_weights(STREAM_FWD, N, K, B);
+    if (B > 8 && B <= wide_max_batch() && vec && g_tune.gemv16 != 0 && streams) {
         // 9..32 samples: the 16-wide streaming kernel (two sample groups beyond 16)
         const int blocks = ceil_div(N, gemv16_fwd_rows_per_block());
         const int step = gemv16_fwd_k_step();
@@ -354,7 +386,7 @@ static int linear_fwd_impl(const float *mu_w, const float *var_w, const float *m
         return TAGI_OK;
     }
 
-    if (B <= gemv_max_batch() && vec) {
+    if (B <= gemv_max_batch() && vec && streams) {
         // slices: short enough for the LDS-resident activations, and enough of
         // them for about two workgroups per CU
         const int variant = (g_tune.gemv_fwd_variant >= 0 &&
@@ -429,7 +461,7 @@ static int linear_bwd_dz_impl(const float *mu_w, const float *jcb, const float *
 
     const bool wide16 = B > 8 && B <= (g_tune.wide32 == 2 ? wide_max_batch() : gemv_max_batch()) &&
                         g_tune.gemv16 != 0;
-    if ((B <= gemv_max_batch() || wide16) && vec) {
+    if ((B <= gemv_max_batch() || wide16) && vec && streams_weights(STREAM_DZ, N, K, B)) {
         const int blocks = ceil_div(K, wide16 ? gemv16_dz_cols_per_block() : gemv_dz_cols_per_block());
         const int step = wide16 ? gemv16_dz_n_step() : gemv_dz_n_step();
         int splits = g_tune.dz_splits > 0 ? g_tune.dz_splits : ceil_div(num_cu(), blocks);
@@ -899,6 +931,37 @@ int tagi_out_update_indexed(const float *mu_a, const float *var_a, const float *
         return TAGI_ERR_INVALID_ARG;
     TAGI_TRY(launch_out_update_indexed(mu_a, var_a, jcb, obs, var_obs, selected_idx, n_obs, n_enc,
                                        n, delta_mu, delta_var, static_cast<hipStream_t>(stream_)));
+    return TAGI_OK;
+}
+
+int tagi_out_update_indexed_reset(const float *mu_a, const float *var_a, const float *jcb,
+                                  const float *obs, const float *var_obs, const int *selected_idx,
+                                  int n_obs, int n_enc, int n, float *delta_mu, float *delta_var,
+                                  size_t delta_len, void *stream_) {
+    if (n < 0 || n_obs <= 0 || n_enc <= 0 || n % n_enc != 0) return TAGI_ERR_INVALID_ARG;
+    if ((n > 0 || delta_len > 0) && (!delta_mu || !delta_var)) return TAGI_ERR_INVALID_ARG;
+    if (n > 0 && (!mu_a || !var_a || !jcb || !obs || !var_obs || !selected_idx))
+        return TAGI_ERR_INVALID_ARG;
+    if ((size_t)(n / n_enc) * n_obs > delta_len) return TAGI_ERR_INVALID_ARG;
+    TAGI_TRY(launch_out_update_indexed_reset(mu_a, var_a, jcb, obs, var_obs, selected_idx, n_obs,
+                                             n_enc, n / n_enc, delta_mu, delta_var, delta_len,
+                                             static_cast<hipStream_t>(stream_)));
+    return TAGI_OK;
+}
+
+int tagi_upload_input(const float *host_mu, const float *host_var, size_t n, float *mu_a,
+                      float *var_a, void *stream_) {
+    if (n > 0 && (!host_mu || !mu_a || !var_a)) return TAGI_ERR_INVALID_ARG;
+    TAGI_TRY(launch_upload_input(host_mu, host_var, n, mu_a, var_a,
+                                 static_cast<hipStream_t>(stream_)));
+    return TAGI_OK;
+}
+
+int tagi_download_outputs(const float *mu_a, const float *var_a, size_t n, float *host_mu,
+                          float *host_var, void *stream_) {
+    if (n > 0 && (!mu_a || !var_a || !host_mu || !host_var)) return TAGI_ERR_INVALID_ARG;
+    TAGI_TRY(launch_download_outputs(mu_a, var_a, n, host_mu, host_var,
+                                     static_cast<hipStream_t>(stream_)));
     return TAGI_OK;
 }
 

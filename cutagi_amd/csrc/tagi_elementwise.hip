@@ -58,6 +58,35 @@ __global__ __launch_bounds__(TPB) void store_states_kernel(
     if (i < n_out) out_jcb[i] = 1.0f;
 }
 
+// Input of a network from pinned host memory straight into the state arrays: the mean
+// is read over the bus by the kernel itself, the variance likewise or (host_var == null)
+// set to zero. One launch on the compute queue instead of two copy-engine transfers and
+// a fill, each of which costs a hand-over between engines on a short dependent chain.
+__global__ __launch_bounds__(TPB) void upload_input_kernel(const float *__restrict__ host_mu,
+                                                           const float *__restrict__ host_var,
+                                                           size_t n, float *__restrict__ mu_a,
+                                                           float *__restrict__ var_a) {
+    const size_t stride = (size_t)gridDim.x * TPB;
+    for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += stride) {
+        mu_a[i] = host_mu[i];
+        var_a[i] = host_var != nullptr ? host_var[i] : 0.f;
+    }
+}
+
+// The other direction: the first n means and variances of a state buffer written
+// straight into pinned host memory by the kernel (one launch and one wait for the
+// stream instead of two synchronous copies).
+__global__ __launch_bounds__(TPB) void download_outputs_kernel(const float *__restrict__ mu_a,
+                                                               const float *__restrict__ var_a,
+                                                               size_t n, float *__restrict__ host_mu,
+                                                               float *__restrict__ host_var) {
+    const size_t stride = (size_t)gridDim.x * TPB;
+    for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += stride) {
+        host_mu[i] = mu_a[i];
+        host_var[i] = var_a[i];
+    }
+}
+
 // p += sign(d) * min(|d|, sqrt(var)/cap); var <= 0 -> 1e-5 and counted. One
 // atomic per wave: the clamped lanes are counted with a ballot.
 __global__ __launch_bounds__(TPB) void param_update_kernel(
@@ -242,6 +271,60 @@ __global__ __launch_bounds__(TPB) void out_update_indexed_kernel(
     }
 }
 
+// The same with the clearing of the innovation buffers included: workgroup b < samples
+// owns sample b's n_obs entries (zeroed, then the selected ones written, in that order
+// behind a barrier); the workgroups after those zero the rest of the buffers. The
+// observations may lie in pinned host memory (read once each).
+__global__ __launch_bounds__(TPB) void out_update_indexed_reset_kernel(
+    const float *__restrict__ mu_a, const float *__restrict__ var_a,
+    const float *__restrict__ jcb, const float *__restrict__ obs,
+    const float *__restrict__ var_obs, const int *__restrict__ sel, int n_obs, int n_enc,
+    int samples, float *__restrict__ dmu, float *__restrict__ dvar, size_t delta_len) {
+    if ((int)blockIdx.x < samples) {
+        const int b = blockIdx.x;
+        // ask for the observations first: they may come over the host link
+        float y = 0.f, vy = 0.f;
+        int s = 0;
+        const bool has = (int)threadIdx.x < n_enc;
+        if (has) {
+            const int col = b * n_enc + threadIdx.x;
+            y = obs[col];
+            vy = var_obs[col];
+            s = sel[col];
+        }
+        const size_t base = (size_t)b * n_obs;
+        for (int i = threadIdx.x; i < n_obs; i += TPB)
+            if (base + i < delta_len) {
+                dmu[base + i] = 0.f;
+                dvar[base + i] = 0.f;
+            }
+        __syncthreads();
+        for (int e = threadIdx.x; e < n_enc; e += TPB) {
+            if (e >= TPB) {      // more than one observation per thread: the later ones
+                const int col = b * n_enc + e;
+                y = obs[col];
+                vy = var_obs[col];
+                s = sel[col];
+            }
+            const size_t idx = base + s - 1;  // sel is 1-based
+            const float j = jcb[idx];
+            const float t = j / (var_a[idx] + vy);
+            if (!(isinf(t) || isnan(t))) {
+                dmu[idx] = t * (y - mu_a[idx]);
+                dvar[idx] = -t * j;
+            }
+        }
+        return;
+    }
+    const size_t first = (size_t)samples * n_obs;
+    const size_t stride = (size_t)(gridDim.x - samples) * TPB;
+    for (size_t i = first + (size_t)(blockIdx.x - samples) * TPB + threadIdx.x; i < delta_len;
+         i += stride) {
+        dmu[i] = 0.f;
+        dvar[i] = 0.f;
+    }
+}
+
 // No __restrict__: the call may run in place (mu_a == mu_z, var_a == var_z).
 __global__ __launch_bounds__(TPB) void relu_kernel(const float *mu_z, const float *var_z,
                                                    size_t n, float *mu_a, float *jcb,
@@ -335,6 +418,38 @@ hipError_t launch_out_update_indexed(const float *mu_a, const float *var_a, cons
     if (n == 0) return hipSuccess;
     hipLaunchKernelGGL(out_update_indexed_kernel, dim3(blocks_for(n, TPB)), dim3(TPB), 0, stream,
                        mu_a, var_a, jcb, obs, var_obs, sel, n_obs, n_enc, n, dmu, dvar);
+    return hipGetLastError();
+}
+
+hipError_t launch_out_update_indexed_reset(const float *mu_a, const float *var_a, const float *jcb,
+                                           const float *obs, const float *var_obs, const int *sel,
+                                           int n_obs, int n_enc, int samples, float *dmu,
+                                           float *dvar, size_t delta_len, hipStream_t stream) {
+    const size_t rest = delta_len > (size_t)samples * n_obs ? delta_len - (size_t)samples * n_obs : 0;
+    unsigned zero_blocks = blocks_for(rest, 4 * TPB);
+    if (zero_blocks > 1024u) zero_blocks = 1024u;
+    if (samples + zero_blocks == 0) return hipSuccess;
+    hipLaunchKernelGGL(out_update_indexed_reset_kernel, dim3(samples + zero_blocks), dim3(TPB), 0,
+                       stream, mu_a, var_a, jcb, obs, var_obs, sel, n_obs, n_enc, samples, dmu,
+                       dvar, delta_len);
+    return hipGetLastError();
+}
+
+hipError_t launch_upload_input(const float *host_mu, const float *host_var, size_t n, float *mu_a,
+                               float *var_a, hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    const unsigned blocks = blocks_for(n, TPB) < 1024u ? blocks_for(n, TPB) : 1024u;
+    hipLaunchKernelGGL(upload_input_kernel, dim3(blocks), dim3(TPB), 0, stream, host_mu, host_var, n,
+                       mu_a, var_a);
+    return hipGetLastError();
+}
+
+hipError_t launch_download_outputs(const float *mu_a, const float *var_a, size_t n, float *host_mu,
+                                   float *host_var, hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    const unsigned blocks = blocks_for(n, TPB) < 1024u ? blocks_for(n, TPB) : 1024u;
+    hipLaunchKernelGGL(download_outputs_kernel, dim3(blocks), dim3(TPB), 0, stream, mu_a, var_a, n,
+                       host_mu, host_var);
     return hipGetLastError();
 }
 

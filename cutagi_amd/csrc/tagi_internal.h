@@ -95,6 +95,14 @@ hipError_t launch_reduce_splits(Epilogue epi, const float *ws0, const float *ws1
                                 const float *e1, float *out0, float *out1, int ldo,
                                 hipStream_t stream, int act = 0, float *out2 = nullptr);
 
+// Forward of small layers in one launch (no slices, no LDS): one wave per 2 rows x 8
+// samples, lanes across the reduction. Needs K % 4 == 0 and 16-byte aligned pointers.
+bool small_fwd_supported(int K, int N, int B);
+hipError_t launch_small_fwd(const float *mu_w, const float *var_w, const float *mu_b,
+                            const float *var_b, const float *mu_a, const float *var_a, int K,
+                            int N, int B, int act, float *out0, float *out1, float *out2,
+                            hipStream_t stream);
+
 // Skinny-batch (B <= 16) streaming kernels: weights are read once from HBM
 // straight into MFMA operand layout, nothing is staged in LDS.
 hipError_t launch_gemv_fwd(const float *mu_w, const float *var_w, const float *mu_a,
@@ -184,6 +192,14 @@ hipError_t launch_out_update_indexed(const float *mu_a, const float *var_a, cons
                                      hipStream_t stream);
 hipError_t launch_relu(const float *mu_z, const float *var_z, size_t n, float *mu_a, float *jcb,
                        float *var_a, hipStream_t stream);
+hipError_t launch_out_update_indexed_reset(const float *mu_a, const float *var_a, const float *jcb,
+                                           const float *obs, const float *var_obs, const int *sel,
+                                           int n_obs, int n_enc, int samples, float *dmu,
+                                           float *dvar, size_t delta_len, hipStream_t stream);
+hipError_t launch_download_outputs(const float *mu_a, const float *var_a, size_t n, float *host_mu,
+                                   float *host_var, hipStream_t stream);
+hipError_t launch_upload_input(const float *host_mu, const float *host_var, size_t n, float *mu_a,
+                               float *var_a, hipStream_t stream);
 
 // Layers between the contractions (tagi_layers.hip)
 hipError_t launch_mixture_relu(const float *mu_z, const float *var_z, size_t n, float *mu_a,

@@ -187,13 +187,19 @@ void OutputUpdater::update_using_indices_raw(BaseHiddenStates &output_states,
     o->size = n;
     o->actual_size = n / output_states.block_size;
     o->idx_size = n;
-    o->upload(mu_obs, var_obs, n, selected_idx, n);
     const int n_enc = (int)(o->idx_size / output_states.block_size);
-    delta->reset_zeros();
-    TAGI_OK_OR_THROW(tagi_out_update_indexed(out->d_mu_a, out->d_var_a, out->jcb_ptr(), o->d_mu_obs,
-                                             o->d_var_obs, o->d_selected_idx, n_obs, n_enc,
-                                             (int)o->size, delta->d_delta_mu, delta->d_delta_var,
-                                             host_stream()));
+    if ((size_t)output_states.block_size * n_obs > delta->size)
+        LOG(LogLevel::ERROR, "Output size does not fit the innovation buffers");
+    // one launch: the kernel reads the observations where they are staged in pinned
+    // memory and clears the rest of the innovation buffers itself
+    const float *mu_at = nullptr, *var_at = nullptr;
+    const int *idx_at = nullptr;
+    o->stage(mu_obs, var_obs, n, selected_idx, &mu_at, &var_at, &idx_at);
+    TAGI_OK_OR_THROW(tagi_out_update_indexed_reset(out->d_mu_a, out->d_var_a, out->jcb_ptr(), mu_at,
+                                                   var_at, idx_at, n_obs, n_enc, (int)n,
+                                                   delta->d_delta_mu, delta->d_delta_var,
+                                                   delta->size, host_stream()));
+    o->staged_work_queued();
 }
 
 void OutputUpdater::update_heteros(BaseHiddenStates &output_states, std::vector<float> &mu_obs,

@@ -16,6 +16,9 @@
 
 namespace tagi_host {
 
+// inputs up to this size are fetched from pinned memory by a kernel (tagi_upload_input)
+static constexpr size_t kKernelUploadMaxBytes = (size_t)1 << 20;
+
 // (declared in host_util.h) the stream the host classes queue their device work on
 static hipStream_t g_host_stream = nullptr;
 hipStream_t host_stream() { return g_host_stream; }
@@ -63,7 +66,17 @@ class StagingRing {
         size_t bytes = 0;
         for (int i = 0; i < n; i++) bytes += sizes[i];
         if (bytes == 0) return;
+        void *host = this->stage(parts, sizes, n);
+        HIP_OK(hipMemcpyAsync(dst, host, bytes, hipMemcpyHostToDevice, host_stream()));
+        this->staged_work_queued();
+    }
+    // Copies the pieces back to back into the next pinned slot and returns it; the caller
+    // queues the device work that reads the slot and then calls staged_work_queued().
+    void *stage(const void *const *parts, const size_t *sizes, int n) {
+        size_t bytes = 0;
+        for (int i = 0; i < n; i++) bytes += sizes[i];
         Slot &s = slots_[next_];
+        current_ = next_;
         next_ = (next_ + 1) % SLOTS;
         if (s.event == nullptr) HIP_OK(hipEventCreateWithFlags(&s.event, hipEventDisableTiming));
         if (s.used) HIP_OK(hipEventSynchronize(s.event));
@@ -77,7 +90,10 @@ class StagingRing {
             if (sizes[i]) std::memcpy(static_cast<char *>(s.host) + at, parts[i], sizes[i]);
             at += sizes[i];
         }
-        HIP_OK(hipMemcpyAsync(dst, s.host, bytes, hipMemcpyHostToDevice, host_stream()));
+        return s.host;
+    }
+    void staged_work_queued() {
+        Slot &s = slots_[current_];
         HIP_OK(hipEventRecord(s.event, host_stream()));
         s.used = true;
     }
@@ -90,7 +106,7 @@ class StagingRing {
         bool used = false;
     };
     Slot slots_[SLOTS];
-    int next_ = 0;
+    int next_ = 0, current_ = 0;
 };
 // one ring per device, created on first use and kept until the process ends
 StagingRing &staging_ring(int device_idx) {
@@ -266,10 +282,34 @@ void HiddenStateHip::chunks_to_device(size_t n) {
     jcb_ones = false;
 }
 void HiddenStateHip::to_host() { this->to_host(this->size); }
+// grow-only pinned buffer per device that tagi_download_outputs writes into
+static float *download_buffer(size_t floats, int device_idx) {
+    static float *buf[16] = {};
+    static size_t cap[16] = {};
+    if (device_idx < 0 || device_idx >= 16) LOG(LogLevel::ERROR, "Invalid device index");
+    if (cap[device_idx] < floats) {
+        if (buf[device_idx] != nullptr) HIP_OK(hipHostFree(buf[device_idx]));
+        cap[device_idx] = std::max(floats, (size_t)1 << 14);
+        HIP_OK(hipHostMalloc(reinterpret_cast<void **>(&buf[device_idx]),
+                             cap[device_idx] * sizeof(float), hipHostMallocDefault));
+    }
+    return buf[device_idx];
+}
+
 void HiddenStateHip::to_host(size_t n) {
     n = std::min(n, this->size);
-    d2h(mu_a.data(), d_mu_a, n);
-    d2h(var_a.data(), d_var_a, n);
+    if (n > 0 && n * sizeof(float) <= kKernelUploadMaxBytes) {
+        // small results: one kernel writes both arrays into pinned memory, one wait
+        HIP_OK(hipSetDevice(device_idx));
+        float *host = download_buffer(2 * n, device_idx);
+        TAGI_OK_OR_THROW(tagi_download_outputs(d_mu_a, d_var_a, n, host, host + n, host_stream()));
+        HIP_OK(hipStreamSynchronize(host_stream()));
+        std::memcpy(mu_a.data(), host, n * sizeof(float));
+        std::memcpy(var_a.data(), host + n, n * sizeof(float));
+    } else {
+        d2h(mu_a.data(), d_mu_a, n);
+        d2h(var_a.data(), d_var_a, n);
+    }
     if (jcb_ones)
         std::fill(jcb.begin(), jcb.begin() + n, 1.0f);
     else
@@ -296,11 +336,22 @@ void HiddenStateHip::set_input_raw(const float *mu_x, const float *var_x, size_t
     this->block_size = new_block_size;
     HIP_OK(hipSetDevice(device_idx));
     StagingRing &ring = staging_ring(device_idx);
-    ring.upload(d_mu_a, mu_x, n * sizeof(float));
-    if (var_x != nullptr)
-        ring.upload(d_var_a, var_x, n * sizeof(float));
-    else
-        HIP_OK(hipMemsetAsync(d_var_a, 0, n * sizeof(float), host_stream()));
+    if (n * sizeof(float) <= kKernelUploadMaxBytes) {
+        // small batches: one kernel reads the pinned copy over the bus and fills both arrays
+        // (a copy-engine transfer costs a short dependent chain more than it carries)
+        const void *parts[2] = {mu_x, var_x};
+        const size_t sizes[2] = {n * sizeof(float), var_x != nullptr ? n * sizeof(float) : 0};
+        const float *host = static_cast<const float *>(ring.stage(parts, sizes, 2));
+        TAGI_OK_OR_THROW(tagi_upload_input(host, var_x != nullptr ? host + n : nullptr, n, d_mu_a,
+                                           d_var_a, host_stream()));
+        ring.staged_work_queued();
+    } else {
+        ring.upload(d_mu_a, mu_x, n * sizeof(float));
+        if (var_x != nullptr)
+            ring.upload(d_var_a, var_x, n * sizeof(float));
+        else
+            HIP_OK(hipMemsetAsync(d_var_a, 0, n * sizeof(float), host_stream()));
+    }
     jcb_ones = true;  // the input's Jacobian is one: marked, not written
 }
 void HiddenStateHip::set_size(size_t new_size, size_t new_block_size) {
@@ -510,6 +561,17 @@ void ObservationHip::upload(const float *mu, const float *var, size_t n, const i
         if (ni) ring.upload(d_selected_idx, idx, ni * sizeof(int));
     }
 }
+void ObservationHip::stage(const float *mu, const float *var, size_t n, const int *idx,
+                           const float **mu_at, const float **var_at, const int **idx_at) {
+    HIP_OK(hipSetDevice(device_idx));
+    const void *parts[3] = {mu, var, idx};
+    const size_t sizes[3] = {n * sizeof(float), n * sizeof(float), n * sizeof(int)};
+    char *host = static_cast<char *>(staging_ring(device_idx).stage(parts, sizes, 3));
+    *mu_at = reinterpret_cast<const float *>(host);
+    *var_at = reinterpret_cast<const float *>(host + sizes[0]);
+    *idx_at = reinterpret_cast<const int *>(host + sizes[0] + sizes[1]);
+}
+void ObservationHip::staged_work_queued() { staging_ring(device_idx).staged_work_queued(); }
 void ObservationHip::to_device() {
     this->upload(mu_obs.data(), var_obs.data(), mu_obs.size(), selected_idx.data(),
                  selected_idx.size());

@@ -203,6 +203,12 @@ class ObservationHip : public BaseObservation {
     // Same, straight from caller memory (no host mirror is kept): n observations and
     // variances, n_idx selected indices (idx may be null with n_idx = 0).
     void upload(const float *mu, const float *var, size_t n, const int *idx, size_t n_idx);
+    // Copies the three arrays into pinned host memory that kernels can read and returns
+    // where they lie; the caller queues the kernel that reads them on host_stream() and
+    // then calls staged_work_queued(). The device arrays above are not touched.
+    void stage(const float *mu, const float *var, size_t n, const int *idx, const float **mu_at,
+               const float **var_at, const int **idx_at);
+    void staged_work_queued();
    private:
     void reserve(size_t n, size_t n_idx);
 };

@@ -287,6 +287,20 @@ int tagi_out_update_indexed(const float *mu_a, const float *var_a,
                             int n_obs, int n_enc, int n, float *delta_mu,
                             float *delta_var, void *stream);
 
+/* The same with the clearing of the innovation buffers included (one launch for
+ * DeltaStateCuda::reset_zeros, src/data_struct_cuda.cu:262-275, and the update as
+ * OutputUpdater::update_using_indices runs them, src/base_output_updater.cpp:178-205):
+ * delta_mu / delta_var [0 .. delta_len) end up zero except at the selected entries.
+ * obs, var_obs and selected_idx may point to pinned host memory (each value is read
+ * once), which saves the transfer of the observations. n must be a multiple of n_enc
+ * and (n / n_enc) * n_obs <= delta_len. */
+int tagi_out_update_indexed_reset(const float *mu_a, const float *var_a,
+                                  const float *jcb, const float *obs /* device or pinned host */,
+                                  const float *var_obs /* device or pinned host */,
+                                  const int *selected_idx /* device or pinned host */,
+                                  int n_obs, int n_enc, int n, float *delta_mu,
+                                  float *delta_var, size_t delta_len, void *stream);
+
 /* Output layer with a learned (heteroscedastic) error variance: the 2n output
  * units are pairs, unit 2i the mean output and unit 2i+1 the expected squared error,
  * and obs holds n observations. Unit 2i is updated as in the dense form with the
@@ -299,6 +313,23 @@ int tagi_out_update_heteros(const float *mu_a, const float *var_a,
                             float *delta_mu, float *delta_var, void *stream);
 
 /* ---- ReLU -------------------------------------------------------------------- */
+
+/* A batch of inputs from PINNED host memory (hipHostMalloc) into a state buffer: mu_a
+ * <- host_mu, var_a <- host_var, or zeros when host_var is NULL; n values each. The
+ * kernel reads the host arrays over the bus itself, so the transfer is one launch on
+ * the compute queue; replaces the transfers of HiddenStateCuda::set_input_x +
+ * chunks_to_device (src/data_struct_cuda.cu:58-80, 112-123). The host arrays must stay
+ * untouched until the launch has run (record an event on `stream` after the call). */
+int tagi_upload_input(const float *host_mu /* pinned host */,
+                      const float *host_var /* pinned host, may be NULL */, size_t n,
+                      float *mu_a, float *var_a, void *stream);
+/* The way back: host_mu / host_var (PINNED host memory) <- the first n entries of mu_a /
+ * var_a, written by the kernel itself; valid once `stream` has been synchronised.
+ * Replaces the two transfers of HiddenStateCuda::to_host as Sequential::get_outputs /
+ * output_to_host use it (src/data_struct_cuda.cu:82-110, src/sequential.cpp:470-497). */
+int tagi_download_outputs(const float *mu_a, const float *var_a, size_t n,
+                          float *host_mu /* pinned host */, float *host_var /* pinned host */,
+                          void *stream);
 
 /* mu_a = max(mu_z, 0); jcb, var_a = (0, 0) where that is 0, else (1, var_z);
  * replaces relu_mean_var_cuda (src/activation_cuda.cu), CPU form

@@ -23,7 +23,11 @@ extern "C" {
  * backward on the streaming kernel too), "linear.gemv16.fwd_lines" (1: the 9..16-sample
  * forward that loads whole cache lines and transposes them in LDS), "linear.dw_side" (0: bias innovations and
  * the state-backward fold as launches of their own instead of inside the
- * weight-backward launch), "linear.double_buffer". Conv2d: "conv2d.tile",
+ * weight-backward launch), "linear.double_buffer", "linear.stream_min_weights" (the
+ * smallest weight matrix, in elements, that goes to the streaming kernels; 0 sends every
+ * layer whose batch fits there, < 0 restores the measured thresholds; any value >= 0 also
+ * keeps small layers off their one-launch forward kernel), "linear.small" (0: no
+ * one-launch forward for small layers). Conv2d: "conv2d.tile",
  * "conv2d.splits", "conv2d.dw.tile", "conv2d.dw.splits", "conv2d.group_loads",
  * "conv2d.stencil", "conv2d.phase_order" (0 switches the named path off). */
 int tagi_hip_tune(const char *key /* host */, int value);

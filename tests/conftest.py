@@ -24,3 +24,19 @@ def ref_lib():
     not built (the GPU box has no reference tree)."""
     import oracle
     return oracle.load_ref()
+
+
+@pytest.fixture(params=["by_size", "streaming", "tiled"])
+def linear_kernel_choice(request):
+    """A Linear layer goes to the one-launch kernel for small layers, to the streaming
+    kernels (up to 32 samples) or to the tiled kernel depending on the size of its
+    weight matrix. "by_size" leaves that choice as shipped; "streaming" sends every
+    layer whose batch fits to the streaming kernels and "tiled" every layer to the
+    tiled kernel, so that the small test shapes reach each of them."""
+    from cutagi_amd import capi
+    if request.param == "streaming":
+        capi.tune("linear.stream_min_weights", 0)
+    elif request.param == "tiled":
+        capi.tune("linear.stream_min_weights", 2 ** 31 - 1)
+    yield request.param
+    capi.tune("linear.stream_min_weights", -1)

@@ -41,7 +41,7 @@ def _activate(oracle_lib, name, mu, var):
 @pytest.mark.parametrize("K,N,B", LINEAR)
 @pytest.mark.parametrize("act", ["relu", "mixture_relu"])
 @pytest.mark.parametrize("bias", [True, False])
-def test_linear_forward_with_activation(oracle_lib, K, N, B, act, bias):
+def test_linear_forward_with_activation(oracle_lib, linear_kernel_choice, K, N, B, act, bias):
     import cutagi_amd.functional as F
     d = linear_inputs(K, N, B, seed=3 * K + N + B, bias=bias)
     t = _dev(d)

@@ -29,7 +29,7 @@ def _dev(d):
 
 @pytest.mark.parametrize("K,N,B", SHAPES)
 @pytest.mark.parametrize("bias", [True, False])
-def test_linear_forward(oracle_lib, K, N, B, bias):
+def test_linear_forward(oracle_lib, linear_kernel_choice, K, N, B, bias):
     import cutagi_amd.functional as F
     d = linear_inputs(K, N, B, seed=K + N + B, bias=bias)
     t = _dev(d)
@@ -42,7 +42,7 @@ def test_linear_forward(oracle_lib, K, N, B, bias):
 
 
 @pytest.mark.parametrize("K,N,B", SHAPES)
-def test_linear_backward(oracle_lib, K, N, B):
+def test_linear_backward(oracle_lib, linear_kernel_choice, K, N, B):
     import cutagi_amd.functional as F
     d = linear_inputs(K, N, B, seed=7 * K + N + B, bias=True, jcb_random=True)
     t = _dev(d)
@@ -176,6 +176,7 @@ def test_both_forward_kernels_for_9_to_16_samples(oracle_lib, K, N, B):
     ref = oracle_lib.linear_fwd(d["mu_w"], d["var_w"], d["mu_b"], d["var_b"], d["mu_a"],
                                 d["var_a"], threads=4)
     got = {}
+    capi.tune("linear.stream_min_weights", 0)     # these shapes are small: force the kernels
     try:
         for lines in (1, 0):
             capi.tune("linear.gemv16.fwd_lines", lines)
@@ -185,6 +186,7 @@ def test_both_forward_kernels_for_9_to_16_samples(oracle_lib, K, N, B):
             assert_close(got[lines][1], ref[1], "var_z (lines=%d)" % lines, same_sign=True)
     finally:
         capi.tune("linear.gemv16.fwd_lines", -1)
+        capi.tune("linear.stream_min_weights", -1)
 
 
 @pytest.mark.parametrize("K,N,B", [(1024, 512, 32), (1536, 260, 24), (516, 300, 31)])
@@ -197,12 +199,14 @@ def test_state_backward_streaming_kernel_for_17_to_32_samples(oracle_lib, K, N, 
     t = _dev(d)
     ref = oracle_lib.linear_bwd_dz(d["mu_w"], d["jcb"], d["delta_mu"], d["delta_var"], threads=4)
     capi.tune("linear.gemv32", 2)
+    capi.tune("linear.stream_min_weights", 0)
     try:
         dz = F.linear_bwd_dz(t["mu_w"], t["jcb"], t["delta_mu"], t["delta_var"])
         out = F.linear_bwd(t["mu_w"], t["var_w"], t["var_b"], t["mu_a"], t["jcb"], t["delta_mu"],
                            t["delta_var"])
     finally:
         capi.tune("linear.gemv32", -1)
+        capi.tune("linear.stream_min_weights", -1)
     for got in (dz, out[:2]):
         assert_close(got[0].cpu().numpy(), ref[0], "delta_mu_z")
         assert_close(got[1].cpu().numpy(), ref[1], "delta_var_z", same_sign=True)

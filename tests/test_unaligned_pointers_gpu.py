@@ -53,7 +53,7 @@ LINEAR = [(512, 384, 256), (1024, 256, 8), (1024, 512, 12), (128, 128, 32), (204
 
 
 @pytest.mark.parametrize("K,N,B", LINEAR)
-def test_linear_entry_points_with_offset_pointers(oracle_lib, K, N, B):
+def test_linear_entry_points_with_offset_pointers(oracle_lib, linear_kernel_choice, K, N, B):
     import torch
     from cutagi_amd import capi
     assert K % 4 == 0 and N % 4 == 0

@@ -50,7 +50,7 @@ SEQUENCES = [
 
 
 @pytest.mark.parametrize("first,second", SEQUENCES)
-def test_static_forward_matches_regular_forward(oracle_lib, first, second):
+def test_static_forward_matches_regular_forward(oracle_lib, linear_kernel_choice, first, second):
     for i, (K, N, B) in enumerate((first, second)):
         d = linear_inputs(K, N, B, seed=11 * K + N + B, bias=(i == 0))
         (mu_s, var_s), (mu_r, var_r) = _both(d)
