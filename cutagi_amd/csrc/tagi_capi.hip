@@ -21,7 +21,7 @@ static __device__ __align__(256) float scratch[STATIC_SCRATCH_BYTES / sizeof(flo
 
 namespace {
 
-constexpr int ABI_VERSION = 103;
+constexpr int ABI_VERSION = 104;
 
 #define TAGI_TRY(expr)                          \
     do {                                        \
@@ -182,6 +182,9 @@ bool streams_weights(StreamOp op, int n, int k, int batch) {
     if (op == STREAM_FWD) return weights >= (batch <= 8 ? 8 * M : batch <= 16 ? 2 * M : 8 * M);
     return weights >= (batch <= 8 ? 4 * M : 2 * M);
 }
+
+// the one-launch kernels for small layers, unless a test forces another path
+bool use_small_kernels() { return g_tune.small != 0 && g_tune.stream_min_weights < 0; }
 
 // Tile shape and reduction slices of a tiled launch.
 void plan_gemm(GemmMode mode, GemmParams &p, int forced_splits, int *tile_out) {
@@ -357,7 +360,7 @@ static int linear_fwd_impl(const float *mu_w, const float *var_w, const float *m
     const bool vec = (K % 4 == 0) && aligned16(mu_w) && aligned16(var_w) && aligned16(mu_a) &&
                      aligned16(var_a);
 
-    if (vec && g_tune.small != 0 && g_tune.stream_min_weights < 0 && small_fwd_supported(K, N, B)) {
+    if (vec && use_small_kernels() && small_fwd_supported(K, N, B)) {
         // small layers: one launch, bias and activation included
         TAGI_TRY(launch_small_fwd(mu_w, var_w, e0, e1, mu_a, var_a, K, N, B, act, mu_z, var_z, jcb,
                                   stream));
@@ -461,6 +464,11 @@ static int linear_bwd_dz_impl(const float *mu_w, const float *jcb, const float *
 
     const bool wide16 = B > 8 && B <= (g_tune.wide32 == 2 ? wide_max_batch() : gemv_max_batch()) &&
                         g_tune.gemv16 != 0;
+    if (use_small_kernels() && K % 4 == 0 && aligned16(mu_w) && small_bwd_supported(K, N, B)) {
+        TAGI_TRY(launch_small_dz(mu_w, jcb, delta_mu, delta_var, K, N, B, delta_mu_z, delta_var_z,
+                                 stream));
+        return TAGI_OK;
+    }
     if ((B <= gemv_max_batch() || wide16) && vec && streams_weights(STREAM_DZ, N, K, B)) {
         const int blocks = ceil_div(K, wide16 ? gemv16_dz_cols_per_block() : gemv_dz_cols_per_block());
         const int step = wide16 ? gemv16_dz_n_step() : gemv_dz_n_step();
@@ -522,6 +530,12 @@ static int linear_bwd_dw_impl(const float *var_w, const float *mu_a, const float
     const bool k_vec = (K % 4 == 0) && aligned16(mu_a) && aligned16(var_w) &&
                        aligned16(delta_mu_w) && aligned16(delta_var_w);
 
+    if (use_small_kernels() && k_vec && fold == nullptr && small_dw_supported(K, N, B)) {
+        TAGI_TRY(launch_small_dw(var_w, mu_a, delta_mu, delta_var, K, N, B, delta_mu_w, delta_var_w,
+                                 var_b, delta_mu_b, delta_var_b, stream));
+        if (bias_done) *bias_done = var_b != nullptr;
+        return TAGI_OK;
+    }
     if (B <= gemv_max_batch() && k_vec) {
         TAGI_TRY(launch_gemv_dw(var_w, mu_a, delta_mu, delta_var, K, N, B,
                                 ((g_tune.gemv_rev >= 0 ? g_tune.gemv_rev : 0) >> 2) & 3,
@@ -958,9 +972,12 @@ int tagi_upload_input(const float *host_mu, const float *host_var, size_t n, flo
 }
 
 int tagi_download_outputs(const float *mu_a, const float *var_a, size_t n, float *host_mu,
-                          float *host_var, void *stream_) {
+                          float *host_var, unsigned *host_flag, unsigned flag_value,
+                          void *stream_) {
     if (n > 0 && (!mu_a || !var_a || !host_mu || !host_var)) return TAGI_ERR_INVALID_ARG;
-    TAGI_TRY(launch_download_outputs(mu_a, var_a, n, host_mu, host_var,
+    // with a flag the copy is one workgroup's loop: meant for outputs, not for whole buffers
+    if (host_flag != nullptr && n > ((size_t)1 << 20)) return TAGI_ERR_UNSUPPORTED;
+    TAGI_TRY(launch_download_outputs(mu_a, var_a, n, host_mu, host_var, host_flag, flag_value,
                                      static_cast<hipStream_t>(stream_)));
     return TAGI_OK;
 }

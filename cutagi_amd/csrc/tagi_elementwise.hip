@@ -76,14 +76,25 @@ __global__ __launch_bounds__(TPB) void upload_input_kernel(const float *__restri
 // The other direction: the first n means and variances of a state buffer written
 // straight into pinned host memory by the kernel (one launch and one wait for the
 // stream instead of two synchronous copies).
+// With host_flag given the launch is one workgroup, which writes flag_value there after
+// all of the data (release at system scope): a host thread that polls the flag sees the
+// data complete without waiting for the stream through the runtime.
 __global__ __launch_bounds__(TPB) void download_outputs_kernel(const float *__restrict__ mu_a,
                                                                const float *__restrict__ var_a,
                                                                size_t n, float *__restrict__ host_mu,
-                                                               float *__restrict__ host_var) {
+                                                               float *__restrict__ host_var,
+                                                               unsigned *host_flag,
+                                                               unsigned flag_value) {
     const size_t stride = (size_t)gridDim.x * TPB;
     for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += stride) {
         host_mu[i] = mu_a[i];
         host_var[i] = var_a[i];
+    }
+    if (host_flag != nullptr) {
+        __threadfence_system();
+        __syncthreads();
+        if (threadIdx.x == 0)
+            __hip_atomic_store(host_flag, flag_value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
     }
 }
 
@@ -445,11 +456,13 @@ hipError_t launch_upload_input(const float *host_mu, const float *host_var, size
 }
 
 hipError_t launch_download_outputs(const float *mu_a, const float *var_a, size_t n, float *host_mu,
-                                   float *host_var, hipStream_t stream) {
-    if (n == 0) return hipSuccess;
-    const unsigned blocks = blocks_for(n, TPB) < 1024u ? blocks_for(n, TPB) : 1024u;
+                                   float *host_var, unsigned *host_flag, unsigned flag_value,
+                                   hipStream_t stream) {
+    if (n == 0 && host_flag == nullptr) return hipSuccess;
+    unsigned blocks = blocks_for(n, TPB) < 1024u ? blocks_for(n, TPB) : 1024u;
+    if (host_flag != nullptr || blocks == 0) blocks = 1;   // the flag follows one workgroup's data
     hipLaunchKernelGGL(download_outputs_kernel, dim3(blocks), dim3(TPB), 0, stream, mu_a, var_a, n,
-                       host_mu, host_var);
+                       host_mu, host_var, host_flag, flag_value);
     return hipGetLastError();
 }
 

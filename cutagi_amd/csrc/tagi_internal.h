@@ -103,6 +103,16 @@ hipError_t launch_small_fwd(const float *mu_w, const float *var_w, const float *
                             int N, int B, int act, float *out0, float *out1, float *out2,
                             hipStream_t stream);
 
+// State and weight backward of the same layers, one launch each; the weight backward
+// also writes the bias innovations when var_b is given.
+bool small_bwd_supported(int K, int N, int B);
+bool small_dw_supported(int K, int N, int B);
+hipError_t launch_small_dz(const float *mu_w, const float *jcb, const float *dmu, const float *dvar,
+                           int K, int N, int B, float *out_mu, float *out_var, hipStream_t stream);
+hipError_t launch_small_dw(const float *var_w, const float *mu_a, const float *dmu,
+                           const float *dvar, int K, int N, int B, float *dmu_w, float *dvar_w,
+                           const float *var_b, float *dmu_b, float *dvar_b, hipStream_t stream);
+
 // Skinny-batch (B <= 16) streaming kernels: weights are read once from HBM
 // straight into MFMA operand layout, nothing is staged in LDS.
 hipError_t launch_gemv_fwd(const float *mu_w, const float *var_w, const float *mu_a,
@@ -197,7 +207,8 @@ hipError_t launch_out_update_indexed_reset(const float *mu_a, const float *var_a
                                            int n_obs, int n_enc, int samples, float *dmu,
                                            float *dvar, size_t delta_len, hipStream_t stream);
 hipError_t launch_download_outputs(const float *mu_a, const float *var_a, size_t n, float *host_mu,
-                                   float *host_var, hipStream_t stream);
+                                   float *host_var, unsigned *host_flag, unsigned flag_value,
+                                   hipStream_t stream);
 hipError_t launch_upload_input(const float *host_mu, const float *host_var, size_t n, float *mu_a,
                                float *var_a, hipStream_t stream);
 

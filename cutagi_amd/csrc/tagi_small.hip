@@ -1,4 +1,4 @@
-// Forward of small Linear layers (reference: linear_fwd_mean_var,
+// Small Linear layers in one launch per pass. Forward (reference: linear_fwd_mean_var,
 // src/linear_layer.cpp:19-58; device form src/linear_layer_cuda.cu:27-125): the
 // layers of the MNIST-sized multilayer perceptrons, whose weight matrices fit the L2
 // cache many times over. Such a launch is bound by latency, not by throughput: the
@@ -11,6 +11,16 @@
 // the one store. For reductions longer than 256 the four waves of a workgroup share
 // one tile and each takes a quarter of every 1024 elements (784 inputs: still one
 // round of loads); their sums meet in 512 bytes of LDS. There is no second launch.
+// The code is kept short on purpose: a kernel this brief runs cold, and fetching its
+// instructions is part of its latency (the first version of the butterfly, compiled to
+// select chains, made the launch twice as long).
+//
+// The two backward kernels below follow the same rule - every load of a pass in flight
+// before the first use, no second launch: the state backward (linear_bwd_fc_delta_z,
+// src/linear_layer.cpp:180-219) splits the sum over the output units over eight slices
+// of a workgroup, and the weight backward (linear_bwd_fc_delta_w / _b,
+// src/linear_layer.cpp:221-327) needs no reduction across threads at all (the sum runs
+// over the batch) and writes the bias innovations on the side.
 #include <hip/hip_runtime.h>
 
 #include "tagi_activation.h"
@@ -172,6 +182,141 @@ __global__ __launch_bounds__(SMALL_WAVES * 64) void small_fwd_kernel(
         store_activated(act, mu, var, (size_t)out_b * N + out_n, out0, out1, out2);
 }
 
+// ---- state backward ---------------------------------------------------------------
+// delta_mu_z[b][k] = jcb[b][k] sum_n mu_w[n][k] delta_mu[b][n], delta_var_z with mu_w^2
+// and jcb^2. Workgroup = one sample x 128 input units (32 lanes of 16 bytes) x 8 slices
+// of the output units; slice s takes the units s, s + 8, ...
+constexpr int DZ_LANES = 32, DZ_SLICES = 8, DZ_BATCH = 16;
+
+__global__ __launch_bounds__(DZ_LANES * DZ_SLICES) void small_dz_kernel(
+    const float *__restrict__ mu_w, const float *__restrict__ jcb,
+    const float *__restrict__ dmu, const float *__restrict__ dvar, int K, int N,
+    float *__restrict__ out_mu, float *__restrict__ out_var) {
+    __shared__ float red[DZ_SLICES][DZ_LANES][8];
+    const int kl = threadIdx.x & (DZ_LANES - 1), slice = threadIdx.x / DZ_LANES;
+    const int k = (blockIdx.x * DZ_LANES + kl) * 4;
+    const int b = blockIdx.y;
+    const bool valid = k < K;
+    const float *w_col = mu_w + (valid ? k : 0);
+    const float *dm_row = dmu + (size_t)b * N, *dv_row = dvar + (size_t)b * N;
+    // after the sums: thread t folds entry t % 8 of lane t / 8 over the slices. Its
+    // Jacobian is asked for now, not in a memory round trip of its own at the end.
+    const int kl2 = threadIdx.x >> 3, c = threadIdx.x & 7;
+    const int k2 = (blockIdx.x * DZ_LANES + kl2) * 4 + (c & 3);
+    const size_t at = (size_t)b * K + min(k2, K - 1);
+    const float j = jcb[at];
+    float4 m = make_float4(0.f, 0.f, 0.f, 0.f), v = m;
+    for (int n0 = slice; n0 < N; n0 += DZ_SLICES * DZ_BATCH) {
+        float4 w[DZ_BATCH];
+        float d[DZ_BATCH], dv[DZ_BATCH];
+#pragma unroll
+        for (int u = 0; u < DZ_BATCH; u++) {
+            const int n = n0 + u * DZ_SLICES;
+            const int row = min(n, N - 1);          // rows past the end: read, weighted by zero
+            w[u] = *reinterpret_cast<const float4 *>(w_col + (size_t)row * K);
+            d[u] = dm_row[row];
+            dv[u] = dv_row[row];
+        }
+        __builtin_amdgcn_sched_barrier(0);          // all loads of the batch before any use
+#pragma unroll
+        for (int u = 0; u < DZ_BATCH; u++) {
+            if (n0 + u * DZ_SLICES >= N) d[u] = dv[u] = 0.f;
+            m.x += w[u].x * d[u]; m.y += w[u].y * d[u]; m.z += w[u].z * d[u]; m.w += w[u].w * d[u];
+            v.x += w[u].x * w[u].x * dv[u]; v.y += w[u].y * w[u].y * dv[u];
+            v.z += w[u].z * w[u].z * dv[u]; v.w += w[u].w * w[u].w * dv[u];
+        }
+    }
+    *reinterpret_cast<float4 *>(&red[slice][kl][0]) = m;
+    *reinterpret_cast<float4 *>(&red[slice][kl][4]) = v;
+    __syncthreads();
+    if (k2 >= K) return;
+    float sum = 0.f;
+#pragma unroll
+    for (int s2 = 0; s2 < DZ_SLICES; s2++) sum += red[s2][kl2][c];      // in slice order
+    if (c < 4)
+        out_mu[at] = sum * j;
+    else
+        out_var[at] = sum * j * j;
+}
+
+// ---- weight backward ----------------------------------------------------------------
+// delta_mu_w[n][k] = var_w[n][k] sum_b mu_a[b][k] delta_mu[b][n], delta_var_w with
+// var_w^2, mu_a^2 and delta_var; thread = DW_ROWS output units x 4 input units, DW_BATCH
+// samples per round of loads (2 x 16 up to 16 samples, 1 x 32 beyond). The
+// thread of a row's first input units also has that row's sum of delta over the batch:
+// the bias innovations (x var_b, x var_b^2).
+constexpr int DW_TPB = 256;
+
+template <int DW_ROWS, int DW_BATCH>
+__global__ __launch_bounds__(DW_TPB) void small_dw_kernel(
+    const float *__restrict__ var_w, const float *__restrict__ mu_a,
+    const float *__restrict__ dmu, const float *__restrict__ dvar, int K, int N, int B,
+    float *__restrict__ dmu_w, float *__restrict__ dvar_w, const float *__restrict__ var_b,
+    float *__restrict__ dmu_b, float *__restrict__ dvar_b) {
+    const int K4 = K >> 2;
+    const int item = blockIdx.x * DW_TPB + threadIdx.x;
+    if (item >= ((N + DW_ROWS - 1) / DW_ROWS) * K4) return;
+    const int n0 = (item / K4) * DW_ROWS, k = (item % K4) * 4;
+    int row[DW_ROWS];
+    float4 vw[DW_ROWS], am[DW_ROWS], av[DW_ROWS];
+    float bm[DW_ROWS], bv[DW_ROWS];
+#pragma unroll
+    for (int r = 0; r < DW_ROWS; r++) {
+        row[r] = min(n0 + r, N - 1);
+        vw[r] = *reinterpret_cast<const float4 *>(var_w + (size_t)row[r] * K + k);
+        am[r] = av[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+        bm[r] = bv[r] = 0.f;
+    }
+    for (int b0 = 0; b0 < B; b0 += DW_BATCH) {
+        float4 a[DW_BATCH];
+        float d[DW_BATCH][DW_ROWS], dv[DW_BATCH][DW_ROWS];
+#pragma unroll
+        for (int u = 0; u < DW_BATCH; u++) {
+            const int b = min(b0 + u, B - 1);       // samples past the end: weighted by zero
+            a[u] = *reinterpret_cast<const float4 *>(mu_a + (size_t)b * K + k);
+#pragma unroll
+            for (int r = 0; r < DW_ROWS; r++) {
+                d[u][r] = dmu[(size_t)b * N + row[r]];
+                dv[u][r] = dvar[(size_t)b * N + row[r]];
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);          // all loads of the batch before any use
+#pragma unroll
+        for (int u = 0; u < DW_BATCH; u++) {
+            if (b0 + u >= B) {
+#pragma unroll
+                for (int r = 0; r < DW_ROWS; r++) d[u][r] = dv[u][r] = 0.f;
+            }
+            const float4 sq = make_float4(a[u].x * a[u].x, a[u].y * a[u].y, a[u].z * a[u].z,
+                                          a[u].w * a[u].w);
+#pragma unroll
+            for (int r = 0; r < DW_ROWS; r++) {
+                am[r].x += a[u].x * d[u][r]; am[r].y += a[u].y * d[u][r];
+                am[r].z += a[u].z * d[u][r]; am[r].w += a[u].w * d[u][r];
+                av[r].x += sq.x * dv[u][r]; av[r].y += sq.y * dv[u][r];
+                av[r].z += sq.z * dv[u][r]; av[r].w += sq.w * dv[u][r];
+                bm[r] += d[u][r];
+                bv[r] += dv[u][r];
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < DW_ROWS; r++) {
+        if (n0 + r >= N) break;
+        const size_t at = (size_t)row[r] * K + k;
+        *reinterpret_cast<float4 *>(dmu_w + at) =
+            make_float4(am[r].x * vw[r].x, am[r].y * vw[r].y, am[r].z * vw[r].z, am[r].w * vw[r].w);
+        *reinterpret_cast<float4 *>(dvar_w + at) =
+            make_float4(av[r].x * vw[r].x * vw[r].x, av[r].y * vw[r].y * vw[r].y,
+                        av[r].z * vw[r].z * vw[r].z, av[r].w * vw[r].w * vw[r].w);
+        if (k == 0 && var_b != nullptr) {
+            const float vb = var_b[row[r]];
+            dmu_b[row[r]] = bm[r] * vb;
+            dvar_b[row[r]] = bv[r] * vb * vb;
+        }
+    }
+}
+
 }  // namespace
 
 // Layers this kernel is meant for: up to 64 samples and up to 2^18 weights (512^2),
@@ -197,6 +342,44 @@ hipError_t launch_small_fwd(const float *mu_w, const float *var_w, const float *
     else
         hipLaunchKernelGGL((small_fwd_kernel<RN, RB, SMALL_WAVES>), dim3(tiles), block, 0, stream,
                            mu_w, var_w, mu_b, var_b, mu_a, var_a, K, N, B, act, out0, out1, out2);
+    return hipGetLastError();
+}
+
+// The backward kernels: the same layers (K % 4 == 0; mu_w / var_w / mu_a and the weight
+// innovations 16-byte aligned, which the caller checks).
+bool small_bwd_supported(int K, int N, int B) { return small_fwd_supported(K, N, B); }
+// The weight backward: 9..32 samples (up to 8 the streaming kernel is quicker, beyond 32
+// the tiled one).
+bool small_dw_supported(int K, int N, int B) {
+    return B > 8 && B <= 32 && small_bwd_supported(K, N, B);
+}
+
+hipError_t launch_small_dz(const float *mu_w, const float *jcb, const float *dmu, const float *dvar,
+                           int K, int N, int B, float *out_mu, float *out_var,
+                           hipStream_t stream) {
+    if (K % 4 != 0 || K <= 0 || N <= 0 || B <= 0 || B > 65535) return hipErrorInvalidValue;
+    dim3 grid(((K >> 2) + DZ_LANES - 1) / DZ_LANES, B), block(DZ_LANES * DZ_SLICES);
+    hipLaunchKernelGGL(small_dz_kernel, grid, block, 0, stream, mu_w, jcb, dmu, dvar, K, N, out_mu,
+                       out_var);
+    return hipGetLastError();
+}
+
+// var_b null: no bias innovations (dmu_b / dvar_b unused).
+hipError_t launch_small_dw(const float *var_w, const float *mu_a, const float *dmu,
+                           const float *dvar, int K, int N, int B, float *dmu_w, float *dvar_w,
+                           const float *var_b, float *dmu_b, float *dvar_b, hipStream_t stream) {
+    if (K % 4 != 0 || K <= 0 || N <= 0 || B <= 0) return hipErrorInvalidValue;
+    if (B <= 16) {
+        const int items = ((N + 1) / 2) * (K >> 2);
+        hipLaunchKernelGGL((small_dw_kernel<2, 16>), dim3((items + DW_TPB - 1) / DW_TPB), dim3(DW_TPB),
+                           0, stream, var_w, mu_a, dmu, dvar, K, N, B, dmu_w, dvar_w, var_b, dmu_b,
+                           dvar_b);
+    } else {
+        const int items = N * (K >> 2);
+        hipLaunchKernelGGL((small_dw_kernel<1, 32>), dim3((items + DW_TPB - 1) / DW_TPB), dim3(DW_TPB),
+                           0, stream, var_w, mu_a, dmu, dvar, K, N, B, dmu_w, dvar_w, var_b, dmu_b,
+                           dvar_b);
+    }
     return hipGetLastError();
 }
 

@@ -10,6 +10,8 @@
 #include "../../include/tagi_hip.h"
 
 #include <algorithm>
+#include <atomic>
+#include <chrono>
 #include <cstring>
 
 #include "logger.h"
@@ -292,6 +294,7 @@ static float *download_buffer(size_t floats, int device_idx) {
         cap[device_idx] = std::max(floats, (size_t)1 << 14);
         HIP_OK(hipHostMalloc(reinterpret_cast<void **>(&buf[device_idx]),
                              cap[device_idx] * sizeof(float), hipHostMallocDefault));
+        std::memset(buf[device_idx], 0, 64);      // the completion flag starts cleared
     }
     return buf[device_idx];
 }
@@ -301,9 +304,31 @@ void HiddenStateHip::to_host(size_t n) {
     if (n > 0 && n * sizeof(float) <= kKernelUploadMaxBytes) {
         // small results: one kernel writes both arrays into pinned memory, one wait
         HIP_OK(hipSetDevice(device_idx));
-        float *host = download_buffer(2 * n, device_idx);
-        TAGI_OK_OR_THROW(tagi_download_outputs(d_mu_a, d_var_a, n, host, host + n, host_stream()));
-        HIP_OK(hipStreamSynchronize(host_stream()));
+        // [0]: the flag the kernel sets after the data (64 bytes to itself), then the data
+        float *buf = download_buffer(2 * n + 16, device_idx);
+        unsigned *flag = reinterpret_cast<unsigned *>(buf);
+        float *host = buf + 16;
+        static unsigned sequence = 0;
+        const unsigned expect = ++sequence == 0 ? ++sequence : sequence;   // never the initial 0
+        // (one workgroup copies when a flag is asked for: only for the sizes of outputs)
+        const bool poll = n <= 16384;
+        TAGI_OK_OR_THROW(tagi_download_outputs(d_mu_a, d_var_a, n, host, host + n,
+                                               poll ? flag : nullptr, expect, host_stream()));
+        if (!poll) HIP_OK(hipStreamSynchronize(host_stream()));
+        // Poll the flag: the data is a few hundred bytes behind kernels that take
+        // microseconds, and waking up through the runtime's stream wait costs more than
+        // the wait itself. Bounded: after 2 ms the ordinary wait takes over (which also
+        // reports a failed launch).
+        const auto t0 = std::chrono::steady_clock::now();
+        unsigned spins = 0;
+        while (poll && *static_cast<volatile unsigned *>(flag) != expect) {
+            if ((++spins & 1023u) == 0 &&
+                std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(2)) {
+                HIP_OK(hipStreamSynchronize(host_stream()));
+                break;
+            }
+        }
+        std::atomic_thread_fence(std::memory_order_acquire);
         std::memcpy(mu_a.data(), host, n * sizeof(float));
         std::memcpy(var_a.data(), host + n, n * sizeof(float));
     } else {

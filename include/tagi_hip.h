@@ -325,10 +325,16 @@ int tagi_upload_input(const float *host_mu /* pinned host */,
                       float *mu_a, float *var_a, void *stream);
 /* The way back: host_mu / host_var (PINNED host memory) <- the first n entries of mu_a /
  * var_a, written by the kernel itself; valid once `stream` has been synchronised.
+ * With host_flag (pinned host memory too, may be NULL) the kernel stores flag_value there
+ * after all of the data, with release order at system scope: a host thread that polls
+ * *host_flag until it reads flag_value (then an acquire fence) may read the data without
+ * synchronising the stream; use a value the flag does not hold yet. With a flag n is
+ * limited to 2^20 (TAGI_ERR_UNSUPPORTED beyond).
  * Replaces the two transfers of HiddenStateCuda::to_host as Sequential::get_outputs /
  * output_to_host use it (src/data_struct_cuda.cu:82-110, src/sequential.cpp:470-497). */
 int tagi_download_outputs(const float *mu_a, const float *var_a, size_t n,
                           float *host_mu /* pinned host */, float *host_var /* pinned host */,
+                          unsigned *host_flag /* pinned host or NULL */, unsigned flag_value,
                           void *stream);
 
 /* mu_a = max(mu_z, 0); jcb, var_a = (0, 0) where that is 0, else (1, var_z);

@@ -35,17 +35,30 @@ def test_upload_input_copies_means_and_variances(n, with_var):
 
 
 @pytest.mark.parametrize("n", SIZES)
-def test_download_outputs_writes_pinned_memory(n):
+@pytest.mark.parametrize("with_flag", [False, True])
+def test_download_outputs_writes_pinned_memory(n, with_flag):
     import torch
     from cutagi_amd import capi
     rng = np.random.default_rng(n + 1)
     mu = torch.from_numpy(rng.standard_normal(n + 3).astype(np.float32)).cuda()
     var = torch.from_numpy(rng.uniform(0, 1, n + 3).astype(np.float32)).cuda()
     host = torch.full((2 * n + 2,), -3.0).pin_memory()
+    flag = torch.zeros(16, dtype=torch.int32).pin_memory()
     stream = torch.cuda.current_stream().cuda_stream
     capi.check(capi.lib.tagi_download_outputs(capi.ptr(mu), capi.ptr(var), n, host.data_ptr(),
-                                              host.data_ptr() + 4 * n, stream))
-    torch.cuda.synchronize()
+                                              host.data_ptr() + 4 * n,
+                                              flag.data_ptr() if with_flag else None, 77, stream))
+    if with_flag:
+        # the flag is the completion signal: poll it (bounded), then read without a
+        # stream synchronisation
+        import time
+        t0 = time.time()
+        while int(flag[0]) != 77 and time.time() - t0 < 10.0:
+            pass
+        assert int(flag[0]) == 77
+    else:
+        torch.cuda.synchronize()
+        assert int(flag[0]) == 0
     assert torch.equal(host[:n], mu[:n].cpu())
     assert torch.equal(host[n:2 * n], var[:n].cpu())
     assert float(host[2 * n:].max()) == -3.0
@@ -58,9 +71,10 @@ def test_transfers_reject_null_pointers_and_accept_empty_batches():
     h = torch.zeros(8).pin_memory()
     assert capi.lib.tagi_upload_input(None, None, 8, capi.ptr(x), capi.ptr(x), None) == capi.ERR_INVALID_ARG
     assert capi.lib.tagi_upload_input(h.data_ptr(), None, 8, None, capi.ptr(x), None) == capi.ERR_INVALID_ARG
-    assert capi.lib.tagi_download_outputs(capi.ptr(x), capi.ptr(x), 8, None, h.data_ptr(), None) == capi.ERR_INVALID_ARG
+    assert capi.lib.tagi_download_outputs(capi.ptr(x), capi.ptr(x), 8, None, h.data_ptr(), None, 0, None) == capi.ERR_INVALID_ARG
+    assert capi.lib.tagi_download_outputs(capi.ptr(x), capi.ptr(x), (1 << 20) + 1, h.data_ptr(), h.data_ptr(), h.data_ptr(), 1, None) == capi.ERR_UNSUPPORTED
     assert capi.lib.tagi_upload_input(None, None, 0, None, None, None) == capi.OK
-    assert capi.lib.tagi_download_outputs(None, None, 0, None, None, None) == capi.OK
+    assert capi.lib.tagi_download_outputs(None, None, 0, None, None, None, 0, None) == capi.OK
     torch.cuda.synchronize()
 
 
