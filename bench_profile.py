@@ -10,6 +10,7 @@ of their own, one counter block per run):
     rocprofv3 --pmc WRITE_SIZE --output-format csv -d gpurun_out/pmc_write -o w -- python3 bench.py --no-cpu --extra linear,conv --calibrate --steps 10
     rocprofv3 --pmc SQ_INSTS_VALU_MFMA_MOPS_F32 SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CU_CYCLES SQ_WAVES SQ_WAVE_CYCLES SQ_WAIT_INST_ANY SQ_ACTIVE_INST_VMEM GRBM_GUI_ACTIVE --output-format csv -d gpurun_out/pmc_sq -o sq -- python3 bench.py --no-cpu --extra linear,conv --steps 10
     rocprofv3 --kernel-trace --stats --output-format csv -d gpurun_out/prof_resnet -o resnet -- python3 bench.py --no-cpu --extra resnet18
+    rocprofv3 --kernel-trace --stats --output-format csv -d gpurun_out/prof_mlp -o mlp -- python3 bench.py --no-cpu --extra mlp
 
 and then, anywhere the raw output and a git checkout are at hand,
 
@@ -262,6 +263,42 @@ def resnet(raw, out, stamp):
     print("wrote resnet18_cifar_step_kernel_stats.md")
 
 
+def mlp(raw, out, stamp):
+    tf = find(raw, "prof_mlp", "*kernel_trace.csv")
+    if not tf:
+        return
+    tr = sorted(csv.DictReader(open(tf)), key=lambda r: int(r["Start_Timestamp"]))
+    first = next(i for i, r in enumerate(tr) if "upload_input_kernel" in r["Kernel_Name"])
+    tr = tr[first:]
+    agg = collections.defaultdict(list)
+    order = []
+    for r in tr:
+        k = short(r["Kernel_Name"]) + " [grid %s]" % r.get("Grid_Size_X", r.get("Grid_Size", "?"))
+        if k not in agg:
+            order.append(k)
+        agg[k].append(int(r["End_Timestamp"]) - int(r["Start_Timestamp"]))
+    steps = len(next(v for k, v in agg.items() if k.startswith("out_update_indexed_reset_kernel")))
+    per_step = sum(sum(v) for v in agg.values() if len(v) >= steps // 2) / steps / 1e3
+    with open(os.path.join(out, "mlp_784_128_128_11_step_kernel_stats.md"), "w") as f:
+        f.write("# Kernels of one training step of the 784-128-128-11 perceptron (batch 32)\n\n"
+                "Library built from commit `%s`. Command (one MI355X, repository root):\n\n"
+                "    rocprofv3 --kernel-trace --stats --output-format csv -d gpurun_out/prof_mlp -o mlp -- python3 bench.py --no-cpu --extra mlp\n\n"
+                "Summary written by `python3 bench_profile.py` from `mlp_kernel_trace.csv`: the dispatches from the first input\n"
+                "upload on, %d training steps (warm-up and the HIP-graph replay leg of the same command included; both launch the\n"
+                "same kernels). One step = forward, outputs to the host, output update on 4 selected units per sample, backward,\n"
+                "parameter update: **%d launches, %.1f us of kernel time** (bench.py measures the wall time of the step, which adds\n"
+                "the gaps between dependent launches and the host's turn-around after it has read the outputs).\n\n"
+                "| kernel, in launch order | launches per step | avg us | min us |\n|---|---|---|---|\n"
+                % (stamp, steps, sum(1 for k in order if len(agg[k]) >= steps // 2 for _ in range(round(len(agg[k]) / steps))),
+                   per_step))
+        for k in order:
+            v = agg[k]
+            if len(v) < steps // 2:
+                continue
+            f.write("| `%s` | %.1f | %.1f | %.1f |\n" % (k[:110], len(v) / steps, sum(v) / len(v) / 1e3, min(v) / 1e3))
+    print("wrote mlp_784_128_128_11_step_kernel_stats.md")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--raw", default=os.path.join(ROOT, "gpurun_out"))
@@ -274,6 +311,7 @@ def main():
     traffic(args.raw, args.out, stamp)
     mfma(args.raw, args.out, stamp)
     resnet(args.raw, args.out, stamp)
+    mlp(args.raw, args.out, stamp)
 
 
 if __name__ == "__main__":
