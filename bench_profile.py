@@ -59,12 +59,32 @@ def commit_stamp(given):
         return "unknown"
 
 
-def pmc(path):
-    """Per kernel: average counter values and average duration (us) over its dispatches."""
+# bench.py runs its main workload (Linear 4096^2, batch 256) first and the batch-32 / 64
+# workloads of the same layer later on the same tile kernels: dispatches of a kernel that
+# belongs to the main workload count only up to the first skinny-batch kernel.
+MAIN_ENDS_AT = "gemv_fwd_kernel"
+
+
+def main_workload_only(rows, name_key):
+    """rows (dicts with Start_Timestamp) -> those that precede the first skinny-batch dispatch."""
+    rows = sorted(rows, key=lambda r: int(r["Start_Timestamp"]))
+    for i, r in enumerate(rows):
+        if short(r[name_key]).startswith(MAIN_ENDS_AT):
+            return rows[:i]
+    return rows
+
+
+def pmc(path, main_kernels=()):
+    """Per kernel: average counter values and average duration (us) over its dispatches
+    (for the kernels named in main_kernels: over those of the main workload)."""
     values = collections.defaultdict(lambda: collections.defaultdict(list))
     durations = collections.defaultdict(list)
-    for r in csv.DictReader(open(path)):
+    rows = list(csv.DictReader(open(path)))
+    main_ids = set(id(r) for r in main_workload_only(rows, "Kernel_Name"))
+    for r in rows:
         k = short(r["Kernel_Name"])
+        if k in main_kernels and id(r) not in main_ids:
+            continue
         values[k][r["Counter_Name"]].append(float(r["Counter_Value"]))
         durations[k].append(int(r["End_Timestamp"]) - int(r["Start_Timestamp"]))
     avg = {k: {c: sum(v) / len(v) for c, v in cs.items()} for k, cs in values.items()}
@@ -96,6 +116,7 @@ KERNELS = [
     ("conv_stencil_kernel<true, 32>", "Conv2d delta_z", 5 * CONV_ACT, 4.0 * 64 * 131072 * 576),
     ("conv_stencil_dw_kernel<32>", "Conv2d delta_w", 3 * CONV_ACT, 4.0 * 64 * 131072 * 576),
 ]
+MAIN_KERNELS = tuple(k for k, w, _, _ in KERNELS if "B=256" in w)
 # bench.py's table: (workload, phase) -> kernel
 TRAFFIC_KEYS = [
     (("gemm", "fwd"), KERNELS[0][0]), (("gemm", "bwd_dw"), KERNELS[3][0]), (("gemm", "bwd_dz"), KERNELS[1][0]),
@@ -111,6 +132,13 @@ def kernel_stats(raw, out, stamp):
         return
     rows = list(csv.DictReader(open(stats)))
     avg = {short(r["Name"]): float(r["AverageNs"]) / 1e3 for r in rows}
+    # the kernels of the main workload: their average over that workload's dispatches only
+    per_kernel = collections.defaultdict(list)
+    for r in main_workload_only(list(csv.DictReader(open(trace))), "Kernel_Name"):
+        per_kernel[short(r["Kernel_Name"])].append(int(r["End_Timestamp"]) - int(r["Start_Timestamp"]))
+    for k in MAIN_KERNELS:
+        if per_kernel.get(k):
+            avg[k] = sum(per_kernel[k]) / len(per_kernel[k]) / 1e3
     with open(os.path.join(out, "linear_and_conv2d_bench_kernel_stats.md"), "w") as f:
         f.write("# Kernel durations of the default bench.py run\n\n"
                 "Library built from commit `%s`. Workloads: Linear 4096->4096 batch 256, Linear 8192->8192 batch 8 (and 12, 16),\n"
@@ -125,7 +153,9 @@ def kernel_stats(raw, out, stamp):
             f.write("| `%s` | %s | %.1f | %.1f | %.1f | %s |\n" % (
                 short(r["Name"]), r["Calls"], float(r["AverageNs"]) / 1e3, float(r["MinNs"]) / 1e3,
                 float(r["MaxNs"]) / 1e3, r["Percentage"]))
-        f.write("\nWhich kernel belongs to which workload, with the algorithmic work per launch:\n\n"
+        f.write("\nWhich kernel belongs to which workload, with the algorithmic work per launch (the tile kernels of the batch-256\n"
+                "workload also run the batch-64 one later in the command, which is why their averages above are lower: the rows\n"
+                "below take the dispatches of the batch-256 workload only, i.e. those before the first skinny-batch kernel):\n\n"
                 "| kernel | workload | GFLOP | TFLOP/s at avg | %% of %.1f | MB (inputs + outputs) | GB/s at avg |\n"
                 "|---|---|---|---|---|---|---|\n" % PEAK_TFLOPS)
         for k, w, mb, fl in KERNELS:
@@ -137,7 +167,7 @@ def kernel_stats(raw, out, stamp):
                 "partial sums and bias innovations. The Linear 4096^2 batch 32 / 64 workloads (`extra.mid` of bench.py) run their\n"
                 "state and weight backward on the 32x128 / 64x128 tile kernels listed above under their own template arguments.\n")
         fk = KERNELS[0][0]
-        tr = sorted(csv.DictReader(open(trace)), key=lambda r: int(r["Start_Timestamp"]))
+        tr = main_workload_only(list(csv.DictReader(open(trace))), "Kernel_Name")
         folds = []
         for a, b in zip(tr, tr[1:]):
             if short(a["Kernel_Name"]) == fk and short(b["Kernel_Name"]).startswith("reduce_splits_kernel<0"):
@@ -154,8 +184,8 @@ def traffic(raw, out, stamp):
     ff, wf = find(raw, "pmc_fetch", "*counter_collection.csv"), find(raw, "pmc_write", "*counter_collection.csv")
     if not ff or not wf:
         return
-    fa, _ = pmc(ff)
-    wa, _ = pmc(wf)
+    fa, _ = pmc(ff, MAIN_KERNELS)
+    wa, _ = pmc(wf, MAIN_KERNELS)
     ck = [k for k in fa if "copyBuffer" in k][0]
     fs, ws = 1048576.0 / fa[ck]["FETCH_SIZE"], 1048576.0 / wa[ck]["WRITE_SIZE"]
     with open(os.path.join(out, "linear_and_conv2d_hbm_traffic_counters.md"), "w") as f:
@@ -195,7 +225,7 @@ def mfma(raw, out, stamp):
     sf = find(raw, "pmc_sq", "*counter_collection.csv")
     if not sf:
         return
-    sa, sd = pmc(sf)
+    sa, sd = pmc(sf, MAIN_KERNELS)
     with open(os.path.join(out, "linear_and_conv2d_mfma_utilisation_counters.md"), "w") as f:
         f.write("# MFMA utilisation counters, all bench.py kernels\n\n"
                 "Library built from commit `%s`. Command (one MI355X, repository root):\n\n"
