@@ -327,6 +327,7 @@ int tagi_hip_tune(const char *key, int value) {
     else if (!strcmp(key, "conv2d.group_loads")) g_conv2d_group_loads = value;
     else if (!strcmp(key, "conv2d.stencil")) g_conv2d_stencil = value;
     else if (!strcmp(key, "conv2d.phase_order")) g_conv2d_phase_order = value;
+    else if (!strcmp(key, "conv2d.s2_all")) g_conv2d_s2_all = value < 0 ? 1 : value;
     else if (!strcmp(key, "linear.tile")) g_tune.tile = value;
     else if (!strcmp(key, "linear.double_buffer")) g_gemm_double_buffer = value < 0 ? 1 : value;
     else if (!strcmp(key, "conv2d.dw.splits")) g_tune.conv_dw_splits = value;
@@ -740,6 +741,11 @@ static int conv2d_bwd_dz_impl(const float *mu_w, const float *jcb, const float *
         const int tiles = ceil_div(fi, gemm_tile_rows(tile)) * ceil_div(B * wihi, gemm_tile_cols(tile));
         if (tiles >= 2 * num_cu() && tiles < 4 * num_cu() && ki * ki * fo >= 3 * 8 * gemm_k_tile())
             splits = 3;
+    }
+    if (conv2d_bwd_dz_s2_all(mu_w, delta_mu_out, delta_var_out, B, fo, woho, wihi, fi, ki, nr)) {
+        // all four phases of a pixel block in one workgroup, one workgroup per CU
+        tile = 1;  // 64 x 128 (tile ids as in pick_tile)
+        splits = conv2d_bwd_dz_s2_all_splits(B, fo, woho, fi);
     }
     if (g_tune.conv_splits > 0) splits = g_tune.conv_splits;
     if (g_tune.conv_tile >= 0 && g_tune.conv_tile < gemm_tile_count()) tile = g_tune.conv_tile;

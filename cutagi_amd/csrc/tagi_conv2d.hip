@@ -756,21 +756,31 @@ inline int lcm_int(int a, int b) {
     return a / x * b;
 }
 
-// `stencil_s2`: output map width when the strided state-backward stencil kernel applies.
+// `s2_all`: output map width when the stride-2 state-backward stencil kernel applies.
 template <class P, bool DZ>
 hipError_t run_sliced(int tile, int splits, int stencil, float *ws0, float *ws1, ConvParams &p,
-                      hipStream_t stream, int stencil_s2 = 0) {
+                      hipStream_t stream, int s2_all = 0) {
     // the state backward re-states its slices per tile in whole output channels
-    const int unit = (stencil || stencil_s2) ? 288 : DZ ? lcm_int(KT, p.k2) : KT;
+    // (the stencil kernels: in whole groups of 32 channels)
+    const int unit = (stencil || s2_all) ? 32 * p.k2 : DZ ? lcm_int(KT, p.k2) : KT;
     const int per = ceil_div(ceil_div(p.R, splits), unit) * unit;
     p.splits = ceil_div(p.R, per);
     p.r_per_split = per;
     p.ws0 = ws0;
     p.ws1 = ws1;
-    hipError_t e = stencil_s2 ? launch_conv_stencil_s2_dz(stencil_s2, p, stream)
+    hipError_t e = s2_all     ? (p.k2 == 9 ? launch_conv_stencil_s2_all_dz<3>(s2_all, p, stream)
+                                           : launch_conv_stencil_s2_all_dz<2>(s2_all, p, stream))
                    : stencil  ? launch_conv_stencil<DZ>(stencil, p, stream)
                               : launch_tiles<P>(tile, p, stream);
     if (e != hipSuccess || p.splits == 1) return e;
+    if constexpr (DZ) {
+        // phase-ordered columns of a stride-2 layer: fold in the order of the output
+        const uintptr_t ptrs = reinterpret_cast<uintptr_t>(p.out0) | reinterpret_cast<uintptr_t>(p.out1) |
+                               reinterpret_cast<uintptr_t>(p.e0) | reinterpret_cast<uintptr_t>(p.res0) |
+                               reinterpret_cast<uintptr_t>(p.res1);
+        if (p.perm_s == 2 && p.perm_w % 2 == 0 && (ptrs & 7u) == 0 && g_conv2d_s2_all)
+            return launch_reduce_store_s2_pairs(p, stream);
+    }
     return launch_reduce_store<P>(p, stream);
 }
 }  // namespace
@@ -778,6 +788,28 @@ hipError_t run_sliced(int tile, int splits, int stencil, float *ws0, float *ws1,
 int g_conv2d_group_loads = 1;
 int g_conv2d_stencil = 1;
 int g_conv2d_phase_order = 1;
+int g_conv2d_s2_all = 1;
+
+// Output map width when the state backward of a stride-2 layer runs on the kernel that
+// keeps all four phases in one workgroup (3x3 with padding on the right and bottom, or
+// 2x2 without padding; the kernel verifies the tables), 0 otherwise.
+int conv2d_bwd_dz_s2_all(const float *mu_w, const float *dmu, const float *dvar, int B, int fo,
+                         int woho, int wihi, int fi, int ki, int nr) {
+    if (!g_conv2d_stencil || !g_conv2d_s2_all || !g_conv2d_phase_order) return 0;
+    if (!((ki == 3 && nr == 4) || (ki == 2 && nr == 1))) return 0;
+    if (wihi != 4 * woho || fo % 32 != 0 || fi % 64 != 0 || ((long long)B * woho) % 128 != 0 ||
+        !aligned16(mu_w) || !aligned16(dmu) || !aligned16(dvar))
+        return 0;
+    return s2_out_width(woho);
+}
+
+// Its reduction slices: one workgroup per CU is resident; whole groups of 32 channels.
+int conv2d_bwd_dz_s2_all_splits(int B, int fo, int woho, int fi) {
+    const int tiles = (fi / 64) * (int)((long long)B * woho / 128);
+    int s = tiles > 0 ? num_cu() / tiles : 1;
+    if (s > fo / 32) s = fo / 32;
+    return s < 1 ? 1 : s;
+}
 
 hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
                              const float *var_b, const float *mu_a, const float *var_a,
@@ -832,13 +864,11 @@ hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float
     if (g_conv2d_stencil && ki == 3 && nr == 9 && woho == wihi && fo % 8 == 0 && fi % 64 == 0 &&
         tile == TILE_64x128 && aligned16(mu_w) && aligned16(dmu) && aligned16(dvar))
         stencil = stencil_width(wihi);
-    // 3x3, stride 2, padding on the right and bottom (the kernel verifies the tables)
-    int stencil_s2 = 0;
-    if (g_conv2d_stencil && ki == 3 && nr == 4 && wihi == 4 * woho && p.perm_s == 2 &&
-        fo % 32 == 0 && fi % 64 == 0 && tile == TILE_64x128 && ((long long)B * woho) % 128 == 0 &&
-        aligned16(dmu) && aligned16(dvar))
-        stencil_s2 = s2_out_width(woho);
-    return run_sliced<ConvDzProblem, true>(tile, splits, stencil, ws0, ws1, p, stream, stencil_s2);
+    // stride 2, 3x3 with padding on the right and bottom or 2x2 (the kernel verifies the tables)
+    const int s2_all = (p.perm_s == 2 && tile == TILE_64x128)
+                           ? conv2d_bwd_dz_s2_all(mu_w, dmu, dvar, B, fo, woho, wihi, fi, ki, nr)
+                           : 0;
+    return run_sliced<ConvDzProblem, true>(tile, splits, stencil, ws0, ws1, p, stream, s2_all);
 }
 
 // Workgroups of the weight-backward kernel that one CU holds at a time.

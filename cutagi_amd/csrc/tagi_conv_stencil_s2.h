@@ -1,23 +1,17 @@
-// Regular-stencil kernels for the strided convolutions of a ResNet: 3x3 kernel,
-// stride 2, one pixel of padding on the right and bottom only (the reference's
-// padding type 2: tap (ky, kx) of output pixel (oy, ox) reads input pixel
-// (2*oy + ky, 2*ox + kx), src/indices.cpp:63-103), on square input maps of width
-// 8, 16 or 32. As in tagi_conv_stencil.h every workgroup first CHECKS the index
-// tables it was given against that stencil, for its own pixels, and runs the
-// table-driven loop if anything differs.
+// Regular-stencil kernel for the state backward of the stride-2 convolutions of a
+// ResNet: the 3x3 kernel with one pixel of padding on the right and bottom only (the
+// reference's padding type 2) and the 2x2 projection without padding - in both, tap
+// (ky, kx) of output pixel (oy, ox) reads input pixel (2*oy + ky, 2*ox + kx)
+// (src/indices.cpp:63-103) - on square input maps of width 8, 16 or 32. As in
+// tagi_conv_stencil.h every workgroup first CHECKS the index tables it was given against
+// that stencil, for its own pixels, and runs the table-driven loop if anything differs.
 //
-// State backward. An input pixel (y, x) is reached through the taps whose parity
-// matches its own: ky = y mod 2 (mod 2), kx likewise, i.e. through 4, 2, 2 or 1 of
-// the 9 taps by phase (y mod 2, x mod 2), from the output pixels
-// ((y - ky) / 2, (x - kx) / 2). With the columns numbered phase by phase
-// (ConvParams::perm_s = 2) a 128-column tile holds pixels (2*ly + py, 2*lx + px) of
-// ONE phase, and on the (ly, lx) grid of that phase the contraction is a small
-// stencil over the innovation maps: taps at offsets (-(ky / 2), -(kx / 2)), all in
-// {-1, 0}. So the workgroup stages the innovation rows of its channels once, with a
-// zero halo on top and left, and every tap is a constant offset into that patch. A
-// k-tile holds 32 / T output channels for a phase with T taps, which makes every
-// k-tile 16 MFMA steps per k-half whatever the phase; only the weights of the
-// phase's taps are staged.
+// An input pixel (y, x) is reached through the taps whose parity matches its own:
+// ky = y (mod 2), kx likewise, i.e. through 4, 2, 2 or 1 of the 9 taps (one of the 4) by
+// phase (y mod 2, x mod 2), from the output pixels ((y - ky) / 2, (x - kx) / 2). With the
+// columns numbered phase by phase (ConvParams::perm_s = 2), the pixels (2*ly + py,
+// 2*lx + px) of a phase form an (ly, lx) grid on which the contraction is a small stencil
+// over the innovation maps: taps at offsets (-(ky / 2), -(kx / 2)), all in {-1, 0}.
 //
 // Included by tagi_conv2d.hip after tagi_conv_stencil.h.
 #pragma once
@@ -25,25 +19,27 @@
 namespace tagi {
 namespace {
 
-// ---- state backward ------------------------------------------------------------------
+// ---- all four phases in one workgroup ----------------------------------------------------
+// The four phases of a block of input pixels (2*ly + py, 2*lx + px) read the SAME
+// innovation patch (output pixels (ly - a, lx - c), a, c in {0, 1}), each through its own
+// taps. A workgroup that keeps four accumulator sets therefore stages the patch once
+// and runs all KS*KS taps per staged channel pair - the reduction of a tile is KS*KS*fo
+// long, as in the unit-stride stencil, instead of 1..4 taps * fo - and pays the table
+// check, the first loads and the wind-down once per 4 x 64 x 128 outputs. Covers the
+// 3x3 kernel and the 2x2 projection of a residual block (one tap per phase, no halo).
+// (A workgroup per phase tile, the first form of this kernel, reduced over 1..4 taps * fo
+// only and reached 36-55 % of the matrix peak on ResNet-18's three layers.) The weights of an output channel, w[f][(m0+row)*T + t] for the
+// tile's 64 rows, are 64*T consecutive floats and are staged in that order.
+// 128 accumulator registers per lane: one 8-wave workgroup per CU.
 
-// Taps of the phase class: PY / PX = parity of the input row / column.
-template <int PY, int PX>
-struct PhaseTaps {
-    static constexpr int TY = PY == 0 ? 2 : 1, TX = PX == 0 ? 2 : 1, T = TY * TX;
-    // the i-th tap of the phase (row-major over its rows and columns)
-    static constexpr int ky(int i) { return PY == 0 ? 2 * (i / TX) : 1; }
-    static constexpr int kx(int i) { return PX == 0 ? 2 * (i % TX) : 1; }
-};
-
-// Expected (tap, output pixel) occurrences of input pixel (y, x) on a 2*WO-wide map;
-// returns the tap mask, out[t] = 1-based output pixel of tap t.
-template <int WO>
-__device__ __forceinline__ int s2_occurrences(int y, int x, int (&out)[9]) {
+// Expected (tap, output pixel) occurrences of input pixel (y, x) on a 2*WO-wide map for a
+// KS x KS kernel (KS = 2 or 3); returns the tap mask, out[t] = 1-based output pixel of tap t.
+template <int WO, int KS>
+__device__ __forceinline__ int s2k_occurrences(int y, int x, int (&out)[KS * KS]) {
     int mask = 0;
 #pragma unroll
-    for (int t = 0; t < 9; t++) {
-        const int ky = t / 3, kx = t - ky * 3;
+    for (int t = 0; t < KS * KS; t++) {
+        const int ky = t / KS, kx = t - ky * KS;
         const int ny = y - ky, nx = x - kx;
         const bool hit = ny >= 0 && nx >= 0 && (ny & 1) == 0 && (nx & 1) == 0 &&
                          (ny >> 1) < WO && (nx >> 1) < WO;
@@ -53,92 +49,177 @@ __device__ __forceinline__ int s2_occurrences(int y, int x, int (&out)[9]) {
     return mask;
 }
 
-// Do FCzwa_1 [wihi][nr] / Szz_ud [nr][wihi] list exactly those occurrences for the
-// pixels of columns n0 .. n0+127 (any order within a pixel's list)? Uniform verdict.
-// `scratch` holds 130 ints of LDS.
-template <int WO>
-__device__ __forceinline__ bool s2_dz_tables_ok(const ConvParams &p, int n0, int tid, int nthreads,
-                                                int *scratch) {
-    int *flag = scratch, *seen = scratch + 2;
-    if (tid == 0) *flag = 1;
-    if (tid < 128) seen[tid] = 0;
+// Do the two tables list exactly those occurrences for the 4 x 128 pixels of the tile
+// (phase-ordered columns ph * per_phase + q0 + c)? Thread (ph, c) owns one pixel and its
+// whole list (at most NR entries), all requested before any is looked at. Uniform verdict;
+// `scratch`: one int of LDS.
+template <int WO, int KS>
+__device__ __forceinline__ bool s2_all_tables_ok(const ConvParams &p, int q0, int per_phase,
+                                                 int tid, int *scratch) {
+    constexpr int T = KS * KS, NR = KS == 3 ? 4 : 1;
+    if (tid == 0) *scratch = 1;
     __syncthreads();
-    bool ok = p.nr >= 1 && p.nr <= 9;
-    const int entries = 128 * min(max(p.nr, 1), 9);
-    for (int e = tid; e < entries; e += nthreads) {
-        const int j = e >> 7, c = e & 127, n = n0 + c;
-        if (n >= p.N) continue;
-        const int px = dz_column(p, n).px;
-        const int o = p.idx2[j * p.wihi + px], tap = p.idx[px * p.nr + j];
-        if (o <= -1) continue;
-        if (tap < 1 || tap > 9) {
-            ok = false;
-            continue;
-        }
-        int want[9];
-        const int y = px / (2 * WO), x = px - y * (2 * WO);
-        const int mask = s2_occurrences<WO>(y, x, want);
-        const int t = tap - 1;
-        int w = 0;
+    bool ok = p.nr == NR;
+    if (ok) {
+        const int ph = tid >> 7, c = tid & 127;
+        const int px = dz_column(p, ph * per_phase + q0 + c).px;
+        int o[NR], tap[NR];
 #pragma unroll
-        for (int q = 0; q < 9; q++) w = q == t ? want[q] : w;
-        ok = ok && (mask >> t & 1) && o == w;
-        if (atomicOr(&seen[c], 1 << t) >> t & 1) ok = false;  // listed twice
-    }
-    __syncthreads();
-    if (tid < 128 && n0 + tid < p.N) {
-        const int px = dz_column(p, n0 + tid).px;
-        int want[9];
+        for (int j = 0; j < NR; j++) {
+            o[j] = p.idx2[j * p.wihi + px];
+            tap[j] = p.idx[px * NR + j];
+        }
+        int want[T];
         const int y = px / (2 * WO), x = px - y * (2 * WO);
-        ok = ok && seen[tid] == s2_occurrences<WO>(y, x, want);
+        const int mask = s2k_occurrences<WO, KS>(y, x, want);
+        int seen = 0;
+#pragma unroll
+        for (int j = 0; j < NR; j++) {
+            if (o[j] <= -1) continue;
+            if (tap[j] < 1 || tap[j] > T) {
+                ok = false;
+                continue;
+            }
+            const int t = tap[j] - 1;
+            int w = 0;
+#pragma unroll
+            for (int q = 0; q < T; q++) w = q == t ? want[q] : w;
+            ok = ok && o[j] == w && !(seen >> t & 1);
+            seen |= 1 << t;
+        }
+        ok = ok && seen == mask;
     }
-    if (!ok) *flag = 0;
+    if (!ok) *scratch = 0;
     __syncthreads();
-    const bool verdict = __builtin_amdgcn_readfirstlane(*flag) != 0;
+    const bool verdict = __builtin_amdgcn_readfirstlane(*scratch) != 0;
     __syncthreads();
     return verdict;
 }
 
-template <int WO, int T>
-struct S2DzGeom {
+// The epilogue of ConvDzProblem::store_with for two neighbouring input pixels at once.
+__device__ __forceinline__ bool s2_pair_stores_ok(const ConvParams &p) {
+    const uintptr_t all = reinterpret_cast<uintptr_t>(p.out0) | reinterpret_cast<uintptr_t>(p.out1) |
+                          reinterpret_cast<uintptr_t>(p.e0) |
+                          (p.res_mode ? reinterpret_cast<uintptr_t>(p.res0) |
+                                            reinterpret_cast<uintptr_t>(p.res1)
+                                      : 0);
+    return (all & 7u) == 0;
+}
+__device__ __forceinline__ void s2_finish_pair(const ConvParams &p, size_t at, float2 mu, float2 var,
+                                               float2 e, float2 r0, float2 r1) {
+    if (p.res_mode == 1) {
+        mu.x += r0.x; mu.y += r0.y;
+        var.x += r1.x; var.y += r1.y;
+    }
+    mu.x *= e.x; mu.y *= e.y;
+    var.x *= e.x * e.x; var.y *= e.y * e.y;
+    if (p.res_mode == 2) {
+        mu.x += r0.x; mu.y += r0.y;
+        var.x += r1.x; var.y += r1.y;
+    }
+    *reinterpret_cast<float2 *>(p.out0 + at) = mu;
+    *reinterpret_cast<float2 *>(p.out1 + at) = var;
+}
+// Accumulator register v of a lane is row row0 + 8*(v/4) + v%4 (tile_epilogue's layout);
+// (ma, va) / (mb, vb): the sums of input pixels (y, 2*lx) / (y, 2*lx + 1) of image b.
+template <int WO>
+__device__ __forceinline__ void s2_store_row_pairs(const ConvParams &p, floatx16 (&ma)[1][1],
+                                                   floatx16 (&va)[1][1], floatx16 (&mb)[1][1],
+                                                   floatx16 (&vb)[1][1], int row0, int b, int y,
+                                                   int lx) {
+    constexpr int WI = 2 * WO;
+    const size_t base = ((size_t)b * p.fi) * (WI * WI) + (size_t)y * WI + 2 * lx;
+    const float2 zero = make_float2(0.f, 0.f);
+    // the epilogue operands of eight rows are requested before their first store (a load
+    // that follows a store waits for it)
+#pragma unroll
+    for (int h = 0; h < 16; h += 8) {
+        float2 e[8], r0[8], r1[8];
+#pragma unroll
+        for (int v = h; v < h + 8; v++) {
+            const size_t at = base + (size_t)(row0 + 8 * (v / 4) + (v % 4)) * (WI * WI);
+            e[v - h] = *reinterpret_cast<const float2 *>(p.e0 + at);
+            r0[v - h] = p.res_mode ? *reinterpret_cast<const float2 *>(p.res0 + at) : zero;
+            r1[v - h] = p.res_mode ? *reinterpret_cast<const float2 *>(p.res1 + at) : zero;
+        }
+#pragma unroll
+        for (int v = h; v < h + 8; v++) {
+            const size_t at = base + (size_t)(row0 + 8 * (v / 4) + (v % 4)) * (WI * WI);
+            s2_finish_pair(p, at, make_float2(ma[0][0][v], mb[0][0][v]),
+                           make_float2(va[0][0][v], vb[0][0][v]), e[v - h], r0[v - h], r1[v - h]);
+        }
+    }
+}
+
+// Fold of a sliced reduction for phase-ordered columns (perm_s = 2) in the order of the
+// OUTPUT: a thread owns two neighbouring input pixels (y, 2*lx), (y, 2*lx + 1) of one
+// channel, whose partial sums lie in the two column phases of row phase y mod 2 at the
+// same offset - consecutive threads read consecutive partial sums of either phase and
+// write consecutive pairs. ws0/ws1 [split][M][N]; W = p.perm_w (even).
+__global__ __launch_bounds__(256) void reduce_store_s2_pairs_kernel(ConvParams p) {
+    const int W = p.perm_w, ws = W / 2;
+    const size_t pairs = (size_t)p.M * p.N / 2;
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= pairs) return;
+    // i = ((b * M + m) * W + y) * ws + lx : the order of the output tensor
+    const int lx = (int)(i % ws);
+    size_t rest = i / ws;
+    const int y = (int)(rest % W);
+    rest /= W;
+    const int m = (int)(rest % p.M), b = (int)(rest / p.M);
+    const int per_img = p.wihi / 4, per_phase = p.B * per_img;
+    const size_t col = (size_t)((y & 1) * 2) * per_phase + (size_t)b * per_img + (y >> 1) * ws + lx;
+    const size_t total = (size_t)p.M * p.N, src = (size_t)m * p.N + col;
+    float2 mu = make_float2(0.f, 0.f), var = mu;
+#pragma unroll 4
+    for (int s = 0; s < p.splits; s++) {
+        mu.x += p.ws0[s * total + src];
+        mu.y += p.ws0[s * total + src + per_phase];
+        var.x += p.ws1[s * total + src];
+        var.y += p.ws1[s * total + src + per_phase];
+    }
+    const size_t at = ((size_t)b * p.M + m) * p.wihi + (size_t)y * W + 2 * lx;
+    const float2 zero = make_float2(0.f, 0.f);
+    s2_finish_pair(p, at, mu, var, *reinterpret_cast<const float2 *>(p.e0 + at),
+                   p.res_mode ? *reinterpret_cast<const float2 *>(p.res0 + at) : zero,
+                   p.res_mode ? *reinterpret_cast<const float2 *>(p.res1 + at) : zero);
+}
+
+inline hipError_t launch_reduce_store_s2_pairs(const ConvParams &p, hipStream_t stream) {
+    const size_t pairs = (size_t)p.M * p.N / 2;
+    hipLaunchKernelGGL(reduce_store_s2_pairs_kernel, dim3((unsigned)((pairs + 255) / 256)), dim3(256),
+                       0, stream, p);
+    return hipGetLastError();
+}
+
+template <int WO, int KS>
+struct S2AllGeom {
     using G = StencilGeom<WO>;               // patch layout of one channel: rows -1 .. RPI, zero halo
-    // output channels per k-tile (the narrowest maps hold eight images per tile: their
-    // patch is kept to 16 channels so that two workgroups still share a CU)
-    static constexpr int KC = (WO == 4 && T == 1) ? 16 : 32 / T;
+    static constexpr int T = KS * KS;
+    static constexpr int KC = WO == 4 ? 8 : 16;            // output channels per k-tile
     static constexpr int PATCH = KC * G::CS;
-    // rows -1 .. RPI-1 are read (taps reach up and left only); the bottom halo row is
-    // never loaded and stays zero
     static constexpr int UNITS = KC * G::SEGS * (G::RPI + 1) * (WO / 4);
     static constexpr int P_SLOTS = (UNITS + 511) / 512;
-    static constexpr int WS = 64 + 4;        // weight tile [T][KC][64 rows + 4]
-    static constexpr int W_FLOATS = T * KC * WS;
-    static constexpr int W_SLOTS = T * KC * 64 / 512;  // 4
-    static constexpr int LDS_FLOATS = W_FLOATS + 2 * PATCH;
+    static constexpr int WROW = 64 * T;                    // floats of one output channel
+    static constexpr int W_VEC = KC * WROW / 4;            // 16-byte pieces per k-tile
+    static constexpr int W_SLOTS = (W_VEC + 511) / 512;
+    static constexpr int LDS_FLOATS = KC * WROW + 2 * PATCH;
 };
 
-// One 64 x 128 tile of one phase on a verified stencil. c_begin / c_end: output
-// channels of the reduction slice (multiples of 32).
-template <int WO, int PY, int PX>
-__device__ __forceinline__ void s2_dz_body(const ConvParams &p, float *lds, int m0, int n0,
-                                           int split, int c_begin, int c_end) {
-    using PT = PhaseTaps<PY, PX>;
-    constexpr int T = PT::T;
-    using S = S2DzGeom<WO, T>;
+template <int WO, int KS>
+__device__ __forceinline__ void s2_all_body(const ConvParams &p, float *lds, int m0, int q0,
+                                            int per_phase, int split, int c_begin, int c_end) {
+    using S = S2AllGeom<WO, KS>;
     using G = StencilGeom<WO>;
-    constexpr int W = WO, H = WO, NT = 512, KC = S::KC;
+    constexpr int W = WO, H = WO, NT = 512, KC = S::KC, T = S::T;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wrow = (wave / 4) * 32, wcol = (wave % 4) * 32, half = lane >> 5;
-    float *lds_w = lds;                 // [T][KC][WS]
-    float *lds_p = lds + S::W_FLOATS;   // [PATCH][2]: (delta_mu, delta_var) interleaved
+    float *lds_w = lds;                      // [KC][64 rows * T], memory order
+    float *lds_p = lds + KC * S::WROW;       // [PATCH][2]: (delta_mu, delta_var) interleaved
 
     for (int i = tid; i < 2 * S::PATCH; i += NT) lds_p[i] = 0.f;
 
-    // position of the tile inside its phase: pixels (b, ly, lx) in the order of the
-    // innovation maps
-    const int per_phase = p.B * W * H;
-    const int q0 = n0 % per_phase;
-
-    // patch units of this thread
+    // patch units of this thread (rows -1 .. RPI-1 of each segment; taps reach up and left)
     size_t punit[S::P_SLOTS];
     int pdst[S::P_SLOTS];
     bool p_ok[S::P_SLOTS];
@@ -160,140 +241,221 @@ __device__ __forceinline__ void s2_dz_body(const ConvParams &p, float *lds, int 
     }
     const size_t pstep = (size_t)KC * (W * H);
 
-    // weight elements of this thread: w[f][m0 + row][tap ti], row fastest
+    // weight pieces of this thread: 16 bytes of w[c_begin + f][(m0 + row) * T + t]
     size_t wsrc[S::W_SLOTS];
     int wdst[S::W_SLOTS];
+    bool w_ok[S::W_SLOTS];
 #pragma unroll
     for (int i = 0; i < S::W_SLOTS; i++) {
-        const int e = tid + i * NT, row = e & 63, rest = e >> 6, f = rest % KC, ti = rest / KC;
-        int tap = 0;
-#pragma unroll
-        for (int q = 0; q < T; q++) tap = q == ti ? PT::ky(q) * 3 + PT::kx(q) : tap;
-        wsrc[i] = ((size_t)(c_begin + f) * p.fi + m0 + row) * 9 + tap;
-        wdst[i] = (ti * KC + f) * S::WS + row;
+        const int e = tid + i * NT;
+        w_ok[i] = e < S::W_VEC;
+        const int id = w_ok[i] ? e : 0;
+        const int f = id / (S::WROW / 4), q = id - f * (S::WROW / 4);
+        wsrc[i] = ((size_t)(c_begin + f) * p.fi + m0) * T + 4 * q;
+        wdst[i] = f * S::WROW + 4 * q;
     }
-    const size_t wstep = (size_t)KC * p.fi * 9;
+    const size_t wstep = (size_t)KC * p.fi * T;
 
-    floatx16 acc0[1][1], acc1[1][1];
+    // one accumulator pair per phase (py, px), named one by one: an array of them indexed
+    // by the tap's phase is kept in scratch memory by the compiler
+    floatx16 m00[1][1], m01[1][1], m10[1][1], m11[1][1], v00[1][1], v01[1][1], v10[1][1], v11[1][1];
 #pragma unroll
     for (int v = 0; v < 16; v++) {
-        acc0[0][0][v] = 0.f;
-        acc1[0][0][v] = 0.f;
+        m00[0][0][v] = m01[0][0][v] = m10[0][0][v] = m11[0][0][v] = 0.f;
+        v00[0][0][v] = v01[0][0][v] = v10[0][0][v] = v11[0][0][v] = 0.f;
     }
 
-    float4 rp0[S::P_SLOTS], rp1[S::P_SLOTS];
-    float rw[S::W_SLOTS];
-
-#define TAGI_S2DZ_FETCH()                                                             \
+    // staging registers, named one by one (arrays of them end up in scratch memory)
+    static_assert(S::W_SLOTS <= 5 && S::P_SLOTS <= 2, "staging registers below");
+    float4 rw0, rw1, rw2, rw3, rw4, rpa0, rpa1, rpb0, rpb1;
+    rw0 = rw1 = rw2 = rw3 = rw4 = rpa0 = rpa1 = rpb0 = rpb1 = make_float4(0.f, 0.f, 0.f, 0.f);
+#define TAGI_S2ALL_WLOAD(i)                                                           \
+    if (i < S::W_SLOTS) {                                                             \
+        rw##i = *reinterpret_cast<const float4 *>(p.w0 + wsrc[i < S::W_SLOTS ? i : 0]); \
+        if (w_ok[i < S::W_SLOTS ? i : 0]) wsrc[i < S::W_SLOTS ? i : 0] += wstep;      \
+    }
+#define TAGI_S2ALL_WPUT(i)                                                            \
+    if (i < S::W_SLOTS && w_ok[i < S::W_SLOTS ? i : 0])                               \
+        *reinterpret_cast<float4 *>(lds_w + wdst[i < S::W_SLOTS ? i : 0]) = rw##i;
+#define TAGI_S2ALL_PLOAD(i, A_, B_)                                                   \
+    if (i < S::P_SLOTS) {                                                             \
+        A_ = *reinterpret_cast<const float4 *>(p.d0 + punit[i < S::P_SLOTS ? i : 0]); \
+        B_ = *reinterpret_cast<const float4 *>(p.d1 + punit[i < S::P_SLOTS ? i : 0]); \
+        if (p_ok[i < S::P_SLOTS ? i : 0]) punit[i < S::P_SLOTS ? i : 0] += pstep;     \
+    }
+#define TAGI_S2ALL_PPUT(i, A_, B_)                                                    \
+    if (i < S::P_SLOTS && p_ok[i < S::P_SLOTS ? i : 0]) {                             \
+        float *dst_ = lds_p + 2 * pdst[i < S::P_SLOTS ? i : 0];                       \
+        *reinterpret_cast<float4 *>(dst_) = make_float4(A_.x, B_.x, A_.y, B_.y);      \
+        *reinterpret_cast<float4 *>(dst_ + 4) = make_float4(A_.z, B_.z, A_.w, B_.w);  \
+    }
+#define TAGI_S2ALL_FETCH()                                                            \
     do {                                                                              \
-        _Pragma("unroll") for (int i = 0; i < S::W_SLOTS; i++) {                      \
-            rw[i] = p.w0[wsrc[i]];                                                    \
-            wsrc[i] += wstep;                                                         \
-        }                                                                             \
-        _Pragma("unroll") for (int i = 0; i < S::P_SLOTS; i++) {                      \
-            rp0[i] = *reinterpret_cast<const float4 *>(p.d0 + punit[i]);              \
-            rp1[i] = *reinterpret_cast<const float4 *>(p.d1 + punit[i]);              \
-            if (p_ok[i]) punit[i] += pstep;                                           \
-        }                                                                             \
+        TAGI_S2ALL_WLOAD(0) TAGI_S2ALL_WLOAD(1) TAGI_S2ALL_WLOAD(2)                   \
+        TAGI_S2ALL_WLOAD(3) TAGI_S2ALL_WLOAD(4)                                       \
+        TAGI_S2ALL_PLOAD(0, rpa0, rpb0) TAGI_S2ALL_PLOAD(1, rpa1, rpb1)               \
     } while (0)
-#define TAGI_S2DZ_COMMIT()                                                            \
+#define TAGI_S2ALL_COMMIT()                                                           \
     do {                                                                              \
-        _Pragma("unroll") for (int i = 0; i < S::W_SLOTS; i++) lds_w[wdst[i]] = rw[i]; \
-        _Pragma("unroll") for (int i = 0; i < S::P_SLOTS; i++) if (p_ok[i]) {         \
-            *reinterpret_cast<float4 *>(lds_p + 2 * pdst[i]) =                        \
-                make_float4(rp0[i].x, rp1[i].x, rp0[i].y, rp1[i].y);                  \
-            *reinterpret_cast<float4 *>(lds_p + 2 * pdst[i] + 4) =                    \
-                make_float4(rp0[i].z, rp1[i].z, rp0[i].w, rp1[i].w);                  \
-        }                                                                             \
+        TAGI_S2ALL_WPUT(0) TAGI_S2ALL_WPUT(1) TAGI_S2ALL_WPUT(2)                      \
+        TAGI_S2ALL_WPUT(3) TAGI_S2ALL_WPUT(4)                                         \
+        TAGI_S2ALL_PPUT(0, rpa0, rpb0) TAGI_S2ALL_PPUT(1, rpa1, rpb1)                 \
     } while (0)
 
     // operand addresses of this lane: patch cell (row ly - 1, column lx - 1) of its pixel
-    // for output channel `half` of a pair; weights of its row
+    // for output channel `half` of a pair; the T weights of its row
     const int pix = wcol + (lane & 31), prow = pix / W, px = pix - prow * W;
     const float *bp = lds_p + 2 * (half * G::CS + (prow / G::RPI) * G::SEG +
                                    (prow % G::RPI) * G::RS + G::XO - 1 + px);
-    const float *wp = lds_w + half * S::WS + wrow + (lane & 31);
+    const float *wp = lds_w + half * S::WROW + (wrow + (lane & 31)) * T;
 
     __syncthreads();  // patch zeroed
     if (c_begin < c_end) {
-        TAGI_S2DZ_FETCH();
-        TAGI_S2DZ_COMMIT();
+        TAGI_S2ALL_FETCH();
+        TAGI_S2ALL_COMMIT();
     }
     __syncthreads();
 
     for (int c0 = c_begin; c0 < c_end; c0 += KC) {
         const bool more = c0 + KC < c_end;
-        if (more) TAGI_S2DZ_FETCH();
+        if (more) TAGI_S2ALL_FETCH();
 #pragma unroll
         for (int pair = 0; pair < KC / 2; pair++) {
+            // the innovations of output pixels (ly - a, lx - c)
+            float2 y[2][2];
 #pragma unroll
-            for (int ti = 0; ti < T; ti++) {
-                // tap (ky, kx) brings the innovation of output pixel (ly - ky/2, lx - kx/2)
-                const int off = (1 - PT::ky(ti) / 2) * G::RS + (1 - PT::kx(ti) / 2);
-                const float2 y = *reinterpret_cast<const float2 *>(bp + 2 * (2 * pair * G::CS + off));
-                const float w = wp[(ti * KC + 2 * pair) * S::WS];
-                acc0[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(w, y.x, acc0[0][0], 0, 0, 0);
-                acc1[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(w * w, y.y, acc1[0][0], 0, 0, 0);
+            for (int a = 0; a < (KS + 1) / 2; a++)
+#pragma unroll
+                for (int c = 0; c < (KS + 1) / 2; c++)
+                    y[a][c] = *reinterpret_cast<const float2 *>(
+                        bp + 2 * (2 * pair * G::CS + (1 - a) * G::RS + (1 - c)));
+            // tap (ky, kx): phase (ky & 1, kx & 1), innovation of output pixel (ly - ky/2, lx - kx/2)
+#define TAGI_S2ALL_TAP(W_, M_, V_, Y_)                                                        \
+    do {                                                                                      \
+        const float w_ = (W_);                                                                \
+        M_[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(w_, (Y_).x, M_[0][0], 0, 0, 0);       \
+        V_[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(w_ * w_, (Y_).y, V_[0][0], 0, 0, 0);  \
+    } while (0)
+            if constexpr (KS == 2) {
+                // 16 bytes per lane: rows at a stride of four floats would share banks
+                const float4 w4 = *reinterpret_cast<const float4 *>(wp + 2 * pair * S::WROW);
+                TAGI_S2ALL_TAP(w4.x, m00, v00, y[0][0]);
+                TAGI_S2ALL_TAP(w4.y, m01, v01, y[0][0]);
+                TAGI_S2ALL_TAP(w4.z, m10, v10, y[0][0]);
+                TAGI_S2ALL_TAP(w4.w, m11, v11, y[0][0]);
+            } else {
+                const float *wq = wp + 2 * pair * S::WROW;   // stride 9 between rows: no conflicts
+                TAGI_S2ALL_TAP(wq[0], m00, v00, y[0][0]);
+                TAGI_S2ALL_TAP(wq[1], m01, v01, y[0][0]);
+                TAGI_S2ALL_TAP(wq[2], m00, v00, y[0][1]);
+                TAGI_S2ALL_TAP(wq[3], m10, v10, y[0][0]);
+                TAGI_S2ALL_TAP(wq[4], m11, v11, y[0][0]);
+                TAGI_S2ALL_TAP(wq[5], m10, v10, y[0][1]);
+                TAGI_S2ALL_TAP(wq[6], m00, v00, y[1][0]);
+                TAGI_S2ALL_TAP(wq[7], m01, v01, y[1][0]);
+                TAGI_S2ALL_TAP(wq[8], m00, v00, y[1][1]);
             }
+#undef TAGI_S2ALL_TAP
         }
         __syncthreads();
         if (more) {
-            TAGI_S2DZ_COMMIT();
+            TAGI_S2ALL_COMMIT();
             __syncthreads();
         }
     }
-#undef TAGI_S2DZ_FETCH
-#undef TAGI_S2DZ_COMMIT
-    tile_epilogue<ConvDzProblem, 64, 128, 2, 4>(p, acc0, acc1, m0, n0, split);
+#undef TAGI_S2ALL_FETCH
+#undef TAGI_S2ALL_COMMIT
+#undef TAGI_S2ALL_WLOAD
+#undef TAGI_S2ALL_WPUT
+#undef TAGI_S2ALL_PLOAD
+#undef TAGI_S2ALL_PPUT
+    if (p.splits > 1 || !s2_pair_stores_ok(p)) {
+        // partial sums (contiguous in the phase-ordered workspace), or outputs that are
+        // not 8-byte aligned: phase by phase
+        tile_epilogue<ConvDzProblem, 64, 128, 2, 4>(p, m00, v00, m0, q0, split);
+        tile_epilogue<ConvDzProblem, 64, 128, 2, 4>(p, m01, v01, m0, per_phase + q0, split);
+        tile_epilogue<ConvDzProblem, 64, 128, 2, 4>(p, m10, v10, m0, 2 * per_phase + q0, split);
+        tile_epilogue<ConvDzProblem, 64, 128, 2, 4>(p, m11, v11, m0, 3 * per_phase + q0, split);
+        return;
+    }
+    // Complete sums: the two column phases of a lane's pixel are neighbours in memory
+    // ((2*ly + py, 2*lx) and (2*ly + py, 2*lx + 1)), so they leave as one 8-byte store
+    // and a wave writes whole rows. (Phase by phase the same outputs are 4-byte stores
+    // two elements apart: 89 of 173 us at 64 -> 128 channels on 32 x 32 maps.)
+    const int q = q0 + pix, b = q / (W * H), l = q - b * (W * H), ly = l / W, lx = l - ly * W;
+    const int row0 = m0 + wrow + 4 * half;
+    s2_store_row_pairs<W>(p, m00, v00, m01, v01, row0, b, 2 * ly, lx);
+    s2_store_row_pairs<W>(p, m10, v10, m11, v11, row0, b, 2 * ly + 1, lx);
 }
 
-template <int WO>
-struct S2DzLds {
+template <int WO, int KS>
+struct S2AllLds {
     using P = ConvDzProblem;
     static constexpr int XF = TileGeom<P::XK, 64>::floats, YF = TileGeom<P::YK, 128>::floats;
     static constexpr int GENERIC = P::NX * XF + P::NY * YF;
-    static constexpr int a = S2DzGeom<WO, 4>::LDS_FLOATS, b = S2DzGeom<WO, 2>::LDS_FLOATS,
-                         c = S2DzGeom<WO, 1>::LDS_FLOATS;
-    static constexpr int m1 = a > b ? a : b, m2 = m1 > c ? m1 : c;
-    static constexpr int FLOATS = m2 > GENERIC ? m2 : GENERIC;
+    static constexpr int MINE = S2AllGeom<WO, KS>::LDS_FLOATS;
+    static constexpr int FLOATS = MINE > GENERIC ? MINE : GENERIC;
 };
 
-// One 64 x 128 tile per workgroup of 8 waves; columns are numbered phase by phase
-// (perm_s = 2) and a tile lies inside one phase (batch * WO * WO is a multiple of 128).
-template <int WO>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4)))
-void conv_stencil_s2_dz_kernel(ConvParams p) {
+// One workgroup of 8 waves per 64 input channels x 128 base pixels x 4 phases; grid.x =
+// (fi / 64) * (B * WO * WO / 128), grid.y = reduction slices (whole groups of 32 output
+// channels). Tables that are not the expected stencil: the four phase tiles run through
+// the table-driven loop one after the other.
+template <int WO, int KS>
+__global__ __launch_bounds__(512) void conv_stencil_s2_all_dz_kernel(ConvParams p) {
     using P = ConvDzProblem;
-    using L = S2DzLds<WO>;
+    using L = S2AllLds<WO, KS>;
     __shared__ __attribute__((aligned(16))) float lds[L::FLOATS];
     extern __shared__ __attribute__((aligned(16))) int lds_extra[];
 
-    const int tiles_n = (p.N + 127) / 128;
+    const int per_phase = p.B * WO * WO;
+    const int tiles_q = per_phase / 128;
     const int split = blockIdx.y;
-    const int tile = P::place_tile(p, blockIdx.x, split, gridDim.x);
-    const int m0 = (tile / tiles_n) * 64, n0 = (tile % tiles_n) * 128;
+    const int m0 = (blockIdx.x / tiles_q) * 64, q0 = (blockIdx.x % tiles_q) * 128;
     const int r_begin = split * p.r_per_split;
     const int r_end = min(p.R, r_begin + p.r_per_split);
 
-    if (s2_dz_tables_ok<WO>(p, n0, threadIdx.x, 512, lds_extra)) {
-        const int phase = n0 / (p.B * WO * WO);
-        const int c_begin = r_begin / 9, c_end = r_end / 9;
-        switch (phase) {
-            case 0: s2_dz_body<WO, 0, 0>(p, lds, m0, n0, split, c_begin, c_end); break;
-            case 1: s2_dz_body<WO, 0, 1>(p, lds, m0, n0, split, c_begin, c_end); break;
-            case 2: s2_dz_body<WO, 1, 0>(p, lds, m0, n0, split, c_begin, c_end); break;
-            default: s2_dz_body<WO, 1, 1>(p, lds, m0, n0, split, c_begin, c_end); break;
-        }
+    if (s2_all_tables_ok<WO, KS>(p, q0, per_phase, threadIdx.x, lds_extra)) {
+        s2_all_body<WO, KS>(p, lds, m0, q0, per_phase, split, r_begin / (KS * KS), r_end / (KS * KS));
         return;
     }
-    typename P::Ctx ctx;
-    P::prologue(p, ctx, lds_extra, threadIdx.x, 512, m0, n0, 64, 128, r_begin, r_end);
-    __syncthreads();
-    int r_lo = r_begin, r_hi = r_end;
-    P::adjust_range(p, ctx, r_lo, r_hi);
-    mfma_tile_body<P, 64, 128, 2, 4, 0>(p, ctx, reinterpret_cast<float (*)[L::XF]>(lds),
-                                        reinterpret_cast<float (*)[L::YF]>(lds + P::NX * L::XF), m0,
-                                        n0, split, r_lo, r_hi);
+    for (int ph = 0; ph < 4; ph++) {
+        const int n0 = ph * per_phase + q0;
+        __syncthreads();  // the previous phase's tables and tiles are done with
+        typename P::Ctx ctx;
+        P::prologue(p, ctx, lds_extra, threadIdx.x, 512, m0, n0, 64, 128, r_begin, r_end);
+        __syncthreads();
+        int r_lo = r_begin, r_hi = r_end;
+        P::adjust_range(p, ctx, r_lo, r_hi);
+        mfma_tile_body<P, 64, 128, 2, 4, 0>(p, ctx, reinterpret_cast<float (*)[L::XF]>(lds),
+                                            reinterpret_cast<float (*)[L::YF]>(lds + P::NX * L::XF),
+                                            m0, n0, split, r_lo, r_hi);
+    }
+}
+
+template <int KS>
+inline hipError_t launch_conv_stencil_s2_all_dz(int wo, const ConvParams &p, hipStream_t stream) {
+    using P = ConvDzProblem;
+    const dim3 grid((p.M / 64) * (p.B * wo * wo / 128), p.splits);
+    const size_t extra = P::extra_lds_bytes(p, 64, 128);
+    if (extra > kTileExtraLdsMax) return hipErrorInvalidValue;
+#define TAGI_LAUNCH_S2ALL(WD)                                                                      \
+    case WD: {                                                                                     \
+        static PerDeviceOnce once;                                                                 \
+        hipError_t e = allow_dynamic_lds(                                                          \
+            once, reinterpret_cast<const void *>(conv_stencil_s2_all_dz_kernel<WD, KS>),           \
+            (int)kTileExtraLdsMax);                                                                \
+        if (e != hipSuccess) return e;                                                             \
+        hipLaunchKernelGGL((conv_stencil_s2_all_dz_kernel<WD, KS>), grid, dim3(512), extra, stream, p); \
+        return hipGetLastError();                                                                  \
+    }
+    switch (wo) {
+        TAGI_LAUNCH_S2ALL(4)
+        TAGI_LAUNCH_S2ALL(8)
+        TAGI_LAUNCH_S2ALL(16)
+    }
+#undef TAGI_LAUNCH_S2ALL
+    return hipErrorInvalidValue;
 }
 
 // Output map width for which the strided kernels exist, 0 otherwise.
@@ -301,30 +463,6 @@ inline int s2_out_width(int out_pixels) {
     for (int w : {4, 8, 16})
         if (w * w == out_pixels) return w;
     return 0;
-}
-
-inline hipError_t launch_conv_stencil_s2_dz(int wo, const ConvParams &p, hipStream_t stream) {
-    using P = ConvDzProblem;
-    const dim3 grid(((p.M + 63) / 64) * ((p.N + 127) / 128), p.splits);
-    const size_t extra = P::extra_lds_bytes(p, 64, 128);
-    if (extra > kTileExtraLdsMax) return hipErrorInvalidValue;
-#define TAGI_LAUNCH_S2DZ(WD)                                                                    \
-    case WD: {                                                                                  \
-        static PerDeviceOnce once;                                                              \
-        hipError_t e = allow_dynamic_lds(                                                       \
-            once, reinterpret_cast<const void *>(conv_stencil_s2_dz_kernel<WD>),                \
-            (int)kTileExtraLdsMax);                                                             \
-        if (e != hipSuccess) return e;                                                          \
-        hipLaunchKernelGGL((conv_stencil_s2_dz_kernel<WD>), grid, dim3(512), extra, stream, p); \
-        return hipGetLastError();                                                               \
-    }
-    switch (wo) {
-        TAGI_LAUNCH_S2DZ(4)
-        TAGI_LAUNCH_S2DZ(8)
-        TAGI_LAUNCH_S2DZ(16)
-    }
-#undef TAGI_LAUNCH_S2DZ
-    return hipErrorInvalidValue;
 }
 
 }  // namespace

@@ -251,6 +251,10 @@ extern int g_conv2d_group_loads;
 extern int g_conv2d_stencil;
 // 0 keeps the natural column order in the conv2d state backward of strided layers.
 extern int g_conv2d_phase_order;
+extern int g_conv2d_s2_all;   // 0: no all-phase kernel for the strided state backward
+int conv2d_bwd_dz_s2_all(const float *mu_w, const float *dmu, const float *dvar, int B, int fo,
+                         int woho, int wihi, int fi, int ki, int nr);
+int conv2d_bwd_dz_s2_all_splits(int B, int fo, int woho, int fi);
 
 hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
                              const float *var_b, const float *mu_a, const float *var_a,

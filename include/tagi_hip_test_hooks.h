@@ -29,7 +29,8 @@ extern "C" {
  * keeps small layers off their one-launch forward kernel), "linear.small" (0: no
  * one-launch forward for small layers). Conv2d: "conv2d.tile",
  * "conv2d.splits", "conv2d.dw.tile", "conv2d.dw.splits", "conv2d.group_loads",
- * "conv2d.stencil", "conv2d.phase_order" (0 switches the named path off). */
+ * "conv2d.stencil", "conv2d.phase_order", "conv2d.s2_all" (0 switches the named path
+ * off; s2_all: the stride-2 state backward that keeps all four phases in one workgroup). */
 int tagi_hip_tune(const char *key /* host */, int value);
 
 #ifdef __cplusplus

@@ -35,6 +35,11 @@ GEOMS = [
     (3, 2, 1, 2, 16, 128, 96, 2),  # 8x8 output maps, two images per tile
     (3, 2, 1, 2, 8, 64, 160, 8),   # 4x4 output maps, eight images per tile
     (3, 2, 1, 2, 16, 64, 640, 2),  # long reduction: sliced
+    # 2x2 s2 projections with whole groups of channels: the all-phase state backward
+    (2, 2, 0, 1, 32, 64, 64, 1),
+    (2, 2, 0, 1, 16, 128, 96, 2),
+    (2, 2, 0, 1, 8, 64, 160, 8),
+    (2, 2, 0, 1, 16, 64, 640, 2),
 ]
 
 
@@ -190,8 +195,8 @@ def test_conv2d_stencil_kernels_agree_with_the_table_path():
 
 
 def test_conv2d_strided_stencil_kernels_agree_with_the_table_path():
-    """3x3 stride 2: the same inputs through the strided stencil kernels and, with the
-    stencil kernels switched off, through the table-driven ones."""
+    """3x3 stride 2: the same inputs with the stencil kernels on (the state backward has
+    one) and, with them switched off, through the table-driven kernels."""
     import torch
     import cutagi_amd.functional as F
     from cutagi_amd import capi
@@ -222,6 +227,66 @@ def test_conv2d_strided_stencil_kernels_agree_with_the_table_path():
             switched.append(name)
     # a different summation order shows that the switch switched the state backward
     assert "delta_mu_z" in switched
+
+
+@pytest.mark.parametrize("geom", [(3, 2, 1, 2, 32, 64, 64, 1), (3, 2, 1, 2, 16, 128, 96, 2),
+                                  (3, 2, 1, 2, 8, 64, 160, 8), (3, 2, 1, 2, 16, 64, 640, 2),
+                                  (2, 2, 0, 1, 16, 64, 96, 2)])
+def test_conv2d_strided_state_backward_kernels_agree(oracle_lib, geom):
+    """The stride-2 state backward on its stencil kernel (one workgroup for all four
+    phases of a pixel block; default) and on the table-driven kernel, switched off either
+    by its own switch or with all stencil kernels. All give the oracle's result, and the
+    stencil kernel differs from the table-driven one in its summation order."""
+    import cutagi_amd.functional as F
+    from cutagi_amd import capi
+    k, s, p, pt, wi, fi, fo, B = geom
+    idx, d, t, ti, wihi, woho = _setup(oracle_lib, geom, False, seed=21)
+    ref = oracle_lib.conv2d_bwd_dz(d["mu_w"], d["jcb"], d["delta_mu"], d["delta_var"],
+                                   idx["FCzwa_1"], idx["Szz_ud"], woho, fo, wihi, fi, k, idx["h"],
+                                   B, threads=4)
+    got = {}
+    try:
+        for name, all_phase, stencil in (("all", 1, 1), ("own_switch", 0, 1), ("tables", 1, 0)):
+            capi.tune("conv2d.s2_all", all_phase)
+            capi.tune("conv2d.stencil", stencil)
+            dz = F.conv2d_bwd_dz(t["mu_w"], t["jcb"], t["delta_mu"], t["delta_var"], ti["FCzwa_1"],
+                                 ti["Szz_ud"], woho, fo, wihi, fi, k, idx["h"], B)
+            got[name] = (dz[0].cpu().numpy(), dz[1].cpu().numpy())
+            assert_close(got[name][0], ref[0], "delta_mu_z (%s)" % name)
+            assert_close(got[name][1], ref[1], "delta_var_z (%s)" % name, same_sign=True)
+    finally:
+        capi.tune("conv2d.s2_all", 1)
+        capi.tune("conv2d.stencil", 1)
+    assert not np.array_equal(got["all"][0], got["tables"][0])
+    assert np.array_equal(got["own_switch"][0], got["tables"][0])
+
+
+def test_conv2d_projection_tables_of_another_geometry_take_the_table_path(oracle_lib):
+    """2x2 stride 2: every input pixel has one occurrence. One pixel's entry is pointed
+    at another output pixel: the workgroup that owns it runs the table-driven loop for
+    its four phase tiles, and the result is what the tables say."""
+    import torch
+    import cutagi_amd.functional as F
+    from cutagi_amd import capi
+    k, wi, fi, fo, B = 2, 16, 64, 32, 2
+    idx = capi.conv2d_build_idx(k, 2, wi, wi, 0, 1, k * k * fi * fo + 1)
+    wihi, woho, h = wi * wi, idx["wo"] * idx["ho"], idx["h"]
+    assert h == 1
+    zud = idx["Szz_ud"].copy()
+    zud[41] = (zud[41] % woho) + 1
+    d = conv_inputs(fi, fo, k, wihi, woho, B, seed=10, bias=False, jcb_random=True)
+    t = {n: (None if v is None else torch.from_numpy(v).cuda()) for n, v in d.items()}
+    dz = F.conv2d_bwd_dz(t["mu_w"], t["jcb"], t["delta_mu"], t["delta_var"],
+                         torch.from_numpy(idx["FCzwa_1"]).cuda(), torch.from_numpy(zud).cuda(),
+                         woho, fo, wihi, fi, k, h, B)
+    ref = oracle_lib.conv2d_bwd_dz(d["mu_w"], d["jcb"], d["delta_mu"], d["delta_var"],
+                                   idx["FCzwa_1"], zud, woho, fo, wihi, fi, k, h, B, threads=4)
+    assert_close(dz[0].cpu().numpy(), ref[0], "delta_mu_z")
+    assert_close(dz[1].cpu().numpy(), ref[1], "delta_var_z", same_sign=True)
+    clean = oracle_lib.conv2d_bwd_dz(d["mu_w"], d["jcb"], d["delta_mu"], d["delta_var"],
+                                     idx["FCzwa_1"], idx["Szz_ud"], woho, fo, wihi, fi, k, h, B,
+                                     threads=4)
+    assert not np.array_equal(clean[0], ref[0])
 
 
 def test_conv2d_strided_tables_of_another_geometry_take_the_table_path(oracle_lib):
