@@ -759,16 +759,25 @@ inline int lcm_int(int a, int b) {
 // `s2_all`: output map width when the stride-2 state-backward stencil kernel applies.
 template <class P, bool DZ>
 hipError_t run_sliced(int tile, int splits, int stencil, float *ws0, float *ws1, ConvParams &p,
-                      hipStream_t stream, int s2_all = 0) {
+                      hipStream_t stream, int s2_all = 0, int s2_fwd = 0) {
     // the state backward re-states its slices per tile in whole output channels
     // (the stencil kernels: in whole groups of 32 channels)
-    const int unit = (stencil || s2_all) ? 32 * p.k2 : DZ ? lcm_int(KT, p.k2) : KT;
+    const int unit = (stencil || s2_all || s2_fwd) ? 32 * p.k2 : DZ ? lcm_int(KT, p.k2) : KT;
     const int per = ceil_div(ceil_div(p.R, splits), unit) * unit;
     p.splits = ceil_div(p.R, per);
     p.r_per_split = per;
     p.ws0 = ws0;
     p.ws1 = ws1;
-    hipError_t e = s2_all     ? (p.k2 == 9 ? launch_conv_stencil_s2_all_dz<3>(s2_all, p, stream)
+    hipError_t e = hipSuccess;
+    if constexpr (!DZ) {
+        if (s2_fwd) {
+            e = p.k2 == 9 ? launch_conv_stencil_s2_fwd<3>(s2_fwd, p, stream)
+                          : launch_conv_stencil_s2_fwd<2>(s2_fwd, p, stream);
+            if (e != hipSuccess || p.splits == 1) return e;
+            return launch_reduce_store<P>(p, stream);
+        }
+    }
+    e = s2_all     ? (p.k2 == 9 ? launch_conv_stencil_s2_all_dz<3>(s2_all, p, stream)
                                            : launch_conv_stencil_s2_all_dz<2>(s2_all, p, stream))
                    : stencil  ? launch_conv_stencil<DZ>(stencil, p, stream)
                               : launch_tiles<P>(tile, p, stream);
@@ -830,7 +839,15 @@ hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float 
     if (g_conv2d_stencil && vec && ki == 3 && woho == wihi && fi % 8 == 0 && fo % 64 == 0 &&
         tile == TILE_64x128 && aligned16(mu_a) && aligned16(var_a))
         stencil = stencil_width(wihi);
-    if (vec) return run_sliced<ConvFwdProblem<true>, false>(tile, splits, stencil, ws0, ws1, p, stream);
+    // stride 2 on a square map, 3x3 with padding on the right and bottom or 2x2 (the
+    // kernel verifies the table)
+    int s2_fwd = 0;
+    if (g_conv2d_stencil && g_conv2d_s2_all && vec && (ki == 3 || ki == 2) && wihi == 4 * woho &&
+        fi % 8 == 0 && fo % 64 == 0 && tile == TILE_64x128 && aligned16(mu_a) && aligned16(var_a))
+        s2_fwd = s2_out_width(woho);
+    if (vec)
+        return run_sliced<ConvFwdProblem<true>, false>(tile, splits, stencil, ws0, ws1, p, stream, 0,
+                                                       s2_fwd);
     return run_sliced<ConvFwdProblem<false>, false>(tile, splits, 0, ws0, ws1, p, stream);
 }
 

@@ -458,6 +458,271 @@ inline hipError_t launch_conv_stencil_s2_all_dz(int wo, const ConvParams &p, hip
     return hipErrorInvalidValue;
 }
 
+// ---- forward ---------------------------------------------------------------------------
+// Output tile = 64 output channels x 128 output pixels = 128/WO whole output rows. The
+// input rows those pixels read (2*oy + ky) are staged once per channel with 16-byte
+// loads - 2*RPI + KS - 2 rows of 2*WO values per segment, plus one zero cell on the right
+// and, where the last row leaves the image, a zero row: the padding of the 3x3 kernel -
+// and tap (ky, kx) of a lane's pixel is the constant offset ky*RS + kx from the cell
+// (2*oy, 2*ox) when the MFMA operand is read. A k-tile is 4 channels x 9 taps or
+// 8 channels x 4 taps; lanes 0-31 / 32-63 of an MFMA step take the first / second half
+// of its channels at the same (channel, tap) position, the weights stay in memory order.
+template <int WO, int KS>
+struct S2FwdGeom {
+    static constexpr int W = WO, H = WO, WI = 2 * WO, T = KS * KS;
+    static constexpr int KC = KS == 3 ? 4 : 8;             // channels per k-tile
+    static constexpr int VPH = KC / 2 * T;                 // reduction steps per k-half
+    static constexpr int NR = 128 / W;                     // output rows per tile
+    static constexpr int RPI = NR < H ? NR : H;            // rows of one image among them
+    static constexpr int SEGS = NR / RPI;                  // images (segments) per tile
+    static constexpr int PR = 2 * RPI + KS - 2;            // staged input rows per segment
+    static constexpr int RS = WI + 4;                      // values, one zero cell, 3 unused
+    static constexpr int SEG = PR * RS;
+    static constexpr int CS = SEGS * SEG + 4;
+    static constexpr int PATCH = KC * CS;                  // floats per staged array
+    static constexpr int UNITS = KC * SEGS * PR * (WI / 4);  // 16-byte loads per array
+    static constexpr int P_SLOTS = (UNITS + 511) / 512;
+    static constexpr int AS = KC * T + (KC * T == 36 ? 8 : 12);  // 44: rows on distinct bank groups
+    static constexpr int A_VEC = 64 * KC * T / 4;          // 16-byte loads per weight array
+    static constexpr int A_SLOTS = (A_VEC + 511) / 512;
+    static constexpr int LDS_FLOATS = 2 * 64 * AS + 2 * PATCH;
+    static_assert(P_SLOTS <= 2 && A_SLOTS <= 2 && VPH % 2 == 0 && (KC * T) % 4 == 0, "staging slots");
+};
+
+// Expected Fmwa_2 entry (1-based input pixel, -1 = padding) of tap t of output pixel o.
+template <int WO, int KS>
+__device__ __forceinline__ int s2_fmwa(int o, int t) {
+    const int oy = o / WO, ox = o - oy * WO;
+    const int iy = 2 * oy + t / KS, ix = 2 * ox + t % KS;
+    return (iy < 2 * WO && ix < 2 * WO) ? iy * (2 * WO) + ix + 1 : -1;
+}
+
+// Does Fmwa_2 [woho][T] describe that stencil for the pixels n0 .. n0+127? Uniform verdict;
+// entries are requested in batches before any is looked at. `scratch`: one int of LDS.
+template <int WO, int KS>
+__device__ __forceinline__ bool s2_fwd_tables_ok(const ConvParams &p, int n0, int tid, int *scratch) {
+    constexpr int T = KS * KS, PAIRS = 128 * T, ITER = (PAIRS + 511) / 512;
+    if (tid == 0) *scratch = 1;
+    __syncthreads();
+    int got[ITER], want[ITER];
+#pragma unroll
+    for (int i = 0; i < ITER; i++) {
+        const int e = tid + i * 512, c = e / T, t = e - c * T, n = n0 + c;
+        const bool live = e < PAIRS && n < p.N;
+        const int o = live ? n % p.woho : 0;
+        got[i] = p.idx[live ? o * T + t : 0];
+        want[i] = live ? s2_fmwa<WO, KS>(o, t) : got[i];
+    }
+    bool ok = true;
+#pragma unroll
+    for (int i = 0; i < ITER; i++) ok = ok && got[i] == want[i];
+    if (!ok) *scratch = 0;
+    __syncthreads();
+    const bool verdict = __builtin_amdgcn_readfirstlane(*scratch) != 0;
+    __syncthreads();
+    return verdict;
+}
+
+// One 64 x 128 tile on a verified stencil. c_begin / c_end: input channels of the
+// reduction slice (multiples of KC).
+template <int WO, int KS>
+__device__ __forceinline__ void s2_fwd_body(const ConvParams &p, float *lds, int m0, int n0,
+                                            int split, int c_begin, int c_end) {
+    using G = S2FwdGeom<WO, KS>;
+    constexpr int W = WO, H = WO, WI = G::WI, NT = 512, KC = G::KC, T = G::T;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wrow = (wave / 4) * 32, wcol = (wave % 4) * 32, half = lane >> 5;
+    float *lds_a = lds;                      // [2 arrays][64 rows][AS]: KC*T values per row, memory order
+    float *lds_p = lds + 2 * 64 * G::AS;     // [PATCH][2]: (mu_a, var_a) interleaved
+
+    for (int i = tid; i < 2 * G::PATCH; i += NT) lds_p[i] = 0.f;
+
+    // patch units of this thread: channel pc, segment, staged row pr, columns 4*x4 ..
+    size_t punit[G::P_SLOTS];
+    int pdst[G::P_SLOTS];
+    bool p_ok[G::P_SLOTS];
+#pragma unroll
+    for (int i = 0; i < G::P_SLOTS; i++) {
+        int u = tid + i * NT;
+        const bool live = u < G::UNITS;
+        u = live ? u : 0;
+        const int x4 = u % (WI / 4);
+        u /= (WI / 4);
+        const int pr = u % G::PR;
+        u /= G::PR;
+        const int seg = u % G::SEGS, pc = u / G::SEGS;
+        const int grow = n0 / W + seg * G::RPI;  // first output row of the segment, over the batch
+        const int img = grow / H, y = 2 * (grow % H) + pr;
+        p_ok[i] = live && y < 2 * H && img < p.B;
+        punit[i] = p_ok[i] ? ((size_t)img * p.fi + c_begin + pc) * (WI * WI) + y * WI + 4 * x4 : 0;
+        pdst[i] = pc * G::CS + seg * G::SEG + pr * G::RS + 4 * x4;
+    }
+    const size_t pstep = (size_t)KC * (WI * WI);
+
+    // weight pieces of this thread: 16 bytes of w[m0 + row][c_begin*T + 4q ..]
+    size_t asrc[G::A_SLOTS];
+    int adst[G::A_SLOTS];
+    bool a_ok[G::A_SLOTS];
+#pragma unroll
+    for (int i = 0; i < G::A_SLOTS; i++) {
+        const int e = tid + i * NT;
+        a_ok[i] = e < G::A_VEC;
+        const int id = a_ok[i] ? e : 0;
+        const int row = id / (KC * T / 4), q = id - row * (KC * T / 4);
+        asrc[i] = (size_t)(m0 + row) * p.R + (size_t)c_begin * T + 4 * q;
+        adst[i] = row * G::AS + 4 * q;
+    }
+    const size_t astep = (size_t)KC * T;
+
+    floatx16 acc0[1][1], acc1[1][1];
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        acc0[0][0][v] = 0.f;
+        acc1[0][0][v] = 0.f;
+    }
+
+    // staging registers, named one by one (arrays of them end up in scratch memory)
+    float4 rm0, rm1, rv0, rv1, rpa0, rpa1, rpb0, rpb1;
+    rm0 = rm1 = rv0 = rv1 = rpa0 = rpa1 = rpb0 = rpb1 = make_float4(0.f, 0.f, 0.f, 0.f);
+#define TAGI_S2FWD_ALOAD(i)                                                           \
+    if (i < G::A_SLOTS) {                                                             \
+        rm##i = *reinterpret_cast<const float4 *>(p.w0 + asrc[i < G::A_SLOTS ? i : 0]); \
+        rv##i = *reinterpret_cast<const float4 *>(p.w1 + asrc[i < G::A_SLOTS ? i : 0]); \
+        if (a_ok[i < G::A_SLOTS ? i : 0]) asrc[i < G::A_SLOTS ? i : 0] += astep;      \
+    }
+#define TAGI_S2FWD_APUT(i)                                                            \
+    if (i < G::A_SLOTS && a_ok[i < G::A_SLOTS ? i : 0]) {                             \
+        *reinterpret_cast<float4 *>(lds_a + adst[i < G::A_SLOTS ? i : 0]) = rm##i;    \
+        *reinterpret_cast<float4 *>(lds_a + 64 * G::AS + adst[i < G::A_SLOTS ? i : 0]) = rv##i; \
+    }
+#define TAGI_S2FWD_PLOAD(i, A_, B_)                                                   \
+    if (i < G::P_SLOTS) {                                                             \
+        A_ = *reinterpret_cast<const float4 *>(p.a0 + punit[i < G::P_SLOTS ? i : 0]); \
+        B_ = *reinterpret_cast<const float4 *>(p.a1 + punit[i < G::P_SLOTS ? i : 0]); \
+        if (p_ok[i < G::P_SLOTS ? i : 0]) punit[i < G::P_SLOTS ? i : 0] += pstep;     \
+    }
+#define TAGI_S2FWD_PPUT(i, A_, B_)                                                    \
+    if (i < G::P_SLOTS && p_ok[i < G::P_SLOTS ? i : 0]) {                             \
+        float *dst_ = lds_p + 2 * pdst[i < G::P_SLOTS ? i : 0];                       \
+        *reinterpret_cast<float4 *>(dst_) = make_float4(A_.x, B_.x, A_.y, B_.y);      \
+        *reinterpret_cast<float4 *>(dst_ + 4) = make_float4(A_.z, B_.z, A_.w, B_.w);  \
+    }
+#define TAGI_S2FWD_FETCH()                                                            \
+    do {                                                                              \
+        TAGI_S2FWD_ALOAD(0) TAGI_S2FWD_ALOAD(1)                                       \
+        TAGI_S2FWD_PLOAD(0, rpa0, rpb0) TAGI_S2FWD_PLOAD(1, rpa1, rpb1)               \
+    } while (0)
+#define TAGI_S2FWD_COMMIT()                                                           \
+    do {                                                                              \
+        TAGI_S2FWD_APUT(0) TAGI_S2FWD_APUT(1)                                         \
+        TAGI_S2FWD_PPUT(0, rpa0, rpb0) TAGI_S2FWD_PPUT(1, rpa1, rpb1)                 \
+    } while (0)
+
+    // operand addresses of this lane: patch cell (2*oy, 2*ox) of its pixel in the first
+    // channel of its k-half; its row's values of that half
+    const int pix = wcol + (lane & 31), prow = pix / W, px = pix - prow * W;
+    const float *bp = lds_p + 2 * (half * (KC / 2) * G::CS + (prow / G::RPI) * G::SEG +
+                                   2 * (prow % G::RPI) * G::RS + 2 * px);
+    const float *a0 = lds_a + (wrow + (lane & 31)) * G::AS + half * G::VPH;
+    const float *a1 = a0 + 64 * G::AS;
+
+    __syncthreads();  // patch zeroed
+    if (c_begin < c_end) {
+        TAGI_S2FWD_FETCH();
+        TAGI_S2FWD_COMMIT();
+    }
+    __syncthreads();
+
+    for (int c0 = c_begin; c0 < c_end; c0 += KC) {
+        const bool more = c0 + KC < c_end;
+        if (more) TAGI_S2FWD_FETCH();
+#pragma unroll
+        for (int g = 0; g < G::VPH / 2; g++) {
+            const float2 am = *reinterpret_cast<const float2 *>(a0 + 2 * g);
+            const float2 av = *reinterpret_cast<const float2 *>(a1 + 2 * g);
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                const int s = 2 * g + e, ch = s / T, t = s - ch * T, ky = t / KS, kx = t - ky * KS;
+                const float2 y = *reinterpret_cast<const float2 *>(bp + 2 * (ch * G::CS + ky * G::RS + kx));
+                const float w = e ? am.y : am.x, wv = e ? av.y : av.x;
+                // mean: mu_w mu_a; variance: var_w (var_a + mu_a^2) + mu_w^2 var_a
+                acc0[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(w, y.x, acc0[0][0], 0, 0, 0);
+                acc1[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(wv, y.x * y.x + y.y, acc1[0][0], 0, 0, 0);
+                acc1[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(w * w, y.y, acc1[0][0], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+        if (more) {
+            TAGI_S2FWD_COMMIT();
+            __syncthreads();
+        }
+    }
+#undef TAGI_S2FWD_FETCH
+#undef TAGI_S2FWD_COMMIT
+#undef TAGI_S2FWD_ALOAD
+#undef TAGI_S2FWD_APUT
+#undef TAGI_S2FWD_PLOAD
+#undef TAGI_S2FWD_PPUT
+    tile_epilogue<ConvFwdProblem<true>, 64, 128, 2, 4>(p, acc0, acc1, m0, n0, split);
+}
+
+// One 64 x 128 tile per workgroup of 8 waves: verified stencil -> s2_fwd_body, anything
+// else -> the table-driven loop of the generic tile kernel.
+template <int WO, int KS>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4)))
+void conv_stencil_s2_fwd_kernel(ConvParams p) {
+    using G = S2FwdGeom<WO, KS>;
+    using P = ConvFwdProblem<true>;
+    constexpr int XF = TileGeom<P::XK, 64>::floats, YF = TileGeom<P::YK, 128>::floats;
+    constexpr int GENERIC = P::NX * XF + P::NY * YF;
+    __shared__ __attribute__((aligned(16))) float lds[GENERIC > G::LDS_FLOATS ? GENERIC : G::LDS_FLOATS];
+    extern __shared__ __attribute__((aligned(16))) int lds_extra[];
+
+    const int tiles_n = (p.N + 127) / 128;
+    const int tile = blockIdx.x, split = blockIdx.y;
+    const int m0 = (tile / tiles_n) * 64, n0 = (tile % tiles_n) * 128;
+    const int r_begin = split * p.r_per_split;
+    const int r_end = min(p.R, r_begin + p.r_per_split);
+
+    if (s2_fwd_tables_ok<WO, KS>(p, n0, threadIdx.x, lds_extra)) {
+        s2_fwd_body<WO, KS>(p, lds, m0, n0, split, r_begin / (KS * KS), r_end / (KS * KS));
+        return;
+    }
+    typename P::Ctx ctx;
+    P::prologue(p, ctx, lds_extra, threadIdx.x, 512, m0, n0, 64, 128, r_begin, r_end);
+    __syncthreads();
+    int r_lo = r_begin, r_hi = r_end;
+    P::adjust_range(p, ctx, r_lo, r_hi);
+    mfma_tile_body<P, 64, 128, 2, 4, 0>(p, ctx, reinterpret_cast<float (*)[XF]>(lds),
+                                        reinterpret_cast<float (*)[YF]>(lds + P::NX * XF), m0, n0,
+                                        split, r_lo, r_hi);
+}
+
+template <int KS>
+inline hipError_t launch_conv_stencil_s2_fwd(int wo, const ConvParams &p, hipStream_t stream) {
+    using P = ConvFwdProblem<true>;
+    const dim3 grid(((p.M + 63) / 64) * ((p.N + 127) / 128), p.splits);
+    const size_t extra = P::extra_lds_bytes(p, 64, 128);
+    if (extra > kTileExtraLdsMax) return hipErrorInvalidValue;
+#define TAGI_LAUNCH_S2FWD(WD)                                                                      \
+    case WD: {                                                                                     \
+        static PerDeviceOnce once;                                                                 \
+        hipError_t e = allow_dynamic_lds(                                                          \
+            once, reinterpret_cast<const void *>(conv_stencil_s2_fwd_kernel<WD, KS>),              \
+            (int)kTileExtraLdsMax);                                                                \
+        if (e != hipSuccess) return e;                                                             \
+        hipLaunchKernelGGL((conv_stencil_s2_fwd_kernel<WD, KS>), grid, dim3(512), extra, stream, p); \
+        return hipGetLastError();                                                                  \
+    }
+    switch (wo) {
+        TAGI_LAUNCH_S2FWD(4)
+        TAGI_LAUNCH_S2FWD(8)
+        TAGI_LAUNCH_S2FWD(16)
+    }
+#undef TAGI_LAUNCH_S2FWD
+    return hipErrorInvalidValue;
+}
+
 // Output map width for which the strided kernels exist, 0 otherwise.
 inline int s2_out_width(int out_pixels) {
     for (int w : {4, 8, 16})

@@ -35,6 +35,9 @@ GEOMS = [
     (3, 2, 1, 2, 16, 128, 96, 2),  # 8x8 output maps, two images per tile
     (3, 2, 1, 2, 8, 64, 160, 8),   # 4x4 output maps, eight images per tile
     (3, 2, 1, 2, 16, 64, 640, 2),  # long reduction: sliced
+    (3, 2, 1, 2, 32, 8, 64, 3),    # strided forward stencil only: 8 input channels, last tile partial... (3 x 256 pixels)
+    (3, 2, 1, 2, 8, 24, 64, 5),    # 4x4 output maps, 80 pixels: one partial tile
+    (2, 2, 0, 1, 16, 40, 128, 3),  # 2x2 forward stencil: 192 pixels, partial second tile
     # 2x2 s2 projections with whole groups of channels: the all-phase state backward
     (2, 2, 0, 1, 32, 64, 64, 1),
     (2, 2, 0, 1, 16, 128, 96, 2),
@@ -225,8 +228,35 @@ def test_conv2d_strided_stencil_kernels_agree_with_the_table_path():
         assert_close(a, b, name, same_sign=name in SAME_SIGN)
         if not np.array_equal(a, b):
             switched.append(name)
-    # a different summation order shows that the switch switched the state backward
-    assert "delta_mu_z" in switched
+    # a different summation order shows that the switch switched the forward and the
+    # state backward
+    assert "delta_mu_z" in switched and "mu_z" in switched
+
+
+@pytest.mark.parametrize("k,pad,pt", [(3, 1, 2), (2, 0, 1)])
+def test_conv2d_strided_forward_with_an_altered_table_takes_the_table_path(oracle_lib, k, pad, pt):
+    """The strided forward stencil is chosen by sizes and checks the table it is given.
+    One entry of Fmwa_2 is pointed at another input pixel: the tile that owns it runs the
+    table-driven loop, and the result is what the table says."""
+    import torch
+    import cutagi_amd.functional as F
+    from cutagi_amd import capi
+    wi, fi, fo, B = 16, 32, 64, 3
+    idx = capi.conv2d_build_idx(k, 2, wi, wi, pad, pt, k * k * fi * fo + 1)
+    wihi, woho = wi * wi, idx["wo"] * idx["ho"]
+    table = idx["Fmwa_2"].copy()
+    table[21 * k * k + 1] = 7          # output pixel 21, tap 1: reads input pixel 7 instead
+    d = conv_inputs(fi, fo, k, wihi, woho, B, seed=12, bias=True, jcb_random=True)
+    t = {n: (None if v is None else torch.from_numpy(v).cuda()) for n, v in d.items()}
+    z = F.conv2d_fwd(t["mu_w"], t["var_w"], t["mu_b"], t["var_b"], t["mu_a"], t["var_a"],
+                     torch.from_numpy(table).cuda(), woho, fo, wihi, fi, k, B)
+    ref = oracle_lib.conv2d_fwd(d["mu_w"], d["var_w"], d["mu_b"], d["var_b"], d["mu_a"], d["var_a"],
+                                table, woho, fo, wihi, fi, k, B, threads=4)
+    assert_close(z[0].cpu().numpy(), ref[0], "mu_z")
+    assert_close(z[1].cpu().numpy(), ref[1], "var_z", same_sign=True)
+    clean = oracle_lib.conv2d_fwd(d["mu_w"], d["var_w"], d["mu_b"], d["var_b"], d["mu_a"],
+                                  d["var_a"], idx["Fmwa_2"], woho, fo, wihi, fi, k, B, threads=4)
+    assert not np.array_equal(clean[0], ref[0])
 
 
 @pytest.mark.parametrize("geom", [(3, 2, 1, 2, 32, 64, 64, 1), (3, 2, 1, 2, 16, 128, 96, 2),
