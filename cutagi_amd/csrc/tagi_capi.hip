@@ -805,7 +805,9 @@ int tagi_conv2d_bwd_dw(const float *var_w, const float *var_b, const float *mu_a
     // (three full rounds of resident workgroups: a partly filled last round
     // costs as much time as a full one)
     const bool stencil = conv2d_bwd_dw_stencil(mu_a, delta_mu_out, delta_var_out, B, fo, woho, wihi,
-                                               fi, ki, tile) != 0;
+                                               fi, ki, tile) != 0 ||
+                         conv2d_bwd_dw_s2(mu_a, delta_mu_out, delta_var_out, B, fo, woho, wihi, fi,
+                                          ki, tile) != 0;
     int splits = g_tune.conv_dw_splits > 0 ? g_tune.conv_dw_splits
                  : stencil                 ? conv2d_bwd_dw_stencil_splits(out_tiles)
                                            : 3 * conv2d_bwd_dw_blocks_per_cu(tile) * num_cu() / out_tiles;

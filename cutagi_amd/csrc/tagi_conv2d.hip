@@ -931,6 +931,17 @@ int conv2d_bwd_dw_stencil(const float *mu_a, const float *dmu, const float *dvar
     return stencil_width(wihi);
 }
 
+// The same for the stride-2 layers (3x3 with padding on the right and bottom, 2x2 without):
+// output map width when the weight backward runs on their stencil kernel, 0 otherwise.
+int conv2d_bwd_dw_s2(const float *mu_a, const float *dmu, const float *dvar, int B, int fo,
+                     int woho, int wihi, int fi, int ki, int tile) {
+    if (!g_conv2d_stencil || !g_conv2d_s2_all || (ki != 3 && ki != 2) || wihi != 4 * woho ||
+        fi % 64 != 0 || fo % 64 != 0 || ((long long)B * woho) % 64 != 0 || tile != TILE_64x64 ||
+        !aligned16(mu_a) || !aligned16(dmu) || !aligned16(dvar))
+        return 0;
+    return s2_out_width(woho);
+}
+
 // Reduction slices for the stencil kernel (two 8-wave workgroups per CU): the
 // fewest rounds of resident workgroups that are at least 95 % full, else the
 // fullest of up to four rounds. A partly filled round costs as much as a full one.
@@ -962,12 +973,15 @@ hipError_t launch_conv2d_bwd_dw(const float *var_w, const float *mu_a, const flo
     p.M = fo; p.N = p.k2 * fi; p.R = B * woho;
     const bool vec = (woho % 4 == 0) && aligned16(dmu) && aligned16(dvar);
     const int stencil = conv2d_bwd_dw_stencil(mu_a, dmu, dvar, B, fo, woho, wihi, fi, ki, tile);
-    const int unit = stencil ? 64 : KT;
+    const int s2 = conv2d_bwd_dw_s2(mu_a, dmu, dvar, B, fo, woho, wihi, fi, ki, tile);
+    const int unit = (stencil || s2) ? 64 : KT;
     int per = ceil_div(ceil_div(p.R, splits), unit) * unit;
     p.splits = ceil_div(p.R, per);
     p.r_per_split = per;
     p.ws0 = ws0; p.ws1 = ws1;
     hipError_t e = stencil ? launch_conv_stencil_dw(stencil, p, stream)
+                   : s2    ? (ki == 3 ? launch_conv_stencil_s2_dw<3>(s2, p, stream)
+                                      : launch_conv_stencil_s2_dw<2>(s2, p, stream))
                    : vec   ? launch_tiles<ConvDwVecProblem>(tile, p, stream)
                            : launch_tiles<ConvDwProblem<false>>(tile, p, stream);
     if (e != hipSuccess) return e;

@@ -723,6 +723,257 @@ inline hipError_t launch_conv_stencil_s2_fwd(int wo, const ConvParams &p, hipStr
     return hipErrorInvalidValue;
 }
 
+// ---- weight backward -----------------------------------------------------------------------
+//   D[fo][(c,t)] = sum over (b, output pixel) of delta[b][fo][pixel] * a[b][c][2*pixel + tap t]
+// As the unit-stride kernel of tagi_conv_stencil.h: rows are output channels, the 64
+// columns of a tile are consecutive (channel, tap) pairs (8 channels of 9 taps or 16 of 4),
+// the reduction runs over output pixels 64 at a time = 64/WO whole output rows, whose input
+// rows are staged per k-tile (every cell rewritten, zero where a row leaves the image). A
+// lane's column fixes its (channel, tap) = one LDS base address; the pixel of a reduction
+// step is an immediate offset - here two cells per output pixel and two rows per output row.
+template <int WO, int KS>
+struct S2DwGeom {
+    static constexpr int W = WO, H = WO, WI = 2 * WO, T = KS * KS;
+    static constexpr int KP = 64;                          // output pixels per k-tile
+    static constexpr int KC = KS == 3 ? 8 : 16;            // channels a column tile can touch
+    static constexpr int NR = KP / W;                      // output rows per k-tile
+    static constexpr int RPI = NR < H ? NR : H;
+    static constexpr int SEGS = NR / RPI;
+    static constexpr int PR = 2 * RPI + KS - 2;            // staged input rows per segment
+    static constexpr int RS = WI + 4;                      // values, one zero cell, 3 unused
+    static constexpr int SEG = PR * RS;
+    static constexpr int CS = SEGS * SEG + 4;
+    static constexpr int PATCH = KC * CS;
+    static constexpr int UNITS = KC * SEGS * PR * (WI / 4);
+    static constexpr int P_SLOTS = (UNITS + 511) / 512;
+    static constexpr int AS = KP + 4;                      // innovation tile [64 rows][64 pixels + 4]
+    static constexpr int LOG_PIX = WO == 4 ? 4 : WO == 8 ? 6 : 8;
+    static_assert(P_SLOTS <= 2 && KP % W == 0 && NR % RPI == 0 && H % RPI == 0, "tile geometry");
+    // LDS offset of the cell (2*oy, 2*ox) of output pixel k (0..63) of the k-tile
+    static constexpr int pixel_offset(int k) {
+        return ((k / W) / RPI) * SEG + 2 * ((k / W) % RPI) * RS + 2 * (k % W);
+    }
+};
+
+template <int WO, int KS>
+__device__ __forceinline__ void s2_dw_body(const ConvParams &p, float *lds, int m0, int n0,
+                                           int split, int r_begin, int r_end) {
+    using G = S2DwGeom<WO, KS>;
+    constexpr int W = G::W, H = G::H, WI = G::WI, T = G::T, NT = 512, PIX = W * H, PIXI = WI * WI;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // eight waves: 2 x 2 sub-tiles of 32 x 32, each held by two waves that take the
+    // first / second 32 pixels of every k-tile and add up at the end
+    const int kgroup = wave >> 2;
+    const int wrow = ((wave & 3) / 2) * 32, wcol = (wave & 1) * 32, half = lane >> 5;
+    float *lds_a = lds;                        // [2][64][AS]
+    float *lds_p = lds + 2 * 64 * G::AS;       // [PATCH]
+    const int c_lo = n0 / T;                   // first channel of the column tile
+
+    for (int i = tid; i < G::PATCH; i += NT) lds_p[i] = 0.f;
+
+    // patch units: channel pc, segment, staged row pr, columns 4*x4 ... Output rows are
+    // counted over the whole batch; `grow` is the first output row of the k-tile.
+    int pseg[G::P_SLOTS], prw[G::P_SLOTS], pdst[G::P_SLOTS], pchan[G::P_SLOTS];
+    bool has_unit[G::P_SLOTS];
+#pragma unroll
+    for (int i = 0; i < G::P_SLOTS; i++) {
+        int u = tid + i * NT;
+        has_unit[i] = u < G::UNITS;
+        u = has_unit[i] ? u : 0;
+        const int x4 = u % (WI / 4);
+        u /= (WI / 4);
+        prw[i] = u % G::PR;
+        u /= G::PR;
+        pseg[i] = u % G::SEGS;
+        const int pc = u / G::SEGS;
+        // channels past the layer's last one (a partial last column tile) are never read
+        has_unit[i] = has_unit[i] && c_lo + pc < p.fi;
+        pdst[i] = pc * G::CS + pseg[i] * G::SEG + prw[i] * G::RS + 4 * x4;
+        pchan[i] = (c_lo + (has_unit[i] ? pc : 0)) * PIXI + 4 * x4;
+    }
+    int grow = r_begin / W;
+
+    // innovation pieces: 16 bytes at pixel 4*q of rows tid/16 + 32*i
+    const int q = tid % 16, arow = tid / 16;
+    int gpix = r_begin + 4 * q;  // output pixel counted over the whole batch
+
+    floatx16 acc0[1][1], acc1[1][1];
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        acc0[0][0][v] = 0.f;
+        acc1[0][0][v] = 0.f;
+    }
+
+    float4 ra00, ra01, ra10, ra11, rp0, rp1;
+    rp0 = rp1 = make_float4(0.f, 0.f, 0.f, 0.f);
+    bool rp_ok0 = false, rp_ok1 = false;
+#define TAGI_S2DW_PLOAD(i, R_, OK_)                                                        \
+    if (i < G::P_SLOTS) {                                                                  \
+        const int j_ = i < G::P_SLOTS ? i : 0;                                             \
+        const int g_ = grow + pseg[j_] * G::RPI, img_ = g_ / H, y_ = 2 * (g_ - img_ * H) + prw[j_]; \
+        OK_ = has_unit[j_] && y_ < 2 * H && img_ < p.B;                                    \
+        R_ = *reinterpret_cast<const float4 *>(                                            \
+            p.a0 + (OK_ ? (size_t)img_ * p.fi * PIXI + pchan[j_] + y_ * WI : 0));          \
+    }
+#define TAGI_S2DW_PPUT(i, R_, OK_)                                                         \
+    if (i < G::P_SLOTS && has_unit[i < G::P_SLOTS ? i : 0])                                \
+        *reinterpret_cast<float4 *>(lds_p + pdst[i < G::P_SLOTS ? i : 0]) =                \
+            OK_ ? R_ : make_float4(0.f, 0.f, 0.f, 0.f);
+#define TAGI_S2DW_FETCH()                                                                  \
+    do {                                                                                   \
+        const int b_ = gpix >> G::LOG_PIX, o_ = gpix & (PIX - 1);                          \
+        const size_t at_ = ((size_t)b_ * p.fo + m0 + arow) * PIX + o_;                     \
+        ra00 = *reinterpret_cast<const float4 *>(p.d0 + at_);                              \
+        ra10 = *reinterpret_cast<const float4 *>(p.d1 + at_);                              \
+        ra01 = *reinterpret_cast<const float4 *>(p.d0 + at_ + (size_t)32 * PIX);           \
+        ra11 = *reinterpret_cast<const float4 *>(p.d1 + at_ + (size_t)32 * PIX);           \
+        gpix += G::KP;                                                                     \
+        TAGI_S2DW_PLOAD(0, rp0, rp_ok0) TAGI_S2DW_PLOAD(1, rp1, rp_ok1)                    \
+        grow += G::NR;                                                                     \
+    } while (0)
+#define TAGI_S2DW_COMMIT()                                                                 \
+    do {                                                                                   \
+        float *d0_ = lds_a + arow * G::AS + 4 * q, *d1_ = d0_ + 64 * G::AS;                \
+        *reinterpret_cast<float4 *>(d0_) = ra00;                                           \
+        *reinterpret_cast<float4 *>(d0_ + 32 * G::AS) = ra01;                              \
+        *reinterpret_cast<float4 *>(d1_) = ra10;                                           \
+        *reinterpret_cast<float4 *>(d1_ + 32 * G::AS) = ra11;                              \
+        TAGI_S2DW_PPUT(0, rp0, rp_ok0) TAGI_S2DW_PPUT(1, rp1, rp_ok1)                      \
+    } while (0)
+
+    // operand addresses of this lane: its column is (channel, tap)
+    const int n = min(n0 + wcol + (lane & 31), p.N - 1);
+    const int ch = n / T - c_lo, t = n - (n / T) * T, ky = t / KS, kx = t - ky * KS;
+    const float *bp = lds_p + ch * G::CS + ky * G::RS + kx + (half ? G::pixel_offset(4) : 0) +
+                      (kgroup ? G::pixel_offset(32) : 0);
+    const float *a0 = lds_a + (wrow + (lane & 31)) * G::AS + 4 * half + 32 * kgroup;
+    const float *a1 = a0 + 64 * G::AS;
+
+    __syncthreads();  // patch zeroed
+    if (r_begin < r_end) {
+        TAGI_S2DW_FETCH();
+        TAGI_S2DW_COMMIT();
+    }
+    __syncthreads();
+
+    for (int r0 = r_begin; r0 < r_end; r0 += G::KP) {
+        const bool more = r0 + G::KP < r_end;
+        if (more) TAGI_S2DW_FETCH();
+#pragma unroll
+        for (int kk = 0; kk < G::KP / 2; kk += 8) {
+            const float4 dm = *reinterpret_cast<const float4 *>(a0 + kk);
+            const float4 dv = *reinterpret_cast<const float4 *>(a1 + kk);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float y = bp[G::pixel_offset(kk + e)];
+                acc0[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(comp4(dm, e), y, acc0[0][0], 0, 0, 0);
+                acc1[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(comp4(dv, e), y * y, acc1[0][0], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+        if (more) {
+            TAGI_S2DW_COMMIT();
+            __syncthreads();
+        }
+    }
+#undef TAGI_S2DW_FETCH
+#undef TAGI_S2DW_COMMIT
+#undef TAGI_S2DW_PLOAD
+#undef TAGI_S2DW_PPUT
+
+    // the second pixel group hands its sums over through LDS ([value][lane] layout)
+    float *xch = lds;
+    if (kgroup == 1) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            xch[v * 256 + (tid - 256)] = acc0[0][0][v];
+            xch[(16 + v) * 256 + (tid - 256)] = acc1[0][0][v];
+        }
+    }
+    __syncthreads();
+    if (kgroup == 1) return;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        acc0[0][0][v] += xch[v * 256 + tid];
+        acc1[0][0][v] += xch[(16 + v) * 256 + tid];
+    }
+    tile_epilogue<ConvDwVecProblem, 64, 64, 2, 2>(p, acc0, acc1, m0, n0, split);
+}
+
+template <int WO, int KS>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4)))
+void conv_stencil_s2_dw_kernel(ConvParams p) {
+    using G = S2DwGeom<WO, KS>;
+    using P = ConvDwVecProblem;
+    constexpr int T = KS * KS;
+    constexpr int XF = TileGeom<P::XK, 64>::floats, YF = TileGeom<P::YK, 64>::floats;
+    constexpr int GENERIC = P::NX * XF + P::NY * YF;
+    constexpr int STENCIL = 2 * 64 * G::AS + G::PATCH;
+    static_assert(2 * 64 * G::AS >= 32 * 256, "the innovation tiles hold the final exchange");
+    __shared__ __attribute__((aligned(16))) float lds[GENERIC > STENCIL ? GENERIC : STENCIL];
+    __shared__ int regular_flag;
+
+    const int tiles_n = (p.N + 63) / 64;
+    int tile = blockIdx.x, split = blockIdx.y;
+    if (gridDim.y % 8 == 0) {
+        // all column tiles of one reduction slice on one XCD (see mfma_tile_kernel)
+        const int id = blockIdx.y * gridDim.x + blockIdx.x;
+        const int qq = id >> 3;
+        tile = qq % gridDim.x;
+        split = (qq / gridDim.x) * 8 + (id & 7);
+    }
+    const int m0 = (tile / tiles_n) * 64, n0 = (tile % tiles_n) * 64;
+    const int r_begin = split * p.r_per_split;
+    const int r_end = min(p.R, r_begin + p.r_per_split);
+
+    // the output pixels of this slice, per image position: all of Fmwa_2 once the slice is
+    // as long as a map; entries are requested six at a time before any is looked at
+    if (threadIdx.x == 0) regular_flag = 1;
+    __syncthreads();
+    {
+        const int total = min(max(r_end - r_begin, 0), p.woho) * T;
+        bool ok = true;
+        for (int base = threadIdx.x; base < total; base += 6 * 512) {
+            int got[6], want[6];
+#pragma unroll
+            for (int i = 0; i < 6; i++) {
+                const int e = base + i * 512, c = e / T, t = e - c * T;
+                const bool live = e < total;
+                const int o = live ? (r_begin + c) & (WO * WO - 1) : 0;
+                got[i] = p.idx[live ? o * T + t : 0];
+                want[i] = live ? s2_fmwa<WO, KS>(o, t) : got[i];
+            }
+#pragma unroll
+            for (int i = 0; i < 6; i++) ok = ok && got[i] == want[i];
+        }
+        if (!ok) regular_flag = 0;
+    }
+    __syncthreads();
+    if (__builtin_amdgcn_readfirstlane(regular_flag)) {
+        s2_dw_body<WO, KS>(p, lds, m0, n0, split, r_begin, r_end);
+        return;
+    }
+    // table-driven loop: written for four waves; the other four leave
+    if (threadIdx.x >= 256) return;
+    typename P::Ctx ctx;
+    P::prologue(p, ctx, nullptr, threadIdx.x, 256, m0, n0, 64, 64, r_begin, r_end);
+    mfma_tile_body<P, 64, 64, 2, 2, 0>(p, ctx, reinterpret_cast<float (*)[XF]>(lds),
+                                       reinterpret_cast<float (*)[YF]>(lds + P::NX * XF), m0, n0,
+                                       split, r_begin, r_end);
+}
+
+template <int KS>
+inline hipError_t launch_conv_stencil_s2_dw(int wo, const ConvParams &p, hipStream_t stream) {
+    const dim3 grid(((p.M + 63) / 64) * ((p.N + 63) / 64), p.splits);
+    switch (wo) {
+        case 4: hipLaunchKernelGGL((conv_stencil_s2_dw_kernel<4, KS>), grid, dim3(512), 0, stream, p); break;
+        case 8: hipLaunchKernelGGL((conv_stencil_s2_dw_kernel<8, KS>), grid, dim3(512), 0, stream, p); break;
+        case 16: hipLaunchKernelGGL((conv_stencil_s2_dw_kernel<16, KS>), grid, dim3(512), 0, stream, p); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 // Output map width for which the strided kernels exist, 0 otherwise.
 inline int s2_out_width(int out_pixels) {
     for (int w : {4, 8, 16})

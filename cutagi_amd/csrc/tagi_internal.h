@@ -271,6 +271,8 @@ int conv2d_bwd_dw_blocks_per_cu(int tile);
 int conv2d_bwd_dw_stencil(const float *mu_a, const float *dmu, const float *dvar, int B, int fo,
                           int woho, int wihi, int fi, int ki, int tile);
 int conv2d_bwd_dw_stencil_splits(int out_tiles);
+int conv2d_bwd_dw_s2(const float *mu_a, const float *dmu, const float *dvar, int B, int fo,
+                     int woho, int wihi, int fi, int ki, int tile);
 hipError_t launch_conv2d_bwd_dw(const float *var_w, const float *mu_a, const float *dmu,
                                 const float *dvar, const int *aidx, int B, int fo, int woho,
                                 int wihi, int fi, int ki, int tile, int splits, float *ws0, float *ws1,

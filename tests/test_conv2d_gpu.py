@@ -228,9 +228,41 @@ def test_conv2d_strided_stencil_kernels_agree_with_the_table_path():
         assert_close(a, b, name, same_sign=name in SAME_SIGN)
         if not np.array_equal(a, b):
             switched.append(name)
-    # a different summation order shows that the switch switched the forward and the
-    # state backward
-    assert "delta_mu_z" in switched and "mu_z" in switched
+    # a different summation order shows that the switch switched all three passes
+    assert "delta_mu_z" in switched and "mu_z" in switched and "delta_mu_w" in switched
+
+
+@pytest.mark.parametrize("k,pad,pt", [(3, 1, 2), (2, 0, 1)])
+def test_conv2d_strided_weight_backward_with_an_altered_table_takes_the_table_path(oracle_lib, k,
+                                                                                   pad, pt):
+    """The same for the weight backward (64 input and output channels, whole 64-pixel
+    k-tiles): with one entry of Fmwa_2 altered, the slices that see it run the
+    table-driven loop; with the table intact the stencil kernel gives the oracle's result
+    in another summation order than the table-driven kernel."""
+    import torch
+    import cutagi_amd.functional as F
+    from cutagi_amd import capi
+    wi, fi, fo, B = 16, 64, 64, 3
+    idx = capi.conv2d_build_idx(k, 2, wi, wi, pad, pt, k * k * fi * fo + 1)
+    wihi, woho = wi * wi, idx["wo"] * idx["ho"]
+    table = idx["Fmwa_2"].copy()
+    table[21 * k * k + 1] = 7
+    d = conv_inputs(fi, fo, k, wihi, woho, B, seed=13, bias=True, jcb_random=True)
+    t = {n: (None if v is None else torch.from_numpy(v).cuda()) for n, v in d.items()}
+    for tab in (table, idx["Fmwa_2"]):
+        dw = F.conv2d_bwd_dw(t["var_w"], t["var_b"], t["mu_a"], t["delta_mu"], t["delta_var"],
+                             torch.from_numpy(tab).cuda(), B, fo, woho, wihi, fi, k)
+        ref = oracle_lib.conv2d_bwd_dw(d["var_w"], d["var_b"], d["mu_a"], d["delta_mu"],
+                                       d["delta_var"], tab, B, fo, woho, wihi, fi, k, threads=4)
+        assert_close(dw[0].cpu().numpy(), ref[0], "delta_mu_w")
+        assert_close(dw[1].cpu().numpy(), ref[1], "delta_var_w", same_sign=True)
+    capi.tune("conv2d.stencil", 0)
+    try:
+        off = F.conv2d_bwd_dw(t["var_w"], t["var_b"], t["mu_a"], t["delta_mu"], t["delta_var"],
+                              torch.from_numpy(idx["Fmwa_2"]).cuda(), B, fo, woho, wihi, fi, k)
+    finally:
+        capi.tune("conv2d.stencil", 1)
+    assert not np.array_equal(off[0].cpu().numpy(), dw[0].cpu().numpy())
 
 
 @pytest.mark.parametrize("k,pad,pt", [(3, 1, 2), (2, 0, 1)])
