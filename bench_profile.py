@@ -264,9 +264,9 @@ def resnet(raw, out, stamp):
     steps = len(agg["avgpool_fwd_kernel"])
     total = sum(sum(v) for v in agg.values())
     groups = collections.OrderedDict([
-        ("Conv2d, regular-stencil kernels (3x3 stride 1; state backward of 3x3 stride 2)", lambda k: k.startswith("conv_stencil")),
-        ("Conv2d, table-driven tile kernels (strided 3x3 forward / weight backward, 2x2 projections, stem)",
-         lambda k: k.startswith("mfma_tile_kernel<Conv")),
+        ("Conv2d, regular-stencil kernels, 3x3 stride 1", lambda k: k.startswith("conv_stencil") and "_s2_" not in k),
+        ("Conv2d, regular-stencil kernels, stride 2 (3x3 and the 2x2 projections)", lambda k: k.startswith("conv_stencil_s2")),
+        ("Conv2d, table-driven tile kernels (the 3-channel stem)", lambda k: k.startswith("mfma_tile_kernel<Conv")),
         ("BatchNorm2d passes", lambda k: k.startswith("bn_")),
         ("folds of sliced reductions", lambda k: k.startswith("reduce_")),
     ])
@@ -287,7 +287,7 @@ def resnet(raw, out, stamp):
         f.write("| everything else (residual / pooling / Linear head / update / transfers) | %.3f | %.1f |\n\n"
                 % (rest / 1e6 / steps, rest / total * 100))
         f.write("| kernel | calls per step | avg us | ms per step | % of kernel time |\n|---|---|---|---|---|\n")
-        for k, v in sorted(agg.items(), key=lambda kv: -sum(kv[1]))[:34]:
+        for k, v in sorted(agg.items(), key=lambda kv: -sum(kv[1]))[:46]:
             f.write("| `%s` | %.1f | %.1f | %.3f | %.1f |\n" % (
                 k[:100], len(v) / steps, sum(v) / len(v) / 1e3, sum(v) / 1e6 / steps, sum(v) / total * 100))
     print("wrote resnet18_cifar_step_kernel_stats.md")
