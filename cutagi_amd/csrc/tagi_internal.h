@@ -251,7 +251,7 @@ extern int g_conv2d_group_loads;
 extern int g_conv2d_stencil;
 // 0 keeps the natural column order in the conv2d state backward of strided layers.
 extern int g_conv2d_phase_order;
-extern int g_conv2d_s2_all;   // 0: no all-phase kernel for the strided state backward
+extern int g_conv2d_s2_all;   // 0: no stencil kernels for the stride-2 layers
 int conv2d_bwd_dz_s2_all(const float *mu_w, const float *dmu, const float *dvar, int B, int fo,
                          int woho, int wihi, int fi, int ki, int nr);
 int conv2d_bwd_dz_s2_all_splits(int B, int fo, int woho, int fi);

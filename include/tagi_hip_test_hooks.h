@@ -30,7 +30,9 @@ extern "C" {
  * one-launch forward for small layers). Conv2d: "conv2d.tile",
  * "conv2d.splits", "conv2d.dw.tile", "conv2d.dw.splits", "conv2d.group_loads",
  * "conv2d.stencil", "conv2d.phase_order", "conv2d.s2_all" (0 switches the named path
- * off; s2_all: the stride-2 state backward that keeps all four phases in one workgroup). */
+ * off; s2_all: the stencil kernels of the stride-2 layers - forward, state backward with
+ * all four phases in one workgroup and its pair-wise fold, weight backward - which leaves
+ * those layers on the table-driven kernels). */
 int tagi_hip_tune(const char *key /* host */, int value);
 
 #ifdef __cplusplus
