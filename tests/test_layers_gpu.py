@@ -31,6 +31,41 @@ def test_mixture_relu(oracle_lib):
     assert got.min() >= floor and mu_a.cpu().numpy().min() >= floor
 
 
+def test_mixture_relu_distribution_function_in_the_tails():
+    """The activation computes the normal density and distribution function from one
+    exponential and a fitted Mills ratio. The Jacobian it returns IS the distribution
+    function: elementwise relative error against float64 (scipy) from alpha = -9 to 9,
+    where Phi spans 1e-19 .. 1 - the rms-normalised parity metric above would not see a
+    wrong tail - and the first moment against its float64 closed form where that is not
+    a difference of nearly equal terms (alpha >= -2)."""
+    import torch
+    from scipy.stats import norm
+    import cutagi_amd.functional as F
+    alpha = np.linspace(-9.0, 9.0, 360001)
+    sd = np.float32(0.75)
+    mu = (alpha * float(sd)).astype(np.float32)
+    var = np.full_like(mu, sd * sd)
+    mu_a, var_a, jcb = F.mixture_relu_fwd(torch.from_numpy(mu).cuda(), torch.from_numpy(var).cuda())
+    a64 = mu.astype(np.float64) / np.sqrt(var.astype(np.float64))     # what the kernel was given
+    want = norm.cdf(a64)
+    rel = np.abs(jcb.cpu().numpy().astype(np.float64) / want - 1.0)
+    # fp32: alpha carries 6e-8 of rounding, which the tail amplifies by about alpha^2
+    assert rel.max() <= 2e-5, rel.max()
+    assert rel[np.abs(a64) <= 3].max() <= 2e-6
+    keep = a64 >= -2.0
+    s64 = np.sqrt(var.astype(np.float64))
+    first = mu.astype(np.float64) * want + s64 * norm.pdf(a64)
+    rel1 = np.abs(mu_a.cpu().numpy().astype(np.float64)[keep] / first[keep] - 1.0)
+    assert rel1.max() <= 5e-6, rel1.max()
+    # degenerate inputs: zero variance (alpha = +-inf) and huge |alpha|
+    m = np.array([2.0, -2.0, 1e4, -1e4, 0.5], np.float32)
+    v = np.array([0.0, 0.0, 1e-6, 1e-6, 1e-30], np.float32)
+    o = [x.cpu().numpy() for x in F.mixture_relu_fwd(torch.from_numpy(m).cuda(), torch.from_numpy(v).cuda())]
+    np.testing.assert_allclose(o[0], [2.0, 1e-6, 1e4, 1e-6, 0.5], rtol=1e-6)
+    np.testing.assert_allclose(o[2], [1.0, 0.0, 1.0, 0.0, 1.0], atol=1e-30)
+    assert np.all(o[1] >= 1e-6) and np.all(np.isfinite(o[1]))
+
+
 # (wihi, fi, B): feature maps of the ResNet-18 configuration scaled down in
 # batch, odd sizes, one sample per chunk, and the fully-connected form (wihi = 1)
 BN_SHAPES = [(1024, 64, 4), (256, 128, 3), (16, 512, 8), (49, 5, 7), (1, 300, 16), (9, 3, 2),
