@@ -21,7 +21,7 @@ static __device__ __align__(256) float scratch[STATIC_SCRATCH_BYTES / sizeof(flo
 
 namespace {
 
-constexpr int ABI_VERSION = 104;
+constexpr int ABI_VERSION = 105;
 
 #define TAGI_TRY(expr)                          \
     do {                                        \
@@ -328,6 +328,7 @@ int tagi_hip_tune(const char *key, int value) {
     else if (!strcmp(key, "conv2d.stencil")) g_conv2d_stencil = value;
     else if (!strcmp(key, "conv2d.phase_order")) g_conv2d_phase_order = value;
     else if (!strcmp(key, "conv2d.s2_all")) g_conv2d_s2_all = value < 0 ? 1 : value;
+    else if (!strcmp(key, "conv2d.bwd_pair")) g_conv2d_bwd_pair = value < 0 ? 1 : value;
     else if (!strcmp(key, "linear.tile")) g_tune.tile = value;
     else if (!strcmp(key, "linear.double_buffer")) g_gemm_double_buffer = value < 0 ? 1 : value;
     else if (!strcmp(key, "conv2d.dw.splits")) g_tune.conv_dw_splits = value;
@@ -825,6 +826,66 @@ int tagi_conv2d_bwd_dw(const float *var_w, const float *var_b, const float *mu_a
         TAGI_TRY(launch_conv2d_bwd_db(var_b, delta_mu_out, delta_var_out, B, fo, woho, chunks,
                                       ws + 2 * part, delta_mu_b, delta_var_b, stream));
     }
+    return TAGI_OK;
+}
+
+int tagi_conv2d_bwd(const float *mu_w, const float *var_w, const float *var_b, const float *mu_a,
+                    const float *jcb, const float *delta_mu_out, const float *delta_var_out,
+                    const int *aidx, const int *zw_idx, const int *zud_idx, int B, int fo, int woho,
+                    int wihi, int fi, int ki, int nr, int bias, int state_update, int param_update,
+                    const float *res_mu, const float *res_var, int res_mode, float *delta_mu,
+                    float *delta_var, float *delta_mu_w, float *delta_var_w, float *delta_mu_b,
+                    float *delta_var_b, void *stream_) {
+    if (res_mu != nullptr && (!res_var || (res_mode != 1 && res_mode != 2) || !state_update))
+        return TAGI_ERR_INVALID_ARG;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const bool both = state_update && param_update && mu_w && var_w && mu_a && jcb && delta_mu_out &&
+                      delta_var_out && aidx && zw_idx && zud_idx && delta_mu && delta_var &&
+                      delta_mu_w && delta_var_w && B > 0 && fo > 0 && woho > 0 && wihi > 0 && fi > 0 &&
+                      ki > 0 && nr > 0 && (!bias || (var_b && delta_mu_b && delta_var_b)) &&
+                      conv_sizes_ok(B, fo, woho, fi, wihi, ki) && g_tune.conv_tile < 0 &&
+                      g_tune.conv_dw_tile < 0;
+    if (both && conv2d_bwd_pair(mu_w, mu_a, delta_mu_out, delta_var_out, B, fo, woho, wihi, fi, ki, nr)) {
+        // both contractions on their stencil kernels: one launch for the two tile grids
+        int tile_z = 0, splits_z = 1;
+        conv2d_plan(fi, B * wihi, ki * ki * fo, &tile_z, &splits_z);
+        if (g_tune.conv_splits > 0) splits_z = g_tune.conv_splits;
+        const int out_tiles = ceil_div(fo, 64) * ceil_div(ki * ki * fi, 64);
+        int splits_w = g_tune.conv_dw_splits > 0 ? g_tune.conv_dw_splits
+                                                 : conv2d_bwd_dw_stencil_splits(out_tiles);
+        const int max_splits = ceil_div(B * woho, 256);
+        if (splits_w > max_splits) splits_w = max_splits;
+        if (splits_w < 1) splits_w = 1;
+        if (tile_z == 1) {  // 64 x 128, the tile of the state-backward stencil
+            const size_t part_z = splits_z > 1 ? (size_t)splits_z * fi * B * wihi : 0;
+            const size_t part_w = (size_t)splits_w * fo * ki * ki * fi;
+            const int chunks = 64;  // slices of the (b, o) range in the bias reduction
+            float *ws = nullptr;
+            int rc = workspace_get((2 * part_z + 2 * part_w + 2 * (size_t)chunks * fo) * sizeof(float),
+                                   stream, &ws);
+            if (rc != TAGI_OK) return rc;
+            float *wz = ws, *ww = ws + 2 * part_z;
+            TAGI_TRY(launch_conv2d_bwd_pair(mu_w, var_w, mu_a, jcb, delta_mu_out, delta_var_out, aidx,
+                                            zw_idx, zud_idx, B, fo, woho, wihi, fi, ki, nr, splits_z,
+                                            wz, wz + part_z, splits_w, ww, ww + part_w, res_mu,
+                                            res_var, res_mode, delta_mu, delta_var, delta_mu_w,
+                                            delta_var_w, stream));
+            if (bias)
+                TAGI_TRY(launch_conv2d_bwd_db(var_b, delta_mu_out, delta_var_out, B, fo, woho, chunks,
+                                              ww + 2 * part_w, delta_mu_b, delta_var_b, stream));
+            return TAGI_OK;
+        }
+    }
+    if (param_update) {
+        int rc = tagi_conv2d_bwd_dw(var_w, var_b, mu_a, delta_mu_out, delta_var_out, aidx, B, fo, woho,
+                                    wihi, fi, ki, bias, delta_mu_w, delta_var_w, delta_mu_b,
+                                    delta_var_b, stream_);
+        if (rc != TAGI_OK) return rc;
+    }
+    if (state_update)
+        return conv2d_bwd_dz_impl(mu_w, jcb, delta_mu_out, delta_var_out, zw_idx, zud_idx, woho, fo,
+                                  wihi, fi, ki, nr, B, delta_mu, delta_var, stream_, res_mu, res_var,
+                                  res_mode);
     return TAGI_OK;
 }
 

@@ -851,12 +851,14 @@ hipError_t launch_conv2d_fwd(const float *mu_w, const float *var_w, const float 
     return run_sliced<ConvFwdProblem<false>, false>(tile, splits, 0, ws0, ws1, p, stream);
 }
 
-hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *dmu,
-                                const float *dvar, const int *zw_idx, const int *zud_idx,
-                                int woho, int fo, int wihi, int fi, int ki, int nr, int B,
-                                int tile, int splits, float *ws0, float *ws1, float *out_dmu,
-                                float *out_dvar, hipStream_t stream, const float *res_mu,
-                                const float *res_var, int res_mode) {
+namespace {
+// Problem description of the state backward; *stencil / *s2_all: map width when the
+// unit-stride / stride-2 stencil kernel applies, 0 otherwise.
+ConvParams dz_params(const float *mu_w, const float *jcb, const float *dmu, const float *dvar,
+                     const int *zw_idx, const int *zud_idx, int woho, int fo, int wihi, int fi,
+                     int ki, int nr, int B, int tile, float *out_dmu, float *out_dvar,
+                     const float *res_mu, const float *res_var, int res_mode, int *stencil,
+                     int *s2_all) {
     const int k2 = ki * ki;
     ConvParams p = {};
     p.res0 = res_mu; p.res1 = res_var; p.res_mode = res_mu != nullptr ? res_mode : 0;
@@ -877,14 +879,36 @@ hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float
             p.perm_w = w;
         }
     }
-    int stencil = 0;
+    *stencil = 0;
     if (g_conv2d_stencil && ki == 3 && nr == 9 && woho == wihi && fo % 8 == 0 && fi % 64 == 0 &&
         tile == TILE_64x128 && aligned16(mu_w) && aligned16(dmu) && aligned16(dvar))
-        stencil = stencil_width(wihi);
+        *stencil = stencil_width(wihi);
     // stride 2, 3x3 with padding on the right and bottom or 2x2 (the kernel verifies the tables)
-    const int s2_all = (p.perm_s == 2 && tile == TILE_64x128)
-                           ? conv2d_bwd_dz_s2_all(mu_w, dmu, dvar, B, fo, woho, wihi, fi, ki, nr)
-                           : 0;
+    *s2_all = (p.perm_s == 2 && tile == TILE_64x128)
+                  ? conv2d_bwd_dz_s2_all(mu_w, dmu, dvar, B, fo, woho, wihi, fi, ki, nr)
+                  : 0;
+    return p;
+}
+
+// Reduction slices of a launch: whole `unit`s per slice.
+void plan_slices(ConvParams &p, int splits, int unit, float *ws0, float *ws1) {
+    const int per = ceil_div(ceil_div(p.R, splits), unit) * unit;
+    p.splits = ceil_div(p.R, per);
+    p.r_per_split = per;
+    p.ws0 = ws0;
+    p.ws1 = ws1;
+}
+}  // namespace
+
+hipError_t launch_conv2d_bwd_dz(const float *mu_w, const float *jcb, const float *dmu,
+                                const float *dvar, const int *zw_idx, const int *zud_idx,
+                                int woho, int fo, int wihi, int fi, int ki, int nr, int B,
+                                int tile, int splits, float *ws0, float *ws1, float *out_dmu,
+                                float *out_dvar, hipStream_t stream, const float *res_mu,
+                                const float *res_var, int res_mode) {
+    int stencil = 0, s2_all = 0;
+    ConvParams p = dz_params(mu_w, jcb, dmu, dvar, zw_idx, zud_idx, woho, fo, wihi, fi, ki, nr, B,
+                             tile, out_dmu, out_dvar, res_mu, res_var, res_mode, &stencil, &s2_all);
     return run_sliced<ConvDzProblem, true>(tile, splits, stencil, ws0, ws1, p, stream, s2_all);
 }
 
@@ -962,23 +986,28 @@ int conv2d_bwd_dw_stencil_splits(int out_tiles) {
     return best;
 }
 
-hipError_t launch_conv2d_bwd_dw(const float *var_w, const float *mu_a, const float *dmu,
-                                const float *dvar, const int *aidx, int B, int fo, int woho,
-                                int wihi, int fi, int ki, int tile, int splits, float *ws0, float *ws1,
-                                float *dmu_w, float *dvar_w, hipStream_t stream) {
+namespace {
+ConvParams dw_params(const float *var_w, const float *mu_a, const float *dmu, const float *dvar,
+                     const int *aidx, int B, int fo, int woho, int wihi, int fi, int ki,
+                     float *dmu_w, float *dvar_w) {
     ConvParams p = {};
     p.a0 = mu_a; p.d0 = dmu; p.d1 = dvar; p.e0 = var_w; p.idx = aidx;
     p.out0 = dmu_w; p.out1 = dvar_w;
     p.woho = woho; p.fo = fo; p.wihi = wihi; p.fi = fi; p.k2 = ki * ki; p.B = B;
     p.M = fo; p.N = p.k2 * fi; p.R = B * woho;
+    return p;
+}
+}  // namespace
+
+hipError_t launch_conv2d_bwd_dw(const float *var_w, const float *mu_a, const float *dmu,
+                                const float *dvar, const int *aidx, int B, int fo, int woho,
+                                int wihi, int fi, int ki, int tile, int splits, float *ws0, float *ws1,
+                                float *dmu_w, float *dvar_w, hipStream_t stream) {
+    ConvParams p = dw_params(var_w, mu_a, dmu, dvar, aidx, B, fo, woho, wihi, fi, ki, dmu_w, dvar_w);
     const bool vec = (woho % 4 == 0) && aligned16(dmu) && aligned16(dvar);
     const int stencil = conv2d_bwd_dw_stencil(mu_a, dmu, dvar, B, fo, woho, wihi, fi, ki, tile);
     const int s2 = conv2d_bwd_dw_s2(mu_a, dmu, dvar, B, fo, woho, wihi, fi, ki, tile);
-    const int unit = (stencil || s2) ? 64 : KT;
-    int per = ceil_div(ceil_div(p.R, splits), unit) * unit;
-    p.splits = ceil_div(p.R, per);
-    p.r_per_split = per;
-    p.ws0 = ws0; p.ws1 = ws1;
+    plan_slices(p, splits, (stencil || s2) ? 64 : KT, ws0, ws1);
     hipError_t e = stencil ? launch_conv_stencil_dw(stencil, p, stream)
                    : s2    ? (ki == 3 ? launch_conv_stencil_s2_dw<3>(s2, p, stream)
                                       : launch_conv_stencil_s2_dw<2>(s2, p, stream))
@@ -988,6 +1017,50 @@ hipError_t launch_conv2d_bwd_dw(const float *var_w, const float *mu_a, const flo
     if (p.splits > 1)
         e = launch_reduce_splits(EPI_SCALE, ws0, ws1, p.splits, p.M, p.N, var_w, nullptr, dmu_w,
                                  dvar_w, p.N, stream);
+    return e;
+}
+
+int g_conv2d_bwd_pair = 1;
+
+// Map width when the state backward and the weight backward of a layer can share one
+// launch (both on their unit-stride stencil kernels), 0 otherwise.
+int conv2d_bwd_pair(const float *mu_w, const float *mu_a, const float *dmu, const float *dvar, int B,
+                    int fo, int woho, int wihi, int fi, int ki, int nr) {
+    if (!g_conv2d_bwd_pair || !g_conv2d_stencil || ki != 3 || nr != 9 || woho != wihi ||
+        fo % 64 != 0 || fi % 64 != 0 || !aligned16(mu_w))
+        return 0;
+    return conv2d_bwd_dw_stencil(mu_a, dmu, dvar, B, fo, woho, wihi, fi, ki, TILE_64x64);
+}
+
+// Both backward contractions of a layer for which conv2d_bwd_pair() holds: one launch for
+// the two tile grids, then the folds of whichever is sliced. (z: state backward, 64 x 128
+// tiles; w: weight backward, 64 x 64 tiles; workspaces of their own.)
+hipError_t launch_conv2d_bwd_pair(const float *mu_w, const float *var_w, const float *mu_a,
+                                  const float *jcb, const float *dmu, const float *dvar,
+                                  const int *aidx, const int *zw_idx, const int *zud_idx, int B,
+                                  int fo, int woho, int wihi, int fi, int ki, int nr, int splits_z,
+                                  float *wz0, float *wz1, int splits_w, float *ww0, float *ww1,
+                                  const float *res_mu, const float *res_var, int res_mode,
+                                  float *out_dmu, float *out_dvar, float *dmu_w, float *dvar_w,
+                                  hipStream_t stream) {
+    int stencil = 0, s2_all = 0;
+    ConvParams pz = dz_params(mu_w, jcb, dmu, dvar, zw_idx, zud_idx, woho, fo, wihi, fi, ki, nr, B,
+                              TILE_64x128, out_dmu, out_dvar, res_mu, res_var, res_mode, &stencil,
+                              &s2_all);
+    ConvParams pw = dw_params(var_w, mu_a, dmu, dvar, aidx, B, fo, woho, wihi, fi, ki, dmu_w, dvar_w);
+    const int width = conv2d_bwd_pair(mu_w, mu_a, dmu, dvar, B, fo, woho, wihi, fi, ki, nr);
+    if (width == 0 || stencil != width) return hipErrorInvalidValue;
+    plan_slices(pz, splits_z, 32 * pz.k2, wz0, wz1);
+    plan_slices(pw, splits_w, 64, ww0, ww1);
+    hipError_t e = launch_conv_stencil_bwd_pair(width, pz, pw, stream);
+    if (e != hipSuccess) return e;
+    if (pz.splits > 1) {
+        e = launch_reduce_store<ConvDzProblem>(pz, stream);
+        if (e != hipSuccess) return e;
+    }
+    if (pw.splits > 1)
+        e = launch_reduce_splits(EPI_SCALE, ww0, ww1, pw.splits, pw.M, pw.N, var_w, nullptr, dmu_w,
+                                 dvar_w, pw.N, stream);
     return e;
 }
 

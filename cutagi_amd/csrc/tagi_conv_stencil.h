@@ -306,21 +306,25 @@ __device__ __forceinline__ void stencil_body(const ConvParams &p, float *lds, in
     tile_epilogue<P, 64, 128, 2, 4>(p, acc0, acc1, m0, n0, split);
 }
 
-// One 64 x 128 tile per workgroup of 8 waves: verified stencil -> stencil_body,
-// anything else -> the table-driven loop of the generic tile kernel.
+// LDS floats a workgroup of conv_stencil_kernel<DZ, WIDTH> needs (stencil or table-driven loop).
 template <bool DZ, int WIDTH>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4)))
-void conv_stencil_kernel(ConvParams p) {
+constexpr int stencil_lds_floats() {
     using G = StencilGeom<WIDTH>;
     using P = typename std::conditional<DZ, ConvDzProblem, ConvFwdProblem<true>>::type;
     constexpr int XF = TileGeom<P::XK, 64>::floats, YF = TileGeom<P::YK, 128>::floats;
     constexpr int GENERIC = P::NX * XF + P::NY * YF;
     constexpr int STENCIL = (DZ ? 1 : 2) * 64 * G::AS + 2 * G::PATCH;
-    __shared__ __attribute__((aligned(16))) float lds[GENERIC > STENCIL ? GENERIC : STENCIL];
-    extern __shared__ __attribute__((aligned(16))) int lds_extra[];
+    return GENERIC > STENCIL ? GENERIC : STENCIL;
+}
 
+// One 64 x 128 tile by a workgroup of 8 waves: verified stencil -> stencil_body,
+// anything else -> the table-driven loop of the generic tile kernel.
+template <bool DZ, int WIDTH>
+__device__ __forceinline__ void conv_stencil_block(const ConvParams &p, float *lds, int *lds_extra,
+                                                   int tile, int split) {
+    using P = typename std::conditional<DZ, ConvDzProblem, ConvFwdProblem<true>>::type;
+    constexpr int XF = TileGeom<P::XK, 64>::floats, YF = TileGeom<P::YK, 128>::floats;
     const int tiles_n = (p.N + 127) / 128;
-    const int tile = blockIdx.x, split = blockIdx.y;
     const int m0 = (tile / tiles_n) * 64, n0 = (tile % tiles_n) * 128;
     const int r_begin = split * p.r_per_split;
     const int r_end = min(p.R, r_begin + p.r_per_split);
@@ -337,6 +341,14 @@ void conv_stencil_kernel(ConvParams p) {
     mfma_tile_body<P, 64, 128, 2, 4, 0>(p, ctx, reinterpret_cast<float (*)[XF]>(lds),
                                         reinterpret_cast<float (*)[YF]>(lds + P::NX * XF), m0, n0,
                                         split, r_lo, r_hi);
+}
+
+template <bool DZ, int WIDTH>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4)))
+void conv_stencil_kernel(ConvParams p) {
+    __shared__ __attribute__((aligned(16))) float lds[stencil_lds_floats<DZ, WIDTH>()];
+    extern __shared__ __attribute__((aligned(16))) int lds_extra[];
+    conv_stencil_block<DZ, WIDTH>(p, lds, lds_extra, blockIdx.x, blockIdx.y);
 }
 
 // Map width for which the stencil kernel exists, 0 otherwise (pixels = width^2).
@@ -528,25 +540,32 @@ __device__ __forceinline__ void stencil_dw_body(const ConvParams &p, float *lds,
 }
 
 template <int WIDTH>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4)))
-void conv_stencil_dw_kernel(ConvParams p) {
+constexpr int stencil_dw_lds_floats() {
     using G = StencilDwGeom<WIDTH>;
     using P = ConvDwVecProblem;
     constexpr int XF = TileGeom<P::XK, 64>::floats, YF = TileGeom<P::YK, 64>::floats;
     constexpr int GENERIC = P::NX * XF + P::NY * YF;
     constexpr int STENCIL = 2 * 64 * G::AS + G::PATCH;
     static_assert(2 * 64 * G::AS >= 32 * 256, "the innovation tiles hold the final exchange");
-    __shared__ __attribute__((aligned(16))) float lds[GENERIC > STENCIL ? GENERIC : STENCIL];
-    __shared__ int regular_flag;
+    return GENERIC > STENCIL ? GENERIC : STENCIL;
+}
 
+// One 64 x 64 tile of one reduction slice by a workgroup of 8 waves; (bx, by) of a
+// (gx, gy) = (tiles, slices) grid. `regular_flag`: one int of LDS.
+template <int WIDTH>
+__device__ __forceinline__ void conv_stencil_dw_block(const ConvParams &p, float *lds,
+                                                      int *regular_flag, int bx, int by, int gx,
+                                                      int gy) {
+    using P = ConvDwVecProblem;
+    constexpr int XF = TileGeom<P::XK, 64>::floats, YF = TileGeom<P::YK, 64>::floats;
     const int tiles_n = (p.N + 63) / 64;
-    int tile = blockIdx.x, split = blockIdx.y;
-    if (gridDim.y % 8 == 0) {
+    int tile = bx, split = by;
+    if (gy % 8 == 0) {
         // all column tiles of one reduction slice on one XCD (see mfma_tile_kernel)
-        const int id = blockIdx.y * gridDim.x + blockIdx.x;
+        const int id = by * gx + bx;
         const int qq = id >> 3;
-        tile = qq % gridDim.x;
-        split = (qq / gridDim.x) * 8 + (id & 7);
+        tile = qq % gx;
+        split = (qq / gx) * 8 + (id & 7);
     }
     const int m0 = (tile / tiles_n) * 64, n0 = (tile % tiles_n) * 64;
     const int r_begin = split * p.r_per_split;
@@ -555,7 +574,7 @@ void conv_stencil_dw_kernel(ConvParams p) {
     // the pixels of this slice, per image position: all of Fmwa_2 once the slice
     // is as long as a map. Entries are requested six at a time before any is
     // looked at (one memory latency per batch, not per entry).
-    if (threadIdx.x == 0) regular_flag = 1;
+    if (threadIdx.x == 0) *regular_flag = 1;
     __syncthreads();
     {
         const int total = min(max(r_end - r_begin, 0), p.woho) * 9;
@@ -573,10 +592,10 @@ void conv_stencil_dw_kernel(ConvParams p) {
 #pragma unroll
             for (int i = 0; i < 6; i++) ok = ok && got[i] == want[i];
         }
-        if (!ok) regular_flag = 0;
+        if (!ok) *regular_flag = 0;
     }
     __syncthreads();
-    if (__builtin_amdgcn_readfirstlane(regular_flag)) {
+    if (__builtin_amdgcn_readfirstlane(*regular_flag)) {
         stencil_dw_body<WIDTH>(p, lds, m0, n0, split, r_begin, r_end);
         return;
     }
@@ -588,6 +607,66 @@ void conv_stencil_dw_kernel(ConvParams p) {
     mfma_tile_body<P, 64, 64, 2, 2, 0>(p, ctx, reinterpret_cast<float (*)[XF]>(lds),
                                        reinterpret_cast<float (*)[YF]>(lds + P::NX * XF), m0, n0,
                                        split, r_begin, r_end);
+}
+
+template <int WIDTH>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4)))
+void conv_stencil_dw_kernel(ConvParams p) {
+    __shared__ __attribute__((aligned(16))) float lds[stencil_dw_lds_floats<WIDTH>()];
+    __shared__ int regular_flag;
+    conv_stencil_dw_block<WIDTH>(p, lds, &regular_flag, blockIdx.x, blockIdx.y, gridDim.x, gridDim.y);
+}
+
+// State backward and weight backward of one layer in ONE launch: the first `blocks_z`
+// workgroups are the state backward's (tile, slice) grid, the rest the weight backward's.
+// The two contractions read the same innovations and are independent; as one grid the
+// workgroups of the second start where those of the first leave CUs free, so neither
+// kernel's ramp-up (table check, first loads) nor its tail runs on an otherwise idle chip.
+template <int WIDTH>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4)))
+void conv_stencil_bwd_pair_kernel(ConvParams pz, ConvParams pw, int blocks_z, int tiles_z,
+                                  int tiles_w, int splits_w) {
+    constexpr int FZ = stencil_lds_floats<true, WIDTH>(), FW = stencil_dw_lds_floats<WIDTH>();
+    __shared__ __attribute__((aligned(16))) float lds[FZ > FW ? FZ : FW];
+    __shared__ int regular_flag;
+    extern __shared__ __attribute__((aligned(16))) int lds_extra[];
+    const int id = blockIdx.x;
+    if (id < blocks_z) {
+        conv_stencil_block<true, WIDTH>(pz, lds, lds_extra, id % tiles_z, id / tiles_z);
+    } else {
+        const int j = id - blocks_z;
+        conv_stencil_dw_block<WIDTH>(pw, lds, &regular_flag, j % tiles_w, j / tiles_w, tiles_w, splits_w);
+    }
+}
+
+inline hipError_t launch_conv_stencil_bwd_pair(int width, const ConvParams &pz, const ConvParams &pw,
+                                               hipStream_t stream) {
+    using P = ConvDzProblem;
+    const int tiles_z = ((pz.M + 63) / 64) * ((pz.N + 127) / 128);
+    const int tiles_w = ((pw.M + 63) / 64) * ((pw.N + 63) / 64);
+    const int blocks_z = tiles_z * pz.splits;
+    const dim3 grid(blocks_z + tiles_w * pw.splits);
+    const size_t extra = P::extra_lds_bytes(pz, 64, 128);
+    if (extra > kTileExtraLdsMax) return hipErrorInvalidValue;
+#define TAGI_LAUNCH_PAIR(WD)                                                                       \
+    case WD: {                                                                                     \
+        static PerDeviceOnce once;                                                                 \
+        hipError_t e = allow_dynamic_lds(                                                          \
+            once, reinterpret_cast<const void *>(conv_stencil_bwd_pair_kernel<WD>),                \
+            (int)kTileExtraLdsMax);                                                                \
+        if (e != hipSuccess) return e;                                                             \
+        hipLaunchKernelGGL((conv_stencil_bwd_pair_kernel<WD>), grid, dim3(512), extra, stream, pz, \
+                           pw, blocks_z, tiles_z, tiles_w, pw.splits);                             \
+        return hipGetLastError();                                                                  \
+    }
+    switch (width) {
+        TAGI_LAUNCH_PAIR(4)
+        TAGI_LAUNCH_PAIR(8)
+        TAGI_LAUNCH_PAIR(16)
+        TAGI_LAUNCH_PAIR(32)
+    }
+#undef TAGI_LAUNCH_PAIR
+    return hipErrorInvalidValue;
 }
 
 inline hipError_t launch_conv_stencil_dw(int width, const ConvParams &p, hipStream_t stream) {

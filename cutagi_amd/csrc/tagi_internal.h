@@ -277,6 +277,18 @@ hipError_t launch_conv2d_bwd_dw(const float *var_w, const float *mu_a, const flo
                                 const float *dvar, const int *aidx, int B, int fo, int woho,
                                 int wihi, int fi, int ki, int tile, int splits, float *ws0, float *ws1,
                                 float *dmu_w, float *dvar_w, hipStream_t stream);
+// 0: state and weight backward of a layer always as launches of their own
+extern int g_conv2d_bwd_pair;
+int conv2d_bwd_pair(const float *mu_w, const float *mu_a, const float *dmu, const float *dvar, int B,
+                    int fo, int woho, int wihi, int fi, int ki, int nr);
+hipError_t launch_conv2d_bwd_pair(const float *mu_w, const float *var_w, const float *mu_a,
+                                  const float *jcb, const float *dmu, const float *dvar,
+                                  const int *aidx, const int *zw_idx, const int *zud_idx, int B,
+                                  int fo, int woho, int wihi, int fi, int ki, int nr, int splits_z,
+                                  float *wz0, float *wz1, int splits_w, float *ww0, float *ww1,
+                                  const float *res_mu, const float *res_var, int res_mode,
+                                  float *out_dmu, float *out_dvar, float *dmu_w, float *dvar_w,
+                                  hipStream_t stream);
 hipError_t launch_conv2d_bwd_db(const float *var_b, const float *dmu, const float *dvar, int B,
                                 int fo, int woho, int chunks, float *scratch, float *dmu_b,
                                 float *dvar_b, hipStream_t stream);

@@ -168,6 +168,30 @@ def conv2d_bwd_dw(var_w, var_b, mu_a, delta_mu, delta_var, aidx, B, fo, woho, wi
     return om, ov, bm, bv
 
 
+def conv2d_bwd(mu_w, var_w, var_b, mu_a, jcb, delta_mu, delta_var, aidx, zw_idx, zud_idx, B, fo,
+               woho, wihi, fi, ki, nr, state_update=True, param_update=True, res_mu=None,
+               res_var=None, res_mode=0):
+    """Both backward contractions in one call: (delta_mu_z, delta_var_z, delta_mu_w,
+    delta_var_w, delta_mu_b, delta_var_b), None where a part is switched off."""
+    _chk(mu_w, var_w, var_b, mu_a, jcb, delta_mu, delta_var, aidx, zw_idx, zud_idx, res_mu, res_var)
+    dev = mu_w.device
+    nw = ki * ki * fi * fo
+    bias = var_b is not None
+    zm = torch.empty(B * fi * wihi, device=dev) if state_update else None
+    zv = torch.empty(B * fi * wihi, device=dev) if state_update else None
+    wm = torch.empty(nw, device=dev) if param_update else None
+    wv = torch.empty(nw, device=dev) if param_update else None
+    bm = torch.empty(fo, device=dev) if bias and param_update else None
+    bv = torch.empty(fo, device=dev) if bias and param_update else None
+    capi.check(capi.lib.tagi_conv2d_bwd(
+        capi.ptr(mu_w), capi.ptr(var_w), capi.ptr(var_b), capi.ptr(mu_a), capi.ptr(jcb),
+        capi.ptr(delta_mu), capi.ptr(delta_var), capi.ptr(aidx), capi.ptr(zw_idx), capi.ptr(zud_idx),
+        B, fo, woho, wihi, fi, ki, nr, int(bias), int(state_update), int(param_update),
+        capi.ptr(res_mu), capi.ptr(res_var), res_mode, capi.ptr(zm), capi.ptr(zv), capi.ptr(wm),
+        capi.ptr(wv), capi.ptr(bm), capi.ptr(bv), _stream()))
+    return zm, zv, wm, wv, bm, bv
+
+
 def store_states(mu_a, jcb, n_in, bwd_mu_a, bwd_jcb, out_jcb, n_out):
     capi.check(capi.lib.tagi_store_states(capi.ptr(mu_a), capi.ptr(jcb), n_in, capi.ptr(bwd_mu_a),
                                           capi.ptr(bwd_jcb), capi.ptr(out_jcb), n_out, _stream()))

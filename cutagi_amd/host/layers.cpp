@@ -685,30 +685,17 @@ void Conv2dHip::backward(BaseDeltaStates &input_delta_states, BaseDeltaStates &o
     auto *bwd = dynamic_cast<BackwardStateHip *>(this->bwd_states.get());
     const int batch_size = (int)input_delta_states.block_size;
     const int woho = (int)(out_width * out_height), wihi = (int)(in_width * in_height);
-    if (param_update)
-        TAGI_OK_OR_THROW(tagi_conv2d_bwd_dw(d_var_w, d_var_b, bwd->d_mu_a, din->d_delta_mu,
-                                            din->d_delta_var, d_idx_mwa_2, batch_size,
-                                            (int)out_channels, woho, wihi, (int)in_channels,
-                                            (int)kernel_size, bias ? 1 : 0, d_delta_mu_w,
-                                            d_delta_var_w, d_delta_mu_b, d_delta_var_b, host_stream()));
-    if (state_udapte) {
-        if (input_size * batch_size > dout->size)
-            LOG(LogLevel::ERROR, "Delta state buffer too small for " + this->get_layer_info());
-        if (res_mu != nullptr)
-            TAGI_OK_OR_THROW(tagi_conv2d_bwd_dz_res(
-                d_mu_w, bwd->jcb_ptr(), din->d_delta_mu, din->d_delta_var, d_idx_cov_zwa_1,
-                d_idx_var_z_ud, woho, (int)out_channels, wihi, (int)in_channels, (int)kernel_size,
-                row_zw, batch_size, res_mu, res_var, res_mode, dout->d_delta_mu,
-                dout->d_delta_var, host_stream()));
-        else
-            TAGI_OK_OR_THROW(tagi_conv2d_bwd_dz(d_mu_w, bwd->jcb_ptr(), din->d_delta_mu,
-                                                din->d_delta_var, d_idx_cov_zwa_1, d_idx_var_z_ud,
-                                                woho, (int)out_channels, wihi, (int)in_channels,
-                                                (int)kernel_size, row_zw, batch_size,
-                                                dout->d_delta_mu, dout->d_delta_var, host_stream()));
-    } else if (res_mu != nullptr) {
+    if (state_udapte && input_size * batch_size > dout->size)
+        LOG(LogLevel::ERROR, "Delta state buffer too small for " + this->get_layer_info());
+    if (!state_udapte && res_mu != nullptr)
         LOG(LogLevel::ERROR, "Residual innovations handed to a layer that skips its state update");
-    }
+    // one call for both contractions: where they run on the stencil kernels they share a launch
+    TAGI_OK_OR_THROW(tagi_conv2d_bwd(
+        d_mu_w, d_var_w, d_var_b, bwd->d_mu_a, bwd->jcb_ptr(), din->d_delta_mu, din->d_delta_var,
+        d_idx_mwa_2, d_idx_cov_zwa_1, d_idx_var_z_ud, batch_size, (int)out_channels, woho, wihi,
+        (int)in_channels, (int)kernel_size, row_zw, bias ? 1 : 0, state_udapte ? 1 : 0,
+        param_update ? 1 : 0, res_mu, res_var, res_mode, dout->d_delta_mu, dout->d_delta_var,
+        d_delta_mu_w, d_delta_var_w, d_delta_mu_b, d_delta_var_b, host_stream()));
 }
 
 // ---- ReLU ---------------------------------------------------------------------------------

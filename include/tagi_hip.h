@@ -206,6 +206,25 @@ int tagi_conv2d_bwd_dw(const float *var_w, const float *var_b,
                        float *delta_mu_w, float *delta_var_w,
                        float *delta_mu_b, float *delta_var_b, void *stream);
 
+/* All of Conv2dCuda::backward (src/conv2d_layer_cuda.cu:349-476) in one call: the state
+ * innovations (state_update; with res_mu / res_var != NULL also the residual add of
+ * tagi_conv2d_bwd_dz_res) and the weight / bias innovations (param_update; bias ones
+ * only when bias != 0). Where both contractions run on their regular-stencil kernels
+ * (3x3, stride 1, "same" padding, whole groups of 64 channels) they share ONE launch:
+ * the two tile grids are independent, and as one grid neither kernel's ramp-up nor its
+ * tail leaves the chip idle. Otherwise the same as tagi_conv2d_bwd_dw followed by
+ * tagi_conv2d_bwd_dz(_res). Uses the workspace. */
+int tagi_conv2d_bwd(const float *mu_w, const float *var_w, const float *var_b,
+                    const float *mu_a, const float *jcb,
+                    const float *delta_mu_out, const float *delta_var_out,
+                    const int *aidx, const int *zw_idx, const int *zud_idx, int B,
+                    int fo, int woho, int wihi, int fi, int ki, int nr, int bias,
+                    int state_update, int param_update,
+                    const float *res_mu /* may be NULL */, const float *res_var,
+                    int res_mode, float *delta_mu, float *delta_var,
+                    float *delta_mu_w, float *delta_var_w, float *delta_mu_b,
+                    float *delta_var_b, void *stream);
+
 /* ---- layer glue ------------------------------------------------------------ */
 
 /* Keep what the backward pass needs and reset the output Jacobian; replaces

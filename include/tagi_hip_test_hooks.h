@@ -32,7 +32,8 @@ extern "C" {
  * "conv2d.stencil", "conv2d.phase_order", "conv2d.s2_all" (0 switches the named path
  * off; s2_all: the stencil kernels of the stride-2 layers - forward, state backward with
  * all four phases in one workgroup and its pair-wise fold, weight backward - which leaves
- * those layers on the table-driven kernels). */
+ * those layers on the table-driven kernels; "conv2d.bwd_pair": 0 gives the state and the
+ * weight backward of tagi_conv2d_bwd launches of their own). */
 int tagi_hip_tune(const char *key /* host */, int value);
 
 #ifdef __cplusplus

@@ -463,3 +463,84 @@ def test_conv2d_state_backward_with_residual(oracle_lib, geom, mode):
     torch.cuda.synchronize()
     assert_close(om.cpu().numpy(), want[0], "delta_mu_z + residual")
     assert_close(ov.cpu().numpy(), want[1], "delta_var_z + residual", same_sign=True)
+
+
+# eligible for the shared launch (3x3 s1 p1, whole groups of 64 channels, whole 64-pixel
+# k-tiles), sliced state backward, and shapes that fall back to two launches
+PAIR_GEOMS = [(3, 1, 1, 1, 16, 64, 64, 4), (3, 1, 1, 1, 32, 64, 64, 2), (3, 1, 1, 1, 8, 128, 64, 3),
+              (3, 1, 1, 1, 4, 320, 128, 8), (3, 1, 1, 1, 4, 320, 64, 5), (3, 2, 1, 2, 16, 64, 64, 4),
+              (2, 2, 0, 1, 8, 64, 130, 2), (3, 1, 1, 1, 8, 4, 8, 3)]
+
+
+@pytest.mark.parametrize("geom", PAIR_GEOMS)
+@pytest.mark.parametrize("res_mode", [0, 1, 2])
+def test_conv2d_backward_in_one_call(oracle_lib, geom, res_mode):
+    """tagi_conv2d_bwd against the oracle and, bit for bit, against the separate entry
+    points (same kernels, whether they share a launch or not); with and without a
+    residual, with the parts switched off one at a time."""
+    import torch
+    import cutagi_amd.functional as F
+    from cutagi_amd import capi
+    k, s, p, pt, wi, fi, fo, B = geom
+    idx, d, t, ti, wihi, woho = _setup(oracle_lib, geom, True, seed=31 + res_mode)
+    rng = np.random.default_rng(5)
+    res = None
+    if res_mode:
+        res = [torch.from_numpy((rng.standard_normal(B * fi * wihi) * 0.1).astype(np.float32)).cuda(),
+               torch.from_numpy(rng.uniform(0, 1e-3, B * fi * wihi).astype(np.float32)).cuda()]
+    args = (t["mu_w"], t["var_w"], t["var_b"], t["mu_a"], t["jcb"], t["delta_mu"], t["delta_var"],
+            ti["Fmwa_2"], ti["FCzwa_1"], ti["Szz_ud"], B, fo, woho, wihi, fi, k, idx["h"])
+    kw = dict(res_mu=res[0] if res else None, res_var=res[1] if res else None, res_mode=res_mode)
+    got = F.conv2d_bwd(*args, **kw)
+    # the separate entry points
+    dw = F.conv2d_bwd_dw(t["var_w"], t["var_b"], t["mu_a"], t["delta_mu"], t["delta_var"],
+                         ti["Fmwa_2"], B, fo, woho, wihi, fi, k)
+    zm, zv = torch.empty(B * fi * wihi, device="cuda"), torch.empty(B * fi * wihi, device="cuda")
+    if res_mode:
+        capi.check(capi.lib.tagi_conv2d_bwd_dz_res(
+            capi.ptr(t["mu_w"]), capi.ptr(t["jcb"]), capi.ptr(t["delta_mu"]), capi.ptr(t["delta_var"]),
+            capi.ptr(ti["FCzwa_1"]), capi.ptr(ti["Szz_ud"]), woho, fo, wihi, fi, k, idx["h"], B,
+            capi.ptr(res[0]), capi.ptr(res[1]), res_mode, capi.ptr(zm), capi.ptr(zv),
+            torch.cuda.current_stream().cuda_stream))
+    else:
+        zm, zv = F.conv2d_bwd_dz(t["mu_w"], t["jcb"], t["delta_mu"], t["delta_var"], ti["FCzwa_1"],
+                                 ti["Szz_ud"], woho, fo, wihi, fi, k, idx["h"], B)
+    for name, a, b in zip(("delta_mu_z", "delta_var_z", "delta_mu_w", "delta_var_w", "delta_mu_b",
+                           "delta_var_b"), got, (zm, zv) + tuple(dw)):
+        assert torch.equal(a, b), name
+    # the oracle (the residual is applied as ConvDz does: before or after the Jacobian)
+    ref = oracle_lib.conv2d_bwd_dz(d["mu_w"], d["jcb"], d["delta_mu"], d["delta_var"],
+                                   idx["FCzwa_1"], idx["Szz_ud"], woho, fo, wihi, fi, k, idx["h"],
+                                   B, threads=4)
+    if res_mode == 0:
+        assert_close(got[0].cpu().numpy(), ref[0], "delta_mu_z")
+        assert_close(got[1].cpu().numpy(), ref[1], "delta_var_z", same_sign=True)
+    rw = oracle_lib.conv2d_bwd_dw(d["var_w"], d["var_b"], d["mu_a"], d["delta_mu"], d["delta_var"],
+                                  idx["Fmwa_2"], B, fo, woho, wihi, fi, k, threads=4)
+    assert_close(got[2].cpu().numpy(), rw[0], "delta_mu_w")
+    assert_close(got[3].cpu().numpy(), rw[1], "delta_var_w", same_sign=True)
+    # parts switched off
+    only_w = F.conv2d_bwd(*args, state_update=False)
+    assert only_w[0] is None and torch.equal(only_w[2], got[2]) and torch.equal(only_w[4], got[4])
+    only_z = F.conv2d_bwd(*args, param_update=False, **kw)
+    assert only_z[2] is None and torch.equal(only_z[0], got[0]) and torch.equal(only_z[1], got[1])
+
+
+def test_conv2d_backward_pair_launch_can_be_switched_off(oracle_lib):
+    """"conv2d.bwd_pair" = 0 gives two launches; the results are the same bits."""
+    import torch
+    import cutagi_amd.functional as F
+    from cutagi_amd import capi
+    geom = (3, 1, 1, 1, 16, 64, 128, 4)
+    k, s, p, pt, wi, fi, fo, B = geom
+    idx, d, t, ti, wihi, woho = _setup(oracle_lib, geom, False, seed=40)
+    args = (t["mu_w"], t["var_w"], None, t["mu_a"], t["jcb"], t["delta_mu"], t["delta_var"],
+            ti["Fmwa_2"], ti["FCzwa_1"], ti["Szz_ud"], B, fo, woho, wihi, fi, k, idx["h"])
+    a = F.conv2d_bwd(*args)
+    capi.tune("conv2d.bwd_pair", 0)
+    try:
+        b = F.conv2d_bwd(*args)
+    finally:
+        capi.tune("conv2d.bwd_pair", 1)
+    for x, y in zip(a[:4], b[:4]):
+        assert torch.equal(x, y)
