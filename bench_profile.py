@@ -113,8 +113,8 @@ KERNELS = [
     ("gemv_dw_kernel<16, true>", "Linear 8192^2 B=12 and B=16 delta_w (+delta_b)", 3 * K3 * K3 * 4 / MB, 4.0 * 14 * K3 * K3),
     ("gemv16_fwd_kernel<2>", "Linear 4096^2 B=32 forward", 2 * K2 * K2 * 4 / MB, 6.0 * 32 * K2 * K2),
     ("conv_stencil_kernel<false, 32>", "Conv2d 3x3 64->64 @32x32 B=128 forward", 4 * CONV_ACT, 6.0 * 64 * 131072 * 576),
-    ("conv_stencil_kernel<true, 32>", "Conv2d delta_z", 5 * CONV_ACT, 4.0 * 64 * 131072 * 576),
-    ("conv_stencil_dw_kernel<32>", "Conv2d delta_w", 3 * CONV_ACT, 4.0 * 64 * 131072 * 576),
+    ("conv_stencil_bwd_pair_kernel<32>", "Conv2d delta_z + delta_w (one launch)", 6 * CONV_ACT,
+     8.0 * 64 * 131072 * 576),
 ]
 MAIN_KERNELS = tuple(k for k, w, _, _ in KERNELS if "B=256" in w)
 # bench.py's table: (workload, phase) -> kernel
