@@ -613,6 +613,18 @@ int tagi_linear_bwd(const float *mu_w, const float *var_w, const float *var_b, c
     int rc = TAGI_OK;
     if (param_update && bias && (!var_b || !delta_mu_b || !delta_var_b))
         return TAGI_ERR_INVALID_ARG;
+    if (state_update && param_update && use_small_kernels() && g_tune.dw_side != 0 && mu_w && var_w &&
+        mu_a && jcb && delta_mu && delta_var && delta_mu_z && delta_var_z && delta_mu_w &&
+        delta_var_w && K > 0 && N > 0 && B > 0 && K % 4 == 0 && aligned16(mu_w) && aligned16(mu_a) &&
+        aligned16(var_w) && aligned16(delta_mu_w) && aligned16(delta_var_w) &&
+        small_bwd_supported(K, N, B) && small_dw_supported(K, N, B)) {
+        // a small layer: both contractions (and the bias innovations) in one launch
+        TAGI_TRY(launch_small_bwd_pair(mu_w, var_w, mu_a, jcb, delta_mu, delta_var, K, N, B,
+                                       delta_mu_z, delta_var_z, delta_mu_w, delta_var_w,
+                                       bias ? var_b : nullptr, delta_mu_b, delta_var_b,
+                                       static_cast<hipStream_t>(stream)));
+        return TAGI_OK;
+    }
     DzFold fold;
     if (state_update) {
         rc = linear_bwd_dz_impl(mu_w, jcb, delta_mu, delta_var, K, N, B, delta_mu_z, delta_var_z,

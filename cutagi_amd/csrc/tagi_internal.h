@@ -113,6 +113,12 @@ hipError_t launch_small_dw(const float *var_w, const float *mu_a, const float *d
                            const float *dvar, int K, int N, int B, float *dmu_w, float *dvar_w,
                            const float *var_b, float *dmu_b, float *dvar_b, hipStream_t stream);
 
+hipError_t launch_small_bwd_pair(const float *mu_w, const float *var_w, const float *mu_a,
+                                 const float *jcb, const float *dmu, const float *dvar, int K, int N,
+                                 int B, float *out_mu, float *out_var, float *dmu_w, float *dvar_w,
+                                 const float *var_b, float *dmu_b, float *dvar_b,
+                                 hipStream_t stream);
+
 // Skinny-batch (B <= 16) streaming kernels: weights are read once from HBM
 // straight into MFMA operand layout, nothing is staged in LDS.
 hipError_t launch_gemv_fwd(const float *mu_w, const float *var_w, const float *mu_a,

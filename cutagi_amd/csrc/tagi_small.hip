@@ -188,21 +188,21 @@ __global__ __launch_bounds__(SMALL_WAVES * 64) void small_fwd_kernel(
 // of the output units; slice s takes the units s, s + 8, ...
 constexpr int DZ_LANES = 32, DZ_SLICES = 8, DZ_BATCH = 16;
 
-__global__ __launch_bounds__(DZ_LANES * DZ_SLICES) void small_dz_kernel(
+// (bx, b): column block and sample of the workgroup; red: 8 KB of LDS
+__device__ __forceinline__ void small_dz_block(
     const float *__restrict__ mu_w, const float *__restrict__ jcb,
     const float *__restrict__ dmu, const float *__restrict__ dvar, int K, int N,
-    float *__restrict__ out_mu, float *__restrict__ out_var) {
-    __shared__ float red[DZ_SLICES][DZ_LANES][8];
+    float *__restrict__ out_mu, float *__restrict__ out_var, int bx, int b,
+    float (*red)[DZ_LANES][8]) {
     const int kl = threadIdx.x & (DZ_LANES - 1), slice = threadIdx.x / DZ_LANES;
-    const int k = (blockIdx.x * DZ_LANES + kl) * 4;
-    const int b = blockIdx.y;
+    const int k = (bx * DZ_LANES + kl) * 4;
     const bool valid = k < K;
     const float *w_col = mu_w + (valid ? k : 0);
     const float *dm_row = dmu + (size_t)b * N, *dv_row = dvar + (size_t)b * N;
     // after the sums: thread t folds entry t % 8 of lane t / 8 over the slices. Its
     // Jacobian is asked for now, not in a memory round trip of its own at the end.
     const int kl2 = threadIdx.x >> 3, c = threadIdx.x & 7;
-    const int k2 = (blockIdx.x * DZ_LANES + kl2) * 4 + (c & 3);
+    const int k2 = (bx * DZ_LANES + kl2) * 4 + (c & 3);
     const size_t at = (size_t)b * K + min(k2, K - 1);
     const float j = jcb[at];
     float4 m = make_float4(0.f, 0.f, 0.f, 0.f), v = m;
@@ -239,6 +239,14 @@ __global__ __launch_bounds__(DZ_LANES * DZ_SLICES) void small_dz_kernel(
         out_var[at] = sum * j * j;
 }
 
+__global__ __launch_bounds__(DZ_LANES * DZ_SLICES) void small_dz_kernel(
+    const float *__restrict__ mu_w, const float *__restrict__ jcb,
+    const float *__restrict__ dmu, const float *__restrict__ dvar, int K, int N,
+    float *__restrict__ out_mu, float *__restrict__ out_var) {
+    __shared__ float red[DZ_SLICES][DZ_LANES][8];
+    small_dz_block(mu_w, jcb, dmu, dvar, K, N, out_mu, out_var, blockIdx.x, blockIdx.y, red);
+}
+
 // ---- weight backward ----------------------------------------------------------------
 // delta_mu_w[n][k] = var_w[n][k] sum_b mu_a[b][k] delta_mu[b][n], delta_var_w with
 // var_w^2, mu_a^2 and delta_var; thread = DW_ROWS output units x 4 input units, DW_BATCH
@@ -248,13 +256,13 @@ __global__ __launch_bounds__(DZ_LANES * DZ_SLICES) void small_dz_kernel(
 constexpr int DW_TPB = 256;
 
 template <int DW_ROWS, int DW_BATCH>
-__global__ __launch_bounds__(DW_TPB) void small_dw_kernel(
+__device__ __forceinline__ void small_dw_block(
     const float *__restrict__ var_w, const float *__restrict__ mu_a,
     const float *__restrict__ dmu, const float *__restrict__ dvar, int K, int N, int B,
     float *__restrict__ dmu_w, float *__restrict__ dvar_w, const float *__restrict__ var_b,
-    float *__restrict__ dmu_b, float *__restrict__ dvar_b) {
+    float *__restrict__ dmu_b, float *__restrict__ dvar_b, int block) {
     const int K4 = K >> 2;
-    const int item = blockIdx.x * DW_TPB + threadIdx.x;
+    const int item = block * DW_TPB + threadIdx.x;
     if (item >= ((N + DW_ROWS - 1) / DW_ROWS) * K4) return;
     const int n0 = (item / K4) * DW_ROWS, k = (item % K4) * 4;
     int row[DW_ROWS];
@@ -315,6 +323,39 @@ __global__ __launch_bounds__(DW_TPB) void small_dw_kernel(
             dvar_b[row[r]] = bv[r] * vb * vb;
         }
     }
+}
+
+template <int DW_ROWS, int DW_BATCH>
+__global__ __launch_bounds__(DW_TPB) void small_dw_kernel(
+    const float *__restrict__ var_w, const float *__restrict__ mu_a,
+    const float *__restrict__ dmu, const float *__restrict__ dvar, int K, int N, int B,
+    float *__restrict__ dmu_w, float *__restrict__ dvar_w, const float *__restrict__ var_b,
+    float *__restrict__ dmu_b, float *__restrict__ dvar_b) {
+    small_dw_block<DW_ROWS, DW_BATCH>(var_w, mu_a, dmu, dvar, K, N, B, dmu_w, dvar_w, var_b, dmu_b,
+                                      dvar_b, blockIdx.x);
+}
+
+// Both backward kernels of a layer as one grid: the first blocks_z workgroups are the
+// state backward's (column block, sample) pairs, the rest the weight backward's. The two
+// read the same innovations and do not depend on each other; at these sizes a launch
+// costs more than what it computes.
+struct SmallBwdArgs {
+    const float *mu_w, *var_w, *mu_a, *jcb, *dmu, *dvar, *var_b;
+    float *out_mu, *out_var, *dmu_w, *dvar_w, *dmu_b, *dvar_b;
+    int K, N, B, blocks_z, blocks_zx;
+};
+static_assert(DZ_LANES * DZ_SLICES == DW_TPB, "one workgroup size for both parts");
+
+template <int DW_ROWS, int DW_BATCH>
+__global__ __launch_bounds__(DW_TPB) void small_bwd_pair_kernel(SmallBwdArgs a) {
+    __shared__ float red[DZ_SLICES][DZ_LANES][8];
+    const int id = blockIdx.x;
+    if (id < a.blocks_z)
+        small_dz_block(a.mu_w, a.jcb, a.dmu, a.dvar, a.K, a.N, a.out_mu, a.out_var,
+                       id % a.blocks_zx, id / a.blocks_zx, red);
+    else
+        small_dw_block<DW_ROWS, DW_BATCH>(a.var_w, a.mu_a, a.dmu, a.dvar, a.K, a.N, a.B, a.dmu_w,
+                                          a.dvar_w, a.var_b, a.dmu_b, a.dvar_b, id - a.blocks_z);
 }
 
 }  // namespace
@@ -379,6 +420,32 @@ hipError_t launch_small_dw(const float *var_w, const float *mu_a, const float *d
         hipLaunchKernelGGL((small_dw_kernel<1, 32>), dim3((items + DW_TPB - 1) / DW_TPB), dim3(DW_TPB),
                            0, stream, var_w, mu_a, dmu, dvar, K, N, B, dmu_w, dvar_w, var_b, dmu_b,
                            dvar_b);
+    }
+    return hipGetLastError();
+}
+
+// State and weight backward (+ bias innovations when var_b is given) of a layer for which
+// small_bwd_supported and small_dw_supported hold, in one launch.
+hipError_t launch_small_bwd_pair(const float *mu_w, const float *var_w, const float *mu_a,
+                                 const float *jcb, const float *dmu, const float *dvar, int K, int N,
+                                 int B, float *out_mu, float *out_var, float *dmu_w, float *dvar_w,
+                                 const float *var_b, float *dmu_b, float *dvar_b,
+                                 hipStream_t stream) {
+    if (K % 4 != 0 || K <= 0 || N <= 0 || B <= 0) return hipErrorInvalidValue;
+    SmallBwdArgs a;
+    a.mu_w = mu_w; a.var_w = var_w; a.mu_a = mu_a; a.jcb = jcb; a.dmu = dmu; a.dvar = dvar;
+    a.var_b = var_b; a.out_mu = out_mu; a.out_var = out_var; a.dmu_w = dmu_w; a.dvar_w = dvar_w;
+    a.dmu_b = dmu_b; a.dvar_b = dvar_b; a.K = K; a.N = N; a.B = B;
+    a.blocks_zx = ((K >> 2) + DZ_LANES - 1) / DZ_LANES;
+    a.blocks_z = a.blocks_zx * B;
+    if (B <= 16) {
+        const int items = ((N + 1) / 2) * (K >> 2);
+        hipLaunchKernelGGL((small_bwd_pair_kernel<2, 16>), dim3(a.blocks_z + (items + DW_TPB - 1) / DW_TPB),
+                           dim3(DW_TPB), 0, stream, a);
+    } else {
+        const int items = N * (K >> 2);
+        hipLaunchKernelGGL((small_bwd_pair_kernel<1, 32>), dim3(a.blocks_z + (items + DW_TPB - 1) / DW_TPB),
+                           dim3(DW_TPB), 0, stream, a);
     }
     return hipGetLastError();
 }
