@@ -57,6 +57,7 @@ SIGNATURES = {
     "tagi_out_update_indexed": (_i, [_vp] * 6 + [_i] * 3 + [_vp] * 3),
     "tagi_out_update_indexed_reset": (_i, [_vp] * 6 + [_i, _i, _i, _vp, _vp, _sz, _vp]),
     "tagi_conv2d_bwd": (_i, [_vp] * 10 + [_i] * 10 + [_vp, _vp, _i] + [_vp] * 7),
+    "tagi_batchnorm2d_fwd_train": (_i, [_vp] * 8 + [_i, _f, _f, _i, _i, _i] + [_vp] * 7),
     "tagi_upload_input": (_i, [_vp, _vp, _sz, _vp, _vp, _vp]),
     "tagi_download_outputs": (_i, [_vp, _vp, _sz, _vp, _vp, _vp, ctypes.c_uint, _vp]),
     "tagi_relu_fwd": (_i, [_vp, _vp, _sz, _vp, _vp, _vp, _vp]),

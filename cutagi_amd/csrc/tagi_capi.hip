@@ -21,7 +21,7 @@ static __device__ __align__(256) float scratch[STATIC_SCRATCH_BYTES / sizeof(flo
 
 namespace {
 
-constexpr int ABI_VERSION = 105;
+constexpr int ABI_VERSION = 106;
 
 #define TAGI_TRY(expr)                          \
     do {                                        \
@@ -329,6 +329,7 @@ int tagi_hip_tune(const char *key, int value) {
     else if (!strcmp(key, "conv2d.phase_order")) g_conv2d_phase_order = value;
     else if (!strcmp(key, "conv2d.s2_all")) g_conv2d_s2_all = value < 0 ? 1 : value;
     else if (!strcmp(key, "conv2d.bwd_pair")) g_conv2d_bwd_pair = value < 0 ? 1 : value;
+    else if (!strcmp(key, "batchnorm.fused_train")) g_bn_fused_train = value < 0 ? 1 : value;
     else if (!strcmp(key, "linear.tile")) g_tune.tile = value;
     else if (!strcmp(key, "linear.double_buffer")) g_gemm_double_buffer = value < 0 ? 1 : value;
     else if (!strcmp(key, "conv2d.dw.splits")) g_tune.conv_dw_splits = value;
@@ -1114,6 +1115,28 @@ static int batchnorm2d_fwd_impl(const float *mu_w, const float *var_w, const flo
     TAGI_TRY(launch_batchnorm2d_fwd(mu_w, var_w, bias ? mu_b : nullptr, bias ? var_b : nullptr,
                                     mu_a, var_a, mu_norm, var_norm, epsilon, wihi, fi, B, mu_z,
                                     var_z, static_cast<hipStream_t>(stream), mu_res, var_res));
+    return TAGI_OK;
+}
+
+int tagi_batchnorm2d_fwd_train(const float *mu_w, const float *var_w, const float *mu_b,
+                               const float *var_b, const float *mu_a, const float *var_a,
+                               const float *mu_res, const float *var_res, int bias, float momentum,
+                               float epsilon, int wihi, int fi, int B, float *mu_s, float *var_s,
+                               float *mu_ra, float *var_ra, float *mu_z, float *var_z,
+                               void *stream) {
+    if (!mu_w || !var_w || !mu_a || !var_a || !mu_s || !var_s || !mu_ra || !var_ra || !mu_z || !var_z)
+        return TAGI_ERR_INVALID_ARG;
+    if (bias && (!mu_b || !var_b)) return TAGI_ERR_INVALID_ARG;
+    if ((mu_res == nullptr) != (var_res == nullptr)) return TAGI_ERR_INVALID_ARG;
+    if (!bn_sizes_ok(wihi, fi, B)) return TAGI_ERR_INVALID_ARG;
+    float *ws = nullptr;
+    int rc = workspace_get(batchnorm2d_scratch_floats(fi, B) * sizeof(float),
+                           static_cast<hipStream_t>(stream), &ws);
+    if (rc != TAGI_OK) return rc;
+    TAGI_TRY(launch_batchnorm2d_fwd_train(mu_w, var_w, bias ? mu_b : nullptr, bias ? var_b : nullptr,
+                                          mu_a, var_a, mu_res, var_res, momentum, epsilon, wihi, fi,
+                                          B, ws, mu_s, var_s, mu_ra, var_ra, mu_z, var_z,
+                                          static_cast<hipStream_t>(stream)));
     return TAGI_OK;
 }
 

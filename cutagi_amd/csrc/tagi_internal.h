@@ -226,6 +226,13 @@ hipError_t launch_batchnorm2d_stats(const float *mu_a, const float *var_a, int w
                                     int B, float momentum, float *scratch, float *mu_s,
                                     float *var_s, float *mu_ra, float *var_ra,
                                     hipStream_t stream);
+extern int g_bn_fused_train;  // 0: statistics merged by a launch of their own
+hipError_t launch_batchnorm2d_fwd_train(const float *mu_w, const float *var_w, const float *mu_b,
+                                        const float *var_b, const float *mu_a, const float *var_a,
+                                        const float *mu_res, const float *var_res, float momentum,
+                                        float epsilon, int wihi, int fi, int B, float *scratch,
+                                        float *mu_s, float *var_s, float *mu_ra, float *var_ra,
+                                        float *mu_z, float *var_z, hipStream_t stream);
 hipError_t launch_batchnorm2d_fwd(const float *mu_w, const float *var_w, const float *mu_b,
                                   const float *var_b, const float *mu_a, const float *var_a,
                                   const float *mu_norm, const float *var_norm, float epsilon,

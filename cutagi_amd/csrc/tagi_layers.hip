@@ -226,6 +226,95 @@ __global__ __launch_bounds__(TPB) void bn_fwd_vec_kernel(
     *reinterpret_cast<float4 *>(var_z + i) = ov;
 }
 
+// Training-mode forward with the merge of the statistics inside: bn_stats_final_kernel's
+// work is done per workgroup, for the channel maps the workgroup touches (the partial
+// statistics are a few cache-resident floats per channel), which saves that kernel's
+// launch. A workgroup owns FT_ITER * TPB consecutive groups of four pixels; thread t < maps
+// merges the chunks of map t's channel in chunk order (the same arithmetic as
+// bn_stats_final_kernel, so mean and variance are the same bits) and leaves them in LDS;
+// the one workgroup that holds the start of map (image 0, channel c) also writes the batch
+// statistics and moves the running averages. The normalisation is bn_fwd_vec_kernel's.
+constexpr int FT_ITER = 4, FT_MAX_MAPS = FT_ITER * TPB / 4 + 1;   // wihi >= 16
+
+__global__ __launch_bounds__(TPB) void bn_fwd_train_vec_kernel(
+    const float *__restrict__ mu_w, const float *__restrict__ var_w,
+    const float *__restrict__ mu_b, const float *__restrict__ var_b,
+    const float *__restrict__ mu_a, const float *__restrict__ var_a,
+    const float *__restrict__ part, int chunks, float momentum, float epsilon, int wihi, int fi,
+    size_t n4, const float *__restrict__ mu_res, const float *__restrict__ var_res,
+    float *__restrict__ mu_s, float *__restrict__ var_s, float *__restrict__ mu_ra,
+    float *__restrict__ var_ra, float *__restrict__ mu_z, float *__restrict__ var_z) {
+    __shared__ float s_mean[FT_MAX_MAPS], s_var[FT_MAX_MAPS];
+    const int w4 = wihi >> 2;
+    const size_t first = (size_t)blockIdx.x * (FT_ITER * TPB);
+    const size_t end = min(n4, first + (size_t)FT_ITER * TPB);
+    const size_t map_first = first / w4, map_last = (end - 1) / w4;
+    const int maps = (int)(map_last - map_first + 1);
+    for (int t = threadIdx.x; t < maps; t += TPB) {
+        const size_t map = map_first + t;
+        const int c = (int)(map % fi);
+        float n = 0.f, mean = 0.f, m2 = 0.f, sum_var = 0.f;
+        for (int q = 0; q < chunks; q++) {
+            const float *o = part + ((size_t)c * chunks + q) * 4;
+            const float nb = o[0];
+            if (nb <= 0.f) continue;
+            const float delta = o[1] - mean, tot = n + nb;
+            mean += delta * (nb / tot);
+            m2 += o[2] + delta * delta * (n * nb / tot);
+            n = tot;
+            sum_var += o[3];
+        }
+        const float var = (m2 + sum_var) / (n - 1.f);
+        s_mean[t] = mean;
+        s_var[t] = var;
+        if (map < (size_t)fi && map * w4 >= first) {   // image 0: once per channel
+            mu_s[c] = mean;
+            var_s[c] = var;
+            mu_ra[c] = mu_ra[c] * momentum + mean * (1.f - momentum);
+            var_ra[c] = var_ra[c] * momentum + var * (1.f - momentum);
+        }
+    }
+    __syncthreads();
+    const bool has_b = mu_b != nullptr, has_r = mu_res != nullptr;
+#pragma unroll
+    for (int it = 0; it < FT_ITER; it++) {
+        const size_t i4 = first + (size_t)it * TPB + threadIdx.x;
+        if (i4 >= end) break;
+        const size_t i = i4 * 4, map = i4 / w4;
+        const int c = (int)(map % fi), li = (int)(map - map_first);
+        const float4 ma = *reinterpret_cast<const float4 *>(mu_a + i);
+        const float4 va = *reinterpret_cast<const float4 *>(var_a + i);
+        float4 rm = make_float4(0.f, 0.f, 0.f, 0.f), rv = rm;
+        if (has_r) {
+            rm = *reinterpret_cast<const float4 *>(mu_res + i);
+            rv = *reinterpret_cast<const float4 *>(var_res + i);
+        }
+        const float inv = 1.0f / sqrtf(s_var[li] + epsilon);
+        const float mw = mu_w[c], vw = var_w[c], mean = s_mean[li];
+        const float bm = has_b ? mu_b[c] : 0.f, bv = has_b ? var_b[c] : 0.f;
+        auto one = [&](float a, float v, float r0, float r1, float &mz, float &vz) {
+            const float d = a - mean;
+            mz = inv * d * mw;
+            vz = inv * inv * (v * (mw * mw + vw) + vw * d * d);
+            if (has_b) {
+                mz += bm;
+                vz += bv;
+            }
+            if (has_r) {
+                mz += r0;
+                vz += r1;
+            }
+        };
+        float4 om, ov;
+        one(ma.x, va.x, rm.x, rv.x, om.x, ov.x);
+        one(ma.y, va.y, rm.y, rv.y, om.y, ov.y);
+        one(ma.z, va.z, rm.z, rv.z, om.z, ov.z);
+        one(ma.w, va.w, rm.w, rv.w, om.w, ov.w);
+        *reinterpret_cast<float4 *>(mu_z + i) = om;
+        *reinterpret_cast<float4 *>(var_z + i) = ov;
+    }
+}
+
 // Backward of one (chunk, channel): the state innovations element by element,
 // and partial sums of the four parameter innovations of the channel.
 template <bool VEC>
@@ -438,6 +527,38 @@ hipError_t launch_batchnorm2d_stats(const float *mu_a, const float *var_a, int w
                            mu_a, var_a, wihi, fi, B, per, scratch);
     hipLaunchKernelGGL(bn_stats_final_kernel, dim3((fi + 63) / 64), dim3(64), 0, stream, scratch,
                        fi, chunks, momentum, mu_s, var_s, mu_ra, var_ra);
+    return hipGetLastError();
+}
+
+int g_bn_fused_train = 1;
+
+// Statistics + normalisation of a training-mode forward: two launches where the 16-byte
+// path applies (partial statistics, then the forward that merges them itself), otherwise
+// the three of launch_batchnorm2d_stats + launch_batchnorm2d_fwd.
+hipError_t launch_batchnorm2d_fwd_train(const float *mu_w, const float *var_w, const float *mu_b,
+                                        const float *var_b, const float *mu_a, const float *var_a,
+                                        const float *mu_res, const float *var_res, float momentum,
+                                        float epsilon, int wihi, int fi, int B, float *scratch,
+                                        float *mu_s, float *var_s, float *mu_ra, float *var_ra,
+                                        float *mu_z, float *var_z, hipStream_t stream) {
+    const bool vec = wihi % 4 == 0 && wihi >= 16 && aligned16(mu_a) && aligned16(var_a) &&
+                     aligned16(mu_z) && aligned16(var_z) && aligned16(mu_res) && aligned16(var_res);
+    if (!vec || !g_bn_fused_train) {
+        hipError_t e = launch_batchnorm2d_stats(mu_a, var_a, wihi, fi, B, momentum, scratch, mu_s,
+                                                var_s, mu_ra, var_ra, stream);
+        if (e != hipSuccess) return e;
+        return launch_batchnorm2d_fwd(mu_w, var_w, mu_b, var_b, mu_a, var_a, mu_s, var_s, epsilon,
+                                      wihi, fi, B, mu_z, var_z, stream, mu_res, var_res);
+    }
+    int per = 0;
+    const int chunks = bn_chunks(fi, B, &per);
+    hipLaunchKernelGGL(bn_stats_partial_kernel<true>, dim3(chunks, fi), dim3(TPB), 0, stream, mu_a,
+                       var_a, wihi, fi, B, per, scratch);
+    const size_t n4 = (size_t)B * fi * wihi / 4;
+    hipLaunchKernelGGL(bn_fwd_train_vec_kernel, dim3(blocks_for(n4, FT_ITER * TPB)), dim3(TPB), 0,
+                       stream, mu_w, var_w, mu_b, var_b, mu_a, var_a, scratch, chunks, momentum,
+                       epsilon, wihi, fi, n4, mu_res, var_res, mu_s, var_s, mu_ra, var_ra, mu_z,
+                       var_z);
     return hipGetLastError();
 }
 

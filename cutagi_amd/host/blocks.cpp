@@ -241,22 +241,22 @@ void BatchNorm2dHip::forward(BaseHiddenStates &input_states, BaseHiddenStates &o
     if (this->training) {
         if (batch_size * wihi < 2)
             LOG(LogLevel::ERROR, "BatchNorm2d needs more than one value per feature in training");
-        TAGI_OK_OR_THROW(tagi_batchnorm2d_stats(in->d_mu_a, in->d_var_a, wihi, fi, batch_size,
-                                                momentum, d_mu_norm_batch, d_var_norm_batch,
-                                                d_mu_ra, d_var_ra, host_stream()));
-    }
-    const float *mu_target = this->training ? d_mu_norm_batch : d_mu_ra;
-    const float *var_target = this->training ? d_var_norm_batch : d_var_ra;
-    if (res_mu != nullptr)
+        // statistics, running averages and the normalisation (+ the residual add) in one call
+        TAGI_OK_OR_THROW(tagi_batchnorm2d_fwd_train(
+            d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a, in->d_var_a, res_mu, res_var,
+            bias ? 1 : 0, momentum, epsilon, wihi, fi, batch_size, d_mu_norm_batch, d_var_norm_batch,
+            d_mu_ra, d_var_ra, out->d_mu_a, out->d_var_a, host_stream()));
+    } else if (res_mu != nullptr) {
         TAGI_OK_OR_THROW(tagi_batchnorm2d_fwd_res(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a,
-                                                  in->d_var_a, mu_target, var_target, res_mu,
-                                                  res_var, bias ? 1 : 0, epsilon, wihi, fi,
-                                                  batch_size, out->d_mu_a, out->d_var_a, host_stream()));
-    else
+                                                  in->d_var_a, d_mu_ra, d_var_ra, res_mu, res_var,
+                                                  bias ? 1 : 0, epsilon, wihi, fi, batch_size,
+                                                  out->d_mu_a, out->d_var_a, host_stream()));
+    } else {
         TAGI_OK_OR_THROW(tagi_batchnorm2d_fwd(d_mu_w, d_var_w, d_mu_b, d_var_b, in->d_mu_a,
-                                              in->d_var_a, mu_target, var_target, bias ? 1 : 0,
-                                              epsilon, wihi, fi, batch_size, out->d_mu_a,
-                                              out->d_var_a, host_stream()));
+                                              in->d_var_a, d_mu_ra, d_var_ra, bias ? 1 : 0, epsilon,
+                                              wihi, fi, batch_size, out->d_mu_a, out->d_var_a,
+                                              host_stream()));
+    }
     out->jcb_ones = true;
     if (this->training) this->store_states_for_training_hip(*in, *out);
 }

@@ -410,6 +410,22 @@ int tagi_batchnorm2d_fwd_res(const float *mu_w, const float *var_w,
                              float epsilon, int wihi, int fi, int B, float *mu_z,
                              float *var_z, void *stream);
 
+/* A training-mode forward in one call: tagi_batchnorm2d_stats followed by
+ * tagi_batchnorm2d_fwd (mu_res == NULL) or tagi_batchnorm2d_fwd_res with the batch
+ * statistics, i.e. all of BatchNorm2dCuda::forward in training mode
+ * (src/batchnorm_layer_cuda.cu:915-959). The results are the same bits; where the
+ * 16-byte path applies the statistics are merged by the normalising kernel itself (two
+ * launches instead of three). mu_s / var_s receive the batch statistics (the backward
+ * pass needs them), mu_ra / var_ra are updated. Uses the workspace. */
+int tagi_batchnorm2d_fwd_train(const float *mu_w, const float *var_w,
+                               const float *mu_b, const float *var_b,
+                               const float *mu_a, const float *var_a,
+                               const float *mu_res /* may be NULL */,
+                               const float *var_res, int bias, float momentum,
+                               float epsilon, int wihi, int fi, int B, float *mu_s,
+                               float *var_s, float *mu_ra, float *var_ra,
+                               float *mu_z, float *var_z, void *stream);
+
 /* All of BatchNorm2dCuda::backward (src/batchnorm_layer_cuda.cu:969-1102) in one
  * call: state innovations (state_update) and the per-channel weight / bias
  * innovations (param_update; bias ones only when bias != 0). mu_a and jcb are the

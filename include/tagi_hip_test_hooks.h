@@ -33,7 +33,8 @@ extern "C" {
  * off; s2_all: the stencil kernels of the stride-2 layers - forward, state backward with
  * all four phases in one workgroup and its pair-wise fold, weight backward - which leaves
  * those layers on the table-driven kernels; "conv2d.bwd_pair": 0 gives the state and the
- * weight backward of tagi_conv2d_bwd launches of their own). */
+ * weight backward of tagi_conv2d_bwd launches of their own). "batchnorm.fused_train": 0
+ * gives tagi_batchnorm2d_fwd_train a launch of its own for the merge of the statistics. */
 int tagi_hip_tune(const char *key /* host */, int value);
 
 #ifdef __cplusplus

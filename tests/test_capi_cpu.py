@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(capi.lib, n), "missing export: " + n
         assert n in capi.SIGNATURES, "binding missing for: " + n
     assert sorted(capi.SIGNATURES) == names
-    assert capi.version() == 105
+    assert capi.version() == 106
 
 
 def test_error_strings_and_device_count():

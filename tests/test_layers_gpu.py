@@ -117,6 +117,67 @@ def test_batchnorm2d(oracle_lib, wihi, fi, B, bias):
     assert float(out[1].max()) <= 0 and float(out[3].max()) <= 0
 
 
+@pytest.mark.parametrize("wihi,fi,B", BN_SHAPES + [(16, 70, 9), (64, 256, 8), (20, 6, 3)])
+@pytest.mark.parametrize("bias", [True, False])
+@pytest.mark.parametrize("residual", [False, True])
+def test_batchnorm2d_training_forward_in_one_call(oracle_lib, wihi, fi, B, bias, residual):
+    """tagi_batchnorm2d_fwd_train = statistics, running averages, normalisation and the
+    optional residual add. Bit for bit what the separate entry points give (the fused
+    kernel repeats their arithmetic), with the merge of the statistics inside the
+    normalising kernel and as a launch of its own; and the oracle's result."""
+    import torch
+    from cutagi_amd import capi
+    d = batchnorm_inputs(wihi, fi, B, seed=3 * wihi + fi + B)
+    t = _dev(d)
+    n = B * fi * wihi
+    rng = np.random.default_rng(n)
+    res = None
+    if residual:
+        res = [torch.from_numpy(rng.standard_normal(n).astype(np.float32)).cuda(),
+               torch.from_numpy(rng.uniform(0.01, 0.5, n).astype(np.float32)).cuda()]
+    mb, vb = (t["mu_b"], t["var_b"]) if bias else (None, None)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def fused():
+        ra = [t["mu_ra"].clone(), t["var_ra"].clone()]
+        st = [torch.empty(fi, device="cuda"), torch.empty(fi, device="cuda")]
+        z = [torch.empty(n, device="cuda"), torch.empty(n, device="cuda")]
+        capi.check(capi.lib.tagi_batchnorm2d_fwd_train(
+            capi.ptr(t["mu_w"]), capi.ptr(t["var_w"]), capi.ptr(mb), capi.ptr(vb), capi.ptr(t["mu_a"]),
+            capi.ptr(t["var_a"]), capi.ptr(res[0]) if res else None, capi.ptr(res[1]) if res else None,
+            int(bias), 0.9, 1e-5, wihi, fi, B, capi.ptr(st[0]), capi.ptr(st[1]), capi.ptr(ra[0]),
+            capi.ptr(ra[1]), capi.ptr(z[0]), capi.ptr(z[1]), stream))
+        return st + ra + z
+
+    got = fused()
+    capi.tune("batchnorm.fused_train", 0)
+    try:
+        plain = fused()
+    finally:
+        capi.tune("batchnorm.fused_train", 1)
+    # the separate entry points
+    import cutagi_amd.functional as F
+    ra = [t["mu_ra"].clone(), t["var_ra"].clone()]
+    st = F.batchnorm2d_stats(t["mu_a"], t["var_a"], wihi, fi, B, 0.9, ra[0], ra[1])
+    z = [torch.empty(n, device="cuda"), torch.empty(n, device="cuda")]
+    if residual:
+        capi.check(capi.lib.tagi_batchnorm2d_fwd_res(
+            capi.ptr(t["mu_w"]), capi.ptr(t["var_w"]), capi.ptr(mb), capi.ptr(vb), capi.ptr(t["mu_a"]),
+            capi.ptr(t["var_a"]), capi.ptr(st[0]), capi.ptr(st[1]), capi.ptr(res[0]), capi.ptr(res[1]),
+            int(bias), 1e-5, wihi, fi, B, capi.ptr(z[0]), capi.ptr(z[1]), stream))
+    else:
+        z = list(F.batchnorm2d_fwd(t["mu_w"], t["var_w"], mb, vb, t["mu_a"], t["var_a"], st[0], st[1],
+                                   1e-5, wihi, fi, B))
+    names = ("mu_s", "var_s", "mu_ra", "var_ra", "mu_z", "var_z")
+    for name, a, b, c in zip(names, got, plain, list(st) + ra + z):
+        assert torch.equal(a, c), name + " (fused merge)"
+        assert torch.equal(b, c), name + " (merge as a launch of its own)"
+    ref_s = oracle_lib.batchnorm2d_stats(d["mu_a"], d["var_a"], wihi, fi, B, 0.9, d["mu_ra"],
+                                         d["var_ra"], 4)
+    for name, a, r in zip(names[:4], got[:4], ref_s):
+        assert_close(a.cpu().numpy(), r, name)
+
+
 def test_batchnorm2d_backward_switches(oracle_lib):
     import cutagi_amd.functional as F
     import torch
