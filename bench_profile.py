@@ -62,14 +62,14 @@ def commit_stamp(given):
 # bench.py runs its main workload (Linear 4096^2, batch 256) first and the batch-32 / 64
 # workloads of the same layer later on the same tile kernels: dispatches of a kernel that
 # belongs to the main workload count only up to the first skinny-batch kernel.
-MAIN_ENDS_AT = "gemv_fwd_kernel"
+MAIN_ENDS_AT = ("gemv_fwd_kernel", "gemv16_fwd_kernel")
 
 
 def main_workload_only(rows, name_key):
     """rows (dicts with Start_Timestamp) -> those that precede the first skinny-batch dispatch."""
     rows = sorted(rows, key=lambda r: int(r["Start_Timestamp"]))
     for i, r in enumerate(rows):
-        if short(r[name_key]).startswith(MAIN_ENDS_AT):
+        if short(r[name_key]).startswith(MAIN_ENDS_AT):  # (a tuple of prefixes)
             return rows[:i]
     return rows
 
@@ -105,24 +105,27 @@ KERNELS = [
     ("linear_dw_side_kernel<LinearProblem<2, true, true, true>, 64, 128, 2, 4>",
      "Linear 4096^2 B=256 delta_w + delta_z fold + delta_b (inside the backward call)",
      (3 * K2 * K2 + B2 * K2 + 2 * B2 * K2) * 4 / MB, 4.0 * B2 * K2 * K2),
-    ("gemv_fwd_kernel<2, 2, 1>", "Linear 8192^2 B=8 forward", 2 * K3 * K3 * 4 / MB, 6.0 * B3 * K3 * K3),
+    ("gemv16_fwd_kernel<1, 1>", "Linear 8192^2 B=8, 12 and 16 forward", 2 * K3 * K3 * 4 / MB, 6.0 * 12 * K3 * K3),
     ("gemv_dz_kernel<2>", "Linear 8192^2 B=8 delta_z", K3 * K3 * 4 / MB, 4.0 * B3 * K3 * K3),
     ("gemv_dw_kernel<8, true>", "Linear 8192^2 B=8 delta_w (+delta_b)", 3 * K3 * K3 * 4 / MB, 4.0 * B3 * K3 * K3),
-    ("gemv16_fwd_kernel<1>", "Linear 8192^2 B=12 and B=16 forward", 2 * K3 * K3 * 4 / MB, 6.0 * 14 * K3 * K3),
-    ("gemv16_dz_kernel<1>", "Linear 8192^2 B=12 and B=16 delta_z", K3 * K3 * 4 / MB, 4.0 * 14 * K3 * K3),
+    ("gemv16_dz_kernel<1, false>", "Linear 8192^2 B=12 and B=16 delta_z", K3 * K3 * 4 / MB, 4.0 * 14 * K3 * K3),
     ("gemv_dw_kernel<16, true>", "Linear 8192^2 B=12 and B=16 delta_w (+delta_b)", 3 * K3 * K3 * 4 / MB, 4.0 * 14 * K3 * K3),
-    ("gemv16_fwd_kernel<2>", "Linear 4096^2 B=32 forward", 2 * K2 * K2 * 4 / MB, 6.0 * 32 * K2 * K2),
+    ("gemv16_fwd_kernel<2, 2>", "Linear 4096^2 B=32 forward", 2 * K2 * K2 * 4 / MB, 6.0 * 32 * K2 * K2),
     ("conv_stencil_kernel<false, 32>", "Conv2d 3x3 64->64 @32x32 B=128 forward", 4 * CONV_ACT, 6.0 * 64 * 131072 * 576),
     ("conv_stencil_bwd_pair_kernel<32>", "Conv2d delta_z + delta_w (one launch)", 6 * CONV_ACT,
      8.0 * 64 * 131072 * 576),
 ]
 MAIN_KERNELS = tuple(k for k, w, _, _ in KERNELS if "B=256" in w)
 # bench.py's table: (workload, phase) -> kernel
+_BY_WORKLOAD = {w: k for k, w, _, _ in KERNELS}
 TRAFFIC_KEYS = [
     (("gemm", "fwd"), KERNELS[0][0]), (("gemm", "bwd_dw"), KERNELS[3][0]), (("gemm", "bwd_dz"), KERNELS[1][0]),
-    (("skinny", "fwd"), KERNELS[4][0]), (("skinny", "bwd_dz"), KERNELS[5][0]), (("skinny", "bwd_dw"), KERNELS[6][0]),
-    (("skinny12", "fwd"), KERNELS[7][0]), (("skinny12", "bwd_dz"), KERNELS[8][0]), (("skinny12", "bwd_dw"), KERNELS[9][0]),
-    (("conv", "fwd"), KERNELS[11][0]),
+    (("skinny", "fwd"), _BY_WORKLOAD["Linear 8192^2 B=8, 12 and 16 forward"]),
+    (("skinny", "bwd_dz"), _BY_WORKLOAD["Linear 8192^2 B=8 delta_z"]),
+    (("skinny", "bwd_dw"), _BY_WORKLOAD["Linear 8192^2 B=8 delta_w (+delta_b)"]),
+    (("skinny12", "bwd_dz"), _BY_WORKLOAD["Linear 8192^2 B=12 and B=16 delta_z"]),
+    (("skinny12", "bwd_dw"), _BY_WORKLOAD["Linear 8192^2 B=12 and B=16 delta_w (+delta_b)"]),
+    (("conv", "fwd"), _BY_WORKLOAD["Conv2d 3x3 64->64 @32x32 B=128 forward"]),
 ]
 
 

@@ -109,6 +109,7 @@ struct Tuning {
     // walk rows from the end, high bit: XCD-aware column mapping
     int gemv_rev = -1;
     int gemv16 = -1;    // 0: 9..16 samples on the 4x4x1 kernels too
+    int gemv16_min = -1;  // smallest batch the 16-wide forward takes (default 5)
     int wide32 = -1;    // 0: 17..32 samples on the tiled kernels; 2: state backward streams too
     int dw_side = -1;   // 0: bias innovations and the state-backward fold as launches of their own
     // >= 0: the smallest weight matrix (elements) the streaming kernels take, whatever the
@@ -338,8 +339,10 @@ int tagi_hip_tune(const char *key, int value) {
     else if (!strcmp(key, "linear.gemv.reverse")) g_tune.gemv_rev = value;
     else if (!strcmp(key, "linear.dw_side")) g_tune.dw_side = value;
     else if (!strcmp(key, "linear.gemv16")) g_tune.gemv16 = value;
+    else if (!strcmp(key, "linear.gemv16.min_batch")) g_tune.gemv16_min = value;
     else if (!strcmp(key, "linear.gemv32")) g_tune.wide32 = value;
-    else if (!strcmp(key, "linear.gemv16.fwd_lines")) g_gemv16_fwd_lines = value < 0 ? 0 : value;
+    else if (!strcmp(key, "linear.gemv16.dz_streaming")) g_gemv16_dz_streaming = value < 0 ? 0 : value;
+    else if (!strcmp(key, "linear.gemv16.whole_lines")) g_gemv16_fwd_whole_lines = value;
     else if (!strcmp(key, "linear.stream_min_weights")) g_tune.stream_min_weights = value;
     else if (!strcmp(key, "linear.small")) g_tune.small = value;
     else return TAGI_ERR_INVALID_ARG;
@@ -370,7 +373,8 @@ static int linear_fwd_impl(const float *mu_w, const float *var_w, const float *m
         return TAGI_OK;
     }
     const bool streams = streams_weights(STREAM_FWD, N, K, B);
-    if (B > 8 && B <= wide_max_batch() && vec && g_tune.gemv16 != 0 && streams) {
+    if (B >= (g_tune.gemv16_min > 0 ? g_tune.gemv16_min : 5) && B <= wide_max_batch() && vec &&
+        g_tune.gemv16 != 0 && streams) {
         // 9..32 samples: the 16-wide streaming kernel (two sample groups beyond 16)
         const int blocks = ceil_div(N, gemv16_fwd_rows_per_block());
         const int step = gemv16_fwd_k_step();

@@ -17,6 +17,7 @@
 // Reduction slices (gridDim.y) write partial sums [slice][B][cols]; the caller
 // folds them, together with the bias or Jacobian epilogue, in reduce_splits.
 #include "tagi_internal.h"
+#include "tagi_stage.h"
 
 namespace tagi {
 
@@ -103,17 +104,6 @@ __global__ __launch_bounds__(FWD_WAVES * 64) void gemv_fwd_kernel(
     const int rot = (swz & 2) ? ((row_block * FWD_WAVES + wave) * 2 * KSTEP) % k_per_split : 0;
 
     // stage the slice of the activations: [sample][k], zero beyond B and kr
-    const int k4s = k_per_split / 4;
-    for (int e = tid; e < 4 * H * k4s; e += FWD_WAVES * 64) {
-        const int b = e / k4s, k = (e - b * k4s) * 4;
-        float4 m = zero4(), v = zero4();
-        if (b < B && k < kr) {
-            m = ld4(mu_a + (size_t)b * K + k_begin + k);
-            v = ld4(var_a + (size_t)b * K + k_begin + k);
-        }
-        *reinterpret_cast<float4 *>(s_mu + b * S + k) = m;
-        *reinterpret_cast<float4 *>(s_var + b * S + k) = v;
-    }
 
     // Weight loads are never predicated (a predicated load costs a branch and
     // makes the compiler wait for every outstanding load): rows beyond N read row
@@ -186,6 +176,12 @@ __global__ __launch_bounds__(FWD_WAVES * 64) void gemv_fwd_kernel(
     const int span = (swz & 2) ? k_per_split : (kr + 2 * KSTEP - 1) / (2 * KSTEP) * (2 * KSTEP);
     auto wrap = [&](int p) { return p >= k_per_split ? p - k_per_split : p; };
     load(sm[0], sv[0], rot);
+    __builtin_amdgcn_sched_barrier(0);  // the first weights are on their way while the slice is staged
+    stage_slice_pairs<FWD_WAVES * 64>(mu_a, var_a, 4 * H, B, K, k_begin, kr, k_per_split, tid,
+                                      [&](int b, int k, float4 m, float4 v) {
+                                          *reinterpret_cast<float4 *>(s_mu + b * S + k) = m;
+                                          *reinterpret_cast<float4 *>(s_var + b * S + k) = v;
+                                      });
     __syncthreads();
     for (int kb = 0; kb < span; kb += 2 * KSTEP) {
         // (the last pair has nothing left to prefetch: it re-reads the stage that
@@ -303,17 +299,6 @@ __global__ __launch_bounds__(DZ_WAVES * 64) void gemv_dz_kernel(
             x[u] = ldw_dz(w + (size_t)min(n_begin + r + u, n_last) * K);
     };
     // stage this slice of the innovations: [sample][n], zero beyond B and nr
-    const int n4s = n_per_split / 4;
-    for (int e = tid; e < 4 * H * n4s; e += DZ_WAVES * 64) {
-        const int b = e / n4s, n = (e - b * n4s) * 4;
-        float4 m = zero4(), v = zero4();
-        if (b < B && n < nr) {
-            m = ld4(dmu + (size_t)b * N + n_begin + n);
-            v = ld4(dvar + (size_t)b * N + n_begin + n);
-        }
-        *reinterpret_cast<float4 *>(s_dm + b * S + n) = m;
-        *reinterpret_cast<float4 *>(s_dv + b * S + n) = v;
-    }
 
     floatx4 acc0[4][H], acc1[4][H];
 #pragma unroll
@@ -349,6 +334,12 @@ __global__ __launch_bounds__(DZ_WAVES * 64) void gemv_dz_kernel(
     };
 
     load(st[0], r_lo);
+    __builtin_amdgcn_sched_barrier(0);  // the first weights are on their way while the slice is staged
+    stage_slice_pairs<DZ_WAVES * 64>(dmu, dvar, 4 * H, B, N, n_begin, nr, n_per_split, tid,
+                                     [&](int b, int n, float4 m, float4 v) {
+                                         *reinterpret_cast<float4 *>(s_dm + b * S + n) = m;
+                                         *reinterpret_cast<float4 *>(s_dv + b * S + n) = v;
+                                     });
     __syncthreads();
     for (int r = r_lo; r < r_hi; r += 2 * STAGE) {
         load(st[1], r + STAGE);

@@ -10,6 +10,7 @@
 //
 // The weight backward of tagi_gemv.hip serves every B <= 16 and is not repeated.
 #include "tagi_internal.h"
+#include "tagi_stage.h"
 
 namespace tagi {
 
@@ -19,6 +20,32 @@ namespace {
 
 __device__ __forceinline__ float4 ld4(const float *p) {
     return *reinterpret_cast<const float4 *>(p);
+}
+__device__ __forceinline__ float4 ldnt4(const float *p) {
+    const floatx4 v = __builtin_nontemporal_load(reinterpret_cast<const floatx4 *>(p));
+    return make_float4(v[0], v[1], v[2], v[3]);
+}
+// Lanes of the banks in BANKS (a bank = four lanes of a row of sixteen) take `from` of
+// the lane eight further round the row; the others keep `keep`.
+template <int BANKS>
+__device__ __forceinline__ float take_ror8(float keep, float from) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(keep), __float_as_int(from),
+                                                      0x128 /* row_ror:8 */, 0xF, BANKS, false));
+}
+// a: loaded by lane (i, kk) from row i % 8 of the group, b: from row 8 + i % 8, both at
+// chunk kk + 4 * (i / 8) of the 32-element window. Afterwards a is chunk kk and b chunk
+// kk + 4 of row i: lanes i < 8 keep a and take b from the a of lane i + 8, lanes i >= 8
+// keep b and take a from the b of lane i - 8.
+__device__ __forceinline__ void swap_halves(float4 &a, float4 &b) {
+    const float4 a0 = a;
+    a.x = take_ror8<0xC>(a0.x, b.x);
+    a.y = take_ror8<0xC>(a0.y, b.y);
+    a.z = take_ror8<0xC>(a0.z, b.z);
+    a.w = take_ror8<0xC>(a0.w, b.w);
+    b.x = take_ror8<0x3>(b.x, a0.x);
+    b.y = take_ror8<0x3>(b.y, a0.y);
+    b.z = take_ror8<0x3>(b.z, a0.z);
+    b.w = take_ror8<0x3>(b.w, a0.w);
 }
 __device__ __forceinline__ float4 zero4() { return make_float4(0.f, 0.f, 0.f, 0.f); }
 __device__ __forceinline__ float comp(const float4 &v, int t) {
@@ -31,7 +58,7 @@ __device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
 }
 
-constexpr int W16_WAVES = 8;
+constexpr int W16_WAVES = 16;   // forward: one workgroup of sixteen waves per CU
 constexpr int W16_SAMPLES = 16;
 
 // ---------------------------------------------------------------------------
@@ -54,7 +81,10 @@ constexpr int F16_PAD = 4;       // LDS row stride % 32 == 4
 
 // NG: groups of 16 samples (1: up to 16 samples, 2: up to 32 - every weight fragment
 // then feeds two MFMAs, one per group, from the same registers).
-template <int NG>
+// WL: load instructions cover whole 128-byte lines (8 rows x 128 bytes each, two of them
+// for the wave's sixteen rows) with streaming loads; lanes i and i ^ 8 then exchange one
+// float4 each to arrive at the operand layout (see swap_halves).
+template <int NG, int WL>
 __global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_kernel(
     const float *__restrict__ mu_w, const float *__restrict__ var_w,
     const float *__restrict__ mu_a, const float *__restrict__ var_a, int K, int N, int B,
@@ -86,30 +116,24 @@ __global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_kernel(
     const int rot = ((row_block * W16_WAVES + wave) * 2 * KSTEP) % k_per_split;
 
     // stage the slice of the activations: [sample][k], zero beyond B and kr
-    const int k4s = k_per_split / 4;
-    for (int e = tid; e < NS * k4s; e += W16_WAVES * 64) {
-        const int b = e / k4s, k = (e - b * k4s) * 4;
-        float4 m = zero4(), v = zero4();
-        if (b < B && k < kr) {
-            m = ld4(mu_a + (size_t)b * K + k_begin + k);
-            v = ld4(var_a + (size_t)b * K + k_begin + k);
-        }
-        *reinterpret_cast<float4 *>(s_mu + b * S + k) = m;
-        *reinterpret_cast<float4 *>(s_var + b * S + k) = v;
-    }
 
     // Weight loads are never predicated: rows beyond N read row N-1 and are
     // dropped at the end, reduction elements beyond the slice read the last float4
     // of the row and meet zero activations.
     const int n0 = row_block * ROWS_PER_BLOCK + wave * (RG * 16);
+    // WL: wm / wv point at row (i % 8) of the group's first eight rows, the second
+    // eight lie `hi` floats further; the lane's chunk of the 32-element window is
+    // kk + 4 * (i / 8)
     const float *wm[RG], *wv[RG];
+    size_t hi[RG];
 #pragma unroll
     for (int rg = 0; rg < RG; rg++) {
-        const int row = min(n0 + 16 * rg + i, N - 1);
+        const int row = min(n0 + 16 * rg + (WL ? (i & 7) : i), N - 1);
         wm[rg] = mu_w + (size_t)row * K;
         wv[rg] = var_w + (size_t)row * K;
+        hi[rg] = (size_t)(min(n0 + 16 * rg + 8 + (i & 7), N - 1) - row) * K;
     }
-    const int k_lane = k_begin + 4 * kk, k_last = K - 4;
+    const int k_lane = k_begin + 4 * (WL ? kk + 4 * (i >> 3) : kk), k_last = K - 4;
 
     // the two variance terms have accumulators of their own, so that no MFMA waits
     // for the one issued just before it
@@ -125,6 +149,21 @@ __global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_kernel(
 
     float4 sm[2][RG][C], sv[2][RG][C];
     auto load = [&](float4(&m)[RG][C], float4(&v)[RG][C], int kb) {
+        if (WL) {
+            static_assert(!WL || C % 2 == 0, "a 128-byte line is two chunks of 16 elements");
+#pragma unroll
+            for (int c = 0; c < C; c += 2) {
+                const int k = min(k_lane + kb + 16 * c, k_last);
+#pragma unroll
+                for (int rg = 0; rg < RG; rg++) {
+                    m[rg][c] = WL == 1 ? ldnt4(wm[rg] + k) : ld4(wm[rg] + k);
+                    v[rg][c] = WL == 1 ? ldnt4(wv[rg] + k) : ld4(wv[rg] + k);
+                    m[rg][c + 1] = WL == 1 ? ldnt4(wm[rg] + hi[rg] + k) : ld4(wm[rg] + hi[rg] + k);
+                    v[rg][c + 1] = WL == 1 ? ldnt4(wv[rg] + hi[rg] + k) : ld4(wv[rg] + hi[rg] + k);
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int c = 0; c < C; c++) {
             const int k = min(k_lane + kb + 16 * c, k_last);
@@ -135,7 +174,16 @@ __global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_kernel(
             }
         }
     };
-    auto multiply = [&](const float4(&cm)[RG][C], const float4(&cv)[RG][C], int kb) {
+    auto multiply = [&](float4(&cm)[RG][C], float4(&cv)[RG][C], int kb) {
+        if (WL) {
+#pragma unroll
+            for (int c = 0; c < C; c += 2)
+#pragma unroll
+                for (int rg = 0; rg < RG; rg++) {
+                    swap_halves(cm[rg][c], cm[rg][c + 1]);
+                    swap_halves(cv[rg][c], cv[rg][c + 1]);
+                }
+        }
 #pragma unroll
         for (int c = 0; c < C; c++) {
             const int at = kb + 16 * c + 4 * kk;
@@ -167,6 +215,12 @@ __global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_kernel(
     // rotated by `rot`
     auto wrap = [&](int p) { return p >= k_per_split ? p - k_per_split : p; };
     load(sm[0], sv[0], rot);
+    __builtin_amdgcn_sched_barrier(0);  // the first weights are on their way while the slice is staged
+    stage_slice_pairs<W16_WAVES * 64>(mu_a, var_a, NS, B, K, k_begin, kr, k_per_split, tid,
+                                      [&](int b, int k, float4 m, float4 v) {
+                                          *reinterpret_cast<float4 *>(s_mu + b * S + k) = m;
+                                          *reinterpret_cast<float4 *>(s_var + b * S + k) = v;
+                                      });
     __syncthreads();
     for (int kb = 0; kb < k_per_split; kb += 2 * KSTEP) {
         const int p0 = wrap(rot + kb), p1 = p0 + KSTEP;
@@ -209,157 +263,6 @@ __global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// Forward, loading whole cache lines (not the default: it measures the same as the
-// kernel above, which says that half-line requests are not what holds that one at
-// 5 TB/s). The MFMA wants lane (i, kk) to hold row i,
-// which makes a load instruction of the kernel above touch sixteen rows, half a
-// 128-byte line each. Here a load instruction covers 4 rows x 256 bytes instead
-// (lane (r = l/16, q = l%16): row 4*j + r of the wave's sixteen, reduction elements
-// 4*q .. 4*q+3 of a 64-element stage, j = 0..3), and the wave turns the stage into
-// the operand layout through a small LDS tile of its own, [16 rows][64 + 4]: four
-// 16-byte writes and four 16-byte reads per lane and array, no barrier (the tile
-// belongs to the wave; LDS operations of a wave complete in order). Component t of
-// the float4 a lane reads back is A[i][kk] of MFMA t as before.
-// ---------------------------------------------------------------------------
-constexpr int T16_STAGE = 64;             // reduction elements per stage
-constexpr int T16_TS = T16_STAGE + 4;     // row stride of the transposition tile
-constexpr int T16_TILE = 16 * T16_TS;     // floats per array and wave
-constexpr int T16_DEPTH = 2;              // register stages (4 measured slower: 131 vs 114 us at 8192^2, batch 16)
-
-__global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_lines_kernel(
-    const float *__restrict__ mu_w, const float *__restrict__ var_w,
-    const float *__restrict__ mu_a, const float *__restrict__ var_a, int K, int N, int B,
-    int k_per_split, int splits, float *__restrict__ ws0, float *__restrict__ ws1) {
-    extern __shared__ __attribute__((aligned(16))) float lds[];
-    constexpr int ROWS_PER_BLOCK = W16_WAVES * 16;
-    const int S = k_per_split + F16_PAD;
-    float *s_mu = lds, *s_var = lds + W16_SAMPLES * S;
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int i = lane & 15, kk = lane >> 4;  // operand layout: row i, reduction slot kk
-    float *t_mu = lds + 2 * W16_SAMPLES * S + wave * 2 * T16_TILE, *t_var = t_mu + T16_TILE;
-    int row_block, split;
-    const int id = blockIdx.x, row_blocks = gridDim.x / splits;
-    if (row_blocks % 8 == 0) {
-        const int xcd = id & 7, local = id >> 3;
-        split = local % splits;
-        row_block = (local / splits) * 8 + xcd;
-    } else {
-        row_block = id % row_blocks;
-        split = id / row_blocks;
-    }
-    const int k_begin = split * k_per_split;
-    const int kr = min(K, k_begin + k_per_split) - k_begin;
-    const int rot = ((row_block * W16_WAVES + wave) * 2 * T16_STAGE) % k_per_split;
-
-    const int k4s = k_per_split / 4;
-    for (int e = tid; e < W16_SAMPLES * k4s; e += W16_WAVES * 64) {
-        const int b = e / k4s, k = (e - b * k4s) * 4;
-        float4 m = zero4(), v = zero4();
-        if (b < B && k < kr) {
-            m = ld4(mu_a + (size_t)b * K + k_begin + k);
-            v = ld4(var_a + (size_t)b * K + k_begin + k);
-        }
-        *reinterpret_cast<float4 *>(s_mu + b * S + k) = m;
-        *reinterpret_cast<float4 *>(s_var + b * S + k) = v;
-    }
-
-    // load layout: lane (r = kk, q = i) -> rows 4*j + r, elements 4*q ..; rows beyond N
-    // read row N-1 and are dropped at the end, elements beyond the slice read the last
-    // float4 of the row and meet zero activations
-    const int n0 = row_block * ROWS_PER_BLOCK + wave * 16;
-    const float *wm[4], *wv[4];
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int row = min(n0 + 4 * j + kk, N - 1);
-        wm[j] = mu_w + (size_t)row * K;
-        wv[j] = var_w + (size_t)row * K;
-    }
-    const int k_lane = k_begin + 4 * i, k_last = K - 4;
-
-    floatx4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0, acc2 = acc0;
-
-    float4 gm[T16_DEPTH][4], gv[T16_DEPTH][4];
-#define TAGI_T16_LOAD(buf, kb)                                      \
-    do {                                                            \
-        const int k_ = min(k_lane + (kb), k_last);                  \
-        _Pragma("unroll") for (int j = 0; j < 4; j++) {             \
-            gm[buf][j] = ld4(wm[j] + k_);                           \
-            gv[buf][j] = ld4(wv[j] + k_);                           \
-        }                                                           \
-    } while (0)
-    // registers -> the wave's tile -> operand layout -> MFMAs, one stage
-#define TAGI_T16_MULTIPLY(buf, kb)                                                               \
-    do {                                                                                         \
-        _Pragma("unroll") for (int j = 0; j < 4; j++) {                                          \
-            *reinterpret_cast<float4 *>(t_mu + (4 * j + kk) * T16_TS + 4 * i) = gm[buf][j];      \
-            *reinterpret_cast<float4 *>(t_var + (4 * j + kk) * T16_TS + 4 * i) = gv[buf][j];     \
-        }                                                                                        \
-        __builtin_amdgcn_wave_barrier(); /* other lanes' writes are read below */                \
-        _Pragma("unroll") for (int c = 0; c < 4; c++) {                                          \
-            const int at = (kb) + 16 * c + 4 * kk;                                               \
-            const float4 w = *reinterpret_cast<const float4 *>(t_mu + i * T16_TS + 16 * c + 4 * kk);  \
-            const float4 u = *reinterpret_cast<const float4 *>(t_var + i * T16_TS + 16 * c + 4 * kk); \
-            const float4 am = *reinterpret_cast<const float4 *>(s_mu + i * S + at);              \
-            const float4 av = *reinterpret_cast<const float4 *>(s_var + i * S + at);             \
-            const float4 as = make_float4(av.x + am.x * am.x, av.y + am.y * am.y,                \
-                                          av.z + am.z * am.z, av.w + am.w * am.w);               \
-            const float4 q = sq4(w);                                                             \
-            _Pragma("unroll") for (int t = 0; t < 4; t++) {                                      \
-                acc0 = mfma16(comp(w, t), comp(am, t), acc0);                                    \
-                acc1 = mfma16(comp(u, t), comp(as, t), acc1);                                    \
-                acc2 = mfma16(comp(q, t), comp(av, t), acc2);                                    \
-            }                                                                                    \
-        }                                                                                        \
-        __builtin_amdgcn_wave_barrier(); /* the tile is rewritten by the next stage */           \
-    } while (0)
-
-    // T16_DEPTH register stages in turn: while stage s is multiplied, the loads of the
-    // next T16_DEPTH - 1 stages are in flight (one workgroup per CU: the registers are
-    // there, and it is what keeps enough bytes on their way). Positions are inside the
-    // slice, rotated by `rot`; the last stages prefetch positions that wrap around
-    // (cached, never multiplied).
-    auto pos = [&](int p) {
-        p += rot;
-        while (p >= k_per_split) p -= k_per_split;
-        return p;
-    };
-#pragma unroll
-    for (int u = 0; u < T16_DEPTH - 1; u++) TAGI_T16_LOAD(u, pos(u * T16_STAGE));
-    __syncthreads();
-    for (int kb = 0; kb < k_per_split; kb += T16_DEPTH * T16_STAGE) {
-#pragma unroll
-        for (int u = 0; u < T16_DEPTH; u++) {
-            TAGI_T16_LOAD((u + T16_DEPTH - 1) % T16_DEPTH, pos(kb + (u + T16_DEPTH - 1) * T16_STAGE));
-            __builtin_amdgcn_sched_barrier(0);
-            TAGI_T16_MULTIPLY(u, pos(kb + u * T16_STAGE));
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
-#undef TAGI_T16_LOAD
-#undef TAGI_T16_MULTIPLY
-
-    // register v of lane l: row n0 + 4*(l/16) + v, sample l%16
-    const int b = lane & 15;
-    if (b < B) {
-        const int n = n0 + 4 * (lane >> 4);
-        const size_t at = ((size_t)split * B + b) * N + n;
-        const floatx4 m = acc0, v = acc1 + acc2;
-        if ((N & 3) == 0 && n + 3 < N) {
-            *reinterpret_cast<float4 *>(ws0 + at) = make_float4(m[0], m[1], m[2], m[3]);
-            *reinterpret_cast<float4 *>(ws1 + at) = make_float4(v[0], v[1], v[2], v[3]);
-        } else {
-#pragma unroll
-            for (int c = 0; c < 4; c++)
-                if (n + c < N) {
-                    ws0[at + c] = m[c];
-                    ws1[at + c] = v[c];
-                }
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------
 // State backward. A wave owns 64 consecutive input columns; the eight waves of a
 // workgroup sit side by side (512 columns) and walk the same slice of output
 // rows, so the staged innovations of the slice serve all of them and no wave
@@ -373,10 +276,14 @@ __global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_lines_kernel(
 // ---------------------------------------------------------------------------
 constexpr int Z16_ST = 4;      // 4-row steps per register stage (= steps per LDS float4)
 constexpr int Z16_PADQ = 1;    // plane stride per/4 + 4: spreads the kk planes over the banks
-constexpr int Z16_WAVES = 8;   // side by side, 64 columns each (4 measured slower)
+#ifndef TAGI_Z16_WAVES
+#define TAGI_Z16_WAVES 8
+#endif
+constexpr int Z16_WAVES = TAGI_Z16_WAVES;   // side by side, 64 columns each (4 measured slower)
 constexpr int Z16_COLS = Z16_WAVES * 64;
 
-template <int NG>
+// NT: streaming loads for the weights (every line is read once, by one instruction)
+template <int NG, bool NT>
 __global__ __launch_bounds__(Z16_WAVES * 64) void gemv16_dz_kernel(
     const float *__restrict__ mu_w, const float *__restrict__ dmu,
     const float *__restrict__ dvar, int K, int N, int B, int n_per_split,
@@ -405,21 +312,18 @@ __global__ __launch_bounds__(Z16_WAVES * 64) void gemv16_dz_kernel(
     auto load = [&](float4(&x)[ST], int s) {
 #pragma unroll
         for (int u = 0; u < ST; u++)
-            x[u] = ld4(w + (size_t)min(n_begin + 4 * (s + u) + kk, n_last) * K);
+            x[u] = NT ? ldnt4(w + (size_t)min(n_begin + 4 * (s + u) + kk, n_last) * K)
+                      : ld4(w + (size_t)min(n_begin + 4 * (s + u) + kk, n_last) * K);
     };
     load(st[0], 0);
     // stage the innovations: global [sample][n] -> LDS [sample][n % 4][n / 4]
-    for (int e = tid; e < NS * steps; e += Z16_WAVES * 64) {
-        const int b = e / steps, step = e - b * steps;
-        float4 m = zero4(), v = zero4();
-        if (b < B && n_begin + 4 * step < N) {  // N % 4 == 0 on this path
-            m = ld4(dmu + (size_t)b * N + n_begin + 4 * step);
-            v = ld4(dvar + (size_t)b * N + n_begin + 4 * step);
-        }
-        float *pm = s_dm + b * S + step, *pv = s_dv + b * S + step;
-        pm[0] = m.x; pm[Q] = m.y; pm[2 * Q] = m.z; pm[3 * Q] = m.w;
-        pv[0] = v.x; pv[Q] = v.y; pv[2 * Q] = v.z; pv[3 * Q] = v.w;
-    }
+    // (N % 4 == 0 on this path)
+    stage_slice_pairs<Z16_WAVES * 64>(dmu, dvar, NS, B, N, n_begin, N - n_begin, n_per_split, tid,
+                                      [&](int b, int n, float4 m, float4 v) {
+                                          float *pm = s_dm + b * S + n / 4, *pv = s_dv + b * S + n / 4;
+                                          pm[0] = m.x; pm[Q] = m.y; pm[2 * Q] = m.z; pm[3 * Q] = m.w;
+                                          pv[0] = v.x; pv[Q] = v.y; pv[2 * Q] = v.z; pv[3 * Q] = v.w;
+                                      });
 
     floatx4 acc0[NG][4], acc1[NG][4];
 #pragma unroll
@@ -486,28 +390,16 @@ __global__ __launch_bounds__(Z16_WAVES * 64) void gemv16_dz_kernel(
 
 constexpr int F16_KROUND = 2 * F16_KSTEP;                     // slices: whole pairs of stages
 constexpr int Z16_NSTEP = 2 * Z16_ST * 4;                     // rows: whole pairs of stages
-constexpr size_t W16_LDS_BUDGET = 72 * 1024;                  // two workgroups per CU
+constexpr size_t W16_LDS_BUDGET = 72 * 1024;                  // slices of 512 elements for 16 samples
 
 }  // namespace
 
-// 1: the forward that loads whole cache lines and transposes them in LDS. Measured equal
-// to the direct kernel (8192^2, batch 16: 113.6 vs 113.9 us per call), so the simpler one
-// stays the default.
-int g_gemv16_fwd_lines = 0;
-
 int gemv16_fwd_rows_per_block() { return W16_WAVES * F16_RG * 16; }
-int gemv16_fwd_k_step() { return g_gemv16_fwd_lines ? T16_DEPTH * T16_STAGE : F16_KROUND; }
+int gemv16_fwd_k_step() { return F16_KROUND; }
 // sample slots the kernels stage for a batch of B: 16 up to 16 samples, 32 beyond
 static int sample_slots(int B) { return B <= W16_SAMPLES ? W16_SAMPLES : 2 * W16_SAMPLES; }
 int gemv16_max_batch() { return 2 * W16_SAMPLES; }
 int gemv16_fwd_max_slice(int B) {
-    if (g_gemv16_fwd_lines && B <= W16_SAMPLES) {
-        // one workgroup per CU: the activations of a slice plus the waves' tiles
-        const size_t budget = 150 * 1024 - (size_t)W16_WAVES * 2 * T16_TILE * sizeof(float);
-        int s = (int)(budget / (2 * W16_SAMPLES * sizeof(float)) - F16_PAD) /
-                (T16_DEPTH * T16_STAGE) * (T16_DEPTH * T16_STAGE);
-        return s > 512 ? 512 : s;
-    }
     return (int)(W16_LDS_BUDGET / (2 * sample_slots(B) * sizeof(float)) - F16_PAD) / F16_KROUND *
            F16_KROUND;
 }
@@ -516,6 +408,29 @@ int gemv16_dz_n_step() { return Z16_NSTEP; }
 int gemv16_dz_max_slice(int B) {
     return (int)(W16_LDS_BUDGET / (2 * sample_slots(B) * sizeof(float)) - 16 * Z16_PADQ) /
            Z16_NSTEP * Z16_NSTEP;
+}
+
+// Forward load pattern. 1: whole 128-byte lines with streaming loads, 2: whole lines
+// with plain loads, 0: sixteen rows x 64 bytes per instruction with plain loads,
+// -1: by size - streaming loads when the two weight matrices are larger than the
+// 256 MB memory-side cache (they cannot stay in it from one call to the next, and not
+// allocating them leaves it to everything else), plain loads of whole lines otherwise.
+// Measured per forward call, batch 16: 8192^2 115 / 104 / 108 us for 0 / 1 / 2 with
+// eight waves per workgroup and 100 us for 1 with sixteen; 4096^2 28.2 / 32.0 / 27.9 us.
+int g_gemv16_fwd_whole_lines = -1;
+
+template <int NG, int WL>
+static hipError_t run_gemv16_fwd(dim3 grid, dim3 block, size_t lds, hipStream_t stream,
+                                 const float *mu_w, const float *var_w, const float *mu_a,
+                                 const float *var_a, int K, int N, int B, int k_per_split,
+                                 int splits, float *ws0, float *ws1) {
+    static PerDeviceOnce once;
+    hipError_t e = allow_dynamic_lds(
+        once, reinterpret_cast<const void *>(gemv16_fwd_kernel<NG, WL>), 160 * 1024);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((gemv16_fwd_kernel<NG, WL>), grid, block, lds, stream, mu_w, var_w, mu_a,
+                       var_a, K, N, B, k_per_split, splits, ws0, ws1);
+    return hipGetLastError();
 }
 
 // k_per_split: a multiple of gemv16_fwd_k_step(), at most gemv16_fwd_max_slice(B);
@@ -529,31 +444,28 @@ hipError_t launch_gemv16_fwd(const float *mu_w, const float *var_w, const float 
     size_t lds = (size_t)2 * sample_slots(B) * (k_per_split + F16_PAD) * sizeof(float);
     const int rows = gemv16_fwd_rows_per_block();
     dim3 grid(((N + rows - 1) / rows) * splits), block(W16_WAVES * 64);
-    if (g_gemv16_fwd_lines && B <= W16_SAMPLES) {
-        lds += (size_t)W16_WAVES * 2 * T16_TILE * sizeof(float);
-        static PerDeviceOnce once_lines;
-        hipError_t e = allow_dynamic_lds(
-            once_lines, reinterpret_cast<const void *>(gemv16_fwd_lines_kernel), 160 * 1024);
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(gemv16_fwd_lines_kernel, grid, block, lds, stream, mu_w, var_w, mu_a,
-                           var_a, K, N, B, k_per_split, splits, ws0, ws1);
-        return hipGetLastError();
-    }
-    if (B <= W16_SAMPLES) {
-        static PerDeviceOnce once;
-        hipError_t e = allow_dynamic_lds(
-            once, reinterpret_cast<const void *>(gemv16_fwd_kernel<1>), 160 * 1024);
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(gemv16_fwd_kernel<1>, grid, block, lds, stream, mu_w, var_w, mu_a, var_a,
-                           K, N, B, k_per_split, splits, ws0, ws1);
-    } else {
-        static PerDeviceOnce once2;
-        hipError_t e = allow_dynamic_lds(
-            once2, reinterpret_cast<const void *>(gemv16_fwd_kernel<2>), 160 * 1024);
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(gemv16_fwd_kernel<2>, grid, block, lds, stream, mu_w, var_w, mu_a, var_a,
-                           K, N, B, k_per_split, splits, ws0, ws1);
-    }
+#define TAGI_RUN16(NG, WL)                                                                     \
+    run_gemv16_fwd<NG, WL>(grid, block, lds, stream, mu_w, var_w, mu_a, var_a, K, N, B, k_per_split, \
+                           splits, ws0, ws1)
+    int wl = g_gemv16_fwd_whole_lines;
+    if (wl < 0 || wl > 2) wl = (size_t)N * K * 2 * sizeof(float) > ((size_t)256 << 20) ? 1 : 2;
+    if (B <= W16_SAMPLES) return wl == 1 ? TAGI_RUN16(1, 1) : wl == 2 ? TAGI_RUN16(1, 2) : TAGI_RUN16(1, 0);
+    return wl == 1 ? TAGI_RUN16(2, 1) : wl == 2 ? TAGI_RUN16(2, 2) : TAGI_RUN16(2, 0);
+#undef TAGI_RUN16
+}
+
+int g_gemv16_dz_streaming = 0;
+
+template <int NG, bool NT>
+static hipError_t run_gemv16_dz(dim3 grid, dim3 block, size_t lds, hipStream_t stream,
+                                const float *mu_w, const float *dmu, const float *dvar, int K, int N,
+                                int B, int n_per_split, float *ws0, float *ws1) {
+    static PerDeviceOnce once;
+    hipError_t e = allow_dynamic_lds(
+        once, reinterpret_cast<const void *>(gemv16_dz_kernel<NG, NT>), 160 * 1024);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((gemv16_dz_kernel<NG, NT>), grid, block, lds, stream, mu_w, dmu, dvar, K, N, B,
+                       n_per_split, ws0, ws1);
     return hipGetLastError();
 }
 
@@ -569,22 +481,12 @@ hipError_t launch_gemv16_dz(const float *mu_w, const float *dmu, const float *dv
     const size_t lds = (size_t)2 * sample_slots(B) * (n_per_split + 16 * Z16_PADQ) * sizeof(float);
     const int cols = gemv16_dz_cols_per_block();
     dim3 grid((K + cols - 1) / cols, splits), block(Z16_WAVES * 64);
-    if (B <= W16_SAMPLES) {
-        static PerDeviceOnce once;
-        hipError_t e = allow_dynamic_lds(
-            once, reinterpret_cast<const void *>(gemv16_dz_kernel<1>), 160 * 1024);
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(gemv16_dz_kernel<1>, grid, block, lds, stream, mu_w, dmu, dvar, K, N, B,
-                           n_per_split, ws0, ws1);
-    } else {
-        static PerDeviceOnce once2;
-        hipError_t e = allow_dynamic_lds(
-            once2, reinterpret_cast<const void *>(gemv16_dz_kernel<2>), 160 * 1024);
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(gemv16_dz_kernel<2>, grid, block, lds, stream, mu_w, dmu, dvar, K, N, B,
-                           n_per_split, ws0, ws1);
-    }
-    return hipGetLastError();
+#define TAGI_RUN16Z(NG, NT) \
+    run_gemv16_dz<NG, NT>(grid, block, lds, stream, mu_w, dmu, dvar, K, N, B, n_per_split, ws0, ws1)
+    const bool nt = g_gemv16_dz_streaming != 0;
+    if (B <= W16_SAMPLES) return nt ? TAGI_RUN16Z(1, true) : TAGI_RUN16Z(1, false);
+    return nt ? TAGI_RUN16Z(2, true) : TAGI_RUN16Z(2, false);
+#undef TAGI_RUN16Z
 }
 
 }  // namespace tagi

@@ -20,8 +20,12 @@ extern "C" {
  * "linear.gemv.fwd_variant", "linear.gemv.reverse", "linear.gemv16" (0: 9..16
  * samples on the kernels for up to 8), "linear.gemv32" (0: the forward of 17..32
  * samples on the tiled kernel instead of the 16-wide streaming one; 2: their state
- * backward on the streaming kernel too), "linear.gemv16.fwd_lines" (1: the 9..16-sample
- * forward that loads whole cache lines and transposes them in LDS), "linear.dw_side" (0: bias innovations and
+ * backward on the streaming kernel too), "linear.gemv16.whole_lines" (load
+ * pattern of the 9..32-sample forward: 1 whole 128-byte lines with streaming loads, 2
+ * whole lines with plain loads, 0 sixteen rows x 64 bytes per instruction; < 0 by
+ * size), "linear.gemv16.dz_streaming" (1: streaming loads in the 9..32-sample state
+ * backward), "linear.gemv16.min_batch" (smallest batch that takes the 16-wide forward,
+ * 9 by default), "linear.dw_side" (0: bias innovations and
  * the state-backward fold as launches of their own instead of inside the
  * weight-backward launch), "linear.double_buffer", "linear.stream_min_weights" (the
  * smallest weight matrix, in elements, that goes to the streaming kernels; 0 sends every

@@ -163,12 +163,13 @@ def test_pack_size_network_at_its_real_size():
 
 
 @pytest.mark.parametrize("K,N,B", [(1024, 512, 16), (1536, 260, 12), (72, 1028, 10),
-                                   (2052, 300, 13), (4096, 256, 9)])
-def test_both_forward_kernels_for_9_to_16_samples(oracle_lib, K, N, B):
-    """The 16-wide streaming forward exists twice: loading the MFMA operand layout
-    directly (16 rows x 64 bytes per instruction, the default), and loading whole cache
-    lines that a wave-private LDS tile turns into that layout (same speed, kept as a
-    switch)."""
+                                   (2052, 300, 13), (4096, 256, 9), (516, 1000, 20),
+                                   (2048, 1027 * 4, 32), (36, 52, 12)])
+def test_forward_load_patterns_for_9_to_16_samples(oracle_lib, K, N, B):
+    """The 16-wide streaming forward loads its weights in one of three ways: whole
+    128-byte lines with streaming loads (lanes then exchange a float4), whole lines with
+    plain loads, or sixteen rows x 64 bytes per instruction. The library picks by size;
+    the three must agree bit for bit (the same registers reach the same MFMAs)."""
     import cutagi_amd.functional as F
     from cutagi_amd import capi
     d = linear_inputs(K, N, B, seed=K + N + B, bias=True)
@@ -178,14 +179,17 @@ def test_both_forward_kernels_for_9_to_16_samples(oracle_lib, K, N, B):
     got = {}
     capi.tune("linear.stream_min_weights", 0)     # these shapes are small: force the kernels
     try:
-        for lines in (1, 0):
-            capi.tune("linear.gemv16.fwd_lines", lines)
+        for pattern in (0, 1, 2):
+            capi.tune("linear.gemv16.whole_lines", pattern)
             z = F.linear_fwd(t["mu_w"], t["var_w"], t["mu_b"], t["var_b"], t["mu_a"], t["var_a"])
-            got[lines] = (z[0].cpu().numpy(), z[1].cpu().numpy())
-            assert_close(got[lines][0], ref[0], "mu_z (lines=%d)" % lines)
-            assert_close(got[lines][1], ref[1], "var_z (lines=%d)" % lines, same_sign=True)
+            got[pattern] = (z[0].cpu().numpy(), z[1].cpu().numpy())
+            assert_close(got[pattern][0], ref[0], "mu_z (pattern %d)" % pattern)
+            assert_close(got[pattern][1], ref[1], "var_z (pattern %d)" % pattern, same_sign=True)
+        for pattern in (1, 2):
+            assert np.array_equal(got[pattern][0], got[0][0])
+            assert np.array_equal(got[pattern][1], got[0][1])
     finally:
-        capi.tune("linear.gemv16.fwd_lines", -1)
+        capi.tune("linear.gemv16.whole_lines", -1)
         capi.tune("linear.stream_min_weights", -1)
 
 
