@@ -170,9 +170,10 @@ int wide_max_batch() {
 // where reading the weights is what takes the time; on smaller layers a launch is bound by
 // latency and the tiled kernel's many short slices finish sooner. Thresholds from kernel
 // times at 128^2 .. 4096^2 (weights in elements):
-//   forward        <= 8 samples: 8M (4096^2: 29 against 39 us; 2048^2: 25 against 19 us)
-//                  9..16: 2M (2048^2: 15.6 against 19.7 us; 1024^2: 15.3 against 13.3 us)
-//                  17..32: 8M (4096^2: 36 against 41 us; 2048^2: 22.4 against 21.3 us)
+//   forward        <= 4 samples: 8M (4096^2: 29 against 39 us; 2048^2: 25 against 19 us)
+//                  5..16: 4M (2048^2: 15.0 against 18-19 us; 2048 x 1024: 14.7-15.4 against
+//                  13.7-15.1 us)
+//                  17..32: 8M (4096 x 2048: 23.4 against 28 us; 2048^2: 21.6 against 21.0 us)
 //   state backward <= 8 samples: 4M (4096^2: 19-22 against 28 us; 1024^2: 13-16 against 11 us)
 //                  9..16: 2M (2048x1024: 13.5 against 14.4 us; 1024^2: 12.7 against 12.2 us)
 enum StreamOp { STREAM_FWD, STREAM_DZ };
@@ -180,7 +181,7 @@ bool streams_weights(StreamOp op, int n, int k, int batch) {
     const long long weights = (long long)n * k;
     if (g_tune.stream_min_weights >= 0) return weights >= g_tune.stream_min_weights;
     const long long M = 1ll << 20;
-    if (op == STREAM_FWD) return weights >= (batch <= 8 ? 8 * M : batch <= 16 ? 2 * M : 8 * M);
+    if (op == STREAM_FWD) return weights >= (batch <= 4 ? 8 * M : batch <= 16 ? 4 * M : 8 * M);
     return weights >= (batch <= 8 ? 4 * M : 2 * M);
 }
 
@@ -341,7 +342,7 @@ int tagi_hip_tune(const char *key, int value) {
     else if (!strcmp(key, "linear.gemv16")) g_tune.gemv16 = value;
     else if (!strcmp(key, "linear.gemv16.min_batch")) g_tune.gemv16_min = value;
     else if (!strcmp(key, "linear.gemv32")) g_tune.wide32 = value;
-    else if (!strcmp(key, "linear.gemv16.dz_streaming")) g_gemv16_dz_streaming = value < 0 ? 0 : value;
+    else if (!strcmp(key, "linear.gemv16.fwd_waves")) g_gemv16_fwd_waves = value;
     else if (!strcmp(key, "linear.gemv16.whole_lines")) g_gemv16_fwd_whole_lines = value;
     else if (!strcmp(key, "linear.stream_min_weights")) g_tune.stream_min_weights = value;
     else if (!strcmp(key, "linear.small")) g_tune.small = value;
@@ -376,7 +377,7 @@ static int linear_fwd_impl(const float *mu_w, const float *var_w, const float *m
     if (B >= (g_tune.gemv16_min > 0 ? g_tune.gemv16_min : 5) && B <= wide_max_batch() && vec &&
         g_tune.gemv16 != 0 && streams) {
         // 9..32 samples: the 16-wide streaming kernel (two sample groups beyond 16)
-        const int blocks = ceil_div(N, gemv16_fwd_rows_per_block());
+        const int blocks = ceil_div(N, gemv16_fwd_rows_per_block(N, K, B));
         const int step = gemv16_fwd_k_step();
         int splits = g_tune.fwd_splits > 0 ? g_tune.fwd_splits : ceil_div(2 * num_cu(), blocks);
         const int max_splits = ceil_div(K, 4 * step);

@@ -58,7 +58,6 @@ __device__ __forceinline__ floatx4 mfma16(float a, float b, floatx4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
 }
 
-constexpr int W16_WAVES = 16;   // forward: one workgroup of sixteen waves per CU
 constexpr int W16_SAMPLES = 16;
 
 // ---------------------------------------------------------------------------
@@ -84,14 +83,16 @@ constexpr int F16_PAD = 4;       // LDS row stride % 32 == 4
 // WL: load instructions cover whole 128-byte lines (8 rows x 128 bytes each, two of them
 // for the wave's sixteen rows) with streaming loads; lanes i and i ^ 8 then exchange one
 // float4 each to arrive at the operand layout (see swap_halves).
-template <int NG, int WL>
-__global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_kernel(
+// WAVES: 16 (one workgroup per CU, 256 rows share a staged slice) where that still gives
+// every CU a workgroup, 8 on smaller matrices.
+template <int NG, int WL, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemv16_fwd_kernel(
     const float *__restrict__ mu_w, const float *__restrict__ var_w,
     const float *__restrict__ mu_a, const float *__restrict__ var_a, int K, int N, int B,
     int k_per_split, int splits, float *__restrict__ ws0, float *__restrict__ ws1) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int RG = F16_RG, C = F16_C, KSTEP = F16_KSTEP;
-    constexpr int ROWS_PER_BLOCK = W16_WAVES * RG * 16;
+    constexpr int ROWS_PER_BLOCK = WAVES * RG * 16;
     constexpr int NS = NG * W16_SAMPLES;
     const int S = k_per_split + F16_PAD;
     float *s_mu = lds, *s_var = lds + NS * S;
@@ -113,7 +114,7 @@ __global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_kernel(
     const int k_begin = split * k_per_split;
     const int kr = min(K, k_begin + k_per_split) - k_begin;
     // each wave walks its slice from a different starting point (sums commute)
-    const int rot = ((row_block * W16_WAVES + wave) * 2 * KSTEP) % k_per_split;
+    const int rot = ((row_block * WAVES + wave) * 2 * KSTEP) % k_per_split;
 
     // stage the slice of the activations: [sample][k], zero beyond B and kr
 
@@ -216,7 +217,7 @@ __global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_kernel(
     auto wrap = [&](int p) { return p >= k_per_split ? p - k_per_split : p; };
     load(sm[0], sv[0], rot);
     __builtin_amdgcn_sched_barrier(0);  // the first weights are on their way while the slice is staged
-    stage_slice_pairs<W16_WAVES * 64>(mu_a, var_a, NS, B, K, k_begin, kr, k_per_split, tid,
+    stage_slice_pairs<WAVES * 64>(mu_a, var_a, NS, B, K, k_begin, kr, k_per_split, tid,
                                       [&](int b, int k, float4 m, float4 v) {
                                           *reinterpret_cast<float4 *>(s_mu + b * S + k) = m;
                                           *reinterpret_cast<float4 *>(s_var + b * S + k) = v;
@@ -276,14 +277,13 @@ __global__ __launch_bounds__(W16_WAVES * 64) void gemv16_fwd_kernel(
 // ---------------------------------------------------------------------------
 constexpr int Z16_ST = 4;      // 4-row steps per register stage (= steps per LDS float4)
 constexpr int Z16_PADQ = 1;    // plane stride per/4 + 4: spreads the kk planes over the banks
-#ifndef TAGI_Z16_WAVES
-#define TAGI_Z16_WAVES 8
-#endif
-constexpr int Z16_WAVES = TAGI_Z16_WAVES;   // side by side, 64 columns each (4 measured slower)
+constexpr int Z16_WAVES = 8;   // side by side, 64 columns each (4 measured slower)
 constexpr int Z16_COLS = Z16_WAVES * 64;
 
-// NT: streaming loads for the weights (every line is read once, by one instruction)
-template <int NG, bool NT>
+// (Measured and left out, 8192^2, batch 16, per call: streaming loads for the weights 60
+// against 57 us; sixteen waves side by side 74 us; sixteen waves as two halves of the
+// slice's rows that meet in LDS 58 against 56 us.)
+template <int NG>
 __global__ __launch_bounds__(Z16_WAVES * 64) void gemv16_dz_kernel(
     const float *__restrict__ mu_w, const float *__restrict__ dmu,
     const float *__restrict__ dvar, int K, int N, int B, int n_per_split,
@@ -312,8 +312,7 @@ __global__ __launch_bounds__(Z16_WAVES * 64) void gemv16_dz_kernel(
     auto load = [&](float4(&x)[ST], int s) {
 #pragma unroll
         for (int u = 0; u < ST; u++)
-            x[u] = NT ? ldnt4(w + (size_t)min(n_begin + 4 * (s + u) + kk, n_last) * K)
-                      : ld4(w + (size_t)min(n_begin + 4 * (s + u) + kk, n_last) * K);
+            x[u] = ld4(w + (size_t)min(n_begin + 4 * (s + u) + kk, n_last) * K);
     };
     load(st[0], 0);
     // stage the innovations: global [sample][n] -> LDS [sample][n % 4][n / 4]
@@ -394,7 +393,16 @@ constexpr size_t W16_LDS_BUDGET = 72 * 1024;                  // slices of 512 e
 
 }  // namespace
 
-int gemv16_fwd_rows_per_block() { return W16_WAVES * F16_RG * 16; }
+// Waves per forward workgroup: -1 by size, else 8 or 16.
+int g_gemv16_fwd_waves = -1;
+static int fwd_waves(int N, int K, int B) {
+    if (g_gemv16_fwd_waves == 8 || g_gemv16_fwd_waves == 16) return g_gemv16_fwd_waves;
+    // Sixteen where 256-row blocks x 512-element slices still number two per CU, for up
+    // to sixteen samples. Forward call, 16 against 8 waves: 8192^2 batch 16 99.7 / 103.9
+    // us, batch 8 93.0 / 96.4; 8192 x 4096 batch 16 52.5 / 47.3; 8192^2 batch 32 150 / 144.
+    return B <= W16_SAMPLES && (long long)N * K >= 2ll * num_cu() * 256 * 512 ? 16 : 8;
+}
+int gemv16_fwd_rows_per_block(int N, int K, int B) { return fwd_waves(N, K, B) * F16_RG * 16; }
 int gemv16_fwd_k_step() { return F16_KROUND; }
 // sample slots the kernels stage for a batch of B: 16 up to 16 samples, 32 beyond
 static int sample_slots(int B) { return B <= W16_SAMPLES ? W16_SAMPLES : 2 * W16_SAMPLES; }
@@ -419,16 +427,16 @@ int gemv16_dz_max_slice(int B) {
 // eight waves per workgroup and 100 us for 1 with sixteen; 4096^2 28.2 / 32.0 / 27.9 us.
 int g_gemv16_fwd_whole_lines = -1;
 
-template <int NG, int WL>
-static hipError_t run_gemv16_fwd(dim3 grid, dim3 block, size_t lds, hipStream_t stream,
+template <int NG, int WL, int WAVES>
+static hipError_t run_gemv16_fwd(dim3 grid, size_t lds, hipStream_t stream,
                                  const float *mu_w, const float *var_w, const float *mu_a,
                                  const float *var_a, int K, int N, int B, int k_per_split,
                                  int splits, float *ws0, float *ws1) {
     static PerDeviceOnce once;
     hipError_t e = allow_dynamic_lds(
-        once, reinterpret_cast<const void *>(gemv16_fwd_kernel<NG, WL>), 160 * 1024);
+        once, reinterpret_cast<const void *>(gemv16_fwd_kernel<NG, WL, WAVES>), 160 * 1024);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((gemv16_fwd_kernel<NG, WL>), grid, block, lds, stream, mu_w, var_w, mu_a,
+    hipLaunchKernelGGL((gemv16_fwd_kernel<NG, WL, WAVES>), grid, dim3(WAVES * 64), lds, stream, mu_w, var_w, mu_a,
                        var_a, K, N, B, k_per_split, splits, ws0, ws1);
     return hipGetLastError();
 }
@@ -442,11 +450,13 @@ hipError_t launch_gemv16_fwd(const float *mu_w, const float *var_w, const float 
         k_per_split > gemv16_fwd_max_slice(B) || (long long)k_per_split * splits < K)
         return hipErrorInvalidValue;
     size_t lds = (size_t)2 * sample_slots(B) * (k_per_split + F16_PAD) * sizeof(float);
-    const int rows = gemv16_fwd_rows_per_block();
-    dim3 grid(((N + rows - 1) / rows) * splits), block(W16_WAVES * 64);
-#define TAGI_RUN16(NG, WL)                                                                     \
-    run_gemv16_fwd<NG, WL>(grid, block, lds, stream, mu_w, var_w, mu_a, var_a, K, N, B, k_per_split, \
-                           splits, ws0, ws1)
+    const int rows = gemv16_fwd_rows_per_block(N, K, B);
+    dim3 grid(((N + rows - 1) / rows) * splits);
+#define TAGI_RUN16(NG, WL)                                                                          \
+    (rows == 256 ? run_gemv16_fwd<NG, WL, 16>(grid, lds, stream, mu_w, var_w, mu_a, var_a, K, N, B, \
+                                              k_per_split, splits, ws0, ws1)                       \
+                 : run_gemv16_fwd<NG, WL, 8>(grid, lds, stream, mu_w, var_w, mu_a, var_a, K, N, B,  \
+                                             k_per_split, splits, ws0, ws1))
     int wl = g_gemv16_fwd_whole_lines;
     if (wl < 0 || wl > 2) wl = (size_t)N * K * 2 * sizeof(float) > ((size_t)256 << 20) ? 1 : 2;
     if (B <= W16_SAMPLES) return wl == 1 ? TAGI_RUN16(1, 1) : wl == 2 ? TAGI_RUN16(1, 2) : TAGI_RUN16(1, 0);
@@ -454,17 +464,15 @@ hipError_t launch_gemv16_fwd(const float *mu_w, const float *var_w, const float 
 #undef TAGI_RUN16
 }
 
-int g_gemv16_dz_streaming = 0;
-
-template <int NG, bool NT>
+template <int NG>
 static hipError_t run_gemv16_dz(dim3 grid, dim3 block, size_t lds, hipStream_t stream,
                                 const float *mu_w, const float *dmu, const float *dvar, int K, int N,
                                 int B, int n_per_split, float *ws0, float *ws1) {
     static PerDeviceOnce once;
     hipError_t e = allow_dynamic_lds(
-        once, reinterpret_cast<const void *>(gemv16_dz_kernel<NG, NT>), 160 * 1024);
+        once, reinterpret_cast<const void *>(gemv16_dz_kernel<NG>), 160 * 1024);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((gemv16_dz_kernel<NG, NT>), grid, block, lds, stream, mu_w, dmu, dvar, K, N, B,
+    hipLaunchKernelGGL((gemv16_dz_kernel<NG>), grid, block, lds, stream, mu_w, dmu, dvar, K, N, B,
                        n_per_split, ws0, ws1);
     return hipGetLastError();
 }
@@ -481,12 +489,9 @@ hipError_t launch_gemv16_dz(const float *mu_w, const float *dmu, const float *dv
     const size_t lds = (size_t)2 * sample_slots(B) * (n_per_split + 16 * Z16_PADQ) * sizeof(float);
     const int cols = gemv16_dz_cols_per_block();
     dim3 grid((K + cols - 1) / cols, splits), block(Z16_WAVES * 64);
-#define TAGI_RUN16Z(NG, NT) \
-    run_gemv16_dz<NG, NT>(grid, block, lds, stream, mu_w, dmu, dvar, K, N, B, n_per_split, ws0, ws1)
-    const bool nt = g_gemv16_dz_streaming != 0;
-    if (B <= W16_SAMPLES) return nt ? TAGI_RUN16Z(1, true) : TAGI_RUN16Z(1, false);
-    return nt ? TAGI_RUN16Z(2, true) : TAGI_RUN16Z(2, false);
-#undef TAGI_RUN16Z
+    if (B <= W16_SAMPLES)
+        return run_gemv16_dz<1>(grid, block, lds, stream, mu_w, dmu, dvar, K, N, B, n_per_split, ws0, ws1);
+    return run_gemv16_dz<2>(grid, block, lds, stream, mu_w, dmu, dvar, K, N, B, n_per_split, ws0, ws1);
 }
 
 }  // namespace tagi

@@ -151,8 +151,8 @@ hipError_t launch_gemv16_dz(const float *mu_w, const float *dmu, const float *dv
                             hipStream_t stream);
 // 1: the 9..16-sample forward kernel that loads whole cache lines (default 0)
 extern int g_gemv16_fwd_whole_lines;
-extern int g_gemv16_dz_streaming;
-int gemv16_fwd_rows_per_block();
+int gemv16_fwd_rows_per_block(int N, int K, int B);
+extern int g_gemv16_fwd_waves;
 int gemv16_fwd_k_step();
 int gemv16_fwd_max_slice(int B);
 int gemv16_max_batch();  // 32: two groups of sixteen samples

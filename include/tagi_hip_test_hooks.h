@@ -23,8 +23,8 @@ extern "C" {
  * backward on the streaming kernel too), "linear.gemv16.whole_lines" (load
  * pattern of the 9..32-sample forward: 1 whole 128-byte lines with streaming loads, 2
  * whole lines with plain loads, 0 sixteen rows x 64 bytes per instruction; < 0 by
- * size), "linear.gemv16.dz_streaming" (1: streaming loads in the 9..32-sample state
- * backward), "linear.gemv16.min_batch" (smallest batch that takes the 16-wide forward,
+ * size), "linear.gemv16.fwd_waves" (8 or 16 waves per workgroup of that forward, < 0 by
+ * size), "linear.gemv16.min_batch" (smallest batch that takes the 16-wide forward,
  * 9 by default), "linear.dw_side" (0: bias innovations and
  * the state-backward fold as launches of their own instead of inside the
  * weight-backward launch), "linear.double_buffer", "linear.stream_min_weights" (the
