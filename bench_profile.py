@@ -105,12 +105,12 @@ KERNELS = [
     ("linear_dw_side_kernel<LinearProblem<2, true, true, true>, 64, 128, 2, 4>",
      "Linear 4096^2 B=256 delta_w + delta_z fold + delta_b (inside the backward call)",
      (3 * K2 * K2 + B2 * K2 + 2 * B2 * K2) * 4 / MB, 4.0 * B2 * K2 * K2),
-    ("gemv16_fwd_kernel<1, 1>", "Linear 8192^2 B=8, 12 and 16 forward", 2 * K3 * K3 * 4 / MB, 6.0 * 12 * K3 * K3),
+    ("gemv16_fwd_kernel<1, 3, 16>", "Linear 8192^2 B=8, 12 and 16 forward", 2 * K3 * K3 * 4 / MB, 6.0 * 12 * K3 * K3),
     ("gemv_dz_kernel<2>", "Linear 8192^2 B=8 delta_z", K3 * K3 * 4 / MB, 4.0 * B3 * K3 * K3),
     ("gemv_dw_kernel<8, true>", "Linear 8192^2 B=8 delta_w (+delta_b)", 3 * K3 * K3 * 4 / MB, 4.0 * B3 * K3 * K3),
-    ("gemv16_dz_kernel<1, false>", "Linear 8192^2 B=12 and B=16 delta_z", K3 * K3 * 4 / MB, 4.0 * 14 * K3 * K3),
+    ("gemv16_dz_kernel<1>", "Linear 8192^2 B=12 and B=16 delta_z", K3 * K3 * 4 / MB, 4.0 * 14 * K3 * K3),
     ("gemv_dw_kernel<16, true>", "Linear 8192^2 B=12 and B=16 delta_w (+delta_b)", 3 * K3 * K3 * 4 / MB, 4.0 * 14 * K3 * K3),
-    ("gemv16_fwd_kernel<2, 2>", "Linear 4096^2 B=32 forward", 2 * K2 * K2 * 4 / MB, 6.0 * 32 * K2 * K2),
+    ("gemv16_fwd_kernel<2, 2, 8>", "Linear 4096^2 B=32 forward", 2 * K2 * K2 * 4 / MB, 6.0 * 32 * K2 * K2),
     ("conv_stencil_kernel<false, 32>", "Conv2d 3x3 64->64 @32x32 B=128 forward", 4 * CONV_ACT, 6.0 * 64 * 131072 * 576),
     ("conv_stencil_bwd_pair_kernel<32>", "Conv2d delta_z + delta_w (one launch)", 6 * CONV_ACT,
      8.0 * 64 * 131072 * 576),

@@ -166,10 +166,10 @@ def test_pack_size_network_at_its_real_size():
                                    (2052, 300, 13), (4096, 256, 9), (516, 1000, 20),
                                    (2048, 1027 * 4, 32), (36, 52, 12)])
 def test_forward_load_patterns_for_9_to_16_samples(oracle_lib, K, N, B):
-    """The 16-wide streaming forward loads its weights in one of three ways: whole
-    128-byte lines with streaming loads (lanes then exchange a float4), whole lines with
-    plain loads, or sixteen rows x 64 bytes per instruction. The library picks by size;
-    the three must agree bit for bit (the same registers reach the same MFMAs)."""
+    """The 16-wide streaming forward loads its weights as whole 128-byte lines (lanes
+    then exchange a float4) with streaming loads, plain loads or one of each per matrix,
+    or as sixteen rows x 64 bytes per instruction. The library picks by size; all must
+    agree bit for bit (the same registers reach the same MFMAs)."""
     import cutagi_amd.functional as F
     from cutagi_amd import capi
     d = linear_inputs(K, N, B, seed=K + N + B, bias=True)
@@ -181,14 +181,14 @@ def test_forward_load_patterns_for_9_to_16_samples(oracle_lib, K, N, B):
     try:
         for waves in (8, 16):                     # workgroups of 128 or 256 rows
             capi.tune("linear.gemv16.fwd_waves", waves)
-            for pattern in (0, 1, 2):
+            for pattern in (0, 1, 2, 3):
                 capi.tune("linear.gemv16.whole_lines", pattern)
                 z = F.linear_fwd(t["mu_w"], t["var_w"], t["mu_b"], t["var_b"], t["mu_a"], t["var_a"])
                 got[pattern] = (z[0].cpu().numpy(), z[1].cpu().numpy())
                 what = "(pattern %d, %d waves)" % (pattern, waves)
                 assert_close(got[pattern][0], ref[0], "mu_z " + what)
                 assert_close(got[pattern][1], ref[1], "var_z " + what, same_sign=True)
-            for pattern in (1, 2):
+            for pattern in (1, 2, 3):
                 assert np.array_equal(got[pattern][0], got[0][0])
                 assert np.array_equal(got[pattern][1], got[0][1])
     finally:
