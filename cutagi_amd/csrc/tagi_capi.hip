@@ -109,7 +109,7 @@ struct Tuning {
     // walk rows from the end, high bit: XCD-aware column mapping
     int gemv_rev = -1;
     int gemv16 = -1;    // 0: 9..16 samples on the 4x4x1 kernels too
-    int gemv16_min = -1;  // smallest batch the 16-wide forward takes (default 5)
+    int gemv16_min = -1;  // smallest batch the 16-wide forward takes (default 1)
     int wide32 = -1;    // 0: 17..32 samples on the tiled kernels; 2: state backward streams too
     int dw_side = -1;   // 0: bias innovations and the state-backward fold as launches of their own
     // >= 0: the smallest weight matrix (elements) the streaming kernels take, whatever the
@@ -170,9 +170,8 @@ int wide_max_batch() {
 // where reading the weights is what takes the time; on smaller layers a launch is bound by
 // latency and the tiled kernel's many short slices finish sooner. Thresholds from kernel
 // times at 128^2 .. 4096^2 (weights in elements):
-//   forward        <= 4 samples: 8M (4096^2: 29 against 39 us; 2048^2: 25 against 19 us)
-//                  5..16: 4M (2048^2: 15.0 against 18-19 us; 2048 x 1024: 14.7-15.4 against
-//                  13.7-15.1 us)
+//   forward        <= 16 samples: 4M (2048^2: 15.0 against 17-19 us; 2048 x 1024: 14.7-15.4
+//                  against 13.7-15.1 us)
 //                  17..32: 8M (4096 x 2048: 23.4 against 28 us; 2048^2: 21.6 against 21.0 us)
 //   state backward <= 8 samples: 4M (4096^2: 19-22 against 28 us; 1024^2: 13-16 against 11 us)
 //                  9..16: 2M (2048x1024: 13.5 against 14.4 us; 1024^2: 12.7 against 12.2 us)
@@ -181,7 +180,7 @@ bool streams_weights(StreamOp op, int n, int k, int batch) {
     const long long weights = (long long)n * k;
     if (g_tune.stream_min_weights >= 0) return weights >= g_tune.stream_min_weights;
     const long long M = 1ll << 20;
-    if (op == STREAM_FWD) return weights >= (batch <= 4 ? 8 * M : batch <= 16 ? 4 * M : 8 * M);
+    if (op == STREAM_FWD) return weights >= (batch <= 16 ? 4 * M : 8 * M);
     return weights >= (batch <= 8 ? 4 * M : 2 * M);
 }
 
@@ -374,7 +373,7 @@ static int linear_fwd_impl(const float *mu_w, const float *var_w, const float *m
         return TAGI_OK;
     }
     const bool streams = streams_weights(STREAM_FWD, N, K, B);
-    if (B >= (g_tune.gemv16_min > 0 ? g_tune.gemv16_min : 5) && B <= wide_max_batch() && vec &&
+    if (B >= (g_tune.gemv16_min > 0 ? g_tune.gemv16_min : 1) && B <= wide_max_batch() && vec &&
         g_tune.gemv16 != 0 && streams) {
         // 9..32 samples: the 16-wide streaming kernel (two sample groups beyond 16)
         const int blocks = ceil_div(N, gemv16_fwd_rows_per_block(N, K, B));

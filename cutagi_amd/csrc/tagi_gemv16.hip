@@ -157,10 +157,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv16_fwd_kernel(
                 const int k = min(k_lane + kb + 16 * c, k_last);
 #pragma unroll
                 for (int rg = 0; rg < RG; rg++) {
-                    m[rg][c] = WL == 1 ? ldnt4(wm[rg] + k) : ld4(wm[rg] + k);
-                    v[rg][c] = WL != 2 ? ldnt4(wv[rg] + k) : ld4(wv[rg] + k);
-                    m[rg][c + 1] = WL == 1 ? ldnt4(wm[rg] + hi[rg] + k) : ld4(wm[rg] + hi[rg] + k);
-                    v[rg][c + 1] = WL != 2 ? ldnt4(wv[rg] + hi[rg] + k) : ld4(wv[rg] + hi[rg] + k);
+                    m[rg][c] = (WL == 1 || WL == 4) ? ldnt4(wm[rg] + k) : ld4(wm[rg] + k);
+                    v[rg][c] = (WL == 1 || WL == 3) ? ldnt4(wv[rg] + k) : ld4(wv[rg] + k);
+                    m[rg][c + 1] = (WL == 1 || WL == 4) ? ldnt4(wm[rg] + hi[rg] + k) : ld4(wm[rg] + hi[rg] + k);
+                    v[rg][c + 1] = (WL == 1 || WL == 3) ? ldnt4(wv[rg] + hi[rg] + k) : ld4(wv[rg] + hi[rg] + k);
                 }
             }
             return;
@@ -420,14 +420,17 @@ int gemv16_dz_max_slice(int B) {
 
 // Forward load pattern. 0: sixteen rows x 64 bytes per instruction, plain loads; 1: whole
 // 128-byte lines, streaming loads; 2: whole lines, plain loads; 3: whole lines, plain
-// loads for mu_w and streaming loads for var_w; -1: by size - 3 when the two weight
-// matrices are larger than the 256 MB memory-side cache, 2 otherwise (smaller matrices
-// stay in it from one call to the next: 4096^2, batch 16, 32.0 us with streaming loads
-// against 27.9). Measured per forward call at 8192^2, batch 16: 115 / 104 / 108 us for
-// 0 / 1 / 2 with eight waves per workgroup, 100 us for 1 with sixteen. 3 costs the
-// forward nothing against 1 and leaves mu_w, not var_w, in that cache, which the state
-// backward of the same layer reads next: forward + backward 293 -> 283 us at batch 16,
-// 288 -> 280 us at batch 12 (the backward of up to 8 samples neither gains nor loses).
+// loads for mu_w and streaming loads for var_w; 4: the other way round; -1: by size
+// against the 256 MB memory-side cache. Both matrices fit: 2 (they stay in it from one
+// call to the next: 4096^2, batch 16, 27.9 us against 32.0 with streaming loads).
+// Neither fits: 1. One fits: the forward streams one matrix and leaves the other in the
+// cache for the backward of the same layer - var_w for the weight backward up to 8
+// samples (4), mu_w for the 16-wide state backward beyond (3; that kernel's own plain
+// loads would push var_w out again). Measured at 8192^2 per forward call, batch 16:
+// 115 / 104 / 108 us for 0 / 1 / 2 with eight waves per workgroup, 100 us for 1 with
+// sixteen, 3 and 4 the same as 1; forward + backward: batch 16 293 -> 283 us with 3
+// (291 with 4), batch 8 265 -> 252 us with 4 (264 with 3). This helps where a layer's
+// backward follows its forward closely; elsewhere it is neutral.
 int g_gemv16_fwd_whole_lines = -1;
 
 template <int NG, int WL, int WAVES>
@@ -461,10 +464,13 @@ hipError_t launch_gemv16_fwd(const float *mu_w, const float *var_w, const float 
                  : run_gemv16_fwd<NG, WL, 8>(grid, lds, stream, mu_w, var_w, mu_a, var_a, K, N, B,  \
                                              k_per_split, splits, ws0, ws1))
     int wl = g_gemv16_fwd_whole_lines;
-    if (wl < 0 || wl > 3) wl = (size_t)N * K * 2 * sizeof(float) > ((size_t)256 << 20) ? 3 : 2;
+    if (wl < 0 || wl > 4) {
+        const size_t matrix = (size_t)N * K * sizeof(float), cache = (size_t)256 << 20;
+        wl = 2 * matrix <= cache ? 2 : matrix > cache ? 1 : B <= 8 ? 4 : 3;
+    }
     if (B <= W16_SAMPLES)
-        return wl == 1 ? TAGI_RUN16(1, 1) : wl == 2 ? TAGI_RUN16(1, 2) : wl == 3 ? TAGI_RUN16(1, 3) : TAGI_RUN16(1, 0);
-    return wl == 1 ? TAGI_RUN16(2, 1) : wl == 2 ? TAGI_RUN16(2, 2) : wl == 3 ? TAGI_RUN16(2, 3) : TAGI_RUN16(2, 0);
+        return wl == 1 ? TAGI_RUN16(1, 1) : wl == 2 ? TAGI_RUN16(1, 2) : wl == 3 ? TAGI_RUN16(1, 3) : wl == 4 ? TAGI_RUN16(1, 4) : TAGI_RUN16(1, 0);
+    return wl == 1 ? TAGI_RUN16(2, 1) : wl == 2 ? TAGI_RUN16(2, 2) : wl == 3 ? TAGI_RUN16(2, 3) : wl == 4 ? TAGI_RUN16(2, 4) : TAGI_RUN16(2, 0);
 #undef TAGI_RUN16
 }
 

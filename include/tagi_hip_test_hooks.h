@@ -21,11 +21,12 @@ extern "C" {
  * samples on the kernels for up to 8), "linear.gemv32" (0: the forward of 17..32
  * samples on the tiled kernel instead of the 16-wide streaming one; 2: their state
  * backward on the streaming kernel too), "linear.gemv16.whole_lines" (load
- * pattern of the 5..32-sample forward: 1 whole 128-byte lines with streaming loads, 2
+ * pattern of the 16-wide streaming forward: 1 whole 128-byte lines with streaming loads, 2
  * whole lines with plain loads, 3 whole lines with plain loads for mu_w and streaming
- * loads for var_w, 0 sixteen rows x 64 bytes per instruction; < 0 by size), "linear.gemv16.fwd_waves" (8 or 16 waves per workgroup of that forward, < 0 by
+ * loads for var_w, 4 the other way round, 0 sixteen rows x 64 bytes per instruction;
+ * < 0 by size), "linear.gemv16.fwd_waves" (8 or 16 waves per workgroup of that forward, < 0 by
  * size), "linear.gemv16.min_batch" (smallest batch that takes the 16-wide forward,
- * 9 by default), "linear.dw_side" (0: bias innovations and
+ * 1 by default; the 4x4x1 forward serves the batches below it), "linear.dw_side" (0: bias innovations and
  * the state-backward fold as launches of their own instead of inside the
  * weight-backward launch), "linear.double_buffer", "linear.stream_min_weights" (the
  * smallest weight matrix, in elements, that goes to the streaming kernels; 0 sends every

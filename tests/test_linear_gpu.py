@@ -181,14 +181,14 @@ def test_forward_load_patterns_for_9_to_16_samples(oracle_lib, K, N, B):
     try:
         for waves in (8, 16):                     # workgroups of 128 or 256 rows
             capi.tune("linear.gemv16.fwd_waves", waves)
-            for pattern in (0, 1, 2, 3):
+            for pattern in (0, 1, 2, 3, 4):
                 capi.tune("linear.gemv16.whole_lines", pattern)
                 z = F.linear_fwd(t["mu_w"], t["var_w"], t["mu_b"], t["var_b"], t["mu_a"], t["var_a"])
                 got[pattern] = (z[0].cpu().numpy(), z[1].cpu().numpy())
                 what = "(pattern %d, %d waves)" % (pattern, waves)
                 assert_close(got[pattern][0], ref[0], "mu_z " + what)
                 assert_close(got[pattern][1], ref[1], "var_z " + what, same_sign=True)
-            for pattern in (1, 2, 3):
+            for pattern in (1, 2, 3, 4):
                 assert np.array_equal(got[pattern][0], got[0][0])
                 assert np.array_equal(got[pattern][1], got[0][1])
     finally:
