@@ -105,9 +105,10 @@ KERNELS = [
     ("linear_dw_side_kernel<LinearProblem<2, true, true, true>, 64, 128, 2, 4>",
      "Linear 4096^2 B=256 delta_w + delta_z fold + delta_b (inside the backward call)",
      (3 * K2 * K2 + B2 * K2 + 2 * B2 * K2) * 4 / MB, 4.0 * B2 * K2 * K2),
-    ("gemv16_fwd_kernel<1, 3, 16>", "Linear 8192^2 B=8, 12 and 16 forward", 2 * K3 * K3 * 4 / MB, 6.0 * 12 * K3 * K3),
+    ("gemv16_fwd_kernel<1, 4, 16>", "Linear 8192^2 B=8 forward", 2 * K3 * K3 * 4 / MB, 6.0 * B3 * K3 * K3),
     ("gemv_dz_kernel<2>", "Linear 8192^2 B=8 delta_z", K3 * K3 * 4 / MB, 4.0 * B3 * K3 * K3),
     ("gemv_dw_kernel<8, true>", "Linear 8192^2 B=8 delta_w (+delta_b)", 3 * K3 * K3 * 4 / MB, 4.0 * B3 * K3 * K3),
+    ("gemv16_fwd_kernel<1, 3, 16>", "Linear 8192^2 B=12 and B=16 forward", 2 * K3 * K3 * 4 / MB, 6.0 * 14 * K3 * K3),
     ("gemv16_dz_kernel<1>", "Linear 8192^2 B=12 and B=16 delta_z", K3 * K3 * 4 / MB, 4.0 * 14 * K3 * K3),
     ("gemv_dw_kernel<16, true>", "Linear 8192^2 B=12 and B=16 delta_w (+delta_b)", 3 * K3 * K3 * 4 / MB, 4.0 * 14 * K3 * K3),
     ("gemv16_fwd_kernel<2, 2, 8>", "Linear 4096^2 B=32 forward", 2 * K2 * K2 * 4 / MB, 6.0 * 32 * K2 * K2),
@@ -120,9 +121,10 @@ MAIN_KERNELS = tuple(k for k, w, _, _ in KERNELS if "B=256" in w)
 _BY_WORKLOAD = {w: k for k, w, _, _ in KERNELS}
 TRAFFIC_KEYS = [
     (("gemm", "fwd"), KERNELS[0][0]), (("gemm", "bwd_dw"), KERNELS[3][0]), (("gemm", "bwd_dz"), KERNELS[1][0]),
-    (("skinny", "fwd"), _BY_WORKLOAD["Linear 8192^2 B=8, 12 and 16 forward"]),
+    (("skinny", "fwd"), _BY_WORKLOAD["Linear 8192^2 B=8 forward"]),
     (("skinny", "bwd_dz"), _BY_WORKLOAD["Linear 8192^2 B=8 delta_z"]),
     (("skinny", "bwd_dw"), _BY_WORKLOAD["Linear 8192^2 B=8 delta_w (+delta_b)"]),
+    (("skinny12", "fwd"), _BY_WORKLOAD["Linear 8192^2 B=12 and B=16 forward"]),
     (("skinny12", "bwd_dz"), _BY_WORKLOAD["Linear 8192^2 B=12 and B=16 delta_z"]),
     (("skinny12", "bwd_dw"), _BY_WORKLOAD["Linear 8192^2 B=12 and B=16 delta_w (+delta_b)"]),
     (("conv", "fwd"), _BY_WORKLOAD["Conv2d 3x3 64->64 @32x32 B=128 forward"]),
