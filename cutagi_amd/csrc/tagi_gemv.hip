@@ -11,8 +11,10 @@
 // streaming kernel.
 //
 // The forward and state-backward kernels here are instantiated for up to 16
-// samples but dispatched for B <= 8; 9..16 samples take the 16x16x4 kernels of
-// tagi_gemv16.hip. The weight backward serves every B <= 16.
+// samples. As dispatched, the state backward serves B <= 8 (9..16 samples take the
+// 16x16x4 kernel of tagi_gemv16.hip) and the forward none: the 16x16x4 forward
+// measured faster for every batch, and this one stays behind a test switch
+// ("linear.gemv16.min_batch"). The weight backward serves every B <= 16.
 //
 // Reduction slices (gridDim.y) write partial sums [slice][B][cols]; the caller
 // folds them, together with the bias or Jacobian epilogue, in reduce_splits.

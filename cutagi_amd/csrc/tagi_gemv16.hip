@@ -1,4 +1,6 @@
-// Skinny-batch kernels of the TAGI Linear layer for 9 <= B <= 16, gfx950.
+// Skinny-batch kernels of the TAGI Linear layer on 16-wide MFMAs, gfx950: the forward
+// for every batch up to 32 (two groups of sixteen samples beyond 16), the state
+// backward for 9 <= B <= 16.
 //
 // Same plan as tagi_gemv.hip (the weight matrices stream from HBM once, straight
 // into MFMA operand layout; the few activations / innovations sit in LDS), but on
