@@ -131,12 +131,18 @@ int pick_tile(int rows) {
     return 2;
 }
 
-// Reduction slices so that a launch reaches about two workgroups per CU, while
-// every slice keeps at least `min_tiles` k-tiles of work.
+// Reduction slices so that a launch reaches about two workgroups per CU (one where that
+// takes more than eight slices), while every slice keeps at least `min_tiles` k-tiles of
+// work.
 int pick_splits(int tiles, int reduction, int forced, int min_tiles = 8) {
     const int kt = gemm_k_tile();
     const int k_tiles = ceil_div(reduction, kt);
     int s = forced > 0 ? forced : ceil_div(2 * num_cu(), tiles);
+    // Beyond eight slices the partial sums cost more than the second workgroup per CU
+    // gives: one per CU then (4096^2, forward + backward: batch 64 163 -> 156 us with 8
+    // instead of 16 slices, batch 128 272 -> 270 us with 4 instead of 8; batch 256 and
+    // 512 are faster with two per CU, 496 against 500 us and 947 against 958 us).
+    if (forced <= 0 && s > 8) s = std::max(8, ceil_div(num_cu(), tiles));
     int cap = k_tiles / min_tiles > 0 ? k_tiles / min_tiles : 1;
     // A launch that leaves most of the chip empty is bound by the latency of its
     // k-tile loop (one memory round trip per k-tile, nothing else on the CU to hide
